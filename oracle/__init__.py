@@ -1,0 +1,254 @@
+"""ctypes binding of the CPU oracle (``oracle/libppml_oracle.so``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py`` -- as the checker, never as the thing measured or shipped.
+The GPU package never imports this module.
+
+Array conventions follow the reference: Q8_0 blocks are 34-byte records ``{fp16 d; int8 qs[32]}``
+held here as ``uint8`` arrays of shape ``[..., nblocks, 34]``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libppml_oracle.so")
+_REF_PATH = os.path.join(_HERE, "_ref", "libppml_ref_half.so")
+
+QK = 32
+BLOCK_BYTES = 34
+
+
+def build(force: bool = False) -> None:
+    """Compile the oracle (and the reference's HalfUtils.h wrapper when the reference is mounted)."""
+    args = ["make", "-C", _HERE]
+    if force:
+        args.append("-B")
+    subprocess.run(args, check=True, stdout=subprocess.DEVNULL)
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = C.CDLL(_LIB_PATH)
+    f32p, i32p, vp = C.POINTER(C.c_float), C.POINTER(C.c_int32), C.c_void_p
+    i64 = C.c_int64
+    lib.orc_fp32_to_fp16.restype = C.c_uint16
+    lib.orc_fp32_to_fp16.argtypes = [C.c_float]
+    lib.orc_fp16_to_fp32.restype = C.c_float
+    lib.orc_fp16_to_fp32.argtypes = [C.c_uint16]
+    lib.orc_quantize_q8_0.restype = C.c_int
+    lib.orc_quantize_q8_0.argtypes = [f32p, vp, i64]
+    lib.orc_q8_0_repacked_bytes.restype = C.c_size_t
+    lib.orc_q8_0_repacked_bytes.argtypes = [i64]
+    lib.orc_repack_q8_0.restype = None
+    lib.orc_repack_q8_0.argtypes = [vp, i64, vp]
+    lib.orc_unrepack_q8_0.restype = None
+    lib.orc_unrepack_q8_0.argtypes = [vp, i64, vp]
+    lib.orc_dequantize_q8_0.restype = None
+    lib.orc_dequantize_q8_0.argtypes = [vp, f32p, i64]
+    lib.orc_q8_block_sums.restype = C.c_int
+    lib.orc_q8_block_sums.argtypes = [vp, vp, i32p, C.c_int, C.c_int, C.c_int]
+    lib.orc_mul_mat_q8q8.restype = C.c_int
+    lib.orc_mul_mat_q8q8.argtypes = [vp, vp, f32p] + [C.c_int] * 6
+    lib.orc_mul_mat_q8.restype = C.c_int
+    lib.orc_mul_mat_q8.argtypes = [vp, f32p, f32p] + [C.c_int] * 7
+    lib.orc_mul_mat_f32.restype = None
+    lib.orc_mul_mat_f32.argtypes = [f32p, f32p, f32p, C.c_int, C.c_int, C.c_int, f32p, C.c_int]
+    lib.orc_out_prod.restype = None
+    lib.orc_out_prod.argtypes = [f32p, f32p, f32p] + [i64] * 12 + [C.c_int]
+    lib.orc_outer_prod_mean.restype = None
+    lib.orc_outer_prod_mean.argtypes = [f32p, f32p, f32p] + [i64] * 4 + [C.c_int]
+    lib.orc_outer_product_mean_value.restype = None
+    lib.orc_outer_product_mean_value.argtypes = [f32p, f32p, f32p] + [i64] * 4 + [C.c_int]
+    lib.orc_attention_scores.restype = None
+    lib.orc_attention_scores.argtypes = [f32p, f32p, f32p] + [i64] * 5 + [C.c_int]
+    lib.orc_max_threads.restype = C.c_int
+    return lib
+
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        _lib = _load()
+    return _lib
+
+
+def ref_half_lib():
+    """The reference's own HalfUtils.h compiled as-is, or None when it was never built."""
+    if not os.path.exists(_REF_PATH):
+        return None
+    ref = C.CDLL(_REF_PATH)
+    ref.ref_fp32_to_fp16.restype = C.c_uint16
+    ref.ref_fp32_to_fp16.argtypes = [C.c_float]
+    ref.ref_fp16_to_fp32.restype = C.c_float
+    ref.ref_fp16_to_fp32.argtypes = [C.c_uint16]
+    ref.ref_sweep_fp32_to_fp16.restype = C.c_int64
+    ref.ref_sweep_fp32_to_fp16.argtypes = [C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32)]
+    return ref
+
+
+def _f32(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _fp(a: np.ndarray):
+    return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _vp(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def max_threads() -> int:
+    return int(lib().orc_max_threads())
+
+
+def fp32_to_fp16(x: float) -> int:
+    return int(lib().orc_fp32_to_fp16(C.c_float(x)))
+
+
+def fp16_to_fp32(h: int) -> float:
+    return float(lib().orc_fp16_to_fp32(C.c_uint16(h)))
+
+
+def quantize_q8_0(x) -> np.ndarray:
+    """f32 [..., K] -> uint8 [..., K/32, 34] (QuantBlocks.h:62-79)."""
+    x = _f32(x)
+    n = x.size
+    if n % QK:
+        raise ValueError("element count is not a multiple of 32")
+    out = np.empty((n // QK, BLOCK_BYTES), dtype=np.uint8)
+    rc = lib().orc_quantize_q8_0(_fp(x), _vp(out), n)
+    assert rc == 0
+    return out.reshape(x.shape[:-1] + (x.shape[-1] // QK, BLOCK_BYTES))
+
+
+def block_scales_bits(blocks: np.ndarray) -> np.ndarray:
+    return np.ascontiguousarray(blocks[..., :2]).view(np.uint16)[..., 0]
+
+
+def block_quants(blocks: np.ndarray) -> np.ndarray:
+    return np.ascontiguousarray(blocks[..., 2:]).view(np.int8)
+
+
+def repack_q8_0(blocks: np.ndarray) -> np.ndarray:
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    nb = blocks.size // BLOCK_BYTES
+    out = np.empty(nb * BLOCK_BYTES, dtype=np.uint8)
+    lib().orc_repack_q8_0(_vp(blocks), nb, _vp(out))
+    return out
+
+
+def unrepack_q8_0(packed: np.ndarray) -> np.ndarray:
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    nb = packed.size // BLOCK_BYTES
+    out = np.empty((nb, BLOCK_BYTES), dtype=np.uint8)
+    lib().orc_unrepack_q8_0(_vp(packed), nb, _vp(out))
+    return out
+
+
+def dequantize_q8_0(blocks: np.ndarray) -> np.ndarray:
+    blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+    nb = blocks.size // BLOCK_BYTES
+    out = np.empty(nb * QK, dtype=np.float32)
+    lib().orc_dequantize_q8_0(_vp(blocks), _fp(out), nb * QK)
+    return out.reshape(blocks.shape[:-2] + (blocks.shape[-2] * QK,))
+
+
+def q8_block_sums(wq: np.ndarray, xq: np.ndarray) -> np.ndarray:
+    """wq [M, nblk, 34], xq [N, nblk, 34] -> int32 [N, M, nblk]."""
+    wq = np.ascontiguousarray(wq, dtype=np.uint8)
+    xq = np.ascontiguousarray(xq, dtype=np.uint8)
+    M, nblk = wq.shape[0], wq.shape[1]
+    N = xq.shape[0]
+    out = np.empty((N, M, nblk), dtype=np.int32)
+    rc = lib().orc_q8_block_sums(_vp(wq), _vp(xq), out.ctypes.data_as(C.POINTER(C.c_int32)),
+                                 M, N, nblk * QK)
+    assert rc == 0, rc
+    return out
+
+
+def mul_mat_q8q8(wq, xq, c_trans=1, fma=1, nthreads=0) -> np.ndarray:
+    wq = np.ascontiguousarray(wq, dtype=np.uint8)
+    xq = np.ascontiguousarray(xq, dtype=np.uint8)
+    M, nblk = wq.shape[0], wq.shape[1]
+    N = xq.shape[0]
+    out = np.empty((N, M) if c_trans else (M, N), dtype=np.float32)
+    rc = lib().orc_mul_mat_q8q8(_vp(wq), _vp(xq), _fp(out), M, N, nblk * QK, c_trans, fma, nthreads)
+    assert rc == 0, rc
+    return out
+
+
+def mul_mat_q8(w, x, wtype=0, c_trans=1, fma=1, nthreads=0) -> np.ndarray:
+    """w: Q8_0 weight bytes (wtype 0: [M, K/32, 34]; wtype 2: flat Q8_0R), x f32 [N, K]."""
+    x = _f32(x)
+    N, K = x.shape
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    M = w.size // (K // QK * BLOCK_BYTES)
+    out = np.empty((N, M) if c_trans else (M, N), dtype=np.float32)
+    rc = lib().orc_mul_mat_q8(_vp(w), _fp(x), _fp(out), M, N, K, wtype, c_trans, fma, nthreads)
+    if rc:
+        raise RuntimeError(f"orc_mul_mat_q8 rc={rc}")
+    return out
+
+
+def mul_mat_f32(a, b, bias=None, nthreads=0) -> np.ndarray:
+    """a [M,K], b [N,K] -> [M,N] (CPUKernels.cpp:763-771)."""
+    a, b = _f32(a), _f32(b)
+    M, K = a.shape
+    N = b.shape[0]
+    out = np.empty((M, N), dtype=np.float32)
+    bp = None
+    if bias is not None:
+        bias = _f32(bias)
+        bp = _fp(bias)
+    lib().orc_mul_mat_f32(_fp(a), _fp(b), _fp(out), M, K, N, bp, nthreads)
+    return out
+
+
+def out_prod(s0, s1, nthreads=0) -> np.ndarray:
+    """Arrays are numpy-shaped outermost first: s0 [ne03,ne02,ne01,ne00], s1 [ne13,ne12,ne11,ne10]
+    -> dst [ne3,ne2,ne1(=ne10),ne0(=ne00)] (CPUKernels.cpp:787-887)."""
+    s0, s1 = _f32(s0), _f32(s1)
+    ne03, ne02, ne01, ne00 = s0.shape
+    ne13, ne12, ne11, ne10 = s1.shape
+    ne0, ne1, ne2, ne3 = ne00, ne10, max(ne02, ne12), max(ne03, ne13)
+    out = np.empty((ne3, ne2, ne1, ne0), dtype=np.float32)
+    lib().orc_out_prod(_fp(s0), _fp(s1), _fp(out), ne00, ne01, ne02, ne03, ne10, ne11, ne12, ne13,
+                       ne0, ne1, ne2, ne3, nthreads)
+    return out
+
+
+def outer_prod_mean(left, right, D, L, N, B, nthreads=0) -> np.ndarray:
+    """Graph form; flat buffers indexed exactly as CPUKernels.cpp:1006-1028."""
+    left, right = _f32(left).ravel(), _f32(right).ravel()
+    out = np.empty(D * D * L * L * B, dtype=np.float32)
+    lib().orc_outer_prod_mean(_fp(left), _fp(right), _fp(out), D, L, N, B, nthreads)
+    return out
+
+
+def outer_product_mean_value(left, right, nthreads=0) -> np.ndarray:
+    """Value form: left/right (B,N,L,D) -> (B,L,L,D*D) (MathUtils.cpp:387-437)."""
+    left, right = _f32(left), _f32(right)
+    B, N, L, D = left.shape
+    out = np.empty((B, L, L, D * D), dtype=np.float32)
+    lib().orc_outer_product_mean_value(_fp(left), _fp(right), _fp(out), B, N, L, D, nthreads)
+    return out
+
+
+def attention_scores(q, k, nthreads=0) -> np.ndarray:
+    """Q (NQ,H,D,Lq), K (NQ,H,D,Lk) -> (NQ,H,Lq,Lk) incl. 1/sqrt(D) (Attention.cpp:58-79)."""
+    q, k = _f32(q), _f32(k)
+    NQ, H, D, Lq = q.shape
+    Lk = k.shape[3]
+    out = np.empty((NQ, H, Lq, Lk), dtype=np.float32)
+    lib().orc_attention_scores(_fp(q), _fp(k), _fp(out), NQ, H, D, Lq, Lk, nthreads)
+    return out

@@ -1,0 +1,368 @@
+/*
+ * ppml_oracle.c -- CPU restatement of the reference's matrix-multiplication path.
+ *
+ * TEST INFRASTRUCTURE ONLY (see ppml_oracle.h).  Build: `make -C oracle`
+ * (gcc -O2 -ffp-contract=off -fopenmp; no fast-math, so every float operation rounds
+ * exactly as the reference's x86-64 -O2 build, which has no FMA contraction).
+ *
+ * Pinning status (what fixes each function besides the reference text):
+ *   orc_fp32_to_fp16 / orc_fp16_to_fp32 : own bit-level algorithm, checked against the
+ *       reference's HalfUtils.h compiled as-is (oracle/_ref) and against numpy float16.
+ *   orc_quantize_q8_0 : closed form per block; invariants (arg-max -> +-127, zero block ->
+ *       d=0,q=0, |x - d*q| <= d/2), a hand-checked vector, and an independent
+ *       double-precision restatement on random blocks.
+ *   orc_repack/unrepack : round trip + plane offsets.
+ *   orc_q8_block_sums   : exact integers, brute force with numpy int64.
+ *   orc_mul_mat_q8q8    : PARITY UNPINNED by any reference-held test (the reference's own
+ *       Q8 tests are absent from its tree and its CPU backend has no Q8 kernel); pinned
+ *       by the closed form sum_ib float(sumi)*(dw*da) evaluated in float64 and by the
+ *       dequantised f32 GEMM special case.
+ *   orc_mul_mat_f32     : the reference's MulMat test inputs (tests/test_cuda.cpp:133-167),
+ *       whose products and sums are exact in binary32, against integer arithmetic.
+ *   orc_out_prod        : the reference's OutProd inputs (tests/test_cuda.cpp:207-245, 262-341),
+ *       exact, plus broadcast special cases against numpy einsum.
+ *   orc_outer_prod_mean : graph form; no reference-held vector covers its index decode and the
+ *       reference kernel cannot be compiled here (CUDA headers absent) -- pinned only by numpy
+ *       einsum over the layout stated at src/backend/CPUKernels.cpp:975-981.
+ *   orc_outer_product_mean_value : known answers of tests/test_outer_product_mean.cpp:10-70.
+ *   orc_attention_scores: einsum special case and the 1/sqrt(D) closed form.
+ */
+#include "ppml_oracle.h"
+
+#include <math.h>
+#include <string.h>
+#include <stdlib.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static int pick_threads(int nthreads) {
+#ifdef _OPENMP
+    if (nthreads <= 0) return omp_get_max_threads();
+    return nthreads;
+#else
+    (void)nthreads;
+    return 1;
+#endif
+}
+
+int orc_max_threads(void) { return pick_threads(0); }
+
+/* ------------------------------------------------------------------ fp16 */
+/* Same function as include/ppml/HalfUtils.h:42-52 (round to nearest even, NaN -> sign|0x7E00),
+ * written as explicit exponent/mantissa arithmetic rather than the reference's float-add trick. */
+uint16_t orc_fp32_to_fp16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, sizeof u);
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    const uint32_t mag = u & 0x7fffffffu;
+    if (mag > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);           /* NaN */
+    if (mag >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);          /* >= 65520 -> inf */
+    if (mag < 0x38800000u) {                                            /* below 2^-14: subnormal half */
+        if (mag < 0x33000000u) return (uint16_t)sign;                   /* < 2^-25 -> 0 */
+        const int e = (int)(mag >> 23);                                 /* biased exponent, 102..112 */
+        const uint32_t m = (mag & 0x7fffffu) | 0x800000u;               /* 24-bit significand */
+        const int shift = 126 - e;                                      /* result = m >> shift, 14..24 */
+        uint32_t h = m >> shift;
+        const uint32_t rem = m & ((1u << shift) - 1u);
+        const uint32_t half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (h & 1u))) h++;
+        return (uint16_t)(sign | h);
+    }
+    uint32_t h = (((mag >> 23) - 112u) << 10) | ((mag & 0x7fffffu) >> 13);
+    const uint32_t rem = mag & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++;             /* carry may bump the exponent */
+    return (uint16_t)(sign | h);
+}
+
+/* include/ppml/HalfUtils.h:26-37 (exact widening) */
+float orc_fp16_to_fp32(uint16_t h) {
+    const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 0x1fu;
+    uint32_t m = h & 0x3ffu;
+    uint32_t u;
+    if (e == 0x1fu) {
+        u = sign | 0x7f800000u | (m << 13);
+    } else if (e != 0) {
+        u = sign | ((e + 112u) << 23) | (m << 13);
+    } else if (m == 0) {
+        u = sign;
+    } else {
+        int ee = 113;
+        while (!(m & 0x400u)) { m <<= 1; ee--; }
+        u = sign | ((uint32_t)ee << 23) | ((m & 0x3ffu) << 13);
+    }
+    float f;
+    memcpy(&f, &u, sizeof f);
+    return f;
+}
+
+/* ------------------------------------------------------------------ Q8_0 */
+static inline uint16_t blk_d_bits(const uint8_t *blk) {
+    uint16_t d;
+    memcpy(&d, blk, 2);
+    return d;
+}
+
+/* include/ppml/QuantBlocks.h:62-79 */
+int orc_quantize_q8_0(const float *src, void *dst_blocks, int64_t n) {
+    if (n % ORC_QK8_0 != 0) return 1;
+    const int64_t nb = n / ORC_QK8_0;
+    uint8_t *out = (uint8_t *)dst_blocks;
+    for (int64_t b = 0; b < nb; ++b) {
+        const float *x = src + b * ORC_QK8_0;
+        float amax = 0.0f;
+        for (int i = 0; i < ORC_QK8_0; ++i) amax = fmaxf(amax, fabsf(x[i]));
+        const float d = amax / 127.0f;
+        const float inv = (amax == 0.0f) ? 0.0f : 1.0f / d;   /* the f32 d, not its fp16 rounding */
+        const uint16_t dh = orc_fp32_to_fp16(d);
+        uint8_t *blk = out + b * ORC_Q8_0_BLOCK_BYTES;
+        memcpy(blk, &dh, 2);
+        for (int i = 0; i < ORC_QK8_0; ++i) {
+            float q = roundf(x[i] * inv);                     /* half away from zero */
+            q = q > 127.0f ? 127.0f : (q < -127.0f ? -127.0f : q);
+            ((int8_t *)(blk + 2))[i] = (int8_t)q;
+        }
+    }
+    return 0;
+}
+
+/* include/ppml/QuantBlocks.h:119-121 */
+size_t orc_q8_0_repacked_bytes(int64_t numel) {
+    return (size_t)(numel / ORC_QK8_0) * (ORC_QK8_0 + 2);
+}
+
+/* include/ppml/QuantBlocks.h:123-133 */
+void orc_repack_q8_0(const void *src_blocks, int64_t nblocks, void *dst) {
+    const uint8_t *src = (const uint8_t *)src_blocks;
+    uint8_t *qs = (uint8_t *)dst;
+    uint8_t *d = qs + nblocks * ORC_QK8_0;
+    for (int64_t b = 0; b < nblocks; ++b) {
+        memcpy(qs + b * ORC_QK8_0, src + b * ORC_Q8_0_BLOCK_BYTES + 2, ORC_QK8_0);
+        memcpy(d + b * 2, src + b * ORC_Q8_0_BLOCK_BYTES, 2);
+    }
+}
+
+/* include/ppml/QuantBlocks.h:136-145 */
+void orc_unrepack_q8_0(const void *src, int64_t nblocks, void *dst_blocks) {
+    const uint8_t *qs = (const uint8_t *)src;
+    const uint8_t *d = qs + nblocks * ORC_QK8_0;
+    uint8_t *dst = (uint8_t *)dst_blocks;
+    for (int64_t b = 0; b < nblocks; ++b) {
+        memcpy(dst + b * ORC_Q8_0_BLOCK_BYTES + 2, qs + b * ORC_QK8_0, ORC_QK8_0);
+        memcpy(dst + b * ORC_Q8_0_BLOCK_BYTES, d + b * 2, 2);
+    }
+}
+
+/* include/ppml/QuantBlocks.h:164-170 */
+void orc_dequantize_q8_0(const void *src_blocks, float *dst, int64_t n) {
+    const uint8_t *src = (const uint8_t *)src_blocks;
+    const int64_t nb = n / ORC_QK8_0;
+    for (int64_t b = 0; b < nb; ++b) {
+        const uint8_t *blk = src + b * ORC_Q8_0_BLOCK_BYTES;
+        const float d = orc_fp16_to_fp32(blk_d_bits(blk));
+        const int8_t *q = (const int8_t *)(blk + 2);
+        for (int i = 0; i < ORC_QK8_0; ++i) dst[b * ORC_QK8_0 + i] = d * (float)q[i];
+    }
+}
+
+static inline int32_t block_dot(const uint8_t *wb, const uint8_t *xb) {
+    const int8_t *w = (const int8_t *)(wb + 2);
+    const int8_t *x = (const int8_t *)(xb + 2);
+    int32_t s = 0;
+    for (int i = 0; i < ORC_QK8_0; ++i) s += (int32_t)w[i] * (int32_t)x[i];
+    return s;
+}
+
+/* the integer part of src/cuda/MulMatQ8Kernel.cu:120-139 */
+int orc_q8_block_sums(const void *w_blocks, const void *x_blocks, int32_t *sums,
+                      int M, int N, int K) {
+    if (!w_blocks || !x_blocks || !sums || M <= 0 || N <= 0 || K <= 0) return 1;
+    if (K % ORC_QK8_0) return 2;
+    const int nblk = K / ORC_QK8_0;
+    const uint8_t *W = (const uint8_t *)w_blocks;
+    const uint8_t *X = (const uint8_t *)x_blocks;
+    for (int n = 0; n < N; ++n)
+        for (int m = 0; m < M; ++m)
+            for (int ib = 0; ib < nblk; ++ib)
+                sums[((int64_t)n * M + m) * nblk + ib] =
+                    block_dot(W + ((int64_t)m * nblk + ib) * ORC_Q8_0_BLOCK_BYTES,
+                              X + ((int64_t)n * nblk + ib) * ORC_Q8_0_BLOCK_BYTES);
+    return 0;
+}
+
+/* src/cuda/MulMatQ8Kernel.cu:108-145: one output = blocks ascending,
+ * acc += float(sumi) * (d_w * d_a); d_w*d_a is the exact f32 product of two halves. */
+int orc_mul_mat_q8q8(const void *w_blocks, const void *x_blocks, float *C,
+                     int M, int N, int K, int c_trans, int fma, int nthreads) {
+    if (!w_blocks || !x_blocks || !C || M <= 0 || N <= 0 || K <= 0) return 1;
+    if (K % ORC_QK8_0) return 2;
+    const int nblk = K / ORC_QK8_0;
+    const uint8_t *W = (const uint8_t *)w_blocks;
+    const uint8_t *X = (const uint8_t *)x_blocks;
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(dynamic, 4) num_threads(nt)
+    for (int n = 0; n < N; ++n) {
+        const uint8_t *xrow = X + (int64_t)n * nblk * ORC_Q8_0_BLOCK_BYTES;
+        for (int m = 0; m < M; ++m) {
+            const uint8_t *wrow = W + (int64_t)m * nblk * ORC_Q8_0_BLOCK_BYTES;
+            float acc = 0.0f;
+            for (int ib = 0; ib < nblk; ++ib) {
+                const uint8_t *wb = wrow + ib * ORC_Q8_0_BLOCK_BYTES;
+                const uint8_t *xb = xrow + ib * ORC_Q8_0_BLOCK_BYTES;
+                const int32_t sumi = block_dot(wb, xb);
+                const float s = orc_fp16_to_fp32(blk_d_bits(wb)) * orc_fp16_to_fp32(blk_d_bits(xb));
+                if (fma) {
+                    acc = fmaf((float)sumi, s, acc);
+                } else {
+                    const float t = (float)sumi * s;
+                    acc = acc + t;
+                }
+            }
+            if (c_trans) C[(int64_t)n * M + m] = acc;
+            else         C[(int64_t)m * N + n] = acc;
+        }
+    }
+    return 0;
+}
+
+/* src/cuda/MulMatQ8Kernel.cu:476-547 with Q8_0 activations (QuantBlocks.h:62-79 per row). */
+int orc_mul_mat_q8(const void *W, const float *X, float *C, int M, int N, int K,
+                   int wtype, int c_trans, int fma, int nthreads) {
+    if (!W || !X || !C || M <= 0 || N <= 0 || K <= 0) return 1;
+    if (K % ORC_QK8_0) return 2;
+    if (wtype != 0 && wtype != 2) return 5;
+    const int64_t nblk = K / ORC_QK8_0;
+    uint8_t *xq = (uint8_t *)malloc((size_t)N * nblk * ORC_Q8_0_BLOCK_BYTES);
+    if (!xq) return 3;
+    uint8_t *wq = NULL;
+    const void *wblocks = W;
+    if (wtype == 2) {
+        wq = (uint8_t *)malloc((size_t)M * nblk * ORC_Q8_0_BLOCK_BYTES);
+        if (!wq) { free(xq); return 3; }
+        orc_unrepack_q8_0(W, (int64_t)M * nblk, wq);
+        wblocks = wq;
+    }
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(static) num_threads(nt)
+    for (int n = 0; n < N; ++n)
+        orc_quantize_q8_0(X + (int64_t)n * K, xq + (int64_t)n * nblk * ORC_Q8_0_BLOCK_BYTES, K);
+    const int rc = orc_mul_mat_q8q8(wblocks, xq, C, M, N, K, c_trans, fma, nthreads);
+    free(xq);
+    free(wq);
+    return rc;
+}
+
+/* ------------------------------------------------------------------ f32 */
+/* src/backend/CPUKernels.cpp:763-771: rows handed out one at a time, bias enters the
+ * accumulator first, k ascending, separate multiply and add. */
+void orc_mul_mat_f32(const float *a, const float *b, float *d, int M, int K, int N,
+                     const float *bias, int nthreads) {
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(nt)
+    for (int i = 0; i < M; ++i) {
+        for (int j = 0; j < N; ++j) {
+            float sum = bias ? bias[j] : 0.0f;
+            for (int k = 0; k < K; ++k) sum += a[(int64_t)i * K + k] * b[(int64_t)j * K + k];
+            d[j + (int64_t)i * N] = sum;
+        }
+    }
+}
+
+/* src/backend/CPUKernels.cpp:787-887: dst zeroed, then for each dst row (i1,i2,i3)
+ * d_row[i0] += s0[i0,k,i02,i03] * s1[i1,k,i2,i3], k ascending (the reference's K-blocking of
+ * 32 and row-blocking of 16 leave the per-element order unchanged); src0 planes broadcast
+ * with i02 = i2 / (ne2/ne02), i03 = i3 / (ne3/ne03). */
+void orc_out_prod(const float *s0, const float *s1, float *dst,
+                  int64_t ne00, int64_t ne01, int64_t ne02, int64_t ne03,
+                  int64_t ne10, int64_t ne11, int64_t ne12, int64_t ne13,
+                  int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3, int nthreads) {
+    (void)ne13;
+    const int64_t nr = ne1 * ne2 * ne3;
+    const int64_t dps2 = ne2 / ne02;
+    const int64_t dps3 = ne3 / ne03;
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(static) num_threads(nt)
+    for (int64_t ir = 0; ir < nr; ++ir) {
+        const int64_t i3 = ir / (ne2 * ne1);
+        const int64_t i2 = (ir - i3 * ne2 * ne1) / ne1;
+        const int64_t i1 = ir - i3 * ne2 * ne1 - i2 * ne1;
+        const int64_t i02 = i2 / dps2;
+        const int64_t i03 = i3 / dps3;
+        float *d_row = dst + (i1 * ne0 + i2 * ne0 * ne1 + i3 * ne0 * ne1 * ne2);
+        for (int64_t i0 = 0; i0 < ne0; ++i0) d_row[i0] = 0.0f;
+        for (int64_t k = 0; k < ne01; ++k) {
+            const float *a = s0 + (k * ne00 + i02 * ne00 * ne01 + i03 * ne00 * ne01 * ne02);
+            const float bv = s1[i1 + k * ne10 + i2 * ne10 * ne11 + i3 * ne10 * ne11 * ne12];
+            for (int64_t i0 = 0; i0 < ne00; ++i0) d_row[i0] += a[i0] * bv;
+        }
+    }
+}
+
+/* src/backend/CPUKernels.cpp:982-1032: flat output index decoded b -> j -> i -> d2 -> d1,
+ * inputs indexed ((d*L + i)*N + n)*B + b, sum over n ascending, 1/N applied after the sum. */
+void orc_outer_prod_mean(const float *left, const float *right, float *dst,
+                         int64_t D, int64_t L, int64_t N, int64_t B, int nthreads) {
+    const float inv_N = 1.0f / (float)N;
+    const int64_t total = D * D * L * L * B;
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(static) num_threads(nt)
+    for (int64_t idx = 0; idx < total; ++idx) {
+        int64_t t = idx;
+        const int64_t b = t % B; t /= B;
+        const int64_t j = t % L; t /= L;
+        const int64_t i = t % L; t /= L;
+        const int64_t d2 = t % D; t /= D;
+        const int64_t d1 = t;
+        float sum = 0.0f;
+        for (int64_t n = 0; n < N; ++n)
+            sum += left[((d1 * L + i) * N + n) * B + b] * right[((d2 * L + j) * N + n) * B + b];
+        dst[idx] = sum * inv_N;
+    }
+}
+
+/* src/ops/MathUtils.cpp:387-437: left/right (B,N,L,D) row-major -> dst (B,L,L,D*D). */
+void orc_outer_product_mean_value(const float *left, const float *right, float *dst,
+                                  int64_t B, int64_t N, int64_t L, int64_t D, int nthreads) {
+    const float inv_N = 1.0f / (float)N;
+    const int64_t D2 = D * D;
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(static) collapse(2) num_threads(nt)
+    for (int64_t b = 0; b < B; ++b)
+        for (int64_t i = 0; i < L; ++i)
+            for (int64_t j = 0; j < L; ++j)
+                for (int64_t d1 = 0; d1 < D; ++d1)
+                    for (int64_t d2 = 0; d2 < D; ++d2) {
+                        float sum = 0.0f;
+                        for (int64_t n = 0; n < N; ++n)
+                            sum += left[((b * N + n) * L + i) * D + d1] *
+                                   right[((b * N + n) * L + j) * D + d2];
+                        dst[((b * L + i) * L + j) * D2 + (d1 * D + d2)] = sum * inv_N;
+                    }
+}
+
+/* src/modules/Attention.cpp:58-79: Q,K value layout (NQ,H,D,L); scores (NQ,H,Lq,Lk),
+ * scaled by 1/sqrt(D) after the sum. */
+void orc_attention_scores(const float *Q, const float *K, float *scores,
+                          int64_t NQ, int64_t H, int64_t D, int64_t Lq, int64_t Lk, int nthreads) {
+    const float inv_scale = 1.0f / sqrtf((float)D);
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(static) collapse(2) num_threads(nt)
+    for (int64_t b = 0; b < NQ; ++b)
+        for (int64_t h = 0; h < H; ++h)
+            for (int64_t i = 0; i < Lq; ++i)
+                for (int64_t j = 0; j < Lk; ++j) {
+                    float s = 0.0f;
+                    const float *qp = Q + ((b * H + h) * D) * Lq + i;
+                    const float *kp = K + ((b * H + h) * D) * Lk + j;
+                    for (int64_t d = 0; d < D; ++d) s += qp[d * Lq] * kp[d * Lk];
+                    scores[((b * H + h) * Lq + i) * Lk + j] = s * inv_scale;
+                }
+}

@@ -1,0 +1,80 @@
+/*
+ * ppml_oracle.h -- CPU restatement of the reference's matrix-multiplication path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This library is the checker for the HIP kernels: it is
+ * loaded by the test-suite, by the smoke check and by the benchmark's cpu_baseline leg.
+ * Nothing in the shipped GPU path may call it; the GPU library has no CPU fallback.
+ *
+ * Every function cites the reference file:line whose loop it restates
+ * (paths relative to the reference tree).  Storage conventions are the reference's:
+ *   block_q8_0  = { fp16 d; int8 qs[32]; }  34 bytes, 2-byte aligned   (include/ppml/QuantBlocks.h:33-36)
+ *   Q8_0R       = qs plane [nblocks][32] followed by d plane [nblocks] fp16 (QuantBlocks.h:113-135)
+ *
+ * Pinning status of each function is recorded next to its definition in ppml_oracle.c.
+ */
+#ifndef PPML_ORACLE_H
+#define PPML_ORACLE_H
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ORC_QK8_0 32
+#define ORC_Q8_0_BLOCK_BYTES 34
+
+/* include/ppml/HalfUtils.h:26-52 */
+uint16_t orc_fp32_to_fp16(float f);
+float    orc_fp16_to_fp32(uint16_t h);
+
+/* include/ppml/QuantBlocks.h:62-79 ; returns 0 on success, 1 if n % 32 != 0 */
+int  orc_quantize_q8_0(const float *src, void *dst_blocks, int64_t n);
+/* include/ppml/QuantBlocks.h:123-145 */
+size_t orc_q8_0_repacked_bytes(int64_t numel);
+void orc_repack_q8_0(const void *src_blocks, int64_t nblocks, void *dst);
+void orc_unrepack_q8_0(const void *src, int64_t nblocks, void *dst_blocks);
+/* include/ppml/QuantBlocks.h:164-170 */
+void orc_dequantize_q8_0(const void *src_blocks, float *dst, int64_t n);
+
+/* per-block int32 sums of src/cuda/MulMatQ8Kernel.cu:120-139:
+ * sums[(n*M + m)*nblk + ib] = sum_{i<32} W[m][ib].qs[i] * X[n][ib].qs[i]      */
+int  orc_q8_block_sums(const void *w_blocks, const void *x_blocks, int32_t *sums,
+                       int M, int N, int K);
+
+/* src/cuda/MulMatQ8Kernel.cu:108-145 on two Q8_0 operands (M = weight rows, N = activation rows).
+ * c_trans 0: C[m*N+n]   c_trans 1: C[n*M+m].   fma != 0 -> acc = fmaf(float(sumi), dw*da, acc)
+ * (what nvcc's default contraction makes of the reference line), fma == 0 -> rounded product
+ * then rounded add.  returns 0 ok, 1 bad args, 2 K % 32.                                      */
+int  orc_mul_mat_q8q8(const void *w_blocks, const void *x_blocks, float *C,
+                      int M, int N, int K, int c_trans, int fma, int nthreads);
+/* Whole Q8_0 linear: quantize every activation row with orc_quantize_q8_0, then the loop above.
+ * wtype 0 = interleaved block_q8_0, 2 = Q8_0R; others -> 5 (src/cuda/MulMatQ8Kernel.cu:476-547). */
+int  orc_mul_mat_q8(const void *W, const float *X, float *C, int M, int N, int K,
+                    int wtype, int c_trans, int fma, int nthreads);
+
+/* src/backend/CPUKernels.cpp:763-771 ; bias may be NULL */
+void orc_mul_mat_f32(const float *a, const float *b, float *d, int M, int K, int N,
+                     const float *bias, int nthreads);
+/* src/backend/CPUKernels.cpp:787-887 */
+void orc_out_prod(const float *s0, const float *s1, float *dst,
+                  int64_t ne00, int64_t ne01, int64_t ne02, int64_t ne03,
+                  int64_t ne10, int64_t ne11, int64_t ne12, int64_t ne13,
+                  int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3, int nthreads);
+/* src/backend/CPUKernels.cpp:982-1032 */
+void orc_outer_prod_mean(const float *left, const float *right, float *dst,
+                         int64_t D, int64_t L, int64_t N, int64_t B, int nthreads);
+/* src/ops/MathUtils.cpp:387-437 */
+void orc_outer_product_mean_value(const float *left, const float *right, float *dst,
+                                  int64_t B, int64_t N, int64_t L, int64_t D, int nthreads);
+/* src/modules/Attention.cpp:58-79 (scores only, before bias and softmax) */
+void orc_attention_scores(const float *Q, const float *K, float *scores,
+                          int64_t NQ, int64_t H, int64_t D, int64_t Lq, int64_t Lk, int nthreads);
+
+int orc_max_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,349 @@
+"""Pins the CPU oracle before anything is compared against it.
+
+Each check is chosen so that a plausible mistake in the restatement (dropped term, wrong sign or
+index, transposed operand, wrong rounding mode) fails: the reference's own test inputs and known
+answers where it holds them, the reference's HalfUtils.h compiled as-is where that was built, and
+otherwise closed forms, invariants, library special cases and brute force on small inputs.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+
+# ----------------------------------------------------------------------------- fp16
+def _interesting_floats():
+    rng = np.random.default_rng(7)
+    bits = [0x00000000, 0x80000000, 0x33000000, 0x33000001, 0x32ffffff, 0x33800000, 0x387fe000,
+            0x387fffff, 0x38800000, 0x38801000, 0x38800fff, 0x38801001, 0x477fe000, 0x477fefff,
+            0x477ff000, 0x477fffff, 0x47800000, 0x7f7fffff, 0x7f800000, 0xff800000, 0x7fc00000,
+            0xffc00001, 0x3f800000, 0x3f801000, 0x3f803000, 0x3f802fff, 0x3a9ff000]
+    rnd = rng.integers(0, 2**32, size=200000, dtype=np.uint64).astype(np.uint32)
+    # dense coverage of the half range incl. subnormals and ties
+    ties = (np.arange(0, 0x7c00, dtype=np.uint32) << 13) + 0x38000000
+    return np.concatenate([np.array(bits, dtype=np.uint32), rnd, ties, ties + 0x1000, ties + 0x0fff,
+                           ties + 0x1001])
+
+
+def test_fp32_to_fp16_matches_numpy(oracle):
+    u = _interesting_floats()
+    f = u.view(np.float32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = f.astype(np.float16).view(np.uint16)
+    got = np.array([oracle.fp32_to_fp16(float(x)) if not np.isnan(x) else 0 for x in f], dtype=np.uint16)
+    ok = np.isnan(f) | (got == want)
+    assert ok.all(), (hex(int(u[~ok][0])), hex(int(got[~ok][0])), hex(int(want[~ok][0])))
+    # NaN keeps its sign and becomes the quiet pattern (HalfUtils.h:51)
+    assert oracle.lib().orc_fp32_to_fp16(C.c_float(float("nan"))) & 0x7fff == 0x7e00
+
+
+def test_fp16_to_fp32_all_patterns(oracle):
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([oracle.fp16_to_fp32(int(x)) for x in h], dtype=np.float32)
+    nan = np.isnan(want)
+    assert (np.isnan(got) == nan).all()
+    assert (got.view(np.uint32)[~nan] == want.view(np.uint32)[~nan]).all()
+
+
+def test_fp16_against_compiled_reference(oracle):
+    ref = oracle.ref_half_lib()
+    if ref is None:
+        pytest.skip("oracle/_ref was not built (reference tree absent at build time)")
+    for h in range(65536):
+        a, b = oracle.fp16_to_fp32(h), ref.ref_fp16_to_fp32(h)
+        assert (a != a and b != b) or np.float32(a).view(np.uint32) == np.float32(b).view(np.uint32), hex(h)
+    fn = C.cast(oracle.lib().orc_fp32_to_fp16, C.c_void_p)
+    first = C.c_uint32(0)
+    # every 251st binary32 pattern (17M values) plus two offset sweeps around the tie patterns
+    for start, stride in ((0, 251), (0x1000, 0x2000), (0x0fff, 0x2000), (0x1001, 0x2000)):
+        bad = ref.ref_sweep_fp32_to_fp16(fn, start, stride, C.byref(first))
+        assert bad == 0, (bad, hex(first.value))
+
+
+# ----------------------------------------------------------------------------- quantize
+def test_quantize_hand_checked_vector(oracle):
+    x = (0.01 * (np.arange(32, dtype=np.float64) - 15.5)).astype(np.float32)
+    blk = oracle.quantize_q8_0(x)
+    assert blk.shape == (1, 34)
+    assert int(oracle.block_scales_bits(blk)[0]) == 0x1500
+    q = oracle.block_quants(blk)[0]
+    assert q[0] == -127 and q[31] == 127
+    # symmetric ramp: q is odd-symmetric and monotone
+    assert (q == -q[::-1]).all() and (np.diff(q.astype(int)) >= 0).all()
+
+
+def test_quantize_zero_block_and_rejects_ragged(oracle):
+    blk = oracle.quantize_q8_0(np.zeros(64, dtype=np.float32))
+    assert (blk == 0).all()                      # d = +0 and q = 0 (QuantBlocks.h:70)
+    with pytest.raises(ValueError):
+        oracle.quantize_q8_0(np.zeros(33, dtype=np.float32))
+    x = np.zeros(31, dtype=np.float32)
+    out = np.zeros(34, dtype=np.uint8)
+    rc = oracle.lib().orc_quantize_q8_0(x.ctypes.data_as(C.POINTER(C.c_float)), out.ctypes.data_as(C.c_void_p), 31)
+    assert rc == 1
+
+
+def test_quantize_invariants_and_independent_rounding(oracle):
+    rng = np.random.default_rng(1)
+    x = np.concatenate([
+        rng.standard_normal(32 * 2000).astype(np.float32),
+        (rng.standard_normal(32 * 500) * 0.02).astype(np.float32),
+        (rng.standard_normal(32 * 500) * 1e-6).astype(np.float32),
+        (rng.standard_normal(32 * 100) * 1e4).astype(np.float32),
+    ]).reshape(-1, 32)
+    blk = oracle.quantize_q8_0(x)[:, 0, :]
+    q = oracle.block_quants(blk).astype(np.int64)
+    dbits = oracle.block_scales_bits(blk)
+    amax = np.abs(x).max(axis=1)
+    # scale: fp16(RNE) of the binary32 quotient amax/127 -- numpy's own division and half rounding
+    d32 = (amax / np.float32(127.0)).astype(np.float32)
+    assert (dbits == d32.astype(np.float16).view(np.uint16)).all()
+    # the arg-max element maps to +-127, nothing leaves [-127,127]
+    arg = np.abs(x).argmax(axis=1)
+    rows = np.arange(x.shape[0])
+    assert (np.abs(q[rows, arg]) == 127).all()
+    assert (np.sign(q[rows, arg]) == np.sign(x[rows, arg])).all()
+    assert q.min() >= -127 and q.max() <= 127
+    # reconstruction error is at most half a step of the f32 scale
+    err = np.abs(x.astype(np.float64) - d32[:, None].astype(np.float64) * q)
+    assert (err <= 0.5 * d32[:, None].astype(np.float64) * (1 + 1e-5)).all()
+    # independent statement in float64: q = round-half-away(x / d); may differ from the binary32
+    # product x*(1/d) only when the exact quotient sits on a rounding boundary
+    t = x.astype(np.float64) / d32[:, None].astype(np.float64)
+    want = np.sign(t) * np.floor(np.abs(t) + 0.5)
+    want = np.clip(want, -127, 127).astype(np.int64)
+    diff = want != q
+    frac = np.abs(np.abs(t) - np.floor(np.abs(t)) - 0.5)
+    assert (frac[diff] < 2e-5).all() and diff.mean() < 1e-4
+
+
+def test_quantize_ties_round_away_from_zero(oracle):
+    # amax = 127 -> d = 1, inv = 1: the quantizer is round() itself
+    x = np.zeros(32, dtype=np.float32)
+    x[0] = 127.0
+    x[1:9] = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 0.49999997, -0.49999997]
+    q = oracle.block_quants(oracle.quantize_q8_0(x))[0]
+    assert list(q[:9]) == [127, 1, -1, 2, -2, 3, -3, 0, 0]
+
+
+def test_quantize_ignores_nan_in_absmax(oracle):
+    # std::fmax drops NaN (QuantBlocks.h:67): the scale comes from the finite elements
+    x = np.ones(32, dtype=np.float32)
+    x[3] = np.nan
+    x[5] = -2.0
+    blk = oracle.quantize_q8_0(x)
+    assert int(oracle.block_scales_bits(blk)[0]) == int(np.float32(2.0 / 127.0).astype(np.float16).view(np.uint16))
+    assert oracle.block_quants(blk)[0][5] == -127
+
+
+def test_repack_round_trip_and_planes(oracle):
+    rng = np.random.default_rng(2)
+    blk = oracle.quantize_q8_0(rng.standard_normal((6, 96)).astype(np.float32))
+    flat = blk.reshape(-1, 34)
+    nb = flat.shape[0]
+    packed = oracle.repack_q8_0(flat)
+    assert packed.size == nb * 34 == oracle.lib().orc_q8_0_repacked_bytes(nb * 32)
+    assert (packed[: nb * 32].reshape(nb, 32) == flat[:, 2:]).all()
+    assert (packed[nb * 32:].reshape(nb, 2) == flat[:, :2]).all()
+    assert (oracle.unrepack_q8_0(packed) == flat).all()
+
+
+def test_dequantize_closed_form(oracle):
+    rng = np.random.default_rng(3)
+    blk = oracle.quantize_q8_0(rng.standard_normal((4, 64)).astype(np.float32))
+    d = oracle.block_scales_bits(blk).view(np.float16).astype(np.float32)
+    want = (d[..., None] * oracle.block_quants(blk).astype(np.float32)).reshape(4, 64)
+    assert (oracle.dequantize_q8_0(blk) == want).all()
+
+
+# ----------------------------------------------------------------------------- Q8 dot
+def _q8_case(rng, M, N, K):
+    w = (rng.standard_normal((M, K)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    return w, x
+
+
+def test_block_sums_brute_force(oracle):
+    rng = np.random.default_rng(4)
+    w, x = _q8_case(rng, 7, 5, 96)
+    wq, xq = oracle.quantize_q8_0(w), oracle.quantize_q8_0(x)
+    got = oracle.q8_block_sums(wq, xq)
+    want = np.einsum("mbi,nbi->nmb", oracle.block_quants(wq).astype(np.int64), oracle.block_quants(xq).astype(np.int64))
+    assert (got == want).all()
+    # extreme block: |sum| reaches 32*127*127 without overflow
+    hi = np.full((1, 32), 5.0, dtype=np.float32)
+    s = oracle.q8_block_sums(oracle.quantize_q8_0(hi), oracle.quantize_q8_0(-hi))
+    assert int(s[0, 0, 0]) == -32 * 127 * 127
+
+
+@pytest.mark.parametrize("c_trans", [0, 1])
+def test_q8_matmul_closed_form(oracle, c_trans):
+    rng = np.random.default_rng(5)
+    M, N, K = 9, 6, 128
+    w, x = _q8_case(rng, M, N, K)
+    wq, xq = oracle.quantize_q8_0(w), oracle.quantize_q8_0(x)
+    sums = oracle.q8_block_sums(wq, xq).astype(np.float64)                 # [N, M, nblk]
+    dw = oracle.block_scales_bits(wq).view(np.float16).astype(np.float64)    # [M, nblk]
+    da = oracle.block_scales_bits(xq).view(np.float16).astype(np.float64)    # [N, nblk]
+    exact = np.einsum("nmb,mb,nb->nm", sums, dw, da)
+    for fma in (0, 1):
+        got = oracle.mul_mat_q8q8(wq, xq, c_trans=c_trans, fma=fma).astype(np.float64)
+        got = got if c_trans else got.T
+        assert np.abs(got - exact).max() <= 1e-6 * np.abs(exact).max()
+    # special case: equals the f32 GEMM of the dequantised operands up to f32 summation error
+    deq = oracle.mul_mat_f32(oracle.dequantize_q8_0(xq), oracle.dequantize_q8_0(wq)).astype(np.float64)
+    assert np.abs(deq - exact).max() <= 1e-5 * np.abs(exact).max()
+    # and approximates the unquantised product to quantisation accuracy
+    full = x.astype(np.float64) @ w.astype(np.float64).T
+    assert np.abs(full - exact).max() <= 0.02 * np.abs(full).max()
+
+
+def test_q8_matmul_end_to_end_and_layouts(oracle):
+    rng = np.random.default_rng(6)
+    M, N, K = 8, 5, 64
+    w, x = _q8_case(rng, M, N, K)
+    wq = oracle.quantize_q8_0(w)
+    a = oracle.mul_mat_q8(wq, x, wtype=0, c_trans=1)
+    b = oracle.mul_mat_q8(oracle.repack_q8_0(wq), x, wtype=2, c_trans=1)
+    c = oracle.mul_mat_q8(wq, x, wtype=0, c_trans=0)
+    assert (a == b).all() and (a == c.T).all()
+    assert (a == oracle.mul_mat_q8q8(wq, oracle.quantize_q8_0(x))).all()
+    with pytest.raises(RuntimeError):
+        oracle.mul_mat_q8(wq, x, wtype=1)
+    # single-block single-output order check: acc = fma(float(sumi), dw*da, 0)
+    one = oracle.mul_mat_q8q8(wq[:1, :1], oracle.quantize_q8_0(x)[:1, :1])
+    s = int(oracle.q8_block_sums(wq[:1, :1], oracle.quantize_q8_0(x)[:1, :1])[0, 0, 0])
+    dw = oracle.block_scales_bits(wq)[0, 0].view(np.float16).astype(np.float32)
+    da = oracle.block_scales_bits(oracle.quantize_q8_0(x))[0, 0].view(np.float16).astype(np.float32)
+    assert one[0, 0] == np.float32(s) * np.float32(dw * da)
+
+
+# ----------------------------------------------------------------------------- f32 mul_mat
+def test_mul_mat_reference_test_inputs_exact(oracle):
+    # tests/test_cuda.cpp:133-167: every product is a multiple of 1/8 and every partial sum is small,
+    # so binary32 holds all of them exactly and the answer equals integer arithmetic.
+    M, K, N = 17, 9, 23
+    A = ((np.arange(M * K) % 11) * 0.5 - 2.0).astype(np.float32).reshape(M, K)
+    B = ((np.arange(N * K) % 13) * 0.25 + 0.5).astype(np.float32).reshape(N, K)
+    got = oracle.mul_mat_f32(A, B)
+    Ai = np.rint(A.astype(np.float64) * 2).astype(np.int64)
+    Bi = np.rint(B.astype(np.float64) * 4).astype(np.int64)
+    want = (Ai @ Bi.T) / 8.0
+    assert got.shape == (M, N) and (got.astype(np.float64) == want).all()
+    bias = ((np.arange(N) % 5) * 0.125 - 0.25).astype(np.float32)
+    got_b = oracle.mul_mat_f32(A, B, bias)
+    assert (got_b.astype(np.float64) == want + bias.astype(np.float64)[None, :]).all()
+    for nt in (1, 3):
+        assert (oracle.mul_mat_f32(A, B, bias, nthreads=nt) == got_b).all()
+
+
+def test_mul_mat_bias_enters_first_and_k_ascending(oracle):
+    # 1e8 + 1 - 1e8: only "bias first, then k ascending" gives 0; bias last would give 1.
+    a = np.array([[1.0, 1.0]], dtype=np.float32)
+    b = np.array([[1.0, -1e8]], dtype=np.float32)
+    assert oracle.mul_mat_f32(a, b, np.array([1e8], dtype=np.float32))[0, 0] == 0.0
+    # ascending k: (1e8 + 1) - 1e8 = 0, descending would give 1
+    a = np.array([[1e8, 1.0, -1e8]], dtype=np.float32)
+    b = np.ones((1, 3), dtype=np.float32)
+    assert oracle.mul_mat_f32(a, b)[0, 0] == 0.0
+
+
+def test_mul_mat_random_vs_float64(oracle):
+    rng = np.random.default_rng(8)
+    A = rng.standard_normal((33, 70)).astype(np.float32)
+    B = rng.standard_normal((21, 70)).astype(np.float32)
+    want = A.astype(np.float64) @ B.astype(np.float64).T
+    assert np.abs(oracle.mul_mat_f32(A, B) - want).max() < 1e-4
+
+
+# ----------------------------------------------------------------------------- out_prod
+def test_out_prod_reference_small_inputs_exact(oracle):
+    # tests/test_cuda.cpp:207-245
+    C0, C1, K = 4, 5, 3
+    a = ((np.arange(C0 * K) % 7) * 0.5).astype(np.float32).reshape(1, 1, K, C0)
+    b = ((np.arange(C1 * K) % 9) * 0.25 - 1.0).astype(np.float32).reshape(1, 1, K, C1)
+    got = oracle.out_prod(a, b)
+    want = np.einsum("ki,kj->ji", a[0, 0].astype(np.float64), b[0, 0].astype(np.float64))
+    assert got.shape == (1, 1, C1, C0) and (got[0, 0].astype(np.float64) == want).all()
+
+
+def test_out_prod_reference_real_shape_exact(oracle):
+    # tests/test_cuda.cpp:262-341: L=51, K=51, 16x64 planes; inputs are multiples of 1/16 and 1/8,
+    # so the sums are exact in binary32 whatever the order.
+    L, K, P2, P3 = 51, 51, 16, 64
+    nA = L * K * P2 * P3
+    A = ((np.arange(nA) % 13) * 0.0625 - 0.5).astype(np.float32).reshape(P3, P2, K, L)
+    B = ((np.arange(nA) % 7) * 0.125 - 0.25).astype(np.float32).reshape(P3, P2, K, L)
+    got = oracle.out_prod(A, B)
+    for i3, i2 in ((0, 0), (P3 - 1, P2 - 1), (17, 5)):
+        want = np.einsum("ki,kj->ji", A[i3, i2].astype(np.float64), B[i3, i2].astype(np.float64))
+        assert (got[i3, i2].astype(np.float64) == want).all()
+
+
+def test_out_prod_broadcasts_src0_planes(oracle):
+    # CPUKernels.cpp:836-858: i02 = i2 / (ne2/ne02), i03 = i3 / (ne3/ne03)
+    rng = np.random.default_rng(9)
+    s0 = rng.integers(-4, 5, size=(2, 3, 5, 6)).astype(np.float32)      # ne03=2, ne02=3
+    s1 = rng.integers(-4, 5, size=(4, 6, 5, 7)).astype(np.float32)      # ne13=4, ne12=6
+    got = oracle.out_prod(s0, s1)
+    s0b = np.repeat(np.repeat(s0, 2, axis=0), 2, axis=1)
+    want = np.einsum("pqki,pqkj->pqji", s0b.astype(np.float64), s1.astype(np.float64))
+    assert got.shape == (4, 6, 7, 6) and (got.astype(np.float64) == want).all()
+
+
+# ----------------------------------------------------------------------------- outer product mean
+def test_opm_value_known_answers(oracle):
+    # tests/test_outer_product_mean.cpp:10-50
+    left = np.array([1, 2, 3, 4, 5, 6, 7, 8], dtype=np.float32).reshape(1, 2, 2, 2)
+    right = np.array([1, 0, 0, 1, 1, 1, 0, 0], dtype=np.float32).reshape(1, 2, 2, 2)
+    o = oracle.outer_product_mean_value(left, right)
+    assert o.shape == (1, 2, 2, 4)
+    assert list(o[0, 0, 0]) == [3.0, 2.5, 4.0, 3.0]
+    assert o[0, 1, 1, 0] == 0.0 and o[0, 1, 1, 3] == 2.0
+    # tests/test_outer_product_mean.cpp:52-70
+    left = np.array([[n + i for i in range(2)] for n in range(3)], dtype=np.float32).reshape(1, 3, 2, 1)
+    o = oracle.outer_product_mean_value(left, np.ones((1, 3, 2, 1), dtype=np.float32))
+    assert np.allclose(o.ravel(), [1.0, 1.0, 2.0, 2.0], rtol=1e-7)
+
+
+def test_opm_value_vs_einsum(oracle):
+    rng = np.random.default_rng(10)
+    l = rng.integers(-3, 4, size=(2, 4, 3, 5)).astype(np.float32)
+    r = rng.integers(-3, 4, size=(2, 4, 3, 5)).astype(np.float32)
+    want = np.einsum("bnid,bnje->bijde", l.astype(np.float64), r.astype(np.float64)).reshape(2, 3, 3, 25) / 4.0
+    assert (oracle.outer_product_mean_value(l, r).astype(np.float64) == want).all()
+
+
+def test_opm_graph_form_vs_einsum(oracle):
+    # Layout stated at src/backend/CPUKernels.cpp:975-981: left[d,i,n,b] at ((d*L+i)*N+n)*B+b and
+    # dst[(d1*D+d2), i, j, b] at (((d1*D+d2)*L+i)*L+j)*B+b.  D != L != N != B so that any swapped
+    # pair of indices changes the result.
+    rng = np.random.default_rng(11)
+    D, L, N, B = 3, 4, 8, 2
+    l = rng.integers(-3, 4, size=(D, L, N, B)).astype(np.float32)
+    r = rng.integers(-3, 4, size=(D, L, N, B)).astype(np.float32)
+    got = oracle.outer_prod_mean(l, r, D, L, N, B).reshape(D, D, L, L, B)
+    want = np.einsum("dinb,ejnb->deijb", l.astype(np.float64), r.astype(np.float64)) / N
+    assert (got.astype(np.float64) == want).all()
+    # 1/N multiplies the finished sum (CPUKernels.cpp:995,1028): with N=3 sum*inv differs from sum/3
+    D, L, N, B = 1, 1, 3, 1
+    l = np.array([1.0, 1.0, 1.0], dtype=np.float32)
+    got = oracle.outer_prod_mean(l, l, D, L, N, B)
+    assert got[0] == np.float32(3.0) * (np.float32(1.0) / np.float32(3.0))
+
+
+# ----------------------------------------------------------------------------- attention scores
+def test_attention_scores_vs_einsum(oracle):
+    rng = np.random.default_rng(12)
+    NQ, H, D, Lq, Lk = 2, 3, 16, 5, 7
+    q = rng.integers(-3, 4, size=(NQ, H, D, Lq)).astype(np.float32)
+    k = rng.integers(-3, 4, size=(NQ, H, D, Lk)).astype(np.float32)
+    got = oracle.attention_scores(q, k)
+    s = np.einsum("bhdi,bhdj->bhij", q.astype(np.float64), k.astype(np.float64)).astype(np.float32)
+    want = s * (np.float32(1.0) / np.sqrt(np.float32(D)))          # 1/sqrt(16) = 0.25 exactly
+    assert (got == want).all()
+    # equals the graph path: out_prod(K,Q) then a scale node (Attention.cpp:264-270)
+    kk = np.ascontiguousarray(k.reshape(NQ, H, D, Lk))
+    op = oracle.out_prod(kk, q)                                      # [NQ,H,Lq,Lk]
+    assert (op * np.float32(0.25) == got).all()
