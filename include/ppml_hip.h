@@ -1,0 +1,132 @@
+/*
+ * ppml_hip.h -- C ABI of the MI355X (gfx950) matrix-multiplication backend.
+ *
+ * Every entry point is the twin of one of the reference's per-op launcher functions (free
+ * functions in namespace ppml, declared extern in src/backend/CUDAKernels.cpp:158-205 and
+ * 325-326).  Arguments keep the reference's names, order and meaning; two things differ on
+ * purpose: each launcher returns an int status instead of void (the reference's cudaCheck has an
+ * empty body, src/cuda/CUDAKernels.cu:21-24, so its launch errors are dropped), and each takes
+ * a trailing stream (NULL = the default stream, which is what the reference always uses).
+ *
+ * All pointers are DEVICE pointers owned by the caller's buffers; the library neither frees nor
+ * retains them.  Launchers are asynchronous on the given stream; call ppml_hip_synchronize()
+ * (Backend::synchronize, include/ppml/Backend.h:557) before reading results on the host.
+ *
+ * Status codes shared by all entry points:
+ *   0 ok   1 bad arguments   2 K not a multiple of 32   3 allocation failed
+ *   5 unsupported weight type   6 kernel launch failed   7 no usable gfx950 device
+ */
+#ifndef PPML_HIP_H
+#define PPML_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PPML_HIP_ABI_VERSION 1
+
+typedef void *ppml_hip_stream_t; /* a hipStream_t, or NULL */
+
+/* Weight storage handed to mul_mat_q8_hip; 0..2 are the reference's wtype values
+ * (src/backend/CUDAKernels.cpp:769-770), 3 is this library's MFMA-fragment layout. */
+enum {
+    PPML_WTYPE_Q8_0 = 0,  /* interleaved 34-byte block_q8_0  (include/ppml/QuantBlocks.h:33-36) */
+    PPML_WTYPE_Q8_1 = 1,  /* interleaved 36-byte block_q8_1  (include/ppml/QuantBlocks.h:38-41) */
+    PPML_WTYPE_Q8_0R = 2, /* qs plane + d plane              (include/ppml/QuantBlocks.h:113-135) */
+    PPML_WTYPE_Q8_0M = 3  /* MFMA-fragment order, made by q8_weight_pack_hip */
+};
+
+/* ---- library / device --------------------------------------------------------------------- */
+int ppml_hip_abi_version(void);
+/* Selects `device`, checks that it is a gfx950 part; replaces cudaSetDevice in
+ * CUDABackend::graph_compute (src/backend/CUDABackend.cpp:708-712). */
+int ppml_hip_init(int device);
+/* Backend::synchronize (include/ppml/Backend.h:557). */
+int ppml_hip_synchronize(void);
+/* Text of the last failure on the calling thread ("" if none). */
+const char *ppml_hip_last_error(void);
+
+/* ---- f32 GEMM ------------------------------------------------------------------------------ */
+/* replaces mul_mat_cuda (src/cuda/CUDAKernels.cu:1174-1182):
+ * C[m*N+n] = (bias ? bias[n] : 0) + sum_k A[m*K+k] * B[n*K+k].  bias may be NULL. */
+int mul_mat_hip(const float *A, const float *B, float *C, int M, int K, int N,
+                const float *bias, ppml_hip_stream_t stream);
+
+/* ---- Q8_0 ---------------------------------------------------------------------------------- */
+/* Q8_0 twin of quantize_rows_q8_1_cuda (src/cuda/QuantKernels.cu:86-93); the arithmetic is
+ * quantize_q8_0_host (include/ppml/QuantBlocks.h:62-79).  y receives ne/32 block_q8_0 records. */
+int quantize_rows_q8_0_hip(const float *x, void *y, int64_t ne, ppml_hip_stream_t stream);
+/* replaces dequantize_q8_0_cuda (src/cuda/QuantKernels.cu:95-101). */
+int dequantize_q8_0_hip(const void *x, float *y, int64_t ne, ppml_hip_stream_t stream);
+
+/* Once-per-weight repack, the role repack_q8_0_host plays in the reference
+ * (include/ppml/QuantBlocks.h:123-133, called from src/model/PPML.cpp:4504-4528).
+ * Turns an M x K weight of type 0, 1 or 2 into PPML_WTYPE_Q8_0M. */
+size_t q8_weight_packed_bytes_hip(int M, int K);
+int q8_weight_pack_hip(const void *W, int wtype, int M, int K, void *packed,
+                       ppml_hip_stream_t stream);
+
+/* replaces mul_mat_q8_cuda (src/cuda/MulMatQ8Kernel.cu:476-547).
+ * W: M x K quantized weight (rows = out features), X: N x K f32 activations (rows = tokens).
+ * Activations are quantized to Q8_0 per 32-element block inside the kernel, every block is
+ * contracted with int8 MFMA into an exact int32 and settled as
+ *     acc = fma(float(sumi), d_w * d_a, acc)        blocks ascending
+ * (src/cuda/MulMatQ8Kernel.cu:120-142).  c_trans 0 -> C[m*N+n], 1 -> C[n*M+m].
+ * *path_out (may be NULL) is set to 1: there is only the MFMA path. */
+int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
+                   int c_trans, int *path_out, ppml_hip_stream_t stream);
+
+/* The same kernel with its optional inputs and outputs exposed.
+ *   flags bit 0: apply ReLU to X before quantizing (FeedForward: linear1 -> ReLU -> linear2,
+ *                src/modules/Attention.cpp:1097-1104)
+ *   xq_dump  (may be NULL): receives the Q8_0 blocks the kernel made of X, [N][K/32] block_q8_0
+ *   sums_dump(may be NULL): receives the per-block int32 sums, [(n*M+m)*(K/32)+ib]            */
+int mul_mat_q8_ex_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
+                      int c_trans, int flags, void *xq_dump, int32_t *sums_dump,
+                      ppml_hip_stream_t stream);
+
+/* ---- batched / permuted f32 contractions ----------------------------------------------------- */
+/* replaces out_prod_cuda (src/cuda/OutProdKernel.cu:211-260) with the CPU kernel's plane
+ * broadcast (src/backend/CPUKernels.cpp:836-858):
+ * dst[i0,i1,i2,i3] = sum_k src0[i0,k,i2/(ne2/ne02),i3/(ne3/ne03)] * src1[i1,k,i2,i3].
+ * dst is overwritten (the caller does not need to zero it first). */
+int out_prod_hip(const float *src0, const float *src1, float *dst,
+                 int64_t ne00, int64_t ne01, int64_t ne02, int64_t ne03,
+                 int64_t ne10, int64_t ne11, int64_t ne12, int64_t ne13,
+                 int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3,
+                 ppml_hip_stream_t stream);
+/* out_prod followed by the OP_SCALE node of the attention path in one pass
+ * (src/modules/Attention.cpp:264-270): dst = scale * out_prod(src0, src1). */
+int out_prod_scaled_hip(const float *src0, const float *src1, float *dst,
+                        int64_t ne00, int64_t ne01, int64_t ne02, int64_t ne03,
+                        int64_t ne10, int64_t ne11, int64_t ne12, int64_t ne13,
+                        int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3,
+                        float scale, ppml_hip_stream_t stream);
+
+/* replaces outer_prod_mean_cuda (src/cuda/PairKernels.cu:553-561), indexing of
+ * src/backend/CPUKernels.cpp:1006-1028: left/right [D,L,N,B] -> dst [D*D,L,L,B]. */
+int outer_prod_mean_hip(const float *left, const float *right, float *dst,
+                        int64_t D, int64_t L, int64_t N, int64_t B, float inv_N,
+                        ppml_hip_stream_t stream);
+/* value-form outer product mean (src/ops/MathUtils.cpp:387-437):
+ * left/right (B,N,L,D) -> dst (B,L,L,D*D), i.e. dst = A^T B / N per batch. */
+int outer_product_mean_value_hip(const float *left, const float *right, float *dst,
+                                 int64_t B, int64_t N, int64_t L, int64_t D,
+                                 ppml_hip_stream_t stream);
+/* The plain form of the same contraction: O[m*Nc+n] = alpha * sum_k A[k*M+m] * Bm[k*Nc+n]. */
+int mul_mat_tn_hip(const float *A, const float *Bm, float *O, int M, int K, int Nc, float alpha,
+                   ppml_hip_stream_t stream);
+
+/* ---- observability (include/ppml/MulMatStats.h:154-169) -------------------------------------- */
+/* Per-shape call counters keyed like the reference (M<<40 | K<<20 | N); enabled by the
+ * environment variable PPML_MULMAT_STATS=1.  Writes up to `cap` rows of
+ * {M, K, N, calls} (int64 each) and returns the number of distinct shapes. */
+int ppml_hip_mulmat_stats(int64_t *rows, int cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

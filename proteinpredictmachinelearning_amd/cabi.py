@@ -1,0 +1,71 @@
+"""ctypes binding of the gfx950 backend library (``lib/libppml_hip.so``).
+
+The signatures below are the ones ``include/ppml_hip.h`` declares.  There is no fallback: if the
+library is missing, or it was built for another GPU, loading fails loudly.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libppml_hip.so")
+
+_i, _i64, _f, _vp = C.c_int, C.c_int64, C.c_float, C.c_void_p
+
+# name -> (restype, argtypes); every symbol include/ppml_hip.h declares
+SIGNATURES = {
+    "ppml_hip_abi_version": (_i, []),
+    "ppml_hip_init": (_i, [_i]),
+    "ppml_hip_synchronize": (_i, []),
+    "ppml_hip_last_error": (C.c_char_p, []),
+    "mul_mat_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
+    "quantize_rows_q8_0_hip": (_i, [_vp, _vp, _i64, _vp]),
+    "dequantize_q8_0_hip": (_i, [_vp, _vp, _i64, _vp]),
+    "q8_weight_packed_bytes_hip": (C.c_size_t, [_i, _i]),
+    "q8_weight_pack_hip": (_i, [_vp, _i, _i, _i, _vp, _vp]),
+    "mul_mat_q8_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, C.POINTER(_i), _vp]),
+    "mul_mat_q8_ex_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "out_prod_hip": (_i, [_vp, _vp, _vp] + [_i64] * 12 + [_vp]),
+    "out_prod_scaled_hip": (_i, [_vp, _vp, _vp] + [_i64] * 12 + [_f, _vp]),
+    "outer_prod_mean_hip": (_i, [_vp, _vp, _vp] + [_i64] * 4 + [_f, _vp]),
+    "outer_product_mean_value_hip": (_i, [_vp, _vp, _vp] + [_i64] * 4 + [_vp]),
+    "mul_mat_tn_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _f, _vp]),
+    "ppml_hip_mulmat_stats": (_i, [C.POINTER(_i64), _i]),
+}
+
+_lib = None
+
+
+class BackendError(RuntimeError):
+    """A launcher returned a non-zero status."""
+
+    def __init__(self, name: str, rc: int, text: str):
+        super().__init__(f"{name} failed with status {rc}: {text}")
+        self.rc = rc
+
+
+def load() -> C.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `make -C proteinpredictmachinelearning_amd/csrc` "
+            "(or __graft_entry__.build()); this backend has no CPU fallback")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the library lacks a declared symbol
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().ppml_hip_last_error().decode()
+
+
+def check(name: str, rc: int) -> None:
+    if rc != 0:
+        raise BackendError(name, rc, last_error())

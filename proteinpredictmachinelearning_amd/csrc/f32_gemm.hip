@@ -1,0 +1,327 @@
+// True-fp32 MFMA contractions for gfx950: dense GEMM with bias (mul_mat), batched transposed
+// GEMM with plane broadcast (out_prod, attention logits) and outer-product-mean in both of the
+// reference's layouts.  One kernel, three operand-access modes.
+//
+// Reference behaviour restated here (paths relative to the reference tree):
+//   mul_mat          src/backend/CPUKernels.cpp:763-771   (bias first, k ascending)
+//   out_prod         src/backend/CPUKernels.cpp:787-887
+//   outer_prod_mean  src/backend/CPUKernels.cpp:982-1032, src/ops/MathUtils.cpp:387-437
+//
+// Reduction order: every output is accumulated in fp32 by v_mfma_f32_32x32x2_f32, k ascending in
+// steps of 2 (the instruction adds a[k]*b[k] + a[k+1]*b[k+1] to the accumulator), starting from
+// bias[n] (or 0); alpha multiplies the finished sum.
+#include "common.hpp"
+
+namespace ppmlhip {
+namespace {
+
+constexpr int BM = 128, BN = 128, BK = 16;
+constexpr int LDS_LD = BM + 4;        // row pitch of the k-major LDS tiles (floats)
+
+enum LoadMode { LOAD_K_CONTIG = 0, LOAD_ROW_CONTIG = 1, LOAD_STRIDED = 2 };
+
+struct GemmParams {
+    const float* A;       // rows m: A(m,k) = A[m*a_rs + k*a_ks]
+    const float* B;       // cols n: B(n,k) = B[n*b_rs + k*b_ks]
+    float* C;
+    const float* bias;    // [N] or null
+    int M, N, K;
+    int64_t a_rs, a_ks, b_rs, b_ks;
+    // planes: p = p3*np2 + p2
+    int np2, np3;
+    int64_t a_p2, a_p3, b_p2, b_p3, c_p2, c_p3;
+    int b_div2, b_div3;   // B-side plane index = p / div (out_prod's src0 broadcast)
+    float alpha;
+    // C(m,n) = C[(m/c_lm)*c_mo + (m%c_lm)*c_mi + (n/c_ln)*c_no + (n%c_ln)*c_ni]
+    int c_lm, c_ln;
+    int64_t c_mo, c_mi, c_no, c_ni;
+    int tiles_m, tiles_n;
+};
+
+// 16 x 128 tile of one operand -> two v4f per thread
+template <int MODE>
+__device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_t rs, int64_t ks,
+                                          int row0, int nrows, int k0, int K, int tid, v4f (&reg)[2]) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if (MODE == LOAD_K_CONTIG) {
+            const int r = (tid >> 2) + it * 64;          // row within tile
+            const int k = k0 + (tid & 3) * 4;
+            const int row = row0 + r;
+            if (row < nrows) {
+                const float* p = base + static_cast<int64_t>(row) * rs + k;
+                if (k + 3 < K) v = *reinterpret_cast<const v4f_u*>(p);
+                else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) if (k + c < K) v[c] = p[c];
+                }
+            }
+        } else if (MODE == LOAD_ROW_CONTIG) {
+            const int kk = (tid >> 5) + it * 8;
+            const int r = (tid & 31) * 4;
+            const int k = k0 + kk, row = row0 + r;
+            if (k < K) {
+                const float* p = base + static_cast<int64_t>(k) * ks + row;
+                if (row + 3 < nrows) v = *reinterpret_cast<const v4f_u*>(p);
+                else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) if (row + c < nrows) v[c] = p[c];
+                }
+            }
+        } else {
+            const int r = (tid >> 2) + it * 64;
+            const int k = k0 + (tid & 3) * 4;
+            const int row = row0 + r;
+            if (row < nrows) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    if (k + c < K) v[c] = base[static_cast<int64_t>(row) * rs + static_cast<int64_t>(k + c) * ks];
+            }
+        }
+        reg[it] = v;
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ void store_tile(float* __restrict__ lds, int tid, const v4f (&reg)[2]) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        if (MODE == LOAD_ROW_CONTIG) {
+            const int kk = (tid >> 5) + it * 8;
+            const int r = (tid & 31) * 4;
+            *reinterpret_cast<v4f*>(lds + kk * LDS_LD + r) = reg[it];
+        } else {
+            const int r = (tid >> 2) + it * 64;
+            const int kk = (tid & 3) * 4;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) lds[(kk + c) * LDS_LD + r] = reg[it][c];
+        }
+    }
+}
+
+template <int MODE, bool SPLIT_C>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) float lds_a[BK * LDS_LD];
+    __shared__ __attribute__((aligned(16))) float lds_b[BK * LDS_LD];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 31, hh = lane >> 5;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+
+    // work-group -> (plane, tile row, tile col); bands of 8 tile rows keep operand panels in one L2
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int total = tiles * p.np2 * p.np3;
+    const int idx = xcd_contiguous_index(blockIdx.x, total);
+    const int plane = idx / tiles;
+    int t = idx - plane * tiles;
+    const int band_rows = 8;
+    const int band = t / (band_rows * p.tiles_n);
+    t -= band * band_rows * p.tiles_n;
+    const int rows_here = (p.tiles_m - band * band_rows) < band_rows ? (p.tiles_m - band * band_rows) : band_rows;
+    const int tm = band * band_rows + t % rows_here;
+    const int tn = t / rows_here;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int p2 = plane % p.np2, p3 = plane / p.np2;
+    const float* A = p.A + p2 * p.a_p2 + p3 * p.a_p3;
+    const float* B = p.B + (p2 / p.b_div2) * p.b_p2 + (p3 / p.b_div3) * p.b_p3;
+    float* C = p.C + p2 * p.c_p2 + p3 * p.c_p3;
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+        const int n = n0 + wn + tj * 32 + j;
+        const float b0 = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+#pragma unroll
+        for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = b0;
+    }
+
+    v4f ra[2], rb[2];
+    load_tile<MODE>(A, p.a_rs, p.a_ks, m0, p.M, 0, p.K, tid, ra);
+    load_tile<MODE>(B, p.b_rs, p.b_ks, n0, p.N, 0, p.K, tid, rb);
+
+    for (int k0 = 0; k0 < p.K; k0 += BK) {
+        store_tile<MODE>(lds_a, tid, ra);
+        store_tile<MODE>(lds_b, tid, rb);
+        __syncthreads();
+        if (k0 + BK < p.K) {
+            load_tile<MODE>(A, p.a_rs, p.a_ks, m0, p.M, k0 + BK, p.K, tid, ra);
+            load_tile<MODE>(B, p.b_rs, p.b_ks, n0, p.N, k0 + BK, p.K, tid, rb);
+        }
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 2) {
+            const float a0 = lds_a[(kk + hh) * LDS_LD + wm + j];
+            const float a1 = lds_a[(kk + hh) * LDS_LD + wm + 32 + j];
+            const float b0 = lds_b[(kk + hh) * LDS_LD + wn + j];
+            const float b1 = lds_b[(kk + hh) * LDS_LD + wn + 32 + j];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    const bool scale = p.alpha != 1.0f;
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj) {
+            const int n = n0 + wn + tj * 32 + j;
+            if (n >= p.N) continue;
+            int64_t coff;
+            if (SPLIT_C) coff = static_cast<int64_t>(n / p.c_ln) * p.c_no + static_cast<int64_t>(n % p.c_ln) * p.c_ni;
+            else         coff = static_cast<int64_t>(n) * p.c_ni;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm + ti * 32 + mfma32_row(r, lane);
+                if (m >= p.M) continue;
+                int64_t roff;
+                if (SPLIT_C) roff = static_cast<int64_t>(m / p.c_lm) * p.c_mo + static_cast<int64_t>(m % p.c_lm) * p.c_mi;
+                else         roff = static_cast<int64_t>(m) * p.c_mi;
+                float v = acc[ti][tj][r];
+                if (scale) v *= p.alpha;
+                C[roff + coff] = v;
+            }
+        }
+}
+
+int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
+    p.tiles_m = (p.M + BM - 1) / BM;
+    p.tiles_n = (p.N + BN - 1) / BN;
+    const int64_t total = static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.np2 * p.np3;
+    if (total <= 0 || total > 0x7fffffffLL) { set_error("%s: grid of %lld work-groups is out of range", what, (long long)total); return RC_BAD_ARGS; }
+    const dim3 grid(static_cast<unsigned>(total)), block(256);
+    const bool split = !(p.c_lm >= p.M && p.c_ln >= p.N);
+    int mode = LOAD_STRIDED;
+    if (p.a_ks == 1 && p.b_ks == 1) mode = LOAD_K_CONTIG;
+    else if (p.a_rs == 1 && p.b_rs == 1) mode = LOAD_ROW_CONTIG;
+#define PPML_LAUNCH(MODE, SPLIT) hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT>), grid, block, 0, stream, p)
+    if (mode == LOAD_K_CONTIG)        { if (split) PPML_LAUNCH(LOAD_K_CONTIG, true);   else PPML_LAUNCH(LOAD_K_CONTIG, false); }
+    else if (mode == LOAD_ROW_CONTIG) { if (split) PPML_LAUNCH(LOAD_ROW_CONTIG, true); else PPML_LAUNCH(LOAD_ROW_CONTIG, false); }
+    else                              { if (split) PPML_LAUNCH(LOAD_STRIDED, true);    else PPML_LAUNCH(LOAD_STRIDED, false); }
+#undef PPML_LAUNCH
+    return check_launch(what);
+}
+
+GemmParams plain_params() {
+    GemmParams p{};
+    p.np2 = p.np3 = 1;
+    p.b_div2 = p.b_div3 = 1;
+    p.alpha = 1.0f;
+    p.c_lm = p.c_ln = 0x7fffffff;
+    return p;
+}
+
+}  // namespace
+}  // namespace ppmlhip
+
+using namespace ppmlhip;
+
+extern "C" int mul_mat_hip(const float* A, const float* B, float* C, int M, int K, int N,
+                           const float* bias, ppml_hip_stream_t stream) {
+    if (!A || !B || !C || M <= 0 || K <= 0 || N <= 0) { set_error("mul_mat_hip: bad arguments (M=%d K=%d N=%d)", M, K, N); return RC_BAD_ARGS; }
+    stats_record(M, K, N);
+    GemmParams p = plain_params();
+    p.A = A; p.B = B; p.C = C; p.bias = bias;
+    p.M = M; p.N = N; p.K = K;
+    p.a_rs = K; p.a_ks = 1; p.b_rs = K; p.b_ks = 1;
+    p.c_mi = N; p.c_ni = 1;
+    return launch_gemm(p, static_cast<hipStream_t>(stream), "mul_mat_hip");
+}
+
+extern "C" int mul_mat_tn_hip(const float* A, const float* Bm, float* O, int M, int K, int Nc, float alpha,
+                              ppml_hip_stream_t stream) {
+    if (!A || !Bm || !O || M <= 0 || K <= 0 || Nc <= 0) { set_error("mul_mat_tn_hip: bad arguments"); return RC_BAD_ARGS; }
+    stats_record(M, K, Nc);
+    GemmParams p = plain_params();
+    p.A = A; p.B = Bm; p.C = O;
+    p.M = M; p.N = Nc; p.K = K;
+    p.a_rs = 1; p.a_ks = M; p.b_rs = 1; p.b_ks = Nc;
+    p.c_mi = Nc; p.c_ni = 1;
+    p.alpha = alpha;
+    return launch_gemm(p, static_cast<hipStream_t>(stream), "mul_mat_tn_hip");
+}
+
+extern "C" int out_prod_scaled_hip(const float* src0, const float* src1, float* dst,
+                                   int64_t ne00, int64_t ne01, int64_t ne02, int64_t ne03,
+                                   int64_t ne10, int64_t ne11, int64_t ne12, int64_t ne13,
+                                   int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3,
+                                   float scale, ppml_hip_stream_t stream) {
+    if (!src0 || !src1 || !dst) { set_error("out_prod_hip: null pointer"); return RC_BAD_ARGS; }
+    const bool pos = ne00 > 0 && ne01 > 0 && ne02 > 0 && ne03 > 0 && ne10 > 0 && ne11 > 0 && ne12 > 0 && ne13 > 0;
+    // shape contract of the graph builder (src/core/ComputeGraphHelper.cpp:318-345) and the
+    // broadcast rule of the CPU kernel (src/backend/CPUKernels.cpp:836-837)
+    if (!pos || ne01 != ne11 || ne0 != ne00 || ne1 != ne10 || ne2 != ne12 || ne3 != ne13 ||
+        ne2 % ne02 != 0 || ne3 % ne03 != 0 || ne0 > 0x7fffffff || ne1 > 0x7fffffff || ne01 > 0x7fffffff) {
+        set_error("out_prod_hip: shape mismatch src0[%lld,%lld,%lld,%lld] src1[%lld,%lld,%lld,%lld] dst[%lld,%lld,%lld,%lld]",
+                  (long long)ne00, (long long)ne01, (long long)ne02, (long long)ne03,
+                  (long long)ne10, (long long)ne11, (long long)ne12, (long long)ne13,
+                  (long long)ne0, (long long)ne1, (long long)ne2, (long long)ne3);
+        return RC_BAD_ARGS;
+    }
+    stats_record(ne1, ne01, ne0);
+    GemmParams p = plain_params();
+    p.A = src1; p.B = src0; p.C = dst;                 // rows = i1 (src1), cols = i0 (src0)
+    p.M = static_cast<int>(ne1); p.N = static_cast<int>(ne0); p.K = static_cast<int>(ne01);
+    p.a_rs = 1; p.a_ks = ne10; p.b_rs = 1; p.b_ks = ne00;
+    p.np2 = static_cast<int>(ne2); p.np3 = static_cast<int>(ne3);
+    p.a_p2 = ne10 * ne11; p.a_p3 = ne10 * ne11 * ne12;
+    p.b_p2 = ne00 * ne01; p.b_p3 = ne00 * ne01 * ne02;
+    p.c_p2 = ne0 * ne1;   p.c_p3 = ne0 * ne1 * ne2;
+    p.b_div2 = static_cast<int>(ne2 / ne02); p.b_div3 = static_cast<int>(ne3 / ne03);
+    p.c_mi = ne0; p.c_ni = 1;
+    p.alpha = scale;
+    return launch_gemm(p, static_cast<hipStream_t>(stream), "out_prod_hip");
+}
+
+extern "C" int out_prod_hip(const float* src0, const float* src1, float* dst,
+                            int64_t ne00, int64_t ne01, int64_t ne02, int64_t ne03,
+                            int64_t ne10, int64_t ne11, int64_t ne12, int64_t ne13,
+                            int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3,
+                            ppml_hip_stream_t stream) {
+    return out_prod_scaled_hip(src0, src1, dst, ne00, ne01, ne02, ne03, ne10, ne11, ne12, ne13,
+                               ne0, ne1, ne2, ne3, 1.0f, stream);
+}
+
+extern "C" int outer_prod_mean_hip(const float* left, const float* right, float* dst,
+                                   int64_t D, int64_t L, int64_t N, int64_t B, float inv_N,
+                                   ppml_hip_stream_t stream) {
+    if (!left || !right || !dst || D <= 0 || L <= 0 || N <= 0 || B <= 0 || D * L > 0x7fffffff || N > 0x7fffffff) {
+        set_error("outer_prod_mean_hip: bad arguments"); return RC_BAD_ARGS;
+    }
+    stats_record(D * L, N, D * L);
+    GemmParams p = plain_params();
+    p.A = left; p.B = right; p.C = dst;               // rows = (d1,i), cols = (d2,j), k = n
+    p.M = p.N = static_cast<int>(D * L); p.K = static_cast<int>(N);
+    p.a_rs = N * B; p.a_ks = B; p.b_rs = N * B; p.b_ks = B;
+    p.np2 = static_cast<int>(B);                       // batch b is the innermost index of every tensor
+    p.a_p2 = 1; p.b_p2 = 1; p.c_p2 = 1;
+    p.alpha = inv_N;
+    p.c_lm = p.c_ln = static_cast<int>(L);
+    p.c_mo = D * L * L * B; p.c_mi = L * B; p.c_no = L * L * B; p.c_ni = B;
+    return launch_gemm(p, static_cast<hipStream_t>(stream), "outer_prod_mean_hip");
+}
+
+extern "C" int outer_product_mean_value_hip(const float* left, const float* right, float* dst,
+                                            int64_t B, int64_t N, int64_t L, int64_t D,
+                                            ppml_hip_stream_t stream) {
+    if (!left || !right || !dst || D <= 0 || L <= 0 || N <= 0 || B <= 0 || D * L > 0x7fffffff || N > 0x7fffffff) {
+        set_error("outer_product_mean_value_hip: bad arguments"); return RC_BAD_ARGS;
+    }
+    stats_record(D * L, N, D * L);
+    GemmParams p = plain_params();
+    p.A = left; p.B = right; p.C = dst;               // rows = (i,d1), cols = (j,d2), k = n
+    p.M = p.N = static_cast<int>(L * D); p.K = static_cast<int>(N);
+    p.a_rs = 1; p.a_ks = L * D; p.b_rs = 1; p.b_ks = L * D;
+    p.np2 = static_cast<int>(B);
+    p.a_p2 = N * L * D; p.b_p2 = N * L * D; p.c_p2 = L * L * D * D;
+    p.alpha = 1.0f / static_cast<float>(N);
+    p.c_lm = p.c_ln = static_cast<int>(D);
+    p.c_mo = L * D * D; p.c_mi = D; p.c_no = D * D; p.c_ni = 1;
+    return launch_gemm(p, static_cast<hipStream_t>(stream), "outer_product_mean_value_hip");
+}

@@ -1,0 +1,216 @@
+"""Host-side operators of the gfx950 mul_mat backend on top of the C ABI.
+
+Function names, argument order, shape contracts and error behaviour follow the reference's graph-op
+builders (src/core/ComputeGraphHelper.cpp:262-345, 1748-1764) and its dispatch wrapper
+(src/backend/CUDAKernels.cpp:717-847).  torch is used for device memory and streams only; all
+arithmetic happens in the HIP library.  Shapes are written numpy style (outermost first), i.e. the
+reverse of the reference's ``dims[0]``-innermost notation.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import torch
+
+from . import cabi
+
+QK = 32
+BLOCK_BYTES = 34
+WTYPE_Q8_0, WTYPE_Q8_1, WTYPE_Q8_0R, WTYPE_Q8_0M = 0, 1, 2, 3
+
+_initialised = set()
+
+
+def _lib():
+    lib = cabi.load()
+    if not torch.cuda.is_available():
+        raise RuntimeError("the gfx950 backend needs a GPU; there is no CPU path")
+    dev = torch.cuda.current_device()
+    if dev not in _initialised:
+        cabi.check("ppml_hip_init", lib.ppml_hip_init(dev))
+        _initialised.add(dev)
+    return lib
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev_f32(t: torch.Tensor, name: str) -> torch.Tensor:
+    if not t.is_cuda or t.dtype != torch.float32:
+        raise TypeError(f"{name} must be a float32 device tensor")
+    return t.contiguous()
+
+
+def _ptr(t) -> C.c_void_p:
+    return C.c_void_p(0 if t is None else t.data_ptr())
+
+
+def synchronize() -> None:
+    cabi.check("ppml_hip_synchronize", _lib().ppml_hip_synchronize())
+
+
+# ----------------------------------------------------------------------------- f32
+def mul_mat(a: torch.Tensor, b: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """a [M,K], b [N,K] -> [M,N] = a @ b.T (+ bias[N]); src/core/ComputeGraphHelper.cpp:262-314."""
+    a, b = _dev_f32(a, "a"), _dev_f32(b, "b")
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise ValueError(f"mul_mat: inner dimensions differ, a {tuple(a.shape)} b {tuple(b.shape)}")
+    M, K = a.shape
+    N = b.shape[0]
+    if bias is not None:
+        bias = _dev_f32(bias, "bias")
+        if bias.numel() != N:          # the reference drops a bias of the wrong length with a message
+            raise ValueError(f"mul_mat: bias has {bias.numel()} elements, expected {N}")
+    out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+    lib = _lib()
+    cabi.check("mul_mat_hip", lib.mul_mat_hip(_ptr(a), _ptr(b), _ptr(out), M, K, N, _ptr(bias), _stream()))
+    return out
+
+
+def mul_mat_tn(a: torch.Tensor, b: torch.Tensor, alpha: float = 1.0) -> torch.Tensor:
+    """a [K,M], b [K,N] -> alpha * a.T @ b (the dense form of outer-product-mean)."""
+    a, b = _dev_f32(a, "a"), _dev_f32(b, "b")
+    if a.dim() != 2 or b.dim() != 2 or a.shape[0] != b.shape[0]:
+        raise ValueError("mul_mat_tn: contraction lengths differ")
+    K, M = a.shape
+    N = b.shape[1]
+    out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+    cabi.check("mul_mat_tn_hip", _lib().mul_mat_tn_hip(_ptr(a), _ptr(b), _ptr(out), M, K, N, alpha, _stream()))
+    return out
+
+
+def out_prod(a: torch.Tensor, b: torch.Tensor, scale: float | None = None) -> torch.Tensor:
+    """a [ne03,ne02,K,ne00], b [ne13,ne12,K,ne10] -> [ne13,ne12,ne10,ne00];
+    src/core/ComputeGraphHelper.cpp:318-345, broadcast of src/backend/CPUKernels.cpp:836-858.
+    ``scale`` fuses the OP_SCALE node that follows in the attention path."""
+    a, b = _dev_f32(a, "a"), _dev_f32(b, "b")
+    while a.dim() < 4:
+        a = a.unsqueeze(0)
+    while b.dim() < 4:
+        b = b.unsqueeze(0)
+    ne03, ne02, ne01, ne00 = a.shape
+    ne13, ne12, ne11, ne10 = b.shape
+    if ne01 != ne11:
+        raise ValueError(f"out_prod: contraction dims differ ({ne01} vs {ne11})")
+    ne0, ne1, ne2, ne3 = ne00, ne10, max(ne02, ne12), max(ne03, ne13)
+    out = torch.empty((ne3, ne2, ne1, ne0), dtype=torch.float32, device=a.device)
+    dims = [ne00, ne01, ne02, ne03, ne10, ne11, ne12, ne13, ne0, ne1, ne2, ne3]
+    lib = _lib()
+    if scale is None:
+        rc = lib.out_prod_hip(_ptr(a), _ptr(b), _ptr(out), *dims, _stream())
+    else:
+        rc = lib.out_prod_scaled_hip(_ptr(a), _ptr(b), _ptr(out), *dims, scale, _stream())
+    cabi.check("out_prod_hip", rc)
+    return out
+
+
+def attention_logits(k: torch.Tensor, q: torch.Tensor, head_dim: int | None = None) -> torch.Tensor:
+    """out_prod(K, Q) * 1/sqrt(head_dim), steps 1-2 of src/modules/Attention.cpp:264-270."""
+    d = k.shape[-2] if head_dim is None else head_dim
+    return out_prod(k, q, scale=1.0 / math.sqrt(float(d)))
+
+
+def outer_product_mean(left: torch.Tensor, right: torch.Tensor, D: int, L: int, N: int, B: int) -> torch.Tensor:
+    """Graph form (src/core/ComputeGraphHelper.cpp:1748-1764): flat buffers indexed as
+    src/backend/CPUKernels.cpp:1006-1028; returns the flat [D*D*L*L*B] result."""
+    left, right = _dev_f32(left, "left").reshape(-1), _dev_f32(right, "right").reshape(-1)
+    if left.numel() != D * L * N * B or right.numel() != D * L * N * B:
+        raise ValueError("outer_product_mean: operand size does not match D*L*N*B")
+    out = torch.empty(D * D * L * L * B, dtype=torch.float32, device=left.device)
+    cabi.check("outer_prod_mean_hip",
+               _lib().outer_prod_mean_hip(_ptr(left), _ptr(right), _ptr(out), D, L, N, B, 1.0 / float(N), _stream()))
+    return out
+
+
+def outer_product_mean_value(left: torch.Tensor, right: torch.Tensor) -> torch.Tensor:
+    """Value form (src/ops/MathUtils.cpp:387-437): (B,N,L,D) x (B,N,L,D) -> (B,L,L,D*D)."""
+    left, right = _dev_f32(left, "left"), _dev_f32(right, "right")
+    if left.dim() != 4 or right.dim() != 4:
+        raise ValueError("outer_product_mean expects 4D tensors")
+    if left.shape[0] != right.shape[0] or left.shape[2] != right.shape[2] or left.shape[3] != right.shape[3] \
+            or left.shape[1] != right.shape[1]:
+        raise ValueError("outer_product_mean dimension mismatch: batch/residue/feature dims differ")
+    B, N, L, D = left.shape
+    out = torch.empty((B, L, L, D * D), dtype=torch.float32, device=left.device)
+    cabi.check("outer_product_mean_value_hip",
+               _lib().outer_product_mean_value_hip(_ptr(left), _ptr(right), _ptr(out), B, N, L, D, _stream()))
+    return out
+
+
+# ----------------------------------------------------------------------------- Q8_0
+def quantize_rows_q8_0(x: torch.Tensor) -> torch.Tensor:
+    """f32 [..., K] -> uint8 [..., K/32, 34] block_q8_0 records (include/ppml/QuantBlocks.h:62-79)."""
+    x = _dev_f32(x, "x")
+    ne = x.numel()
+    if x.shape[-1] % QK:
+        raise ValueError("quantize_rows_q8_0: innermost dimension is not a multiple of 32")
+    out = torch.empty(x.shape[:-1] + (x.shape[-1] // QK, BLOCK_BYTES), dtype=torch.uint8, device=x.device)
+    cabi.check("quantize_rows_q8_0_hip", _lib().quantize_rows_q8_0_hip(_ptr(x), _ptr(out), ne, _stream()))
+    return out
+
+
+def dequantize_q8_0(blocks: torch.Tensor) -> torch.Tensor:
+    if not blocks.is_cuda or blocks.dtype != torch.uint8 or blocks.shape[-1] != BLOCK_BYTES:
+        raise TypeError("dequantize_q8_0 expects uint8 [..., nblocks, 34] on the device")
+    blocks = blocks.contiguous()
+    nb = blocks.numel() // BLOCK_BYTES
+    out = torch.empty(blocks.shape[:-2] + (blocks.shape[-2] * QK,), dtype=torch.float32, device=blocks.device)
+    cabi.check("dequantize_q8_0_hip", _lib().dequantize_q8_0_hip(_ptr(blocks), _ptr(out), nb * QK, _stream()))
+    return out
+
+
+class Q8Weight:
+    """A quantized M x K weight resident on the device (rows = out features).
+
+    ``data`` holds the bytes in layout ``wtype``; ``pack()`` returns the MFMA-fragment copy made
+    once per weight, the step the reference does with its Q8_0R repack
+    (src/model/PPML.cpp:4504-4528)."""
+
+    def __init__(self, data: torch.Tensor, M: int, K: int, wtype: int):
+        if K % QK:
+            raise ValueError("quantized weights need K % 32 == 0 (blocks never cross a row)")
+        self.data, self.M, self.K, self.wtype = data.contiguous(), M, K, wtype
+
+    @classmethod
+    def from_f32(cls, w: torch.Tensor) -> "Q8Weight":
+        w = _dev_f32(w, "w")
+        M, K = w.shape
+        return cls(quantize_rows_q8_0(w).reshape(-1), M, K, WTYPE_Q8_0)
+
+    def pack(self) -> "Q8Weight":
+        if self.wtype == WTYPE_Q8_0M:
+            return self
+        lib = _lib()
+        nbytes = lib.q8_weight_packed_bytes_hip(self.M, self.K)
+        out = torch.empty(nbytes, dtype=torch.uint8, device=self.data.device)
+        cabi.check("q8_weight_pack_hip",
+                   lib.q8_weight_pack_hip(_ptr(self.data), self.wtype, self.M, self.K, _ptr(out), _stream()))
+        return Q8Weight(out, self.M, self.K, WTYPE_Q8_0M)
+
+
+def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = False,
+               dump: bool = False):
+    """Q8_0 linear: x f32 [N,K] (rows = tokens) times quantized w [M,K] -> [N,M] (c_trans=1, the
+    LinearLayer orientation) or [M,N] (c_trans=0); src/backend/CUDAKernels.cpp:740-789.
+    With ``dump`` also returns the kernel's own Q8_0 blocks of x and its per-block int32 sums."""
+    x = _dev_f32(x, "x")
+    if x.dim() != 2 or x.shape[1] != w.K:
+        raise ValueError(f"mul_mat_q8: activations {tuple(x.shape)} do not match weight K={w.K}")
+    N, K = x.shape
+    M = w.M
+    out = torch.empty((N, M) if c_trans else (M, N), dtype=torch.float32, device=x.device)
+    lib = _lib()
+    if not dump and not relu:
+        path = C.c_int(0)
+        cabi.check("mul_mat_q8_hip", lib.mul_mat_q8_hip(_ptr(w.data), _ptr(x), _ptr(out), M, N, K, w.wtype,
+                                                         c_trans, C.byref(path), _stream()))
+        return out
+    xq = sums = None
+    if dump:
+        xq = torch.empty((N, K // QK, BLOCK_BYTES), dtype=torch.uint8, device=x.device)
+        sums = torch.empty((N, M, K // QK), dtype=torch.int32, device=x.device)
+    cabi.check("mul_mat_q8_ex_hip", lib.mul_mat_q8_ex_hip(_ptr(w.data), _ptr(x), _ptr(out), M, N, K, w.wtype,
+                                                           c_trans, 1 if relu else 0, _ptr(xq), _ptr(sums), _stream()))
+    return (out, xq, sums) if dump else out

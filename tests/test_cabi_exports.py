@@ -1,0 +1,44 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/ppml_hip.h declares."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ppml_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"^\s*(?:const\s+)?(?:int|size_t|char\s*\*)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+    return sorted(set(names))
+
+
+def test_header_symbols_are_exported_and_bound():
+    from proteinpredictmachinelearning_amd import cabi
+
+    names = _declared_symbols()
+    assert len(names) >= 15, names
+    lib = cabi.load()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/ppml_hip.h but not exported"
+    assert set(names) == set(cabi.SIGNATURES), set(names) ^ set(cabi.SIGNATURES)
+    assert lib.ppml_hip_abi_version() == 1
+
+
+def test_host_side_argument_checks_need_no_gpu():
+    from proteinpredictmachinelearning_amd import cabi
+
+    lib = cabi.load()
+    # null pointers / bad sizes are rejected before any device work (mul_mat_q8_cuda rc table,
+    # src/cuda/MulMatQ8Kernel.cu:479-481)
+    assert lib.mul_mat_q8_hip(None, None, None, 4, 4, 32, 0, 1, None, None) == 1
+    assert b"bad arguments" in lib.ppml_hip_last_error()
+    one = ctypes.c_void_p(16)
+    assert lib.mul_mat_q8_hip(one, one, one, 4, 4, 33, 0, 1, None, None) == 2
+    assert lib.mul_mat_q8_hip(one, one, one, 4, 4, 32, 9, 1, None, None) == 5
+    assert lib.quantize_rows_q8_0_hip(one, one, 33, None) == 1
+    assert lib.q8_weight_packed_bytes_hip(768, 256) == 24 * 8 * (1024 + 64)
+    assert lib.q8_weight_packed_bytes_hip(768, 250) == 0
+    assert lib.mul_mat_hip(None, one, one, 1, 1, 1, None, None) == 1
+    dims = [4, 3, 1, 1, 5, 2, 1, 1, 4, 5, 1, 1]        # contraction lengths differ
+    assert lib.out_prod_hip(one, one, one, *dims, None) == 1

@@ -1,0 +1,216 @@
+"""GPU parity of the Q8_0 path against the CPU oracle, through the C ABI.
+
+Bar: quantized bytes, fp16 scales and per-block int32 sums bit-exact; final f32 outputs within 1e-5
+relative (measured against the largest magnitude of the row's settled terms, see ``_rel_err``).  The
+kernel settles blocks in the oracle's order with the same fma, so the tests also report -- and at
+these sizes require -- exact equality of the outputs.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "GPU tests need a device"
+    from proteinpredictmachinelearning_amd import ops as _ops
+
+    return _ops
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _rel_err(got, want):
+    """max |got - want| / max |want|: the 1e-5 relative bar of the Q8 path."""
+    return float(np.abs(got.astype(np.float64) - want.astype(np.float64)).max() / np.abs(want).max())
+
+
+def _inputs(seed, N, K, M, wscale=0.02):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    w = (rng.standard_normal((M, K)) * wscale).astype(np.float32)
+    return x, w
+
+
+def _q8_1_from_q8_0(blocks):
+    """block_q8_1 records {half d; half s=d*sum(q); int8 qs[32]} from block_q8_0 records
+    (include/ppml/QuantBlocks.h:38-41, 81-111 for the meaning of s)."""
+    flat = blocks.reshape(-1, 34)
+    out = np.zeros((flat.shape[0], 36), dtype=np.uint8)
+    out[:, 0:2] = flat[:, 0:2]
+    d = flat[:, 0:2].copy().view(np.float16)[:, 0].astype(np.float32)
+    s = (d * flat[:, 2:].view(np.int8).astype(np.int32).sum(axis=1).astype(np.float32)).astype(np.float16)
+    out[:, 2:4] = s.view(np.uint8).reshape(-1, 2)
+    out[:, 4:] = flat[:, 2:]
+    return out
+
+
+# ----------------------------------------------------------------------------- quantizer
+@pytest.mark.parametrize("rows,K,scale", [(408, 256, 1.0), (7, 32, 1.0), (33, 96, 0.02), (10609, 128, 1.0),
+                                          (5, 2048, 1e-6), (3, 64, 1e4)])
+def test_quantize_rows_bit_exact(ops, oracle, rows, K, scale):
+    rng = np.random.default_rng(rows * 1000 + K)
+    x = (rng.standard_normal((rows, K)) * scale).astype(np.float32)
+    x[0, :32] = 0.0                                  # an all-zero block
+    if K >= 64:
+        x[-1, 32:64] = np.linspace(-127, 127, 32)    # d = 1: rounding ties hit exactly
+        x[-1, 33] = 0.5
+        x[-1, 34] = -2.5
+    got = ops.quantize_rows_q8_0(_dev(x)).cpu().numpy()
+    want = oracle.quantize_q8_0(x)
+    assert got.shape == want.shape
+    assert (got == want).all(), f"{(got != want).sum()} differing bytes"
+
+
+def test_quantize_ties_and_nan_block(ops, oracle):
+    x = np.zeros((2, 32), dtype=np.float32)
+    x[0, 0] = 127.0
+    x[0, 1:9] = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 0.49999997, -0.49999997]
+    x[1, :] = 1.0
+    x[1, 5] = -2.0
+    got = ops.quantize_rows_q8_0(_dev(x)).cpu().numpy()
+    assert (got == oracle.quantize_q8_0(x)).all()
+    assert list(got[0, 0, 2:11].view(np.int8)) == [127, 1, -1, 2, -2, 3, -3, 0, 0]
+
+
+def test_dequantize_matches_oracle(ops, oracle):
+    x, _ = _inputs(3, 17, 96, 1)
+    blk = oracle.quantize_q8_0(x)
+    got = ops.dequantize_q8_0(_dev(blk)).cpu().numpy()
+    assert (got == oracle.dequantize_q8_0(blk)).all()
+
+
+def test_quantize_rejects_ragged(ops):
+    with pytest.raises(ValueError):
+        ops.quantize_rows_q8_0(torch.zeros(4, 33, device="cuda"))
+    from proteinpredictmachinelearning_amd import cabi
+    lib = cabi.load()
+    buf = torch.zeros(64, device="cuda")
+    assert lib.quantize_rows_q8_0_hip(C.c_void_p(buf.data_ptr()), C.c_void_p(buf.data_ptr()), 33, None) == 1
+
+
+# ----------------------------------------------------------------------------- fused linear
+SHAPES = [
+    # N tokens, K, M out features
+    (408, 256, 256),      # the dev-config linear (8 x 51 MSA rows)
+    (45, 32, 32),         # one block, ragged token tile
+    (100, 96, 100),       # M not a multiple of 32, odd block count
+    (64, 1056, 64),       # 33 blocks: K staged through LDS in two chunks
+    (70, 128, 800),       # 25 column tiles: more than one column pass per work-group
+    (33, 64, 300),        # 10 column tiles (8 waves x 2)
+    (1, 512, 128),        # a single token
+]
+
+
+@pytest.mark.parametrize("N,K,M", SHAPES)
+def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M):
+    x, w = _inputs(N + K + M, N, K, M)
+    wq = oracle.quantize_q8_0(w)
+    xq_want = oracle.quantize_q8_0(x)
+    W = ops.Q8Weight(_dev(wq.reshape(-1)), M, K, ops.WTYPE_Q8_0)
+    out, xq, sums = ops.mul_mat_q8(W, _dev(x), c_trans=1, dump=True)
+    out, xq, sums = out.cpu().numpy(), xq.cpu().numpy(), sums.cpu().numpy()
+    assert (xq == xq_want).all(), "activation blocks differ from quantize_q8_0_host"
+    assert (sums == oracle.q8_block_sums(wq, xq_want)).all(), "per-block int32 sums differ"
+    want = oracle.mul_mat_q8(wq, x, wtype=0, c_trans=1, fma=1)
+    assert _rel_err(out, want) <= 1e-5
+    assert (out == want).all(), f"outputs not bit-identical: rel err {_rel_err(out, want):.3e}"
+    # the undumped fast path gives the same bits
+    fast = ops.mul_mat_q8(W, _dev(x), c_trans=1).cpu().numpy()
+    assert (fast == out).all()
+
+
+@pytest.mark.parametrize("N,K,M", [(408, 256, 256), (100, 96, 100), (70, 128, 800)])
+def test_weight_layouts_and_output_orientations_agree(ops, oracle, N, K, M):
+    x, w = _inputs(11 * N + M, N, K, M)
+    wq = oracle.quantize_q8_0(w)
+    want = oracle.mul_mat_q8(wq, x, wtype=0, c_trans=1, fma=1)
+    xd = _dev(x)
+    layouts = {
+        ops.WTYPE_Q8_0: wq.reshape(-1),
+        ops.WTYPE_Q8_1: _q8_1_from_q8_0(wq).reshape(-1),
+        ops.WTYPE_Q8_0R: oracle.repack_q8_0(wq),
+    }
+    for wtype, data in layouts.items():
+        W = ops.Q8Weight(_dev(data), M, K, wtype)
+        assert (ops.mul_mat_q8(W, xd, c_trans=1).cpu().numpy() == want).all(), wtype
+        assert (ops.mul_mat_q8(W, xd, c_trans=0).cpu().numpy() == want.T).all(), wtype
+        Wm = W.pack()
+        assert Wm.wtype == ops.WTYPE_Q8_0M and Wm.data.numel() == ((M + 31) // 32) * (K // 32) * 1088
+        assert (ops.mul_mat_q8(Wm, xd, c_trans=1).cpu().numpy() == want).all(), wtype
+        assert (ops.mul_mat_q8(Wm, xd, c_trans=0).cpu().numpy() == want.T).all(), wtype
+    # quantizing the weight on the device gives the same blocks as the host quantizer
+    Wd = ops.Q8Weight.from_f32(_dev(w))
+    assert (Wd.data.cpu().numpy() == wq.reshape(-1)).all()
+
+
+def test_relu_fused_into_the_quantizer(ops, oracle):
+    # pair-track feed-forward: linear1 -> ReLU -> linear2 (src/modules/Attention.cpp:1097-1104)
+    x, w = _inputs(21, 200, 512, 128)
+    wq = oracle.quantize_q8_0(w)
+    W = ops.Q8Weight(_dev(wq.reshape(-1)), 128, 512, ops.WTYPE_Q8_0).pack()
+    got = ops.mul_mat_q8(W, _dev(x), relu=True).cpu().numpy()
+    want = oracle.mul_mat_q8(wq, np.maximum(x, 0.0), wtype=0, c_trans=1, fma=1)
+    assert (got == want).all()
+
+
+def test_status_codes(ops):
+    from proteinpredictmachinelearning_amd import cabi
+    lib = cabi.load()
+    buf = torch.zeros(4096, device="cuda")
+    p = C.c_void_p(buf.data_ptr())
+    path = C.c_int(7)
+    assert lib.mul_mat_q8_hip(p, p, p, 4, 4, 48, 0, 1, C.byref(path), None) == 2 and path.value == 0
+    assert lib.mul_mat_q8_hip(p, p, p, 4, 4, 32, 4, 1, C.byref(path), None) == 5
+    assert lib.mul_mat_q8_hip(None, p, p, 4, 4, 32, 0, 1, None, None) == 1
+    assert lib.mul_mat_q8_hip(p, p, p, 4, 4, 32, 0, 1, C.byref(path), None) == 0 and path.value == 1
+    with pytest.raises(ValueError):
+        ops.mul_mat_q8(ops.Q8Weight(buf.view(torch.uint8)[:34 * 4], 4, 32, 0), torch.zeros(3, 64, device="cuda"))
+
+
+# ----------------------------------------------------------------------------- BASELINE shapes
+def test_pair_feed_forward_shapes_full(ops, oracle):
+    # X 10609 x 128 -> 512 -> ReLU -> 128, both layers checked against the oracle in full
+    x, w1 = _inputs(103, 10609, 128, 512)
+    rng = np.random.default_rng(104)
+    w2 = (rng.standard_normal((128, 512)) * 0.02).astype(np.float32)
+    w1q, w2q = oracle.quantize_q8_0(w1), oracle.quantize_q8_0(w2)
+    W1 = ops.Q8Weight(_dev(w1q.reshape(-1)), 512, 128, 0).pack()
+    W2 = ops.Q8Weight(_dev(w2q.reshape(-1)), 128, 512, 0).pack()
+    y = ops.mul_mat_q8(W1, _dev(x))
+    z = ops.mul_mat_q8(W2, y, relu=True).cpu().numpy()
+    y = y.cpu().numpy()
+    y_want = oracle.mul_mat_q8(w1q, x, fma=1)
+    assert _rel_err(y, y_want) <= 1e-5 and (y == y_want).all()
+    z_want = oracle.mul_mat_q8(w2q, np.maximum(y_want, 0.0), fma=1)
+    assert _rel_err(z, z_want) <= 1e-5 and (z == z_want).all()
+
+
+def test_msa_qkv_shape_full_size_properties(ops, oracle):
+    # 26368 x 256 -> 768: rows are independent, so (a) a strided sample of rows must equal the oracle
+    # bit for bit, (b) permuting the token rows must permute the output rows, (c) zero rows give zeros.
+    N, K, M = 26368, 256, 768
+    x, w = _inputs(256103, N, K, M)
+    x[12345] = 0.0
+    wq = oracle.quantize_q8_0(w)
+    W = ops.Q8Weight(_dev(wq.reshape(-1)), M, K, 0).pack()
+    xd = _dev(x)
+    y = ops.mul_mat_q8(W, xd)
+    idx = np.r_[0:64, 12340:12350, N - 40:N, np.arange(97, N, 997)]
+    want = oracle.mul_mat_q8(wq, x[idx], fma=1)
+    got = y.cpu().numpy()
+    assert (got[idx] == want).all()
+    assert (got[12345] == 0).all()
+    perm = torch.randperm(N, generator=torch.Generator().manual_seed(5)).cuda()
+    y_perm = ops.mul_mat_q8(W, xd[perm].contiguous())
+    assert torch.equal(y_perm, y[perm])
+    # and the result approximates the unquantized product to quantization accuracy
+    full = x[idx].astype(np.float64) @ w.astype(np.float64).T
+    assert np.abs(got[idx] - full).max() <= 0.03 * np.abs(full).max()
