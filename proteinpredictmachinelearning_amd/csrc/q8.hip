@@ -99,68 +99,80 @@ __global__ __launch_bounds__(256) void dequantize_q8_0_kernel(const uint8_t* __r
 // is laid out the same way, so whatever order the instruction walks K in, equal K meets equal K.
 //
 // PPML_WTYPE_Q8_0M stores exactly these fragments: for tile ct and block b the 64 lanes' 16
-// bytes are consecutive (1 KiB), followed by one fp16 scale plane [ct][b][32].  Rows beyond M
-// are zero, so kernels never need a row guard on the weight side.
+// bytes are consecutive (1 KiB), followed by one fp16 scale plane [ct][b][32].  The tile count is
+// rounded up to even and rows beyond M are zero, so kernels need no guard on the weight side.
 // ------------------------------------------------------------------------------------------
-struct WFrag {
-    v4i q;
-    float d;
+__host__ __device__ inline int packed_tiles(int M) { return (((M + 31) / 32) + 1) & ~1; }
+
+struct WGeom {
+    const uint8_t* W;
+    int M, nblk, mct_pad;
 };
 
+// 16 quants of weight row 32*ct + (lane & 31), k-half lane >> 5, block b
 template <int WT>
-__device__ __forceinline__ WFrag load_wfrag(const uint8_t* __restrict__ W, int M, int nblk, int mct,
-                                            int ct, int b, int lane) {
-    WFrag f;
-    const int j = lane & 31, hh = lane >> 5;
-    const int m = ct * 32 + j;
+__device__ __forceinline__ v4i load_wq(const WGeom& g, int ct, int b, int lane) {
     if (WT == PPML_WTYPE_Q8_0M) {
-        const int64_t frag = static_cast<int64_t>(ct) * nblk + b;
-        f.q = *reinterpret_cast<const v4i*>(W + (frag * 64 + lane) * 16);
-        const uint16_t* dplane = reinterpret_cast<const uint16_t*>(W + static_cast<int64_t>(mct) * nblk * 1024);
-        f.d = half_bits_to_float(dplane[frag * 32 + j]);
-        return f;
+        ct = ct < g.mct_pad ? ct : g.mct_pad - 1;     // tiles past the end repeat the last one; never stored
+        const int64_t frag = static_cast<int64_t>(ct) * g.nblk + b;
+        return *reinterpret_cast<const v4i*>(g.W + (frag * 64 + lane) * 16);
     }
-    if (m >= M) {
-        f.q = v4i{0, 0, 0, 0};
-        f.d = 0.0f;
-        return f;
-    }
-    const int64_t blk = static_cast<int64_t>(m) * nblk + b;
+    const int hh = lane >> 5;
+    int m = ct * 32 + (lane & 31);
+    m = m < g.M ? m : g.M - 1;                        // rows past the end repeat the last one; never stored
+    const int64_t blk = static_cast<int64_t>(m) * g.nblk + b;
+    v4i q;
     if (WT == PPML_WTYPE_Q8_0R) {
         typedef int v4i_u __attribute__((ext_vector_type(4), aligned(4)));
-        f.q = *reinterpret_cast<const v4i_u*>(W + blk * 32 + hh * 16);
-        const uint16_t* dplane = reinterpret_cast<const uint16_t*>(W + static_cast<int64_t>(M) * nblk * 32);
-        f.d = half_bits_to_float(dplane[blk]);
+        q = *reinterpret_cast<const v4i_u*>(g.W + blk * 32 + hh * 16);
     } else if (WT == PPML_WTYPE_Q8_0) {
-        const uint8_t* p = W + blk * Q8_0_BYTES;       // 2-byte aligned
-        const uint16_t* q16 = reinterpret_cast<const uint16_t*>(p + 2 + hh * 16);
+        const uint16_t* q16 = reinterpret_cast<const uint16_t*>(g.W + blk * Q8_0_BYTES + 2 + hh * 16);  // 2-byte aligned
 #pragma unroll
         for (int c = 0; c < 4; ++c)
-            f.q[c] = static_cast<int>(static_cast<uint32_t>(q16[2 * c]) | (static_cast<uint32_t>(q16[2 * c + 1]) << 16));
-        f.d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(p));
+            q[c] = static_cast<int>(static_cast<uint32_t>(q16[2 * c]) | (static_cast<uint32_t>(q16[2 * c + 1]) << 16));
     } else {                                           // Q8_1: {half d; half s; int8 qs[32]}, 4-byte aligned
-        const uint8_t* p = W + blk * Q8_1_BYTES;
-        const int* q32 = reinterpret_cast<const int*>(p + 4 + hh * 16);
+        const int* q32 = reinterpret_cast<const int*>(g.W + blk * Q8_1_BYTES + 4 + hh * 16);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) f.q[c] = q32[c];
-        f.d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(p));
+        for (int c = 0; c < 4; ++c) q[c] = q32[c];
     }
-    return f;
+    return q;
+}
+
+// fp16 scale bits of weight row 32*ct + (lane & 31), block b
+template <int WT>
+__device__ __forceinline__ uint16_t load_wd(const WGeom& g, int ct, int b, int lane) {
+    if (WT == PPML_WTYPE_Q8_0M) {
+        ct = ct < g.mct_pad ? ct : g.mct_pad - 1;
+        const uint16_t* dplane = reinterpret_cast<const uint16_t*>(g.W + static_cast<int64_t>(g.mct_pad) * g.nblk * 1024);
+        return dplane[(static_cast<int64_t>(ct) * g.nblk + b) * 32 + (lane & 31)];
+    }
+    int m = ct * 32 + (lane & 31);
+    m = m < g.M ? m : g.M - 1;
+    const int64_t blk = static_cast<int64_t>(m) * g.nblk + b;
+    if (WT == PPML_WTYPE_Q8_0R) {
+        const uint16_t* dplane = reinterpret_cast<const uint16_t*>(g.W + static_cast<int64_t>(g.M) * g.nblk * 32);
+        return dplane[blk];
+    }
+    const int stride = (WT == PPML_WTYPE_Q8_0) ? Q8_0_BYTES : Q8_1_BYTES;
+    return *reinterpret_cast<const uint16_t*>(g.W + blk * stride);
 }
 
 template <int WT>
 __global__ __launch_bounds__(64) void q8_weight_pack_kernel(const uint8_t* __restrict__ W,
                                                             uint8_t* __restrict__ out, int M, int nblk,
-                                                            int mct) {
+                                                            int mct_pad) {
     const int frag = blockIdx.x;                       // ct * nblk + b
     const int ct = frag / nblk, b = frag - ct * nblk;
     const int lane = threadIdx.x;
-    // source types never take the Q8_0M branch of load_wfrag
-    const WFrag f = load_wfrag<WT>(W, M, nblk, mct, ct, b, lane);
-    *reinterpret_cast<v4i*>(out + (static_cast<int64_t>(frag) * 64 + lane) * 16) = f.q;
+    const WGeom g{W, M, nblk, mct_pad};
+    const bool live = ct * 32 + (lane & 31) < M;
+    v4i q = load_wq<WT>(g, ct, b, lane);
+    uint16_t d = load_wd<WT>(g, ct, b, lane);
+    if (!live) { q = v4i{0, 0, 0, 0}; d = 0; }
+    *reinterpret_cast<v4i*>(out + (static_cast<int64_t>(frag) * 64 + lane) * 16) = q;
     if (lane < 32) {
-        uint16_t* dplane = reinterpret_cast<uint16_t*>(out + static_cast<int64_t>(mct) * nblk * 1024);
-        dplane[static_cast<int64_t>(frag) * 32 + lane] = __half_as_ushort(__float2half_rn(f.d));  // exact: d is a half
+        uint16_t* dplane = reinterpret_cast<uint16_t*>(out + static_cast<int64_t>(mct_pad) * nblk * 1024);
+        dplane[static_cast<int64_t>(frag) * 32 + lane] = d;
     }
 }
 
@@ -170,42 +182,128 @@ __global__ __launch_bounds__(64) void q8_weight_pack_kernel(const uint8_t* __res
 //   phase 1  the work-group streams its 32 x K slice of X once from HBM (16-byte loads, 8 lanes
 //            per Q8 block, block absmax by DPP), quantizes it and leaves it in LDS already in
 //            MFMA-fragment order, scales beside it as f32.  Nothing quantized goes back to HBM.
-//   phase 2  wave w owns P consecutive 32-column tiles of the output.  For every block b
-//            (ascending) it issues one v_mfma_i32_32x32x32_i8 per tile -> exact int32 block sums,
-//            one v_mfma_f32_32x32x2_f32 that forms the 32x32 scale products d_a[row]*d_w[col]
-//            (each the exact product of two halves; the second K slot is zero), and settles
-//            acc = fma(float(sumi), d_w*d_a, acc) on the VALU.
+//   phase 2  wave w owns P consecutive 32-column tiles of the output (P even).  For every block
+//            b (ascending) and every pair of tiles it issues two v_mfma_i32_32x32x32_i8 -> exact
+//            int32 block sums, and one v_mfma_f32_32x32x1_2b_f32 whose two 32x32 outer products
+//            are the scale products d_a[row]*d_w[col] of both tiles (each the exact product of two
+//            halves), then settles acc = fma(float(sumi), d_w*d_a, acc) on the VALU.  The weight
+//            fragments of block b+1 are requested as soon as the MFMAs of block b have read theirs.
 //   phase 3  each half-wave store instruction writes one full 128-byte line of a C row.
 //
 // LDS per work-group: KC * 1152 bytes (KC = blocks staged at once, at most 32).
 // ------------------------------------------------------------------------------------------
 constexpr int TILE_TOK = 32;
 constexpr int KC_MAX = 32;          // blocks of K staged in LDS at once (K = 1024 per chunk)
+constexpr int UB = 4;               // quantizer units (8 rows x 1 block) a wave keeps in flight
+
+typedef float v32f __attribute__((ext_vector_type(32)));
+
+// Read cursor over the weight data of one pair of column tiles (ct, ct+1): 32-bit byte offsets
+// from the weight base, advanced by a fixed stride per Q8 block.
+template <int WT>
+struct WPair {
+    uint32_t oq0, oq1, od;   // offsets of this lane's fragment of tile ct, of tile ct+1, and of its scale
+    v4i q0, q1;              // fragments of block b
+    uint32_t d_bits;         // fp16 scale of tile ct (lanes 0-31) / ct+1 (lanes 32-63); converted at use
+
+    static constexpr uint32_t q_stride() {
+        return WT == PPML_WTYPE_Q8_0M ? 1024u : WT == PPML_WTYPE_Q8_0R ? 32u : WT == PPML_WTYPE_Q8_0 ? 34u : 36u;
+    }
+    static constexpr uint32_t d_stride() {
+        return WT == PPML_WTYPE_Q8_0M ? 64u : WT == PPML_WTYPE_Q8_0R ? 2u : WT == PPML_WTYPE_Q8_0 ? 34u : 36u;
+    }
+    __device__ __forceinline__ void init(const WGeom& g, int ct, int lane) {
+        const uint32_t j = lane & 31, hh = lane >> 5;
+        const uint32_t nblk = g.nblk;
+        if (WT == PPML_WTYPE_Q8_0M) {
+            // tiles past the end repeat the last pair; their results are never stored
+            const uint32_t c = ct + 1 < g.mct_pad ? ct : g.mct_pad - 2;
+            oq0 = (c * nblk * 64u + lane) * 16u;
+            oq1 = oq0 + nblk * 1024u;
+            od = static_cast<uint32_t>(g.mct_pad) * nblk * 1024u + ((c + hh) * nblk * 32u + j) * 2u;
+            return;
+        }
+        // rows past the end repeat the last row; their results are never stored
+        uint32_t m0 = ct * 32 + j, m1 = m0 + 32;
+        const uint32_t last = g.M - 1;
+        m0 = m0 < last ? m0 : last;
+        m1 = m1 < last ? m1 : last;
+        const uint32_t md = hh ? m1 : m0;
+        if (WT == PPML_WTYPE_Q8_0R) {
+            oq0 = m0 * nblk * 32u + hh * 16u;
+            oq1 = m1 * nblk * 32u + hh * 16u;
+            od = static_cast<uint32_t>(g.M) * nblk * 32u + md * nblk * 2u;
+        } else if (WT == PPML_WTYPE_Q8_0) {
+            oq0 = m0 * nblk * 34u + 2u + hh * 16u;
+            oq1 = m1 * nblk * 34u + 2u + hh * 16u;
+            od = md * nblk * 34u;
+        } else {                                       // Q8_1: {half d; half s; int8 qs[32]}
+            oq0 = m0 * nblk * 36u + 4u + hh * 16u;
+            oq1 = m1 * nblk * 36u + 4u + hh * 16u;
+            od = md * nblk * 36u;
+        }
+    }
+    static __device__ __forceinline__ v4i load_q(const uint8_t* __restrict__ W, uint32_t off) {
+        if (WT == PPML_WTYPE_Q8_0M) return *reinterpret_cast<const v4i*>(W + off);
+        if (WT == PPML_WTYPE_Q8_0) {                   // 2-byte aligned records
+            const uint16_t* q16 = reinterpret_cast<const uint16_t*>(W + off);
+            v4i q;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                q[c] = static_cast<int>(static_cast<uint32_t>(q16[2 * c]) | (static_cast<uint32_t>(q16[2 * c + 1]) << 16));
+            return q;
+        }
+        typedef int v4i_u __attribute__((ext_vector_type(4), aligned(4)));
+        return *reinterpret_cast<const v4i_u*>(W + off);
+    }
+    __device__ __forceinline__ void load(const uint8_t* __restrict__ W) {
+        q0 = load_q(W, oq0);
+        q1 = load_q(W, oq1);
+        d_bits = *reinterpret_cast<const uint16_t*>(W + od);
+    }
+    __device__ __forceinline__ void advance() {
+        oq0 += q_stride();
+        oq1 += q_stride();
+        od += d_stride();
+    }
+};
 
 template <int NW, int P, int WT, bool DUMP>
-__global__ __launch_bounds__(NW * 64) void q8_linear_kernel(
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void q8_linear_kernel(
     const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
-    int M, int N, int nblk, int mct, int c_trans, int relu,
+    int M, int N, int nblk, int c_trans, int relu,
     uint8_t* __restrict__ xq_dump, int32_t* __restrict__ sums_dump) {
+    static_assert(P % 2 == 0, "column tiles are processed in pairs");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int kc = nblk < KC_MAX ? nblk : KC_MAX;
-    v4i* lds_a = reinterpret_cast<v4i*>(lds);                              // [kc][64] fragments
-    float* lds_d = reinterpret_cast<float*>(lds + static_cast<size_t>(kc) * 1024);  // [kc][32]
+    v4i* lds_a = reinterpret_cast<v4i*>(lds);                                        // [kc][64] fragments
+    float* lds_d = reinterpret_cast<float*>(lds + static_cast<size_t>(kc) * 1024);   // [kc][32]
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int j = lane & 31, hh = lane >> 5;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: keeps tile addressing scalar
+    const int j = lane & 31;
     const int tok0 = blockIdx.x * TILE_TOK;
     const int K = nblk * QK;
+    const int mct = (M + 31) / 32;
+    const WGeom g{W, M, nblk, packed_tiles(M)};
 
-    const int cols_per_pass = NW * P;                  // 32-column tiles covered by one pass
-    for (int ct_base = 0; ct_base < mct; ct_base += cols_per_pass) {
+    for (int ct_base = 0; ct_base < mct; ct_base += NW * P) {
         const int ct0 = ct_base + wave * P;
         v16f acc[P];
 #pragma unroll
         for (int p = 0; p < P; ++p)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[p][r] = 0.0f;
+
+        WPair<WT> wp[P / 2];
+        if (ct0 < mct) {
+#pragma unroll
+            for (int pp = 0; pp < P / 2; ++pp) {
+                wp[pp].init(g, ct0 + 2 * pp, lane);
+                wp[pp].load(W);                        // block 0, in flight while X is quantized
+            }
+        }
 
         for (int b0 = 0; b0 < nblk; b0 += kc) {
             const int nb = (nblk - b0) < kc ? (nblk - b0) : kc;
@@ -214,25 +312,24 @@ __global__ __launch_bounds__(NW * 64) void q8_linear_kernel(
             if (ct_base == 0 || nblk > kc) {
                 if (b0 > 0 || ct_base > 0) __syncthreads();        // previous readers are done
                 const int units = nb * 4;                          // (8 rows) x (1 block) per wave step
-                const int g = lane >> 3, c8 = lane & 7;
-                for (int u0 = wave; u0 < units; u0 += NW * 4) {
-                    v4f xv[4];
+                const int grp = lane >> 3, c8 = lane & 7;
+                for (int u0 = wave; u0 < units; u0 += NW * UB) {
+                    v4f xv[UB];
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) {
-                        const int u = u0 + s * NW;
-                        const int row = (u & 3) * 8 + g;
-                        const int bl = u >> 2;
-                        const int tok = tok0 + row;
-                        xv[s] = v4f{0.f, 0.f, 0.f, 0.f};
-                        if (u < units && tok < N)
-                            xv[s] = *reinterpret_cast<const v4f_u*>(
-                                X + static_cast<int64_t>(tok) * K + (b0 + bl) * QK + c8 * 4);
+                    for (int s = 0; s < UB; ++s) {
+                        int u = u0 + s * NW;
+                        u = u < units ? u : units - 1;             // surplus slots repeat the last unit
+                        const int row = (u & 3) * 8 + grp;
+                        int tok = tok0 + row;
+                        tok = tok < N ? tok : N - 1;               // rows past the end repeat the last row
+                        xv[s] = *reinterpret_cast<const v4f_u*>(
+                            X + static_cast<int64_t>(tok) * K + (b0 + (u >> 2)) * QK + c8 * 4);
                     }
 #pragma unroll
-                    for (int s = 0; s < 4; ++s) {
+                    for (int s = 0; s < UB; ++s) {
                         const int u = u0 + s * NW;
-                        if (u >= units) continue;                  // wave-uniform
-                        const int row = (u & 3) * 8 + g;
+                        if (u >= units) break;                     // wave-uniform
+                        const int row = (u & 3) * 8 + grp;
                         const int bl = u >> 2;
                         v4f x = xv[s];
                         if (relu) {
@@ -259,35 +356,46 @@ __global__ __launch_bounds__(NW * 64) void q8_linear_kernel(
                 __syncthreads();
             }
 
-            // ---------------- phase 2: blocks ascending, P column tiles per wave
+            // ---------------- phase 2: blocks ascending, P column tiles per wave, in pairs
             if (ct0 < mct) {
                 for (int bl = 0; bl < nb; ++bl) {
                     const int b = b0 + bl;
+                    const bool more = b + 1 < nblk;                                // last block: harmless re-read
                     const v4i afrag = lds_a[bl * 64 + lane];
-                    const float da_lane = (hh == 0) ? lds_d[bl * 32 + j] : 0.0f;   // K slot 0 only
+                    const float da_lane = lds_d[bl * 32 + j];                      // rows of both scale blocks
 #pragma unroll
-                    for (int p = 0; p < P; ++p) {
-                        const int ct = ct0 + p;
-                        if (ct >= mct) break;                                      // wave-uniform
-                        const WFrag wf = load_wfrag<WT>(W, M, nblk, mct, ct, b, lane);
+                    for (int pp = 0; pp < P / 2; ++pp) {
                         v16i zero_i;
-                        v16f zero_f;
+                        v32f zero_f;
 #pragma unroll
-                        for (int r = 0; r < 16; ++r) { zero_i[r] = 0; zero_f[r] = 0.0f; }
-                        // rows = activation rows (A operand), columns = weight rows (B operand)
-                        const v16i sumi = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, wf.q, zero_i, 0, 0, 0);
-                        const float dw_lane = (hh == 0) ? wf.d : 0.0f;
-                        const v16f scale = __builtin_amdgcn_mfma_f32_32x32x2f32(da_lane, dw_lane, zero_f, 0, 0, 0);
+                        for (int r = 0; r < 16; ++r) zero_i[r] = 0;
 #pragma unroll
-                        for (int r = 0; r < 16; ++r)
-                            acc[p][r] = __builtin_fmaf(static_cast<float>(sumi[r]), scale[r], acc[p][r]);
+                        for (int r = 0; r < 32; ++r) zero_f[r] = 0.0f;
+                        // rows = activation rows (A operand), columns = weight rows (B operand);
+                        // the longest instruction goes first so the first settle can start earliest
+                        const float dw_lane = half_bits_to_float(static_cast<uint16_t>(wp[pp].d_bits));
+                        const v32f scale = __builtin_amdgcn_mfma_f32_32x32x1f32(da_lane, dw_lane, zero_f, 0, 0, 0);
+                        const v16i sum0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, wp[pp].q0, zero_i, 0, 0, 0);
+                        const v16i sum1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, wp[pp].q1, zero_i, 0, 0, 0);
+                        // request block b+1 now that the MFMAs have read block b; it lands during the settle
+                        __builtin_amdgcn_sched_barrier(0);
+                        if (more) wp[pp].advance();
+                        wp[pp].load(W);
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            acc[2 * pp][r] = __builtin_fmaf(static_cast<float>(sum0[r]), scale[r], acc[2 * pp][r]);
+                            acc[2 * pp + 1][r] = __builtin_fmaf(static_cast<float>(sum1[r]), scale[16 + r], acc[2 * pp + 1][r]);
+                        }
                         if (DUMP && sums_dump) {
 #pragma unroll
                             for (int r = 0; r < 16; ++r) {
                                 const int tok = tok0 + mfma32_row(r, lane);
-                                const int m = ct * 32 + j;
-                                if (tok < N && m < M)
-                                    sums_dump[(static_cast<int64_t>(tok) * M + m) * nblk + b] = sumi[r];
+                                const int m0 = (ct0 + 2 * pp) * 32 + j;
+                                if (tok < N && m0 < M)
+                                    sums_dump[(static_cast<int64_t>(tok) * M + m0) * nblk + b] = sum0[r];
+                                if (tok < N && m0 + 32 < M)
+                                    sums_dump[(static_cast<int64_t>(tok) * M + m0 + 32) * nblk + b] = sum1[r];
                             }
                         }
                     }
@@ -296,17 +404,30 @@ __global__ __launch_bounds__(NW * 64) void q8_linear_kernel(
         }
 
         // ---------------- phase 3: store
+        if (ct0 < mct) {
+            const bool full = (tok0 + TILE_TOK <= N) && (c_trans != 0);
+            if (full) {
+                float* crow = C + static_cast<int64_t>(tok0 + 4 * (lane >> 5)) * M + ct0 * 32 + j;
 #pragma unroll
-        for (int p = 0; p < P; ++p) {
-            const int ct = ct0 + p;
-            if (ct >= mct) break;
-            const int m = ct * 32 + j;
+                for (int p = 0; p < P; ++p) {
+                    if ((ct0 + p) * 32 + j < M) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int tok = tok0 + mfma32_row(r, lane);
-                if (tok < N && m < M) {
-                    if (c_trans) C[static_cast<int64_t>(tok) * M + m] = acc[p][r];
-                    else         C[static_cast<int64_t>(m) * N + tok] = acc[p][r];
+                        for (int r = 0; r < 16; ++r)
+                            __builtin_nontemporal_store(acc[p][r], crow + static_cast<int64_t>(8 * (r >> 2) + (r & 3)) * M + p * 32);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < P; ++p) {
+                    const int m = (ct0 + p) * 32 + j;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int tok = tok0 + mfma32_row(r, lane);
+                        if (tok < N && m < M) {
+                            if (c_trans) C[static_cast<int64_t>(tok) * M + m] = acc[p][r];
+                            else         C[static_cast<int64_t>(m) * N + tok] = acc[p][r];
+                        }
+                    }
                 }
             }
         }
@@ -316,17 +437,16 @@ __global__ __launch_bounds__(NW * 64) void q8_linear_kernel(
 template <int NW, int P, int WT>
 int launch_q8_linear(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
                      int relu, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
-    const int mct = (M + 31) / 32;
     const int kc = nblk < KC_MAX ? nblk : KC_MAX;
     const size_t lds = static_cast<size_t>(kc) * (1024 + 32 * sizeof(float));
     const dim3 grid((N + TILE_TOK - 1) / TILE_TOK), block(NW * 64);
     if (xq_dump || sums_dump)
         hipLaunchKernelGGL((q8_linear_kernel<NW, P, WT, true>), grid, block, lds, stream,
-                           static_cast<const uint8_t*>(W), X, C, M, N, nblk, mct, c_trans, relu,
+                           static_cast<const uint8_t*>(W), X, C, M, N, nblk, c_trans, relu,
                            static_cast<uint8_t*>(xq_dump), sums_dump);
     else
         hipLaunchKernelGGL((q8_linear_kernel<NW, P, WT, false>), grid, block, lds, stream,
-                           static_cast<const uint8_t*>(W), X, C, M, N, nblk, mct, c_trans, relu,
+                           static_cast<const uint8_t*>(W), X, C, M, N, nblk, c_trans, relu,
                            static_cast<uint8_t*>(nullptr), static_cast<int32_t*>(nullptr));
     return check_launch("q8_linear_kernel");
 }
@@ -335,11 +455,11 @@ template <int WT>
 int dispatch_q8_linear(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
                        int relu, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
     const int mct = (M + 31) / 32;
-    // waves split the output columns; pick the shape with the least idle tiles
-    if (mct <= 4)  return launch_q8_linear<4, 1, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
-    if (mct <= 8)  return launch_q8_linear<8, 1, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
-    if (mct <= 16) return launch_q8_linear<8, 2, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
-    return launch_q8_linear<8, 3, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
+    // waves split the output columns; pick the shape with the fewest idle column tiles
+    if (mct <= 4)  return launch_q8_linear<2, 2, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
+    if (mct <= 8)  return launch_q8_linear<4, 2, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
+    if (mct <= 16) return launch_q8_linear<4, 4, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
+    return launch_q8_linear<4, 6, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
 }
 
 }  // namespace
@@ -367,14 +487,14 @@ extern "C" int dequantize_q8_0_hip(const void* x, float* y, int64_t ne, ppml_hip
 
 extern "C" size_t q8_weight_packed_bytes_hip(int M, int K) {
     if (M <= 0 || K <= 0 || (K % QK) != 0) return 0;
-    const size_t mct = (static_cast<size_t>(M) + 31) / 32;
-    return mct * static_cast<size_t>(K / QK) * (1024 + 32 * sizeof(uint16_t));
+    const size_t tiles = static_cast<size_t>(packed_tiles(M));
+    return tiles * static_cast<size_t>(K / QK) * (1024 + 32 * sizeof(uint16_t));
 }
 
 extern "C" int q8_weight_pack_hip(const void* W, int wtype, int M, int K, void* packed, ppml_hip_stream_t stream) {
     if (!W || !packed || M <= 0 || K <= 0) { set_error("q8_weight_pack_hip: bad arguments"); return RC_BAD_ARGS; }
     if ((K % QK) != 0) { set_error("q8_weight_pack_hip: K=%d is not a multiple of 32", K); return RC_K_NOT_32; }
-    const int nblk = K / QK, mct = (M + 31) / 32;
+    const int nblk = K / QK, mct = packed_tiles(M);
     const dim3 grid(mct * nblk), block(64);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint8_t* w = static_cast<const uint8_t*>(W);

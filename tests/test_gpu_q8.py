@@ -143,7 +143,8 @@ def test_weight_layouts_and_output_orientations_agree(ops, oracle, N, K, M):
         assert (ops.mul_mat_q8(W, xd, c_trans=1).cpu().numpy() == want).all(), wtype
         assert (ops.mul_mat_q8(W, xd, c_trans=0).cpu().numpy() == want.T).all(), wtype
         Wm = W.pack()
-        assert Wm.wtype == ops.WTYPE_Q8_0M and Wm.data.numel() == ((M + 31) // 32) * (K // 32) * 1088
+        tiles = (((M + 31) // 32) + 1) // 2 * 2          # the packed layout holds an even number of 32-row tiles
+        assert Wm.wtype == ops.WTYPE_Q8_0M and Wm.data.numel() == tiles * (K // 32) * 1088
         assert (ops.mul_mat_q8(Wm, xd, c_trans=1).cpu().numpy() == want).all(), wtype
         assert (ops.mul_mat_q8(Wm, xd, c_trans=0).cpu().numpy() == want.T).all(), wtype
     # quantizing the weight on the device gives the same blocks as the host quantizer
