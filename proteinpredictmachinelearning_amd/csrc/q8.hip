@@ -14,49 +14,75 @@ namespace {
 // Quantizer arithmetic shared by the standalone and the fused kernel.
 // ------------------------------------------------------------------------------------------
 
-// max over each aligned group of 8 lanes (one Q8 block when every lane holds 4 elements)
-__device__ __forceinline__ float group8_max(float v) {
+// max over each aligned group of 4 lanes (one Q8 block when every lane holds 8 elements)
+__device__ __forceinline__ float group4_max(float v) {
     float o;
     o = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));  // lane ^ 1
     v = fmaxf(v, o);
     o = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));  // lane ^ 2
     v = fmaxf(v, o);
-    o = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false)); // 7 - lane (half row mirror)
-    v = fmaxf(v, o);
     return v;
 }
 
 struct BlockQuant {
-    uint32_t q4;      // this lane's 4 quants, element c in byte c
-    uint16_t d_bits;  // fp16 scale of the block
+    uint32_t q_lo, q_hi;  // this lane's 8 quants, element c in byte c % 4 of word c / 4
+    uint16_t d_bits;      // fp16 scale of the block
 };
 
-// x holds elements 4*c8 .. 4*c8+3 of one 32-element block, the 8 lanes of an aligned group hold
-// the whole block.  IEEE division, round half away from zero, clamp to +-127.
-__device__ __forceinline__ BlockQuant quantize_block_lane(v4f x) {
+// round(t) for |t| <= 200 as one add and one truncating convert: adding the largest float below
+// one half (with t's sign) carries exactly the ties and nothing else over the integer boundary,
+// so the result equals (int)roundf(t) -- half away from zero -- for every binary32 t in range
+// (checked exhaustively against roundf on the host).
+__device__ __forceinline__ int round_half_away_to_int(float t) {
+    const float h = __int_as_float((__float_as_int(t) & 0x80000000) | 0x3effffff);
+    return static_cast<int>(t + h);
+}
+
+__device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
+    const uint32_t ab = __builtin_amdgcn_perm(static_cast<uint32_t>(b), static_cast<uint32_t>(a), 0x0c0c0400u);
+    const uint32_t cd = __builtin_amdgcn_perm(static_cast<uint32_t>(d), static_cast<uint32_t>(c), 0x0c0c0400u);
+    return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
+}
+
+// x0,x1 hold elements 8*c4 .. 8*c4+7 of one 32-element block, the 4 lanes of an aligned group hold
+// the whole block.  IEEE division for the scale and its reciprocal, round half away from zero,
+// clamp to +-127 (include/ppml/QuantBlocks.h:62-79).
+__device__ __forceinline__ BlockQuant quantize_block_lane(v4f x0, v4f x1) {
     float amax = 0.0f;
-    amax = fmaxf(amax, fabsf(x[0]));   // fmaxf drops NaN like std::fmax
-    amax = fmaxf(amax, fabsf(x[1]));
-    amax = fmaxf(amax, fabsf(x[2]));
-    amax = fmaxf(amax, fabsf(x[3]));
-    amax = group8_max(amax);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) amax = fmaxf(amax, fabsf(x0[c]));   // fmaxf drops NaN like std::fmax
+#pragma unroll
+    for (int c = 0; c < 4; ++c) amax = fmaxf(amax, fabsf(x1[c]));
+    amax = group4_max(amax);
     const float d = amax / 127.0f;
     const float inv = (amax == 0.0f) ? 0.0f : 1.0f / d;
     BlockQuant out;
     out.d_bits = __half_as_ushort(__float2half_rn(d));
-    uint32_t packed = 0;
+    int q[8];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        float q = roundf(x[c] * inv);
-        q = q > 127.0f ? 127.0f : (q < -127.0f ? -127.0f : q);
-        packed |= (static_cast<uint32_t>(static_cast<int>(q)) & 0xffu) << (8 * c);
+        q[c] = round_half_away_to_int(x0[c] * inv);
+        q[4 + c] = round_half_away_to_int(x1[c] * inv);
     }
-    out.q4 = packed;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) q[c] = q[c] > 127 ? 127 : (q[c] < -127 ? -127 : q[c]);
+    out.q_lo = pack4(q[0], q[1], q[2], q[3]);
+    out.q_hi = pack4(q[4], q[5], q[6], q[7]);
     return out;
 }
 
 __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
     return __half2float(__ushort_as_half(h));
+}
+
+// 8 quants of block `blk` (2-byte aligned 34-byte record) written by the lane that owns them
+__device__ __forceinline__ void store_block_part(uint8_t* blk, int c4, const BlockQuant& bq) {
+    uint16_t* q16 = reinterpret_cast<uint16_t*>(blk + 2 + c4 * 8);
+    q16[0] = static_cast<uint16_t>(bq.q_lo & 0xffffu);
+    q16[1] = static_cast<uint16_t>(bq.q_lo >> 16);
+    q16[2] = static_cast<uint16_t>(bq.q_hi & 0xffffu);
+    q16[3] = static_cast<uint16_t>(bq.q_hi >> 16);
+    if (c4 == 0) *reinterpret_cast<uint16_t*>(blk) = bq.d_bits;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -66,18 +92,16 @@ __global__ __launch_bounds__(256) void quantize_rows_q8_0_kernel(const float* __
                                                                  uint8_t* __restrict__ y,
                                                                  int64_t nblocks) {
     const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    int64_t ib = t >> 3;
-    const int c8 = static_cast<int>(t & 7);
+    int64_t ib = t >> 2;
+    const int c4 = static_cast<int>(t & 3);
     const bool live = ib < nblocks;
-    if (!live) ib = nblocks - 1;                       // keep the whole 8-lane group convergent
-    const v4f xv = *reinterpret_cast<const v4f_u*>(x + ib * QK + c8 * 4);
-    const BlockQuant bq = quantize_block_lane(xv);
+    if (!live) ib = nblocks - 1;                       // keep the whole 4-lane group convergent
+    const float* src = x + ib * QK + c4 * 8;
+    const v4f x0 = *reinterpret_cast<const v4f_u*>(src);
+    const v4f x1 = *reinterpret_cast<const v4f_u*>(src + 4);
+    const BlockQuant bq = quantize_block_lane(x0, x1);
     if (!live) return;
-    uint8_t* blk = y + ib * Q8_0_BYTES;               // 2-byte aligned only
-    uint16_t* q16 = reinterpret_cast<uint16_t*>(blk + 2 + c8 * 4);
-    q16[0] = static_cast<uint16_t>(bq.q4 & 0xffffu);
-    q16[1] = static_cast<uint16_t>(bq.q4 >> 16);
-    if (c8 == 0) *reinterpret_cast<uint16_t*>(blk) = bq.d_bits;
+    store_block_part(y + ib * Q8_0_BYTES, c4, bq);
 }
 
 __global__ __launch_bounds__(256) void dequantize_q8_0_kernel(const uint8_t* __restrict__ x,
@@ -179,22 +203,43 @@ __global__ __launch_bounds__(64) void q8_weight_pack_kernel(const uint8_t* __res
 // ------------------------------------------------------------------------------------------
 // Fused Q8_0 linear:  C = Q8_0(X) . W^T   for one tile of 32 activation rows per work-group.
 //
-//   phase 1  the work-group streams its 32 x K slice of X once from HBM (16-byte loads, 8 lanes
+//   phase 1  the work-group streams its 32 x K slice of X once from HBM (16-byte loads, 4 lanes
 //            per Q8 block, block absmax by DPP), quantizes it and leaves it in LDS already in
 //            MFMA-fragment order, scales beside it as f32.  Nothing quantized goes back to HBM.
-//   phase 2  wave w owns P consecutive 32-column tiles of the output (P even).  For every block
-//            b (ascending) and every pair of tiles it issues two v_mfma_i32_32x32x32_i8 -> exact
-//            int32 block sums, and one v_mfma_f32_32x32x1_2b_f32 whose two 32x32 outer products
-//            are the scale products d_a[row]*d_w[col] of both tiles (each the exact product of two
-//            halves), then settles acc = fma(float(sumi), d_w*d_a, acc) on the VALU.  The weight
-//            fragments of block b+1 are requested as soon as the MFMAs of block b have read theirs.
-//   phase 3  each half-wave store instruction writes one full 128-byte line of a C row.
+//   phase 2  the waves share out the output columns in pairs of 32-column tiles.  For one pair a
+//            wave walks the blocks in ascending order; per block it issues two
+//            v_mfma_i32_32x32x32_i8 -> exact int32 block sums, and one v_mfma_f32_32x32x1_2b_f32
+//            whose two 32x32 outer products are the scale products d_w[col]*d_a[row] of both tiles
+//            (each the exact product of two halves), then settles
+//            acc = fma(float(sumi), d_w*d_a, acc) on the VALU.  The weight fragments of the next
+//            block are requested as soon as the MFMAs of this one have read theirs.
+//   phase 3  the pair is stored at once (16 bytes per lane), so the output streams to HBM while the
+//            other pairs are still being computed; only 32 accumulator registers are ever live,
+//            which lets four work-groups share a CU.
 //
-// LDS per work-group: KC * 1152 bytes (KC = blocks staged at once, at most 32).
+// MFMA roles: A = weight rows (output rows of the instruction), B = activation rows (output
+// columns), so a lane ends up with 4 consecutive output features of one token per register quad.
+//
+// LDS per work-group: kc * 1152 bytes, kc = blocks of K staged at once (at most KC_MAX).  For longer
+// rows K is walked in chunks and the partial result of every output is carried in C itself, which
+// keeps the per-output block order intact.
 // ------------------------------------------------------------------------------------------
+#ifdef PPML_Q8_TRACE
+// Development aid, compiled out of the library: per-wave timestamps of the kernel's phases.
+__device__ unsigned long long* g_q8_trace = nullptr;
+#define PPML_TRACE_MARK(slot)                                                                      \
+    do {                                                                                           \
+        if (g_q8_trace && (threadIdx.x & 63) == 0)                                                 \
+            g_q8_trace[(static_cast<size_t>(blockIdx.x) * NW + (threadIdx.x >> 6)) * 32 + (slot)] = \
+                __builtin_amdgcn_s_memrealtime();   /* 100 MHz, common to the whole device */      \
+    } while (0)
+#else
+#define PPML_TRACE_MARK(slot) do {} while (0)
+#endif
+
 constexpr int TILE_TOK = 32;
-constexpr int KC_MAX = 32;          // blocks of K staged in LDS at once (K = 1024 per chunk)
-constexpr int UB = 4;               // quantizer units (8 rows x 1 block) a wave keeps in flight
+constexpr int KC_MAX = 56;          // blocks of K staged in LDS at once (63 KiB)
+constexpr int UB = 4;               // quantizer units (8 rows x 2 blocks) a wave keeps in flight
 
 typedef float v32f __attribute__((ext_vector_type(32)));
 
@@ -203,7 +248,7 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 template <int WT>
 struct WPair {
     uint32_t oq0, oq1, od;   // offsets of this lane's fragment of tile ct, of tile ct+1, and of its scale
-    v4i q0, q1;              // fragments of block b
+    v4i q0, q1;              // fragments of the current block
     uint32_t d_bits;         // fp16 scale of tile ct (lanes 0-31) / ct+1 (lanes 32-63); converted at use
 
     static constexpr uint32_t q_stride() {
@@ -212,15 +257,16 @@ struct WPair {
     static constexpr uint32_t d_stride() {
         return WT == PPML_WTYPE_Q8_0M ? 64u : WT == PPML_WTYPE_Q8_0R ? 2u : WT == PPML_WTYPE_Q8_0 ? 34u : 36u;
     }
-    __device__ __forceinline__ void init(const WGeom& g, int ct, int lane) {
+    // cursor at block b of the pair starting at tile ct
+    __device__ __forceinline__ void init(const WGeom& g, int ct, int b, int lane) {
         const uint32_t j = lane & 31, hh = lane >> 5;
         const uint32_t nblk = g.nblk;
         if (WT == PPML_WTYPE_Q8_0M) {
-            // tiles past the end repeat the last pair; their results are never stored
+            // pairs past the end repeat the last pair; their results are never stored
             const uint32_t c = ct + 1 < g.mct_pad ? ct : g.mct_pad - 2;
-            oq0 = (c * nblk * 64u + lane) * 16u;
+            oq0 = ((c * nblk + b) * 64u + lane) * 16u;
             oq1 = oq0 + nblk * 1024u;
-            od = static_cast<uint32_t>(g.mct_pad) * nblk * 1024u + ((c + hh) * nblk * 32u + j) * 2u;
+            od = static_cast<uint32_t>(g.mct_pad) * nblk * 1024u + (((c + hh) * nblk + b) * 32u + j) * 2u;
             return;
         }
         // rows past the end repeat the last row; their results are never stored
@@ -230,17 +276,17 @@ struct WPair {
         m1 = m1 < last ? m1 : last;
         const uint32_t md = hh ? m1 : m0;
         if (WT == PPML_WTYPE_Q8_0R) {
-            oq0 = m0 * nblk * 32u + hh * 16u;
-            oq1 = m1 * nblk * 32u + hh * 16u;
-            od = static_cast<uint32_t>(g.M) * nblk * 32u + md * nblk * 2u;
+            oq0 = (m0 * nblk + b) * 32u + hh * 16u;
+            oq1 = (m1 * nblk + b) * 32u + hh * 16u;
+            od = static_cast<uint32_t>(g.M) * nblk * 32u + (md * nblk + b) * 2u;
         } else if (WT == PPML_WTYPE_Q8_0) {
-            oq0 = m0 * nblk * 34u + 2u + hh * 16u;
-            oq1 = m1 * nblk * 34u + 2u + hh * 16u;
-            od = md * nblk * 34u;
+            oq0 = (m0 * nblk + b) * 34u + 2u + hh * 16u;
+            oq1 = (m1 * nblk + b) * 34u + 2u + hh * 16u;
+            od = (md * nblk + b) * 34u;
         } else {                                       // Q8_1: {half d; half s; int8 qs[32]}
-            oq0 = m0 * nblk * 36u + 4u + hh * 16u;
-            oq1 = m1 * nblk * 36u + 4u + hh * 16u;
-            od = md * nblk * 36u;
+            oq0 = (m0 * nblk + b) * 36u + 4u + hh * 16u;
+            oq1 = (m1 * nblk + b) * 36u + 4u + hh * 16u;
+            od = (md * nblk + b) * 36u;
         }
     }
     static __device__ __forceinline__ v4i load_q(const uint8_t* __restrict__ W, uint32_t off) {
@@ -268,198 +314,490 @@ struct WPair {
     }
 };
 
-template <int NW, int P, int WT, bool DUMP>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2))) void q8_linear_kernel(
+// address of C(tok, m) and whether a lane may touch it
+struct COut {
+    float* C;
+    int M, N, c_trans;
+    __device__ __forceinline__ float* at(int tok, int m) const {
+        return c_trans ? C + static_cast<int64_t>(tok) * M + m : C + static_cast<int64_t>(m) * N + tok;
+    }
+};
+
+template <int NW, int WT, bool DUMP>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void q8_linear_kernel(
     const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
-    int M, int N, int nblk, int c_trans, int relu,
+    int M, int N, int nblk, int kc, int c_trans, int relu,
     uint8_t* __restrict__ xq_dump, int32_t* __restrict__ sums_dump) {
-    static_assert(P % 2 == 0, "column tiles are processed in pairs");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    const int kc = nblk < KC_MAX ? nblk : KC_MAX;
     v4i* lds_a = reinterpret_cast<v4i*>(lds);                                        // [kc][64] fragments
     float* lds_d = reinterpret_cast<float*>(lds + static_cast<size_t>(kc) * 1024);   // [kc][32]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: keeps tile addressing scalar
-    const int j = lane & 31;
+    const int j = lane & 31, hh = lane >> 5;
     const int tok0 = blockIdx.x * TILE_TOK;
     const int K = nblk * QK;
-    const int mct = (M + 31) / 32;
+    const int npairs = (M + 63) / 64;
     const WGeom g{W, M, nblk, packed_tiles(M)};
+    const COut out{C, M, N, c_trans};
+    const int tok = tok0 + j;                          // this lane's activation row in every MFMA result
+    PPML_TRACE_MARK(0);
 
-    for (int ct_base = 0; ct_base < mct; ct_base += NW * P) {
-        const int ct0 = ct_base + wave * P;
-        v16f acc[P];
+    for (int b0 = 0; b0 < nblk; b0 += kc) {
+        const int nb = (nblk - b0) < kc ? (nblk - b0) : kc;
+        // ---------------- phase 1: quantize X[tok0..+32][b0*32 .. (b0+nb)*32) into LDS
+        if (b0 > 0) __syncthreads();                   // readers of the previous chunk are done
+        WPair<WT> wp;
+        {
+            const int npair_b = (nb + 1) >> 1;
+            const int units = npair_b * 4;             // (8 rows) x (2 blocks) per wave step
+            const int grp = lane >> 2, c4 = lane & 3;
+            const int urow = grp & 7, ublk = grp >> 3; // row and block within the unit
+            for (int u0 = wave; u0 < units; u0 += NW * UB) {
+                v4f xv[UB][2];
 #pragma unroll
-        for (int p = 0; p < P; ++p)
+                for (int s = 0; s < UB; ++s) {
+                    int u = u0 + s * NW;
+                    u = u < units ? u : units - 1;     // surplus slots repeat the last unit
+                    int bl = (u >> 2) * 2 + ublk;
+                    bl = bl < nb ? bl : nb - 1;        // odd block count: repeat the last block
+                    int t = tok0 + (u & 3) * 8 + urow;
+                    t = t < N ? t : N - 1;             // rows past the end repeat the last row
+                    const float* src = X + static_cast<int64_t>(t) * K + (b0 + bl) * QK + c4 * 8;
+                    xv[s][0] = *reinterpret_cast<const v4f_u*>(src);
+                    xv[s][1] = *reinterpret_cast<const v4f_u*>(src + 4);
+                }
+                if (u0 == wave && wave < npairs) {
+                    // first weight block of this wave's first pair: requested behind the activation
+                    // loads, lands while they are being quantized
+                    wp.init(g, 2 * wave, b0, lane);
+                    wp.load(W);
+                }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[p][r] = 0.0f;
-
-        WPair<WT> wp[P / 2];
-        if (ct0 < mct) {
+                for (int s = 0; s < UB; ++s) {
+                    const int u = u0 + s * NW;
+                    if (u >= units) break;             // wave-uniform
+                    const int row = (u & 3) * 8 + urow;
+                    const int bl = (u >> 2) * 2 + ublk;
+                    v4f x0 = xv[s][0], x1 = xv[s][1];
+                    if (relu) {
 #pragma unroll
-            for (int pp = 0; pp < P / 2; ++pp) {
-                wp[pp].init(g, ct0 + 2 * pp, lane);
-                wp[pp].load(W);                        // block 0, in flight while X is quantized
-            }
-        }
-
-        for (int b0 = 0; b0 < nblk; b0 += kc) {
-            const int nb = (nblk - b0) < kc ? (nblk - b0) : kc;
-            // ---------------- phase 1: quantize X[tok0..+32][b0*32 .. (b0+nb)*32) into LDS
-            // (skipped when the whole K is already staged from an earlier column pass)
-            if (ct_base == 0 || nblk > kc) {
-                if (b0 > 0 || ct_base > 0) __syncthreads();        // previous readers are done
-                const int units = nb * 4;                          // (8 rows) x (1 block) per wave step
-                const int grp = lane >> 3, c8 = lane & 7;
-                for (int u0 = wave; u0 < units; u0 += NW * UB) {
-                    v4f xv[UB];
-#pragma unroll
-                    for (int s = 0; s < UB; ++s) {
-                        int u = u0 + s * NW;
-                        u = u < units ? u : units - 1;             // surplus slots repeat the last unit
-                        const int row = (u & 3) * 8 + grp;
-                        int tok = tok0 + row;
-                        tok = tok < N ? tok : N - 1;               // rows past the end repeat the last row
-                        xv[s] = *reinterpret_cast<const v4f_u*>(
-                            X + static_cast<int64_t>(tok) * K + (b0 + (u >> 2)) * QK + c8 * 4);
+                        for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
                     }
-#pragma unroll
-                    for (int s = 0; s < UB; ++s) {
-                        const int u = u0 + s * NW;
-                        if (u >= units) break;                     // wave-uniform
-                        const int row = (u & 3) * 8 + grp;
-                        const int bl = u >> 2;
-                        v4f x = xv[s];
-                        if (relu) {
-#pragma unroll
-                            for (int c = 0; c < 4; ++c) x[c] = fmaxf(x[c], 0.0f);
-                        }
-                        const BlockQuant bq = quantize_block_lane(x);
-                        // fragment order: block bl, k-half c8/4, row, dword c8%4
-                        int* dst = reinterpret_cast<int*>(lds_a) + ((bl * 64 + (c8 >> 2) * 32 + row) * 4 + (c8 & 3));
-                        *dst = static_cast<int>(bq.q4);
-                        if (c8 == 0) lds_d[bl * 32 + row] = half_bits_to_float(bq.d_bits);
+                    const BlockQuant bq = quantize_block_lane(x0, x1);
+                    if (bl < nb) {
+                        // fragment order: block bl, k-half c4/2, row, dword pair c4%2
+                        uint2* dst = reinterpret_cast<uint2*>(lds_a) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
+                        *dst = uint2{bq.q_lo, bq.q_hi};
+                        if (c4 == 0) lds_d[bl * 32 + row] = half_bits_to_float(bq.d_bits);
                         if (DUMP && xq_dump) {
-                            const int tok = tok0 + row;
-                            if (tok < N) {
-                                uint8_t* blk = xq_dump + (static_cast<int64_t>(tok) * nblk + b0 + bl) * Q8_0_BYTES;
-                                uint16_t* q16 = reinterpret_cast<uint16_t*>(blk + 2 + c8 * 4);
-                                q16[0] = static_cast<uint16_t>(bq.q4 & 0xffffu);
-                                q16[1] = static_cast<uint16_t>(bq.q4 >> 16);
-                                if (c8 == 0) *reinterpret_cast<uint16_t*>(blk) = bq.d_bits;
-                            }
+                            const int t = tok0 + row;
+                            if (t < N)
+                                store_block_part(xq_dump + (static_cast<int64_t>(t) * nblk + b0 + bl) * Q8_0_BYTES, c4, bq);
                         }
                     }
                 }
-                __syncthreads();
             }
-
-            // ---------------- phase 2: blocks ascending, P column tiles per wave, in pairs
-            if (ct0 < mct) {
-                for (int bl = 0; bl < nb; ++bl) {
-                    const int b = b0 + bl;
-                    const bool more = b + 1 < nblk;                                // last block: harmless re-read
-                    const v4i afrag = lds_a[bl * 64 + lane];
-                    const float da_lane = lds_d[bl * 32 + j];                      // rows of both scale blocks
-#pragma unroll
-                    for (int pp = 0; pp < P / 2; ++pp) {
-                        v16i zero_i;
-                        v32f zero_f;
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) zero_i[r] = 0;
-#pragma unroll
-                        for (int r = 0; r < 32; ++r) zero_f[r] = 0.0f;
-                        // rows = activation rows (A operand), columns = weight rows (B operand);
-                        // the longest instruction goes first so the first settle can start earliest
-                        const float dw_lane = half_bits_to_float(static_cast<uint16_t>(wp[pp].d_bits));
-                        const v32f scale = __builtin_amdgcn_mfma_f32_32x32x1f32(da_lane, dw_lane, zero_f, 0, 0, 0);
-                        const v16i sum0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, wp[pp].q0, zero_i, 0, 0, 0);
-                        const v16i sum1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag, wp[pp].q1, zero_i, 0, 0, 0);
-                        // request block b+1 now that the MFMAs have read block b; it lands during the settle
-                        __builtin_amdgcn_sched_barrier(0);
-                        if (more) wp[pp].advance();
-                        wp[pp].load(W);
-                        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            acc[2 * pp][r] = __builtin_fmaf(static_cast<float>(sum0[r]), scale[r], acc[2 * pp][r]);
-                            acc[2 * pp + 1][r] = __builtin_fmaf(static_cast<float>(sum1[r]), scale[16 + r], acc[2 * pp + 1][r]);
-                        }
-                        if (DUMP && sums_dump) {
-#pragma unroll
-                            for (int r = 0; r < 16; ++r) {
-                                const int tok = tok0 + mfma32_row(r, lane);
-                                const int m0 = (ct0 + 2 * pp) * 32 + j;
-                                if (tok < N && m0 < M)
-                                    sums_dump[(static_cast<int64_t>(tok) * M + m0) * nblk + b] = sum0[r];
-                                if (tok < N && m0 + 32 < M)
-                                    sums_dump[(static_cast<int64_t>(tok) * M + m0 + 32) * nblk + b] = sum1[r];
-                            }
-                        }
-                    }
-                }
+            if (units <= wave && wave < npairs) {      // this wave had nothing to quantize
+                wp.init(g, 2 * wave, b0, lane);
+                wp.load(W);
             }
         }
+        PPML_TRACE_MARK(1);
+        __syncthreads();
+        PPML_TRACE_MARK(2);
 
-        // ---------------- phase 3: store
-        if (ct0 < mct) {
-            const bool full = (tok0 + TILE_TOK <= N) && (c_trans != 0);
-            if (full) {
-                float* crow = C + static_cast<int64_t>(tok0 + 4 * (lane >> 5)) * M + ct0 * 32 + j;
+        // ---------------- phase 2 + 3: one pair of column tiles at a time
+        for (int pr = wave; pr < npairs; pr += NW) {
+            const int ct = 2 * pr;
+            v16f acc0, acc1;
+            if (b0 == 0) {
 #pragma unroll
-                for (int p = 0; p < P; ++p) {
-                    if ((ct0 + p) * 32 + j < M) {
-#pragma unroll
-                        for (int r = 0; r < 16; ++r)
-                            __builtin_nontemporal_store(acc[p][r], crow + static_cast<int64_t>(8 * (r >> 2) + (r & 3)) * M + p * 32);
-                    }
-                }
+                for (int r = 0; r < 16; ++r) { acc0[r] = 0.0f; acc1[r] = 0.0f; }
             } else {
+                // later chunk of a long row: the running sums were parked in C
 #pragma unroll
-                for (int p = 0; p < P; ++p) {
-                    const int m = (ct0 + p) * 32 + j;
+                for (int r = 0; r < 16; ++r) {
+                    const int m = ct * 32 + mfma32_row(r, lane);
+                    acc0[r] = (tok < N && m < M) ? *out.at(tok, m) : 0.0f;
+                    acc1[r] = (tok < N && m + 32 < M) ? *out.at(tok, m + 32) : 0.0f;
+                }
+            }
+            for (int bl = 0; bl < nb; ++bl) {
+                const v4i afrag = lds_a[bl * 64 + lane];
+                const float da_lane = lds_d[bl * 32 + j];                  // columns of both scale blocks
+                v16i zero_i;
+                v32f zero_f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) zero_i[r] = 0;
+#pragma unroll
+                for (int r = 0; r < 32; ++r) zero_f[r] = 0.0f;
+                // the longest instruction goes first so the first settle can start earliest
+                const float dw_lane = half_bits_to_float(static_cast<uint16_t>(wp.d_bits));
+                const v32f scale = __builtin_amdgcn_mfma_f32_32x32x1f32(dw_lane, da_lane, zero_f, 0, 0, 0);
+                const v16i sum0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wp.q0, afrag, zero_i, 0, 0, 0);
+                const v16i sum1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wp.q1, afrag, zero_i, 0, 0, 0);
+                // request the next block (or the first block of this wave's next pair) now that the
+                // MFMAs have read this one; it lands during the settle
+                __builtin_amdgcn_sched_barrier(0);
+                if (bl + 1 < nb) wp.advance();
+                else if (pr + NW < npairs) wp.init(g, ct + 2 * NW, b0, lane);
+                wp.load(W);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    acc0[r] = __builtin_fmaf(static_cast<float>(sum0[r]), scale[r], acc0[r]);
+                    acc1[r] = __builtin_fmaf(static_cast<float>(sum1[r]), scale[16 + r], acc1[r]);
+                }
+                if (DUMP && sums_dump) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
-                        const int tok = tok0 + mfma32_row(r, lane);
-                        if (tok < N && m < M) {
-                            if (c_trans) C[static_cast<int64_t>(tok) * M + m] = acc[p][r];
-                            else         C[static_cast<int64_t>(m) * N + tok] = acc[p][r];
+                        const int m = ct * 32 + mfma32_row(r, lane);
+                        if (tok < N && m < M)
+                            sums_dump[(static_cast<int64_t>(tok) * M + m) * nblk + b0 + bl] = sum0[r];
+                        if (tok < N && m + 32 < M)
+                            sums_dump[(static_cast<int64_t>(tok) * M + m + 32) * nblk + b0 + bl] = sum1[r];
+                    }
+                }
+            }
+            // ---------------- phase 3: store the pair
+            if (tok < N) {
+                if (c_trans) {
+                    float* crow = C + static_cast<int64_t>(tok) * M + ct * 32 + 4 * hh;
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const int m = (ct + t) * 32 + 8 * q + 4 * hh;
+                            const v16f& a = t ? acc1 : acc0;
+                            if (m + 3 < M) {
+                                v4f v = {a[4 * q], a[4 * q + 1], a[4 * q + 2], a[4 * q + 3]};
+                                *reinterpret_cast<v4f_u*>(crow + t * 32 + 8 * q) = v;
+                            } else {
+#pragma unroll
+                                for (int c = 0; c < 4; ++c)
+                                    if (m + c < M) crow[t * 32 + 8 * q + c] = a[4 * q + c];
+                            }
                         }
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int m = ct * 32 + mfma32_row(r, lane);
+                        if (m < M) C[static_cast<int64_t>(m) * N + tok] = acc0[r];
+                        if (m + 32 < M) C[static_cast<int64_t>(m + 32) * N + tok] = acc1[r];
                     }
                 }
             }
         }
+        PPML_TRACE_MARK(3);
     }
+    PPML_TRACE_MARK(4);
 }
 
-template <int NW, int P, int WT>
+template <int NW, int WT>
 int launch_q8_linear(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
                      int relu, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
     const int kc = nblk < KC_MAX ? nblk : KC_MAX;
     const size_t lds = static_cast<size_t>(kc) * (1024 + 32 * sizeof(float));
     const dim3 grid((N + TILE_TOK - 1) / TILE_TOK), block(NW * 64);
     if (xq_dump || sums_dump)
-        hipLaunchKernelGGL((q8_linear_kernel<NW, P, WT, true>), grid, block, lds, stream,
-                           static_cast<const uint8_t*>(W), X, C, M, N, nblk, c_trans, relu,
+        hipLaunchKernelGGL((q8_linear_kernel<NW, WT, true>), grid, block, lds, stream,
+                           static_cast<const uint8_t*>(W), X, C, M, N, nblk, kc, c_trans, relu,
                            static_cast<uint8_t*>(xq_dump), sums_dump);
     else
-        hipLaunchKernelGGL((q8_linear_kernel<NW, P, WT, false>), grid, block, lds, stream,
-                           static_cast<const uint8_t*>(W), X, C, M, N, nblk, c_trans, relu,
+        hipLaunchKernelGGL((q8_linear_kernel<NW, WT, false>), grid, block, lds, stream,
+                           static_cast<const uint8_t*>(W), X, C, M, N, nblk, kc, c_trans, relu,
                            static_cast<uint8_t*>(nullptr), static_cast<int32_t*>(nullptr));
     return check_launch("q8_linear_kernel");
+}
+
+// ------------------------------------------------------------------------------------------
+// Weight-stationary form of the same linear, for Q8_0M weights small enough to live in registers
+// (M*K up to 256 Ki elements: every projection the reference quantizes, src/model/PPML.cpp:4434-4437).
+//
+// One work-group of 8 waves per CU walks over token tiles.  Wave w keeps the fragments and scales
+// of its TPW column tiles in VGPRs for the whole kernel, so the inner loop has no weight traffic at
+// all and the only vector-memory operations are the activation loads and the output stores:
+//
+//   loads of tile i+1 are issued before the MFMA work of tile i and its stores, so waiting for
+//   them never waits for a store (the VMEM counter retires in order), and the activation read,
+//   the arithmetic and the output write of neighbouring tiles overlap inside one work-group.
+//
+// Per column tile the blocks are walked in ascending order.  Each step issues the two MFMAs of
+// block b+1 -- v_mfma_i32_32x32x32_i8 for the exact block sums and v_mfma_f32_32x32x2_f32 for the
+// 32x32 scale products d_a[row]*d_w[col] (second K slot zero) -- and then settles block b on the
+// VALU, so the matrix pipe runs one block ahead of the VALU and neither waits for the other.  A
+// tile is stored as soon as its last block is settled, under the arithmetic of the next tile.
+// MFMA roles: A = activation rows, B = weight rows, so a store instruction writes two full
+// 128-byte lines.  LDS holds two quantized tiles so a single barrier per tile is enough.
+// ------------------------------------------------------------------------------------------
+// A value the optimizer cannot see through (always 1).  Branching on it puts the guarded code in a
+// basic block of its own: the fully unrolled MFMA steps below would otherwise all be issued up
+// front, since nothing orders them, and their result registers would spill.
+__device__ __forceinline__ int opaque_one() {
+    int one = 1;
+    asm volatile("" : "+s"(one));
+    return one;
+}
+
+template <int NW, int TPW, int NBLK, bool DUMP>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void q8_linear_ws_kernel(
+    const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
+    int M, int N, int ntiles, int relu,
+    uint8_t* __restrict__ xq_dump, int32_t* __restrict__ sums_dump) {
+    static_assert(NBLK % 2 == 0, "the quantizer stages blocks in pairs");
+    constexpr int K = NBLK * QK;
+    constexpr int NUNITS = 2 * NBLK;                   // (8 rows) x (2 blocks) each
+    constexpr int UPW = (NUNITS + NW - 1) / NW;        // units per wave
+    constexpr int STEPS = TPW * NBLK;
+    // LDS: two quantized activation tiles (fragments + scales) and this work-group's weight scales.
+    // Scale rows are 64 wide with lanes 32..63 zero: they feed K slot 1 of the scale MFMA.
+    extern __shared__ __attribute__((aligned(16))) uint8_t ws_lds[];
+    v4i (*lds_a)[NBLK * 64] = reinterpret_cast<v4i (*)[NBLK * 64]>(ws_lds);
+    float (*lds_d)[NBLK * 64] = reinterpret_cast<float (*)[NBLK * 64]>(ws_lds + 2 * NBLK * 1024);
+    float* lds_wd = reinterpret_cast<float*>(ws_lds + 2 * NBLK * 1024 + 2 * NBLK * 256);   // [NW*TPW][NBLK][64]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const int mct_pad = packed_tiles(M);
+    const int grp = lane >> 2, c4 = lane & 3;
+    const int urow = grp & 7, ublk = grp >> 3;
+    const __amdgpu_buffer_rsrc_t c_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(C, 0, N * M * 4, 0x00020000);   // raw dword buffer over C
+
+    auto load_tile = [&](int tile, v4f (&xv)[UPW][2]) {
+#pragma unroll
+        for (int s = 0; s < UPW; ++s) {
+            int u = wave + s * NW;
+            u = u < NUNITS ? u : NUNITS - 1;
+            const int bl = (u >> 2) * 2 + ublk;
+            int t = tile * TILE_TOK + (u & 3) * 8 + urow;
+            t = t < N ? t : N - 1;                     // rows past the end repeat the last row
+            const float* src = X + static_cast<int64_t>(t) * K + bl * QK + c4 * 8;
+            xv[s][0] = *reinterpret_cast<const v4f_u*>(src);
+            xv[s][1] = *reinterpret_cast<const v4f_u*>(src + 4);
+        }
+    };
+
+    // The first activation tile is requested before the weights: it has the longer way to come,
+    // and it keeps these loads older than at least a tile's worth of later memory operations on
+    // every path into the loop, which is what lets the wait in front of the quantizer skip them.
+    v4f xv[UPW][2];
+    int tile = blockIdx.x;
+    PPML_TRACE_MARK(0);
+    if (tile < ntiles) load_tile(tile, xv);
+
+    // ---- resident weights: fragments of TPW column tiles in registers, their scales in LDS
+    v4i wq[TPW][NBLK];
+    float* my_wd = lds_wd + static_cast<size_t>(wave) * TPW * NBLK * 64 + lane;
+    {
+        const uint16_t* dplane = reinterpret_cast<const uint16_t*>(W + static_cast<size_t>(mct_pad) * NBLK * 1024);
+#pragma unroll
+        for (int t = 0; t < TPW; ++t) {
+            int ct = wave * TPW + t;
+            ct = ct < mct_pad ? ct : mct_pad - 1;      // tiles past the end repeat the last one; never stored
+#pragma unroll
+            for (int b = 0; b < NBLK; ++b) {
+                wq[t][b] = *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(ct * NBLK + b) * 64 + lane) * 16);
+                const float d = half_bits_to_float(dplane[(ct * NBLK + b) * 32 + j]);
+                my_wd[(t * NBLK + b) * 64] = hh ? 0.0f : d;
+            }
+        }
+    }
+    for (int i = tid; i < 2 * NBLK * 64; i += NW * 64) (&lds_d[0][0])[i] = 0.0f;
+    __syncthreads();
+
+    // quantizes the tile held in xv into LDS buffer `buf`
+    auto quantize_tile = [&](int buf, int tok0, v4f (&xv)[UPW][2]) {
+#pragma unroll
+        for (int s = 0; s < UPW; ++s) {
+            const int u = wave + s * NW;
+            if (u >= NUNITS) break;                    // wave-uniform
+            const int row = (u & 3) * 8 + urow;
+            const int bl = (u >> 2) * 2 + ublk;
+            v4f x0 = xv[s][0], x1 = xv[s][1];
+            if (relu) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
+            }
+            const BlockQuant bq = quantize_block_lane(x0, x1);
+            uint2* dst = reinterpret_cast<uint2*>(lds_a[buf]) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
+            *dst = uint2{bq.q_lo, bq.q_hi};
+            if (c4 == 0) lds_d[buf][bl * 64 + row] = half_bits_to_float(bq.d_bits);
+            if (DUMP && xq_dump) {
+                const int t = tok0 + row;
+                if (t < N) store_block_part(xq_dump + (static_cast<int64_t>(t) * NBLK + bl) * Q8_0_BYTES, c4, bq);
+            }
+        }
+    };
+
+    if (tile < ntiles) quantize_tile(0, tile * TILE_TOK, xv);
+    __syncthreads();
+    PPML_TRACE_MARK(1);
+
+    // Step at which the next tile is quantized: late enough for its loads (issued at the top of the
+    // iteration) to have arrived, early enough that the output stores on both sides of it keep
+    // the write path busy through it.
+    constexpr int QSTEP = ((2 * STEPS / 3) / 2) * 2;
+
+    for (int it = 0; tile < ntiles; tile += gridDim.x, ++it) {
+        const int buf = it & 1;
+        const int tok0 = tile * TILE_TOK;
+        const int next = tile + static_cast<int>(gridDim.x);
+        const bool has_next = next < ntiles;
+        // ---------------- request the next tile; it arrives under this tile's arithmetic
+        if (has_next) load_tile(next, xv);
+        PPML_TRACE_MARK(2 + 4 * it);
+
+        // ---------------- MFMA one block ahead of the settle; tiles in turn, blocks ascending
+        v16i zero_i;
+        v16f zero_f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { zero_i[r] = 0; zero_f[r] = 0.0f; }
+        // Two result buffers used alternately: step st settles one while the MFMAs of step st+1
+        // fill the other.  Steps go in pairs so the buffers swap roles by name, not by copying.
+        v16i sum_a, sum_b;
+        v16f scl_a, scl_b;
+        v16f acc;
+        auto issue = [&](int st, v16i& sum, v16f& scl) {
+            const int t = st / NBLK, b = st % NBLK;
+            const v4i a = lds_a[buf][b * 64 + lane];
+            const float da = lds_d[buf][b * 64 + lane];
+            sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, wq[t][b], zero_i, 0, 0, 0);
+            scl = __builtin_amdgcn_mfma_f32_32x32x2f32(da, my_wd[(t * NBLK + b) * 64], zero_f, 0, 0, 0);
+        };
+        auto settle = [&](int st, const v16i& sum, const v16f& scl) {
+            const int t = st / NBLK, b = st % NBLK;
+            if (b == 0) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(static_cast<float>(sum[r]), scl[r], 0.0f);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(static_cast<float>(sum[r]), scl[r], acc[r]);
+            }
+            const int m = (wave * TPW + t) * 32 + j;   // this lane's output feature
+            if (DUMP && sums_dump) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int tok = tok0 + mfma32_row(r, lane);
+                    if (tok < N && m < M) sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b] = sum[r];
+                }
+            }
+            if (b == NBLK - 1) {
+                // The tile is complete: each half-wave store writes one full 128-byte line of a C
+                // row.  Buffer stores with a bounds-checked offset: lanes past the edge of C pass an
+                // offset beyond the buffer and are dropped by the hardware, so every wave issues
+                // exactly 16 stores here and the memory counter stays predictable.
+                const uint32_t base = (static_cast<uint32_t>(tok0 + 4 * hh) * M + m) * 4u;
+                const uint32_t out_of_range = 0xfffffff0u;
+                if (tok0 + TILE_TOK <= N) {
+                    const uint32_t b0 = m < M ? base : out_of_range;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[r]), c_rsrc, b0,
+                                                              (8 * (r >> 2) + (r & 3)) * M * 4, 0);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const bool ok = m < M && tok0 + mfma32_row(r, lane) < N;
+                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[r]), c_rsrc, ok ? base : out_of_range,
+                                                              (8 * (r >> 2) + (r & 3)) * M * 4, 0);
+                    }
+                }
+            }
+        };
+        static_assert(STEPS % 2 == 0, "steps are taken in pairs");
+        issue(0, sum_a, scl_a);
+#pragma unroll
+        for (int st = 0; st < STEPS; st += 2) {
+            if (!opaque_one()) continue;               // one basic block per pair of steps, see opaque_one()
+            if (st == QSTEP && has_next) {
+                quantize_tile(buf ^ 1, next * TILE_TOK, xv);
+                PPML_TRACE_MARK(3 + 4 * it);
+            }
+            issue(st + 1, sum_b, scl_b);
+            settle(st, sum_a, scl_a);
+            if (st + 2 < STEPS) issue(st + 2, sum_a, scl_a);
+            settle(st + 1, sum_b, scl_b);
+        }
+        PPML_TRACE_MARK(4 + 4 * it);
+        __syncthreads();                               // next tile quantized, this tile's LDS reads done
+        PPML_TRACE_MARK(5 + 4 * it);
+    }
+}
+
+int device_cu_count() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        return n;
+    }();
+    return cus;
+}
+
+template <int TPW, int NBLK>
+int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int relu,
+                        void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
+    constexpr int NW = 8;
+    const int ntiles = (N + TILE_TOK - 1) / TILE_TOK;
+    // one resident work-group per CU; with more tiles than CUs every work-group takes the same
+    // number of tiles (824 tiles on 256 CUs: 206 work-groups x 4 rather than 256 x 3 + 56 x 1)
+    const int cus = device_cu_count();
+    const int rounds = (ntiles + cus - 1) / cus;
+    const int wgs = (ntiles + rounds - 1) / rounds;
+    const dim3 grid(wgs), block(NW * 64);
+    constexpr size_t lds = 2 * NBLK * 1024 + 2 * NBLK * 256 + static_cast<size_t>(NW) * TPW * NBLK * 256;
+    if (lds > 64 * 1024) {
+        static const hipError_t attr_fast = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(&q8_linear_ws_kernel<NW, TPW, NBLK, false>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+        static const hipError_t attr_dump = hipFuncSetAttribute(
+            reinterpret_cast<const void*>(&q8_linear_ws_kernel<NW, TPW, NBLK, true>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+        if (attr_fast != hipSuccess || attr_dump != hipSuccess) {
+            (void)hipGetLastError();
+            return -1;                                  // fall back to the general kernel
+        }
+    }
+    if (xq_dump || sums_dump)
+        hipLaunchKernelGGL((q8_linear_ws_kernel<NW, TPW, NBLK, true>), grid, block, lds, stream,
+                           static_cast<const uint8_t*>(W), X, C, M, N, ntiles, relu,
+                           static_cast<uint8_t*>(xq_dump), sums_dump);
+    else
+        hipLaunchKernelGGL((q8_linear_ws_kernel<NW, TPW, NBLK, false>), grid, block, lds, stream,
+                           static_cast<const uint8_t*>(W), X, C, M, N, ntiles, relu,
+                           static_cast<uint8_t*>(nullptr), static_cast<int32_t*>(nullptr));
+    return check_launch("q8_linear_ws_kernel");
+}
+
+// returns -1 when the shape has no weight-stationary instance
+int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
+                     int relu, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
+    if (!c_trans) return -1;
+    if (static_cast<int64_t>(N) * M * 4 >= 0x7fff0000LL) return -1;   // the kernel addresses C with 32-bit byte offsets
+    const int mct = (M + 31) / 32;
+    const int tpw = (mct + 7) / 8;
+#define PPML_WS(TPW, NBLK) if (tpw == TPW && nblk == NBLK) return launch_q8_linear_ws<TPW, NBLK>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
+    PPML_WS(1, 4);  PPML_WS(2, 4);  PPML_WS(3, 4);  PPML_WS(4, 4);
+    PPML_WS(1, 8);  PPML_WS(2, 8);  PPML_WS(3, 8);
+    PPML_WS(1, 16);
+#undef PPML_WS
+    return -1;
 }
 
 template <int WT>
 int dispatch_q8_linear(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
                        int relu, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
-    const int mct = (M + 31) / 32;
-    // waves split the output columns; pick the shape with the fewest idle column tiles
-    if (mct <= 4)  return launch_q8_linear<2, 2, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
-    if (mct <= 8)  return launch_q8_linear<4, 2, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
-    if (mct <= 16) return launch_q8_linear<4, 4, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
-    return launch_q8_linear<4, 6, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
+    // four waves share a token tile; with at most two pairs of column tiles two waves are enough
+    if (M <= 128) return launch_q8_linear<2, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
+    return launch_q8_linear<4, WT>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, stream);
 }
 
 }  // namespace
@@ -470,7 +808,7 @@ using namespace ppmlhip;
 extern "C" int quantize_rows_q8_0_hip(const float* x, void* y, int64_t ne, ppml_hip_stream_t stream) {
     if (!x || !y || ne <= 0 || (ne % QK) != 0) { set_error("quantize_rows_q8_0_hip: bad arguments (ne=%lld)", (long long)ne); return RC_BAD_ARGS; }
     const int64_t nblocks = ne / QK;
-    const int64_t threads = nblocks * 8;
+    const int64_t threads = nblocks * 4;
     const unsigned grid = static_cast<unsigned>((threads + 255) / 256);
     hipLaunchKernelGGL(quantize_rows_q8_0_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
                        x, static_cast<uint8_t*>(y), nblocks);
@@ -521,7 +859,11 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
         case PPML_WTYPE_Q8_0:  return dispatch_q8_linear<PPML_WTYPE_Q8_0>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_1:  return dispatch_q8_linear<PPML_WTYPE_Q8_1>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0R: return dispatch_q8_linear<PPML_WTYPE_Q8_0R>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
-        case PPML_WTYPE_Q8_0M: return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
+        case PPML_WTYPE_Q8_0M: {
+            const int rc = try_q8_linear_ws(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
+            if (rc >= 0) return rc;
+            return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
+        }
         default: set_error("mul_mat_q8_hip: unsupported wtype %d", wtype); return RC_WTYPE;
     }
 }

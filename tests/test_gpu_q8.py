@@ -109,12 +109,25 @@ SHAPES = [
 ]
 
 
+SHAPES += [
+    # shapes with a weight-stationary instance when the weight is packed (K/32 in {4,8,16})
+    (300, 128, 512),      # pair feed-forward up-projection, ragged last token tile
+    (200, 512, 128),      # pair feed-forward down-projection
+    (1000, 256, 768),     # MSA QKV projection: more token tiles than one pass of work-groups on a small grid
+    (77, 256, 700),       # output features not a multiple of 32 (and not of 4 at the edge tile)
+    (9000, 128, 100),     # more token tiles than CUs: the persistent loop and its double buffer
+]
+
+
+@pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("N,K,M", SHAPES)
-def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M):
+def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packed):
     x, w = _inputs(N + K + M, N, K, M)
     wq = oracle.quantize_q8_0(w)
     xq_want = oracle.quantize_q8_0(x)
     W = ops.Q8Weight(_dev(wq.reshape(-1)), M, K, ops.WTYPE_Q8_0)
+    if packed:
+        W = W.pack()
     out, xq, sums = ops.mul_mat_q8(W, _dev(x), c_trans=1, dump=True)
     out, xq, sums = out.cpu().numpy(), xq.cpu().numpy(), sums.cpu().numpy()
     assert (xq == xq_want).all(), "activation blocks differ from quantize_q8_0_host"
