@@ -26,8 +26,8 @@ INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA, published
 FP32_MFMA_PEAK_TFLOPS = 157.3
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE
-# scaled by the same counters on a copy kernel of known size); None until measured.
-MEASURED_TRAFFIC_BYTES = None
+# scaled by the same counters on a 1 GiB copy: factors 2.000 and 1.000).
+MEASURED_TRAFFIC_BYTES = 109_890_000   # 28.89 MB read + 81.00 MB written per launch
 
 
 def q8_bytes(rows, K, N):
@@ -42,6 +42,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configured shapes")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 1 GiB device copy, the kernel of known size against which the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (no collectives, no sharding); "
@@ -185,6 +188,14 @@ def main() -> int:
         steps, warm = 10, 3
         f32_case(opm, (2 * 256 * 12288 + 12288 * 12288) * 4, 2.0 * 12288 * 12288 * 256, "opm_dense_12288x256x12288")
         out["extra"] = extra
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_(generator=gen)   # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["copy_calibration"] = {"bytes_read": src.numel() * 4, "bytes_written": dst.numel() * 4, "launches": 5}
 
     print(json.dumps(out))
     return 0
