@@ -1,0 +1,57 @@
+/*
+ * ppml_hip_backend.h -- C ABI over the C++ host side (ppml_hip_backend.hpp): build a few tensor
+ * nodes, bind device memory, run them through the backend's graph executor.
+ *
+ * This is the shape the reference's own tests use (tests/test_cuda.cpp:39-51, 108-110: make device
+ * leaves, make one node, graph_compute, synchronize, copy back), exposed without C++ types so that
+ * tests and other languages can drive the executor.  It has no counterpart among the reference's
+ * launcher functions; those are in ppml_hip.h.
+ *
+ * Status values returned by graph_compute / pack_weight are the reference's
+ * enum class Status {SUCCESS = 0, ALLOC_FAILED, NOT_SUPPORTED, ABORTED} (include/ppml/Backend.h:168-173).
+ */
+#ifndef PPML_HIP_BACKEND_H
+#define PPML_HIP_BACKEND_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ppml_hip_backend ppml_hip_backend;
+typedef struct ppml_hip_tensor ppml_hip_tensor;
+
+ppml_hip_backend *ppml_hip_backend_create(int device);
+void ppml_hip_backend_destroy(ppml_hip_backend *b);
+const char *ppml_hip_backend_name(const ppml_hip_backend *b);
+const char *ppml_hip_backend_last_error(const ppml_hip_backend *b);
+int ppml_hip_backend_priority(const ppml_hip_backend *b);
+void ppml_hip_backend_synchronize(ppml_hip_backend *b);
+
+/* op / type are the reference's tensor_op / tensor_type values; dims[0] is the innermost dimension */
+ppml_hip_tensor *ppml_hip_tensor_create(int op, int type, int ndim, const int64_t *dims);
+void ppml_hip_tensor_destroy(ppml_hip_tensor *t);
+void ppml_hip_tensor_set_src(ppml_hip_tensor *t, int slot, ppml_hip_tensor *src);
+void ppml_hip_tensor_set_data(ppml_hip_tensor *t, void *device_ptr);
+void ppml_hip_tensor_set_view(ppml_hip_tensor *t, ppml_hip_tensor *view_src, size_t byte_offset);
+void ppml_hip_tensor_set_param(ppml_hip_tensor *t, int index, float value);
+size_t ppml_hip_tensor_nbytes(const ppml_hip_tensor *t);
+int ppml_hip_tensor_type(const ppml_hip_tensor *t);
+/* allocate device storage through the backend's BufferType and copy host data in / out */
+int ppml_hip_tensor_upload(ppml_hip_backend *b, ppml_hip_tensor *t, const void *host, size_t nbytes);
+int ppml_hip_tensor_download(ppml_hip_backend *b, const ppml_hip_tensor *t, void *host, size_t nbytes);
+
+/* The rule is a function of the node alone: b may be NULL, which lets a scheduler on a host without
+ * a device ask the question (Backend::supports_op, include/ppml/Backend.h:571). */
+int ppml_hip_backend_supports_op(const ppml_hip_backend *b, const ppml_hip_tensor *node);
+/* 1: a scheduler owns allocation, graph_compute allocates nothing (Backend.h skip_alloc_) */
+void ppml_hip_backend_set_skip_alloc(ppml_hip_backend *b, int on);
+int ppml_hip_backend_graph_compute(ppml_hip_backend *b, ppml_hip_tensor **nodes, int n);
+int ppml_hip_backend_pack_weight(ppml_hip_backend *b, ppml_hip_tensor *weight);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,146 @@
+// ppml_hip_backend.hpp -- C++ host side of the gfx950 backend, above the C ABI of ppml_hip.h.
+//
+// It mirrors the part of the reference's backend plug-in interface that the matrix-multiplication
+// path goes through (include/ppml/Backend.h:550-605 `Backend`, 252-329 `BufferType`/`Buffer`,
+// 168-173 `Status`) on a field-compatible subset of the reference's tensor node
+// (include/ppml/Tensor.h:443-464: op, type, dims, src[], data, buffer, view_src, op_params), so that
+// the executor logic -- which nodes are skipped, how views are resolved, what is rejected, how
+// failures map to Status -- can be exercised without the rest of the reference.  A maintainer of
+// the reference needs only the C ABI; this class shows what the adapter around it does.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+namespace ppmlhip {
+
+// numeric values of the reference's enums (include/ppml/Tensor.h:35-64 and 136-278)
+enum TensorType : int {
+    TENSOR_TYPE_F32 = 0,
+    TENSOR_TYPE_F16 = 1,
+    TENSOR_TYPE_Q8_0 = 8,
+    TENSOR_TYPE_Q8_1 = 9,
+    TENSOR_TYPE_Q8_0R = 19,
+    TENSOR_TYPE_Q8_0M = 64,   // this backend's MFMA-fragment layout; never leaves the device
+};
+
+enum TensorOp : int {
+    OP_NONE = 0,
+    OP_MUL_MAT = 30,
+    OP_OUT_PROD = 32,
+    OP_SCALE = 33,
+    OP_RESHAPE = 37,
+    OP_VIEW = 38,
+    OP_OUTER_PROD_MEAN = 102,
+};
+
+// include/ppml/Backend.h:168-173
+enum class Status : int { SUCCESS = 0, ALLOC_FAILED, NOT_SUPPORTED, ABORTED };
+
+// include/ppml/Tensor.h:72-133
+bool is_quantized_type(int t);
+bool is_quantized_type_supported(int t);
+int quant_block_elems(int t);
+size_t quant_block_bytes(int t);
+
+class Buffer;
+
+// The fields of the reference's tensor node that this path reads.
+struct Tensor {
+    int op = OP_NONE;
+    int type = TENSOR_TYPE_F32;
+    int ndim = 0;
+    int64_t dims[4] = {1, 1, 1, 1};       // dims[0] innermost
+    Tensor* src[10] = {nullptr};
+    void* data = nullptr;
+    Buffer* buffer = nullptr;
+    size_t buffer_offs = 0;
+    Tensor* view_src = nullptr;           // OP_VIEW / OP_RESHAPE share their source's storage
+    size_t view_offs = 0;
+    float op_params[16] = {0};
+
+    int64_t numel() const { return dims[0] * dims[1] * dims[2] * dims[3]; }
+    // include/ppml/Tensor.h:327-352
+    bool quant_shape_valid() const;
+    size_t nbytes() const;
+};
+
+// include/ppml/Backend.h:252-272
+class BufferType {
+public:
+    const char* get_name() const { return "HIP"; }
+    void* alloc(size_t size) const;
+    void free(void* p) const;
+    size_t get_alignment() const { return 128; }
+    size_t get_alloc_size(const Tensor* t) const { return t->nbytes(); }
+    bool is_host() const { return false; }
+    static const BufferType* instance();
+};
+
+// include/ppml/Backend.h:275-329, 355-432 (device semantics: blocking copies)
+class Buffer {
+public:
+    Buffer(const BufferType* type, size_t size);
+    ~Buffer();
+    Buffer(const Buffer&) = delete;
+    Buffer& operator=(const Buffer&) = delete;
+    void* data() const { return base_; }
+    size_t size() const { return size_; }
+    bool is_host() const { return false; }
+    bool set_tensor(Tensor* t, const void* host, size_t offs, size_t n);
+    bool get_tensor(const Tensor* t, void* host, size_t offs, size_t n) const;
+    bool memset_tensor(Tensor* t, int value, size_t offs, size_t n);
+    bool contains(const void* p, size_t n) const;
+
+private:
+    const BufferType* type_;
+    void* base_ = nullptr;
+    size_t size_ = 0;
+};
+
+using ComputeGraph = std::vector<Tensor*>;   // nodes in evaluation order
+
+// src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-416 (OP_OUTER_PROD_MEAN);
+// a function of the node alone, so it can be asked without a device
+bool node_supported(const Tensor* node);
+
+// include/ppml/Backend.h:550-605; executor obligations of src/backend/CUDABackend.cpp:708-1086
+class HipBackend {
+public:
+    explicit HipBackend(int device);
+    ~HipBackend();
+    const char* get_name() const { return "HIP-gfx950"; }
+    Status graph_compute(ComputeGraph* graph);
+    void synchronize();
+    bool supports_op(const Tensor* node) const { return node_supported(node); }
+    const BufferType* buffer_type() const { return BufferType::instance(); }
+    bool supports_buffer_type(const BufferType* t) const { return t == BufferType::instance(); }
+    int priority() const { return 1; }                   // include/ppml/Backend.h:949
+    bool vram_budgeted() const { return true; }
+    bool skip_alloc() const { return skip_alloc_; }
+    void set_skip_alloc(bool v) { skip_alloc_ = v; }
+    const std::string& last_error() const { return error_; }
+
+    // Once-per-weight step of src/model/PPML.cpp:4504-4528: turns a Q8_0 / Q8_1 / Q8_0R weight node
+    // into the MFMA-fragment layout in a buffer owned by this backend.
+    Status pack_weight(Tensor* weight);
+
+private:
+    Status dispatch_node(Tensor* node);                  // src/backend/CUDAKernels.cpp:351-, 717-847
+    Status kernel_mul_mat(Tensor* node);
+    Status kernel_out_prod(Tensor* node);
+    Status kernel_outer_prod_mean(Tensor* node);
+    bool resolve_views(Tensor* node);                    // src/backend/CUDABackend.cpp:800-819
+    bool device_pointer_ok(const Tensor* t) const;       // src/backend/CUDABackend.cpp:894-973
+    Status fail(Status s, const std::string& why);
+
+    int device_;
+    bool skip_alloc_ = false;
+    std::string error_;
+    std::vector<std::unique_ptr<Buffer>> owned_;         // node outputs allocated here, packed weights
+};
+
+}  // namespace ppmlhip

@@ -34,6 +34,30 @@ SIGNATURES = {
     "ppml_hip_mulmat_stats": (_i, [C.POINTER(_i64), _i]),
 }
 
+# every symbol include/ppml_hip_backend.h declares (the executor driver above the launchers)
+BACKEND_SIGNATURES = {
+    "ppml_hip_backend_create": (_vp, [_i]),
+    "ppml_hip_backend_destroy": (None, [_vp]),
+    "ppml_hip_backend_name": (C.c_char_p, [_vp]),
+    "ppml_hip_backend_last_error": (C.c_char_p, [_vp]),
+    "ppml_hip_backend_priority": (_i, [_vp]),
+    "ppml_hip_backend_synchronize": (None, [_vp]),
+    "ppml_hip_tensor_create": (_vp, [_i, _i, _i, C.POINTER(_i64)]),
+    "ppml_hip_tensor_destroy": (None, [_vp]),
+    "ppml_hip_tensor_set_src": (None, [_vp, _i, _vp]),
+    "ppml_hip_tensor_set_data": (None, [_vp, _vp]),
+    "ppml_hip_tensor_set_view": (None, [_vp, _vp, C.c_size_t]),
+    "ppml_hip_tensor_set_param": (None, [_vp, _i, _f]),
+    "ppml_hip_tensor_nbytes": (C.c_size_t, [_vp]),
+    "ppml_hip_tensor_type": (_i, [_vp]),
+    "ppml_hip_tensor_upload": (_i, [_vp, _vp, _vp, C.c_size_t]),
+    "ppml_hip_tensor_download": (_i, [_vp, _vp, _vp, C.c_size_t]),
+    "ppml_hip_backend_supports_op": (_i, [_vp, _vp]),
+    "ppml_hip_backend_set_skip_alloc": (None, [_vp, _i]),
+    "ppml_hip_backend_graph_compute": (_i, [_vp, C.POINTER(_vp), _i]),
+    "ppml_hip_backend_pack_weight": (_i, [_vp, _vp]),
+}
+
 _lib = None
 
 
@@ -54,7 +78,7 @@ def load() -> C.CDLL:
             f"{LIB_PATH} is missing: build it with `make -C proteinpredictmachinelearning_amd/csrc` "
             "(or __graft_entry__.build()); this backend has no CPU fallback")
     lib = C.CDLL(LIB_PATH)
-    for name, (res, args) in SIGNATURES.items():
+    for name, (res, args) in list(SIGNATURES.items()) + list(BACKEND_SIGNATURES.items()):
         fn = getattr(lib, name)          # AttributeError if the library lacks a declared symbol
         fn.restype = res
         fn.argtypes = args

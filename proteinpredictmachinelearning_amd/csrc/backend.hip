@@ -1,0 +1,461 @@
+// Host side of the gfx950 backend: the executor that walks a list of tensor nodes and hands the
+// matrix-multiplication ops to the launchers of ppml_hip.h.  No kernels in this file.
+//
+// What it mirrors of the reference:
+//   supports_op      src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-416 (OP_OUTER_PROD_MEAN)
+//   graph_compute    src/backend/CUDABackend.cpp:708-1086 (skip no-op nodes, resolve view sources,
+//                    refuse host / out-of-buffer pointers, dispatch, launch error -> ABORTED)
+//   node -> launcher src/backend/CUDAKernels.cpp:717-847 (mul_mat), 1537-1565 (out_prod), 1204-1221 (outer_prod_mean)
+//
+// Two deliberate differences, both on failure paths only:
+//   * the reference's quantized mul_mat prints and returns normally when the launcher fails, so the
+//     node is silently left unwritten (CUDAKernels.cpp:735-763); here every launcher failure ends
+//     graph_compute with NOT_SUPPORTED (bad arguments) or ABORTED (device error);
+//   * a view source is bound to root data PLUS the accumulated view offsets; the reference binds the
+//     root pointer itself (CUDABackend.cpp:812-819) and relies on its allocator having bound offset
+//     views beforehand.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <new>
+
+#include "../../include/ppml_hip.h"
+#include "../../include/ppml_hip_backend.h"
+#include "../../include/ppml_hip_backend.hpp"
+
+namespace ppmlhip {
+
+// ------------------------------------------------------------------------------------------------
+// type helpers (include/ppml/Tensor.h:72-133)
+bool is_quantized_type(int t) {
+    return t == TENSOR_TYPE_Q8_0 || t == TENSOR_TYPE_Q8_1 || t == TENSOR_TYPE_Q8_0R || t == TENSOR_TYPE_Q8_0M;
+}
+bool is_quantized_type_supported(int t) { return is_quantized_type(t); }
+int quant_block_elems(int t) { return is_quantized_type(t) ? 32 : 1; }
+size_t quant_block_bytes(int t) {
+    switch (t) {
+        case TENSOR_TYPE_Q8_0:
+        case TENSOR_TYPE_Q8_0R:
+        case TENSOR_TYPE_Q8_0M: return 34;
+        case TENSOR_TYPE_Q8_1: return 36;
+        case TENSOR_TYPE_F16: return 2;
+        default: return 4;
+    }
+}
+
+bool Tensor::quant_shape_valid() const {
+    if (!is_quantized_type(type)) return true;
+    return ndim >= 1 && dims[0] > 0 && dims[0] % quant_block_elems(type) == 0;
+}
+
+size_t Tensor::nbytes() const {
+    const int64_t n = numel();
+    if (n <= 0) return 0;
+    if (type == TENSOR_TYPE_Q8_0M) {
+        if (!quant_shape_valid()) return 0;
+        return q8_weight_packed_bytes_hip(static_cast<int>(n / dims[0]), static_cast<int>(dims[0]));
+    }
+    if (is_quantized_type(type)) {
+        if (!quant_shape_valid()) return 0;
+        return static_cast<size_t>(n / quant_block_elems(type)) * quant_block_bytes(type);
+    }
+    return static_cast<size_t>(n) * quant_block_bytes(type);
+}
+
+// ------------------------------------------------------------------------------------------------
+// BufferType / Buffer (include/ppml/Backend.h:252-329)
+void* BufferType::alloc(size_t size) const {
+    void* p = nullptr;
+    if (size == 0) size = get_alignment();
+    if (hipMalloc(&p, size) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    return p;
+}
+void BufferType::free(void* p) const {
+    if (p) (void)hipFree(p);
+}
+const BufferType* BufferType::instance() {
+    static const BufferType t;
+    return &t;
+}
+
+Buffer::Buffer(const BufferType* type, size_t size) : type_(type), size_(size) { base_ = type_->alloc(size); }
+Buffer::~Buffer() { type_->free(base_); }
+
+bool Buffer::contains(const void* p, size_t n) const {
+    const char* b = static_cast<const char*>(base_);
+    const char* q = static_cast<const char*>(p);
+    return base_ && q >= b && n <= size_ && q + n <= b + size_;
+}
+bool Buffer::set_tensor(Tensor* t, const void* host, size_t offs, size_t n) {
+    if (!t || !t->data || !host || !contains(static_cast<char*>(t->data) + offs, n)) return false;
+    return hipMemcpy(static_cast<char*>(t->data) + offs, host, n, hipMemcpyHostToDevice) == hipSuccess;
+}
+bool Buffer::get_tensor(const Tensor* t, void* host, size_t offs, size_t n) const {
+    if (!t || !t->data || !host || !contains(static_cast<const char*>(t->data) + offs, n)) return false;
+    return hipMemcpy(host, static_cast<const char*>(t->data) + offs, n, hipMemcpyDeviceToHost) == hipSuccess;
+}
+bool Buffer::memset_tensor(Tensor* t, int value, size_t offs, size_t n) {
+    if (!t || !t->data || !contains(static_cast<char*>(t->data) + offs, n)) return false;
+    return hipMemset(static_cast<char*>(t->data) + offs, value, n) == hipSuccess;
+}
+
+// ------------------------------------------------------------------------------------------------
+HipBackend::HipBackend(int device) : device_(device) {
+    if (ppml_hip_init(device) != 0) error_ = ppml_hip_last_error();
+}
+HipBackend::~HipBackend() {
+    (void)hipSetDevice(device_);
+    (void)hipDeviceSynchronize();
+}
+
+Status HipBackend::fail(Status s, const std::string& why) {
+    error_ = why;
+    return s;
+}
+
+void HipBackend::synchronize() {
+    (void)hipSetDevice(device_);
+    (void)hipDeviceSynchronize();
+}
+
+bool node_supported(const Tensor* node) {
+    if (!node) return false;
+    const Tensor* src0 = node->src[0];
+    const Tensor* src1 = node->src[1];
+    switch (node->op) {
+        case OP_NONE:
+        case OP_VIEW:
+        case OP_RESHAPE:
+            return true;
+        case OP_MUL_MAT: {
+            if (!src1) return true;
+            // the bias epilogue exists on the f32 path only
+            if (node->src[2] && ((src0 && src0->type != TENSOR_TYPE_F32) || src1->type != TENSOR_TYPE_F32)) return false;
+            if (is_quantized_type(src1->type) || (src0 && is_quantized_type(src0->type))) {
+                if (!src0) return false;
+                const bool q0 = is_quantized_type(src0->type), q1 = is_quantized_type(src1->type);
+                if (q0 == q1) return false;     // exactly one side is the quantized weight
+                const Tensor* w = q0 ? src0 : src1;
+                const Tensor* a = q0 ? src1 : src0;
+                return w->quant_shape_valid() && is_quantized_type_supported(w->type) &&
+                       a->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32;
+            }
+            // F16 x F16 is served by the reference's own kernels, not by this backend
+            return src0 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
+                   node->type == TENSOR_TYPE_F32;
+        }
+        case OP_OUT_PROD:
+            return src0 && src1 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
+                   node->type == TENSOR_TYPE_F32;
+        case OP_OUTER_PROD_MEAN:
+            if (!src0 || !src1) return false;
+            if (src0->type != TENSOR_TYPE_F32 || src1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32) return false;
+            return src0->ndim == 4 && src1->ndim == 4 && src0->dims[0] > 0 && src0->dims[2] > 0;
+        default:
+            return false;
+    }
+}
+
+// Follows view_src (or, for OP_VIEW / OP_RESHAPE nodes built with only src[0] set, src[0]) to the
+// tensor that carries the storage and binds every unbound source of `node` to it.
+bool HipBackend::resolve_views(Tensor* node) {
+    for (Tensor* src : node->src) {
+        if (!src || src->data) continue;
+        Tensor* r = src;
+        size_t offs = 0;
+        for (int guard = 0; guard < 64; ++guard) {
+            Tensor* nxt = r->view_src;
+            if (!nxt && (r->op == OP_VIEW || r->op == OP_RESHAPE)) nxt = r->src[0];
+            if (!nxt) break;
+            offs += r->view_offs;
+            r = nxt;
+        }
+        if (r == src || !r->data) continue;
+        src->data = static_cast<char*>(r->data) + offs;
+        src->buffer = r->buffer;
+        src->buffer_offs = r->buffer_offs + offs;
+    }
+    return true;
+}
+
+bool HipBackend::device_pointer_ok(const Tensor* t) const {
+    if (!t || !t->data) return false;
+    hipPointerAttribute_t attr{};
+    if (hipPointerGetAttributes(&attr, t->data) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    if (attr.type != hipMemoryTypeDevice && attr.type != hipMemoryTypeManaged) return false;
+    if (t->buffer) {
+        const size_t need = t->nbytes();
+        if (!t->buffer->contains(t->data, need)) return false;
+    }
+    return true;
+}
+
+static Status status_of_rc(int rc) {
+    if (rc == 0) return Status::SUCCESS;
+    if (rc == 3) return Status::ALLOC_FAILED;
+    if (rc == 6 || rc == 7) return Status::ABORTED;
+    return Status::NOT_SUPPORTED;
+}
+
+Status HipBackend::kernel_mul_mat(Tensor* node) {
+    Tensor* s0 = node->src[0];
+    Tensor* s1 = node->src[1];
+    if (!s0 || !s1) return fail(Status::NOT_SUPPORTED, "mul_mat: missing source");
+    const int64_t M = node->dims[1], N = node->dims[0], K = s0->dims[0];
+    if (s1->dims[0] != K) return fail(Status::NOT_SUPPORTED, "mul_mat: inner dimensions differ");
+    if (s0->numel() != M * K || s1->numel() != N * K)
+        return fail(Status::NOT_SUPPORTED, "mul_mat: source shapes do not match the node's [N, M]");
+    const float* bias = node->src[2] ? static_cast<const float*>(node->src[2]->data) : nullptr;
+    if (node->src[2] && node->src[2]->numel() != N) return fail(Status::NOT_SUPPORTED, "mul_mat: bias length is not N");
+
+    const bool q0 = is_quantized_type(s0->type), q1 = is_quantized_type(s1->type);
+    int rc;
+    if (q0 || q1) {
+        if (bias) return fail(Status::NOT_SUPPORTED, "mul_mat: the quantized path has no bias epilogue");
+        if (q0 == q1) return fail(Status::NOT_SUPPORTED, "mul_mat: exactly one side may be quantized");
+        Tensor* w = q0 ? s0 : s1;
+        Tensor* a = q0 ? s1 : s0;
+        if (!w->quant_shape_valid() || a->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32 || K % 32 != 0)
+            return fail(Status::NOT_SUPPORTED, "mul_mat: unsupported quantized combination");
+        const int wtype = w->type == TENSOR_TYPE_Q8_1 ? PPML_WTYPE_Q8_1
+                        : w->type == TENSOR_TYPE_Q8_0R ? PPML_WTYPE_Q8_0R
+                        : w->type == TENSOR_TYPE_Q8_0M ? PPML_WTYPE_Q8_0M : PPML_WTYPE_Q8_0;
+        // weight rows are the out features: with the weight in src0 they index the node's dims[1]
+        const int64_t Mq = q0 ? M : N, Nq = q0 ? N : M;
+        const int c_trans = q0 ? 0 : 1;
+        int path = 0;
+        rc = mul_mat_q8_hip(w->data, static_cast<const float*>(a->data), static_cast<float*>(node->data),
+                            static_cast<int>(Mq), static_cast<int>(Nq), static_cast<int>(K), wtype, c_trans, &path,
+                            nullptr);
+    } else {
+        if (s0->type != TENSOR_TYPE_F32 || s1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32)
+            return fail(Status::NOT_SUPPORTED, "mul_mat: only F32 x F32 -> F32 besides the quantized path");
+        rc = mul_mat_hip(static_cast<const float*>(s0->data), static_cast<const float*>(s1->data),
+                         static_cast<float*>(node->data), static_cast<int>(M), static_cast<int>(K),
+                         static_cast<int>(N), bias, nullptr);
+    }
+    if (rc != 0) return fail(status_of_rc(rc), std::string("mul_mat: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
+static inline int64_t dim_or_1(const Tensor* t, int i) { return t->ndim > i ? t->dims[i] : 1; }
+
+Status HipBackend::kernel_out_prod(Tensor* node) {
+    const Tensor* a = node->src[0];
+    const Tensor* b = node->src[1];
+    if (!a || !b) return fail(Status::NOT_SUPPORTED, "out_prod: missing source");
+    // the reference clears dst first and accumulates; the launcher overwrites dst instead
+    const int rc = out_prod_hip(static_cast<const float*>(a->data), static_cast<const float*>(b->data),
+                                static_cast<float*>(node->data),
+                                a->dims[0], a->dims[1], dim_or_1(a, 2), dim_or_1(a, 3),
+                                b->dims[0], b->dims[1], dim_or_1(b, 2), dim_or_1(b, 3),
+                                node->dims[0], node->dims[1], dim_or_1(node, 2), dim_or_1(node, 3), nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("out_prod: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
+Status HipBackend::kernel_outer_prod_mean(Tensor* node) {
+    const Tensor* l = node->src[0];
+    const Tensor* r = node->src[1];
+    if (!l || !r || !l->data || !r->data || !node->data) return fail(Status::NOT_SUPPORTED, "outer_prod_mean: unbound tensor");
+    const int64_t D = l->dims[0], L = l->dims[1], N = l->dims[2], B = l->dims[3];
+    if (N <= 0) return fail(Status::NOT_SUPPORTED, "outer_prod_mean: N must be positive");
+    if (r->numel() != l->numel() || node->numel() != D * D * L * L * B)
+        return fail(Status::NOT_SUPPORTED, "outer_prod_mean: shapes are not [D,L,N,B] x [D,L,N,B] -> [D*D,L,L,B]");
+    const int rc = outer_prod_mean_hip(static_cast<const float*>(l->data), static_cast<const float*>(r->data),
+                                       static_cast<float*>(node->data), D, L, N, B, 1.0f / static_cast<float>(N),
+                                       nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("outer_prod_mean: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
+Status HipBackend::dispatch_node(Tensor* node) {
+    switch (node->op) {
+        case OP_MUL_MAT: return kernel_mul_mat(node);
+        case OP_OUT_PROD: return kernel_out_prod(node);
+        case OP_OUTER_PROD_MEAN: return kernel_outer_prod_mean(node);
+        default: return fail(Status::NOT_SUPPORTED, "no kernel for op " + std::to_string(node->op));
+    }
+}
+
+Status HipBackend::graph_compute(ComputeGraph* graph) {
+    if (!graph) return fail(Status::NOT_SUPPORTED, "null graph");
+    if (hipSetDevice(device_) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(Status::ABORTED, "cannot select device " + std::to_string(device_));
+    }
+    error_.clear();
+    int index = -1;
+    for (Tensor* node : *graph) {
+        ++index;
+        if (!node) return fail(Status::NOT_SUPPORTED, "null node " + std::to_string(index));
+        if (node->op == OP_NONE || node->op == OP_VIEW || node->op == OP_RESHAPE) continue;
+        resolve_views(node);
+
+        // single-backend mode: outputs nobody allocated get their own device buffer
+        if (!skip_alloc_ && !node->data) {
+            const size_t need = node->nbytes();
+            auto buf = std::make_unique<Buffer>(buffer_type(), need);
+            if (!buf->data()) return fail(Status::ALLOC_FAILED, "cannot allocate " + std::to_string(need) + " bytes for node " + std::to_string(index));
+            node->data = buf->data();
+            node->buffer = buf.get();
+            node->buffer_offs = 0;
+            owned_.push_back(std::move(buf));
+        }
+        // no other backend to fall back to: an unsupported node ends the graph instead of being skipped
+        if (!supports_op(node))
+            return fail(Status::NOT_SUPPORTED, "op " + std::to_string(node->op) + " (node " + std::to_string(index) + ") is not supported");
+
+        if (!device_pointer_ok(node))
+            return fail(Status::NOT_SUPPORTED, "node " + std::to_string(index) + ": output is not device memory inside its buffer");
+        for (int j = 0; j < 10; ++j) {
+            if (node->src[j] && !device_pointer_ok(node->src[j]))
+                return fail(Status::NOT_SUPPORTED, "node " + std::to_string(index) + ": src" + std::to_string(j) +
+                                                    " is not device memory inside its buffer");
+        }
+
+        const Status st = dispatch_node(node);
+        if (st != Status::SUCCESS) return st;
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess)
+            return fail(Status::ABORTED, "launch failed at op " + std::to_string(node->op) + " (node " +
+                                         std::to_string(index) + "): " + hipGetErrorString(e));
+    }
+    return Status::SUCCESS;
+}
+
+Status HipBackend::pack_weight(Tensor* w) {
+    if (!w || !w->data) return fail(Status::NOT_SUPPORTED, "pack_weight: unbound tensor");
+    if (w->type == TENSOR_TYPE_Q8_0M) return Status::SUCCESS;
+    if (!is_quantized_type(w->type) || !w->quant_shape_valid())
+        return fail(Status::NOT_SUPPORTED, "pack_weight: not a Q8 weight with K a multiple of 32");
+    if (hipSetDevice(device_) != hipSuccess) return fail(Status::ABORTED, "cannot select device");
+    const int64_t K = w->dims[0], M = w->numel() / K;
+    const int wtype = w->type == TENSOR_TYPE_Q8_1 ? PPML_WTYPE_Q8_1 : w->type == TENSOR_TYPE_Q8_0R ? PPML_WTYPE_Q8_0R : PPML_WTYPE_Q8_0;
+    const size_t need = q8_weight_packed_bytes_hip(static_cast<int>(M), static_cast<int>(K));
+    auto buf = std::make_unique<Buffer>(buffer_type(), need);
+    if (!buf->data()) return fail(Status::ALLOC_FAILED, "pack_weight: cannot allocate " + std::to_string(need) + " bytes");
+    const int rc = q8_weight_pack_hip(w->data, wtype, static_cast<int>(M), static_cast<int>(K), buf->data(), nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("pack_weight: ") + ppml_hip_last_error());
+    if (hipDeviceSynchronize() != hipSuccess) return fail(Status::ABORTED, "pack_weight: device error");
+    w->data = buf->data();
+    w->buffer = buf.get();
+    w->buffer_offs = 0;
+    w->type = TENSOR_TYPE_Q8_0M;
+    owned_.push_back(std::move(buf));
+    return Status::SUCCESS;
+}
+
+}  // namespace ppmlhip
+
+// ------------------------------------------------------------------------------------------------
+// C ABI of ppml_hip_backend.h
+using namespace ppmlhip;
+
+struct ppml_hip_backend {
+    HipBackend impl;
+    explicit ppml_hip_backend(int device) : impl(device) {}
+};
+struct ppml_hip_tensor {
+    Tensor t;
+    std::unique_ptr<Buffer> own;
+};
+
+extern "C" {
+
+ppml_hip_backend* ppml_hip_backend_create(int device) {
+    auto* b = new (std::nothrow) ppml_hip_backend(device);
+    if (b && !b->impl.last_error().empty()) {   // no gfx950 device: the backend has no other path
+        delete b;
+        return nullptr;
+    }
+    return b;
+}
+void ppml_hip_backend_destroy(ppml_hip_backend* b) { delete b; }
+const char* ppml_hip_backend_name(const ppml_hip_backend* b) { return b ? b->impl.get_name() : ""; }
+const char* ppml_hip_backend_last_error(const ppml_hip_backend* b) { return b ? b->impl.last_error().c_str() : "null backend"; }
+int ppml_hip_backend_priority(const ppml_hip_backend* b) { return b ? b->impl.priority() : 0; }
+void ppml_hip_backend_synchronize(ppml_hip_backend* b) {
+    if (b) b->impl.synchronize();
+}
+
+ppml_hip_tensor* ppml_hip_tensor_create(int op, int type, int ndim, const int64_t* dims) {
+    if (ndim < 0 || ndim > 4 || (ndim > 0 && !dims)) return nullptr;
+    auto* t = new (std::nothrow) ppml_hip_tensor();
+    if (!t) return nullptr;
+    t->t.op = op;
+    t->t.type = type;
+    t->t.ndim = ndim;
+    for (int i = 0; i < ndim; ++i) t->t.dims[i] = dims[i];
+    return t;
+}
+void ppml_hip_tensor_destroy(ppml_hip_tensor* t) { delete t; }
+void ppml_hip_tensor_set_src(ppml_hip_tensor* t, int slot, ppml_hip_tensor* src) {
+    if (t && slot >= 0 && slot < 10) t->t.src[slot] = src ? &src->t : nullptr;
+}
+void ppml_hip_tensor_set_data(ppml_hip_tensor* t, void* device_ptr) {
+    if (!t) return;
+    t->own.reset();
+    t->t.data = device_ptr;
+    t->t.buffer = nullptr;
+    t->t.buffer_offs = 0;
+}
+void ppml_hip_tensor_set_view(ppml_hip_tensor* t, ppml_hip_tensor* view_src, size_t byte_offset) {
+    if (!t) return;
+    t->t.view_src = view_src ? &view_src->t : nullptr;
+    t->t.view_offs = byte_offset;
+}
+void ppml_hip_tensor_set_param(ppml_hip_tensor* t, int index, float value) {
+    if (t && index >= 0 && index < 16) t->t.op_params[index] = value;
+}
+size_t ppml_hip_tensor_nbytes(const ppml_hip_tensor* t) { return t ? t->t.nbytes() : 0; }
+int ppml_hip_tensor_type(const ppml_hip_tensor* t) { return t ? t->t.type : -1; }
+
+int ppml_hip_tensor_upload(ppml_hip_backend* b, ppml_hip_tensor* t, const void* host, size_t nbytes) {
+    if (!b || !t || !host) return static_cast<int>(Status::NOT_SUPPORTED);
+    if (nbytes != t->t.nbytes()) return static_cast<int>(Status::NOT_SUPPORTED);
+    if (!t->own || t->own->size() < nbytes) {
+        t->own = std::make_unique<Buffer>(b->impl.buffer_type(), nbytes);
+        if (!t->own->data()) {
+            t->own.reset();
+            return static_cast<int>(Status::ALLOC_FAILED);
+        }
+    }
+    t->t.data = t->own->data();
+    t->t.buffer = t->own.get();
+    t->t.buffer_offs = 0;
+    return t->own->set_tensor(&t->t, host, 0, nbytes) ? 0 : static_cast<int>(Status::ABORTED);
+}
+int ppml_hip_tensor_download(ppml_hip_backend* b, const ppml_hip_tensor* t, void* host, size_t nbytes) {
+    if (!b || !t || !host || !t->t.data || nbytes > t->t.nbytes()) return static_cast<int>(Status::NOT_SUPPORTED);
+    b->impl.synchronize();
+    if (t->t.buffer) return t->t.buffer->get_tensor(&t->t, host, 0, nbytes) ? 0 : static_cast<int>(Status::ABORTED);
+    return hipMemcpy(host, t->t.data, nbytes, hipMemcpyDeviceToHost) == hipSuccess ? 0 : static_cast<int>(Status::ABORTED);
+}
+
+int ppml_hip_backend_supports_op(const ppml_hip_backend* b, const ppml_hip_tensor* node) {
+    (void)b;
+    return node && node_supported(&node->t) ? 1 : 0;
+}
+int ppml_hip_backend_graph_compute(ppml_hip_backend* b, ppml_hip_tensor** nodes, int n) {
+    if (!b || (n > 0 && !nodes)) return static_cast<int>(Status::NOT_SUPPORTED);
+    ComputeGraph g;
+    g.reserve(n);
+    for (int i = 0; i < n; ++i) g.push_back(nodes[i] ? &nodes[i]->t : nullptr);
+    return static_cast<int>(b->impl.graph_compute(&g));
+}
+int ppml_hip_backend_pack_weight(ppml_hip_backend* b, ppml_hip_tensor* weight) {
+    if (!b || !weight) return static_cast<int>(Status::NOT_SUPPORTED);
+    return static_cast<int>(b->impl.pack_weight(&weight->t));
+}
+void ppml_hip_backend_set_skip_alloc(ppml_hip_backend* b, int on) {
+    if (b) b->impl.set_skip_alloc(on != 0);
+}
+
+}  // extern "C"

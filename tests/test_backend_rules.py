@@ -1,0 +1,77 @@
+"""Scheduling rules and tensor bookkeeping of the executor; no GPU needed.
+
+The table restates what the reference's CUDA backend answers for the three ops of this path
+(src/backend/CUDABackend.cpp:121-163 OP_MUL_MAT, OP_OUT_PROD; 410-416 OP_OUTER_PROD_MEAN).
+"""
+import pytest
+
+from proteinpredictmachinelearning_amd import backend as B
+
+
+def _mm(t0, t1, out=B.F32, bias=None, k0=64, k1=64):
+    s0 = B.Tensor((k0, 5), t0)
+    s1 = B.Tensor((k1, 7), t1)
+    src = [s0, s1] + ([B.Tensor((7,), bias)] if bias is not None else [])
+    return B.Tensor((7, 5), out, B.OP_MUL_MAT, src)
+
+
+@pytest.mark.parametrize("t0,t1,out,bias,want", [
+    (B.F32, B.F32, B.F32, None, True),
+    (B.F32, B.F32, B.F32, B.F32, True),          # bias epilogue: f32 path only
+    (B.F32, B.F32, B.F16, None, False),
+    (B.Q8_0, B.F32, B.F32, None, True),          # weight in src0 (ggml convention)
+    (B.F32, B.Q8_0, B.F32, None, True),          # weight in src1 (LinearLayer convention)
+    (B.F32, B.Q8_1, B.F32, None, True),
+    (B.F32, B.Q8_0R, B.F32, None, True),
+    (B.F32, B.Q8_0M, B.F32, None, True),
+    (B.Q8_0, B.Q8_0, B.F32, None, False),        # exactly one side may be quantized
+    (B.Q8_0, B.F32, B.F32, B.F32, False),        # no bias on the quantized path
+    (B.F32, B.Q8_0, B.F32, B.F32, False),
+    (B.Q8_0, B.F16, B.F32, None, False),         # activations must be f32
+    (B.F32, B.Q8_0, B.F16, None, False),
+    (B.F16, B.F16, B.F32, None, False),          # left to the reference's own kernels
+    (B.F32, B.F16, B.F32, None, False),
+])
+def test_supports_op_mul_mat(t0, t1, out, bias, want):
+    assert B.supports_op(_mm(t0, t1, out, bias)) is want
+
+
+def test_supports_op_rejects_quantized_rows_that_split_a_block():
+    assert B.supports_op(_mm(B.F32, B.Q8_0, k0=48, k1=48)) is False      # 48 % 32 != 0
+    assert B.supports_op(_mm(B.F32, B.Q8_0, k0=96, k1=96)) is True
+
+
+def test_supports_op_other_ops():
+    a = B.Tensor((4, 3, 2, 2))
+    b = B.Tensor((5, 3, 2, 2))
+    assert B.supports_op(B.Tensor((4, 5, 2, 2), B.F32, B.OP_OUT_PROD, [a, b]))
+    assert not B.supports_op(B.Tensor((4, 5, 2, 2), B.F32, B.OP_OUT_PROD, [a]))
+    assert not B.supports_op(B.Tensor((4, 5, 2, 2), B.F16, B.OP_OUT_PROD, [a, b]))
+    l = B.Tensor((3, 4, 8, 2))
+    assert B.supports_op(B.Tensor((9, 4, 4, 2), B.F32, B.OP_OUTER_PROD_MEAN, [l, l]))
+    l3 = B.Tensor((3, 4, 8))
+    assert not B.supports_op(B.Tensor((9, 4, 4, 1), B.F32, B.OP_OUTER_PROD_MEAN, [l3, l3]))
+    # no-op nodes are accepted (and skipped by the executor); everything else belongs to other backends
+    assert B.supports_op(B.Tensor((4,), B.F32, B.OP_VIEW, [a]))
+    assert B.supports_op(B.Tensor((4,), B.F32, B.OP_RESHAPE, [a]))
+    assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_SCALE, [a]))
+    assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_SOFT_MAX, [a]))
+
+
+def test_tensor_nbytes_follows_the_block_records():
+    # include/ppml/Tensor.h:327-352: quantized bytes = blocks * record size; invalid shapes have none
+    assert B.Tensor((256, 768), B.F32).nbytes == 256 * 768 * 4
+    assert B.Tensor((256, 768), B.F16).nbytes == 256 * 768 * 2
+    assert B.Tensor((256, 768), B.Q8_0).nbytes == 768 * 8 * 34
+    assert B.Tensor((256, 768), B.Q8_0R).nbytes == 768 * 8 * 34
+    assert B.Tensor((256, 768), B.Q8_1).nbytes == 768 * 8 * 36
+    assert B.Tensor((250, 768), B.Q8_0).nbytes == 0
+    assert B.Tensor((256, 768), B.Q8_0M).nbytes == 24 * 8 * (1024 + 64)
+    with pytest.raises(ValueError):
+        B.Tensor((1, 2, 3, 4, 5))
+
+
+def test_graph_compute_without_backend_is_refused():
+    from proteinpredictmachinelearning_amd import cabi
+
+    assert cabi.load().ppml_hip_backend_graph_compute(None, None, 0) == B.NOT_SUPPORTED

@@ -6,10 +6,10 @@ import re
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "ppml_hip.h")).read()
+def _declared_symbols(header="ppml_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    names = re.findall(r"^\s*(?:const\s+)?(?:int|size_t|char\s*\*)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+    names = re.findall(r"^\s*(?:const\s+)?(?:int|void|size_t|char\s*\*|ppml_hip_\w+\s*\*)\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
     return sorted(set(names))
 
 
@@ -23,6 +23,17 @@ def test_header_symbols_are_exported_and_bound():
         assert hasattr(lib, n), f"{n} declared in include/ppml_hip.h but not exported"
     assert set(names) == set(cabi.SIGNATURES), set(names) ^ set(cabi.SIGNATURES)
     assert lib.ppml_hip_abi_version() == 1
+
+
+def test_backend_header_symbols_are_exported_and_bound():
+    from proteinpredictmachinelearning_amd import cabi
+
+    names = _declared_symbols("ppml_hip_backend.h")
+    assert len(names) >= 18, names
+    lib = cabi.load()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/ppml_hip_backend.h but not exported"
+    assert set(names) == set(cabi.BACKEND_SIGNATURES), set(names) ^ set(cabi.BACKEND_SIGNATURES)
 
 
 def test_host_side_argument_checks_need_no_gpu():

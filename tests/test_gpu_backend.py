@@ -1,0 +1,144 @@
+"""The executor on the GPU: nodes built like the reference's tests build them
+(tests/test_cuda.cpp:39-51, 108-110), run through graph_compute, compared with the CPU oracle."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+from proteinpredictmachinelearning_amd import backend as B  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def be():
+    return B.Backend(0)
+
+
+def _leaf(be, arr, type=B.F32, dims=None):
+    arr = np.ascontiguousarray(arr)
+    t = B.Tensor(dims if dims is not None else arr.shape[::-1], type)
+    return be.upload(t, arr)
+
+
+def test_identity(be):
+    assert be.name == "HIP-gfx950" and be.priority == 1
+
+
+def test_mul_mat_node_reference_inputs(be, oracle):
+    # tests/test_cuda.cpp:133-167; dims are innermost-first: A [K, M], B [K, N], C [N, M]
+    M, K, N = 17, 9, 23
+    A = ((np.arange(M * K) % 11) * 0.5 - 2.0).astype(np.float32).reshape(M, K)
+    Bm = ((np.arange(N * K) % 13) * 0.25 + 0.5).astype(np.float32).reshape(N, K)
+    bias = ((np.arange(N) % 5) * 0.125 - 0.25).astype(np.float32)
+    a, b, c = _leaf(be, A), _leaf(be, Bm), _leaf(be, bias)
+    node = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [a, b])
+    nodeb = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [a, b, c])
+    assert be.supports_op(node) and be.supports_op(nodeb)
+    assert be.graph_compute([node, nodeb]) == B.SUCCESS, be.last_error
+    assert (be.download(node).reshape(M, N) == oracle.mul_mat_f32(A, Bm)).all()
+    assert (be.download(nodeb).reshape(M, N) == oracle.mul_mat_f32(A, Bm, bias)).all()
+
+
+@pytest.mark.parametrize("wname", ["Q8_0", "Q8_1", "Q8_0R", "packed"])
+@pytest.mark.parametrize("wside", [0, 1])
+def test_quantized_mul_mat_node(be, oracle, wname, wside):
+    rows, K, F = 77, 128, 96        # tokens, in features, out features
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((rows, K)).astype(np.float32)
+    w = (rng.standard_normal((F, K)) * 0.02).astype(np.float32)
+    wq = oracle.quantize_q8_0(w)                                    # [F][K/32] 34-byte records
+    if wname == "Q8_1":                                             # d, s, qs: s is not read
+        rec = np.frombuffer(wq.tobytes(), dtype=np.uint8).reshape(-1, 34)
+        raw = np.concatenate([rec[:, :2], np.zeros((rec.shape[0], 2), np.uint8), rec[:, 2:]], axis=1)
+        wt = _leaf(be, raw.reshape(-1), B.Q8_1, (K, F))
+    elif wname == "Q8_0R":
+        wt = _leaf(be, np.frombuffer(oracle.repack_q8_0(wq).tobytes(), np.uint8), B.Q8_0R, (K, F))
+    else:
+        wt = _leaf(be, np.frombuffer(wq.tobytes(), np.uint8), B.Q8_0, (K, F))
+    if wname == "packed":
+        assert be.pack_weight(wt) == B.SUCCESS, be.last_error
+        assert wt.type == B.Q8_0M
+        assert be.pack_weight(wt) == B.SUCCESS                      # idempotent
+    xt = _leaf(be, x)
+    want = oracle.mul_mat_q8(wq, x, wtype=0, c_trans=1, fma=1)      # [rows][F]
+    if wside == 1:      # mul_mat(x, W): node [F, rows], rows of the result are tokens
+        node = B.Tensor((F, rows), B.F32, B.OP_MUL_MAT, [xt, wt])
+        got = be_run(be, node).reshape(rows, F)
+    else:               # mul_mat(W, x): node [rows, F], rows of the result are out features
+        node = B.Tensor((rows, F), B.F32, B.OP_MUL_MAT, [wt, xt])
+        got = be_run(be, node).reshape(F, rows).T
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6 * np.abs(want).max())
+
+
+def be_run(be, node):
+    assert be.supports_op(node)
+    assert be.graph_compute([node]) == B.SUCCESS, be.last_error
+    return be.download(node)
+
+
+def test_quantized_mul_mat_with_bias_is_refused(be, oracle):
+    x = np.ones((4, 32), np.float32)
+    wq = oracle.quantize_q8_0(np.ones((8, 32), np.float32))
+    wt = _leaf(be, np.frombuffer(wq.tobytes(), np.uint8), B.Q8_0, (32, 8))
+    node = B.Tensor((8, 4), B.F32, B.OP_MUL_MAT, [_leaf(be, x), wt, _leaf(be, np.zeros(8, np.float32))])
+    assert not be.supports_op(node)
+    assert be.graph_compute([node]) == B.NOT_SUPPORTED
+    assert "not supported" in be.last_error
+
+
+def test_out_prod_and_outer_prod_mean_nodes(be, oracle):
+    rng = np.random.default_rng(3)
+    s0 = rng.integers(-3, 4, size=(2, 3, 10, 7)).astype(np.float32)
+    s1 = rng.integers(-3, 4, size=(2, 6, 10, 5)).astype(np.float32)
+    a, b = _leaf(be, s0), _leaf(be, s1)
+    op = B.Tensor((7, 5, 6, 2), B.F32, B.OP_OUT_PROD, [a, b])
+    D, L, N, Bt = 3, 4, 8, 2
+    l = rng.integers(-3, 4, size=D * L * N * Bt).astype(np.float32)
+    r = rng.integers(-3, 4, size=D * L * N * Bt).astype(np.float32)
+    lt, rt = _leaf(be, l, dims=(D, L, N, Bt)), _leaf(be, r, dims=(D, L, N, Bt))
+    opm = B.Tensor((D * D, L, L, Bt), B.F32, B.OP_OUTER_PROD_MEAN, [lt, rt])
+    assert be.graph_compute([op, opm]) == B.SUCCESS, be.last_error
+    assert (be.download(op).reshape(2, 6, 5, 7) == oracle.out_prod(s0, s1)).all()
+    assert (be.download(opm) == oracle.outer_prod_mean(l, r, D, L, N, Bt)).all()
+
+
+def test_view_sources_are_resolved_and_noop_nodes_skipped(be, oracle):
+    # a reshape node built with only src[0] set, and an offset view with view_src set, both feed a
+    # mul_mat (src/backend/CUDABackend.cpp:800-819)
+    M, K, N = 6, 8, 5
+    rng = np.random.default_rng(8)
+    big = rng.integers(-4, 5, size=(2 * M, K)).astype(np.float32)       # two stacked A matrices
+    Bm = rng.integers(-4, 5, size=(N, K)).astype(np.float32)
+    base = _leaf(be, big)
+    second = B.Tensor((K, M), B.F32, B.OP_VIEW).view_of(base, M * K * 4)
+    flat = _leaf(be, Bm.reshape(-1))
+    resh = B.Tensor((K, N), B.F32, B.OP_RESHAPE, [flat])
+    node = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [second, resh])
+    assert be.graph_compute([second, resh, node]) == B.SUCCESS, be.last_error
+    assert (be.download(node).reshape(M, N) == oracle.mul_mat_f32(big[M:], Bm)).all()
+
+
+def test_failure_statuses(be):
+    a = _leaf(be, np.ones((3, 4), np.float32))
+    b = _leaf(be, np.ones((5, 4), np.float32))
+    # an op without a kernel here: NOT_SUPPORTED, nothing launched
+    assert be.graph_compute([B.Tensor((4, 3), B.F32, B.OP_SCALE, [a])]) == B.NOT_SUPPORTED
+    # a source nobody bound
+    ghost = B.Tensor((4, 5))
+    assert be.graph_compute([B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, ghost])]) == B.NOT_SUPPORTED
+    assert "src1" in be.last_error
+    # a host pointer passed off as device memory (src/backend/CUDABackend.cpp:894-973)
+    host = np.ones((5, 4), np.float32)
+    fake = B.Tensor((4, 5)).bind(host.ctypes.data)
+    assert be.graph_compute([B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, fake])]) == B.NOT_SUPPORTED
+    # shapes that do not match the node
+    assert be.graph_compute([B.Tensor((6, 3), B.F32, B.OP_MUL_MAT, [a, b])]) == B.NOT_SUPPORTED
+    # with a scheduler in charge of allocation the executor allocates nothing
+    be.set_skip_alloc(True)
+    try:
+        assert be.graph_compute([B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, b])]) == B.NOT_SUPPORTED
+    finally:
+        be.set_skip_alloc(False)
+    # and the backend still works afterwards
+    node = B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, b])
+    assert be.graph_compute([node]) == B.SUCCESS
+    assert (be.download(node) == 4.0).all()
