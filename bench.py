@@ -122,7 +122,7 @@ def main() -> int:
                    "buffer_rotation": nsets, "weight_layout": "Q8_0M (MFMA fragments)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "q8_linear_kernel", "algorithmic_bytes_per_launch": nbytes,
+                     "kernel": "q8_linear_ws_kernel", "algorithmic_bytes_per_launch": nbytes,
                      "kernel_us": round(ev * 1e6, 2),
                      "int8_mfma_frac": round(nops / ev / 1e12 / INT8_PEAK_TOPS, 4)},
     }

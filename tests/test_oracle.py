@@ -219,6 +219,72 @@ def test_q8_matmul_end_to_end_and_layouts(oracle):
     assert one[0, 0] == np.float32(s) * np.float32(dw * da)
 
 
+def _round_to_f32(v):
+    """Exact rational -> nearest binary32 (ties to even), by integer arithmetic only."""
+    from fractions import Fraction
+
+    if v == 0:
+        return np.float32(0.0)
+    sign = -1 if v < 0 else 1
+    v = abs(Fraction(v))
+    e = v.numerator.bit_length() - v.denominator.bit_length() - 24
+    while v / Fraction(2) ** e >= 2 ** 24:
+        e += 1
+    while v / Fraction(2) ** e < 2 ** 23:
+        e -= 1
+    e = max(e, -149)
+    q = v / Fraction(2) ** e
+    n, rem = divmod(q.numerator, q.denominator)
+    twice = 2 * rem
+    if twice > q.denominator or (twice == q.denominator and n % 2 == 1):
+        n += 1
+    return np.float32(sign * float(n) * 2.0 ** e)       # n < 2^24 + 1 and the scaling are exact in double
+
+
+def test_q8_matmul_settlement_order_bit_exact(oracle):
+    # The settlement acc = fma(float(sumi), dw*da, acc), blocks ascending, redone in exact rational
+    # arithmetic with one rounding per step.  The case is chosen so that the three plausible
+    # mistakes -- multiply and add rounded separately, blocks walked backwards, scales multiplied
+    # into the sum one after the other -- each change at least one output bit.
+    from fractions import Fraction
+
+    rng = np.random.default_rng(12)
+    M, N, K = 6, 5, 256
+    w = (rng.standard_normal((M, K)) * np.exp(rng.standard_normal((M, K // 32)).repeat(32, axis=1))).astype(np.float32)
+    x = (rng.standard_normal((N, K)) * np.exp(rng.standard_normal((N, K // 32)).repeat(32, axis=1))).astype(np.float32)
+    wq, xq = oracle.quantize_q8_0(w), oracle.quantize_q8_0(x)
+    sums = oracle.q8_block_sums(wq, xq)
+    dw = oracle.block_scales_bits(wq).view(np.float16).astype(np.float32)
+    da = oracle.block_scales_bits(xq).view(np.float16).astype(np.float32)
+
+    def settle(order, fused, split_scales=False):
+        out = np.zeros((N, M), np.float32)
+        for n in range(N):
+            for m in range(M):
+                acc = np.float32(0.0)
+                for b in order:
+                    sf = Fraction(int(sums[n, m, b]))
+                    if split_scales:
+                        t = _round_to_f32(sf * Fraction(float(dw[m, b])))
+                        prod = Fraction(float(t)) * Fraction(float(da[n, b]))
+                    else:
+                        prod = sf * Fraction(float(dw[m, b] * da[n, b]))      # dw*da is exact in binary32
+                    if fused:
+                        acc = _round_to_f32(prod + Fraction(float(acc)))
+                    else:
+                        acc = _round_to_f32(Fraction(float(_round_to_f32(prod))) + Fraction(float(acc)))
+                out[n, m] = acc
+        return out
+
+    blocks = list(range(K // 32))
+    want = settle(blocks, fused=True)
+    got = oracle.mul_mat_q8q8(wq, xq, c_trans=1, fma=1)
+    assert (got.view(np.uint32) == want.view(np.uint32)).all()
+    assert (oracle.mul_mat_q8q8(wq, xq, c_trans=1, fma=0).view(np.uint32) == settle(blocks, fused=False).view(np.uint32)).all()
+    for wrong in (settle(blocks, fused=False), settle(blocks[::-1], fused=True), settle(blocks, True, split_scales=True)):
+        assert (wrong.view(np.uint32) != want.view(np.uint32)).any()
+
+
 # ----------------------------------------------------------------------------- f32 mul_mat
 def test_mul_mat_reference_test_inputs_exact(oracle):
     # tests/test_cuda.cpp:133-167: every product is a multiple of 1/8 and every partial sum is small,
