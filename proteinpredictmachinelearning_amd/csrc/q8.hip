@@ -6,6 +6,8 @@
 //   block dot and settlement src/cuda/MulMatQ8Kernel.cu:120-142
 //   launcher contract        src/cuda/MulMatQ8Kernel.cu:476-547, src/cuda/QuantKernels.cu:86-109
 #include "common.hpp"
+#include <type_traits>
+#include <cstdlib>
 
 namespace ppmlhip {
 namespace {
@@ -227,17 +229,24 @@ __global__ __launch_bounds__(64) void q8_weight_pack_kernel(const uint8_t* __res
 #ifdef PPML_Q8_TRACE
 // Development aid, compiled out of the library: per-wave timestamps of the kernel's phases.
 __device__ unsigned long long* g_q8_trace = nullptr;
+__device__ int g_q8_dbg[4] = {0, 0, 0, 0};
+#ifndef PPML_ABL
+#define PPML_ABL 0
+#endif
+#define PPML_DBG(bit) ((PPML_ABL >> (bit)) & 1)   /* compile-time ablation mask of the timeline probe */
 #define PPML_TRACE_MARK(slot)                                                                      \
     do {                                                                                           \
         if (g_q8_trace && (threadIdx.x & 63) == 0)                                                 \
-            g_q8_trace[(static_cast<size_t>(blockIdx.x) * NW + (threadIdx.x >> 6)) * 32 + (slot)] = \
+            g_q8_trace[(static_cast<size_t>(blockIdx.x) * NW + (threadIdx.x >> 6)) * 64 + (slot)] = \
                 __builtin_amdgcn_s_memrealtime();   /* 100 MHz, common to the whole device */      \
     } while (0)
 #else
 #define PPML_TRACE_MARK(slot) do {} while (0)
+#define PPML_DBG(bit) 0
 #endif
 
 constexpr int TILE_TOK = 32;
+constexpr int WS_NBUF = 3;          // quantized activation tiles the weight-stationary kernel keeps in LDS
 constexpr int KC_MAX = 56;          // blocks of K staged in LDS at once (63 KiB)
 constexpr int UB = 4;               // quantizer units (8 rows x 2 blocks) a wave keeps in flight
 
@@ -531,7 +540,8 @@ int launch_q8_linear(const void* W, const float* X, float* C, int M, int N, int 
 // VALU, so the matrix pipe runs one block ahead of the VALU and neither waits for the other.  A
 // tile is stored as soon as its last block is settled, under the arithmetic of the next tile.
 // MFMA roles: A = activation rows, B = weight rows, so a store instruction writes two full
-// 128-byte lines.  LDS holds two quantized tiles so a single barrier per tile is enough.
+// 128-byte lines.  LDS holds three quantized tiles and a count of the waves that have written each,
+// so the loop needs no barrier: waves drift apart by up to a third of a tile instead of meeting.
 // ------------------------------------------------------------------------------------------
 // A value the optimizer cannot see through (always 1).  Branching on it puts the guarded code in a
 // basic block of its own: the fully unrolled MFMA steps below would otherwise all be issued up
@@ -542,8 +552,15 @@ __device__ __forceinline__ int opaque_one() {
     return one;
 }
 
-template <int NW, int TPW, int NBLK, bool DUMP>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void q8_linear_ws_kernel(
+// VGPRs the compiler may allocate in the weight-stationary kernel; the ones above hold the
+// activation tile in flight (see load_tile_async) and are touched by inline assembly only.
+constexpr int ws_staging_regs(int nblk, int nw = 8) {   // 8 registers per unit of (8 rows x 2 blocks) a wave loads
+    return (2 * nblk + nw - 1) / nw * 8 < 16 ? 16 : (2 * nblk + nw - 1) / nw * 8;
+}
+constexpr int ws_compiler_vgprs(int nblk, int nw = 8) { return 256 - ws_staging_regs(nblk, nw); }
+
+template <int NW, int TPW, int NBLK, int WL, bool DUMP>
+__device__ __forceinline__ void q8_linear_ws_body(
     const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
     int M, int N, int ntiles, int relu,
     uint8_t* __restrict__ xq_dump, int32_t* __restrict__ sums_dump) {
@@ -552,12 +569,19 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     constexpr int NUNITS = 2 * NBLK;                   // (8 rows) x (2 blocks) each
     constexpr int UPW = (NUNITS + NW - 1) / NW;        // units per wave
     constexpr int STEPS = TPW * NBLK;
-    // LDS: two quantized activation tiles (fragments + scales) and this work-group's weight scales.
+    // LDS: three quantized activation tiles (fragments + scales) and this work-group's weight scales.
     // Scale rows are 64 wide with lanes 32..63 zero: they feed K slot 1 of the scale MFMA.
     extern __shared__ __attribute__((aligned(16))) uint8_t ws_lds[];
     v4i (*lds_a)[NBLK * 64] = reinterpret_cast<v4i (*)[NBLK * 64]>(ws_lds);
-    float (*lds_d)[NBLK * 64] = reinterpret_cast<float (*)[NBLK * 64]>(ws_lds + 2 * NBLK * 1024);
-    float* lds_wd = reinterpret_cast<float*>(ws_lds + 2 * NBLK * 1024 + 2 * NBLK * 256);   // [NW*TPW][NBLK][64]
+    float (*lds_d)[NBLK * 64] = reinterpret_cast<float (*)[NBLK * 64]>(ws_lds + WS_NBUF * NBLK * 1024);
+    float* lds_wd = reinterpret_cast<float*>(ws_lds + WS_NBUF * NBLK * 1024 + WS_NBUF * NBLK * 256);   // [NW*TPW][NBLK][64]
+    // ready[b]: how many waves have written their share of the tile currently being put in buffer b
+    // (counts up for the life of the kernel; the k-th filling of a buffer is complete at k * NW)
+    unsigned* lds_ready = reinterpret_cast<unsigned*>(ws_lds + WS_NBUF * NBLK * 1024 + WS_NBUF * NBLK * 256 +
+                                                      static_cast<size_t>(NW) * TPW * NBLK * 256);
+    // fragments of the last WL column tiles of every wave, when the register file cannot hold all TPW
+    v4i* lds_wq = reinterpret_cast<v4i*>(ws_lds + WS_NBUF * NBLK * 1024 + WS_NBUF * NBLK * 256 +
+                                         static_cast<size_t>(NW) * TPW * NBLK * 256 + 16);   // [NW][WL][NBLK][64]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -583,16 +607,67 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
         }
     };
 
+    // In-loop form of load_tile.  The vector-memory counter retires in order and counts stores too;
+    // the compiler cannot tell how many output stores follow these loads on every path, so it would
+    // wait for (nearly) all of them before the quantizer touches the data -- and if the loads were
+    // inline assembly with ordinary outputs it would feel free to copy the "results" to other
+    // registers before they have arrived.  So the tile in flight lives in the top STAGE registers,
+    // which the kernel attribute keeps away from the register allocator: load_tile_async() writes
+    // them, take_tile() waits for exactly these loads and only then copies them out.
+    constexpr int STAGE = ws_staging_regs(NBLK, NW);
+    constexpr int STAGE0 = 256 - STAGE;
+    static_assert(UPW * 8 <= STAGE, "staging registers hold one tile share");
+    auto load_tile_async = [&](int tile) {
+#pragma unroll
+        for (int s = 0; s < UPW; ++s) {
+            int u = wave + s * NW;
+            u = u < NUNITS ? u : NUNITS - 1;
+            const int bl = (u >> 2) * 2 + ublk;
+            int t = tile * TILE_TOK + (u & 3) * 8 + urow;
+            t = t < N ? t : N - 1;
+            const float* src = X + static_cast<int64_t>(t) * K + bl * QK + c4 * 8;
+            asm volatile("global_load_dwordx4 v[%1:%2], %0, off\n\tglobal_load_dwordx4 v[%3:%4], %0, off offset:16"
+                         :: "v"(src), "n"(STAGE0 + 8 * s), "n"(STAGE0 + 8 * s + 3), "n"(STAGE0 + 8 * s + 4), "n"(STAGE0 + 8 * s + 7)
+                         : "memory", "v255");
+        }
+    };
+    // `newer` = vector-memory operations issued after load_tile_async: once at most that many are
+    // outstanding, its loads have landed.
+    auto take_tile = [&](auto newer, v4f (&xv)[UPW][2]) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(newer)::value) : "memory");
+#pragma unroll
+        for (int s = 0; s < UPW; ++s) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float e0, e1, e2, e3;
+                asm volatile("v_mov_b32 %0, v[%4]\n\tv_mov_b32 %1, v[%5]\n\tv_mov_b32 %2, v[%6]\n\tv_mov_b32 %3, v[%7]"
+                             : "=v"(e0), "=v"(e1), "=v"(e2), "=v"(e3)
+                             : "n"(STAGE0 + 8 * s + 4 * h), "n"(STAGE0 + 8 * s + 4 * h + 1), "n"(STAGE0 + 8 * s + 4 * h + 2),
+                               "n"(STAGE0 + 8 * s + 4 * h + 3)
+                             : "memory");
+                xv[s][h] = v4f{e0, e1, e2, e3};
+            }
+        }
+    };
+
     // The first activation tile is requested before the weights: it has the longer way to come,
     // and it keeps these loads older than at least a tile's worth of later memory operations on
     // every path into the loop, which is what lets the wait in front of the quantizer skip them.
     v4f xv[UPW][2];
     int tile = blockIdx.x;
     PPML_TRACE_MARK(0);
+#ifdef PPML_Q8_TRACE
+    if (g_q8_dbg[0] > 0) {
+        const int ph = (blockIdx.x / (g_q8_dbg[2] > 0 ? g_q8_dbg[2] : 1)) % g_q8_dbg[0];
+        for (int i = 0; i < ph * g_q8_dbg[1]; ++i) __builtin_amdgcn_s_sleep(8);
+    }
+#endif
     if (tile < ntiles) load_tile(tile, xv);
 
     // ---- resident weights: fragments of TPW column tiles in registers, their scales in LDS
-    v4i wq[TPW][NBLK];
+    static_assert(WL >= 0 && WL < TPW, "at least one column tile stays in registers");
+    v4i wq[TPW - WL][NBLK];
+    v4i* my_wq = lds_wq + static_cast<size_t>(wave) * WL * NBLK * 64 + lane;
     float* my_wd = lds_wd + static_cast<size_t>(wave) * TPW * NBLK * 64 + lane;
     {
         const uint16_t* dplane = reinterpret_cast<const uint16_t*>(W + static_cast<size_t>(mct_pad) * NBLK * 1024);
@@ -602,13 +677,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
             ct = ct < mct_pad ? ct : mct_pad - 1;      // tiles past the end repeat the last one; never stored
 #pragma unroll
             for (int b = 0; b < NBLK; ++b) {
-                wq[t][b] = *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(ct * NBLK + b) * 64 + lane) * 16);
+                const v4i frag = *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(ct * NBLK + b) * 64 + lane) * 16);
+                if (t < TPW - WL) wq[t < TPW - WL ? t : 0][b] = frag;
+                else my_wq[((t - (TPW - WL)) * NBLK + b) * 64] = frag;
                 const float d = half_bits_to_float(dplane[(ct * NBLK + b) * 32 + j]);
                 my_wd[(t * NBLK + b) * 64] = hh ? 0.0f : d;
             }
         }
     }
-    for (int i = tid; i < 2 * NBLK * 64; i += NW * 64) (&lds_d[0][0])[i] = 0.0f;
+    for (int i = tid; i < WS_NBUF * NBLK * 64; i += NW * 64) (&lds_d[0][0])[i] = 0.0f;
+    if (tid < WS_NBUF) lds_ready[tid] = 0u;
     __syncthreads();
 
     // quantizes the tile held in xv into LDS buffer `buf`
@@ -635,23 +713,49 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
         }
     };
 
-    if (tile < ntiles) quantize_tile(0, tile * TILE_TOK, xv);
-    __syncthreads();
+    // A wave announces that its share of a quantized tile is in LDS; consumers poll the count.  The
+    // LDS unit executes one wave's operations in order, so the count becomes visible after the data.
+    auto announce = [&](int buf) {
+        asm volatile("" ::: "memory");
+        if (lane == 0) __hip_atomic_fetch_add(&lds_ready[buf], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        asm volatile("" ::: "memory");
+    };
+    auto await_tile = [&](int buf, unsigned want) {
+        while (__hip_atomic_load(&lds_ready[buf], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < want)
+            __builtin_amdgcn_s_sleep(1);
+        asm volatile("" ::: "memory");
+    };
+
+    if (tile < ntiles) {
+        quantize_tile(0, tile * TILE_TOK, xv);
+        announce(0);
+    }
+    // Every weight fragment has arrived before the loop starts: a load still pending here would make
+    // its first use inside the loop wait for vmcnt(0), i.e. for all output stores, on every iteration.
+    __builtin_amdgcn_s_waitcnt(0x0f70);                // vmcnt(0), other counters untouched
+    // the second tile is requested now and quantized two thirds into the first one
+    if (tile + static_cast<int>(gridDim.x) < ntiles && !PPML_DBG(2)) load_tile_async(tile + static_cast<int>(gridDim.x));
     PPML_TRACE_MARK(1);
 
-    // Step at which the next tile is quantized: late enough for its loads (issued at the top of the
-    // iteration) to have arrived, early enough that the output stores on both sides of it keep
-    // the write path busy through it.
+    // Step at which the next tile is quantized.  Its loads were issued one full round of column tiles
+    // earlier (right after the previous quantization freed the staging registers), so they have
+    // long arrived; the tile after it is requested as soon as this one is in LDS.
     constexpr int QSTEP = ((2 * STEPS / 3) / 2) * 2;
+    // Vector-memory operations issued between a tile's loads and the wait in front of its
+    // quantization: 16 stores per column tile, one round of column tiles (fewer before the first wait).
+    constexpr int NEWER_FIRST = 16 * (QSTEP / NBLK) < 63 ? 16 * (QSTEP / NBLK) : 63;
+    constexpr int NEWER = 16 * TPW < 63 ? 16 * TPW : 63;
 
+    // No barrier inside the loop.  A wave may start tile `it` once all waves have announced it, which
+    // also means all of them are past two thirds of tile it-1; the tile quantized during tile `it`
+    // goes to buffer (it+1) % 3, last read for tile it-2, which every wave has left by then.
     for (int it = 0; tile < ntiles; tile += gridDim.x, ++it) {
-        const int buf = it & 1;
+        const int buf = it % WS_NBUF;
         const int tok0 = tile * TILE_TOK;
         const int next = tile + static_cast<int>(gridDim.x);
         const bool has_next = next < ntiles;
-        // ---------------- request the next tile; it arrives under this tile's arithmetic
-        if (has_next) load_tile(next, xv);
-        PPML_TRACE_MARK(2 + 4 * it);
+        await_tile(buf, static_cast<unsigned>(NW) * static_cast<unsigned>(it / WS_NBUF + 1));
+        PPML_TRACE_MARK(2 + 10 * it);
 
         // ---------------- MFMA one block ahead of the settle; tiles in turn, blocks ascending
         v16i zero_i;
@@ -663,11 +767,17 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
         v16i sum_a, sum_b;
         v16f scl_a, scl_b;
         v16f acc;
+#ifdef PPML_Q8_TRACE
+        sum_a = zero_i; sum_b = zero_i; scl_a = zero_f; scl_b = zero_f;
+#endif
         auto issue = [&](int st, v16i& sum, v16f& scl) {
             const int t = st / NBLK, b = st % NBLK;
+            if (PPML_DBG(5)) return;
             const v4i a = lds_a[buf][b * 64 + lane];
             const float da = lds_d[buf][b * 64 + lane];
-            sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, wq[t][b], zero_i, 0, 0, 0);
+            if (PPML_DBG(4)) { sum[0] += a[0] + wq[0][b][0]; scl[0] += da + my_wd[(t * NBLK + b) * 64]; return; }
+            const v4i w = t < TPW - WL ? wq[t < TPW - WL ? t : 0][b] : my_wq[((t - (TPW - WL)) * NBLK + b) * 64];
+            sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, w, zero_i, 0, 0, 0);
             scl = __builtin_amdgcn_mfma_f32_32x32x2f32(da, my_wd[(t * NBLK + b) * 64], zero_f, 0, 0, 0);
         };
         auto settle = [&](int st, const v16i& sum, const v16f& scl) {
@@ -687,11 +797,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                     if (tok < N && m < M) sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b] = sum[r];
                 }
             }
-            if (b == NBLK - 1) {
+            if (b == NBLK - 1 && !PPML_DBG(0)) {
                 // The tile is complete: each half-wave store writes one full 128-byte line of a C
                 // row.  Buffer stores with a bounds-checked offset: lanes past the edge of C pass an
                 // offset beyond the buffer and are dropped by the hardware, so every wave issues
                 // exactly 16 stores here and the memory counter stays predictable.
+                PPML_TRACE_MARK(2 + 10 * it + 1 + 2 * t);
                 const uint32_t base = (static_cast<uint32_t>(tok0 + 4 * hh) * M + m) * 4u;
                 const uint32_t out_of_range = 0xfffffff0u;
                 if (tok0 + TILE_TOK <= N) {
@@ -708,6 +819,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
                                                               (8 * (r >> 2) + (r & 3)) * M * 4, 0);
                     }
                 }
+                PPML_TRACE_MARK(2 + 10 * it + 2 + 2 * t);
             }
         };
         static_assert(STEPS % 2 == 0, "steps are taken in pairs");
@@ -715,19 +827,46 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
         for (int st = 0; st < STEPS; st += 2) {
             if (!opaque_one()) continue;               // one basic block per pair of steps, see opaque_one()
-            if (st == QSTEP && has_next) {
-                quantize_tile(buf ^ 1, next * TILE_TOK, xv);
-                PPML_TRACE_MARK(3 + 4 * it);
+            if (st == QSTEP && has_next && !PPML_DBG(3)) {
+                PPML_TRACE_MARK(2 + 10 * it + 7);
+                {
+                    v4f xn[UPW][2];
+                    if (it == 0) take_tile(std::integral_constant<int, NEWER_FIRST>{}, xn);
+                    else take_tile(std::integral_constant<int, NEWER>{}, xn);
+                    const int next2 = next + static_cast<int>(gridDim.x);
+                    if (next2 < ntiles && !PPML_DBG(2)) load_tile_async(next2);
+                    quantize_tile((it + 1) % WS_NBUF, next * TILE_TOK, xn);
+                    announce((it + 1) % WS_NBUF);
+                }
+                PPML_TRACE_MARK(2 + 10 * it + 8);
             }
+            if (!PPML_DBG(1) || (st % NBLK) == NBLK - 2) {
             issue(st + 1, sum_b, scl_b);
             settle(st, sum_a, scl_a);
             if (st + 2 < STEPS) issue(st + 2, sum_a, scl_a);
             settle(st + 1, sum_b, scl_b);
+            }
         }
-        PPML_TRACE_MARK(4 + 4 * it);
-        __syncthreads();                               // next tile quantized, this tile's LDS reads done
-        PPML_TRACE_MARK(5 + 4 * it);
+        PPML_TRACE_MARK(2 + 10 * it + 9);
     }
+}
+
+// The attribute takes a literal, hence one kernel per staging size (16 registers up to K = 256, 32 beyond).
+template <int NW, int TPW, int NBLK, int WL, bool DUMP>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(240)))
+void q8_linear_ws_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
+                         int M, int N, int ntiles, int relu, uint8_t* __restrict__ xq_dump,
+                         int32_t* __restrict__ sums_dump) {
+    static_assert(ws_compiler_vgprs(NBLK) == 240, "staging size");
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, relu, xq_dump, sums_dump);
+}
+template <int NW, int TPW, int NBLK, int WL, bool DUMP>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(224)))
+void q8_linear_ws32_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
+                           int M, int N, int ntiles, int relu, uint8_t* __restrict__ xq_dump,
+                           int32_t* __restrict__ sums_dump) {
+    static_assert(ws_compiler_vgprs(NBLK) == 224, "staging size");
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, relu, xq_dump, sums_dump);
 }
 
 int device_cu_count() {
@@ -742,7 +881,7 @@ int device_cu_count() {
     return cus;
 }
 
-template <int TPW, int NBLK>
+template <int TPW, int NBLK, int WL>
 int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int relu,
                         void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
     constexpr int NW = 8;
@@ -753,26 +892,32 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
     const int rounds = (ntiles + cus - 1) / cus;
     const int wgs = (ntiles + rounds - 1) / rounds;
     const dim3 grid(wgs), block(NW * 64);
-    constexpr size_t lds = 2 * NBLK * 1024 + 2 * NBLK * 256 + static_cast<size_t>(NW) * TPW * NBLK * 256;
+    constexpr size_t lds = WS_NBUF * NBLK * 1024 + WS_NBUF * NBLK * 256 + static_cast<size_t>(NW) * TPW * NBLK * 256 + 16 +
+                           static_cast<size_t>(NW) * WL * NBLK * 1024;
+    using KernelFn = void (*)(const uint8_t*, const float*, float*, int, int, int, int, uint8_t*, int32_t*);
+    KernelFn fast, dump;
+    if constexpr (ws_staging_regs(NBLK) == 16) {
+        fast = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false>;
+        dump = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true>;
+    } else {
+        fast = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, false>;
+        dump = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, true>;
+    }
     if (lds > 64 * 1024) {
         static const hipError_t attr_fast = hipFuncSetAttribute(
-            reinterpret_cast<const void*>(&q8_linear_ws_kernel<NW, TPW, NBLK, false>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+            reinterpret_cast<const void*>(fast), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
         static const hipError_t attr_dump = hipFuncSetAttribute(
-            reinterpret_cast<const void*>(&q8_linear_ws_kernel<NW, TPW, NBLK, true>),
-            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+            reinterpret_cast<const void*>(dump), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
         if (attr_fast != hipSuccess || attr_dump != hipSuccess) {
             (void)hipGetLastError();
             return -1;                                  // fall back to the general kernel
         }
     }
     if (xq_dump || sums_dump)
-        hipLaunchKernelGGL((q8_linear_ws_kernel<NW, TPW, NBLK, true>), grid, block, lds, stream,
-                           static_cast<const uint8_t*>(W), X, C, M, N, ntiles, relu,
+        hipLaunchKernelGGL(dump, grid, block, lds, stream, static_cast<const uint8_t*>(W), X, C, M, N, ntiles, relu,
                            static_cast<uint8_t*>(xq_dump), sums_dump);
     else
-        hipLaunchKernelGGL((q8_linear_ws_kernel<NW, TPW, NBLK, false>), grid, block, lds, stream,
-                           static_cast<const uint8_t*>(W), X, C, M, N, ntiles, relu,
+        hipLaunchKernelGGL(fast, grid, block, lds, stream, static_cast<const uint8_t*>(W), X, C, M, N, ntiles, relu,
                            static_cast<uint8_t*>(nullptr), static_cast<int32_t*>(nullptr));
     return check_launch("q8_linear_ws_kernel");
 }
@@ -784,10 +929,11 @@ int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int 
     if (static_cast<int64_t>(N) * M * 4 >= 0x7fff0000LL) return -1;   // the kernel addresses C with 32-bit byte offsets
     const int mct = (M + 31) / 32;
     const int tpw = (mct + 7) / 8;
-#define PPML_WS(TPW, NBLK) if (tpw == TPW && nblk == NBLK) return launch_q8_linear_ws<TPW, NBLK>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
-    PPML_WS(1, 4);  PPML_WS(2, 4);  PPML_WS(3, 4);  PPML_WS(4, 4);
-    PPML_WS(1, 8);  PPML_WS(2, 8);  PPML_WS(3, 8);
-    PPML_WS(1, 16);
+#define PPML_WS(TPW, NBLK, WL) if (tpw == TPW && nblk == NBLK) return launch_q8_linear_ws<TPW, NBLK, WL>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
+    // (column tiles per wave, blocks of K, column tiles whose fragments live in LDS instead of registers)
+    PPML_WS(1, 4, 0);  PPML_WS(2, 4, 0);  PPML_WS(3, 4, 0);  PPML_WS(4, 4, 0);
+    PPML_WS(1, 8, 0);  PPML_WS(2, 8, 0);  PPML_WS(3, 8, 1);
+    PPML_WS(1, 16, 0);
 #undef PPML_WS
     return -1;
 }
