@@ -230,10 +230,6 @@ __global__ __launch_bounds__(64) void q8_weight_pack_kernel(const uint8_t* __res
 // Development aid, compiled out of the library: per-wave timestamps of the kernel's phases.
 __device__ unsigned long long* g_q8_trace = nullptr;
 __device__ int g_q8_dbg[4] = {0, 0, 0, 0};
-#ifndef PPML_ABL
-#define PPML_ABL 0
-#endif
-#define PPML_DBG(bit) ((PPML_ABL >> (bit)) & 1)   /* compile-time ablation mask of the timeline probe */
 #define PPML_TRACE_MARK(slot)                                                                      \
     do {                                                                                           \
         if (g_q8_trace && (threadIdx.x & 63) == 0)                                                 \
@@ -242,7 +238,6 @@ __device__ int g_q8_dbg[4] = {0, 0, 0, 0};
     } while (0)
 #else
 #define PPML_TRACE_MARK(slot) do {} while (0)
-#define PPML_DBG(bit) 0
 #endif
 
 constexpr int TILE_TOK = 32;
@@ -574,18 +569,21 @@ __device__ __forceinline__ void q8_linear_ws_body(
     constexpr int UPW = (NUNITS + NW - 1) / NW;        // units per wave
     constexpr int STEPS = TPW * NBLK;
     // LDS: three quantized activation tiles (fragments + scales) and this work-group's weight scales.
-    // Scale rows are 64 wide with lanes 32..63 zero: they feed K slot 1 of the scale MFMA.
     extern __shared__ __attribute__((aligned(16))) uint8_t ws_lds[];
     v4i (*lds_a)[NBLK * 64] = reinterpret_cast<v4i (*)[NBLK * 64]>(ws_lds);
-    float (*lds_d)[NBLK * 64] = reinterpret_cast<float (*)[NBLK * 64]>(ws_lds + WS_NBUF * NBLK * 1024);
-    float* lds_wd = reinterpret_cast<float*>(ws_lds + WS_NBUF * NBLK * 1024 + WS_NBUF * NBLK * 256);   // [NW*TPW][NBLK][64]
+    constexpr size_t OFF_D = static_cast<size_t>(WS_NBUF) * NBLK * 1024;
+    constexpr size_t OFF_WD = OFF_D + static_cast<size_t>(WS_NBUF) * NBLK * 128;
+    constexpr size_t OFF_READY = OFF_WD + static_cast<size_t>(NW) * TPW * NBLK * 128;
+    constexpr size_t OFF_WQ = OFF_READY + 16;
+    // activation scales [buffer][block][32 rows] and weight scales [wave][column tile][block][32 columns]:
+    // 64 consecutive floats are the operand of one scale MFMA over a pair of blocks
+    float (*lds_d)[NBLK * 32] = reinterpret_cast<float (*)[NBLK * 32]>(ws_lds + OFF_D);
+    float* lds_wd = reinterpret_cast<float*>(ws_lds + OFF_WD);
     // ready[b]: how many waves have written their share of the tile currently being put in buffer b
     // (counts up for the life of the kernel; the k-th filling of a buffer is complete at k * NW)
-    unsigned* lds_ready = reinterpret_cast<unsigned*>(ws_lds + WS_NBUF * NBLK * 1024 + WS_NBUF * NBLK * 256 +
-                                                      static_cast<size_t>(NW) * TPW * NBLK * 256);
+    unsigned* lds_ready = reinterpret_cast<unsigned*>(ws_lds + OFF_READY);
     // fragments of the last WL column tiles of every wave, when the register file cannot hold all TPW
-    v4i* lds_wq = reinterpret_cast<v4i*>(ws_lds + WS_NBUF * NBLK * 1024 + WS_NBUF * NBLK * 256 +
-                                         static_cast<size_t>(NW) * TPW * NBLK * 256 + 16);   // [NW][WL][NBLK][64]
+    v4i* lds_wq = reinterpret_cast<v4i*>(ws_lds + OFF_WQ);   // [NW][WL][NBLK][64]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -666,7 +664,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
     static_assert(WL >= 0 && WL < TPW, "at least one column tile stays in registers");
     v4i wq[TPW - WL][NBLK];
     v4i* my_wq = lds_wq + static_cast<size_t>(wave) * WL * NBLK * 64 + lane;
-    float* my_wd = lds_wd + static_cast<size_t>(wave) * TPW * NBLK * 64 + lane;
+    float* my_wd = lds_wd + static_cast<size_t>(wave) * TPW * NBLK * 32 + lane;
     {
         const uint16_t* dplane = reinterpret_cast<const uint16_t*>(W + static_cast<size_t>(mct_pad) * NBLK * 1024);
 #pragma unroll
@@ -679,12 +677,11 @@ __device__ __forceinline__ void q8_linear_ws_body(
                 if (t < TPW - WL) wq[t < TPW - WL ? t : 0][b] = frag;
                 else my_wq[((t - (TPW - WL)) * NBLK + b) * 64] = frag;
                 const float d = half_bits_to_float(dplane[(ct * NBLK + b) * 32 + j]);
-                my_wd[(t * NBLK + b) * 64] = hh ? 0.0f : d;
+                if (!hh) my_wd[(t * NBLK + b) * 32] = d;
             }
         }
     }
     PPML_TRACE_MARK(42);
-    for (int i = tid; i < WS_NBUF * NBLK * 64; i += NW * 64) (&lds_d[0][0])[i] = 0.0f;
     if (tid < WS_NBUF) lds_ready[tid] = 0u;
     __syncthreads();
     PPML_TRACE_MARK(43);
@@ -705,7 +702,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
             const BlockQuant bq = quantize_block_lane(x0, x1);
             uint2* dst = reinterpret_cast<uint2*>(lds_a[buf]) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
             *dst = uint2{bq.q_lo, bq.q_hi};
-            if (c4 == 0) lds_d[buf][bl * 64 + row] = half_bits_to_float(bq.d_bits);
+            if (c4 == 0) lds_d[buf][bl * 32 + row] = half_bits_to_float(bq.d_bits);
             if (DUMP && xq_dump) {
                 const int t = tok0 + row;
                 if (t < N) store_block_part(xq_dump + (static_cast<int64_t>(t) * NBLK + bl) * Q8_0_BYTES, c4, bq);
@@ -735,7 +732,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
     // its first use inside the loop wait for vmcnt(0), i.e. for all output stores, on every iteration.
     __builtin_amdgcn_s_waitcnt(0x0f70);                // vmcnt(0), other counters untouched
     // the second tile is requested now and quantized two thirds into the first one
-    if (tile + static_cast<int>(gridDim.x) < ntiles && !PPML_DBG(2)) load_tile_async(tile + static_cast<int>(gridDim.x));
+    if (tile + static_cast<int>(gridDim.x) < ntiles) load_tile_async(tile + static_cast<int>(gridDim.x));
     PPML_TRACE_MARK(1);
 
     // Step at which the next tile is quantized.  Its loads were issued one full round of column tiles
@@ -769,27 +766,34 @@ __device__ __forceinline__ void q8_linear_ws_body(
         v16f zero_f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) { zero_i[r] = 0; zero_f[r] = 0.0f; }
-        // Two result buffers used alternately: step st settles one while the MFMAs of step st+1
-        // fill the other.  Steps go in pairs so the buffers swap roles by name, not by copying.
+        // Per pair of blocks: two int8 MFMAs (exact block sums, one result buffer per parity) and one
+        // v_mfma_f32_32x32x1_2b_f32 whose two 32x32 outer products are the scale tables
+        // d_a[row] * d_w[col] of both blocks (each the exact product of two halves).
         v16i sum_a, sum_b;
-        v16f scl_a, scl_b;
+        v32f scl;
+        v32f zero_f2;
+#pragma unroll
+        for (int r = 0; r < 32; ++r) zero_f2[r] = 0.0f;
         v16f acc;
-        // LDS operands of one step, fetched a pair of steps ahead of the MFMAs that consume them
-        struct StepOps { v4i a; v4i w; float da; float dw; };
-        auto fetch = [&](int st, StepOps& o) {
+        // LDS operands of one pair of steps, fetched a pair ahead of the MFMAs that consume them
+        struct PairOps { v4i a0, a1, w0, w1; float da, dw; };
+        auto fetch_pair = [&](int st, PairOps& o) {
             const int t = st / NBLK, b = st % NBLK;
-            o.a = lds_a[buf][b * 64 + lane];
-            o.da = lds_d[buf][b * 64 + lane];
-            o.dw = my_wd[(t * NBLK + b) * 64];
-            if (t >= TPW - WL) o.w = my_wq[((t - (TPW - WL)) * NBLK + b) * 64];
+            o.a0 = lds_a[buf][b * 64 + lane];
+            o.a1 = lds_a[buf][(b + 1) * 64 + lane];
+            o.da = lds_d[buf][b * 32 + lane];          // lanes 0..31: rows of block b, 32..63: of block b + 1
+            o.dw = my_wd[(t * NBLK + b) * 32];
+            if (t >= TPW - WL) {
+                o.w0 = my_wq[((t - (TPW - WL)) * NBLK + b) * 64];
+                o.w1 = my_wq[((t - (TPW - WL)) * NBLK + b + 1) * 64];
+            }
         };
-        auto issue = [&](int st, const StepOps& o, v16i& sum, v16f& scl) {
+        auto block_sum = [&](int st, const v4i& a, const v4i& w_lds) {
             const int t = st / NBLK, b = st % NBLK;
-            const v4i w = t < TPW - WL ? wq[t < TPW - WL ? t : 0][b] : o.w;
-            sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.a, w, zero_i, 0, 0, 0);
-            scl = __builtin_amdgcn_mfma_f32_32x32x2f32(o.da, o.dw, zero_f, 0, 0, 0);
+            const v4i w = t < TPW - WL ? wq[t < TPW - WL ? t : 0][b] : w_lds;
+            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, w, zero_i, 0, 0, 0);
         };
-        auto settle = [&](int st, const v16i& sum, const v16f& scl) {
+        auto settle = [&](int st, const v16i& sum, const v16f scl) {
             const int t = st / NBLK, b = st % NBLK;
             if (b == 0) {
 #pragma unroll
@@ -806,7 +810,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
                     if (tok < N && m < M) sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b] = sum[r];
                 }
             }
-            if (b == NBLK - 1 && !PPML_DBG(0)) {
+            if (b == NBLK - 1) {
                 // The tile is complete: each half-wave store writes one full 128-byte line of a C
                 // row.  Buffer stores with a bounds-checked offset: lanes past the edge of C pass an
                 // offset beyond the buffer and are dropped by the hardware, so every wave issues
@@ -835,43 +839,45 @@ __device__ __forceinline__ void q8_linear_ws_body(
             // One basic block per column tile (see opaque_one()): the accumulator is born and stored
             // inside it, so nothing but loop state crosses the boundary.
             if (!opaque_one()) continue;
-            if (t0 * NBLK == QSTEP_TILE * NBLK && has_next && !PPML_DBG(3)) {
+            if (t0 * NBLK == QSTEP_TILE * NBLK && has_next) {
                 PPML_TRACE_MARK(2 + 10 * it + 7);
                 {
                     v4f xn[UPW][2];
                     if (it == 0) take_tile(std::integral_constant<int, NEWER_FIRST>{}, xn);
                     else take_tile(std::integral_constant<int, NEWER>{}, xn);
                     const int next2 = next + static_cast<int>(gridDim.x);
-                    if (next2 < ntiles && !PPML_DBG(2)) load_tile_async(next2);
+                    if (next2 < ntiles) load_tile_async(next2);
                     quantize_tile((it + 1) % WS_NBUF, next * TILE_TOK, xn);
                     announce((it + 1) % WS_NBUF);
                 }
                 PPML_TRACE_MARK(2 + 10 * it + 8);
             }
-            // Steps go in pairs: even steps use (ops_a, sum_a, scl_a), odd steps the b set, so the sets
-            // swap roles by name.  The MFMAs of a step are issued one settle ahead of their own, with
-            // operands that were fetched a pair ahead; the barriers keep the compiler from sinking
-            // them next to their consumers, where every settle would wait out a whole MFMA.
-            StepOps ops_a, ops_b;
-            fetch(t0 * NBLK, ops_a);
-            fetch(t0 * NBLK + 1, ops_b);
-            issue(t0 * NBLK, ops_a, sum_a, scl_a);
-            if (NBLK > 2) fetch(t0 * NBLK + 2, ops_a);
+            // Pairs of steps use the operand sets pe / po alternately, so they swap roles by name.  A
+            // pair starts by issuing its scale MFMA and the block sum of its second step; the block
+            // sum of the next pair's first step follows the first settle.  The barriers keep the
+            // compiler from sinking MFMAs next to their consumers, where every settle would wait
+            // out a whole MFMA; the one wait left per pair (for the scale table) is covered by the
+            // other wave of the SIMD.
+            PairOps pe, po;
+            const int s0 = t0 * NBLK;
+            fetch_pair(s0, pe);
+            if (NBLK > 2) fetch_pair(s0 + 2, po);
+            sum_a = block_sum(s0, pe.a0, pe.w0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int b0 = 0; b0 < NBLK; b0 += 2) {
-                const int st = t0 * NBLK + b0;
-                issue(st + 1, ops_b, sum_b, scl_b);
-                if (b0 + 3 < NBLK) fetch(st + 3, ops_b);
+            for (int pr = 0; pr < NBLK / 2; ++pr) {
+                const int st = s0 + 2 * pr;
+                PairOps& cur = (pr & 1) ? po : pe;
+                PairOps& nxt = (pr & 1) ? pe : po;
+                scl = __builtin_amdgcn_mfma_f32_32x32x1f32(cur.da, cur.dw, zero_f2, 0, 0, 0);
+                sum_b = block_sum(st + 1, cur.a1, cur.w1);
                 __builtin_amdgcn_sched_barrier(0);
-                settle(st, sum_a, scl_a);
+                settle(st, sum_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
                 __builtin_amdgcn_sched_barrier(0);
-                if (b0 + 2 < NBLK) {
-                    issue(st + 2, ops_a, sum_a, scl_a);
-                    if (b0 + 4 < NBLK) fetch(st + 4, ops_a);
-                }
+                if (2 * pr + 2 < NBLK) sum_a = block_sum(st + 2, nxt.a0, nxt.w0);
+                if (2 * pr + 4 < NBLK) fetch_pair(st + 4, cur);
                 __builtin_amdgcn_sched_barrier(0);
-                settle(st + 1, sum_b, scl_b);
+                settle(st + 1, sum_b, __builtin_shufflevector(scl, scl, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31));
                 __builtin_amdgcn_sched_barrier(0);
             }
             PPML_TRACE_MARK(2 + 10 * it + 1 + t0);
@@ -921,7 +927,7 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
     const int rounds = (ntiles + cus - 1) / cus;
     const int wgs = (ntiles + rounds - 1) / rounds;
     const dim3 grid(wgs), block(NW * 64);
-    constexpr size_t lds = WS_NBUF * NBLK * 1024 + WS_NBUF * NBLK * 256 + static_cast<size_t>(NW) * TPW * NBLK * 256 + 16 +
+    constexpr size_t lds = static_cast<size_t>(WS_NBUF) * NBLK * (1024 + 128) + static_cast<size_t>(NW) * TPW * NBLK * 128 + 16 +
                            static_cast<size_t>(NW) * WL * NBLK * 1024;
     using KernelFn = void (*)(const uint8_t*, const float*, float*, int, int, int, int, uint8_t*, int32_t*);
     KernelFn fast, dump;
