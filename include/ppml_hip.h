@@ -61,6 +61,13 @@ int mul_mat_hip(const float *A, const float *B, float *C, int M, int K, int N,
 int quantize_rows_q8_0_hip(const float *x, void *y, int64_t ne, ppml_hip_stream_t stream);
 /* replaces dequantize_q8_0_cuda (src/cuda/QuantKernels.cu:95-101). */
 int dequantize_q8_0_hip(const void *x, float *y, int64_t ne, ppml_hip_stream_t stream);
+/* replaces quantize_rows_q8_1_cuda (src/cuda/QuantKernels.cu:86-93), the activation quantizer of the
+ * reference's CUDA path: d = vmax / -128 with vmax the signed element of largest magnitude (first one
+ * on equal magnitudes, as the host loop include/ppml/QuantBlocks.h:81-111 picks it), quants clamped to
+ * [-128, 127], s = d * sum(quants).  y receives ne/32 block_q8_1 records (36 bytes). */
+int quantize_rows_q8_1_hip(const float *x, void *y, int64_t ne, ppml_hip_stream_t stream);
+/* replaces dequantize_q8_1_cuda (src/cuda/QuantKernels.cu:103-109). */
+int dequantize_q8_1_hip(const void *x, float *y, int64_t ne, ppml_hip_stream_t stream);
 
 /* Once-per-weight repack, the role repack_q8_0_host plays in the reference
  * (include/ppml/QuantBlocks.h:123-133, called from src/model/PPML.cpp:4504-4528).
@@ -82,6 +89,10 @@ int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K,
 /* The same kernel with its optional inputs and outputs exposed.
  *   flags bit 0: apply ReLU to X before quantizing (FeedForward: linear1 -> ReLU -> linear2,
  *                src/modules/Attention.cpp:1097-1104)
+ *   flags bit 1: quantize X with the Q8_1 rule of quantize_rows_q8_1_hip instead of the Q8_0 rule:
+ *                the numbers mul_mat_q8_cuda itself produces (src/cuda/MulMatQ8Kernel.cu:520-527
+ *                quantizes activations to Q8_1 and settles with their d).  Served by the general
+ *                kernel, not by the weight-stationary one.
  *   xq_dump  (may be NULL): receives the Q8_0 blocks the kernel made of X, [N][K/32] block_q8_0
  *   sums_dump(may be NULL): receives the per-block int32 sums, [(n*M+m)*(K/32)+ib]            */
 int mul_mat_q8_ex_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,

@@ -48,6 +48,9 @@ int ppml_hip_tensor_download(ppml_hip_backend *b, const ppml_hip_tensor *t, void
 int ppml_hip_backend_supports_op(const ppml_hip_backend *b, const ppml_hip_tensor *node);
 /* 1: a scheduler owns allocation, graph_compute allocates nothing (Backend.h skip_alloc_) */
 void ppml_hip_backend_set_skip_alloc(ppml_hip_backend *b, int on);
+/* 0: quantize activations with the Q8_0 rule (default, the CPU contract); 1: with the Q8_1 rule of
+ * the reference's CUDA launcher (src/cuda/MulMatQ8Kernel.cu:483-527) */
+void ppml_hip_backend_set_q8_1_activations(ppml_hip_backend *b, int on);
 int ppml_hip_backend_graph_compute(ppml_hip_backend *b, ppml_hip_tensor **nodes, int n);
 int ppml_hip_backend_pack_weight(ppml_hip_backend *b, ppml_hip_tensor *weight);
 

@@ -123,6 +123,10 @@ public:
     bool skip_alloc() const { return skip_alloc_; }
     void set_skip_alloc(bool v) { skip_alloc_ = v; }
     const std::string& last_error() const { return error_; }
+    // Rule the quantized mul_mat uses for its activations: false = Q8_0 (quantize_q8_0_host, the CPU
+    // contract), true = Q8_1 (what the reference's CUDA launcher does, src/cuda/MulMatQ8Kernel.cu:483-527).
+    void set_q8_1_activations(bool v) { q8_1_activations_ = v; }
+    bool q8_1_activations() const { return q8_1_activations_; }
 
     // Once-per-weight step of src/model/PPML.cpp:4504-4528: turns a Q8_0 / Q8_1 / Q8_0R weight node
     // into the MFMA-fragment layout in a buffer owned by this backend.
@@ -139,6 +143,7 @@ private:
 
     int device_;
     bool skip_alloc_ = false;
+    bool q8_1_activations_ = false;
     std::string error_;
     std::vector<std::unique_ptr<Buffer>> owned_;         // node outputs allocated here, packed weights
 };

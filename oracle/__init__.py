@@ -57,6 +57,10 @@ def _load() -> C.CDLL:
     lib.orc_mul_mat_q8q8.argtypes = [vp, vp, f32p] + [C.c_int] * 6
     lib.orc_mul_mat_q8.restype = C.c_int
     lib.orc_mul_mat_q8.argtypes = [vp, f32p, f32p] + [C.c_int] * 7
+    lib.orc_quantize_q8_1.restype = C.c_int
+    lib.orc_quantize_q8_1.argtypes = [f32p, vp, i64]
+    lib.orc_mul_mat_q8_act.restype = C.c_int
+    lib.orc_mul_mat_q8_act.argtypes = [vp, f32p, f32p] + [C.c_int] * 8
     lib.orc_mul_mat_f32.restype = None
     lib.orc_mul_mat_f32.argtypes = [f32p, f32p, f32p, C.c_int, C.c_int, C.c_int, f32p, C.c_int]
     lib.orc_out_prod.restype = None
@@ -197,6 +201,31 @@ def mul_mat_q8(w, x, wtype=0, c_trans=1, fma=1, nthreads=0) -> np.ndarray:
     rc = lib().orc_mul_mat_q8(_vp(w), _fp(x), _fp(out), M, N, K, wtype, c_trans, fma, nthreads)
     if rc:
         raise RuntimeError(f"orc_mul_mat_q8 rc={rc}")
+    return out
+
+
+def quantize_q8_1(x) -> np.ndarray:
+    """f32 [..., K] -> uint8 [..., K/32, 36] block_q8_1 records (QuantBlocks.h:81-111)."""
+    x = _f32(x)
+    n = x.size
+    if n % QK:
+        raise ValueError("element count is not a multiple of 32")
+    out = np.empty((n // QK, 36), dtype=np.uint8)
+    rc = lib().orc_quantize_q8_1(_fp(x), _vp(out), n)
+    assert rc == 0
+    return out.reshape(x.shape[:-1] + (x.shape[-1] // QK, 36))
+
+
+def mul_mat_q8_act(w, x, act=1, wtype=0, c_trans=1, fma=1, nthreads=0) -> np.ndarray:
+    """mul_mat_q8 with the activation rule selectable (0 = Q8_0, 1 = Q8_1)."""
+    x = _f32(x)
+    N, K = x.shape
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    M = w.size // (K // QK * BLOCK_BYTES)
+    out = np.empty((N, M) if c_trans else (M, N), dtype=np.float32)
+    rc = lib().orc_mul_mat_q8_act(_vp(w), _fp(x), _fp(out), M, N, K, wtype, c_trans, fma, act, nthreads)
+    if rc:
+        raise RuntimeError(f"orc_mul_mat_q8_act rc={rc}")
     return out
 
 

@@ -255,6 +255,73 @@ int orc_mul_mat_q8(const void *W, const float *X, float *C, int M, int N, int K,
     return rc;
 }
 
+/* include/ppml/QuantBlocks.h:81-111 (host) and src/cuda/QuantKernels.cu:29-62 (device): the
+ * activation quantizer of the reference's CUDA path.  Records are {half d, half s, int8 qs[32]}.
+ * vmax is the first element (lowest index) that reaches the largest magnitude (strict `>` scan);
+ * d = vmax / -128 keeps its sign; an all-zero block stores +0; quants clamp to [-128, 127];
+ * s = half(d * float(sum of quants)) with the binary32 d. */
+int orc_quantize_q8_1(const float *src, void *dst_blocks, int64_t n) {
+    if (!src || !dst_blocks || n < 0 || n % ORC_QK8_0) return 1;
+    uint8_t *out = (uint8_t *)dst_blocks;
+    for (int64_t b = 0; b < n / ORC_QK8_0; ++b) {
+        const float *x = src + b * ORC_QK8_0;
+        float amax = 0.0f, vmax = 0.0f;
+        for (int i = 0; i < ORC_QK8_0; ++i) {
+            const float v = x[i];
+            if (fabsf(v) > amax) { amax = fabsf(v); vmax = v; }
+        }
+        const float d = (amax == 0.0f) ? 0.0f : vmax / -128.0f;
+        const float inv = (d == 0.0f) ? 0.0f : 1.0f / d;
+        int32_t qsum = 0;
+        uint8_t *blk = out + b * 36;
+        for (int i = 0; i < ORC_QK8_0; ++i) {
+            float q = roundf(x[i] * inv);
+            q = q > 127.0f ? 127.0f : (q < -128.0f ? -128.0f : q);
+            const int8_t qi = (int8_t)q;
+            blk[4 + i] = (uint8_t)qi;
+            qsum += qi;
+        }
+        const uint16_t dh = orc_fp32_to_fp16(d), sh = orc_fp32_to_fp16(d * (float)qsum);
+        memcpy(blk, &dh, 2);
+        memcpy(blk + 2, &sh, 2);
+    }
+    return 0;
+}
+
+/* The numbers mul_mat_q8_cuda produces (src/cuda/MulMatQ8Kernel.cu:483-527): activations quantized
+ * with the Q8_1 rule above, each block settled with the halves d_w and d_a exactly like the Q8_0
+ * path (120-142); s is not read.  act: 0 = Q8_0 activations (orc_mul_mat_q8), 1 = Q8_1. */
+int orc_mul_mat_q8_act(const void *W, const float *X, float *C, int M, int N, int K,
+                       int wtype, int c_trans, int fma, int act, int nthreads) {
+    if (act == 0) return orc_mul_mat_q8(W, X, C, M, N, K, wtype, c_trans, fma, nthreads);
+    if (act != 1) return 1;
+    if (!W || !X || !C || M <= 0 || N <= 0 || K <= 0) return 1;
+    if (K % ORC_QK8_0) return 2;
+    if (wtype != 0 && wtype != 2) return 5;
+    const int64_t nblk = K / ORC_QK8_0;
+    uint8_t *x1 = (uint8_t *)malloc((size_t)N * nblk * 36);
+    uint8_t *xq = (uint8_t *)malloc((size_t)N * nblk * ORC_Q8_0_BLOCK_BYTES);
+    uint8_t *wq = NULL;
+    if (!x1 || !xq) { free(x1); free(xq); return 3; }
+    const void *wblocks = W;
+    if (wtype == 2) {
+        wq = (uint8_t *)malloc((size_t)M * nblk * ORC_Q8_0_BLOCK_BYTES);
+        if (!wq) { free(x1); free(xq); return 3; }
+        orc_unrepack_q8_0(W, (int64_t)M * nblk, wq);
+        wblocks = wq;
+    }
+    orc_quantize_q8_1(X, x1, (int64_t)N * K);
+    for (int64_t b = 0; b < (int64_t)N * nblk; ++b) {            /* {d, s, qs} -> {d, qs} */
+        memcpy(xq + b * ORC_Q8_0_BLOCK_BYTES, x1 + b * 36, 2);
+        memcpy(xq + b * ORC_Q8_0_BLOCK_BYTES + 2, x1 + b * 36 + 4, 32);
+    }
+    const int rc = orc_mul_mat_q8q8(wblocks, xq, C, M, N, K, c_trans, fma, nthreads);
+    free(x1);
+    free(xq);
+    free(wq);
+    return rc;
+}
+
 /* ------------------------------------------------------------------ f32 */
 /* src/backend/CPUKernels.cpp:763-771: rows handed out one at a time, bias enters the
  * accumulator first, k ascending, separate multiply and add. */

@@ -54,6 +54,14 @@ int  orc_mul_mat_q8q8(const void *w_blocks, const void *x_blocks, float *C,
 int  orc_mul_mat_q8(const void *W, const float *X, float *C, int M, int N, int K,
                     int wtype, int c_trans, int fma, int nthreads);
 
+/* include/ppml/QuantBlocks.h:81-111: the activation quantizer of the reference's CUDA path;
+ * dst receives n/32 block_q8_1 records {fp16 d; fp16 s; int8 qs[32]} (36 bytes). */
+int  orc_quantize_q8_1(const float *src, void *dst_blocks, int64_t n);
+/* orc_mul_mat_q8 with the activation rule selectable: act 0 = Q8_0 (CPU contract), 1 = Q8_1 (what
+ * mul_mat_q8_cuda computes, src/cuda/MulMatQ8Kernel.cu:483-527). */
+int  orc_mul_mat_q8_act(const void *W, const float *X, float *C, int M, int N, int K,
+                        int wtype, int c_trans, int fma, int act, int nthreads);
+
 /* src/backend/CPUKernels.cpp:763-771 ; bias may be NULL */
 void orc_mul_mat_f32(const float *a, const float *b, float *d, int M, int K, int N,
                      const float *bias, int nthreads);

@@ -22,6 +22,8 @@ SIGNATURES = {
     "mul_mat_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "quantize_rows_q8_0_hip": (_i, [_vp, _vp, _i64, _vp]),
     "dequantize_q8_0_hip": (_i, [_vp, _vp, _i64, _vp]),
+    "quantize_rows_q8_1_hip": (_i, [_vp, _vp, _i64, _vp]),
+    "dequantize_q8_1_hip": (_i, [_vp, _vp, _i64, _vp]),
     "q8_weight_packed_bytes_hip": (C.c_size_t, [_i, _i]),
     "q8_weight_pack_hip": (_i, [_vp, _i, _i, _i, _vp, _vp]),
     "mul_mat_q8_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, C.POINTER(_i), _vp]),
@@ -54,6 +56,7 @@ BACKEND_SIGNATURES = {
     "ppml_hip_tensor_download": (_i, [_vp, _vp, _vp, C.c_size_t]),
     "ppml_hip_backend_supports_op": (_i, [_vp, _vp]),
     "ppml_hip_backend_set_skip_alloc": (None, [_vp, _i]),
+    "ppml_hip_backend_set_q8_1_activations": (None, [_vp, _i]),
     "ppml_hip_backend_graph_compute": (_i, [_vp, C.POINTER(_vp), _i]),
     "ppml_hip_backend_pack_weight": (_i, [_vp, _vp]),
 }

@@ -229,10 +229,9 @@ Status HipBackend::kernel_mul_mat(Tensor* node) {
         // weight rows are the out features: with the weight in src0 they index the node's dims[1]
         const int64_t Mq = q0 ? M : N, Nq = q0 ? N : M;
         const int c_trans = q0 ? 0 : 1;
-        int path = 0;
-        rc = mul_mat_q8_hip(w->data, static_cast<const float*>(a->data), static_cast<float*>(node->data),
-                            static_cast<int>(Mq), static_cast<int>(Nq), static_cast<int>(K), wtype, c_trans, &path,
-                            nullptr);
+        rc = mul_mat_q8_ex_hip(w->data, static_cast<const float*>(a->data), static_cast<float*>(node->data),
+                               static_cast<int>(Mq), static_cast<int>(Nq), static_cast<int>(K), wtype, c_trans,
+                               q8_1_activations_ ? 2 : 0, nullptr, nullptr, nullptr);
     } else {
         if (s0->type != TENSOR_TYPE_F32 || s1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32)
             return fail(Status::NOT_SUPPORTED, "mul_mat: only F32 x F32 -> F32 besides the quantized path");
@@ -453,6 +452,9 @@ int ppml_hip_backend_graph_compute(ppml_hip_backend* b, ppml_hip_tensor** nodes,
 int ppml_hip_backend_pack_weight(ppml_hip_backend* b, ppml_hip_tensor* weight) {
     if (!b || !weight) return static_cast<int>(Status::NOT_SUPPORTED);
     return static_cast<int>(b->impl.pack_weight(&weight->t));
+}
+void ppml_hip_backend_set_q8_1_activations(ppml_hip_backend* b, int on) {
+    if (b) b->impl.set_q8_1_activations(on != 0);
 }
 void ppml_hip_backend_set_skip_alloc(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_skip_alloc(on != 0);

@@ -29,6 +29,7 @@ __device__ __forceinline__ float group4_max(float v) {
 struct BlockQuant {
     uint32_t q_lo, q_hi;  // this lane's 8 quants, element c in byte c % 4 of word c / 4
     uint16_t d_bits;      // fp16 scale of the block
+    float d;              // the same scale before rounding to half
 };
 
 // round(t) for |t| <= 200 as one add and one truncating convert: adding the largest float below
@@ -46,28 +47,69 @@ __device__ __forceinline__ uint32_t pack4(int a, int b, int c, int d) {
     return __builtin_amdgcn_perm(cd, ab, 0x05040100u);
 }
 
+// (|v|, v) of the first element of the block that reaches the block's largest magnitude, combined
+// over an aligned group of 4 lanes that hold the block in element order: on equal magnitudes the
+// lower lane wins, as the sequential scan with a strict `>` does (include/ppml/QuantBlocks.h:86-90).
+__device__ __forceinline__ void group4_first_max(float& a, float& v) {
+    const int lane = static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
+    {
+        const float oa = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(a), 0xB1, 0xf, 0xf, false));
+        const float ov = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));
+        const bool low = (lane & 1) == 0;              // this lane is the lower one of the pair
+        const bool keep = low ? (a >= oa) : (a > oa);
+        v = keep ? v : ov;
+        a = keep ? a : oa;
+    }
+    {
+        const float oa = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(a), 0x4E, 0xf, 0xf, false));
+        const float ov = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));
+        const bool low = (lane & 2) == 0;
+        const bool keep = low ? (a >= oa) : (a > oa);
+        v = keep ? v : ov;
+        a = keep ? a : oa;
+    }
+}
+
 // x0,x1 hold elements 8*c4 .. 8*c4+7 of one 32-element block, the 4 lanes of an aligned group hold
-// the whole block.  IEEE division for the scale and its reciprocal, round half away from zero,
-// clamp to +-127 (include/ppml/QuantBlocks.h:62-79).
-__device__ __forceinline__ BlockQuant quantize_block_lane(v4f x0, v4f x1) {
-    float amax = 0.0f;
+// the whole block.  IEEE division for the scale and its reciprocal, round half away from zero.
+//   Q81 = false: d = amax / 127, clamp to +-127             (include/ppml/QuantBlocks.h:62-79)
+//   Q81 = true : d = vmax / -128 with vmax the signed element of largest magnitude, clamp to
+//                [-128, 127]; *qsum receives this lane's share of the sum of the quants
+//                                                            (include/ppml/QuantBlocks.h:81-111)
+template <bool Q81>
+__device__ __forceinline__ BlockQuant quantize_block_lane(v4f x0, v4f x1, int* qsum = nullptr) {
+    float amax = 0.0f, vmax = 0.0f;
+    if (Q81) {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) amax = fmaxf(amax, fabsf(x0[c]));   // fmaxf drops NaN like std::fmax
+        for (int c = 0; c < 8; ++c) {
+            const float x = c < 4 ? x0[c & 3] : x1[c & 3];
+            const bool gt = fabsf(x) > amax;            // false for NaN: ignored like the host's scan
+            vmax = gt ? x : vmax;
+            amax = gt ? fabsf(x) : amax;
+        }
+        group4_first_max(amax, vmax);
+    } else {
 #pragma unroll
-    for (int c = 0; c < 4; ++c) amax = fmaxf(amax, fabsf(x1[c]));
-    amax = group4_max(amax);
-    const float d = amax / 127.0f;
-    const float inv = (amax == 0.0f) ? 0.0f : 1.0f / d;
+        for (int c = 0; c < 4; ++c) amax = fmaxf(amax, fabsf(x0[c]));   // fmaxf drops NaN like std::fmax
+#pragma unroll
+        for (int c = 0; c < 4; ++c) amax = fmaxf(amax, fabsf(x1[c]));
+        amax = group4_max(amax);
+    }
+    const float d = Q81 ? ((amax == 0.0f) ? 0.0f : vmax / -128.0f) : amax / 127.0f;
+    const float inv = (Q81 ? d == 0.0f : amax == 0.0f) ? 0.0f : 1.0f / d;
     BlockQuant out;
     out.d_bits = __half_as_ushort(__float2half_rn(d));
+    out.d = d;
     int q[8];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         q[c] = round_half_away_to_int(x0[c] * inv);
         q[4 + c] = round_half_away_to_int(x1[c] * inv);
     }
+    constexpr int QMIN = Q81 ? -128 : -127;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) q[c] = q[c] > 127 ? 127 : (q[c] < -127 ? -127 : q[c]);
+    for (int c = 0; c < 8; ++c) q[c] = q[c] > 127 ? 127 : (q[c] < QMIN ? QMIN : q[c]);
+    if (Q81 && qsum) *qsum = q[0] + q[1] + q[2] + q[3] + q[4] + q[5] + q[6] + q[7];
     out.q_lo = pack4(q[0], q[1], q[2], q[3]);
     out.q_hi = pack4(q[4], q[5], q[6], q[7]);
     return out;
@@ -101,7 +143,7 @@ __global__ __launch_bounds__(256) void quantize_rows_q8_0_kernel(const float* __
     const float* src = x + ib * QK + c4 * 8;
     const v4f x0 = *reinterpret_cast<const v4f_u*>(src);
     const v4f x1 = *reinterpret_cast<const v4f_u*>(src + 4);
-    const BlockQuant bq = quantize_block_lane(x0, x1);
+    const BlockQuant bq = quantize_block_lane<false>(x0, x1);
     if (!live) return;
     store_block_part(y + ib * Q8_0_BYTES, c4, bq);
 }
@@ -115,6 +157,45 @@ __global__ __launch_bounds__(256) void dequantize_q8_0_kernel(const uint8_t* __r
     const uint8_t* blk = x + ib * Q8_0_BYTES;
     const float d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(blk));
     y[i] = d * static_cast<float>(static_cast<int8_t>(blk[2 + iq]));
+}
+
+// Q8_1 records {half d, half s, int8 qs[32]} (include/ppml/QuantBlocks.h:38-41), s = d * sum(qs)
+__global__ __launch_bounds__(256) void quantize_rows_q8_1_kernel(const float* __restrict__ x,
+                                                                 uint8_t* __restrict__ y,
+                                                                 int64_t nblocks) {
+    const int64_t t = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    int64_t ib = t >> 2;
+    const int c4 = static_cast<int>(t & 3);
+    const bool live = ib < nblocks;
+    if (!live) ib = nblocks - 1;                       // keep the whole 4-lane group convergent
+    const float* src = x + ib * QK + c4 * 8;
+    const v4f x0 = *reinterpret_cast<const v4f_u*>(src);
+    const v4f x1 = *reinterpret_cast<const v4f_u*>(src + 4);
+    int qsum = 0;
+    const BlockQuant bq = quantize_block_lane<true>(x0, x1, &qsum);
+    qsum += __builtin_amdgcn_update_dpp(0, qsum, 0xB1, 0xf, 0xf, false);   // lane ^ 1
+    qsum += __builtin_amdgcn_update_dpp(0, qsum, 0x4E, 0xf, 0xf, false);   // lane ^ 2
+    if (!live) return;
+    uint8_t* blk = y + ib * Q8_1_BYTES;
+    uint32_t* q32 = reinterpret_cast<uint32_t*>(blk + 4 + c4 * 8);       // records are 4-byte aligned
+    q32[0] = bq.q_lo;
+    q32[1] = bq.q_hi;
+    if (c4 == 0) {
+        // s is made from the fp32 scale, like the reference: d * float(sum), then one rounding to half
+        reinterpret_cast<uint16_t*>(blk)[0] = bq.d_bits;
+        reinterpret_cast<uint16_t*>(blk)[1] = __half_as_ushort(__float2half_rn(bq.d * static_cast<float>(qsum)));
+    }
+}
+
+__global__ __launch_bounds__(256) void dequantize_q8_1_kernel(const uint8_t* __restrict__ x,
+                                                              float* __restrict__ y, int64_t ne) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= ne) return;
+    const int64_t ib = i / QK;
+    const int iq = static_cast<int>(i - ib * QK);
+    const uint8_t* blk = x + ib * Q8_1_BYTES;
+    const float d = half_bits_to_float(*reinterpret_cast<const uint16_t*>(blk));
+    y[i] = d * static_cast<float>(static_cast<int8_t>(blk[4 + iq]));
 }
 
 // ------------------------------------------------------------------------------------------
@@ -389,11 +470,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
                     const int row = (u & 3) * 8 + urow;
                     const int bl = (u >> 2) * 2 + ublk;
                     v4f x0 = xv[s][0], x1 = xv[s][1];
-                    if (relu) {
+                    if (relu & 1) {
 #pragma unroll
                         for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
                     }
-                    const BlockQuant bq = quantize_block_lane(x0, x1);
+                    const BlockQuant bq = (relu & 2) ? quantize_block_lane<true>(x0, x1) : quantize_block_lane<false>(x0, x1);
                     if (bl < nb) {
                         // fragment order: block bl, k-half c4/2, row, dword pair c4%2
                         uint2* dst = reinterpret_cast<uint2*>(lds_a) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
@@ -699,7 +780,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
 #pragma unroll
                 for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
             }
-            const BlockQuant bq = quantize_block_lane(x0, x1);
+            const BlockQuant bq = quantize_block_lane<false>(x0, x1);
             uint2* dst = reinterpret_cast<uint2*>(lds_a[buf]) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
             *dst = uint2{bq.q_lo, bq.q_hi};
             if (c4 == 0) lds_d[buf][bl * 32 + row] = half_bits_to_float(bq.d_bits);
@@ -1004,6 +1085,23 @@ extern "C" int dequantize_q8_0_hip(const void* x, float* y, int64_t ne, ppml_hip
     return check_launch("dequantize_q8_0_kernel") ? RC_BAD_ARGS : RC_OK;
 }
 
+extern "C" int quantize_rows_q8_1_hip(const float* x, void* y, int64_t ne, ppml_hip_stream_t stream) {
+    if (!x || !y || ne <= 0 || (ne % QK) != 0) { set_error("quantize_rows_q8_1_hip: bad arguments (ne=%lld)", (long long)ne); return RC_BAD_ARGS; }
+    const int64_t nblocks = ne / QK;
+    const unsigned grid = static_cast<unsigned>((nblocks * 4 + 255) / 256);
+    hipLaunchKernelGGL(quantize_rows_q8_1_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       x, static_cast<uint8_t*>(y), nblocks);
+    return check_launch("quantize_rows_q8_1_kernel") ? RC_BAD_ARGS : RC_OK;   // reference launcher: 0 / 1
+}
+
+extern "C" int dequantize_q8_1_hip(const void* x, float* y, int64_t ne, ppml_hip_stream_t stream) {
+    if (!x || !y || ne <= 0) { set_error("dequantize_q8_1_hip: bad arguments"); return RC_BAD_ARGS; }
+    const unsigned grid = static_cast<unsigned>((ne + 255) / 256);
+    hipLaunchKernelGGL(dequantize_q8_1_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t*>(x), y, ne);
+    return check_launch("dequantize_q8_1_kernel") ? RC_BAD_ARGS : RC_OK;
+}
+
 extern "C" size_t q8_weight_packed_bytes_hip(int M, int K) {
     if (M <= 0 || K <= 0 || (K % QK) != 0) return 0;
     const size_t tiles = static_cast<size_t>(packed_tiles(M));
@@ -1033,17 +1131,20 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
     if (!W || !X || !C || M <= 0 || N <= 0 || K <= 0) { set_error("mul_mat_q8_hip: bad arguments (M=%d N=%d K=%d)", M, N, K); return RC_BAD_ARGS; }
     if ((K % QK) != 0) { set_error("mul_mat_q8_hip: K=%d is not a multiple of 32", K); return RC_K_NOT_32; }
     const int nblk = K / QK;
-    const int relu = flags & 1;
+    const int relu = flags & 1;                        // bit 0: ReLU on X
+    const int act = flags & 3;                         // bit 1: Q8_1 rule for the activations (general kernel only)
     hipStream_t s = static_cast<hipStream_t>(stream);
     stats_record(M, K, N);
     switch (wtype) {
-        case PPML_WTYPE_Q8_0:  return dispatch_q8_linear<PPML_WTYPE_Q8_0>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
-        case PPML_WTYPE_Q8_1:  return dispatch_q8_linear<PPML_WTYPE_Q8_1>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
-        case PPML_WTYPE_Q8_0R: return dispatch_q8_linear<PPML_WTYPE_Q8_0R>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
+        case PPML_WTYPE_Q8_0:  return dispatch_q8_linear<PPML_WTYPE_Q8_0>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
+        case PPML_WTYPE_Q8_1:  return dispatch_q8_linear<PPML_WTYPE_Q8_1>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
+        case PPML_WTYPE_Q8_0R: return dispatch_q8_linear<PPML_WTYPE_Q8_0R>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0M: {
-            const int rc = try_q8_linear_ws(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
-            if (rc >= 0) return rc;
-            return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
+            if (!(act & 2)) {
+                const int rc = try_q8_linear_ws(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
+                if (rc >= 0) return rc;
+            }
+            return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         }
         default: set_error("mul_mat_q8_hip: unsupported wtype %d", wtype); return RC_WTYPE;
     }

@@ -151,6 +151,28 @@ def quantize_rows_q8_0(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def quantize_rows_q8_1(x: torch.Tensor) -> torch.Tensor:
+    """f32 [..., K] -> uint8 [..., K/32, 36] block_q8_1 records, the reference's activation quantizer
+    (include/ppml/QuantBlocks.h:81-111): d = vmax / -128, quants in [-128, 127], s = d * sum(q)."""
+    x = _dev_f32(x, "x")
+    ne = x.numel()
+    if x.shape[-1] % QK:
+        raise ValueError("quantize_rows_q8_1: innermost dimension is not a multiple of 32")
+    out = torch.empty(x.shape[:-1] + (x.shape[-1] // QK, 36), dtype=torch.uint8, device=x.device)
+    cabi.check("quantize_rows_q8_1_hip", _lib().quantize_rows_q8_1_hip(_ptr(x), _ptr(out), ne, _stream()))
+    return out
+
+
+def dequantize_q8_1(blocks: torch.Tensor) -> torch.Tensor:
+    if not blocks.is_cuda or blocks.dtype != torch.uint8 or blocks.shape[-1] != 36:
+        raise TypeError("dequantize_q8_1 expects uint8 [..., nblocks, 36] on the device")
+    blocks = blocks.contiguous()
+    nb = blocks.numel() // 36
+    out = torch.empty(blocks.shape[:-2] + (blocks.shape[-2] * QK,), dtype=torch.float32, device=blocks.device)
+    cabi.check("dequantize_q8_1_hip", _lib().dequantize_q8_1_hip(_ptr(blocks), _ptr(out), nb * QK, _stream()))
+    return out
+
+
 def dequantize_q8_0(blocks: torch.Tensor) -> torch.Tensor:
     if not blocks.is_cuda or blocks.dtype != torch.uint8 or blocks.shape[-1] != BLOCK_BYTES:
         raise TypeError("dequantize_q8_0 expects uint8 [..., nblocks, 34] on the device")
@@ -191,10 +213,14 @@ class Q8Weight:
 
 
 def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = False,
-               dump: bool = False):
+               dump: bool = False, act: str = "q8_0"):
     """Q8_0 linear: x f32 [N,K] (rows = tokens) times quantized w [M,K] -> [N,M] (c_trans=1, the
     LinearLayer orientation) or [M,N] (c_trans=0); src/backend/CUDAKernels.cpp:740-789.
-    With ``dump`` also returns the kernel's own Q8_0 blocks of x and its per-block int32 sums."""
+    With ``dump`` also returns the kernel's own Q8_0 blocks of x and its per-block int32 sums.
+    ``act`` selects the rule the activations are quantized with: "q8_0" (the CPU contract) or
+    "q8_1" (what the reference's CUDA launcher does, src/cuda/MulMatQ8Kernel.cu:483-527)."""
+    if act not in ("q8_0", "q8_1"):
+        raise ValueError("mul_mat_q8: act must be 'q8_0' or 'q8_1'")
     x = _dev_f32(x, "x")
     if x.dim() != 2 or x.shape[1] != w.K:
         raise ValueError(f"mul_mat_q8: activations {tuple(x.shape)} do not match weight K={w.K}")
@@ -202,7 +228,7 @@ def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = Fals
     M = w.M
     out = torch.empty((N, M) if c_trans else (M, N), dtype=torch.float32, device=x.device)
     lib = _lib()
-    if not dump and not relu:
+    if not dump and not relu and act == "q8_0":
         path = C.c_int(0)
         cabi.check("mul_mat_q8_hip", lib.mul_mat_q8_hip(_ptr(w.data), _ptr(x), _ptr(out), M, N, K, w.wtype,
                                                          c_trans, C.byref(path), _stream()))
@@ -212,5 +238,6 @@ def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = Fals
         xq = torch.empty((N, K // QK, BLOCK_BYTES), dtype=torch.uint8, device=x.device)
         sums = torch.empty((N, M, K // QK), dtype=torch.int32, device=x.device)
     cabi.check("mul_mat_q8_ex_hip", lib.mul_mat_q8_ex_hip(_ptr(w.data), _ptr(x), _ptr(out), M, N, K, w.wtype,
-                                                           c_trans, 1 if relu else 0, _ptr(xq), _ptr(sums), _stream()))
+                                                           c_trans, (1 if relu else 0) | (2 if act == "q8_1" else 0),
+                                                           _ptr(xq), _ptr(sums), _stream()))
     return (out, xq, sums) if dump else out

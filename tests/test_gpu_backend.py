@@ -69,6 +69,23 @@ def test_quantized_mul_mat_node(be, oracle, wname, wside):
     np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6 * np.abs(want).max())
 
 
+def test_quantized_mul_mat_node_with_cuda_activation_rule(be, oracle):
+    rows, K, F = 50, 64, 40
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((rows, K)).astype(np.float32)
+    wq = oracle.quantize_q8_0((rng.standard_normal((F, K)) * 0.02).astype(np.float32))
+    wt = _leaf(be, np.frombuffer(wq.tobytes(), np.uint8), B.Q8_0, (K, F))
+    xt = _leaf(be, x)
+    be.set_q8_1_activations(True)
+    try:
+        got = be_run(be, B.Tensor((F, rows), B.F32, B.OP_MUL_MAT, [xt, wt])).reshape(rows, F)
+    finally:
+        be.set_q8_1_activations(False)
+    assert (got == oracle.mul_mat_q8_act(wq, x, act=1)).all()
+    got0 = be_run(be, B.Tensor((F, rows), B.F32, B.OP_MUL_MAT, [xt, wt])).reshape(rows, F)
+    assert (got0 == oracle.mul_mat_q8(wq, x)).all()
+
+
 def be_run(be, node):
     assert be.supports_op(node)
     assert be.graph_compute([node]) == B.SUCCESS, be.last_error

@@ -228,3 +228,58 @@ def test_msa_qkv_shape_full_size_properties(ops, oracle):
     # and the result approximates the unquantized product to quantization accuracy
     full = x[idx].astype(np.float64) @ w.astype(np.float64).T
     assert np.abs(got[idx] - full).max() <= 0.03 * np.abs(full).max()
+
+
+# ----------------------------------------------------------------------------- Q8_1 activation rule
+@pytest.mark.parametrize("rows,K,scale", [(408, 256, 1.0), (7, 32, 1.0), (33, 96, 0.02), (2000, 128, 1.0),
+                                          (5, 2048, 1e-6), (3, 64, 1e4)])
+def test_quantize_rows_q8_1_bit_exact(ops, oracle, rows, K, scale):
+    # the activation quantizer of the reference's CUDA path (include/ppml/QuantBlocks.h:81-111):
+    # d, s and every quant byte for byte
+    rng = np.random.default_rng(rows * 77 + K)
+    x = (rng.standard_normal((rows, K)) * scale).astype(np.float32)
+    x[0, :32] = 0.0                                   # zero block stores +0
+    x[rows - 1, 3], x[rows - 1, 9] = 5.0, -5.0        # equal magnitudes: the first one gives the sign
+    x[rows - 1, K - 32 + 30], x[rows - 1, K - 32 + 2] = 6.0, -6.0
+    x[rows // 2, 7] = np.nan                          # ignored by the scan
+    got = ops.quantize_rows_q8_1(_dev(x)).cpu().numpy()
+    want = oracle.quantize_q8_1(x)
+    assert got.shape == want.shape == (rows, K // 32, 36)
+    nan_blk = (rows // 2, 0)
+    mask = np.ones(got.shape[:2], bool)
+    mask[nan_blk] = False                             # (int8)NaN is not portable: compare that block apart
+    assert (got[mask] == want[mask]).all()
+    assert (got[nan_blk][:2] == want[nan_blk][:2]).all()      # its scale comes from the finite elements
+    back = ops.dequantize_q8_1(_dev(want)).cpu().numpy()
+    d = np.ascontiguousarray(want[..., 0:2]).view(np.float16)[..., 0].astype(np.float32)
+    q = np.ascontiguousarray(want[..., 4:]).view(np.int8).astype(np.float32)
+    assert (back.reshape(rows, K // 32, 32) == d[..., None] * q).all()
+
+
+@pytest.mark.parametrize("wname", ["Q8_0", "Q8_0R", "packed"])
+@pytest.mark.parametrize("N,K,M,c_trans", [(408, 256, 256, 1), (77, 128, 96, 0), (300, 512, 128, 1), (1000, 256, 768, 1)])
+def test_fused_linear_with_q8_1_activations(ops, oracle, wname, N, K, M, c_trans):
+    # what mul_mat_q8_cuda computes (src/cuda/MulMatQ8Kernel.cu:483-527): Q8_1 activations, same
+    # per-block settlement.  Internals and output bit for bit.
+    x, w = _inputs(N + K + M, N, K, M)
+    x[N // 2] *= -3.0
+    wq = oracle.quantize_q8_0(w)
+    if wname == "Q8_0R":
+        W = ops.Q8Weight(_dev(oracle.repack_q8_0(wq)), M, K, 2)
+    else:
+        W = ops.Q8Weight(_dev(wq.reshape(-1)), M, K, 0)
+        if wname == "packed":
+            W = W.pack()
+    y, xq, sums = ops.mul_mat_q8(W, _dev(x), c_trans=c_trans, dump=True, act="q8_1")
+    x1 = oracle.quantize_q8_1(x)
+    want_xq = np.ascontiguousarray(np.concatenate([x1[..., 0:2], x1[..., 4:]], axis=-1))
+    assert (xq.cpu().numpy() == want_xq).all()
+    assert (sums.cpu().numpy() == oracle.q8_block_sums(wq, want_xq)).all()
+    want = oracle.mul_mat_q8_act(wq, x, act=1, c_trans=c_trans)
+    got = y.cpu().numpy()
+    assert _rel_err(got, want) <= 1e-5
+    assert (got == want).all()
+    # without the dump, and the two rules really differ
+    y2 = ops.mul_mat_q8(W, _dev(x), c_trans=c_trans, act="q8_1").cpu().numpy()
+    assert (y2 == want).all()
+    assert (ops.mul_mat_q8(W, _dev(x), c_trans=c_trans).cpu().numpy() != want).any()

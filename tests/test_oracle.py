@@ -157,6 +157,57 @@ def test_dequantize_closed_form(oracle):
     assert (oracle.dequantize_q8_0(blk) == want).all()
 
 
+# ----------------------------------------------------------------------------- Q8_1 activations
+def test_quantize_q8_1_rule(oracle):
+    # include/ppml/QuantBlocks.h:81-111: d = vmax / -128 keeps the sign of the largest element,
+    # which therefore maps to -128; on equal magnitudes the FIRST element decides the sign;
+    # the opposite extreme saturates at +127; s = half(d * sum q) from the binary32 d.
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((40, 32)).astype(np.float32)
+    x[0] = 0.0                                        # zero block: d = +0, q = 0
+    x[1, 5], x[1, 20] = 7.0, -7.0                     # tie: first (+7) wins -> d negative
+    x[2, 5], x[2, 20] = -7.0, 7.0                     # tie the other way round -> d positive
+    x[1, :5] *= 0.1; x[1, 6:20] *= 0.1; x[1, 21:] *= 0.1
+    x[2, :5] *= 0.1; x[2, 6:20] *= 0.1; x[2, 21:] *= 0.1
+    blk = oracle.quantize_q8_1(x.reshape(-1)).reshape(40, 36)
+    d = np.ascontiguousarray(blk[:, 0:2]).view(np.float16)[:, 0].astype(np.float32)
+    s = np.ascontiguousarray(blk[:, 2:4]).view(np.float16)[:, 0]
+    q = np.ascontiguousarray(blk[:, 4:]).view(np.int8).astype(np.int32)
+    assert (blk[0] == 0).all()
+    assert d[1] < 0 and q[1, 5] == -128 and q[1, 20] == 127
+    assert d[2] > 0 and q[2, 5] == -128 and q[2, 20] == 127
+    for r in range(3, 40):
+        i = np.abs(x[r]).argmax()
+        assert q[r, i] == -128                         # the extreme element takes the spare code
+        d32 = np.float32(x[r, i]) / np.float32(-128.0)
+        assert d[r] == np.float32(np.float16(d32))
+        # independent float64 statement of the rounding, away from exact ties
+        t = x[r].astype(np.float64) / np.float64(d32)
+        want = np.clip(np.sign(t) * np.floor(np.abs(t) + 0.5), -128, 127)
+        ok = np.abs(np.abs(t) % 1.0 - 0.5) > 1e-4
+        assert (q[r][ok] == want[ok]).all()
+        assert s[r] == np.float16(d32 * np.float32(q[r].sum()))
+        assert np.abs(x[r] - d32 * q[r]).max() <= abs(d32) * (0.5 + 2 ** -10) + (abs(d32) if q[r].max() == 127 else 0)
+
+
+def test_q8_1_activation_matmul_uses_the_same_settlement(oracle):
+    rng = np.random.default_rng(4)
+    M, N, K = 7, 5, 96
+    w = (rng.standard_normal((M, K)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((N, K)).astype(np.float32)
+    wq = oracle.quantize_q8_0(w)
+    x1 = oracle.quantize_q8_1(x)                                        # [N, nblk, 36]
+    as_q8_0 = np.concatenate([x1[..., 0:2], x1[..., 4:]], axis=-1)      # {d, qs}
+    want = oracle.mul_mat_q8q8(wq, np.ascontiguousarray(as_q8_0))
+    got = oracle.mul_mat_q8_act(wq, x, act=1)
+    assert (got.view(np.uint32) == want.view(np.uint32)).all()
+    assert (oracle.mul_mat_q8_act(wq, x, act=0) == oracle.mul_mat_q8(wq, x)).all()
+    assert (oracle.mul_mat_q8_act(oracle.repack_q8_0(wq), x, act=1, wtype=2) == got).all()
+    assert (oracle.mul_mat_q8_act(wq, x, act=1, c_trans=0) == got.T).all()
+    full = x.astype(np.float64) @ w.astype(np.float64).T
+    assert np.abs(got - full).max() <= 0.02 * np.abs(full).max()
+
+
 # ----------------------------------------------------------------------------- Q8 dot
 def _q8_case(rng, M, N, K):
     w = (rng.standard_normal((M, K)) * 0.02).astype(np.float32)
