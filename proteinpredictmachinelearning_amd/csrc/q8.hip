@@ -973,7 +973,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), 
 void q8_linear_ws_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                          int M, int N, int ntiles, int relu, uint8_t* __restrict__ xq_dump,
                          int32_t* __restrict__ sums_dump) {
-    static_assert(ws_compiler_vgprs(NBLK) == 240, "staging size");
+    static_assert(ws_compiler_vgprs(NBLK, NW) == 240, "staging size");
     q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, relu, xq_dump, sums_dump);
 }
 template <int NW, int TPW, int NBLK, int WL, bool DUMP>
@@ -981,7 +981,16 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), 
 void q8_linear_ws32_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
-    static_assert(ws_compiler_vgprs(NBLK) == 224, "staging size");
+    static_assert(ws_compiler_vgprs(NBLK, NW) == 224, "staging size");
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, relu, xq_dump, sums_dump);
+}
+
+template <int NW, int TPW, int NBLK, int WL, bool DUMP>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(192)))
+void q8_linear_ws64_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
+                           int M, int N, int ntiles, int relu, uint8_t* __restrict__ xq_dump,
+                           int32_t* __restrict__ sums_dump) {
+    static_assert(ws_compiler_vgprs(NBLK, NW) == 192, "staging size");
     q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, relu, xq_dump, sums_dump);
 }
 
@@ -997,14 +1006,14 @@ int device_cu_count() {
     return cus;
 }
 
-template <int TPW, int NBLK, int WL>
+template <int TPW, int NBLK, int WL, int NW = 8>
 int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int relu,
                         void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
-    constexpr int NW = 8;
     const int ntiles = (N + TILE_TOK - 1) / TILE_TOK;
-    // one resident work-group per CU; with more tiles than CUs every work-group takes the same
-    // number of tiles (824 tiles on 256 CUs: 206 work-groups x 4 rather than 256 x 3 + 56 x 1)
-    const int cus = device_cu_count();
+    // Eight waves fill a CU (256 registers each): one resident work-group of 8 waves per CU, or two
+    // of 4.  With more tiles than resident work-groups every work-group takes the same number of
+    // tiles (824 tiles on 256 CUs: 206 work-groups x 4 rather than 256 x 3 + 56 x 1).
+    const int cus = device_cu_count() * (8 / NW);
     const int rounds = (ntiles + cus - 1) / cus;
     const int wgs = (ntiles + rounds - 1) / rounds;
     const dim3 grid(wgs), block(NW * 64);
@@ -1012,12 +1021,16 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
                            static_cast<size_t>(NW) * WL * NBLK * 1024;
     using KernelFn = void (*)(const uint8_t*, const float*, float*, int, int, int, int, uint8_t*, int32_t*);
     KernelFn fast, dump;
-    if constexpr (ws_staging_regs(NBLK) == 16) {
+    if constexpr (ws_staging_regs(NBLK, NW) == 16) {
         fast = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false>;
         dump = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true>;
-    } else {
+    } else if constexpr (ws_staging_regs(NBLK, NW) == 32) {
         fast = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, false>;
         dump = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, true>;
+    } else {
+        static_assert(ws_staging_regs(NBLK, NW) == 64, "no kernel for this staging size");
+        fast = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, false>;
+        dump = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, true>;
     }
     if (lds > 64 * 1024) {
         static const hipError_t attr_fast = hipFuncSetAttribute(
@@ -1045,6 +1058,13 @@ int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int 
     if (static_cast<int64_t>(N) * M * 4 >= 0x7fff0000LL) return -1;   // the kernel addresses C with 32-bit byte offsets
     const int mct = (M + 31) / 32;
     const int tpw = (mct + 7) / 8;
+    // Up to four column tiles: work-groups of four waves, one column tile each and two per CU, so no
+    // wave idles (with eight waves half of them would have no column tile).
+    if (mct <= 4) {
+        if (nblk == 4) return launch_q8_linear_ws<1, 4, 0, 4>(W, X, C, M, N, relu, xq_dump, sums_dump, stream);
+        if (nblk == 8) return launch_q8_linear_ws<1, 8, 0, 4>(W, X, C, M, N, relu, xq_dump, sums_dump, stream);
+        if (nblk == 16) return launch_q8_linear_ws<1, 16, 0, 4>(W, X, C, M, N, relu, xq_dump, sums_dump, stream);
+    }
 #define PPML_WS(TPW, NBLK, WL) if (tpw == TPW && nblk == NBLK) return launch_q8_linear_ws<TPW, NBLK, WL>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
     // (column tiles per wave, blocks of K, column tiles whose fragments live in LDS instead of registers)
     PPML_WS(1, 4, 0);  PPML_WS(2, 4, 0);  PPML_WS(3, 4, 0);  PPML_WS(4, 4, 0);
