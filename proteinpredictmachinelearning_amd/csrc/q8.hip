@@ -642,7 +642,7 @@ constexpr int ws_compiler_vgprs(int nblk, int nw = 8) { return 256 - ws_staging_
 template <int NW, int TPW, int NBLK, int WL, bool DUMP>
 __device__ __forceinline__ void q8_linear_ws_body(
     const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
-    int M, int N, int ntiles, int relu,
+    int M, int N, int ntiles, int npart, int relu,
     uint8_t* __restrict__ xq_dump, int32_t* __restrict__ sums_dump) {
     static_assert(NBLK % 2 == 0, "the quantizer stages blocks in pairs");
     constexpr int K = NBLK * QK;
@@ -737,9 +737,20 @@ __device__ __forceinline__ void q8_linear_ws_body(
     // and it keeps these loads older than at least a tile's worth of later memory operations on
     // every path into the loop, which is what lets the wait in front of the quantizer skip them.
     v4f xv[UPW][2];
-    int tile = blockIdx.x;
+    // This work-group's tiles: blockIdx, blockIdx + grid, ... below `ntiles` in full, then -- when the
+    // tiles left over by whole rounds are few enough -- one more tile of which it computes a single
+    // column tile per wave (tile ntiles + blockIdx / TPW, column part blockIdx % TPW), so that TPW
+    // work-groups share each leftover tile instead of a few work-groups running a whole extra round.
+    const int grid = static_cast<int>(gridDim.x);
+    const int wg = static_cast<int>(blockIdx.x);
+    const int n_full = wg < ntiles ? (ntiles - wg + grid - 1) / grid : 0;
+    const bool has_part = wg < npart;
+    const int n_iter = n_full + (has_part ? 1 : 0);
+    const int part_col = wg % TPW;
+    auto tile_of = [&](int i) { return i < n_full ? wg + i * grid : ntiles + wg / TPW; };
+    int tile = tile_of(0);
     PPML_TRACE_MARK(0);
-    if (tile < ntiles) load_tile(tile, xv);
+    if (n_iter > 0) load_tile(tile, xv);
 
     // ---- resident weights: fragments of TPW column tiles in registers, their scales in LDS
     static_assert(WL >= 0 && WL < TPW, "at least one column tile stays in registers");
@@ -750,7 +761,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
         const uint16_t* dplane = reinterpret_cast<const uint16_t*>(W + static_cast<size_t>(mct_pad) * NBLK * 1024);
 #pragma unroll
         for (int t = 0; t < TPW; ++t) {
-            int ct = wave * TPW + t;
+            int ct = t * NW + wave;                    // round t of the waves covers NW adjacent column tiles
             ct = ct < mct_pad ? ct : mct_pad - 1;      // tiles past the end repeat the last one; never stored
 #pragma unroll
             for (int b = 0; b < NBLK; ++b) {
@@ -776,7 +787,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
             const int row = (u & 3) * 8 + urow;
             const int bl = (u >> 2) * 2 + ublk;
             v4f x0 = xv[s][0], x1 = xv[s][1];
-            if (relu) {
+            if (relu & 1) {
 #pragma unroll
                 for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
             }
@@ -804,7 +815,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
         asm volatile("" ::: "memory");
     };
 
-    if (tile < ntiles) {
+    if (n_iter > 0) {
         quantize_tile(0, tile * TILE_TOK, xv);
         announce(0);
     }
@@ -813,7 +824,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
     // its first use inside the loop wait for vmcnt(0), i.e. for all output stores, on every iteration.
     __builtin_amdgcn_s_waitcnt(0x0f70);                // vmcnt(0), other counters untouched
     // the second tile is requested now and quantized two thirds into the first one
-    if (tile + static_cast<int>(gridDim.x) < ntiles) load_tile_async(tile + static_cast<int>(gridDim.x));
+    if (n_iter > 1) load_tile_async(tile_of(1));
     PPML_TRACE_MARK(1);
 
     // Step at which the next tile is quantized.  Its loads were issued one full round of column tiles
@@ -834,11 +845,13 @@ __device__ __forceinline__ void q8_linear_ws_body(
         for (int i = 0; i < g_q8_dbg[0]; ++i) __builtin_amdgcn_s_sleep(8);   // 512 cycles each
     }
 #endif
-    for (int it = 0; tile < ntiles; tile += gridDim.x, ++it) {
+    for (int it = 0; it < n_iter; ++it) {
+        tile = tile_of(it);
         const int buf = it % WS_NBUF;
         const int tok0 = tile * TILE_TOK;
-        const int next = tile + static_cast<int>(gridDim.x);
-        const bool has_next = next < ntiles;
+        const bool has_next = it + 1 < n_iter;
+        const int next = has_next ? tile_of(it + 1) : tile;
+        const bool partial = it >= n_full;             // compute column tile part_col only
         await_tile(buf, static_cast<unsigned>(NW) * static_cast<unsigned>(it / WS_NBUF + 1));
         PPML_TRACE_MARK(2 + 10 * it);
 
@@ -883,7 +896,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(static_cast<float>(sum[r]), scl[r], acc[r]);
             }
-            const int m = (wave * TPW + t) * 32 + j;   // this lane's output feature
+            const int m = (t * NW + wave) * 32 + j;    // this lane's output feature
             if (DUMP && sums_dump) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
@@ -920,14 +933,14 @@ __device__ __forceinline__ void q8_linear_ws_body(
             // One basic block per column tile (see opaque_one()): the accumulator is born and stored
             // inside it, so nothing but loop state crosses the boundary.
             if (!opaque_one()) continue;
+            if (partial && t0 != part_col) continue;
             if (t0 * NBLK == QSTEP_TILE * NBLK && has_next) {
                 PPML_TRACE_MARK(2 + 10 * it + 7);
                 {
                     v4f xn[UPW][2];
                     if (it == 0) take_tile(std::integral_constant<int, NEWER_FIRST>{}, xn);
                     else take_tile(std::integral_constant<int, NEWER>{}, xn);
-                    const int next2 = next + static_cast<int>(gridDim.x);
-                    if (next2 < ntiles) load_tile_async(next2);
+                    if (it + 2 < n_iter) load_tile_async(tile_of(it + 2));
                     quantize_tile((it + 1) % WS_NBUF, next * TILE_TOK, xn);
                     announce((it + 1) % WS_NBUF);
                 }
@@ -971,27 +984,27 @@ __device__ __forceinline__ void q8_linear_ws_body(
 template <int NW, int TPW, int NBLK, int WL, bool DUMP>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(240)))
 void q8_linear_ws_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
-                         int M, int N, int ntiles, int relu, uint8_t* __restrict__ xq_dump,
+                         int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                          int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 240, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 template <int NW, int TPW, int NBLK, int WL, bool DUMP>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(224)))
 void q8_linear_ws32_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
-                           int M, int N, int ntiles, int relu, uint8_t* __restrict__ xq_dump,
+                           int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 224, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
 template <int NW, int TPW, int NBLK, int WL, bool DUMP>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(192)))
 void q8_linear_ws64_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
-                           int M, int N, int ntiles, int relu, uint8_t* __restrict__ xq_dump,
+                           int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 192, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
 int device_cu_count() {
@@ -1009,17 +1022,26 @@ int device_cu_count() {
 template <int TPW, int NBLK, int WL, int NW = 8>
 int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int relu,
                         void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
-    const int ntiles = (N + TILE_TOK - 1) / TILE_TOK;
     // Eight waves fill a CU (256 registers each): one resident work-group of 8 waves per CU, or two
     // of 4.  With more tiles than resident work-groups every work-group takes the same number of
     // tiles (824 tiles on 256 CUs: 206 work-groups x 4 rather than 256 x 3 + 56 x 1).
     const int cus = device_cu_count() * (8 / NW);
-    const int rounds = (ntiles + cus - 1) / cus;
-    const int wgs = (ntiles + rounds - 1) / rounds;
+    const int all_tiles = (N + TILE_TOK - 1) / TILE_TOK;
+    int wgs, ntiles = all_tiles, npart = 0;
+    const int left = all_tiles % cus;
+    if (all_tiles > cus && left > 0 && left * TPW <= cus && TPW > 1) {
+        // whole rounds on every CU, then the leftover tiles shared by TPW work-groups each
+        wgs = cus;
+        ntiles = all_tiles - left;
+        npart = left * TPW;
+    } else {
+        const int rounds = (all_tiles + cus - 1) / cus;
+        wgs = (all_tiles + rounds - 1) / rounds;
+    }
     const dim3 grid(wgs), block(NW * 64);
     constexpr size_t lds = static_cast<size_t>(WS_NBUF) * NBLK * (1024 + 128) + static_cast<size_t>(NW) * TPW * NBLK * 128 + 16 +
                            static_cast<size_t>(NW) * WL * NBLK * 1024;
-    using KernelFn = void (*)(const uint8_t*, const float*, float*, int, int, int, int, uint8_t*, int32_t*);
+    using KernelFn = void (*)(const uint8_t*, const float*, float*, int, int, int, int, int, uint8_t*, int32_t*);
     KernelFn fast, dump;
     if constexpr (ws_staging_regs(NBLK, NW) == 16) {
         fast = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false>;
@@ -1043,10 +1065,10 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
         }
     }
     if (xq_dump || sums_dump)
-        hipLaunchKernelGGL(dump, grid, block, lds, stream, static_cast<const uint8_t*>(W), X, C, M, N, ntiles, relu,
+        hipLaunchKernelGGL(dump, grid, block, lds, stream, static_cast<const uint8_t*>(W), X, C, M, N, ntiles, npart, relu,
                            static_cast<uint8_t*>(xq_dump), sums_dump);
     else
-        hipLaunchKernelGGL(fast, grid, block, lds, stream, static_cast<const uint8_t*>(W), X, C, M, N, ntiles, relu,
+        hipLaunchKernelGGL(fast, grid, block, lds, stream, static_cast<const uint8_t*>(W), X, C, M, N, ntiles, npart, relu,
                            static_cast<uint8_t*>(nullptr), static_cast<int32_t*>(nullptr));
     return check_launch("q8_linear_ws_kernel");
 }
