@@ -55,6 +55,13 @@ const char *ppml_hip_last_error(void);
 int mul_mat_hip(const float *A, const float *B, float *C, int M, int K, int N,
                 const float *bias, ppml_hip_stream_t stream);
 
+/* replaces mul_mat_cuda_f16 / mul_mat_mma_f16(_smem) (src/cuda/CUDAKernels.cu:1186-1492, declared
+ * src/backend/CUDAKernels.cpp:182-200): A and B hold IEEE halves, [M][K] and [N][K]; every product and the sum
+ * are binary32 (a product of two halves is exact in binary32), C is f32.  bias may be NULL; it is added to
+ * the finished sum, as the CPU kernel does on this branch (src/backend/CPUKernels.cpp:646-672). */
+int mul_mat_f16_hip(const void *A16, const void *B16, float *C, int M, int K, int N,
+                    const float *bias, ppml_hip_stream_t stream);
+
 /* ---- Q8_0 ---------------------------------------------------------------------------------- */
 /* Q8_0 twin of quantize_rows_q8_1_cuda (src/cuda/QuantKernels.cu:86-93); the arithmetic is
  * quantize_q8_0_host (include/ppml/QuantBlocks.h:62-79).  y receives ne/32 block_q8_0 records. */

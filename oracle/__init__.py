@@ -63,6 +63,8 @@ def _load() -> C.CDLL:
     lib.orc_mul_mat_q8_act.argtypes = [vp, f32p, f32p] + [C.c_int] * 8
     lib.orc_mul_mat_f32.restype = None
     lib.orc_mul_mat_f32.argtypes = [f32p, f32p, f32p, C.c_int, C.c_int, C.c_int, f32p, C.c_int]
+    lib.orc_mul_mat_f16.restype = None
+    lib.orc_mul_mat_f16.argtypes = [C.POINTER(C.c_uint16), C.POINTER(C.c_uint16), f32p, C.c_int, C.c_int, C.c_int, f32p, C.c_int]
     lib.orc_out_prod.restype = None
     lib.orc_out_prod.argtypes = [f32p, f32p, f32p] + [i64] * 12 + [C.c_int]
     lib.orc_outer_prod_mean.restype = None
@@ -240,6 +242,21 @@ def mul_mat_f32(a, b, bias=None, nthreads=0) -> np.ndarray:
         bias = _f32(bias)
         bp = _fp(bias)
     lib().orc_mul_mat_f32(_fp(a), _fp(b), _fp(out), M, K, N, bp, nthreads)
+    return out
+
+
+def mul_mat_f16(a16, b16, bias=None, nthreads=0) -> np.ndarray:
+    """a16 [M,K], b16 [N,K] float16 -> f32 [M,N] (CPUKernels.cpp:646-672: binary32 sum, bias last)."""
+    a16 = np.ascontiguousarray(a16, dtype=np.float16)
+    b16 = np.ascontiguousarray(b16, dtype=np.float16)
+    M, K = a16.shape
+    N = b16.shape[0]
+    assert b16.shape[1] == K
+    out = np.empty((M, N), dtype=np.float32)
+    bp = None if bias is None else _fp(_f32(bias))
+    u16p = C.POINTER(C.c_uint16)
+    lib().orc_mul_mat_f16(a16.view(np.uint16).ctypes.data_as(u16p), b16.view(np.uint16).ctypes.data_as(u16p),
+                          _fp(out), M, K, N, bp, nthreads)
     return out
 
 

@@ -339,6 +339,25 @@ void orc_mul_mat_f32(const float *a, const float *b, float *d, int M, int K, int
     }
 }
 
+/* src/backend/CPUKernels.cpp:392-396 (dot_half_row_soft) and 646-672: A and B hold halves, each
+ * product is formed in binary32 (exact: two 11-bit significands), summed k ascending, and the bias
+ * is added to the finished dot product.  (The reference's F16C variant keeps 8 partial sums; this
+ * restates the portable one.) */
+void orc_mul_mat_f16(const uint16_t *a, const uint16_t *b, float *d, int M, int K, int N,
+                     const float *bias, int nthreads) {
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(nt)
+    for (int i = 0; i < M; ++i) {
+        for (int j = 0; j < N; ++j) {
+            float acc = 0.0f;
+            for (int k = 0; k < K; ++k)
+                acc += orc_fp16_to_fp32(a[(int64_t)i * K + k]) * orc_fp16_to_fp32(b[(int64_t)j * K + k]);
+            d[j + (int64_t)i * N] = bias ? (acc + bias[j]) : acc;
+        }
+    }
+}
+
 /* src/backend/CPUKernels.cpp:787-887: dst zeroed, then for each dst row (i1,i2,i3)
  * d_row[i0] += s0[i0,k,i02,i03] * s1[i1,k,i2,i3], k ascending (the reference's K-blocking of
  * 32 and row-blocking of 16 leave the per-element order unchanged); src0 planes broadcast

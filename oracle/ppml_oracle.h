@@ -65,6 +65,10 @@ int  orc_mul_mat_q8_act(const void *W, const float *X, float *C, int M, int N, i
 /* src/backend/CPUKernels.cpp:763-771 ; bias may be NULL */
 void orc_mul_mat_f32(const float *a, const float *b, float *d, int M, int K, int N,
                      const float *bias, int nthreads);
+/* src/backend/CPUKernels.cpp:392-396, 646-672: halves in, binary32 products and sum, bias last */
+void orc_mul_mat_f16(const uint16_t *a, const uint16_t *b, float *d, int M, int K, int N,
+                     const float *bias, int nthreads);
+
 /* src/backend/CPUKernels.cpp:787-887 */
 void orc_out_prod(const float *s0, const float *s1, float *dst,
                   int64_t ne00, int64_t ne01, int64_t ne02, int64_t ne03,

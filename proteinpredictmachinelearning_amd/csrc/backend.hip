@@ -143,9 +143,9 @@ bool node_supported(const Tensor* node) {
                 return w->quant_shape_valid() && is_quantized_type_supported(w->type) &&
                        a->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32;
             }
-            // F16 x F16 is served by the reference's own kernels, not by this backend
-            return src0 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
-                   node->type == TENSOR_TYPE_F32;
+            const bool ok_f32 = src0 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32;
+            const bool ok_f16 = src0 && src0->type == TENSOR_TYPE_F16 && src1->type == TENSOR_TYPE_F16;
+            return (ok_f32 || ok_f16) && node->type == TENSOR_TYPE_F32;
         }
         case OP_OUT_PROD:
             return src0 && src1 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
@@ -232,9 +232,15 @@ Status HipBackend::kernel_mul_mat(Tensor* node) {
         rc = mul_mat_q8_ex_hip(w->data, static_cast<const float*>(a->data), static_cast<float*>(node->data),
                                static_cast<int>(Mq), static_cast<int>(Nq), static_cast<int>(K), wtype, c_trans,
                                q8_1_activations_ ? 2 : 0, nullptr, nullptr, nullptr);
+    } else if (s0->type == TENSOR_TYPE_F16 && s1->type == TENSOR_TYPE_F16) {
+        // src/backend/CUDAKernels.cpp:794-821: F16 x F16 -> F32, no bias epilogue on this path
+        if (bias) return fail(Status::NOT_SUPPORTED, "mul_mat: the F16 path has no bias epilogue");
+        if (node->type != TENSOR_TYPE_F32) return fail(Status::NOT_SUPPORTED, "mul_mat: F16 x F16 gives F32");
+        rc = mul_mat_f16_hip(s0->data, s1->data, static_cast<float*>(node->data), static_cast<int>(M),
+                             static_cast<int>(K), static_cast<int>(N), nullptr, nullptr);
     } else {
         if (s0->type != TENSOR_TYPE_F32 || s1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32)
-            return fail(Status::NOT_SUPPORTED, "mul_mat: only F32 x F32 -> F32 besides the quantized path");
+            return fail(Status::NOT_SUPPORTED, "mul_mat: F32 x F32 or F16 x F16 -> F32 besides the quantized path");
         rc = mul_mat_hip(static_cast<const float*>(s0->data), static_cast<const float*>(s1->data),
                          static_cast<float*>(node->data), static_cast<int>(M), static_cast<int>(K),
                          static_cast<int>(N), bias, nullptr);

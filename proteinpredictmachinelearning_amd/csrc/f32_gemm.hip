@@ -18,7 +18,7 @@ namespace {
 constexpr int BM = 128, BN = 128, BK = 16;
 constexpr int LDS_LD = BM + 4;        // row pitch of the k-major LDS tiles (floats)
 
-enum LoadMode { LOAD_K_CONTIG = 0, LOAD_ROW_CONTIG = 1, LOAD_STRIDED = 2 };
+enum LoadMode { LOAD_K_CONTIG = 0, LOAD_ROW_CONTIG = 1, LOAD_STRIDED = 2, LOAD_K_CONTIG_F16 = 3 };
 
 struct GemmParams {
     const float* A;       // rows m: A(m,k) = A[m*a_rs + k*a_ks]
@@ -37,6 +37,8 @@ struct GemmParams {
     int64_t c_mo, c_mi, c_no, c_ni;
     int tiles_m, tiles_n;
     int stream_c;         // output larger than the last-level cache: write it with streaming stores
+    int f16_in;           // A and B hold IEEE halves (k contiguous); products and sums are binary32
+    int bias_last;        // add the bias to the finished sum instead of starting from it
 };
 
 // 16 x 128 tile of one operand -> two v4f per thread
@@ -56,6 +58,22 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_
                 else {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) if (k + c < K) v[c] = p[c];
+                }
+            }
+        } else if (MODE == LOAD_K_CONTIG_F16) {
+            // the same tile shape read from halves: 4 of them (8 bytes) per thread and pass
+            const int r = (tid >> 2) + it * 64;
+            const int k = k0 + (tid & 3) * 4;
+            const int row = row0 + r;
+            if (row < nrows) {
+                const __half* p = reinterpret_cast<const __half*>(base) + static_cast<int64_t>(row) * rs + k;
+                if (k + 3 < K && (reinterpret_cast<uintptr_t>(p) & 7) == 0) {
+                    const uint2 raw = *reinterpret_cast<const uint2*>(p);
+                    const __half2 lo = *reinterpret_cast<const __half2*>(&raw.x), hi = *reinterpret_cast<const __half2*>(&raw.y);
+                    v[0] = __low2float(lo); v[1] = __high2float(lo); v[2] = __low2float(hi); v[3] = __high2float(hi);
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) if (k + c < K) v[c] = __half2float(p[c]);
                 }
             }
         } else if (MODE == LOAD_ROW_CONTIG) {
@@ -134,7 +152,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj) {
         const int n = n0 + wn + tj * 32 + j;
-        const float b0 = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+        const float b0 = (p.bias && !p.bias_last && n < p.N) ? p.bias[n] : 0.0f;
 #pragma unroll
         for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
@@ -174,6 +192,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
         for (int tj = 0; tj < 2; ++tj) {
             const int n = n0 + wn + tj * 32 + j;
             if (n >= p.N) continue;
+            const float tail_bias = (p.bias && p.bias_last) ? p.bias[n] : 0.0f;
             int64_t coff;
             if (SPLIT_C) coff = static_cast<int64_t>(n / p.c_ln) * p.c_no + static_cast<int64_t>(n % p.c_ln) * p.c_ni;
             else         coff = static_cast<int64_t>(n) * p.c_ni;
@@ -186,6 +205,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
                 else         roff = static_cast<int64_t>(m) * p.c_mi;
                 float v = acc[ti][tj][r];
                 if (scale) v *= p.alpha;
+                if (p.bias_last) v += tail_bias;
                 if (STREAM_C) __builtin_nontemporal_store(v, &C[roff + coff]);
                 else C[roff + coff] = v;
             }
@@ -211,7 +231,8 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
         if (p.stream_c) hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, true>), grid, block, 0, stream, p);  \
         else hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, false>), grid, block, 0, stream, p);    \
     } while (0)
-    if (mode == LOAD_K_CONTIG)        { if (split) PPML_LAUNCH(LOAD_K_CONTIG, true);   else PPML_LAUNCH(LOAD_K_CONTIG, false); }
+    if (p.f16_in)                     { PPML_LAUNCH(LOAD_K_CONTIG_F16, false); }
+    else if (mode == LOAD_K_CONTIG)   { if (split) PPML_LAUNCH(LOAD_K_CONTIG, true);   else PPML_LAUNCH(LOAD_K_CONTIG, false); }
     else if (mode == LOAD_ROW_CONTIG) { if (split) PPML_LAUNCH(LOAD_ROW_CONTIG, true); else PPML_LAUNCH(LOAD_ROW_CONTIG, false); }
     else                              { if (split) PPML_LAUNCH(LOAD_STRIDED, true);    else PPML_LAUNCH(LOAD_STRIDED, false); }
 #undef PPML_LAUNCH
@@ -242,6 +263,20 @@ extern "C" int mul_mat_hip(const float* A, const float* B, float* C, int M, int 
     p.a_rs = K; p.a_ks = 1; p.b_rs = K; p.b_ks = 1;
     p.c_mi = N; p.c_ni = 1;
     return launch_gemm(p, static_cast<hipStream_t>(stream), "mul_mat_hip");
+}
+
+extern "C" int mul_mat_f16_hip(const void* A16, const void* B16, float* C, int M, int K, int N,
+                               const float* bias, ppml_hip_stream_t stream) {
+    if (!A16 || !B16 || !C || M <= 0 || K <= 0 || N <= 0) { set_error("mul_mat_f16_hip: bad arguments (M=%d K=%d N=%d)", M, K, N); return RC_BAD_ARGS; }
+    stats_record(M, K, N);
+    GemmParams p = plain_params();
+    p.A = static_cast<const float*>(A16); p.B = static_cast<const float*>(B16); p.C = C; p.bias = bias;
+    p.M = M; p.N = N; p.K = K;
+    p.a_rs = K; p.a_ks = 1; p.b_rs = K; p.b_ks = 1;      // strides in elements (halves)
+    p.c_mi = N; p.c_ni = 1;
+    p.f16_in = 1;
+    p.bias_last = 1;
+    return launch_gemm(p, static_cast<hipStream_t>(stream), "mul_mat_f16_hip");
 }
 
 extern "C" int mul_mat_tn_hip(const float* A, const float* Bm, float* O, int M, int K, int Nc, float alpha,

@@ -69,6 +69,26 @@ def mul_mat(a: torch.Tensor, b: torch.Tensor, bias: torch.Tensor | None = None) 
     return out
 
 
+def mul_mat_f16(a: torch.Tensor, b: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """F16 x F16 -> F32 mul_mat: a [M,K], b [N,K] float16 on the device, binary32 products and sum,
+    bias (f32 [N]) added to the finished sum (src/backend/CPUKernels.cpp:646-672)."""
+    for t, name in ((a, "a"), (b, "b")):
+        if not t.is_cuda or t.dtype != torch.float16:
+            raise TypeError(f"mul_mat_f16: {name} must be a float16 tensor on the device")
+    a, b = a.contiguous(), b.contiguous()
+    if a.dim() != 2 or b.dim() != 2 or a.shape[1] != b.shape[1]:
+        raise ValueError(f"mul_mat_f16: a {tuple(a.shape)} and b {tuple(b.shape)} do not share K")
+    M, K = a.shape
+    N = b.shape[0]
+    if bias is not None:
+        bias = _dev_f32(bias, "bias")
+        if bias.numel() != N:
+            raise ValueError("mul_mat_f16: bias length is not N")
+    out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+    cabi.check("mul_mat_f16_hip", _lib().mul_mat_f16_hip(_ptr(a), _ptr(b), _ptr(out), M, K, N, _ptr(bias), _stream()))
+    return out
+
+
 def mul_mat_tn(a: torch.Tensor, b: torch.Tensor, alpha: float = 1.0) -> torch.Tensor:
     """a [K,M], b [K,N] -> alpha * a.T @ b (the dense form of outer-product-mean)."""
     a, b = _dev_f32(a, "a"), _dev_f32(b, "b")

@@ -29,7 +29,9 @@ def _mm(t0, t1, out=B.F32, bias=None, k0=64, k1=64):
     (B.F32, B.Q8_0, B.F32, B.F32, False),
     (B.Q8_0, B.F16, B.F32, None, False),         # activations must be f32
     (B.F32, B.Q8_0, B.F16, None, False),
-    (B.F16, B.F16, B.F32, None, False),          # left to the reference's own kernels
+    (B.F16, B.F16, B.F32, None, True),           # halves in, f32 out
+    (B.F16, B.F16, B.F32, B.F32, False),         # no bias epilogue on the F16 path
+    (B.F16, B.F16, B.F16, None, False),
     (B.F32, B.F16, B.F32, None, False),
 ])
 def test_supports_op_mul_mat(t0, t1, out, bias, want):

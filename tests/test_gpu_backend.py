@@ -69,6 +69,21 @@ def test_quantized_mul_mat_node(be, oracle, wname, wside):
     np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-6 * np.abs(want).max())
 
 
+def test_f16_mul_mat_node(be, oracle):
+    M, K, N = 19, 24, 11
+    rng = np.random.default_rng(10)
+    a = rng.integers(-6, 7, size=(M, K)).astype(np.float16)
+    b = rng.integers(-6, 7, size=(N, K)).astype(np.float16)
+    at = _leaf(be, a.view(np.uint8).reshape(-1), B.F16, (K, M))
+    bt = _leaf(be, b.view(np.uint8).reshape(-1), B.F16, (K, N))
+    node = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [at, bt])
+    got = be_run(be, node).reshape(M, N)
+    assert (got == oracle.mul_mat_f16(a, b)).all()
+    withbias = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [at, bt, _leaf(be, np.zeros(N, np.float32))])
+    assert not be.supports_op(withbias)
+    assert be.graph_compute([withbias]) == B.NOT_SUPPORTED
+
+
 def test_quantized_mul_mat_node_with_cuda_activation_rule(be, oracle):
     rows, K, F = 50, 64, 40
     rng = np.random.default_rng(6)

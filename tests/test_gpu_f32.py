@@ -77,6 +77,36 @@ def test_mul_mat_bias_enters_the_accumulator_first(ops):
         ops.mul_mat(a, b, torch.zeros(2, device="cuda"))
 
 
+# ----------------------------------------------------------------------------- F16 mul_mat
+@pytest.mark.parametrize("M,K,N,bias", [(408, 256, 256, False), (17, 9, 23, True), (129, 37, 127, True),
+                                        (300, 70, 260, False), (2000, 128, 512, True), (1, 1, 1, False)])
+def test_mul_mat_f16(ops, oracle, M, K, N, bias):
+    # halves in, binary32 products and sum, bias last (src/backend/CPUKernels.cpp:646-672)
+    rng = np.random.default_rng(M * 3 + K + N)
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    b = (rng.standard_normal((N, K)) * 0.02).astype(np.float16)
+    bv = rng.standard_normal(N).astype(np.float32) if bias else None
+    got = ops.mul_mat_f16(_dev(a), _dev(b), None if bv is None else _dev(bv)).cpu().numpy()
+    want = oracle.mul_mat_f16(a, b, bv)
+    absprod = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64).T + (np.abs(bv)[None, :] if bias else 0)
+    _check(got, want, absprod)
+
+
+def test_mul_mat_f16_exact_on_small_integers(ops, oracle):
+    rng = np.random.default_rng(7)
+    a = rng.integers(-8, 9, size=(65, 40)).astype(np.float16)
+    b = rng.integers(-8, 9, size=(33, 40)).astype(np.float16)
+    bias = rng.integers(-4, 5, size=33).astype(np.float32)
+    got = ops.mul_mat_f16(_dev(a), _dev(b), _dev(bias)).cpu().numpy()
+    assert (got == oracle.mul_mat_f16(a, b, bias)).all()
+    ones = np.ones((1, 2), np.float16)                 # bias last: 2 + 2^24, not (2^24 + 1) + 1
+    assert ops.mul_mat_f16(_dev(ones), _dev(ones), _dev(np.array([2.0 ** 24], np.float32))).item() == 2.0 ** 24 + 2
+    with pytest.raises(TypeError):
+        ops.mul_mat_f16(_dev(a.astype(np.float32)), _dev(b))
+    with pytest.raises(ValueError):
+        ops.mul_mat_f16(_dev(a), _dev(b[:, :39]))
+
+
 # ----------------------------------------------------------------------------- out_prod
 def test_out_prod_reference_small_inputs_exact(ops, oracle):
     # tests/test_cuda.cpp:207-245

@@ -374,6 +374,25 @@ def test_mul_mat_random_vs_float64(oracle):
     assert np.abs(oracle.mul_mat_f32(A, B) - want).max() < 1e-4
 
 
+def test_mul_mat_f16_binary32_sum_and_bias_last(oracle):
+    # src/backend/CPUKernels.cpp:392-396, 646-672
+    rng = np.random.default_rng(2)
+    a = rng.standard_normal((7, 37)).astype(np.float16)
+    b = (rng.standard_normal((5, 37)) * 0.02).astype(np.float16)
+    bias = rng.standard_normal(5).astype(np.float32)
+    got = oracle.mul_mat_f16(a, b, bias)
+    want = a.astype(np.float64) @ b.astype(np.float64).T + bias
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    # equals the f32 kernel on the widened operands when there is no bias (same products, same order)
+    assert (oracle.mul_mat_f16(a, b) == oracle.mul_mat_f32(a.astype(np.float32), b.astype(np.float32))).all()
+    # the bias is added LAST here and FIRST on the f32 branch: with bias 2^24 and two products of 1,
+    # last gives 2 + 2^24 (a binary32 number), first gives (2^24 + 1) + 1 = 2^24 (each +1 is lost)
+    ones = np.ones((1, 2), np.float16)
+    big = np.array([2.0 ** 24], np.float32)
+    assert oracle.mul_mat_f16(ones, ones, big)[0, 0] == np.float32(2.0 ** 24 + 2)
+    assert oracle.mul_mat_f32(ones.astype(np.float32), ones.astype(np.float32), big)[0, 0] == np.float32(2.0 ** 24)
+
+
 # ----------------------------------------------------------------------------- out_prod
 def test_out_prod_reference_small_inputs_exact(oracle):
     # tests/test_cuda.cpp:207-245
