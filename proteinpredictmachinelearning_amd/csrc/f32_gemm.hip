@@ -38,7 +38,6 @@ struct GemmParams {
     int tiles_m, tiles_n;
     int stream_c;         // output larger than the last-level cache: write it with streaming stores
     int f16_in;           // A and B hold IEEE halves (k contiguous); products and sums are binary32
-    int bias_last;        // add the bias to the finished sum instead of starting from it
 };
 
 // 16 x 128 tile of one operand -> two v4f per thread
@@ -148,11 +147,13 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
     const float* B = p.B + (p2 / p.b_div2) * p.b_p2 + (p3 / p.b_div3) * p.b_p3;
     float* C = p.C + p2 * p.c_p2 + p3 * p.c_p3;
 
+    // halves in: the bias joins the finished sum (the CPU branch of the reference adds it last)
+    constexpr bool BIAS_LAST = MODE == LOAD_K_CONTIG_F16;
     v16f acc[2][2];
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj) {
         const int n = n0 + wn + tj * 32 + j;
-        const float b0 = (p.bias && !p.bias_last && n < p.N) ? p.bias[n] : 0.0f;
+        const float b0 = (p.bias && !BIAS_LAST && n < p.N) ? p.bias[n] : 0.0f;
 #pragma unroll
         for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
@@ -192,7 +193,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
         for (int tj = 0; tj < 2; ++tj) {
             const int n = n0 + wn + tj * 32 + j;
             if (n >= p.N) continue;
-            const float tail_bias = (p.bias && p.bias_last) ? p.bias[n] : 0.0f;
+            const float tail_bias = (BIAS_LAST && p.bias) ? p.bias[n] : 0.0f;
             int64_t coff;
             if (SPLIT_C) coff = static_cast<int64_t>(n / p.c_ln) * p.c_no + static_cast<int64_t>(n % p.c_ln) * p.c_ni;
             else         coff = static_cast<int64_t>(n) * p.c_ni;
@@ -205,7 +206,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
                 else         roff = static_cast<int64_t>(m) * p.c_mi;
                 float v = acc[ti][tj][r];
                 if (scale) v *= p.alpha;
-                if (p.bias_last) v += tail_bias;
+                if (BIAS_LAST) v += tail_bias;
                 if (STREAM_C) __builtin_nontemporal_store(v, &C[roff + coff]);
                 else C[roff + coff] = v;
             }
@@ -275,7 +276,6 @@ extern "C" int mul_mat_f16_hip(const void* A16, const void* B16, float* C, int M
     p.a_rs = K; p.a_ks = 1; p.b_rs = K; p.b_ks = 1;      // strides in elements (halves)
     p.c_mi = N; p.c_ni = 1;
     p.f16_in = 1;
-    p.bias_last = 1;
     return launch_gemm(p, static_cast<hipStream_t>(stream), "mul_mat_f16_hip");
 }
 

@@ -750,33 +750,44 @@ __device__ __forceinline__ void q8_linear_ws_body(
     auto tile_of = [&](int i) { return i < n_full ? wg + i * grid : ntiles + wg / TPW; };
     int tile = tile_of(0);
     PPML_TRACE_MARK(0);
+    if (tid < WS_NBUF) lds_ready[tid] = 0u;
+    __syncthreads();                                   // the only barrier of the kernel
     if (n_iter > 0) load_tile(tile, xv);
 
-    // ---- resident weights: fragments of TPW column tiles in registers, their scales in LDS
+    // ---- resident weights: fragments of TPW column tiles in registers, their scales in LDS.  All of
+    // it is requested here, behind the first activation tile, and consumed after that tile has been
+    // quantized: the quantizer runs while the weights are still on their way.
     static_assert(WL >= 0 && WL < TPW, "at least one column tile stays in registers");
     v4i wq[TPW - WL][NBLK];
     v4i* my_wq = lds_wq + static_cast<size_t>(wave) * WL * NBLK * 64 + lane;
     float* my_wd = lds_wd + static_cast<size_t>(wave) * TPW * NBLK * 32 + lane;
+    auto col_tile_of = [&](int t) {
+        const int ct = t * NW + wave;                  // round t of the waves covers NW adjacent column tiles
+        return ct < mct_pad ? ct : mct_pad - 1;        // tiles past the end repeat the last one; never stored
+    };
+#pragma unroll
+    for (int t = 0; t < TPW - WL; ++t) {
+#pragma unroll
+        for (int b = 0; b < NBLK; ++b)
+            wq[t][b] = *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(col_tile_of(t) * NBLK + b) * 64 + lane) * 16);
+    }
+    // scales of one column tile: NBLK x 32 halves, contiguous; a lane takes four at a time
+    constexpr int DCHUNKS = NBLK * 8;                  // groups of four halves per column tile
+    constexpr int DREP = (DCHUNKS + 63) / 64;
+    uint2 draw[TPW][DREP];
     {
         const uint16_t* dplane = reinterpret_cast<const uint16_t*>(W + static_cast<size_t>(mct_pad) * NBLK * 1024);
 #pragma unroll
         for (int t = 0; t < TPW; ++t) {
-            int ct = t * NW + wave;                    // round t of the waves covers NW adjacent column tiles
-            ct = ct < mct_pad ? ct : mct_pad - 1;      // tiles past the end repeat the last one; never stored
 #pragma unroll
-            for (int b = 0; b < NBLK; ++b) {
-                const v4i frag = *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(ct * NBLK + b) * 64 + lane) * 16);
-                if (t < TPW - WL) wq[t < TPW - WL ? t : 0][b] = frag;
-                else my_wq[((t - (TPW - WL)) * NBLK + b) * 64] = frag;
-                const float d = half_bits_to_float(dplane[(ct * NBLK + b) * 32 + j]);
-                if (!hh) my_wd[(t * NBLK + b) * 32] = d;
+            for (int r = 0; r < DREP; ++r) {
+                int ci = lane + 64 * r;
+                ci = ci < DCHUNKS ? ci : DCHUNKS - 1;
+                draw[t][r] = *reinterpret_cast<const uint2*>(dplane + static_cast<size_t>(col_tile_of(t)) * NBLK * 32 + ci * 4);
             }
         }
     }
     PPML_TRACE_MARK(42);
-    if (tid < WS_NBUF) lds_ready[tid] = 0u;
-    __syncthreads();
-    PPML_TRACE_MARK(43);
 
     // quantizes the tile held in xv into LDS buffer `buf`
     auto quantize_tile = [&](int buf, int tok0, v4f (&xv)[UPW][2]) {
@@ -818,6 +829,28 @@ __device__ __forceinline__ void q8_linear_ws_body(
     if (n_iter > 0) {
         quantize_tile(0, tile * TILE_TOK, xv);
         announce(0);
+    }
+    PPML_TRACE_MARK(43);
+    // weight scales and the fragments that live in LDS: written and read by this wave only
+#pragma unroll
+    for (int t = 0; t < TPW; ++t) {
+#pragma unroll
+        for (int r = 0; r < DREP; ++r) {
+            const int ci = lane + 64 * r;
+            if (ci < DCHUNKS) {
+                const uint2 h4 = draw[t][r];
+                const v4f d4{half_bits_to_float(static_cast<uint16_t>(h4.x & 0xffffu)), half_bits_to_float(static_cast<uint16_t>(h4.x >> 16)),
+                             half_bits_to_float(static_cast<uint16_t>(h4.y & 0xffffu)), half_bits_to_float(static_cast<uint16_t>(h4.y >> 16))};
+                *reinterpret_cast<v4f*>(my_wd - lane + t * NBLK * 32 + ci * 4) = d4;
+            }
+        }
+    }
+#pragma unroll
+    for (int t = TPW - WL; t < TPW; ++t) {
+#pragma unroll
+        for (int b = 0; b < NBLK; ++b)
+            my_wq[((t - (TPW - WL)) * NBLK + b) * 64] =
+                *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(col_tile_of(t) * NBLK + b) * 64 + lane) * 16);
     }
     PPML_TRACE_MARK(44);
     // Every weight fragment has arrived before the loop starts: a load still pending here would make
