@@ -313,7 +313,7 @@ __device__ unsigned long long* g_q8_trace = nullptr;
 __device__ int g_q8_dbg[4] = {0, 0, 0, 0};
 #define PPML_TRACE_MARK(slot)                                                                      \
     do {                                                                                           \
-        if (g_q8_trace && (threadIdx.x & 63) == 0)                                                 \
+        if ((PPML_Q8_TRACE == 1 || (slot) == 0 || (slot) >= 60) && g_q8_trace && (threadIdx.x & 63) == 0) \
             g_q8_trace[(static_cast<size_t>(blockIdx.x) * NW + (threadIdx.x >> 6)) * 64 + (slot)] = \
                 __builtin_amdgcn_s_memrealtime();   /* 100 MHz, common to the whole device */      \
     } while (0)
@@ -698,9 +698,21 @@ __device__ __forceinline__ void q8_linear_ws_body(
     // which the kernel attribute keeps away from the register allocator: load_tile_async() writes
     // them, take_tile() waits for exactly these loads and only then copies them out.
     constexpr int STAGE = ws_staging_regs(NBLK, NW);
-    constexpr int STAGE0 = 256 - STAGE;
+    constexpr int STAGE0 = 256 - STAGE;                // two waves per SIMD: 256 registers each
     static_assert(UPW * 8 <= STAGE, "staging registers hold one tile share");
+    // The diagnostic (DUMP) instances leave the fixed registers alone: the extra code of the dumps makes
+    // the compiler spill scalar registers into lanes of a vector register of its choosing, which may be
+    // one of these.  They read each tile with ordinary loads where the fast instances take it over.
+    constexpr bool ASYNC = !DUMP;
+    // Instances short of registers rebuild lane-dependent addresses where they are used, from a copy of
+    // the lane number the optimizer cannot trace, instead of keeping (or spilling) them across the loop.
+    constexpr bool LEAN = STAGE >= 64;
     auto load_tile_async = [&](int tile) {
+        if constexpr (!ASYNC) return;
+        int ln = lane;
+        if (LEAN) asm volatile("" : "+v"(ln));
+        const int grp = ln >> 2, c4 = ln & 3;
+        const int urow = grp & 7, ublk = grp >> 3;
 #pragma unroll
         for (int s = 0; s < UPW; ++s) {
             int u = wave + s * NW;
@@ -709,6 +721,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
             int t = tile * TILE_TOK + (u & 3) * 8 + urow;
             t = t < N ? t : N - 1;
             const float* src = X + static_cast<int64_t>(t) * K + bl * QK + c4 * 8;
+            // the clobber names the top register, which makes the kernel own all 256 of them
             asm volatile("global_load_dwordx4 v[%1:%2], %0, off\n\tglobal_load_dwordx4 v[%3:%4], %0, off offset:16"
                          :: "v"(src), "n"(STAGE0 + 8 * s), "n"(STAGE0 + 8 * s + 3), "n"(STAGE0 + 8 * s + 4), "n"(STAGE0 + 8 * s + 7)
                          : "memory", "v255");
@@ -716,7 +729,11 @@ __device__ __forceinline__ void q8_linear_ws_body(
     };
     // `newer` = vector-memory operations issued after load_tile_async: once at most that many are
     // outstanding, its loads have landed.
-    auto take_tile = [&](auto newer, v4f (&xv)[UPW][2]) {
+    auto take_tile = [&](auto newer, int tile, v4f (&xv)[UPW][2]) {
+        if constexpr (!ASYNC) {
+            load_tile(tile, xv);
+            return;
+        }
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(newer)::value) : "memory");
 #pragma unroll
         for (int s = 0; s < UPW; ++s) {
@@ -791,6 +808,10 @@ __device__ __forceinline__ void q8_linear_ws_body(
 
     // quantizes the tile held in xv into LDS buffer `buf`
     auto quantize_tile = [&](int buf, int tok0, v4f (&xv)[UPW][2]) {
+        int ln = lane;
+        if (LEAN) asm volatile("" : "+v"(ln));
+        const int grp = ln >> 2, c4 = ln & 3;
+        const int urow = grp & 7, ublk = grp >> 3;
 #pragma unroll
         for (int s = 0; s < UPW; ++s) {
             const int u = wave + s * NW;
@@ -944,18 +965,23 @@ __device__ __forceinline__ void q8_linear_ws_body(
                 // exactly 16 stores here and the memory counter stays predictable.
                 const uint32_t base = (static_cast<uint32_t>(tok0 + 4 * hh) * M + m) * 4u;
                 const uint32_t out_of_range = 0xfffffff0u;
+                // Row pitch through a copy the optimizer cannot trace: the sixteen scalar row offsets are
+                // then rebuilt here (a handful of scalar operations) instead of occupying sixteen
+                // scalar registers for the whole kernel, which has none to spare.
+                int pitch = M * 4;
+                asm volatile("" : "+s"(pitch));
                 if (tok0 + TILE_TOK <= N) {
                     const uint32_t b0 = m < M ? base : out_of_range;
 #pragma unroll
                     for (int r = 0; r < 16; ++r)
                         __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[r]), c_rsrc, b0,
-                                                              (8 * (r >> 2) + (r & 3)) * M * 4, WS_STORE_AUX);
+                                                              (8 * (r >> 2) + (r & 3)) * pitch, WS_STORE_AUX);
                 } else {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const bool ok = m < M && tok0 + mfma32_row(r, lane) < N;
                         __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[r]), c_rsrc, ok ? base : out_of_range,
-                                                              (8 * (r >> 2) + (r & 3)) * M * 4, WS_STORE_AUX);
+                                                              (8 * (r >> 2) + (r & 3)) * pitch, WS_STORE_AUX);
                     }
                 }
             }
@@ -971,8 +997,8 @@ __device__ __forceinline__ void q8_linear_ws_body(
                 PPML_TRACE_MARK(2 + 10 * it + 7);
                 {
                     v4f xn[UPW][2];
-                    if (it == 0) take_tile(std::integral_constant<int, NEWER_FIRST>{}, xn);
-                    else take_tile(std::integral_constant<int, NEWER>{}, xn);
+                    if (it == 0) take_tile(std::integral_constant<int, NEWER_FIRST>{}, next, xn);
+                    else take_tile(std::integral_constant<int, NEWER>{}, next, xn);
                     if (it + 2 < n_iter) load_tile_async(tile_of(it + 2));
                     quantize_tile((it + 1) % WS_NBUF, next * TILE_TOK, xn);
                     announce((it + 1) % WS_NBUF);
@@ -987,56 +1013,85 @@ __device__ __forceinline__ void q8_linear_ws_body(
             // other wave of the SIMD.
             PairOps pe, po;
             const int s0 = t0 * NBLK;
+            // Beside 64 staging registers there is no room for a second operand set: one set, refilled as
+            // soon as its MFMAs are issued.
+            constexpr bool TWO_SETS = !LEAN;
             fetch_pair(s0, pe);
-            if (NBLK > 2) fetch_pair(s0 + 2, po);
-            sum_a = block_sum(s0, pe.a0, pe.w0);
+            if (TWO_SETS && NBLK > 2) fetch_pair(s0 + 2, po);
+            if (TWO_SETS) sum_a = block_sum(s0, pe.a0, pe.w0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int pr = 0; pr < NBLK / 2; ++pr) {
                 const int st = s0 + 2 * pr;
-                PairOps& cur = (pr & 1) ? po : pe;
-                PairOps& nxt = (pr & 1) ? pe : po;
-                scl = __builtin_amdgcn_mfma_f32_32x32x1f32(cur.da, cur.dw, zero_f2, 0, 0, 0);
-                sum_b = block_sum(st + 1, cur.a1, cur.w1);
-                __builtin_amdgcn_sched_barrier(0);
-                settle(st, sum_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
-                __builtin_amdgcn_sched_barrier(0);
-                if (2 * pr + 2 < NBLK) sum_a = block_sum(st + 2, nxt.a0, nxt.w0);
-                if (2 * pr + 4 < NBLK) fetch_pair(st + 4, cur);
-                __builtin_amdgcn_sched_barrier(0);
-                settle(st + 1, sum_b, __builtin_shufflevector(scl, scl, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31));
-                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (TWO_SETS) {
+                    PairOps& cur = (pr & 1) ? po : pe;
+                    PairOps& nxt = (pr & 1) ? pe : po;
+                    scl = __builtin_amdgcn_mfma_f32_32x32x1f32(cur.da, cur.dw, zero_f2, 0, 0, 0);
+                    sum_b = block_sum(st + 1, cur.a1, cur.w1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    settle(st, sum_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (2 * pr + 2 < NBLK) sum_a = block_sum(st + 2, nxt.a0, nxt.w0);
+                    if (2 * pr + 4 < NBLK) fetch_pair(st + 4, cur);
+                    __builtin_amdgcn_sched_barrier(0);
+                    settle(st + 1, sum_b, __builtin_shufflevector(scl, scl, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31));
+                    __builtin_amdgcn_sched_barrier(0);
+                } else {
+                    // one block sum alive at a time; the other wave of the SIMD fills the waits
+                    scl = __builtin_amdgcn_mfma_f32_32x32x1f32(pe.da, pe.dw, zero_f2, 0, 0, 0);
+                    sum_a = block_sum(st, pe.a0, pe.w0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    settle(st, sum_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
+                    __builtin_amdgcn_sched_barrier(0);
+                    sum_a = block_sum(st + 1, pe.a1, pe.w1);
+                    if (2 * pr + 2 < NBLK) fetch_pair(st + 2, pe);
+                    __builtin_amdgcn_sched_barrier(0);
+                    settle(st + 1, sum_a, __builtin_shufflevector(scl, scl, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31));
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             PPML_TRACE_MARK(2 + 10 * it + 1 + t0);
         }
         PPML_TRACE_MARK(2 + 10 * it + 9);
     }
+#ifdef PPML_Q8_TRACE
+    // shader clock under this kernel's load: 1024 x 16 x s_nop 15 = 262144 cycles plus loop overhead
+    PPML_TRACE_MARK(60);
+    for (int i = 0; g_q8_trace && i < 1024; ++i)
+        asm volatile("s_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\n"
+                     "s_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15" ::: "memory");
+    PPML_TRACE_MARK(61);
+#endif
 }
 
-// The attribute takes a literal, hence one kernel per staging size (16 registers up to K = 256, 32 beyond).
+// The attribute takes a literal, hence one kernel per staging size (16 registers up to K = 256, 32 or
+// 64 beyond).  On this target the register allocator's budget is TWICE the attribute's value (the
+// value counts architectural and accumulation registers separately): 120 keeps it below v240.  A
+// value the compiler does not honour would go unnoticed until its registers and the staged tile
+// collide, so the build checks the generated code (check_ws_isa.py).
 template <int NW, int TPW, int NBLK, int WL, bool DUMP>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(240)))
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(120)))
 void q8_linear_ws_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                          int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                          int32_t* __restrict__ sums_dump) {
-    static_assert(ws_compiler_vgprs(NBLK, NW) == 240, "staging size");
+    static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 120, "staging size");
     q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 template <int NW, int TPW, int NBLK, int WL, bool DUMP>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(224)))
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(112)))
 void q8_linear_ws32_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
-    static_assert(ws_compiler_vgprs(NBLK, NW) == 224, "staging size");
+    static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 112, "staging size");
     q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
 template <int NW, int TPW, int NBLK, int WL, bool DUMP>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(192)))
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(96)))
 void q8_linear_ws64_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
-    static_assert(ws_compiler_vgprs(NBLK, NW) == 192, "staging size");
+    static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 96, "staging size");
     q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
@@ -1058,7 +1113,7 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
     // Eight waves fill a CU (256 registers each): one resident work-group of 8 waves per CU, or two
     // of 4.  With more tiles than resident work-groups every work-group takes the same number of
     // tiles (824 tiles on 256 CUs: 206 work-groups x 4 rather than 256 x 3 + 56 x 1).
-    const int cus = device_cu_count() * (8 / NW);
+    const int cus = device_cu_count() * (NW == 4 ? 2 : 1);
     const int all_tiles = (N + TILE_TOK - 1) / TILE_TOK;
     int wgs, ntiles = all_tiles, npart = 0;
     const int left = all_tiles % cus;
