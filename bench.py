@@ -27,7 +27,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE
 # scaled by the same counters on a 1 GiB copy: factors 2.000 and 1.000).
-MEASURED_TRAFFIC_BYTES = 109_890_000   # 28.89 MB read + 81.00 MB written per launch
+MEASURED_TRAFFIC_BYTES = 113_570_000   # 28.89 MB read + 81.00 MB written per launch
 
 
 def q8_bytes(rows, K, N):
@@ -38,8 +38,9 @@ def q8_bytes(rows, K, N):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=500,
+                    help="untimed steps; the shader clock needs 1-2 ms of load to reach its steady value")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configured shapes")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -185,7 +186,7 @@ def main() -> int:
             a = torch.randn(256, 12288, device=dev, generator=gen) * 0.1
             b = torch.randn(256, 12288, device=dev, generator=gen) * 0.1
             return (lambda i: ops.mul_mat_tn(a, b, 1.0 / 256)), 1
-        steps, warm = 10, 3
+        steps, warm = 50, 10
         f32_case(opm, (2 * 256 * 12288 + 12288 * 12288) * 4, 2.0 * 12288 * 12288 * 256, "opm_dense_12288x256x12288")
         out["extra"] = extra
 
