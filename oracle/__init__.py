@@ -18,6 +18,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libppml_oracle.so")
 _REF_PATH = os.path.join(_HERE, "_ref", "libppml_ref_half.so")
+_REF_FLASH_PATH = os.path.join(_HERE, "_ref", "libppml_ref_flash.so")
 
 QK = 32
 BLOCK_BYTES = 34
@@ -73,6 +74,8 @@ def _load() -> C.CDLL:
     lib.orc_outer_product_mean_value.argtypes = [f32p, f32p, f32p] + [i64] * 4 + [C.c_int]
     lib.orc_attention_scores.restype = None
     lib.orc_attention_scores.argtypes = [f32p, f32p, f32p] + [i64] * 5 + [C.c_int]
+    lib.orc_flash_attn_forward.restype = C.c_int
+    lib.orc_flash_attn_forward.argtypes = ([C.c_int] * 5 + [C.c_float, C.c_float, C.c_int] + [f32p] * 6 + [C.c_int])
     lib.orc_max_threads.restype = C.c_int
     return lib
 
@@ -298,3 +301,53 @@ def attention_scores(q, k, nthreads=0) -> np.ndarray:
     out = np.empty((NQ, H, Lq, Lk), dtype=np.float32)
     lib().orc_attention_scores(_fp(q), _fp(k), _fp(out), NQ, H, D, Lq, Lk, nthreads)
     return out
+
+
+def _opt_fp(a):
+    return _fp(a) if a is not None else C.POINTER(C.c_float)()
+
+
+def flash_attn_forward(q, k, v, bias=None, causal=False, scale=0.0, eps=1e-9, Bc=64, nthreads=0):
+    """Q, K, V (B,h,L,d), bias (B,h,L,L) or None -> O (B,h,L,d), LSE (B,h,L)  (FlashAttn.cpp:55-135)."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    B, h, L, d = q.shape
+    bias = _f32(bias) if bias is not None else None
+    o = np.empty_like(q)
+    lse = np.empty((B, h, L), dtype=np.float32)
+    rc = lib().orc_flash_attn_forward(B, h, L, d, int(causal), scale, eps, Bc, _fp(q), _fp(k), _fp(v), _opt_fp(bias),
+                                      _fp(o), _fp(lse), nthreads or max_threads())
+    if rc:
+        raise ValueError(f"orc_flash_attn_forward rc={rc}")
+    return o, lse
+
+
+def ref_flash_lib():
+    """The reference's own src/ops/FlashAttn.cpp compiled as-is, or None when it was never built."""
+    if not os.path.exists(_REF_FLASH_PATH):
+        return None
+    ref = C.CDLL(_REF_FLASH_PATH)
+    f32p = C.POINTER(C.c_float)
+    ref.ref_flash_attn_forward.restype = C.c_int
+    ref.ref_flash_attn_forward.argtypes = [C.c_int] * 5 + [C.c_float, C.c_float, C.c_int] + [f32p] * 6
+    ref.ref_flash_attn_forward_plain.restype = C.c_int
+    ref.ref_flash_attn_forward_plain.argtypes = [C.c_int] * 5 + [C.c_float] + [f32p] * 6
+    return ref
+
+
+def ref_flash_attn_forward(q, k, v, bias=None, causal=False, scale=0.0, eps=1e-9, Bc=64, plain=False):
+    """Same arguments through the compiled reference; `plain` = its three-pass routine (no eps)."""
+    ref = ref_flash_lib()
+    if ref is None:
+        return None
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    B, h, L, d = q.shape
+    bias = _f32(bias) if bias is not None else None
+    o = np.empty_like(q)
+    lse = np.empty((B, h, L), dtype=np.float32)
+    if plain:
+        rc = ref.ref_flash_attn_forward_plain(B, h, L, d, int(causal), scale, _fp(q), _fp(k), _fp(v), _opt_fp(bias), _fp(o), _fp(lse))
+    else:
+        rc = ref.ref_flash_attn_forward(B, h, L, d, int(causal), scale, eps, Bc, _fp(q), _fp(k), _fp(v), _opt_fp(bias), _fp(o), _fp(lse))
+    if rc:
+        raise ValueError(f"reference refused the arguments (rc={rc})")
+    return o, lse

@@ -26,6 +26,12 @@
  *       einsum over the layout stated at src/backend/CPUKernels.cpp:975-981.
  *   orc_outer_product_mean_value : known answers of tests/test_outer_product_mean.cpp:10-70.
  *   orc_attention_scores: einsum special case and the 1/sqrt(D) closed form.
+ *   orc_flash_attn_forward : the reference's own src/ops/FlashAttn.cpp compiled as-is
+ *       (oracle/_ref/libppml_ref_flash.so: it needs nothing but its header) -- bit-for-bit on
+ *       random inputs, with and without bias, causal and not, ragged block sizes; plus float64
+ *       softmax attention, closed forms (equal scores -> mean of V, one dominant key -> that
+ *       row of V, shift invariance in the bias, fully masked rows) where the reference build
+ *       is absent.
  */
 #include "ppml_oracle.h"
 
@@ -44,6 +50,74 @@ static int pick_threads(int nthreads) {
     (void)nthreads;
     return 1;
 #endif
+}
+
+/* src/ops/FlashAttn.cpp:55-135.  Same loop nest, same order of the sums (dot product over d ascending,
+ * scale, then bias; block maximum; alpha = exp(m - m_new) with 0 for the first block; P V per output
+ * column over the block's keys ascending; acc = alpha * acc + pv; l = alpha * l + l_tile).  The planes
+ * are independent, so they are spread over threads; within a row nothing is reordered. */
+int orc_flash_attn_forward(int B, int h, int L, int d, int causal, float scale, float softmax_eps, int Bc,
+                           const float *Q, const float *K, const float *V, const float *bias,
+                           float *O, float *LSE, int nthreads) {
+    if (!Q || !K || !V || !O) return 1;
+    if (B <= 0 || h <= 0 || L <= 0 || d <= 0) return 1;
+    if (Bc <= 0) Bc = 64;
+    const float sc = scale > 0.0f ? scale : 1.0f / sqrtf((float)d);
+    const int64_t planes = (int64_t)B * h;
+    if (nthreads <= 0) nthreads = 1;
+#pragma omp parallel for num_threads(nthreads) schedule(dynamic, 1)
+    for (int64_t pl = 0; pl < planes; ++pl) {
+        const float *Qb = Q + pl * (int64_t)L * d, *Kb = K + pl * (int64_t)L * d, *Vb = V + pl * (int64_t)L * d;
+        float *Ob = O + pl * (int64_t)L * d;
+        float *acc = (float *)malloc(sizeof(float) * (size_t)d);
+        float *tile = (float *)malloc(sizeof(float) * (size_t)Bc);
+        for (int i = 0; i < L; ++i) {
+            const float *q = Qb + (int64_t)i * d;
+            const int jmax = causal ? i + 1 : L;
+            float m = -INFINITY, l = 0.0f;
+            for (int dd = 0; dd < d; ++dd) acc[dd] = 0.0f;
+            for (int j0 = 0; j0 < jmax; j0 += Bc) {
+                const int j1 = j0 + Bc < jmax ? j0 + Bc : jmax, nb = j1 - j0;
+                float m_tile = -INFINITY;
+                for (int j = j0; j < j1; ++j) {
+                    const float *k = Kb + (int64_t)j * d;
+                    float s = 0.0f;
+                    for (int dd = 0; dd < d; ++dd) s += q[dd] * k[dd];
+                    s *= sc;
+                    if (bias) s += bias[(pl * L + i) * (int64_t)L + j];
+                    tile[j - j0] = s;
+                    if (s > m_tile) m_tile = s;
+                }
+                const float m_new = m > m_tile ? m : m_tile;
+                const float alpha = (m == -INFINITY) ? 0.0f : expf(m - m_new);
+                float l_tile = 0.0f;
+                for (int j = 0; j < nb; ++j) {
+                    const float p = expf(tile[j] - m_new);
+                    tile[j] = p;
+                    l_tile += p;
+                }
+                for (int dd = 0; dd < d; ++dd) {
+                    float pv = 0.0f;
+                    for (int j = 0; j < nb; ++j) pv += tile[j] * Vb[(int64_t)(j0 + j) * d + dd];
+                    acc[dd] = alpha * acc[dd] + pv;
+                }
+                l = alpha * l + l_tile;
+                m = m_new;
+            }
+            float *o = Ob + (int64_t)i * d;
+            if (l > 0.0f) {
+                const float inv = 1.0f / (l + softmax_eps);
+                for (int dd = 0; dd < d; ++dd) o[dd] = acc[dd] * inv;
+                if (LSE) LSE[pl * L + i] = m + logf(l + softmax_eps);
+            } else {
+                for (int dd = 0; dd < d; ++dd) o[dd] = 0.0f;
+                if (LSE) LSE[pl * L + i] = -INFINITY;
+            }
+        }
+        free(acc);
+        free(tile);
+    }
+    return 0;
 }
 
 int orc_max_threads(void) { return pick_threads(0); }

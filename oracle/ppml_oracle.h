@@ -84,6 +84,14 @@ void orc_outer_product_mean_value(const float *left, const float *right, float *
 void orc_attention_scores(const float *Q, const float *K, float *scores,
                           int64_t NQ, int64_t H, int64_t D, int64_t Lq, int64_t Lk, int nthreads);
 
+/* src/ops/FlashAttn.cpp:55-135 (flash_attn_forward_cpu): O = softmax(scale * Q K^T + bias) V, one pass over
+ * key blocks of Bc with a running maximum and sum.  Q, K, V, O are [B][h][L][d], bias (may be NULL) is
+ * [B][h][L query][L key], LSE (may be NULL) is [B][h][L].  scale <= 0 -> 1/sqrt(d).  A row whose sum
+ * is 0 gets O = 0, LSE = -inf.  returns 0 ok, 1 bad arguments (null pointer, non-positive dimension). */
+int orc_flash_attn_forward(int B, int h, int L, int d, int causal, float scale, float softmax_eps, int Bc,
+                           const float *Q, const float *K, const float *V, const float *bias,
+                           float *O, float *LSE, int nthreads);
+
 int orc_max_threads(void);
 
 #ifdef __cplusplus

@@ -60,3 +60,34 @@ def test_quantizer_hand_vector(oracle):
     assert int(oracle.block_scales_bits(blk).reshape(-1)[0]) == int(g["d_bits"], 16)
     q = oracle.block_quants(blk).reshape(-1)
     assert q[0] == g["q0"] and q[31] == g["q31"]
+
+
+# ----------------------------------------------------------------------------- fused attention forward
+FLASH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "flash_attn_forward.json")
+
+
+def flash_cases():
+    """Inputs and outputs of the reference's own flash_attn_forward_cpu (written by make_flash_attn_vectors.py)."""
+    with open(FLASH) as f:
+        data = json.load(f)
+    for c in data["cases"]:
+        shape = (c["B"], c["h"], c["L"], c["d"])
+        f32 = lambda bits, shp: np.array(bits, dtype=np.uint32).view(np.float32).reshape(shp)  # noqa: E731
+        yield {"cfg": c, "q": f32(c["q"], shape), "k": f32(c["k"], shape), "v": f32(c["v"], shape),
+               "bias": f32(c["bias"], (c["B"], c["h"], c["L"], c["L"])) if c["bias"] is not None else None,
+               "o": f32(c["o"], shape), "lse": f32(c["lse"], shape[:3])}
+
+
+def test_flash_attn_forward_matches_the_reference_vectors_bit_for_bit(oracle):
+    n = 0
+    for c in flash_cases():
+        cfg = c["cfg"]
+        o, lse = oracle.flash_attn_forward(c["q"], c["k"], c["v"], c["bias"], causal=cfg["causal"], scale=cfg["scale"],
+                                           eps=cfg["eps"], Bc=cfg["Bc"])
+        assert (o.view(np.uint32) == c["o"].view(np.uint32)).all(), cfg["L"]
+        assert (lse.view(np.uint32) == c["lse"].view(np.uint32)).all(), cfg["L"]
+        n += 1
+    assert n == 4
+    # the vectors do contain the special row: fully masked -> O = 0, LSE = -inf
+    first = next(flash_cases())
+    assert np.isneginf(first["lse"][0, 0, 1]) and (first["o"][0, 0, 1] == 0).all()

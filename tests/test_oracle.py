@@ -483,3 +483,90 @@ def test_attention_scores_vs_einsum(oracle):
     kk = np.ascontiguousarray(k.reshape(NQ, H, D, Lk))
     op = oracle.out_prod(kk, q)                                      # [NQ,H,Lq,Lk]
     assert (op * np.float32(0.25) == got).all()
+
+
+# ----------------------------------------------------------------------------- fused attention forward
+def _attention_f64(q, k, v, bias, causal, scale, eps):
+    """Textbook softmax attention in float64, written independently of the oracle's loop."""
+    B, h, L, d = q.shape
+    sc = scale if scale > 0 else 1.0 / np.sqrt(d)
+    s = np.einsum("bhid,bhjd->bhij", q.astype(np.float64), k.astype(np.float64)) * sc
+    if bias is not None:
+        s = s + bias.astype(np.float64)
+    if causal:
+        s = np.where(np.tril(np.ones((L, L), dtype=bool)), s, -np.inf)
+    m = s.max(axis=-1, keepdims=True)
+    m = np.where(np.isfinite(m), m, 0.0)
+    e = np.exp(s - m)
+    l = e.sum(axis=-1, keepdims=True)
+    o = np.einsum("bhij,bhjd->bhid", e / (l + eps), v.astype(np.float64))
+    with np.errstate(divide="ignore"):
+        lse = (m + np.log(l + eps))[..., 0]
+    return o, np.where(l[..., 0] > 0, lse, -np.inf)
+
+
+@pytest.mark.parametrize("B,h,L,d,causal,Bc,use_bias", [
+    (2, 3, 37, 8, False, 64, True), (1, 2, 103, 32, False, 64, False), (1, 1, 70, 12, True, 16, True),
+    (2, 1, 5, 4, True, 64, False), (1, 2, 130, 64, False, 32, True), (1, 1, 1, 4, False, 64, True),
+])
+def test_flash_attn_forward_against_the_compiled_reference(oracle, B, h, L, d, causal, Bc, use_bias):
+    if oracle.ref_flash_lib() is None:
+        pytest.skip("oracle/_ref/libppml_ref_flash.so not built (reference tree absent)")
+    rng = np.random.default_rng(L * 131 + d)
+    q, k, v = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(3)]
+    bias = (3 * rng.standard_normal((B, h, L, L))).astype(np.float32) if use_bias else None
+    o, lse = oracle.flash_attn_forward(q, k, v, bias, causal=causal, Bc=Bc)
+    ro, rlse = oracle.ref_flash_attn_forward(q, k, v, bias, causal=causal, Bc=Bc)
+    assert (o.view(np.uint32) == ro.view(np.uint32)).all()
+    assert (lse.view(np.uint32) == rlse.view(np.uint32)).all()
+
+
+@pytest.mark.parametrize("causal,use_bias,scale", [(False, True, 0.0), (True, False, 0.0), (False, False, 0.37), (True, True, 2.0)])
+def test_flash_attn_forward_against_float64_softmax(oracle, causal, use_bias, scale):
+    rng = np.random.default_rng(5)
+    B, h, L, d = 2, 2, 77, 16
+    q, k, v = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(3)]
+    bias = rng.standard_normal((B, h, L, L)).astype(np.float32) if use_bias else None
+    o, lse = oracle.flash_attn_forward(q, k, v, bias, causal=causal, scale=scale, Bc=16)
+    wo, wlse = _attention_f64(q, k, v, bias, causal, scale, 1e-9)
+    assert np.abs(o - wo).max() <= 2e-6 * max(1.0, np.abs(wo).max())
+    assert np.abs(lse - wlse).max() <= 2e-6 * np.abs(wlse).max()
+
+
+def test_flash_attn_forward_closed_forms(oracle):
+    rng = np.random.default_rng(9)
+    B, h, L, d = 1, 2, 40, 8
+    v = rng.standard_normal((B, h, L, d)).astype(np.float32)
+    k = rng.standard_normal((B, h, L, d)).astype(np.float32)
+    zero_q = np.zeros((B, h, L, d), dtype=np.float32)
+    # equal scores: every output row is the mean of V and LSE = log(L) (a swapped Q/K or a dropped
+    # normalisation would not give this); causal: row i is the mean of the first i + 1 rows
+    o, lse = oracle.flash_attn_forward(zero_q, k, v, eps=0.0, Bc=16)
+    assert np.allclose(o, v.mean(axis=2, keepdims=True), atol=1e-6)
+    assert np.allclose(lse, np.log(L), atol=1e-6)
+    o, _ = oracle.flash_attn_forward(zero_q, k, v, causal=True, eps=0.0, Bc=16)
+    want = np.cumsum(v.astype(np.float64), axis=2) / np.arange(1, L + 1)[None, None, :, None]
+    assert np.allclose(o, want, atol=1e-6)
+    # a bias that towers over the scores at key (i * 7) % L picks that row of V: bias is indexed [query][key]
+    q = rng.standard_normal((B, h, L, d)).astype(np.float32)
+    bias = np.zeros((B, h, L, L), dtype=np.float32)
+    pick = (np.arange(L) * 7) % L
+    bias[:, :, np.arange(L), pick] = 200.0
+    o, _ = oracle.flash_attn_forward(q, k, v, bias)
+    assert np.allclose(o, v[:, :, pick, :], atol=1e-6)
+    # adding a constant per query row to the bias changes LSE by that constant and leaves O alone
+    bias = rng.standard_normal((B, h, L, L)).astype(np.float32)
+    shift = rng.standard_normal((B, h, L, 1)).astype(np.float32)
+    o0, l0 = oracle.flash_attn_forward(q, k, v, bias)
+    o1, l1 = oracle.flash_attn_forward(q, k, v, bias + shift)
+    assert np.allclose(o0, o1, atol=2e-6) and np.allclose(l1 - l0, shift[..., 0], atol=1e-5)
+    # the scale multiplies the dot product only, not the bias
+    o2, _ = oracle.flash_attn_forward(2 * q, k, v, bias, scale=0.5)
+    o3, _ = oracle.flash_attn_forward(q, k, v, bias, scale=1.0)
+    assert np.allclose(o2, o3, atol=2e-6)
+    # fully masked row: O = 0 and LSE = -inf; its neighbours are untouched
+    bias[0, 1, 3, :] = -np.inf
+    o4, l4 = oracle.flash_attn_forward(q, k, v, bias)
+    assert (o4[0, 1, 3] == 0).all() and np.isneginf(l4[0, 1, 3]) and np.isfinite(l4[0, 1, 2])
+    # bad arguments are refused, not computed
+    assert oracle.lib().orc_flash_attn_forward(1, 1, 0, 4, 0, 0.0, 0.0, 64, None, None, None, None, None, None, 1) == 1
