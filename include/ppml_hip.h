@@ -138,6 +138,23 @@ int outer_product_mean_value_hip(const float *left, const float *right, float *d
 int mul_mat_tn_hip(const float *A, const float *Bm, float *O, int M, int K, int Nc, float alpha,
                    ppml_hip_stream_t stream);
 
+/* ---- fused attention forward ------------------------------------------------------------------ */
+/* replaces flash_attn_forward_cuda (declared src/backend/CUDAKernels.cpp:174, contract
+ * include/ppml/FlashAttn.h:8-65, called from kernel_flash_attn_ext_cuda, CUDAKernels.cpp:894-903);
+ * the fields of FlashAttnConfig are passed one by one.  The mathematics is that of
+ * flash_attn_forward_cpu (src/ops/FlashAttn.cpp:55-135):
+ *     O = softmax(scale * Q K^T + bias) V,  LSE = m + log(l + softmax_eps),  O = acc / (l + softmax_eps)
+ * Q, K, V, O: [B][h][L][d] f32, 16-byte aligned; bias (may be NULL): [B][h][L query][L key];
+ * LSE (may be NULL): [B][h][L].  scale <= 0 means 1/sqrt(d).  causal: key j <= query i only.
+ * Bc is the reference's key-block width (<= 0 means 64); it does not change the arithmetic except
+ * for one corner the reference has: a row whose first Bc keys are all masked with -inf is written
+ * as O = 0, LSE = -inf even if later keys are not masked, as is a row masked entirely.
+ * returns 0 = ran; 1 = refused (null pointer, non-positive size, d > 64 or d % 4 != 0 -- the
+ * rule of src/backend/CUDABackend.cpp:457-463 -- misaligned pointer, B*h > 65535); 6 = launch error. */
+int flash_attn_forward_hip(int B, int h, int L, int d, int causal, float scale, float softmax_eps, int Bc,
+                           const float *Q, const float *K, const float *V, const float *bias,
+                           float *O, float *LSE, ppml_hip_stream_t stream);
+
 /* ---- observability (include/ppml/MulMatStats.h:154-169) -------------------------------------- */
 /* Per-shape call counters keyed like the reference (M<<40 | K<<20 | N); enabled by the
  * environment variable PPML_MULMAT_STATS=1.  Writes up to `cap` rows of

@@ -1,0 +1,162 @@
+"""GPU parity of the fused attention forward (flash_attn_forward_hip) against the CPU oracle, which is
+itself checked bit for bit against the reference's compiled src/ops/FlashAttn.cpp.
+
+Bar: 1e-4 relative on O (normwise per case, the f32 bar of this backend) and 1e-5 + 1e-5 * |LSE| on
+LSE.  The GPU sums in another order (fp32 MFMA, keys 32 at a time, hardware exp/log), so equality is
+not expected; special rows (fully masked, masked first block) must match exactly: O = 0, LSE = -inf.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+RTOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "GPU tests need a device"
+    from proteinpredictmachinelearning_amd import ops as _ops
+
+    return _ops
+
+
+def _dev(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _run(ops, q, k, v, bias=None, **kw):
+    o, lse = ops.flash_attn_forward(_dev(q), _dev(k), _dev(v), _dev(bias), **kw)
+    ops.synchronize()
+    return o.cpu().numpy(), lse.cpu().numpy()
+
+
+def _check(got_o, got_lse, want_o, want_lse):
+    dead = np.isneginf(want_lse)
+    assert (np.isneginf(got_lse) == dead).all(), "rows written as masked differ"
+    assert (got_o[dead] == 0).all()
+    scale = max(np.abs(want_o).max(), 1e-30)
+    err = np.abs(got_o.astype(np.float64) - want_o).max() / scale
+    assert err <= RTOL, f"O normwise {err:.3e}"
+    live = ~dead
+    lerr = np.abs(got_lse[live].astype(np.float64) - want_lse[live])
+    assert (lerr <= 1e-5 + 1e-5 * np.abs(want_lse[live])).all(), f"LSE {lerr.max():.3e}"
+
+
+CASES = [
+    # B, h, L, d, causal, bias
+    (1, 1, 1, 4, False, False),          # a single key
+    (2, 3, 37, 8, False, True),          # ragged tile, small head
+    (1, 4, 103, 32, False, True),        # pair-track plane of the configured model (L = 103, d = 32)
+    (1, 4, 103, 32, False, False),
+    (1, 2, 128, 32, True, False),        # four full tiles, causal
+    (1, 2, 129, 32, False, True),        # first shape of the eight-wave instance, ragged
+    (2, 2, 256, 32, False, True),        # MSA-track plane (L = 256): bias rows read 16 bytes at a time
+    (1, 2, 300, 32, True, True),         # more keys than one LDS stage holds (256)
+    (1, 2, 70, 64, False, True),         # d = 64 instance
+    (1, 1, 200, 64, True, False),        # d = 64, two LDS stages (128 keys each), causal
+    (1, 2, 45, 20, False, True),         # d not a multiple of 32: padded columns
+    (1, 1, 64, 48, False, False),
+]
+
+
+@pytest.mark.parametrize("B,h,L,d,causal,use_bias", CASES)
+def test_flash_attn_forward_matches_oracle(ops, oracle, B, h, L, d, causal, use_bias):
+    rng = np.random.default_rng(1000 * L + d + int(causal))
+    q, k, v = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(3)]
+    bias = (2 * rng.standard_normal((B, h, L, L))).astype(np.float32) if use_bias else None
+    want_o, want_lse = oracle.flash_attn_forward(q, k, v, bias, causal=causal)
+    got_o, got_lse = _run(ops, q, k, v, bias, causal=causal)
+    _check(got_o, got_lse, want_o, want_lse)
+
+
+def test_reference_golden_vectors(ops):
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "flash_attn_forward.json")
+    with open(path) as f:
+        cases = json.load(f)["cases"]
+    for c in cases:
+        shape = (c["B"], c["h"], c["L"], c["d"])
+        f32 = lambda bits, shp: np.array(bits, dtype=np.uint32).view(np.float32).reshape(shp)  # noqa: E731
+        bias = f32(c["bias"], (c["B"], c["h"], c["L"], c["L"])) if c["bias"] is not None else None
+        got_o, got_lse = _run(ops, f32(c["q"], shape), f32(c["k"], shape), f32(c["v"], shape), bias,
+                              causal=c["causal"], scale=c["scale"], eps=c["eps"], Bc=c["Bc"])
+        _check(got_o, got_lse, f32(c["o"], shape), f32(c["lse"], shape[:3]))
+
+
+def test_scale_eps_and_missing_lse(ops, oracle):
+    rng = np.random.default_rng(3)
+    q, k, v = [rng.standard_normal((1, 2, 50, 16)).astype(np.float32) for _ in range(3)]
+    want_o, want_lse = oracle.flash_attn_forward(q, k, v, None, scale=0.3, eps=0.5)
+    got_o, got_lse = _run(ops, q, k, v, scale=0.3, eps=0.5)
+    _check(got_o, got_lse, want_o, want_lse)
+    o, lse = ops.flash_attn_forward(_dev(q), _dev(k), _dev(v), scale=0.3, eps=0.5, want_lse=False)
+    ops.synchronize()
+    assert lse is None and np.array_equal(o.cpu().numpy(), got_o)
+
+
+def test_masked_rows_and_the_masked_first_block(ops, oracle):
+    rng = np.random.default_rng(4)
+    B, h, L, d = 1, 2, 160, 32
+    q, k, v = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(3)]
+    bias = rng.standard_normal((B, h, L, L)).astype(np.float32)
+    bias[0, 0, 5, :] = -np.inf            # masked entirely
+    bias[0, 0, 6, :64] = -np.inf          # the reference's first block (Bc = 64) masked: row poisoned
+    bias[0, 0, 7, :63] = -np.inf          # one key of a 64-key first block survives; a 32-key first block does not
+    bias[0, 1, 8, 64:] = -np.inf          # only the first block survives: ordinary row
+    bias[0, 1, 9, :32] = -np.inf          # with Bc = 32 this row is poisoned, with 64 it is not
+    for Bc in (64, 32):
+        want_o, want_lse = oracle.flash_attn_forward(q, k, v, bias, Bc=Bc)
+        assert np.isneginf(want_lse[0, 0, 5]) and np.isneginf(want_lse[0, 0, 6]) and np.isfinite(want_lse[0, 1, 8])
+        assert np.isfinite(want_lse[0, 0, 7]) == (Bc == 64)
+        assert np.isneginf(want_lse[0, 1, 9]) == (Bc == 32)
+        got_o, got_lse = _run(ops, q, k, v, bias, Bc=Bc)
+        _check(got_o, got_lse, want_o, want_lse)
+
+
+def test_closed_forms_at_the_configured_sizes(ops):
+    """Size-independent properties at the MSA-track shape (planes 824, L 256, d 32), where the oracle
+    would take minutes: equal scores give the mean of V; V = 1 gives rows of 1; a per-row shift of the
+    bias moves LSE by the shift and leaves O alone."""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    B, h, L, d = 103, 8, 256, 32
+    k = torch.randn(B, h, L, d, device="cuda", generator=g)
+    v = torch.randn(B, h, L, d, device="cuda", generator=g)
+    o, lse = ops.flash_attn_forward(torch.zeros_like(k), k, v, eps=0.0)
+    mean = v.mean(dim=2, keepdim=True)
+    assert float((o - mean).abs().max()) <= 1e-5
+    assert float((lse - float(np.log(L))).abs().max()) <= 1e-5
+    q = torch.randn(B, h, L, d, device="cuda", generator=g)
+    o1, lse1 = ops.flash_attn_forward(q, k, torch.ones_like(v), eps=0.0)
+    assert float((o1 - 1).abs().max()) <= 1e-5
+    Bs, hs = 8, 8
+    bias = torch.randn(Bs, hs, L, L, device="cuda", generator=g)
+    shift = torch.randn(Bs, hs, L, 1, device="cuda", generator=g)
+    qa, ka, va = q[:Bs].contiguous(), k[:Bs].contiguous(), v[:Bs].contiguous()
+    oa, la = ops.flash_attn_forward(qa, ka, va, bias)
+    ob, lb = ops.flash_attn_forward(qa, ka, va, bias + shift)
+    assert float((oa - ob).abs().max()) <= 2e-5
+    assert float((lb - la - shift[..., 0]).abs().max()) <= 2e-5
+    # against torch's own softmax attention in float64 on a few planes
+    s = torch.einsum("bhid,bhjd->bhij", qa.double(), ka.double()) / np.sqrt(d) + bias.double()
+    want = torch.einsum("bhij,bhjd->bhid", torch.softmax(s, dim=-1), va.double())
+    assert float((oa.double() - want).abs().max()) <= RTOL * float(want.abs().max())
+
+
+def test_refused_arguments(ops):
+    from proteinpredictmachinelearning_amd import cabi
+
+    lib = cabi.load()
+    x = torch.zeros(4 * 72, device="cuda")
+    p = x.data_ptr()
+    args = lambda d, ptr=p: (1, 1, 4, d, 0, 0.0, 1e-9, 64, ptr, p, p, None, p, None, None)  # noqa: E731
+    assert lib.flash_attn_forward_hip(*args(72)) == 1          # d > 64 (src/backend/CUDABackend.cpp:457-463)
+    assert lib.flash_attn_forward_hip(*args(6)) == 1           # d % 4 != 0
+    assert lib.flash_attn_forward_hip(*args(8, p + 4)) == 1    # misaligned
+    assert lib.flash_attn_forward_hip(1, 1, 0, 8, 0, 0.0, 1e-9, 64, p, p, p, None, p, None, None) == 1
+    assert lib.flash_attn_forward_hip(1, 1, 4, 8, 0, 0.0, 1e-9, 64, None, p, p, None, p, None, None) == 1
+    assert b"flash_attn_forward_hip" in lib.ppml_hip_last_error()
