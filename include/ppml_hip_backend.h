@@ -36,7 +36,9 @@ void ppml_hip_tensor_destroy(ppml_hip_tensor *t);
 void ppml_hip_tensor_set_src(ppml_hip_tensor *t, int slot, ppml_hip_tensor *src);
 void ppml_hip_tensor_set_data(ppml_hip_tensor *t, void *device_ptr);
 void ppml_hip_tensor_set_view(ppml_hip_tensor *t, ppml_hip_tensor *view_src, size_t byte_offset);
+/* op_params as in the reference's node (include/ppml/Tensor.h:449-450): 32-bit integers, floats stored by bit pattern */
 void ppml_hip_tensor_set_param(ppml_hip_tensor *t, int index, float value);
+void ppml_hip_tensor_set_param_i32(ppml_hip_tensor *t, int index, int value);
 size_t ppml_hip_tensor_nbytes(const ppml_hip_tensor *t);
 int ppml_hip_tensor_type(const ppml_hip_tensor *t);
 /* allocate device storage through the backend's BufferType and copy host data in / out */

@@ -11,6 +11,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <cstring>
 #include <memory>
 #include <string>
 #include <vector>
@@ -34,6 +35,7 @@ enum TensorOp : int {
     OP_SCALE = 33,
     OP_RESHAPE = 37,
     OP_VIEW = 38,
+    OP_FLASH_ATTN_EXT = 75,
     OP_OUTER_PROD_MEAN = 102,
 };
 
@@ -60,7 +62,10 @@ struct Tensor {
     size_t buffer_offs = 0;
     Tensor* view_src = nullptr;           // OP_VIEW / OP_RESHAPE share their source's storage
     size_t view_offs = 0;
-    float op_params[16] = {0};
+    int32_t op_params[16] = {0};          // as in the reference: integers, or the bit pattern of a float
+
+    float param_f32(int i) const { float f; std::memcpy(&f, &op_params[i], sizeof f); return f; }
+    void set_param_f32(int i, float f) { std::memcpy(&op_params[i], &f, sizeof f); }
 
     int64_t numel() const { return dims[0] * dims[1] * dims[2] * dims[3]; }
     // include/ppml/Tensor.h:327-352
@@ -103,8 +108,8 @@ private:
 
 using ComputeGraph = std::vector<Tensor*>;   // nodes in evaluation order
 
-// src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-416 (OP_OUTER_PROD_MEAN);
-// a function of the node alone, so it can be asked without a device
+// src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-416 (OP_OUTER_PROD_MEAN),
+// 457-463 (OP_FLASH_ATTN_EXT); a function of the node alone, so it can be asked without a device
 bool node_supported(const Tensor* node);
 
 // include/ppml/Backend.h:550-605; executor obligations of src/backend/CUDABackend.cpp:708-1086
@@ -137,6 +142,7 @@ private:
     Status kernel_mul_mat(Tensor* node);
     Status kernel_out_prod(Tensor* node);
     Status kernel_outer_prod_mean(Tensor* node);
+    Status kernel_flash_attn_ext(Tensor* node);
     bool resolve_views(Tensor* node);                    // src/backend/CUDABackend.cpp:800-819
     bool device_pointer_ok(const Tensor* t) const;       // src/backend/CUDABackend.cpp:894-973
     Status fail(Status s, const std::string& why);

@@ -17,7 +17,8 @@ from . import cabi
 # tensor_type
 F32, F16, Q8_0, Q8_1, Q8_0R, Q8_0M = 0, 1, 8, 9, 19, 64
 # tensor_op
-OP_NONE, OP_MUL_MAT, OP_OUT_PROD, OP_SCALE, OP_RESHAPE, OP_VIEW, OP_SOFT_MAX, OP_OUTER_PROD_MEAN = 0, 30, 32, 33, 37, 38, 47, 102
+OP_NONE, OP_MUL_MAT, OP_OUT_PROD, OP_SCALE, OP_RESHAPE, OP_VIEW, OP_SOFT_MAX, OP_FLASH_ATTN_EXT, OP_OUTER_PROD_MEAN = \
+    0, 30, 32, 33, 37, 38, 47, 75, 102
 # Status
 SUCCESS, ALLOC_FAILED, NOT_SUPPORTED, ABORTED = 0, 1, 2, 3
 
@@ -52,6 +53,14 @@ class Tensor:
 
     def bind(self, device_ptr: int) -> "Tensor":
         self._lib.ppml_hip_tensor_set_data(self.handle, C.c_void_p(device_ptr))
+        return self
+
+    def set_param(self, index: int, value) -> "Tensor":
+        """op_params[index]: a Python float is stored by its binary32 bit pattern, an int as it is."""
+        if isinstance(value, float):
+            self._lib.ppml_hip_tensor_set_param(self.handle, index, value)
+        else:
+            self._lib.ppml_hip_tensor_set_param_i32(self.handle, index, int(value))
         return self
 
     def view_of(self, base: "Tensor", byte_offset: int = 0) -> "Tensor":

@@ -52,6 +52,7 @@ BACKEND_SIGNATURES = {
     "ppml_hip_tensor_set_data": (None, [_vp, _vp]),
     "ppml_hip_tensor_set_view": (None, [_vp, _vp, C.c_size_t]),
     "ppml_hip_tensor_set_param": (None, [_vp, _i, _f]),
+    "ppml_hip_tensor_set_param_i32": (None, [_vp, _i, _i]),
     "ppml_hip_tensor_nbytes": (C.c_size_t, [_vp]),
     "ppml_hip_tensor_type": (_i, [_vp]),
     "ppml_hip_tensor_upload": (_i, [_vp, _vp, _vp, C.c_size_t]),

@@ -150,6 +150,14 @@ bool node_supported(const Tensor* node) {
         case OP_OUT_PROD:
             return src0 && src1 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
                    node->type == TENSOR_TYPE_F32;
+        case OP_FLASH_ATTN_EXT: {
+            // src/backend/CUDABackend.cpp:457-463: f32, head dimension (dims[0] of the [d,L,h,B] layout)
+            // a multiple of 4 and at most 64
+            if (!src0 || !src1 || !node->src[2]) return false;
+            if (src0->type != TENSOR_TYPE_F32) return false;
+            const int64_t d = src0->dims[0];
+            return d > 0 && d <= 64 && (d % 4) == 0;
+        }
         case OP_OUTER_PROD_MEAN:
             if (!src0 || !src1) return false;
             if (src0->type != TENSOR_TYPE_F32 || src1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32) return false;
@@ -280,11 +288,39 @@ Status HipBackend::kernel_outer_prod_mean(Tensor* node) {
     return Status::SUCCESS;
 }
 
+// src/backend/CUDAKernels.cpp:894-903 with the configuration of CPUKernels.cpp:1384-1398:
+// src 0..2 = Q, K, V in the [d, L, h, B] layout, src 3 = bias or null, src 4 = LSE output or null;
+// op_params: 0 scale (f32), 1 causal, 2 softmax eps (f32), 3 Br, 4 Bc.
+Status HipBackend::kernel_flash_attn_ext(Tensor* node) {
+    const Tensor* q = node->src[0];
+    const Tensor* k = node->src[1];
+    const Tensor* v = node->src[2];
+    if (!q || !k || !v || !q->data || !k->data || !v->data || !node->data)
+        return fail(Status::NOT_SUPPORTED, "flash_attn_ext: unbound tensor");
+    const int64_t d = q->dims[0], L = q->dims[1], h = dim_or_1(q, 2), B = dim_or_1(q, 3);
+    if (k->numel() != q->numel() || v->numel() != q->numel() || node->numel() != q->numel())
+        return fail(Status::NOT_SUPPORTED, "flash_attn_ext: Q, K, V and O differ in size");
+    const Tensor* bias = node->src[3];
+    if (bias && (!bias->data || bias->numel() != B * h * L * L))
+        return fail(Status::NOT_SUPPORTED, "flash_attn_ext: bias is not [L, L, h, B]");
+    Tensor* lse = node->src[4];
+    if (lse && lse->numel() != B * h * L) return fail(Status::NOT_SUPPORTED, "flash_attn_ext: LSE is not [L, h, B]");
+    if (lse && !lse->data) return fail(Status::NOT_SUPPORTED, "flash_attn_ext: LSE buffer is unbound");
+    const int rc = flash_attn_forward_hip(static_cast<int>(B), static_cast<int>(h), static_cast<int>(L), static_cast<int>(d),
+                                          node->op_params[1] != 0, node->param_f32(0), node->param_f32(2), node->op_params[4],
+                                          static_cast<const float*>(q->data), static_cast<const float*>(k->data),
+                                          static_cast<const float*>(v->data), bias ? static_cast<const float*>(bias->data) : nullptr,
+                                          static_cast<float*>(node->data), lse ? static_cast<float*>(lse->data) : nullptr, nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("flash_attn_ext: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
 Status HipBackend::dispatch_node(Tensor* node) {
     switch (node->op) {
         case OP_MUL_MAT: return kernel_mul_mat(node);
         case OP_OUT_PROD: return kernel_out_prod(node);
         case OP_OUTER_PROD_MEAN: return kernel_outer_prod_mean(node);
+        case OP_FLASH_ATTN_EXT: return kernel_flash_attn_ext(node);
         default: return fail(Status::NOT_SUPPORTED, "no kernel for op " + std::to_string(node->op));
     }
 }
@@ -303,14 +339,17 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         if (node->op == OP_NONE || node->op == OP_VIEW || node->op == OP_RESHAPE) continue;
         resolve_views(node);
 
-        // single-backend mode: outputs nobody allocated get their own device buffer
-        if (!skip_alloc_ && !node->data) {
-            const size_t need = node->nbytes();
+        // single-backend mode: outputs nobody allocated get their own device buffer -- the node itself
+        // and the second output the fused attention node carries in src[4] (its LSE buffer)
+        Tensor* outputs[2] = {node, node->op == OP_FLASH_ATTN_EXT ? node->src[4] : nullptr};
+        for (Tensor* out : outputs) {
+            if (!out || skip_alloc_ || out->data) continue;
+            const size_t need = out->nbytes();
             auto buf = std::make_unique<Buffer>(buffer_type(), need);
             if (!buf->data()) return fail(Status::ALLOC_FAILED, "cannot allocate " + std::to_string(need) + " bytes for node " + std::to_string(index));
-            node->data = buf->data();
-            node->buffer = buf.get();
-            node->buffer_offs = 0;
+            out->data = buf->data();
+            out->buffer = buf.get();
+            out->buffer_offs = 0;
             owned_.push_back(std::move(buf));
         }
         // no other backend to fall back to: an unsupported node ends the graph instead of being skipped
@@ -417,6 +456,9 @@ void ppml_hip_tensor_set_view(ppml_hip_tensor* t, ppml_hip_tensor* view_src, siz
     t->t.view_offs = byte_offset;
 }
 void ppml_hip_tensor_set_param(ppml_hip_tensor* t, int index, float value) {
+    if (t && index >= 0 && index < 16) t->t.set_param_f32(index, value);
+}
+void ppml_hip_tensor_set_param_i32(ppml_hip_tensor* t, int index, int value) {
     if (t && index >= 0 && index < 16) t->t.op_params[index] = value;
 }
 size_t ppml_hip_tensor_nbytes(const ppml_hip_tensor* t) { return t ? t->t.nbytes() : 0; }

@@ -60,6 +60,20 @@ def test_supports_op_other_ops():
     assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_SOFT_MAX, [a]))
 
 
+def test_supports_op_fused_attention():
+    # src/backend/CUDABackend.cpp:457-463: Q, K, V present, f32, head dimension (dims[0]) a multiple of 4 up to 64
+    def node(d, type=B.F32, n_src=3):
+        qkv = [B.Tensor((d, 10, 2, 1), type) for _ in range(n_src)]
+        return B.Tensor((d, 10, 2, 1), B.F32, B.OP_FLASH_ATTN_EXT, qkv), qkv
+    for d, want in [(4, True), (32, True), (64, True), (68, False), (6, False), (128, False)]:
+        n, keep = node(d)
+        assert B.supports_op(n) == want, d
+    n, keep = node(32, B.F16)
+    assert not B.supports_op(n)
+    n, keep = node(32, B.F32, n_src=2)
+    assert not B.supports_op(n)
+
+
 def test_tensor_nbytes_follows_the_block_records():
     # include/ppml/Tensor.h:327-352: quantized bytes = blocks * record size; invalid shapes have none
     assert B.Tensor((256, 768), B.F32).nbytes == 256 * 768 * 4

@@ -133,6 +133,33 @@ def test_out_prod_and_outer_prod_mean_nodes(be, oracle):
     assert (be.download(opm) == oracle.outer_prod_mean(l, r, D, L, N, Bt)).all()
 
 
+def test_fused_attention_node(be, oracle):
+    # the node ComputeGraphHelper.cpp:450-484 builds: src 0..2 = Q, K, V as [d, L, h, B], src 3 = bias,
+    # src 4 = LSE output; op_params 0 scale, 1 causal, 2 softmax eps, 3 Br, 4 Bc
+    rng = np.random.default_rng(8)
+    Bt, h, L, d = 2, 3, 77, 32
+    q, k, v = [rng.standard_normal((Bt, h, L, d)).astype(np.float32) for _ in range(3)]
+    bias = rng.standard_normal((Bt, h, L, L)).astype(np.float32)
+    scale = 1.0 / np.sqrt(8.0)                  # the caller's head_dim, not d (Attention.cpp:254-262)
+    for with_bias, causal, with_lse in [(True, False, True), (False, True, False)]:
+        qt, kt, vt = _leaf(be, q), _leaf(be, k), _leaf(be, v)
+        bt = _leaf(be, bias) if with_bias else None
+        lse = B.Tensor((L, h, Bt)) if with_lse else None        # unbound: the executor allocates it
+        node = B.Tensor((d, L, h, Bt), B.F32, B.OP_FLASH_ATTN_EXT, [qt, kt, vt, bt, lse])
+        node.set_param(0, float(scale)).set_param(1, int(causal)).set_param(2, 1e-9).set_param(3, 64).set_param(4, 64)
+        assert be.supports_op(node)
+        assert be.graph_compute([node]) == B.SUCCESS, be.last_error
+        be.synchronize()
+        want_o, want_lse = oracle.flash_attn_forward(q, k, v, bias if with_bias else None, causal=causal, scale=scale)
+        got = be.download(node).reshape(Bt, h, L, d)
+        assert np.abs(got - want_o).max() <= 1e-4 * np.abs(want_o).max()
+        if with_lse:
+            assert np.abs(be.download(lse).reshape(Bt, h, L) - want_lse).max() <= 1e-5 * (1 + np.abs(want_lse).max())
+    # a head dimension the kernel does not take is refused before anything runs
+    bad = B.Tensor((68, 8, 1, 1), B.F32, B.OP_FLASH_ATTN_EXT, [_leaf(be, np.zeros((1, 1, 8, 68), np.float32)) for _ in range(3)])
+    assert be.graph_compute([bad]) == B.NOT_SUPPORTED
+
+
 def test_view_sources_are_resolved_and_noop_nodes_skipped(be, oracle):
     # a reshape node built with only src[0] set, and an offset view with view_src set, both feed a
     # mul_mat (src/backend/CUDABackend.cpp:800-819)
