@@ -182,6 +182,19 @@ def main() -> int:
         f32_case(logits(824, 256, 32), (2 * 824 * 32 * 256 + 824 * 256 * 256) * 4, 2.0 * 824 * 256 * 256 * 32,
                  "attn_logits_msa_824x256x256x32")
 
+        def attention(planes, L, D, with_bias):
+            def make():
+                nb = (4 * planes * L * D + planes * L + (planes * L * L if with_bias else 0)) * 4
+                ns = max(2, int(640e6 // nb) + 1)
+                qkv = [[torch.randn(1, planes, L, D, device=dev, generator=gen) for _ in range(3)] for _ in range(ns)]
+                bs = [torch.randn(1, planes, L, L, device=dev, generator=gen) if with_bias else None for _ in range(ns)]
+                return (lambda i: ops.flash_attn_forward(qkv[i][0], qkv[i][1], qkv[i][2], bs[i])), ns
+            return make
+        for planes, L, D, wb, tag in [(412, 103, 32, True, "pair_412x103x32_bias"), (824, 256, 32, True, "msa_824x256x32_bias"),
+                                      (824, 256, 32, False, "msa_824x256x32")]:
+            f32_case(attention(planes, L, D, wb), (4 * planes * L * D + planes * L + (planes * L * L if wb else 0)) * 4,
+                     4.0 * planes * L * L * D, "fused_attention_" + tag)
+
         def opm():
             a = torch.randn(256, 12288, device=dev, generator=gen) * 0.1
             b = torch.randn(256, 12288, device=dev, generator=gen) * 0.1

@@ -26,14 +26,17 @@
 #include "common.hpp"
 
 #include <cmath>
+#include <type_traits>
 
 namespace ppmlhip {
 namespace {
 
 typedef float v2f __attribute__((ext_vector_type(2)));
 
-template <int DP> struct AttnTiling {
-    static constexpr int CH = DP <= 32 ? 256 : 128;   // keys staged in LDS at a time
+template <int DP, int NW> struct AttnTiling {
+    // keys staged in LDS at a time: about 35 KB per four-wave work-group (four of them share a CU and its
+    // 160 KB), 69 KB per eight-wave one (two per CU)
+    static constexpr int CH = (DP <= 32 ? 256 : 128) / (NW == 4 ? 2 : 1);
     static constexpr int KS = DP + 4;                 // row pitch of K in LDS (floats): 16-byte reads, rows 4 banks apart
     static constexpr int VS = DP;                     // row pitch of V
     static constexpr size_t lds_bytes = static_cast<size_t>(CH) * (KS + VS) * sizeof(float);
@@ -47,7 +50,6 @@ struct AttnParams {
     float scale, eps;
     int head;            // keys of the reference's first block: min(Bc, keys of the row)
     int stage_rows;      // keys staged in LDS at a time: min(CH, L rounded up to 32)
-    int bias_vec;        // bias rows can be read 16 bytes at a time (L % 4 == 0 and an aligned base)
 };
 
 __device__ __forceinline__ float lane_xor32(float x) {
@@ -55,9 +57,12 @@ __device__ __forceinline__ float lane_xor32(float x) {
     return __shfl_xor(x, 32, 64);
 }
 
-template <int DP, int NW>
+// PF: request each tile's bias one tile ahead.  It costs 16 registers, i.e. the fourth wave per SIMD, so only
+// the instance for short sequences uses it: there a work-group is a chain of memory latencies and the
+// machine is far from full anyway.
+template <int DP, int NW, bool PF>
 __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnParams p) {
-    using T = AttnTiling<DP>;
+    using T = AttnTiling<DP, NW>;
     constexpr int KS = T::KS, VS = T::VS;
     constexpr int NB = DP / 32;                       // 32-row blocks of the transposed output
     extern __shared__ __attribute__((aligned(16))) float attn_lds[];
@@ -74,14 +79,16 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
     const bool wave_active = q0 < L;                  // wave-uniform
     const int64_t plane_off = static_cast<int64_t>(plane) * L * d;
 
-    // ---- this lane's slice of its query row: elements half*DP/2 + s, s = 0 .. DP/2-1 (zero past d / past L)
+    constexpr float LOG2E = 1.44269504088896340736f, LN2 = 0.69314718055994530942f;
+    const float sc2 = p.scale * LOG2E;                // scores are kept in the base-2 domain
+    // ---- this lane's slice of its query row, times scale * log2(e): elements half*DP/2 + s, s = 0 .. DP/2-1 (zero past d / past L)
     float qreg[DP / 2];
 #pragma unroll
     for (int s = 0; s < DP / 2; s += 4) {
         const int e = half * (DP / 2) + s;
         v4f x = {0.0f, 0.0f, 0.0f, 0.0f};
         if (q < L && e < d) x = *reinterpret_cast<const v4f*>(p.Q + plane_off + static_cast<int64_t>(q) * d + e);
-        qreg[s] = x[0]; qreg[s + 1] = x[1]; qreg[s + 2] = x[2]; qreg[s + 3] = x[3];
+        qreg[s] = x[0] * sc2; qreg[s + 1] = x[1] * sc2; qreg[s + 2] = x[2] * sc2; qreg[s + 3] = x[3] * sc2;
     }
 
     v16f acc_o[NB];
@@ -95,8 +102,98 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
     const int head_keys = p.head < row_keys ? p.head : row_keys;
     // keys any query of this wave may see (wave-uniform)
     const int wave_keys = p.causal ? (q0 + 32 < L ? q0 + 32 : L) : L;
-    const float* bias_row = p.bias ? p.bias + (static_cast<int64_t>(plane) * L + (q < L ? q : 0)) * L : nullptr;
-    const bool bias_vec = p.bias_vec != 0;
+    // lanes past the last query read the last row (never stored)
+    const float* bias_row = p.bias ? p.bias + (static_cast<int64_t>(plane) * L + (q < L ? q : L - 1)) * L : nullptr;
+
+    // Bias of this lane's 16 keys of the tile starting at key0 (zeros past L), into bias_buf.  Rows of a
+    // length that is no multiple of 4 are read with 16-byte loads all the same (4-byte aligned).
+    float bias_buf[16];
+    auto load_bias = [&](int key0) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int key = key0 + 8 * g + 4 * half;
+            if (key + 3 < L) {
+                const v4f x = *reinterpret_cast<const v4f_u*>(bias_row + key);
+                bias_buf[4 * g] = x[0]; bias_buf[4 * g + 1] = x[1]; bias_buf[4 * g + 2] = x[2]; bias_buf[4 * g + 3] = x[3];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) bias_buf[4 * g + i] = key + i < L ? bias_row[key + i] : 0.0f;
+            }
+        }
+    };
+    if (PF && bias_row && wave_active) load_bias(0);
+
+    // One tile of 32 keys for the wave's 32 queries.  Scores live in the base-2 domain (the query slice
+    // carries scale * log2(e)), so a probability is one subtraction and one v_exp_f32.
+    auto do_tile = [&](auto plain_t, int kt, int key0) {
+        constexpr bool PLAIN = decltype(plain_t)::value;
+        // ---- bias of this lane's 16 keys, requested before the matrix work (or a tile ago)
+        float bv[16];
+        const bool has_bias = bias_row != nullptr;     // wave-uniform
+        if (has_bias) {
+            if (!PF) load_bias(key0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) bv[r] = bias_buf[r];
+            if (PF && key0 + 32 < wave_keys) load_bias(key0 + 32);
+        }
+        // ---- S^T = K_tile . Q^T
+        v16f st;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[r] = 0.0f;
+        const float* krow = lds_k + (kt * 32 + j) * KS + half * (DP / 2);
+#pragma unroll
+        for (int s = 0; s < DP / 2; s += 4) {
+            const v4f kx = *reinterpret_cast<const v4f*>(krow + s);
+            st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[0], qreg[s], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[1], qreg[s + 1], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[2], qreg[s + 2], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[3], qreg[s + 3], st, 0, 0, 0);
+        }
+        // ---- scores of this lane's query: bias, masks; tile maximum
+        float m_tile = -INFINITY;
+        if (has_bias) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) st[r] = __builtin_fmaf(bv[r], LOG2E, st[r]);
+        }
+        if (!PLAIN) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = key0 + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (key >= row_keys) st[r] = -INFINITY;
+                if (key < head_keys) m_head = fmaxf(m_head, st[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) m_tile = fmaxf(m_tile, st[r]);
+        m_tile = fmaxf(m_tile, lane_xor32(m_tile));
+        const float m_new = fmaxf(m_run, m_tile);
+        const float alpha = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+        const float m_sub = (m_new == -INFINITY) ? 0.0f : m_new;       // keeps -inf - -inf out of the exponent
+        float l_tile = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            st[r] = __builtin_amdgcn_exp2f(st[r] - m_sub);
+            l_tile += st[r];
+        }
+        l_tile += lane_xor32(l_tile);
+        l_run = alpha * l_run + l_tile;
+        m_run = m_new;
+        // ---- O^T = alpha * O^T + V^T . P   (the rescale is skipped while no maximum of the wave moves)
+        const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;
+        const float* vbase = lds_v + (kt * 32 + 4 * half) * VS + j;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            if (rescale) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc_o[b][r] *= alpha;
+            }
+#pragma unroll
+            for (int kk = 0; kk < 16; ++kk) {
+                const float vx = vbase[(8 * (kk >> 2) + (kk & 3)) * VS + b * 32];
+                acc_o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx, st[kk], acc_o[b], 0, 0, 0);
+            }
+        }
+    };
 
     const int stage = p.stage_rows;
     for (int c0 = 0; c0 < L; c0 += stage) {
@@ -122,73 +219,11 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
         for (int kt = 0; kt < tiles_here; ++kt) {
             const int key0 = c0 + kt * 32;             // first key of the tile
             if (key0 >= wave_keys) break;              // causal: nothing left for any query of the wave
-            // ---- bias of this lane's 16 keys, requested before the matrix work
-            float bv[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) bv[r] = 0.0f;
-            if (bias_row && q < L) {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int key = key0 + 8 * g + 4 * half;
-                    if (bias_vec && key + 3 < L) {
-                        const v4f x = *reinterpret_cast<const v4f*>(bias_row + key);
-                        bv[4 * g] = x[0]; bv[4 * g + 1] = x[1]; bv[4 * g + 2] = x[2]; bv[4 * g + 3] = x[3];
-                    } else {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) if (key + i < L) bv[4 * g + i] = bias_row[key + i];
-                    }
-                }
-            }
-            // ---- S^T = K_tile . Q^T
-            v16f st;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) st[r] = 0.0f;
-            const float* krow = lds_k + (kt * 32 + j) * KS + half * (DP / 2);
-#pragma unroll
-            for (int s = 0; s < DP / 2; s += 4) {
-                const v4f kx = *reinterpret_cast<const v4f*>(krow + s);
-                st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[0], qreg[s], st, 0, 0, 0);
-                st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[1], qreg[s + 1], st, 0, 0, 0);
-                st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[2], qreg[s + 2], st, 0, 0, 0);
-                st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[3], qreg[s + 3], st, 0, 0, 0);
-            }
-            // ---- scores of this lane's query: scale, bias, masks; tile maximum
-            float m_tile = -INFINITY;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int key = key0 + 8 * (r >> 2) + 4 * half + (r & 3);
-                float s = st[r] * p.scale;
-                s = s + bv[r];
-                if (key >= row_keys) s = -INFINITY;
-                st[r] = s;
-                m_tile = fmaxf(m_tile, s);
-                if (key < head_keys) m_head = fmaxf(m_head, s);
-            }
-            m_tile = fmaxf(m_tile, lane_xor32(m_tile));
-            const float m_new = fmaxf(m_run, m_tile);
-            const float alpha = (m_run == -INFINITY) ? 0.0f : __expf(m_run - m_new);
-            float l_tile = 0.0f;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float pr = (m_new == -INFINITY) ? 0.0f : __expf(st[r] - m_new);
-                st[r] = pr;
-                l_tile += pr;
-            }
-            l_tile += lane_xor32(l_tile);
-            l_run = alpha * l_run + l_tile;
-            m_run = m_new;
-            // ---- O^T = alpha * O^T + V^T . P
-            const float* vbase = lds_v + (kt * 32 + 4 * half) * VS + j;
-#pragma unroll
-            for (int b = 0; b < NB; ++b) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc_o[b][r] *= alpha;
-#pragma unroll
-                for (int kk = 0; kk < 16; ++kk) {
-                    const float vx = vbase[(8 * (kk >> 2) + (kk & 3)) * VS + b * 32];
-                    acc_o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx, st[kk], acc_o[b], 0, 0, 0);
-                }
-            }
+            // A tile is plain when every query of the wave sees all 32 keys and the tile lies behind the
+            // reference's first block; plain tiles skip the masks and the first-block bookkeeping.
+            const bool plain = key0 + 32 <= L && (!p.causal || key0 + 32 <= q0 + 1) && key0 >= p.head;
+            if (plain) do_tile(std::true_type{}, kt, key0);
+            else do_tile(std::false_type{}, kt, key0);
         }
     }
     if (!wave_active || q >= L) return;
@@ -210,13 +245,13 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
                 *reinterpret_cast<v4f*>(orow + dd) = live ? o : v4f{0.0f, 0.0f, 0.0f, 0.0f};
             }
         }
-    if (p.LSE && half == 0) p.LSE[static_cast<int64_t>(plane) * L + q] = live ? m_run + __logf(l_run + p.eps) : -INFINITY;
+    if (p.LSE && half == 0) p.LSE[static_cast<int64_t>(plane) * L + q] = live ? m_run * LN2 + __logf(l_run + p.eps) : -INFINITY;
 }
 
-template <int DP, int NW>
+template <int DP, int NW, bool PF>
 int launch_flash(AttnParams p, hipStream_t stream) {
-    using T = AttnTiling<DP>;
-    auto kernel = &flash_attn_forward_kernel<DP, NW>;
+    using T = AttnTiling<DP, NW>;
+    auto kernel = &flash_attn_forward_kernel<DP, NW, PF>;
     const int l32 = (p.L + 31) / 32 * 32;
     p.stage_rows = l32 < T::CH ? l32 : T::CH;
     const size_t lds = static_cast<size_t>(p.stage_rows) * (T::KS + T::VS) * sizeof(float);
@@ -265,11 +300,12 @@ extern "C" int flash_attn_forward_hip(int B, int h, int L, int d, int causal, fl
     p.scale = scale > 0.0f ? scale : 1.0f / std::sqrt(static_cast<float>(d));   // FlashAttn.cpp:63
     p.eps = softmax_eps;
     p.head = Bc > 0 ? Bc : 64;                        // FlashAttn.cpp:62
-    p.bias_vec = (bias && (L & 3) == 0 && !misaligned(bias)) ? 1 : 0;
     p.stage_rows = 0;                                 // set per instance
     stats_record(static_cast<int64_t>(planes) * L, d, L);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool few_queries = L <= 128;                // four waves cover the plane
-    if (d <= 32) return few_queries ? launch_flash<32, 4>(p, s) : launch_flash<32, 8>(p, s);
-    return few_queries ? launch_flash<64, 4>(p, s) : launch_flash<64, 8>(p, s);
+    // Four-wave work-groups (128 queries): 824 planes of 256 queries make 1648 of them, which spread over
+    // 256 CUs more evenly than 824 eight-wave ones (6.4 per CU against 3.2, each rounded up).
+    const bool short_rows = L <= 128;
+    if (d <= 32) return short_rows ? launch_flash<32, 4, true>(p, s) : launch_flash<32, 4, false>(p, s);
+    return short_rows ? launch_flash<64, 4, true>(p, s) : launch_flash<64, 4, false>(p, s);
 }
