@@ -184,12 +184,26 @@ def main() -> int:
 
         def attention(planes, L, D, with_bias):
             def make():
+                import ctypes as C
                 nb = (4 * planes * L * D + planes * L + (planes * L * L if with_bias else 0)) * 4
                 ns = max(2, int(640e6 // nb) + 1)
                 qkv = [[torch.randn(1, planes, L, D, device=dev, generator=gen) for _ in range(3)] for _ in range(ns)]
                 bs = [torch.randn(1, planes, L, L, device=dev, generator=gen) if with_bias else None for _ in range(ns)]
-                return (lambda i: ops.flash_attn_forward(qkv[i][0], qkv[i][1], qkv[i][2], bs[i])), ns
+                outs = [(torch.empty(1, planes, L, D, device=dev), torch.empty(1, planes, L, device=dev)) for _ in range(ns)]
+                lib, cabi = ops._lib(), ops.cabi
+                stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+                ptr = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None      # noqa: E731
+                argsets = [(1, planes, L, D, 0, 0.0, 1e-9, 64, ptr(qkv[i][0]), ptr(qkv[i][1]), ptr(qkv[i][2]), ptr(bs[i]),
+                            ptr(outs[i][0]), ptr(outs[i][1]), stream) for i in range(ns)]
+
+                def fn(i):
+                    rc = lib.flash_attn_forward_hip(*argsets[i])
+                    if rc:
+                        cabi.check("flash_attn_forward_hip", rc)
+                keep.append((qkv, bs, outs))
+                return fn, ns
             return make
+        keep = []
         for planes, L, D, wb, tag in [(412, 103, 32, True, "pair_412x103x32_bias"), (824, 256, 32, True, "msa_824x256x32_bias"),
                                       (824, 256, 32, False, "msa_824x256x32")]:
             f32_case(attention(planes, L, D, wb), (4 * planes * L * D + planes * L + (planes * L * L if wb else 0)) * 4,
