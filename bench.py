@@ -209,6 +209,25 @@ def main() -> int:
             f32_case(attention(planes, L, D, wb), (4 * planes * L * D + planes * L + (planes * L * L if wb else 0)) * 4,
                      4.0 * planes * L * L * D, "fused_attention_" + tag)
 
+        def bridge():
+            # the [L, D, h, B] -> [D, L, h, B] copy in front of the fused attention node, MSA-track size
+            import ctypes as C
+            ns = 12
+            xs = [torch.randn(824, 32, 256, device=dev, generator=gen) for _ in range(ns)]
+            ys = [torch.empty(824, 256, 32, device=dev) for _ in range(ns)]
+            lib, cabi = ops._lib(), ops.cabi
+            stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            argsets = [(C.c_void_p(xs[i].data_ptr()), C.c_void_p(ys[i].data_ptr()), 824 * 32 * 256, 3, 1, 0, 2, 3,
+                        256, 32, 824, 1, 32, 256, 824, 1, stream) for i in range(ns)]
+
+            def fn(i):
+                rc = lib.permute_hip(*argsets[i])
+                if rc:
+                    cabi.check("permute_hip", rc)
+            keep.append((xs, ys))
+            return fn, ns
+        f32_case(bridge, 2 * 824 * 32 * 256 * 4, 0.0, "permute_attention_bridge_824x256x32")
+
         def opm():
             a = torch.randn(256, 12288, device=dev, generator=gen) * 0.1
             b = torch.randn(256, 12288, device=dev, generator=gen) * 0.1

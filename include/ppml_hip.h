@@ -155,6 +155,20 @@ int flash_attn_forward_hip(int B, int h, int L, int d, int causal, float scale, 
                            const float *Q, const float *K, const float *V, const float *bias,
                            float *O, float *LSE, ppml_hip_stream_t stream);
 
+/* ---- dimension permutation (a real copy) ------------------------------------------------------ */
+/* replaces permute_cuda and transpose_cuda (declared src/backend/CUDAKernels.cpp:137-143, called from
+ * kernel_permute_cuda / kernel_transpose_cuda, 1344-1390); semantics of CPUBackend::kernel_permute
+ * (src/backend/CPUKernels.cpp:1669-1717): dimension p of dst is dimension d_p of src, both dense with
+ * dimension 0 innermost.  s0..s3 are the source sizes, dd0..dd3 the destination sizes, total their
+ * product; entries past ndim are ignored.  This is what mat_transpose(), the operand shuffles of the
+ * backward GEMMs and the layout bridges around the fused attention node are made of.
+ * returns 0 ok, 1 bad arguments (axes that are no permutation -- the reference refuses those too,
+ * CUDAKernels.cpp:1376-1381 -- or sizes that do not match them), 6 launch error. */
+int permute_hip(const float *src, float *dst, int64_t total, int ndim,
+                int32_t d0, int32_t d1, int32_t d2, int32_t d3,
+                int64_t s0, int64_t s1, int64_t s2, int64_t s3,
+                int64_t dd0, int64_t dd1, int64_t dd2, int64_t dd3, ppml_hip_stream_t stream);
+
 /* ---- observability (include/ppml/MulMatStats.h:154-169) -------------------------------------- */
 /* Per-shape call counters keyed like the reference (M<<40 | K<<20 | N); enabled by the
  * environment variable PPML_MULMAT_STATS=1.  Writes up to `cap` rows of

@@ -76,6 +76,8 @@ def _load() -> C.CDLL:
     lib.orc_attention_scores.argtypes = [f32p, f32p, f32p] + [i64] * 5 + [C.c_int]
     lib.orc_flash_attn_forward.restype = C.c_int
     lib.orc_flash_attn_forward.argtypes = ([C.c_int] * 5 + [C.c_float, C.c_float, C.c_int] + [f32p] * 6 + [C.c_int])
+    lib.orc_permute.restype = C.c_int
+    lib.orc_permute.argtypes = [f32p, f32p, C.c_int, C.POINTER(C.c_int32), C.POINTER(i64), C.POINTER(i64)]
     lib.orc_max_threads.restype = C.c_int
     return lib
 
@@ -351,3 +353,18 @@ def ref_flash_attn_forward(q, k, v, bias=None, causal=False, scale=0.0, eps=1e-9
     if rc:
         raise ValueError(f"reference refused the arguments (rc={rc})")
     return o, lse
+
+
+def permute(x, axes) -> np.ndarray:
+    """kernel_permute (CPUKernels.cpp:1669-1717).  `x` is a numpy array whose LAST axis is the reference's
+    dims[0]; `axes` is in the reference's numbering (dimension p of the result is dimension axes[p] of x)."""
+    x = _f32(x)
+    nd = x.ndim
+    sd = list(x.shape[::-1]) + [1] * (4 - nd)
+    ax = [int(a) for a in axes] + list(range(nd, 4))
+    dd = [sd[ax[p]] if 0 <= ax[p] < 4 else 1 for p in range(nd)] + [1] * (4 - nd)
+    out = np.empty(tuple(dd[:nd][::-1]), dtype=np.float32)
+    rc = lib().orc_permute(_fp(x), _fp(out), nd, (C.c_int32 * 4)(*ax), (C.c_int64 * 4)(*sd), (C.c_int64 * 4)(*dd))
+    if rc:
+        raise ValueError(f"orc_permute rc={rc}")
+    return out

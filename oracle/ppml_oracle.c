@@ -26,6 +26,8 @@
  *       einsum over the layout stated at src/backend/CPUKernels.cpp:975-981.
  *   orc_outer_product_mean_value : known answers of tests/test_outer_product_mean.cpp:10-70.
  *   orc_attention_scores: einsum special case and the 1/sqrt(D) closed form.
+ *   orc_permute : numpy.transpose with the axes translated (dst dim p = src dim axes[p], dims[0]
+ *       innermost), identity and inverse permutations, hand-checked 2 x 3 case.
  *   orc_flash_attn_forward : the reference's own src/ops/FlashAttn.cpp compiled as-is
  *       (oracle/_ref/libppml_ref_flash.so: it needs nothing but its header) -- bit-for-bit on
  *       random inputs, with and without bias, causal and not, ragged block sizes; plus float64
@@ -116,6 +118,32 @@ int orc_flash_attn_forward(int B, int h, int L, int d, int causal, float scale, 
         }
         free(acc);
         free(tile);
+    }
+    return 0;
+}
+
+/* src/backend/CPUKernels.cpp:1669-1717: for every destination element, in order, decode its
+ * coordinates (dims[0] innermost), place coordinate p at source dimension axes[p], read that element. */
+int orc_permute(const float *src, float *dst, int ndim, const int32_t axes[4], const int64_t sd_in[4], const int64_t dd_in[4]) {
+    int dims[4] = {0, 1, 2, 3};
+    int64_t sd[4] = {1, 1, 1, 1}, dd[4] = {1, 1, 1, 1};
+    for (int i = 0; i < ndim && i < 4; ++i) {
+        dims[i] = axes[i];
+        if (dims[i] < 0 || dims[i] >= ndim) return 1;
+        sd[i] = sd_in[i];
+        dd[i] = dd_in[i];
+    }
+    const int64_t total = dd[0] * dd[1] * dd[2] * dd[3];
+    for (int64_t idx = 0; idx < total; ++idx) {
+        int64_t t = idx;
+        int64_t jv[4];
+        jv[0] = t % dd[0]; t /= dd[0];
+        jv[1] = t % dd[1]; t /= dd[1];
+        jv[2] = t % dd[2]; t /= dd[2];
+        jv[3] = t;
+        int64_t i[4] = {0, 0, 0, 0};
+        for (int p = 0; p < ndim && p < 4; ++p) i[dims[p]] = jv[p];
+        dst[idx] = src[((i[3] * sd[2] + i[2]) * sd[1] + i[1]) * sd[0] + i[0]];
     }
     return 0;
 }

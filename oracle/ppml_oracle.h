@@ -92,6 +92,11 @@ int orc_flash_attn_forward(int B, int h, int L, int d, int causal, float scale, 
                            const float *Q, const float *K, const float *V, const float *bias,
                            float *O, float *LSE, int nthreads);
 
+/* src/backend/CPUKernels.cpp:1669-1717 (kernel_permute): dimension p of dst is dimension axes[p] of src;
+ * sd = source sizes, dd = destination sizes (dims[0] innermost), entries past ndim ignored.
+ * returns 0 ok, 1 when an axis is outside [0, ndim) -- the reference prints and leaves dst untouched. */
+int orc_permute(const float *src, float *dst, int ndim, const int32_t axes[4], const int64_t sd[4], const int64_t dd[4]);
+
 int orc_max_threads(void);
 
 #ifdef __cplusplus

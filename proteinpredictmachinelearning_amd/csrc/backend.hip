@@ -150,6 +150,10 @@ bool node_supported(const Tensor* node) {
         case OP_OUT_PROD:
             return src0 && src1 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
                    node->type == TENSOR_TYPE_F32;
+        case OP_PERMUTE:
+        case OP_TRANSPOSE:
+            // src/backend/CUDABackend.cpp:113-119
+            return src0 && src0->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32;
         case OP_FLASH_ATTN_EXT: {
             // src/backend/CUDABackend.cpp:457-463: f32, head dimension (dims[0] of the [d,L,h,B] layout)
             // a multiple of 4 and at most 64
@@ -315,12 +319,36 @@ Status HipBackend::kernel_flash_attn_ext(Tensor* node) {
     return Status::SUCCESS;
 }
 
+// src/backend/CUDAKernels.cpp:1344-1390: OP_PERMUTE and OP_TRANSPOSE both carry the axis map in
+// op_params[0..ndim) (dimension p of the node is dimension op_params[p] of src[0]); a map with an entry
+// outside the tensor's dimensions is refused.
+Status HipBackend::kernel_permute(Tensor* node) {
+    const Tensor* a = node->src[0];
+    if (!a || !a->data || !node->data) return fail(Status::NOT_SUPPORTED, "permute: unbound tensor");
+    const int ndim = a->ndim;
+    if (ndim < 1 || ndim > 4 || node->numel() != a->numel()) return fail(Status::NOT_SUPPORTED, "permute: sizes differ");
+    int32_t ax[4] = {0, 1, 2, 3};
+    int64_t sd[4] = {1, 1, 1, 1}, dd[4] = {1, 1, 1, 1};
+    for (int i = 0; i < ndim; ++i) {
+        ax[i] = node->op_params[i];
+        if (ax[i] < 0 || ax[i] >= ndim) return fail(Status::NOT_SUPPORTED, "permute: axis map outside the tensor's dimensions");
+        sd[i] = a->dims[i];
+        dd[i] = node->dims[i];
+    }
+    const int rc = permute_hip(static_cast<const float*>(a->data), static_cast<float*>(node->data), node->numel(), ndim,
+                               ax[0], ax[1], ax[2], ax[3], sd[0], sd[1], sd[2], sd[3], dd[0], dd[1], dd[2], dd[3], nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("permute: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
 Status HipBackend::dispatch_node(Tensor* node) {
     switch (node->op) {
         case OP_MUL_MAT: return kernel_mul_mat(node);
         case OP_OUT_PROD: return kernel_out_prod(node);
         case OP_OUTER_PROD_MEAN: return kernel_outer_prod_mean(node);
         case OP_FLASH_ATTN_EXT: return kernel_flash_attn_ext(node);
+        case OP_PERMUTE:
+        case OP_TRANSPOSE: return kernel_permute(node);
         default: return fail(Status::NOT_SUPPORTED, "no kernel for op " + std::to_string(node->op));
     }
 }

@@ -181,6 +181,23 @@ def flash_attn_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bias: 
     return o, lse
 
 
+def permute(x: torch.Tensor, axes) -> torch.Tensor:
+    """The reference's permute as a copy (src/backend/CPUKernels.cpp:1669-1717).  `x` is a dense tensor whose
+    LAST torch dimension is the reference's dims[0]; `axes` is in the reference's numbering: dimension p of
+    the result (dims[p]) is dimension axes[p] of the source."""
+    x = _dev_f32(x, "x")
+    nd = x.dim()
+    axes = [int(a) for a in axes]
+    if nd < 1 or nd > 4 or sorted(axes) != list(range(nd)):
+        raise ValueError("permute: axes must be a permutation of the tensor's dimensions (at most 4)")
+    sd = list(x.shape[::-1]) + [1] * (4 - nd)                      # reference order: innermost first
+    dd = [sd[axes[p]] for p in range(nd)] + [1] * (4 - nd)
+    ax = axes + list(range(nd, 4))
+    out = torch.empty(tuple(dd[:nd][::-1]), dtype=torch.float32, device=x.device)
+    cabi.check("permute_hip", _lib().permute_hip(_ptr(x), _ptr(out), x.numel(), nd, *ax, *sd, *dd, _stream()))
+    return out
+
+
 # ----------------------------------------------------------------------------- Q8_0
 def quantize_rows_q8_0(x: torch.Tensor) -> torch.Tensor:
     """f32 [..., K] -> uint8 [..., K/32, 34] block_q8_0 records (include/ppml/QuantBlocks.h:62-79)."""

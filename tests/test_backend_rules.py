@@ -91,3 +91,12 @@ def test_graph_compute_without_backend_is_refused():
     from proteinpredictmachinelearning_amd import cabi
 
     assert cabi.load().ppml_hip_backend_graph_compute(None, None, 0) == B.NOT_SUPPORTED
+
+
+def test_supports_op_permute():
+    # src/backend/CUDABackend.cpp:113-119: f32 in, f32 out
+    a = B.Tensor((4, 3, 2, 2))
+    assert B.supports_op(B.Tensor((3, 4, 2, 2), B.F32, B.OP_PERMUTE, [a]))
+    assert B.supports_op(B.Tensor((3, 4, 2, 2), B.F32, B.OP_TRANSPOSE, [a]))
+    assert not B.supports_op(B.Tensor((3, 4, 2, 2), B.F32, B.OP_PERMUTE, []))
+    assert not B.supports_op(B.Tensor((3, 4, 2, 2), B.F16, B.OP_PERMUTE, [a]))

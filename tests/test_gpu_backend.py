@@ -160,6 +160,37 @@ def test_fused_attention_node(be, oracle):
     assert be.graph_compute([bad]) == B.NOT_SUPPORTED
 
 
+def test_fused_attention_subgraph_as_the_reference_builds_it(be, oracle):
+    # ComputeGraphHelper.cpp:450-484: Q, K, V arrive as [L, D, h, B]; three permutes make [D, L, h, B], the fused
+    # node runs, a last permute gives [L, D, h, B] back -- six nodes, all on this backend
+    rng = np.random.default_rng(9)
+    Bt, h, L, d = 2, 2, 40, 16
+    q, k, v = [rng.standard_normal((Bt, h, L, d)).astype(np.float32) for _ in range(3)]     # flash layout values
+    bias = rng.standard_normal((Bt, h, L, L)).astype(np.float32)
+    leaves = [_leaf(be, np.ascontiguousarray(x.transpose(0, 1, 3, 2))) for x in (q, k, v)]    # dims [L, D, h, B]
+    perms = []
+    for t in leaves:
+        n = B.Tensor((d, L, h, Bt), B.F32, B.OP_PERMUTE, [t])
+        for i, a in enumerate((1, 0, 2, 3)):
+            n.set_param(i, a)
+        perms.append(n)
+    flash = B.Tensor((d, L, h, Bt), B.F32, B.OP_FLASH_ATTN_EXT, perms + [_leaf(be, bias), B.Tensor((L, h, Bt))])
+    flash.set_param(0, float(1.0 / np.sqrt(d))).set_param(1, 0).set_param(2, 1e-9).set_param(3, 64).set_param(4, 64)
+    out = B.Tensor((L, d, h, Bt), B.F32, B.OP_TRANSPOSE, [flash])
+    for i, a in enumerate((1, 0, 2, 3)):
+        out.set_param(i, a)
+    assert be.graph_compute(perms + [flash, out]) == B.SUCCESS, be.last_error
+    be.synchronize()
+    want, _ = oracle.flash_attn_forward(q, k, v, bias)
+    got = be.download(out).reshape(Bt, h, d, L).transpose(0, 1, 3, 2)
+    assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+    assert np.array_equal(be.download(perms[0]).reshape(Bt, h, L, d), q)
+    # an axis map outside the tensor's dimensions is refused (src/backend/CUDAKernels.cpp:1376-1381)
+    bad = B.Tensor((d, L, h, Bt), B.F32, B.OP_PERMUTE, [leaves[0]])
+    bad.set_param(0, 7)
+    assert be.graph_compute([bad]) == B.NOT_SUPPORTED
+
+
 def test_view_sources_are_resolved_and_noop_nodes_skipped(be, oracle):
     # a reshape node built with only src[0] set, and an offset view with view_src set, both feed a
     # mul_mat (src/backend/CUDABackend.cpp:800-819)

@@ -570,3 +570,36 @@ def test_flash_attn_forward_closed_forms(oracle):
     assert (o4[0, 1, 3] == 0).all() and np.isneginf(l4[0, 1, 3]) and np.isfinite(l4[0, 1, 2])
     # bad arguments are refused, not computed
     assert oracle.lib().orc_flash_attn_forward(1, 1, 0, 4, 0, 0.0, 0.0, 64, None, None, None, None, None, None, 1) == 1
+
+
+# ----------------------------------------------------------------------------- permute
+def _np_permute(x, axes):
+    """numpy statement of the reference's rule: reference dimension k is numpy axis nd-1-k, and
+    dimension p of the result is dimension axes[p] of the source."""
+    nd = x.ndim
+    return np.ascontiguousarray(np.transpose(x, [nd - 1 - axes[nd - 1 - a] for a in range(nd)]))
+
+
+def test_permute_hand_case_and_numpy(oracle):
+    # dims (reference order) [3, 2]: rows of 3; mat_transpose = axes (1, 0) gives dims [2, 3]
+    x = np.arange(6, dtype=np.float32).reshape(2, 3)
+    assert oracle.permute(x, (1, 0)).tolist() == [[0, 3], [1, 4], [2, 5]]
+    rng = np.random.default_rng(11)
+    import itertools
+    x4 = rng.standard_normal((3, 4, 5, 6)).astype(np.float32)        # reference dims [6, 5, 4, 3]
+    for axes in itertools.permutations(range(4)):
+        got = oracle.permute(x4, axes)
+        assert got.shape == tuple(x4.shape[::-1][a] for a in axes)[::-1]
+        assert np.array_equal(got, _np_permute(x4, axes)), axes
+        inverse = [axes.index(k) for k in range(4)]
+        assert np.array_equal(oracle.permute(got, inverse), x4), axes
+    x3 = rng.standard_normal((4, 5, 6)).astype(np.float32)
+    for axes in itertools.permutations(range(3)):
+        assert np.array_equal(oracle.permute(x3, axes), _np_permute(x3, axes)), axes
+    assert np.array_equal(oracle.permute(x4, (0, 1, 2, 3)), x4)
+    # an axis outside the tensor's dimensions is refused (the reference prints and skips the node)
+    import ctypes as C
+    out = np.zeros(6, dtype=np.float32)
+    rc = oracle.lib().orc_permute(x.ctypes.data_as(C.POINTER(C.c_float)), out.ctypes.data_as(C.POINTER(C.c_float)), 2,
+                                  (C.c_int32 * 4)(2, 0, 2, 3), (C.c_int64 * 4)(3, 2, 1, 1), (C.c_int64 * 4)(2, 3, 1, 1))
+    assert rc == 1 and not out.any()
