@@ -228,6 +228,27 @@ def main() -> int:
             return fn, ns
         f32_case(bridge, 2 * 824 * 32 * 256 * 4, 0.0, "permute_attention_bridge_824x256x32")
 
+        def trimul():
+            # triangle multiplication (outgoing) of the pair track: 128 channels x 103 x 103, contracted length 103
+            import ctypes as C
+            Dc, Lr = 128, 103
+            ns = 40
+            ls = [torch.randn(Dc * Lr * Lr, device=dev, generator=gen) for _ in range(ns)]
+            rs = [torch.randn(Dc * Lr * Lr, device=dev, generator=gen) for _ in range(ns)]
+            os_ = [torch.empty(Dc * Lr * Lr, device=dev) for _ in range(ns)]
+            lib, cabi = ops._lib(), ops.cabi
+            stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+            argsets = [(C.c_void_p(ls[i].data_ptr()), C.c_void_p(rs[i].data_ptr()), C.c_void_p(os_[i].data_ptr()),
+                        Dc, Lr, Lr, Lr, 1, 1.0 / Lr, 1, stream) for i in range(ns)]
+
+            def fn(i):
+                rc = lib.tri_mul_hip(*argsets[i])
+                if rc:
+                    cabi.check("tri_mul_hip", rc)
+            keep.append((ls, rs, os_))
+            return fn, ns
+        f32_case(trimul, 3 * 128 * 103 * 103 * 4, 2.0 * 128 * 103 ** 3, "tri_mul_outgoing_128x103x103x103")
+
         def opm():
             a = torch.randn(256, 12288, device=dev, generator=gen) * 0.1
             b = torch.randn(256, 12288, device=dev, generator=gen) * 0.1

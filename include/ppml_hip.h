@@ -138,6 +138,15 @@ int outer_product_mean_value_hip(const float *left, const float *right, float *d
 int mul_mat_tn_hip(const float *A, const float *Bm, float *O, int M, int K, int Nc, float alpha,
                    ppml_hip_stream_t stream);
 
+/* replaces tri_mul_cuda (src/cuda/PairKernels.cu:514-523, declared src/backend/CUDAKernels.cpp:316-318),
+ * indexing and finite guard of CPUBackend::kernel_tri_mul (src/backend/CPUKernels.cpp:907-968):
+ *   outgoing: dst[((d*I+i)*J+j)*B+b] = inv_L * sum_k left[((d*I+i)*K+k)*B+b] * right[((d*J+j)*K+k)*B+b]
+ *   incoming: dst[((d*I+i)*J+j)*B+b] = inv_L * sum_k left[((d*K+k)*I+i)*B+b] * right[((d*K+k)*J+j)*B+b]
+ * then NaN -> 0 and values beyond +-1e4 -> +-1e4.  One fp32-MFMA contraction per (d, b) plane. */
+int tri_mul_hip(const float *left, const float *right, float *dst,
+                int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float inv_L, int outgoing,
+                ppml_hip_stream_t stream);
+
 /* ---- fused attention forward ------------------------------------------------------------------ */
 /* replaces flash_attn_forward_cuda (declared src/backend/CUDAKernels.cpp:174, contract
  * include/ppml/FlashAttn.h:8-65, called from kernel_flash_attn_ext_cuda, CUDAKernels.cpp:894-903);

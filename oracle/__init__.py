@@ -76,6 +76,8 @@ def _load() -> C.CDLL:
     lib.orc_attention_scores.argtypes = [f32p, f32p, f32p] + [i64] * 5 + [C.c_int]
     lib.orc_flash_attn_forward.restype = C.c_int
     lib.orc_flash_attn_forward.argtypes = ([C.c_int] * 5 + [C.c_float, C.c_float, C.c_int] + [f32p] * 6 + [C.c_int])
+    lib.orc_tri_mul.restype = None
+    lib.orc_tri_mul.argtypes = [f32p, f32p, f32p] + [i64] * 5 + [C.c_float, C.c_int, C.c_int]
     lib.orc_permute.restype = C.c_int
     lib.orc_permute.argtypes = [f32p, f32p, C.c_int, C.POINTER(C.c_int32), C.POINTER(i64), C.POINTER(i64)]
     lib.orc_max_threads.restype = C.c_int
@@ -367,4 +369,13 @@ def permute(x, axes) -> np.ndarray:
     rc = lib().orc_permute(_fp(x), _fp(out), nd, (C.c_int32 * 4)(*ax), (C.c_int64 * 4)(*sd), (C.c_int64 * 4)(*dd))
     if rc:
         raise ValueError(f"orc_permute rc={rc}")
+    return out
+
+
+def tri_mul(left, right, D, I, J, K, B, L, outgoing=True, nthreads=0) -> np.ndarray:
+    """kernel_tri_mul (CPUKernels.cpp:907-968) on flat operands; returns the flat [D*I*J*B] result."""
+    left, right = _f32(left).reshape(-1), _f32(right).reshape(-1)
+    assert left.size == D * I * K * B and right.size == D * J * K * B
+    out = np.empty(D * I * J * B, dtype=np.float32)
+    lib().orc_tri_mul(_fp(left), _fp(right), _fp(out), D, I, J, K, B, L, int(outgoing), nthreads or max_threads())
     return out

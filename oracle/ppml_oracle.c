@@ -26,6 +26,9 @@
  *       einsum over the layout stated at src/backend/CPUKernels.cpp:975-981.
  *   orc_outer_product_mean_value : known answers of tests/test_outer_product_mean.cpp:10-70.
  *   orc_attention_scores: einsum special case and the 1/sqrt(D) closed form.
+ *   orc_tri_mul : numpy einsum over the layout stated at src/backend/CPUKernels.cpp:895-903 (outgoing and
+ *       incoming), exact on small integers; the finite guard on planted NaN / Inf / 1e5 values.  No
+ *       reference-held vector covers it.
  *   orc_permute : numpy.transpose with the axes translated (dst dim p = src dim axes[p], dims[0]
  *       innermost), identity and inverse permutations, hand-checked 2 x 3 case.
  *   orc_flash_attn_forward : the reference's own src/ops/FlashAttn.cpp compiled as-is
@@ -120,6 +123,31 @@ int orc_flash_attn_forward(int B, int h, int L, int d, int causal, float scale, 
         free(tile);
     }
     return 0;
+}
+
+/* src/backend/CPUKernels.cpp:907-968: one output per index, k ascending, sequential binary32 sum. */
+void orc_tri_mul(const float *left, const float *right, float *dst,
+                 int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float L, int outgoing, int nthreads) {
+    const float inv_L = 1.0f / L;
+    const int64_t total = B * I * J * D;
+    if (nthreads <= 0) nthreads = 1;
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+    for (int64_t idx = 0; idx < total; ++idx) {
+        int64_t tmp = idx;
+        const int64_t b = tmp % B; tmp /= B;
+        const int64_t j = tmp % J; tmp /= J;
+        const int64_t i = tmp % I;
+        const int64_t d = tmp / I;
+        float sum = 0.0f;
+        if (outgoing) {
+            for (int64_t k = 0; k < K; ++k) sum += left[((d * I + i) * K + k) * B + b] * right[((d * J + j) * K + k) * B + b];
+        } else {
+            for (int64_t k = 0; k < K; ++k) sum += left[((d * K + k) * I + i) * B + b] * right[((d * K + k) * J + j) * B + b];
+        }
+        float v = sum * inv_L;
+        if (!(v == v) || v > 1e4f || v < -1e4f) v = (v != v) ? 0.0f : (v > 1e4f ? 1e4f : -1e4f);
+        dst[idx] = v;
+    }
 }
 
 /* src/backend/CPUKernels.cpp:1669-1717: for every destination element, in order, decode its

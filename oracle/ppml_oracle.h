@@ -92,6 +92,12 @@ int orc_flash_attn_forward(int B, int h, int L, int d, int causal, float scale, 
                            const float *Q, const float *K, const float *V, const float *bias,
                            float *O, float *LSE, int nthreads);
 
+/* src/backend/CPUKernels.cpp:907-968 (kernel_tri_mul): d outermost, b innermost in every tensor;
+ * outgoing contracts left[d,i,k,b] right[d,j,k,b], incoming left[d,k,i,b] right[d,k,j,b]; result times
+ * 1/L, then the finite guard (NaN -> 0, beyond +-1e4 -> +-1e4). */
+void orc_tri_mul(const float *left, const float *right, float *dst,
+                 int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float L, int outgoing, int nthreads);
+
 /* src/backend/CPUKernels.cpp:1669-1717 (kernel_permute): dimension p of dst is dimension axes[p] of src;
  * sd = source sizes, dd = destination sizes (dims[0] innermost), entries past ndim ignored.
  * returns 0 ok, 1 when an axis is outside [0, ndim) -- the reference prints and leaves dst untouched. */

@@ -150,6 +150,11 @@ bool node_supported(const Tensor* node) {
         case OP_OUT_PROD:
             return src0 && src1 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
                    node->type == TENSOR_TYPE_F32;
+        case OP_TRI_MUL:
+            // src/backend/CUDABackend.cpp:395-402: left, right and the result all 4-D f32
+            if (!src0 || !src1) return false;
+            if (src0->type != TENSOR_TYPE_F32 || src1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32) return false;
+            return src0->ndim == 4 && src1->ndim == 4 && node->ndim == 4;
         case OP_PERMUTE:
         case OP_TRANSPOSE:
             // src/backend/CUDABackend.cpp:113-119
@@ -341,6 +346,26 @@ Status HipBackend::kernel_permute(Tensor* node) {
     return Status::SUCCESS;
 }
 
+// src/backend/CUDAKernels.cpp:1146-1170: the node is [D, I, J, B]; op_params[0] holds L as a float,
+// the low byte of op_params[4] the outgoing flag (ComputeGraphHelper.cpp:409-411); the contracted length
+// is left.dims[2] (outgoing) or left.dims[1] (incoming); L == 0 is refused.
+Status HipBackend::kernel_tri_mul(Tensor* node) {
+    const Tensor* l = node->src[0];
+    const Tensor* r = node->src[1];
+    if (!l || !r || !l->data || !r->data || !node->data) return fail(Status::NOT_SUPPORTED, "tri_mul: unbound tensor");
+    const float L = node->param_f32(0);
+    const bool outgoing = (node->op_params[4] & 0xff) != 0;
+    if (L == 0.0f) return fail(Status::NOT_SUPPORTED, "tri_mul: L is zero");
+    const int64_t D = node->dims[0], I = node->dims[1], J = node->dims[2], B = node->dims[3];
+    const int64_t K = outgoing ? l->dims[2] : l->dims[1];
+    if (l->numel() != D * I * K * B || r->numel() != D * J * K * B)
+        return fail(Status::NOT_SUPPORTED, "tri_mul: operand sizes do not match [D,I,J,B] and the contracted length");
+    const int rc = tri_mul_hip(static_cast<const float*>(l->data), static_cast<const float*>(r->data),
+                               static_cast<float*>(node->data), D, I, J, K, B, 1.0f / L, outgoing ? 1 : 0, nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("tri_mul: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
 Status HipBackend::dispatch_node(Tensor* node) {
     switch (node->op) {
         case OP_MUL_MAT: return kernel_mul_mat(node);
@@ -349,6 +374,7 @@ Status HipBackend::dispatch_node(Tensor* node) {
         case OP_FLASH_ATTN_EXT: return kernel_flash_attn_ext(node);
         case OP_PERMUTE:
         case OP_TRANSPOSE: return kernel_permute(node);
+        case OP_TRI_MUL: return kernel_tri_mul(node);
         default: return fail(Status::NOT_SUPPORTED, "no kernel for op " + std::to_string(node->op));
     }
 }

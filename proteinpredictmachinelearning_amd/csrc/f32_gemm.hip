@@ -38,6 +38,7 @@ struct GemmParams {
     int tiles_m, tiles_n;
     int stream_c;         // output larger than the last-level cache: write it with streaming stores
     int f16_in;           // A and B hold IEEE halves (k contiguous); products and sums are binary32
+    int clamp;            // finite guard in the epilogue (triangle multiplication)
 };
 
 // 16 x 128 tile of one operand -> two v4f per thread
@@ -118,7 +119,10 @@ __device__ __forceinline__ void store_tile(float* __restrict__ lds, int tid, con
     }
 }
 
-template <int MODE, bool SPLIT_C, bool STREAM_C>
+// CLAMP: the finite guard of the triangle multiplication (src/backend/CPUKernels.cpp:957-962): NaN -> 0,
+// values beyond +-1e4 -> +-1e4.  A compile-time property: a run-time test in this store loop costs the
+// other contractions a quarter of their speed.
+template <int MODE, bool SPLIT_C, bool STREAM_C, bool CLAMP = false>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(16))) float lds_a[BK * LDS_LD];
     __shared__ __attribute__((aligned(16))) float lds_b[BK * LDS_LD];
@@ -207,6 +211,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
                 float v = acc[ti][tj][r];
                 if (scale) v *= p.alpha;
                 if (BIAS_LAST) v += tail_bias;
+                if (CLAMP) v = (v != v) ? 0.0f : (v > 1e4f ? 1e4f : (v < -1e4f ? -1e4f : v));
                 if (STREAM_C) __builtin_nontemporal_store(v, &C[roff + coff]);
                 else C[roff + coff] = v;
             }
@@ -232,7 +237,13 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
         if (p.stream_c) hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, true>), grid, block, 0, stream, p);  \
         else hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, false>), grid, block, 0, stream, p);    \
     } while (0)
-    if (p.f16_in)                     { PPML_LAUNCH(LOAD_K_CONTIG_F16, false); }
+    if (p.clamp) {
+        if (split || p.stream_c || p.f16_in) { set_error("%s: no clamped instance for this addressing", what); return RC_BAD_ARGS; }
+        if (mode == LOAD_K_CONTIG) hipLaunchKernelGGL((gemm_f32_kernel<LOAD_K_CONTIG, false, false, true>), grid, block, 0, stream, p);
+        else if (mode == LOAD_ROW_CONTIG) hipLaunchKernelGGL((gemm_f32_kernel<LOAD_ROW_CONTIG, false, false, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((gemm_f32_kernel<LOAD_STRIDED, false, false, true>), grid, block, 0, stream, p);
+    }
+    else if (p.f16_in)                { PPML_LAUNCH(LOAD_K_CONTIG_F16, false); }
     else if (mode == LOAD_K_CONTIG)   { if (split) PPML_LAUNCH(LOAD_K_CONTIG, true);   else PPML_LAUNCH(LOAD_K_CONTIG, false); }
     else if (mode == LOAD_ROW_CONTIG) { if (split) PPML_LAUNCH(LOAD_ROW_CONTIG, true); else PPML_LAUNCH(LOAD_ROW_CONTIG, false); }
     else                              { if (split) PPML_LAUNCH(LOAD_STRIDED, true);    else PPML_LAUNCH(LOAD_STRIDED, false); }
@@ -369,4 +380,29 @@ extern "C" int outer_product_mean_value_hip(const float* left, const float* righ
     p.c_lm = p.c_ln = static_cast<int>(D);
     p.c_mo = L * D * D; p.c_mi = D; p.c_no = D * D; p.c_ni = 1;
     return launch_gemm(p, static_cast<hipStream_t>(stream), "outer_product_mean_value_hip");
+}
+
+extern "C" int tri_mul_hip(const float* left, const float* right, float* dst,
+                           int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float inv_L, int outgoing,
+                           ppml_hip_stream_t stream) {
+    if (!left || !right || !dst || D <= 0 || I <= 0 || J <= 0 || K <= 0 || B <= 0 ||
+        I > 0x7fffffff || J > 0x7fffffff || K > 0x7fffffff || D > 0x7fffffff || B > 0x7fffffff) {
+        set_error("tri_mul_hip: bad arguments"); return RC_BAD_ARGS;
+    }
+    stats_record(I, K, J);
+    GemmParams p = plain_params();
+    p.A = left; p.B = right; p.C = dst;                // rows = i, cols = j, planes = (d, b)
+    p.M = static_cast<int>(I); p.N = static_cast<int>(J); p.K = static_cast<int>(K);
+    if (outgoing) {                                    // left[((d*I+i)*K+k)*B+b], right[((d*J+j)*K+k)*B+b]
+        p.a_rs = K * B; p.a_ks = B; p.b_rs = K * B; p.b_ks = B;
+    } else {                                           // left[((d*K+k)*I+i)*B+b], right[((d*K+k)*J+j)*B+b]
+        p.a_rs = B; p.a_ks = I * B; p.b_rs = B; p.b_ks = J * B;
+    }
+    p.np2 = static_cast<int>(B); p.np3 = static_cast<int>(D);
+    p.a_p2 = 1; p.b_p2 = 1; p.c_p2 = 1;                // batch b is the innermost index of every tensor
+    p.a_p3 = I * K * B; p.b_p3 = J * K * B; p.c_p3 = I * J * B;
+    p.c_mi = J * B; p.c_ni = B;                        // dst[((d*I+i)*J+j)*B+b]
+    p.alpha = inv_L;
+    p.clamp = 1;
+    return launch_gemm(p, static_cast<hipStream_t>(stream), "tri_mul_hip");
 }

@@ -159,6 +159,21 @@ def outer_product_mean_value(left: torch.Tensor, right: torch.Tensor) -> torch.T
     return out
 
 
+def tri_mul(left: torch.Tensor, right: torch.Tensor, D: int, I: int, J: int, K: int, B: int, L: float,
+            outgoing: bool = True) -> torch.Tensor:
+    """Triangle multiplication, graph form (src/backend/CPUKernels.cpp:907-968): flat operands indexed as the
+    kernel does (d outermost, b innermost); returns the flat [D*I*J*B] result incl. the 1/L and the finite guard."""
+    left, right = _dev_f32(left, "left"), _dev_f32(right, "right")
+    if L == 0:
+        raise ValueError("tri_mul: L must not be zero")
+    if left.numel() != D * I * K * B or right.numel() != D * J * K * B:
+        raise ValueError("tri_mul: operand size does not match D, I, J, K, B")
+    out = torch.empty(D * I * J * B, dtype=torch.float32, device=left.device)
+    cabi.check("tri_mul_hip", _lib().tri_mul_hip(_ptr(left), _ptr(right), _ptr(out), D, I, J, K, B, 1.0 / float(L),
+                                                 int(outgoing), _stream()))
+    return out
+
+
 def flash_attn_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bias: torch.Tensor | None = None,
                        causal: bool = False, scale: float = 0.0, eps: float = 1e-9, Bc: int = 64,
                        want_lse: bool = True):

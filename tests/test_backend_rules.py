@@ -100,3 +100,12 @@ def test_supports_op_permute():
     assert B.supports_op(B.Tensor((3, 4, 2, 2), B.F32, B.OP_TRANSPOSE, [a]))
     assert not B.supports_op(B.Tensor((3, 4, 2, 2), B.F32, B.OP_PERMUTE, []))
     assert not B.supports_op(B.Tensor((3, 4, 2, 2), B.F16, B.OP_PERMUTE, [a]))
+
+
+def test_supports_op_tri_mul():
+    # src/backend/CUDABackend.cpp:395-402: both operands and the result 4-D f32
+    l, r = B.Tensor((8, 5, 6, 1)), B.Tensor((8, 4, 6, 1))
+    assert B.supports_op(B.Tensor((8, 5, 4, 1), B.F32, B.OP_TRI_MUL, [l, r]))
+    assert not B.supports_op(B.Tensor((8, 5, 4, 1), B.F32, B.OP_TRI_MUL, [l]))
+    assert not B.supports_op(B.Tensor((8, 5, 4), B.F32, B.OP_TRI_MUL, [l, r]))
+    assert not B.supports_op(B.Tensor((8, 5, 4, 1), B.F32, B.OP_TRI_MUL, [B.Tensor((8, 5, 6, 1), B.F16), r]))

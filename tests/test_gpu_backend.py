@@ -191,6 +191,24 @@ def test_fused_attention_subgraph_as_the_reference_builds_it(be, oracle):
     assert be.graph_compute([bad]) == B.NOT_SUPPORTED
 
 
+def test_tri_mul_node(be, oracle):
+    # ComputeGraphHelper.cpp:390-413: node [D, I, J, B]; op_params[0] = L (float), low byte of op_params[4] = outgoing
+    rng = np.random.default_rng(12)
+    D, I, J, K, Bt = 4, 9, 7, 11, 1
+    for outgoing in (True, False):
+        ldims = (D, I, K, Bt) if outgoing else (D, K, I, Bt)
+        rdims = (D, J, K, Bt) if outgoing else (D, K, J, Bt)
+        left = rng.standard_normal(D * I * K * Bt).astype(np.float32)
+        right = rng.standard_normal(D * J * K * Bt).astype(np.float32)
+        node = B.Tensor((D, I, J, Bt), B.F32, B.OP_TRI_MUL, [_leaf(be, left, dims=ldims), _leaf(be, right, dims=rdims)])
+        node.set_param(0, float(K)).set_param(4, int(outgoing))
+        assert be.graph_compute([node]) == B.SUCCESS, be.last_error
+        want = oracle.tri_mul(left, right, D, I, J, K, Bt, float(K), outgoing)
+        assert np.abs(be.download(node) - want).max() <= 1e-4 * np.abs(want).max()
+    node.set_param(0, 0.0)                              # L == 0 (src/backend/CUDAKernels.cpp:1165)
+    assert be.graph_compute([node]) == B.NOT_SUPPORTED
+
+
 def test_view_sources_are_resolved_and_noop_nodes_skipped(be, oracle):
     # a reshape node built with only src[0] set, and an offset view with view_src set, both feed a
     # mul_mat (src/backend/CUDABackend.cpp:800-819)

@@ -217,3 +217,37 @@ def test_dense_outer_product_mean_stress_shape_properties(ops):
     want = (a[:, rows].double().t() @ b.double()) / N
     err = (o[rows].double() - want).abs().max().item()
     assert err <= RTOL * want.abs().max().item()
+
+
+# ----------------------------------------------------------------------------- triangle multiplication
+@pytest.mark.parametrize("D,I,J,K,Bt,outgoing", [
+    (3, 5, 4, 6, 2, True), (3, 5, 4, 6, 2, False),            # batch innermost: strided operands
+    (16, 103, 103, 103, 1, True), (16, 103, 103, 103, 1, False),   # pair-track shape, a slice of the channels
+    (2, 130, 70, 33, 1, True), (2, 130, 70, 33, 1, False),    # two row tiles, ragged everywhere
+])
+def test_tri_mul(ops, oracle, D, I, J, K, Bt, outgoing):
+    rng = np.random.default_rng(D * 1000 + I)
+    left = rng.standard_normal(D * I * K * Bt).astype(np.float32)
+    right = rng.standard_normal(D * J * K * Bt).astype(np.float32)
+    L = float(K)
+    want = oracle.tri_mul(left, right, D, I, J, K, Bt, L, outgoing)
+    got = ops.tri_mul(_dev(left), _dev(right), D, I, J, K, Bt, L, outgoing).cpu().numpy()
+    _check(got, want)
+    # exact on small integers (every product and partial sum is exact in binary32; 1/L a power of two)
+    li = rng.integers(-4, 5, size=left.size).astype(np.float32)
+    ri = rng.integers(-4, 5, size=right.size).astype(np.float32)
+    got = ops.tri_mul(_dev(li), _dev(ri), D, I, J, K, Bt, 8.0, outgoing).cpu().numpy()
+    assert np.array_equal(got, oracle.tri_mul(li, ri, D, I, J, K, Bt, 8.0, outgoing))
+
+
+def test_tri_mul_finite_guard(ops, oracle):
+    # src/backend/CPUKernels.cpp:957-962
+    left = np.zeros((1, 4, 2, 1), dtype=np.float32)
+    right = np.ones((1, 1, 2, 1), dtype=np.float32)
+    left[0, 0, 0, 0] = np.nan
+    left[0, 1, 0, 0] = 3e4
+    left[0, 2, 0, 0] = -np.inf
+    left[0, 3, 0, 0] = 1.9e4
+    got = ops.tri_mul(_dev(left.reshape(-1)), _dev(right.reshape(-1)), 1, 4, 1, 2, 1, 2.0, True).cpu().numpy()
+    assert got.tolist() == [0.0, 1e4, -1e4, 9.5e3]
+    assert got.tolist() == oracle.tri_mul(left, right, 1, 4, 1, 2, 1, 2.0, True).tolist()

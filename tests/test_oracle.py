@@ -603,3 +603,29 @@ def test_permute_hand_case_and_numpy(oracle):
     rc = oracle.lib().orc_permute(x.ctypes.data_as(C.POINTER(C.c_float)), out.ctypes.data_as(C.POINTER(C.c_float)), 2,
                                   (C.c_int32 * 4)(2, 0, 2, 3), (C.c_int64 * 4)(3, 2, 1, 1), (C.c_int64 * 4)(2, 3, 1, 1))
     assert rc == 1 and not out.any()
+
+
+# ----------------------------------------------------------------------------- triangle multiplication
+def test_tri_mul_against_einsum_and_the_finite_guard(oracle):
+    rng = np.random.default_rng(21)
+    D, I, J, K, Bt, L = 3, 5, 4, 6, 2, 8.0          # 1/8 is exact, small integers keep every sum exact
+    # outgoing: left[d,i,k,b], right[d,j,k,b]; incoming: left[d,k,i,b], right[d,k,j,b] (CPUKernels.cpp:895-903)
+    lo = rng.integers(-4, 5, size=(D, I, K, Bt)).astype(np.float32)
+    ro = rng.integers(-4, 5, size=(D, J, K, Bt)).astype(np.float32)
+    want = np.einsum("dikb,djkb->dijb", lo.astype(np.float64), ro.astype(np.float64)) / L
+    assert np.array_equal(oracle.tri_mul(lo, ro, D, I, J, K, Bt, L, outgoing=True).reshape(D, I, J, Bt), want)
+    li = rng.integers(-4, 5, size=(D, K, I, Bt)).astype(np.float32)
+    ri = rng.integers(-4, 5, size=(D, K, J, Bt)).astype(np.float32)
+    want = np.einsum("dkib,dkjb->dijb", li.astype(np.float64), ri.astype(np.float64)) / L
+    assert np.array_equal(oracle.tri_mul(li, ri, D, I, J, K, Bt, L, outgoing=False).reshape(D, I, J, Bt), want)
+    # the two forms differ (a transposed operand would pass one of the checks above, not both)
+    assert not np.array_equal(oracle.tri_mul(lo, ro, D, I, J, K, Bt, L, True), oracle.tri_mul(lo.reshape(-1), ro.reshape(-1), D, I, J, K, Bt, L, False))
+    # finite guard (CPUKernels.cpp:957-962): NaN -> 0, beyond +-1e4 -> +-1e4, applied after the 1/L
+    l1 = np.zeros((1, 4, 2, 1), dtype=np.float32)
+    r1 = np.ones((1, 1, 2, 1), dtype=np.float32)
+    l1[0, 0, 0, 0] = np.nan
+    l1[0, 1, 0, 0] = 3e4          # 3e4 / 2 = 1.5e4 -> 1e4
+    l1[0, 2, 0, 0] = -np.inf
+    l1[0, 3, 0, 0] = 1.9e4        # 9.5e3 stays
+    got = oracle.tri_mul(l1, r1, 1, 4, 1, 2, 1, 2.0, True)
+    assert got.tolist() == [0.0, 1e4, -1e4, 9.5e3]
