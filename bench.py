@@ -182,7 +182,7 @@ def main() -> int:
         f32_case(logits(824, 256, 32), (2 * 824 * 32 * 256 + 824 * 256 * 256) * 4, 2.0 * 824 * 256 * 256 * 32,
                  "attn_logits_msa_824x256x256x32")
 
-        def attention(planes, L, D, with_bias):
+        def attention(planes, L, D, with_bias, layout=0):
             def make():
                 import ctypes as C
                 nb = (4 * planes * L * D + planes * L + (planes * L * L if with_bias else 0)) * 4
@@ -194,19 +194,21 @@ def main() -> int:
                 stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
                 ptr = lambda t: C.c_void_p(t.data_ptr()) if t is not None else None      # noqa: E731
                 argsets = [(1, planes, L, D, 0, 0.0, 1e-9, 64, ptr(qkv[i][0]), ptr(qkv[i][1]), ptr(qkv[i][2]), ptr(bs[i]),
-                            ptr(outs[i][0]), ptr(outs[i][1]), stream) for i in range(ns)]
+                            ptr(outs[i][0]), ptr(outs[i][1]), layout, stream) for i in range(ns)]
 
                 def fn(i):
-                    rc = lib.flash_attn_forward_hip(*argsets[i])
+                    rc = lib.flash_attn_forward_ex_hip(*argsets[i])
                     if rc:
-                        cabi.check("flash_attn_forward_hip", rc)
+                        cabi.check("flash_attn_forward_ex_hip", rc)
                 keep.append((qkv, bs, outs))
                 return fn, ns
             return make
         keep = []
-        for planes, L, D, wb, tag in [(412, 103, 32, True, "pair_412x103x32_bias"), (824, 256, 32, True, "msa_824x256x32_bias"),
-                                      (824, 256, 32, False, "msa_824x256x32")]:
-            f32_case(attention(planes, L, D, wb), (4 * planes * L * D + planes * L + (planes * L * L if wb else 0)) * 4,
+        # layout 3: Q, K, V and O in the graph's [L, D, h, B] layout, i.e. without the four permutation copies
+        for planes, L, D, wb, lay, tag in [(412, 103, 32, True, 0, "pair_412x103x32_bias"), (824, 256, 32, True, 0, "msa_824x256x32_bias"),
+                                           (824, 256, 32, False, 0, "msa_824x256x32"),
+                                           (824, 256, 32, True, 3, "msa_824x256x32_bias_graph_layout")]:
+            f32_case(attention(planes, L, D, wb, lay), (4 * planes * L * D + planes * L + (planes * L * L if wb else 0)) * 4,
                      4.0 * planes * L * L * D, "fused_attention_" + tag)
 
         def bridge():

@@ -164,6 +164,14 @@ int flash_attn_forward_hip(int B, int h, int L, int d, int causal, float scale, 
                            const float *Q, const float *K, const float *V, const float *bias,
                            float *O, float *LSE, ppml_hip_stream_t stream);
 
+/* The same computation on tensors that have not been through the layout bridges the reference's graph
+ * builder puts around the fused node (src/core/ComputeGraphHelper.cpp:456-458, 483): layout bit 0 -- Q, K
+ * and V are [B][h][d][L] (the graph's [L, D, h, B] tensors); bit 1 -- O is written as [B][h][d][L].  It lets an
+ * executor skip those four permutation copies.  No counterpart in the reference. */
+int flash_attn_forward_ex_hip(int B, int h, int L, int d, int causal, float scale, float softmax_eps, int Bc,
+                              const float *Q, const float *K, const float *V, const float *bias,
+                              float *O, float *LSE, int layout, ppml_hip_stream_t stream);
+
 /* ---- dimension permutation (a real copy) ------------------------------------------------------ */
 /* replaces permute_cuda and transpose_cuda (declared src/backend/CUDAKernels.cpp:137-143, called from
  * kernel_permute_cuda / kernel_transpose_cuda, 1344-1390); semantics of CPUBackend::kernel_permute

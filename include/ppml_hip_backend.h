@@ -53,6 +53,11 @@ void ppml_hip_backend_set_skip_alloc(ppml_hip_backend *b, int on);
 /* 0: quantize activations with the Q8_0 rule (default, the CPU contract); 1: with the Q8_1 rule of
  * the reference's CUDA launcher (src/cuda/MulMatQ8Kernel.cu:483-527) */
 void ppml_hip_backend_set_q8_1_activations(ppml_hip_backend *b, int on);
+/* 1: graph_compute does not execute the {1,0,2,3} permutations the reference's builder wraps around a fused
+ * attention node (src/core/ComputeGraphHelper.cpp:456-458, 483) when the attention node is their only
+ * reader / they are its only reader; the attention kernel takes the other layout itself and the skipped
+ * tensors are never written.  0 (default): every node is executed as it stands. */
+void ppml_hip_backend_set_fuse_attention_bridges(ppml_hip_backend *b, int on);
 int ppml_hip_backend_graph_compute(ppml_hip_backend *b, ppml_hip_tensor **nodes, int n);
 int ppml_hip_backend_pack_weight(ppml_hip_backend *b, ppml_hip_tensor *weight);
 

@@ -135,6 +135,12 @@ public:
     // contract), true = Q8_1 (what the reference's CUDA launcher does, src/cuda/MulMatQ8Kernel.cu:483-527).
     void set_q8_1_activations(bool v) { q8_1_activations_ = v; }
     bool q8_1_activations() const { return q8_1_activations_; }
+    // Off by default.  On: a permutation {1,0,2,3} whose only reader is a fused attention node (all three of
+    // Q, K, V), or that is the only reader of its result, is not executed -- the attention kernel takes that
+    // layout directly -- and the skipped permutation's own tensor is never written.  Only for graphs whose
+    // every reader of those tensors is inside the graph handed to graph_compute.
+    void set_fuse_attention_bridges(bool v) { fuse_attention_bridges_ = v; }
+    bool fuse_attention_bridges() const { return fuse_attention_bridges_; }
 
     // Once-per-weight step of src/model/PPML.cpp:4504-4528: turns a Q8_0 / Q8_1 / Q8_0R weight node
     // into the MFMA-fragment layout in a buffer owned by this backend.
@@ -155,6 +161,8 @@ private:
     int device_;
     bool skip_alloc_ = false;
     bool q8_1_activations_ = false;
+    bool fuse_attention_bridges_ = false;
+    int attn_layout_ = 0;                                // layout bits of the attention node being dispatched
     std::string error_;
     std::vector<std::unique_ptr<Buffer>> owned_;         // node outputs allocated here, packed weights
 };

@@ -99,6 +99,9 @@ class Backend:
     def set_q8_1_activations(self, on: bool) -> None:
         self._lib.ppml_hip_backend_set_q8_1_activations(self.handle, int(on))
 
+    def set_fuse_attention_bridges(self, on: bool) -> None:
+        self._lib.ppml_hip_backend_set_fuse_attention_bridges(self.handle, int(on))
+
     def upload(self, t: Tensor, host: np.ndarray) -> Tensor:
         host = np.ascontiguousarray(host)
         rc = self._lib.ppml_hip_tensor_upload(self.handle, t.handle, host.ctypes.data_as(C.c_void_p), host.nbytes)

@@ -36,6 +36,7 @@ SIGNATURES = {
     "mul_mat_tn_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _f, _vp]),
     "tri_mul_hip": (_i, [_vp, _vp, _vp] + [_i64] * 5 + [_f, _i, _vp]),
     "flash_attn_forward_hip": (_i, [_i] * 5 + [_f, _f, _i] + [_vp] * 7),
+    "flash_attn_forward_ex_hip": (_i, [_i] * 5 + [_f, _f, _i] + [_vp] * 6 + [_i, _vp]),
     "permute_hip": (_i, [_vp, _vp, _i64, _i] + [_i] * 4 + [_i64] * 8 + [_vp]),
     "ppml_hip_mulmat_stats": (_i, [C.POINTER(_i64), _i]),
 }
@@ -62,6 +63,7 @@ BACKEND_SIGNATURES = {
     "ppml_hip_backend_supports_op": (_i, [_vp, _vp]),
     "ppml_hip_backend_set_skip_alloc": (None, [_vp, _i]),
     "ppml_hip_backend_set_q8_1_activations": (None, [_vp, _i]),
+    "ppml_hip_backend_set_fuse_attention_bridges": (None, [_vp, _i]),
     "ppml_hip_backend_graph_compute": (_i, [_vp, C.POINTER(_vp), _i]),
     "ppml_hip_backend_pack_weight": (_i, [_vp, _vp]),
 }

@@ -50,6 +50,8 @@ struct AttnParams {
     float scale, eps;
     int head;            // keys of the reference's first block: min(Bc, keys of the row)
     int stage_rows;      // keys staged in LDS at a time: min(CH, L rounded up to 32)
+    int in_ld;           // Q, K, V are [B][h][d][L] (the graph's [L, D, h, B] tensors, not yet permuted)
+    int out_ld;          // O is written as [B][h][d][L]
 };
 
 __device__ __forceinline__ float lane_xor32(float x) {
@@ -83,12 +85,21 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
     const float sc2 = p.scale * LOG2E;                // scores are kept in the base-2 domain
     // ---- this lane's slice of its query row, times scale * log2(e): elements half*DP/2 + s, s = 0 .. DP/2-1 (zero past d / past L)
     float qreg[DP / 2];
+    if (p.in_ld) {
+        // [d][L]: one element per feature row, lanes along the queries (whole 128-byte runs)
 #pragma unroll
-    for (int s = 0; s < DP / 2; s += 4) {
-        const int e = half * (DP / 2) + s;
-        v4f x = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (q < L && e < d) x = *reinterpret_cast<const v4f*>(p.Q + plane_off + static_cast<int64_t>(q) * d + e);
-        qreg[s] = x[0] * sc2; qreg[s + 1] = x[1] * sc2; qreg[s + 2] = x[2] * sc2; qreg[s + 3] = x[3] * sc2;
+        for (int s = 0; s < DP / 2; ++s) {
+            const int e = half * (DP / 2) + s;
+            qreg[s] = (q < L && e < d) ? p.Q[plane_off + static_cast<int64_t>(e) * L + q] * sc2 : 0.0f;
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < DP / 2; s += 4) {
+            const int e = half * (DP / 2) + s;
+            v4f x = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (q < L && e < d) x = *reinterpret_cast<const v4f*>(p.Q + plane_off + static_cast<int64_t>(q) * d + e);
+            qreg[s] = x[0] * sc2; qreg[s + 1] = x[1] * sc2; qreg[s + 2] = x[2] * sc2; qreg[s + 3] = x[3] * sc2;
+        }
     }
 
     v16f acc_o[NB];
@@ -201,16 +212,45 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
         __syncthreads();
         const int ckeys = L - c0 < stage ? L - c0 : stage;
         const int rows = (ckeys + 31) / 32 * 32;
-        for (int idx = tid; idx < rows * (DP / 4); idx += NW * 64) {
-            const int key = idx / (DP / 4), c = (idx % (DP / 4)) * 4;
-            v4f kx = {0.0f, 0.0f, 0.0f, 0.0f}, vx = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (key < ckeys && c < d) {
-                const int64_t off = plane_off + static_cast<int64_t>(c0 + key) * d + c;
-                kx = *reinterpret_cast<const v4f*>(p.K + off);
-                vx = *reinterpret_cast<const v4f*>(p.V + off);
+        if (p.in_ld) {
+            // source rows run along the keys: four keys of one feature per thread, scattered into the
+            // key-major LDS tiles
+            // (eight lanes read 128 contiguous bytes of one feature row; the LDS writes of a wave then
+            // spread over 16 banks instead of 2)
+            const int kq_n = rows / 4;
+            for (int idx = tid; idx < DP * kq_n; idx += NW * 64) {
+                const int rest = idx >> 3;
+                const int dd = rest % DP, kq = ((rest / DP) * 8 + (idx & 7)) * 4;
+                v4f kx = {0.0f, 0.0f, 0.0f, 0.0f}, vx = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (dd < d) {
+                    const int64_t off = plane_off + static_cast<int64_t>(dd) * L + c0 + kq;
+                    if (kq + 3 < ckeys) {
+                        kx = *reinterpret_cast<const v4f_u*>(p.K + off);
+                        vx = *reinterpret_cast<const v4f_u*>(p.V + off);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            if (kq + i < ckeys) { kx[i] = p.K[off + i]; vx[i] = p.V[off + i]; }
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    lds_k[(kq + i) * KS + dd] = kx[i];
+                    lds_v[(kq + i) * VS + dd] = vx[i];
+                }
             }
-            *reinterpret_cast<v4f*>(lds_k + key * KS + c) = kx;
-            *reinterpret_cast<v4f*>(lds_v + key * VS + c) = vx;
+        } else {
+            for (int idx = tid; idx < rows * (DP / 4); idx += NW * 64) {
+                const int key = idx / (DP / 4), c = (idx % (DP / 4)) * 4;
+                v4f kx = {0.0f, 0.0f, 0.0f, 0.0f}, vx = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (key < ckeys && c < d) {
+                    const int64_t off = plane_off + static_cast<int64_t>(c0 + key) * d + c;
+                    kx = *reinterpret_cast<const v4f*>(p.K + off);
+                    vx = *reinterpret_cast<const v4f*>(p.V + off);
+                }
+                *reinterpret_cast<v4f*>(lds_k + key * KS + c) = kx;
+                *reinterpret_cast<v4f*>(lds_v + key * VS + c) = vx;
+            }
         }
         __syncthreads();
         if (!wave_active) continue;
@@ -234,17 +274,28 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
     m_head = fmaxf(m_head, lane_xor32(m_head));
     const bool live = l_run > 0.0f && m_head > -INFINITY;
     const float inv = live ? 1.0f / (l_run + p.eps) : 0.0f;
-    float* orow = p.O + plane_off + static_cast<int64_t>(q) * d;
+    if (p.out_ld) {
+        // [d][L]: lanes along the queries
 #pragma unroll
-    for (int b = 0; b < NB; ++b)
+        for (int b = 0; b < NB; ++b)
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int dd = b * 32 + 8 * g + 4 * half;
-            if (dd < d) {
-                const v4f o = {acc_o[b][4 * g] * inv, acc_o[b][4 * g + 1] * inv, acc_o[b][4 * g + 2] * inv, acc_o[b][4 * g + 3] * inv};
-                *reinterpret_cast<v4f*>(orow + dd) = live ? o : v4f{0.0f, 0.0f, 0.0f, 0.0f};
+            for (int r = 0; r < 16; ++r) {
+                const int dd = b * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (dd < d) p.O[plane_off + static_cast<int64_t>(dd) * L + q] = live ? acc_o[b][r] * inv : 0.0f;
             }
-        }
+    } else {
+        float* orow = p.O + plane_off + static_cast<int64_t>(q) * d;
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int dd = b * 32 + 8 * g + 4 * half;
+                if (dd < d) {
+                    const v4f o = {acc_o[b][4 * g] * inv, acc_o[b][4 * g + 1] * inv, acc_o[b][4 * g + 2] * inv, acc_o[b][4 * g + 3] * inv};
+                    *reinterpret_cast<v4f*>(orow + dd) = live ? o : v4f{0.0f, 0.0f, 0.0f, 0.0f};
+                }
+            }
+    }
     if (p.LSE && half == 0) p.LSE[static_cast<int64_t>(plane) * L + q] = live ? m_run * LN2 + __logf(l_run + p.eps) : -INFINITY;
 }
 
@@ -272,9 +323,9 @@ int launch_flash(AttnParams p, hipStream_t stream) {
 
 using namespace ppmlhip;
 
-extern "C" int flash_attn_forward_hip(int B, int h, int L, int d, int causal, float scale, float softmax_eps, int Bc,
-                                      const float* Q, const float* K, const float* V, const float* bias,
-                                      float* O, float* LSE, ppml_hip_stream_t stream) {
+extern "C" int flash_attn_forward_ex_hip(int B, int h, int L, int d, int causal, float scale, float softmax_eps, int Bc,
+                                         const float* Q, const float* K, const float* V, const float* bias,
+                                         float* O, float* LSE, int layout, ppml_hip_stream_t stream) {
     if (!Q || !K || !V || !O || B <= 0 || h <= 0 || L <= 0 || d <= 0) {
         set_error("flash_attn_forward_hip: bad arguments (B=%d h=%d L=%d d=%d)", B, h, L, d);
         return RC_BAD_ARGS;
@@ -284,6 +335,7 @@ extern "C" int flash_attn_forward_hip(int B, int h, int L, int d, int causal, fl
         return RC_BAD_ARGS;
     }
     const auto misaligned = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15) != 0; };
+    if (layout < 0 || layout > 3) { set_error("flash_attn_forward_hip: layout %d is not 0..3", layout); return RC_BAD_ARGS; }
     if (misaligned(Q) || misaligned(K) || misaligned(V) || misaligned(O)) {
         set_error("flash_attn_forward_hip: Q, K, V and O must be 16-byte aligned");
         return RC_BAD_ARGS;
@@ -301,6 +353,8 @@ extern "C" int flash_attn_forward_hip(int B, int h, int L, int d, int causal, fl
     p.eps = softmax_eps;
     p.head = Bc > 0 ? Bc : 64;                        // FlashAttn.cpp:62
     p.stage_rows = 0;                                 // set per instance
+    p.in_ld = layout & 1;
+    p.out_ld = (layout >> 1) & 1;
     stats_record(static_cast<int64_t>(planes) * L, d, L);
     hipStream_t s = static_cast<hipStream_t>(stream);
     // Four-wave work-groups (128 queries): 824 planes of 256 queries make 1648 of them, which spread over
@@ -308,4 +362,10 @@ extern "C" int flash_attn_forward_hip(int B, int h, int L, int d, int causal, fl
     const bool short_rows = L <= 128;
     if (d <= 32) return short_rows ? launch_flash<32, 4, true>(p, s) : launch_flash<32, 4, false>(p, s);
     return short_rows ? launch_flash<64, 4, true>(p, s) : launch_flash<64, 4, false>(p, s);
+}
+
+extern "C" int flash_attn_forward_hip(int B, int h, int L, int d, int causal, float scale, float softmax_eps, int Bc,
+                                      const float* Q, const float* K, const float* V, const float* bias,
+                                      float* O, float* LSE, ppml_hip_stream_t stream) {
+    return flash_attn_forward_ex_hip(B, h, L, d, causal, scale, softmax_eps, Bc, Q, K, V, bias, O, LSE, 0, stream);
 }

@@ -18,6 +18,8 @@
 
 #include <cstring>
 #include <new>
+#include <unordered_map>
+#include <unordered_set>
 
 #include "../../include/ppml_hip.h"
 #include "../../include/ppml_hip_backend.h"
@@ -306,7 +308,9 @@ Status HipBackend::kernel_flash_attn_ext(Tensor* node) {
     const Tensor* v = node->src[2];
     if (!q || !k || !v || !q->data || !k->data || !v->data || !node->data)
         return fail(Status::NOT_SUPPORTED, "flash_attn_ext: unbound tensor");
-    const int64_t d = q->dims[0], L = q->dims[1], h = dim_or_1(q, 2), B = dim_or_1(q, 3);
+    // with the leading bridges fused away the sources are still [L, D, h, B]
+    const int64_t d = (attn_layout_ & 1) ? q->dims[1] : q->dims[0], L = (attn_layout_ & 1) ? q->dims[0] : q->dims[1];
+    const int64_t h = dim_or_1(q, 2), B = dim_or_1(q, 3);
     if (k->numel() != q->numel() || v->numel() != q->numel() || node->numel() != q->numel())
         return fail(Status::NOT_SUPPORTED, "flash_attn_ext: Q, K, V and O differ in size");
     const Tensor* bias = node->src[3];
@@ -315,11 +319,12 @@ Status HipBackend::kernel_flash_attn_ext(Tensor* node) {
     Tensor* lse = node->src[4];
     if (lse && lse->numel() != B * h * L) return fail(Status::NOT_SUPPORTED, "flash_attn_ext: LSE is not [L, h, B]");
     if (lse && !lse->data) return fail(Status::NOT_SUPPORTED, "flash_attn_ext: LSE buffer is unbound");
-    const int rc = flash_attn_forward_hip(static_cast<int>(B), static_cast<int>(h), static_cast<int>(L), static_cast<int>(d),
-                                          node->op_params[1] != 0, node->param_f32(0), node->param_f32(2), node->op_params[4],
-                                          static_cast<const float*>(q->data), static_cast<const float*>(k->data),
-                                          static_cast<const float*>(v->data), bias ? static_cast<const float*>(bias->data) : nullptr,
-                                          static_cast<float*>(node->data), lse ? static_cast<float*>(lse->data) : nullptr, nullptr);
+    const int rc = flash_attn_forward_ex_hip(static_cast<int>(B), static_cast<int>(h), static_cast<int>(L), static_cast<int>(d),
+                                             node->op_params[1] != 0, node->param_f32(0), node->param_f32(2), node->op_params[4],
+                                             static_cast<const float*>(q->data), static_cast<const float*>(k->data),
+                                             static_cast<const float*>(v->data), bias ? static_cast<const float*>(bias->data) : nullptr,
+                                             static_cast<float*>(node->data), lse ? static_cast<float*>(lse->data) : nullptr,
+                                             attn_layout_, nullptr);
     if (rc != 0) return fail(status_of_rc(rc), std::string("flash_attn_ext: ") + ppml_hip_last_error());
     return Status::SUCCESS;
 }
@@ -386,16 +391,82 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         return fail(Status::ABORTED, "cannot select device " + std::to_string(device_));
     }
     error_.clear();
+
+    // Optional fusion of the layout bridges around fused attention nodes (ComputeGraphHelper.cpp:456-458,
+    // 483): a permutation {1,0,2,3} that feeds only the attention node, or is the only reader of its result,
+    // is not executed; the attention kernel reads / writes that layout itself.  All three inputs fuse
+    // together or not at all.
+    struct Bridges { bool in = false; Tensor* out = nullptr; };
+    std::unordered_map<const Tensor*, Bridges> fused;
+    std::unordered_set<const Tensor*> skipped;
+    if (fuse_attention_bridges_) {
+        std::unordered_map<const Tensor*, int> uses, position;
+        std::unordered_map<const Tensor*, Tensor*> single_user;
+        int pos = 0;
+        for (Tensor* n : *graph) {
+            if (!n) continue;
+            position[n] = pos++;
+            for (Tensor* s : n->src) if (s) { ++uses[s]; single_user[s] = n; }
+        }
+        const auto is_bridge = [](const Tensor* t) {
+            if (!t || (t->op != OP_PERMUTE && t->op != OP_TRANSPOSE) || t->ndim != 4 || t->type != TENSOR_TYPE_F32) return false;
+            return t->op_params[0] == 1 && t->op_params[1] == 0 && t->op_params[2] == 2 && t->op_params[3] == 3 &&
+                   t->src[0] && t->src[0]->type == TENSOR_TYPE_F32 && t->src[0]->ndim == 4 && !t->view_src;
+        };
+        for (Tensor* n : *graph) {
+            if (!n || n->op != OP_FLASH_ATTN_EXT || !node_supported(n)) continue;
+            Bridges b;
+            b.in = true;
+            for (int s = 0; s < 3; ++s) {
+                const Tensor* pq = n->src[s];
+                b.in = b.in && is_bridge(pq) && uses[pq] == 1 && position.count(pq) && position[pq] < position[n];
+            }
+            // a tensor that feeds two of the three slots (self-attention on one projection) has uses == 2: not fused
+            Tensor* user = uses[n] == 1 ? single_user[n] : nullptr;
+            if (user && is_bridge(user) && user->src[0] == n && position.count(user) && position[user] > position[n])
+                b.out = user;
+            if (!b.in && !b.out) continue;
+            fused[n] = b;
+            if (b.in) for (int s = 0; s < 3; ++s) skipped.insert(n->src[s]);
+            if (b.out) skipped.insert(b.out);
+        }
+    }
+
     int index = -1;
     for (Tensor* node : *graph) {
         ++index;
         if (!node) return fail(Status::NOT_SUPPORTED, "null node " + std::to_string(index));
         if (node->op == OP_NONE || node->op == OP_VIEW || node->op == OP_RESHAPE) continue;
-        resolve_views(node);
+        if (skipped.count(node)) continue;
+
+        // no other backend to fall back to: an unsupported node ends the graph instead of being skipped
+        if (!supports_op(node))
+            return fail(Status::NOT_SUPPORTED, "op " + std::to_string(node->op) + " (node " + std::to_string(index) + ") is not supported");
+
+        // the node as it is executed: for a fused attention node a copy whose sources are the bridges'
+        // sources and whose storage is the trailing bridge's
+        Tensor rewired;
+        Tensor* exec = node;
+        Tensor* storage = node;
+        attn_layout_ = 0;
+        const auto plan = fused.find(node);
+        if (plan != fused.end()) {
+            rewired = *node;
+            exec = &rewired;
+            if (plan->second.in) {
+                for (int s = 0; s < 3; ++s) rewired.src[s] = node->src[s]->src[0];
+                attn_layout_ |= 1;
+            }
+            if (plan->second.out) {
+                storage = plan->second.out;
+                attn_layout_ |= 2;
+            }
+        }
+        resolve_views(exec);
 
         // single-backend mode: outputs nobody allocated get their own device buffer -- the node itself
         // and the second output the fused attention node carries in src[4] (its LSE buffer)
-        Tensor* outputs[2] = {node, node->op == OP_FLASH_ATTN_EXT ? node->src[4] : nullptr};
+        Tensor* outputs[2] = {storage, node->op == OP_FLASH_ATTN_EXT ? node->src[4] : nullptr};
         for (Tensor* out : outputs) {
             if (!out || skip_alloc_ || out->data) continue;
             const size_t need = out->nbytes();
@@ -406,19 +477,22 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
             out->buffer_offs = 0;
             owned_.push_back(std::move(buf));
         }
-        // no other backend to fall back to: an unsupported node ends the graph instead of being skipped
-        if (!supports_op(node))
-            return fail(Status::NOT_SUPPORTED, "op " + std::to_string(node->op) + " (node " + std::to_string(index) + ") is not supported");
+        if (storage != node) {
+            rewired.data = storage->data;
+            rewired.buffer = storage->buffer;
+            rewired.buffer_offs = storage->buffer_offs;
+        }
 
-        if (!device_pointer_ok(node))
+        if (!device_pointer_ok(exec))
             return fail(Status::NOT_SUPPORTED, "node " + std::to_string(index) + ": output is not device memory inside its buffer");
         for (int j = 0; j < 10; ++j) {
-            if (node->src[j] && !device_pointer_ok(node->src[j]))
+            if (exec->src[j] && !device_pointer_ok(exec->src[j]))
                 return fail(Status::NOT_SUPPORTED, "node " + std::to_string(index) + ": src" + std::to_string(j) +
                                                     " is not device memory inside its buffer");
         }
 
-        const Status st = dispatch_node(node);
+        const Status st = dispatch_node(exec);
+        attn_layout_ = 0;
         if (st != Status::SUCCESS) return st;
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess)
@@ -557,6 +631,9 @@ int ppml_hip_backend_pack_weight(ppml_hip_backend* b, ppml_hip_tensor* weight) {
 }
 void ppml_hip_backend_set_q8_1_activations(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_q8_1_activations(on != 0);
+}
+void ppml_hip_backend_set_fuse_attention_bridges(ppml_hip_backend* b, int on) {
+    if (b) b->impl.set_fuse_attention_bridges(on != 0);
 }
 void ppml_hip_backend_set_skip_alloc(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_skip_alloc(on != 0);

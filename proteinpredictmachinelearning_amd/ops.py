@@ -176,23 +176,27 @@ def tri_mul(left: torch.Tensor, right: torch.Tensor, D: int, I: int, J: int, K: 
 
 def flash_attn_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bias: torch.Tensor | None = None,
                        causal: bool = False, scale: float = 0.0, eps: float = 1e-9, Bc: int = 64,
-                       want_lse: bool = True):
+                       want_lse: bool = True, in_ld: bool = False, out_ld: bool = False):
     """Fused attention forward (include/ppml/FlashAttn.h:8-65): Q, K, V (B,h,L,d), bias (B,h,L,L) or None
-    -> O (B,h,L,d) and LSE (B,h,L) (None when not wanted)."""
+    -> O (B,h,L,d) and LSE (B,h,L) (None when not wanted).  in_ld: Q, K, V are (B,h,d,L) instead (the graph
+    tensors before their layout bridge); out_ld: O is returned as (B,h,d,L)."""
     q, k, v = _dev_f32(q, "q"), _dev_f32(k, "k"), _dev_f32(v, "v")
     if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
         raise ValueError("flash_attn_forward: Q, K and V must be 4-D tensors of one shape (B,h,L,d)")
     B, h, L, d = q.shape
+    if in_ld:
+        L, d = d, L
     if bias is not None:
         bias = _dev_f32(bias, "bias")
         if tuple(bias.shape) != (B, h, L, L):
             raise ValueError("flash_attn_forward: bias must be (B,h,L,L)")
-    o = torch.empty_like(q)
+    o = torch.empty((B, h, d, L) if out_ld else (B, h, L, d), dtype=torch.float32, device=q.device)
     lse = torch.empty((B, h, L), dtype=torch.float32, device=q.device) if want_lse else None
-    cabi.check("flash_attn_forward_hip",
-               _lib().flash_attn_forward_hip(B, h, L, d, int(causal), scale, eps, Bc, _ptr(q), _ptr(k), _ptr(v),
-                                             _ptr(bias) if bias is not None else None, _ptr(o),
-                                             _ptr(lse) if lse is not None else None, _stream()))
+    cabi.check("flash_attn_forward_ex_hip",
+               _lib().flash_attn_forward_ex_hip(B, h, L, d, int(causal), scale, eps, Bc, _ptr(q), _ptr(k), _ptr(v),
+                                                _ptr(bias) if bias is not None else None, _ptr(o),
+                                                _ptr(lse) if lse is not None else None,
+                                                int(in_ld) | (int(out_ld) << 1), _stream()))
     return o, lse
 
 

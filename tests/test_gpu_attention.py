@@ -160,3 +160,22 @@ def test_refused_arguments(ops):
     assert lib.flash_attn_forward_hip(1, 1, 0, 8, 0, 0.0, 1e-9, 64, p, p, p, None, p, None, None) == 1
     assert lib.flash_attn_forward_hip(1, 1, 4, 8, 0, 0.0, 1e-9, 64, None, p, p, None, p, None, None) == 1
     assert b"flash_attn_forward_hip" in lib.ppml_hip_last_error()
+
+
+@pytest.mark.parametrize("B,h,L,d,causal,use_bias", [(1, 3, 103, 32, False, True), (2, 2, 256, 32, False, True),
+                                                     (1, 2, 77, 20, True, False), (1, 1, 150, 64, False, True)])
+@pytest.mark.parametrize("in_ld,out_ld", [(True, True), (True, False), (False, True)])
+def test_layouts_without_the_bridges(ops, oracle, B, h, L, d, causal, use_bias, in_ld, out_ld):
+    """Q, K, V handed over as (B,h,d,L) and / or O wanted as (B,h,d,L): the graph tensors on either side of the
+    permutation copies the reference wraps around the node (ComputeGraphHelper.cpp:456-458, 483)."""
+    rng = np.random.default_rng(L + 7 * d)
+    q, k, v = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(3)]
+    bias = rng.standard_normal((B, h, L, L)).astype(np.float32) if use_bias else None
+    want_o, want_lse = oracle.flash_attn_forward(q, k, v, bias, causal=causal)
+    t = (lambda x: np.ascontiguousarray(x.transpose(0, 1, 3, 2))) if in_ld else (lambda x: x)
+    o, lse = ops.flash_attn_forward(_dev(t(q)), _dev(t(k)), _dev(t(v)), _dev(bias), causal=causal, in_ld=in_ld, out_ld=out_ld)
+    ops.synchronize()
+    got_o = o.cpu().numpy()
+    if out_ld:
+        got_o = got_o.transpose(0, 1, 3, 2)
+    _check(got_o, lse.cpu().numpy(), want_o, want_lse)

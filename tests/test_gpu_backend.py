@@ -209,6 +209,66 @@ def test_tri_mul_node(be, oracle):
     assert be.graph_compute([node]) == B.NOT_SUPPORTED
 
 
+def test_fused_attention_subgraph_without_its_bridges(oracle):
+    """The same six-node subgraph with set_fuse_attention_bridges(1): the four permutations are not executed
+    (their tensors stay unbound), the result equals the unfused run; a bridge with a second reader is kept."""
+    be2 = B.Backend(0)
+    rng = np.random.default_rng(10)
+    Bt, h, L, d = 2, 2, 70, 32
+    q, k, v = [rng.standard_normal((Bt, h, L, d)).astype(np.float32) for _ in range(3)]
+    bias = rng.standard_normal((Bt, h, L, L)).astype(np.float32)
+    want, want_lse = oracle.flash_attn_forward(q, k, v, bias)
+
+    def build(extra_reader):
+        leaves = [_leaf(be2, np.ascontiguousarray(x.transpose(0, 1, 3, 2))) for x in (q, k, v)]
+        perms = []
+        for t in leaves:
+            n = B.Tensor((d, L, h, Bt), B.F32, B.OP_PERMUTE, [t])
+            for i, a in enumerate((1, 0, 2, 3)):
+                n.set_param(i, a)
+            perms.append(n)
+        lse = B.Tensor((L, h, Bt))
+        flash = B.Tensor((d, L, h, Bt), B.F32, B.OP_FLASH_ATTN_EXT, perms + [_leaf(be2, bias), lse])
+        flash.set_param(0, float(1.0 / np.sqrt(d))).set_param(1, 0).set_param(2, 1e-9).set_param(3, 64).set_param(4, 64)
+        out = B.Tensor((L, d, h, Bt), B.F32, B.OP_PERMUTE, [flash])
+        for i, a in enumerate((1, 0, 2, 3)):
+            out.set_param(i, a)
+        nodes = perms + [flash, out]
+        if extra_reader:                                # a second reader of the permuted Q: its bridge must run
+            again = B.Tensor((L, d, h, Bt), B.F32, B.OP_PERMUTE, [perms[0]])
+            for i, a in enumerate((1, 0, 2, 3)):
+                again.set_param(i, a)
+            nodes.append(again)
+        return leaves, perms, flash, lse, out, nodes
+
+    be2.set_fuse_attention_bridges(True)
+    leaves, perms, flash, lse, out, nodes = build(False)
+    assert be2.graph_compute(nodes) == B.SUCCESS, be2.last_error
+    be2.synchronize()
+    got = be2.download(out).reshape(Bt, h, d, L).transpose(0, 1, 3, 2)
+    assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+    assert np.abs(be2.download(lse).reshape(Bt, h, L) - want_lse).max() <= 1e-5 * (1 + np.abs(want_lse).max())
+    with pytest.raises(RuntimeError):
+        be2.download(perms[0])                          # never allocated: the bridge was not executed
+    with pytest.raises(RuntimeError):
+        be2.download(flash)
+
+    leaves, perms, flash, lse, out, nodes = build(True)
+    assert be2.graph_compute(nodes) == B.SUCCESS, be2.last_error
+    be2.synchronize()
+    assert np.array_equal(be2.download(perms[0]).reshape(Bt, h, L, d), q)      # inputs not fused this time
+    got = be2.download(out).reshape(Bt, h, d, L).transpose(0, 1, 3, 2)            # the trailing bridge still is
+    assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+    assert np.array_equal(be2.download(nodes[-1]).reshape(Bt, h, d, L), q.transpose(0, 1, 3, 2))
+
+    be2.set_fuse_attention_bridges(False)
+    leaves, perms, flash, lse, out, nodes = build(False)
+    assert be2.graph_compute(nodes) == B.SUCCESS, be2.last_error
+    be2.synchronize()
+    assert np.array_equal(be2.download(perms[1]).reshape(Bt, h, L, d), k)
+    assert np.abs(be2.download(flash).reshape(Bt, h, L, d) - want).max() <= 1e-4 * np.abs(want).max()
+
+
 def test_view_sources_are_resolved_and_noop_nodes_skipped(be, oracle):
     # a reshape node built with only src[0] set, and an offset view with view_src set, both feed a
     # mul_mat (src/backend/CUDABackend.cpp:800-819)
