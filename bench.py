@@ -116,10 +116,10 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8 x int8 -> int32, f32 scale settlement",
+        "dtype": "int8",
         "data": "synthetic (seeded normal draws made on the device)",
         "config": {"workload": "MSA-track QKV Q8_0 linear: X 26368x256 f32 -> Q8_0 on the fly, "
-                               "W 768x256 Q8_0, Y 26368x768 f32 (BASELINE configs[2])",
+                               "W 768x256 Q8_0, Y 26368x768 f32",
                    "buffer_rotation": nsets, "weight_layout": "Q8_0M (MFMA fragments)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,

@@ -189,7 +189,7 @@ def test_status_codes(ops):
         ops.mul_mat_q8(ops.Q8Weight(buf.view(torch.uint8)[:34 * 4], 4, 32, 0), torch.zeros(3, 64, device="cuda"))
 
 
-# ----------------------------------------------------------------------------- BASELINE shapes
+# ----------------------------------------------------------------------------- the configured full-size shapes
 def test_pair_feed_forward_shapes_full(ops, oracle):
     # X 10609 x 128 -> 512 -> ReLU -> 128, both layers checked against the oracle in full
     x, w1 = _inputs(103, 10609, 128, 512)
