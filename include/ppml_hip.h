@@ -147,6 +147,14 @@ int tri_mul_hip(const float *left, const float *right, float *dst,
                 int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float inv_L, int outgoing,
                 ppml_hip_stream_t stream);
 
+/* replaces tri_mul_back_cuda (src/cuda/PairKernels.cu:525-560, declared src/backend/CUDAKernels.cpp:320-323),
+ * mathematics of CPUBackend::kernel_tri_mul_back (src/backend/CPUKernels.cpp:1238-1367): the gradients of
+ * tri_mul_hip's two operands, each 1/L times a contraction of grad [D,I,J,B] with the other operand; gleft or
+ * gright may be NULL (skipped), not both.  No finite guard here, as in the reference. */
+int tri_mul_back_hip(const float *grad, const float *left, const float *right, float *gleft, float *gright,
+                     int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float inv_L, int outgoing,
+                     ppml_hip_stream_t stream);
+
 /* ---- fused attention forward ------------------------------------------------------------------ */
 /* replaces flash_attn_forward_cuda (declared src/backend/CUDAKernels.cpp:174, contract
  * include/ppml/FlashAttn.h:8-65, called from kernel_flash_attn_ext_cuda, CUDAKernels.cpp:894-903);

@@ -39,6 +39,7 @@ enum TensorOp : int {
     OP_TRANSPOSE = 40,
     OP_FLASH_ATTN_EXT = 75,
     OP_TRI_MUL = 100,
+    OP_TRI_MUL_BACK = 101,
     OP_OUTER_PROD_MEAN = 102,
 };
 
@@ -112,7 +113,7 @@ private:
 using ComputeGraph = std::vector<Tensor*>;   // nodes in evaluation order
 
 // src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-416 (OP_OUTER_PROD_MEAN),
-// 113-119 (OP_PERMUTE, OP_TRANSPOSE), 395-402 (OP_TRI_MUL), 457-463 (OP_FLASH_ATTN_EXT); a function of the node alone, so it can be asked without a device
+// 113-119 (OP_PERMUTE, OP_TRANSPOSE), 395-409 (OP_TRI_MUL, OP_TRI_MUL_BACK), 457-463 (OP_FLASH_ATTN_EXT); a function of the node alone, so it can be asked without a device
 bool node_supported(const Tensor* node);
 
 // include/ppml/Backend.h:550-605; executor obligations of src/backend/CUDABackend.cpp:708-1086
@@ -154,6 +155,7 @@ private:
     Status kernel_flash_attn_ext(Tensor* node);
     Status kernel_permute(Tensor* node);
     Status kernel_tri_mul(Tensor* node);
+    Status kernel_tri_mul_back(Tensor* node);
     bool resolve_views(Tensor* node);                    // src/backend/CUDABackend.cpp:800-819
     bool device_pointer_ok(const Tensor* t) const;       // src/backend/CUDABackend.cpp:894-973
     Status fail(Status s, const std::string& why);

@@ -78,6 +78,8 @@ def _load() -> C.CDLL:
     lib.orc_flash_attn_forward.argtypes = ([C.c_int] * 5 + [C.c_float, C.c_float, C.c_int] + [f32p] * 6 + [C.c_int])
     lib.orc_tri_mul.restype = None
     lib.orc_tri_mul.argtypes = [f32p, f32p, f32p] + [i64] * 5 + [C.c_float, C.c_int, C.c_int]
+    lib.orc_tri_mul_back.restype = None
+    lib.orc_tri_mul_back.argtypes = [f32p] * 5 + [i64] * 5 + [C.c_float, C.c_int, C.c_int]
     lib.orc_permute.restype = C.c_int
     lib.orc_permute.argtypes = [f32p, f32p, C.c_int, C.POINTER(C.c_int32), C.POINTER(i64), C.POINTER(i64)]
     lib.orc_max_threads.restype = C.c_int
@@ -379,3 +381,14 @@ def tri_mul(left, right, D, I, J, K, B, L, outgoing=True, nthreads=0) -> np.ndar
     out = np.empty(D * I * J * B, dtype=np.float32)
     lib().orc_tri_mul(_fp(left), _fp(right), _fp(out), D, I, J, K, B, L, int(outgoing), nthreads or max_threads())
     return out
+
+
+def tri_mul_back(grad, left, right, D, I, J, K, B, L, outgoing=True, nthreads=0):
+    """kernel_tri_mul_back (CPUKernels.cpp:1238-1367): returns (gleft, gright), flat, shaped like left and right."""
+    grad, left, right = _f32(grad).reshape(-1), _f32(left).reshape(-1), _f32(right).reshape(-1)
+    assert grad.size == D * I * J * B and left.size == D * I * K * B and right.size == D * J * K * B
+    gl = np.empty(D * I * K * B, dtype=np.float32)
+    gr = np.empty(D * J * K * B, dtype=np.float32)
+    lib().orc_tri_mul_back(_fp(grad), _fp(left), _fp(right), _fp(gl), _fp(gr), D, I, J, K, B, L, int(outgoing),
+                           nthreads or max_threads())
+    return gl, gr

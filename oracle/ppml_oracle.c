@@ -29,6 +29,8 @@
  *   orc_tri_mul : numpy einsum over the layout stated at src/backend/CPUKernels.cpp:895-903 (outgoing and
  *       incoming), exact on small integers; the finite guard on planted NaN / Inf / 1e5 values.  No
  *       reference-held vector covers it.
+ *   orc_tri_mul_back : numpy einsum (exact on small integers) and the adjoint identity
+ *       <grad, tri_mul(l, r)> = <gleft, l> = <gright, r> against orc_tri_mul, both forms.
  *   orc_permute : numpy.transpose with the axes translated (dst dim p = src dim axes[p], dims[0]
  *       innermost), identity and inverse permutations, hand-checked 2 x 3 case.
  *   orc_flash_attn_forward : the reference's own src/ops/FlashAttn.cpp compiled as-is
@@ -147,6 +149,48 @@ void orc_tri_mul(const float *left, const float *right, float *dst,
         float v = sum * inv_L;
         if (!(v == v) || v > 1e4f || v < -1e4f) v = (v != v) ? 0.0f : (v > 1e4f ? 1e4f : -1e4f);
         dst[idx] = v;
+    }
+}
+
+/* src/backend/CPUKernels.cpp:1238-1367: four index decodes, each output one sequential binary32 sum
+ * (j ascending for gleft, i ascending for gright) times 1/L. */
+void orc_tri_mul_back(const float *grad, const float *left, const float *right, float *gleft, float *gright,
+                      int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float L, int outgoing, int nthreads) {
+    const float inv_L = 1.0f / L;
+    if (nthreads <= 0) nthreads = 1;
+    if (gleft) {
+        const int64_t total = D * I * K * B;
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+        for (int64_t idx = 0; idx < total; ++idx) {
+            int64_t tmp = idx, i, k, d;
+            const int64_t b = tmp % B; tmp /= B;
+            if (outgoing) { k = tmp % K; tmp /= K; i = tmp % I; d = tmp / I; }      /* gleft [d,i,k,b] */
+            else          { i = tmp % I; tmp /= I; k = tmp % K; d = tmp / K; }      /* gleft [d,k,i,b] */
+            float sum = 0.0f;
+            for (int64_t j = 0; j < J; ++j) {
+                const float gv = grad[((d * I + i) * J + j) * B + b];
+                const float rv = outgoing ? right[((d * J + j) * K + k) * B + b] : right[((d * K + k) * J + j) * B + b];
+                sum += gv * rv;
+            }
+            gleft[idx] = sum * inv_L;
+        }
+    }
+    if (gright) {
+        const int64_t total = D * J * K * B;
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+        for (int64_t idx = 0; idx < total; ++idx) {
+            int64_t tmp = idx, j, k, d;
+            const int64_t b = tmp % B; tmp /= B;
+            if (outgoing) { k = tmp % K; tmp /= K; j = tmp % J; d = tmp / J; }      /* gright [d,j,k,b] */
+            else          { j = tmp % J; tmp /= J; k = tmp % K; d = tmp / K; }      /* gright [d,k,j,b] */
+            float sum = 0.0f;
+            for (int64_t i = 0; i < I; ++i) {
+                const float gv = grad[((d * I + i) * J + j) * B + b];
+                const float lv = outgoing ? left[((d * I + i) * K + k) * B + b] : left[((d * K + k) * I + i) * B + b];
+                sum += gv * lv;
+            }
+            gright[idx] = sum * inv_L;
+        }
     }
 }
 

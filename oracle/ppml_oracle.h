@@ -98,6 +98,11 @@ int orc_flash_attn_forward(int B, int h, int L, int d, int causal, float scale, 
 void orc_tri_mul(const float *left, const float *right, float *dst,
                  int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float L, int outgoing, int nthreads);
 
+/* src/backend/CPUKernels.cpp:1238-1367 (kernel_tri_mul_back): gleft has left's shape, gright right's;
+ * either may be NULL here (the CPU kernel wants both, the CUDA wrapper accepts one). */
+void orc_tri_mul_back(const float *grad, const float *left, const float *right, float *gleft, float *gright,
+                      int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float L, int outgoing, int nthreads);
+
 /* src/backend/CPUKernels.cpp:1669-1717 (kernel_permute): dimension p of dst is dimension axes[p] of src;
  * sd = source sizes, dd = destination sizes (dims[0] innermost), entries past ndim ignored.
  * returns 0 ok, 1 when an axis is outside [0, ndim) -- the reference prints and leaves dst untouched. */

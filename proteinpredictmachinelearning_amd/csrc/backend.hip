@@ -157,6 +157,11 @@ bool node_supported(const Tensor* node) {
             if (!src0 || !src1) return false;
             if (src0->type != TENSOR_TYPE_F32 || src1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32) return false;
             return src0->ndim == 4 && src1->ndim == 4 && node->ndim == 4;
+        case OP_TRI_MUL_BACK:
+            // src/backend/CUDABackend.cpp:404-409: grad, left, right present, at least one of the two outputs
+            if (!src0 || !src1 || !node->src[2]) return false;
+            if (!node->src[3] && !node->src[4]) return false;
+            return src0->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32;
         case OP_PERMUTE:
         case OP_TRANSPOSE:
             // src/backend/CUDABackend.cpp:113-119
@@ -371,6 +376,31 @@ Status HipBackend::kernel_tri_mul(Tensor* node) {
     return Status::SUCCESS;
 }
 
+// src/backend/CUDAKernels.cpp:1172-1201: src 0 grad [D,I,J,B], 1 left, 2 right, 3 gradient of left (or null),
+// 4 gradient of right (or null); L and the outgoing flag as in the forward node.
+Status HipBackend::kernel_tri_mul_back(Tensor* node) {
+    const Tensor* g = node->src[0];
+    const Tensor* l = node->src[1];
+    const Tensor* r = node->src[2];
+    Tensor* gl = node->src[3];
+    Tensor* gr = node->src[4];
+    if (!g || !l || !r || !g->data || !l->data || !r->data || (!gl && !gr) || (gl && !gl->data) || (gr && !gr->data))
+        return fail(Status::NOT_SUPPORTED, "tri_mul_back: unbound tensor");
+    const float L = node->param_f32(0);
+    const bool outgoing = (node->op_params[4] & 0xff) != 0;
+    if (L == 0.0f) return fail(Status::NOT_SUPPORTED, "tri_mul_back: L is zero");
+    const int64_t D = l->dims[0], B = l->dims[3];
+    const int64_t I = outgoing ? l->dims[1] : l->dims[2], J = outgoing ? r->dims[1] : r->dims[2];
+    const int64_t K = outgoing ? l->dims[2] : l->dims[1];
+    if (g->numel() != D * I * J * B || r->numel() != D * J * K * B || (gl && gl->numel() != l->numel()) || (gr && gr->numel() != r->numel()))
+        return fail(Status::NOT_SUPPORTED, "tri_mul_back: tensor sizes do not match each other");
+    const int rc = tri_mul_back_hip(static_cast<const float*>(g->data), static_cast<const float*>(l->data),
+                                    static_cast<const float*>(r->data), gl ? static_cast<float*>(gl->data) : nullptr,
+                                    gr ? static_cast<float*>(gr->data) : nullptr, D, I, J, K, B, 1.0f / L, outgoing ? 1 : 0, nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("tri_mul_back: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
 Status HipBackend::dispatch_node(Tensor* node) {
     switch (node->op) {
         case OP_MUL_MAT: return kernel_mul_mat(node);
@@ -380,6 +410,7 @@ Status HipBackend::dispatch_node(Tensor* node) {
         case OP_PERMUTE:
         case OP_TRANSPOSE: return kernel_permute(node);
         case OP_TRI_MUL: return kernel_tri_mul(node);
+        case OP_TRI_MUL_BACK: return kernel_tri_mul_back(node);
         default: return fail(Status::NOT_SUPPORTED, "no kernel for op " + std::to_string(node->op));
     }
 }
@@ -466,7 +497,9 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
 
         // single-backend mode: outputs nobody allocated get their own device buffer -- the node itself
         // and the second output the fused attention node carries in src[4] (its LSE buffer)
-        Tensor* outputs[2] = {storage, node->op == OP_FLASH_ATTN_EXT ? node->src[4] : nullptr};
+        // (the backward node of the triangle multiplication carries both of its outputs in src[3] and src[4])
+        Tensor* outputs[3] = {storage, node->op == OP_FLASH_ATTN_EXT || node->op == OP_TRI_MUL_BACK ? node->src[4] : nullptr,
+                              node->op == OP_TRI_MUL_BACK ? node->src[3] : nullptr};
         for (Tensor* out : outputs) {
             if (!out || skip_alloc_ || out->data) continue;
             const size_t need = out->nbytes();

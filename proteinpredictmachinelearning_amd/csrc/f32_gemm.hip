@@ -406,3 +406,40 @@ extern "C" int tri_mul_hip(const float* left, const float* right, float* dst,
     p.clamp = 1;
     return launch_gemm(p, static_cast<hipStream_t>(stream), "tri_mul_hip");
 }
+
+extern "C" int tri_mul_back_hip(const float* grad, const float* left, const float* right, float* gleft, float* gright,
+                                int64_t D, int64_t I, int64_t J, int64_t K, int64_t B, float inv_L, int outgoing,
+                                ppml_hip_stream_t stream) {
+    if (!grad || !left || !right || (!gleft && !gright) || D <= 0 || I <= 0 || J <= 0 || K <= 0 || B <= 0 ||
+        I > 0x7fffffff || J > 0x7fffffff || K > 0x7fffffff || D > 0x7fffffff || B > 0x7fffffff) {
+        set_error("tri_mul_back_hip: bad arguments"); return RC_BAD_ARGS;
+    }
+    // Per (d, b) plane, with grad[i][j] = grad[((d*I+i)*J+j)*B+b]:
+    //   outgoing  gleft[i][k]  = sum_j grad[i][j] * right[j][k]     gright[j][k] = sum_i grad[i][j] * left[i][k]
+    //   incoming  gleft[k][i]  = sum_j grad[i][j] * right[k][j]     gright[k][j] = sum_i grad[i][j] * left[k][i]
+    // Every one is a contraction with one stride per operand index, i.e. a launch of the strided kernel.
+    const auto launch = [&](const float* a, int64_t a_rs, int64_t a_ks, const float* b, int64_t b_rs, int64_t b_ks,
+                            float* c, int64_t c_mi, int64_t c_ni, int64_t M, int64_t N, int64_t Kc,
+                            int64_t a_p3, int64_t b_p3, int64_t c_p3) {
+        stats_record(M, Kc, N);
+        GemmParams p = plain_params();
+        p.A = a; p.B = b; p.C = c;
+        p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(Kc);
+        p.a_rs = a_rs * B; p.a_ks = a_ks * B; p.b_rs = b_rs * B; p.b_ks = b_ks * B;
+        p.c_mi = c_mi * B; p.c_ni = c_ni * B;
+        p.np2 = static_cast<int>(B); p.np3 = static_cast<int>(D);
+        p.a_p2 = 1; p.b_p2 = 1; p.c_p2 = 1;
+        p.a_p3 = a_p3 * B; p.b_p3 = b_p3 * B; p.c_p3 = c_p3 * B;
+        p.alpha = inv_L;
+        return launch_gemm(p, static_cast<hipStream_t>(stream), "tri_mul_back_hip");
+    };
+    int rc = RC_OK;
+    if (outgoing) {
+        if (gleft)  rc = launch(grad, J, 1, right, 1, K, gleft, K, 1, I, K, J, I * J, J * K, I * K);
+        if (rc == RC_OK && gright) rc = launch(grad, 1, J, left, 1, K, gright, K, 1, J, K, I, I * J, I * K, J * K);
+    } else {
+        if (gleft)  rc = launch(grad, J, 1, right, J, 1, gleft, 1, I, I, K, J, I * J, K * J, K * I);
+        if (rc == RC_OK && gright) rc = launch(grad, 1, J, left, I, 1, gright, 1, J, J, K, I, I * J, K * I, K * J);
+    }
+    return rc;
+}

@@ -174,6 +174,22 @@ def tri_mul(left: torch.Tensor, right: torch.Tensor, D: int, I: int, J: int, K: 
     return out
 
 
+def tri_mul_back(grad: torch.Tensor, left: torch.Tensor, right: torch.Tensor, D: int, I: int, J: int, K: int, B: int,
+                 L: float, outgoing: bool = True, want_left: bool = True, want_right: bool = True):
+    """Gradients of tri_mul's operands (src/backend/CPUKernels.cpp:1238-1367); flat tensors, same indexing."""
+    grad, left, right = _dev_f32(grad, "grad"), _dev_f32(left, "left"), _dev_f32(right, "right")
+    if L == 0 or not (want_left or want_right):
+        raise ValueError("tri_mul_back: L must not be zero and at least one gradient must be wanted")
+    if grad.numel() != D * I * J * B or left.numel() != D * I * K * B or right.numel() != D * J * K * B:
+        raise ValueError("tri_mul_back: operand size does not match D, I, J, K, B")
+    gl = torch.empty(D * I * K * B, dtype=torch.float32, device=grad.device) if want_left else None
+    gr = torch.empty(D * J * K * B, dtype=torch.float32, device=grad.device) if want_right else None
+    cabi.check("tri_mul_back_hip",
+               _lib().tri_mul_back_hip(_ptr(grad), _ptr(left), _ptr(right), _ptr(gl) if gl is not None else None,
+                                       _ptr(gr) if gr is not None else None, D, I, J, K, B, 1.0 / float(L), int(outgoing), _stream()))
+    return gl, gr
+
+
 def flash_attn_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bias: torch.Tensor | None = None,
                        causal: bool = False, scale: float = 0.0, eps: float = 1e-9, Bc: int = 64,
                        want_lse: bool = True, in_ld: bool = False, out_ld: bool = False):

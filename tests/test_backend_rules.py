@@ -109,3 +109,13 @@ def test_supports_op_tri_mul():
     assert not B.supports_op(B.Tensor((8, 5, 4, 1), B.F32, B.OP_TRI_MUL, [l]))
     assert not B.supports_op(B.Tensor((8, 5, 4), B.F32, B.OP_TRI_MUL, [l, r]))
     assert not B.supports_op(B.Tensor((8, 5, 4, 1), B.F32, B.OP_TRI_MUL, [B.Tensor((8, 5, 6, 1), B.F16), r]))
+
+
+def test_supports_op_tri_mul_back():
+    # src/backend/CUDABackend.cpp:404-409
+    g, l, r = B.Tensor((8, 5, 4, 1)), B.Tensor((8, 5, 6, 1)), B.Tensor((8, 4, 6, 1))
+    gl, gr = B.Tensor((8, 5, 6, 1)), B.Tensor((8, 4, 6, 1))
+    assert B.supports_op(B.Tensor((1,), B.F32, B.OP_TRI_MUL_BACK, [g, l, r, gl, gr]))
+    assert B.supports_op(B.Tensor((1,), B.F32, B.OP_TRI_MUL_BACK, [g, l, r, None, gr]))
+    assert not B.supports_op(B.Tensor((1,), B.F32, B.OP_TRI_MUL_BACK, [g, l, r]))
+    assert not B.supports_op(B.Tensor((1,), B.F32, B.OP_TRI_MUL_BACK, [g, l, None, gl, gr]))

@@ -269,6 +269,49 @@ def test_fused_attention_subgraph_without_its_bridges(oracle):
     assert np.abs(be2.download(flash).reshape(Bt, h, L, d) - want).max() <= 1e-4 * np.abs(want).max()
 
 
+def test_tri_mul_back_node(be, oracle):
+    # src/backend/CUDAKernels.cpp:1172-1201: outputs live in src[3] / src[4]; unbound ones are allocated here
+    rng = np.random.default_rng(13)
+    D, I, J, K, Bt = 3, 9, 7, 11, 1
+    for outgoing in (True, False):
+        ldims = (D, I, K, Bt) if outgoing else (D, K, I, Bt)
+        rdims = (D, J, K, Bt) if outgoing else (D, K, J, Bt)
+        left = rng.standard_normal(D * I * K * Bt).astype(np.float32)
+        right = rng.standard_normal(D * J * K * Bt).astype(np.float32)
+        grad = rng.standard_normal(D * I * J * Bt).astype(np.float32)
+        gl, gr = B.Tensor(ldims), B.Tensor(rdims)
+        node = B.Tensor((1,), B.F32, B.OP_TRI_MUL_BACK, [_leaf(be, grad, dims=(D, I, J, Bt)), _leaf(be, left, dims=ldims),
+                                                         _leaf(be, right, dims=rdims), gl, gr])
+        node.set_param(0, float(K)).set_param(4, int(outgoing))
+        assert be.graph_compute([node]) == B.SUCCESS, be.last_error
+        want_l, want_r = oracle.tri_mul_back(grad, left, right, D, I, J, K, Bt, float(K), outgoing)
+        assert np.abs(be.download(gl) - want_l).max() <= 1e-4 * np.abs(want_l).max()
+        assert np.abs(be.download(gr) - want_r).max() <= 1e-4 * np.abs(want_r).max()
+
+
+def test_backward_gemms_of_mul_mat_as_the_reference_builds_them(be, oracle):
+    """ComputeGraph.cpp:708-741: for y = mul_mat(A, W) (A dims [K,M], W dims [K,N], y dims [N,M]) the gradients are
+    dA = mul_mat(grad, mat_transpose(W)) and dW = mul_mat(mat_transpose(grad), mat_transpose(A)), where
+    mat_transpose is a permutation copy: five nodes, all on this backend.  Checked against grad @ W and grad^T @ A."""
+    rng = np.random.default_rng(14)
+    M, K, N = 37, 24, 19
+    A = rng.integers(-3, 4, size=(M, K)).astype(np.float32)       # dims [K, M]
+    W = rng.integers(-3, 4, size=(N, K)).astype(np.float32)       # dims [K, N]
+    G = rng.integers(-3, 4, size=(M, N)).astype(np.float32)       # dims [N, M]
+    a, w, g = _leaf(be, A), _leaf(be, W), _leaf(be, G)
+
+    def mat_t(t, dims):
+        n = B.Tensor(dims, B.F32, B.OP_PERMUTE, [t])
+        n.set_param(0, 1).set_param(1, 0)
+        return n
+    wt, gt, at = mat_t(w, (N, K)), mat_t(g, (M, N)), mat_t(a, (M, K))
+    dA = B.Tensor((K, M), B.F32, B.OP_MUL_MAT, [g, wt])          # mul_mat(a, b): dims [b.dims[1], a.dims[1]]
+    dW = B.Tensor((K, N), B.F32, B.OP_MUL_MAT, [gt, at])
+    assert be.graph_compute([wt, dA, gt, at, dW]) == B.SUCCESS, be.last_error
+    assert np.array_equal(be.download(dA).reshape(M, K), G @ W)
+    assert np.array_equal(be.download(dW).reshape(N, K), G.T @ A)
+
+
 def test_view_sources_are_resolved_and_noop_nodes_skipped(be, oracle):
     # a reshape node built with only src[0] set, and an offset view with view_src set, both feed a
     # mul_mat (src/backend/CUDABackend.cpp:800-819)

@@ -251,3 +251,29 @@ def test_tri_mul_finite_guard(ops, oracle):
     got = ops.tri_mul(_dev(left.reshape(-1)), _dev(right.reshape(-1)), 1, 4, 1, 2, 1, 2.0, True).cpu().numpy()
     assert got.tolist() == [0.0, 1e4, -1e4, 9.5e3]
     assert got.tolist() == oracle.tri_mul(left, right, 1, 4, 1, 2, 1, 2.0, True).tolist()
+
+
+@pytest.mark.parametrize("D,I,J,K,Bt,outgoing", [
+    (3, 5, 4, 6, 2, True), (3, 5, 4, 6, 2, False),
+    (8, 103, 103, 103, 1, True), (8, 103, 103, 103, 1, False),
+    (2, 130, 70, 33, 1, True), (2, 130, 70, 33, 1, False),
+])
+def test_tri_mul_back(ops, oracle, D, I, J, K, Bt, outgoing):
+    rng = np.random.default_rng(D * 100 + K)
+    left = rng.standard_normal(D * I * K * Bt).astype(np.float32)
+    right = rng.standard_normal(D * J * K * Bt).astype(np.float32)
+    grad = rng.standard_normal(D * I * J * Bt).astype(np.float32)
+    L = float(K)
+    want_l, want_r = oracle.tri_mul_back(grad, left, right, D, I, J, K, Bt, L, outgoing)
+    gl, gr = ops.tri_mul_back(_dev(grad), _dev(left), _dev(right), D, I, J, K, Bt, L, outgoing)
+    _check(gl.cpu().numpy(), want_l)
+    _check(gr.cpu().numpy(), want_r)
+    # one output only, and exactness on small integers
+    gi = rng.integers(-3, 4, size=grad.size).astype(np.float32)
+    li = rng.integers(-3, 4, size=left.size).astype(np.float32)
+    ri = rng.integers(-3, 4, size=right.size).astype(np.float32)
+    wl, wr = oracle.tri_mul_back(gi, li, ri, D, I, J, K, Bt, 4.0, outgoing)
+    gl, none = ops.tri_mul_back(_dev(gi), _dev(li), _dev(ri), D, I, J, K, Bt, 4.0, outgoing, want_right=False)
+    assert none is None and np.array_equal(gl.cpu().numpy(), wl)
+    none, gr = ops.tri_mul_back(_dev(gi), _dev(li), _dev(ri), D, I, J, K, Bt, 4.0, outgoing, want_left=False)
+    assert none is None and np.array_equal(gr.cpu().numpy(), wr)

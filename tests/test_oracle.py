@@ -629,3 +629,24 @@ def test_tri_mul_against_einsum_and_the_finite_guard(oracle):
     l1[0, 3, 0, 0] = 1.9e4        # 9.5e3 stays
     got = oracle.tri_mul(l1, r1, 1, 4, 1, 2, 1, 2.0, True)
     assert got.tolist() == [0.0, 1e4, -1e4, 9.5e3]
+
+
+def test_tri_mul_back_against_einsum_and_the_adjoint_identity(oracle):
+    rng = np.random.default_rng(22)
+    D, I, J, K, Bt, L = 2, 5, 4, 6, 3, 4.0
+    for outgoing, ls, rs, gl_eq, gr_eq, f_eq in [
+        (True, (D, I, K, Bt), (D, J, K, Bt), "dijb,djkb->dikb", "dijb,dikb->djkb", "dikb,djkb->dijb"),
+        (False, (D, K, I, Bt), (D, K, J, Bt), "dijb,dkjb->dkib", "dijb,dkib->dkjb", "dkib,dkjb->dijb"),
+    ]:
+        left = rng.integers(-3, 4, size=ls).astype(np.float32)
+        right = rng.integers(-3, 4, size=rs).astype(np.float32)
+        grad = rng.integers(-3, 4, size=(D, I, J, Bt)).astype(np.float32)
+        gl, gr = oracle.tri_mul_back(grad, left, right, D, I, J, K, Bt, L, outgoing)
+        g64, l64, r64 = grad.astype(np.float64), left.astype(np.float64), right.astype(np.float64)
+        assert np.array_equal(gl.reshape(ls), np.einsum(gl_eq, g64, r64) / L), outgoing
+        assert np.array_equal(gr.reshape(rs), np.einsum(gr_eq, g64, l64) / L), outgoing
+        # adjoint of the forward map (which the einsum above does not know about): <grad, f(l, r)> = <gleft, l> = <gright, r>
+        fwd = oracle.tri_mul(left, right, D, I, J, K, Bt, L, outgoing).astype(np.float64)
+        assert np.array_equal(fwd.reshape(D, I, J, Bt), np.einsum(f_eq, l64, r64) / L)
+        lhs = float((g64.reshape(-1) * fwd).sum())
+        assert lhs == float((gl.astype(np.float64) * l64.reshape(-1)).sum()) == float((gr.astype(np.float64) * r64.reshape(-1)).sum())
