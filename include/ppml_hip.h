@@ -129,6 +129,13 @@ int out_prod_scaled_hip(const float *src0, const float *src1, float *dst,
 int outer_prod_mean_hip(const float *left, const float *right, float *dst,
                         int64_t D, int64_t L, int64_t N, int64_t B, float inv_N,
                         ppml_hip_stream_t stream);
+/* replaces outer_prod_mean_back_cuda (declared src/backend/CUDAKernels.cpp:327-330), mathematics of
+ * CPUBackend::kernel_outer_prod_mean_back (src/backend/CPUKernels.cpp:1034-1105): grad [D*D,L,L,B], left and
+ * right [D,L,N,B] -> gleft, gright [D,L,N,B] (either may be NULL, not both):
+ *   gleft[d1,i,n,b]  = inv_N * sum_{j,d2} grad[(d1*D+d2),i,j,b] * right[d2,j,n,b]
+ *   gright[d2,j,n,b] = inv_N * sum_{i,d1} grad[(d1*D+d2),i,j,b] * left[d1,i,n,b] */
+int outer_prod_mean_back_hip(const float *grad, const float *left, const float *right, float *gleft, float *gright,
+                             int64_t D, int64_t L, int64_t N, int64_t B, float inv_N, ppml_hip_stream_t stream);
 /* value-form outer product mean (src/ops/MathUtils.cpp:387-437):
  * left/right (B,N,L,D) -> dst (B,L,L,D*D), i.e. dst = A^T B / N per batch. */
 int outer_product_mean_value_hip(const float *left, const float *right, float *dst,

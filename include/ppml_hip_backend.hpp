@@ -41,6 +41,7 @@ enum TensorOp : int {
     OP_TRI_MUL = 100,
     OP_TRI_MUL_BACK = 101,
     OP_OUTER_PROD_MEAN = 102,
+    OP_OUTER_PROD_MEAN_BACK = 103,
 };
 
 // include/ppml/Backend.h:168-173
@@ -112,7 +113,7 @@ private:
 
 using ComputeGraph = std::vector<Tensor*>;   // nodes in evaluation order
 
-// src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-416 (OP_OUTER_PROD_MEAN),
+// src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-421 (OP_OUTER_PROD_MEAN, OP_OUTER_PROD_MEAN_BACK),
 // 113-119 (OP_PERMUTE, OP_TRANSPOSE), 395-409 (OP_TRI_MUL, OP_TRI_MUL_BACK), 457-463 (OP_FLASH_ATTN_EXT); a function of the node alone, so it can be asked without a device
 bool node_supported(const Tensor* node);
 
@@ -156,6 +157,7 @@ private:
     Status kernel_permute(Tensor* node);
     Status kernel_tri_mul(Tensor* node);
     Status kernel_tri_mul_back(Tensor* node);
+    Status kernel_outer_prod_mean_back(Tensor* node);
     bool resolve_views(Tensor* node);                    // src/backend/CUDABackend.cpp:800-819
     bool device_pointer_ok(const Tensor* t) const;       // src/backend/CUDABackend.cpp:894-973
     Status fail(Status s, const std::string& why);

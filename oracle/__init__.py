@@ -78,6 +78,8 @@ def _load() -> C.CDLL:
     lib.orc_flash_attn_forward.argtypes = ([C.c_int] * 5 + [C.c_float, C.c_float, C.c_int] + [f32p] * 6 + [C.c_int])
     lib.orc_tri_mul.restype = None
     lib.orc_tri_mul.argtypes = [f32p, f32p, f32p] + [i64] * 5 + [C.c_float, C.c_int, C.c_int]
+    lib.orc_outer_prod_mean_back.restype = None
+    lib.orc_outer_prod_mean_back.argtypes = [f32p] * 5 + [i64] * 4 + [C.c_int]
     lib.orc_tri_mul_back.restype = None
     lib.orc_tri_mul_back.argtypes = [f32p] * 5 + [i64] * 5 + [C.c_float, C.c_int, C.c_int]
     lib.orc_permute.restype = C.c_int
@@ -391,4 +393,14 @@ def tri_mul_back(grad, left, right, D, I, J, K, B, L, outgoing=True, nthreads=0)
     gr = np.empty(D * J * K * B, dtype=np.float32)
     lib().orc_tri_mul_back(_fp(grad), _fp(left), _fp(right), _fp(gl), _fp(gr), D, I, J, K, B, L, int(outgoing),
                            nthreads or max_threads())
+    return gl, gr
+
+
+def outer_prod_mean_back(grad, left, right, D, L, N, B, nthreads=0):
+    """kernel_outer_prod_mean_back (CPUKernels.cpp:1034-1105): returns (gleft, gright), flat [D*L*N*B] each."""
+    grad, left, right = _f32(grad).reshape(-1), _f32(left).reshape(-1), _f32(right).reshape(-1)
+    assert grad.size == D * D * L * L * B and left.size == D * L * N * B and right.size == D * L * N * B
+    gl = np.empty(D * L * N * B, dtype=np.float32)
+    gr = np.empty(D * L * N * B, dtype=np.float32)
+    lib().orc_outer_prod_mean_back(_fp(grad), _fp(left), _fp(right), _fp(gl), _fp(gr), D, L, N, B, nthreads or max_threads())
     return gl, gr

@@ -29,6 +29,8 @@
  *   orc_tri_mul : numpy einsum over the layout stated at src/backend/CPUKernels.cpp:895-903 (outgoing and
  *       incoming), exact on small integers; the finite guard on planted NaN / Inf / 1e5 values.  No
  *       reference-held vector covers it.
+ *   orc_outer_prod_mean_back : numpy einsum (exact on small integers) and the adjoint identity against
+ *       orc_outer_prod_mean.
  *   orc_tri_mul_back : numpy einsum (exact on small integers) and the adjoint identity
  *       <grad, tri_mul(l, r)> = <gleft, l> = <gright, r> against orc_tri_mul, both forms.
  *   orc_permute : numpy.transpose with the axes translated (dst dim p = src dim axes[p], dims[0]
@@ -125,6 +127,45 @@ int orc_flash_attn_forward(int B, int h, int L, int d, int causal, float scale, 
         free(tile);
     }
     return 0;
+}
+
+/* src/backend/CPUKernels.cpp:1034-1105: per output one sequential binary32 sum, outer loop over the residue
+ * index (j for gleft, i for gright), inner loop over the feature index, then times 1/N. */
+void orc_outer_prod_mean_back(const float *grad, const float *left, const float *right, float *gleft, float *gright,
+                              int64_t D, int64_t L, int64_t N, int64_t B, int nthreads) {
+    const float inv_N = 1.0f / (float)N;
+    const int64_t total = D * L * N * B;
+    if (nthreads <= 0) nthreads = 1;
+    if (gleft) {
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+        for (int64_t idx = 0; idx < total; ++idx) {
+            int64_t tmp = idx;
+            const int64_t b = tmp % B; tmp /= B;
+            const int64_t n = tmp % N; tmp /= N;
+            const int64_t i = tmp % L;
+            const int64_t d1 = tmp / L;
+            float sum = 0.0f;
+            for (int64_t j = 0; j < L; ++j)
+                for (int64_t d2 = 0; d2 < D; ++d2)
+                    sum += grad[(((d1 * D + d2) * L + i) * L + j) * B + b] * right[((d2 * L + j) * N + n) * B + b];
+            gleft[idx] = sum * inv_N;
+        }
+    }
+    if (gright) {
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+        for (int64_t idx = 0; idx < total; ++idx) {
+            int64_t tmp = idx;
+            const int64_t b = tmp % B; tmp /= B;
+            const int64_t n = tmp % N; tmp /= N;
+            const int64_t j = tmp % L;
+            const int64_t d2 = tmp / L;
+            float sum = 0.0f;
+            for (int64_t i = 0; i < L; ++i)
+                for (int64_t d1 = 0; d1 < D; ++d1)
+                    sum += grad[(((d1 * D + d2) * L + i) * L + j) * B + b] * left[((d1 * L + i) * N + n) * B + b];
+            gright[idx] = sum * inv_N;
+        }
+    }
 }
 
 /* src/backend/CPUKernels.cpp:907-968: one output per index, k ascending, sequential binary32 sum. */

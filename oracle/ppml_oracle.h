@@ -77,6 +77,9 @@ void orc_out_prod(const float *s0, const float *s1, float *dst,
 /* src/backend/CPUKernels.cpp:982-1032 */
 void orc_outer_prod_mean(const float *left, const float *right, float *dst,
                          int64_t D, int64_t L, int64_t N, int64_t B, int nthreads);
+/* src/backend/CPUKernels.cpp:1034-1105 (kernel_outer_prod_mean_back); gleft / gright may be NULL */
+void orc_outer_prod_mean_back(const float *grad, const float *left, const float *right, float *gleft, float *gright,
+                              int64_t D, int64_t L, int64_t N, int64_t B, int nthreads);
 /* src/ops/MathUtils.cpp:387-437 */
 void orc_outer_product_mean_value(const float *left, const float *right, float *dst,
                                   int64_t B, int64_t N, int64_t L, int64_t D, int nthreads);

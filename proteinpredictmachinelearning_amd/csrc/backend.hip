@@ -157,6 +157,7 @@ bool node_supported(const Tensor* node) {
             if (!src0 || !src1) return false;
             if (src0->type != TENSOR_TYPE_F32 || src1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32) return false;
             return src0->ndim == 4 && src1->ndim == 4 && node->ndim == 4;
+        case OP_OUTER_PROD_MEAN_BACK:           // src/backend/CUDABackend.cpp:418-421, the same rule
         case OP_TRI_MUL_BACK:
             // src/backend/CUDABackend.cpp:404-409: grad, left, right present, at least one of the two outputs
             if (!src0 || !src1 || !node->src[2]) return false;
@@ -401,6 +402,26 @@ Status HipBackend::kernel_tri_mul_back(Tensor* node) {
     return Status::SUCCESS;
 }
 
+// src/backend/CUDAKernels.cpp:1223-1245: src 0 grad [D*D,L,L,B], 1 left, 2 right [D,L,N,B], 3 / 4 the gradients
+Status HipBackend::kernel_outer_prod_mean_back(Tensor* node) {
+    const Tensor* g = node->src[0];
+    const Tensor* l = node->src[1];
+    const Tensor* r = node->src[2];
+    Tensor* gl = node->src[3];
+    Tensor* gr = node->src[4];
+    if (!g || !l || !r || !g->data || !l->data || !r->data || (!gl && !gr) || (gl && !gl->data) || (gr && !gr->data))
+        return fail(Status::NOT_SUPPORTED, "outer_prod_mean_back: unbound tensor");
+    const int64_t D = l->dims[0], L = l->dims[1], N = l->dims[2], B = l->dims[3];
+    if (N <= 0) return fail(Status::NOT_SUPPORTED, "outer_prod_mean_back: N must be positive");
+    if (g->numel() != D * D * L * L * B || r->numel() != l->numel() || (gl && gl->numel() != l->numel()) || (gr && gr->numel() != l->numel()))
+        return fail(Status::NOT_SUPPORTED, "outer_prod_mean_back: tensor sizes do not match each other");
+    const int rc = outer_prod_mean_back_hip(static_cast<const float*>(g->data), static_cast<const float*>(l->data),
+                                            static_cast<const float*>(r->data), gl ? static_cast<float*>(gl->data) : nullptr,
+                                            gr ? static_cast<float*>(gr->data) : nullptr, D, L, N, B, 1.0f / static_cast<float>(N), nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("outer_prod_mean_back: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
 Status HipBackend::dispatch_node(Tensor* node) {
     switch (node->op) {
         case OP_MUL_MAT: return kernel_mul_mat(node);
@@ -411,6 +432,7 @@ Status HipBackend::dispatch_node(Tensor* node) {
         case OP_TRANSPOSE: return kernel_permute(node);
         case OP_TRI_MUL: return kernel_tri_mul(node);
         case OP_TRI_MUL_BACK: return kernel_tri_mul_back(node);
+        case OP_OUTER_PROD_MEAN_BACK: return kernel_outer_prod_mean_back(node);
         default: return fail(Status::NOT_SUPPORTED, "no kernel for op " + std::to_string(node->op));
     }
 }
@@ -497,9 +519,11 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
 
         // single-backend mode: outputs nobody allocated get their own device buffer -- the node itself
         // and the second output the fused attention node carries in src[4] (its LSE buffer)
-        // (the backward node of the triangle multiplication carries both of its outputs in src[3] and src[4])
-        Tensor* outputs[3] = {storage, node->op == OP_FLASH_ATTN_EXT || node->op == OP_TRI_MUL_BACK ? node->src[4] : nullptr,
-                              node->op == OP_TRI_MUL_BACK ? node->src[3] : nullptr};
+        // (the backward nodes of the triangle multiplication and of outer-product-mean carry both of their
+        // outputs in src[3] and src[4])
+        const bool two_outputs = node->op == OP_TRI_MUL_BACK || node->op == OP_OUTER_PROD_MEAN_BACK;
+        Tensor* outputs[3] = {storage, node->op == OP_FLASH_ATTN_EXT || two_outputs ? node->src[4] : nullptr,
+                              two_outputs ? node->src[3] : nullptr};
         for (Tensor* out : outputs) {
             if (!out || skip_alloc_ || out->data) continue;
             const size_t need = out->nbytes();

@@ -18,7 +18,7 @@ namespace {
 constexpr int BM = 128, BN = 128, BK = 16;
 constexpr int LDS_LD = BM + 4;        // row pitch of the k-major LDS tiles (floats)
 
-enum LoadMode { LOAD_K_CONTIG = 0, LOAD_ROW_CONTIG = 1, LOAD_STRIDED = 2, LOAD_K_CONTIG_F16 = 3 };
+enum LoadMode { LOAD_K_CONTIG = 0, LOAD_ROW_CONTIG = 1, LOAD_STRIDED = 2, LOAD_K_CONTIG_F16 = 3, LOAD_SPLIT_A = 4 };
 
 struct GemmParams {
     const float* A;       // rows m: A(m,k) = A[m*a_rs + k*a_ks]
@@ -39,6 +39,9 @@ struct GemmParams {
     int stream_c;         // output larger than the last-level cache: write it with streaming stores
     int f16_in;           // A and B hold IEEE halves (k contiguous); products and sums are binary32
     int clamp;            // finite guard in the epilogue (triangle multiplication)
+    // LOAD_SPLIT_A: both indices of A are compound, A(m,k) = A[(m/a_lm)*a_mo + (m%a_lm)*a_mi + (k/a_lk)*a_ko + (k%a_lk)*a_ki]
+    int a_lm, a_lk;
+    int64_t a_mo, a_mi, a_ko, a_ki;
 };
 
 // 16 x 128 tile of one operand -> two v4f per thread
@@ -97,6 +100,25 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_
                 for (int c = 0; c < 4; ++c)
                     if (k + c < K) v[c] = base[static_cast<int64_t>(row) * rs + static_cast<int64_t>(k + c) * ks];
             }
+        }
+        reg[it] = v;
+    }
+}
+
+// A tile of an operand whose row and contraction indices are both compound (the gradient tensor of the
+// outer-product-mean backward, indexed [d1][d2][i][j]): one element at a time.
+__device__ __forceinline__ void load_tile_split(const float* __restrict__ base, const GemmParams& p,
+                                                int row0, int nrows, int k0, int K, int tid, v4f (&reg)[2]) {
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        const int row = row0 + (tid >> 2) + it * 64;
+        const int k = k0 + (tid & 3) * 4;
+        if (row < nrows) {
+            const int64_t roff = static_cast<int64_t>(row / p.a_lm) * p.a_mo + static_cast<int64_t>(row % p.a_lm) * p.a_mi;
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (k + c < K) v[c] = base[roff + static_cast<int64_t>((k + c) / p.a_lk) * p.a_ko + static_cast<int64_t>((k + c) % p.a_lk) * p.a_ki];
         }
         reg[it] = v;
     }
@@ -165,16 +187,19 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
     }
 
     v4f ra[2], rb[2];
-    load_tile<MODE>(A, p.a_rs, p.a_ks, m0, p.M, 0, p.K, tid, ra);
-    load_tile<MODE>(B, p.b_rs, p.b_ks, n0, p.N, 0, p.K, tid, rb);
+    constexpr int MODE_B = MODE == LOAD_SPLIT_A ? LOAD_STRIDED : MODE;
+    if (MODE == LOAD_SPLIT_A) load_tile_split(A, p, m0, p.M, 0, p.K, tid, ra);
+    else load_tile<MODE>(A, p.a_rs, p.a_ks, m0, p.M, 0, p.K, tid, ra);
+    load_tile<MODE_B>(B, p.b_rs, p.b_ks, n0, p.N, 0, p.K, tid, rb);
 
     for (int k0 = 0; k0 < p.K; k0 += BK) {
         store_tile<MODE>(lds_a, tid, ra);
         store_tile<MODE>(lds_b, tid, rb);
         __syncthreads();
         if (k0 + BK < p.K) {
-            load_tile<MODE>(A, p.a_rs, p.a_ks, m0, p.M, k0 + BK, p.K, tid, ra);
-            load_tile<MODE>(B, p.b_rs, p.b_ks, n0, p.N, k0 + BK, p.K, tid, rb);
+            if (MODE == LOAD_SPLIT_A) load_tile_split(A, p, m0, p.M, k0 + BK, p.K, tid, ra);
+            else load_tile<MODE>(A, p.a_rs, p.a_ks, m0, p.M, k0 + BK, p.K, tid, ra);
+            load_tile<MODE_B>(B, p.b_rs, p.b_ks, n0, p.N, k0 + BK, p.K, tid, rb);
         }
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 2) {
@@ -237,7 +262,11 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
         if (p.stream_c) hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, true>), grid, block, 0, stream, p);  \
         else hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, false>), grid, block, 0, stream, p);    \
     } while (0)
-    if (p.clamp) {
+    if (p.a_lm > 0) {
+        if (split || p.f16_in || p.clamp) { set_error("%s: no split-operand instance for this addressing", what); return RC_BAD_ARGS; }
+        PPML_LAUNCH(LOAD_SPLIT_A, false);
+    }
+    else if (p.clamp) {
         if (split || p.stream_c || p.f16_in) { set_error("%s: no clamped instance for this addressing", what); return RC_BAD_ARGS; }
         if (mode == LOAD_K_CONTIG) hipLaunchKernelGGL((gemm_f32_kernel<LOAD_K_CONTIG, false, false, true>), grid, block, 0, stream, p);
         else if (mode == LOAD_ROW_CONTIG) hipLaunchKernelGGL((gemm_f32_kernel<LOAD_ROW_CONTIG, false, false, true>), grid, block, 0, stream, p);
@@ -441,5 +470,34 @@ extern "C" int tri_mul_back_hip(const float* grad, const float* left, const floa
         if (gleft)  rc = launch(grad, J, 1, right, J, 1, gleft, 1, I, I, K, J, I * J, K * J, K * I);
         if (rc == RC_OK && gright) rc = launch(grad, 1, J, left, I, 1, gright, 1, J, J, K, I, I * J, K * I, K * J);
     }
+    return rc;
+}
+
+extern "C" int outer_prod_mean_back_hip(const float* grad, const float* left, const float* right, float* gleft, float* gright,
+                                        int64_t D, int64_t L, int64_t N, int64_t B, float inv_N, ppml_hip_stream_t stream) {
+    if (!grad || !left || !right || (!gleft && !gright) || D <= 0 || L <= 0 || N <= 0 || B <= 0 ||
+        D * L > 0x7fffffff || N > 0x7fffffff || B > 0x7fffffff) {
+        set_error("outer_prod_mean_back_hip: bad arguments"); return RC_BAD_ARGS;
+    }
+    // grad[d1][d2][i][j][b]; gleft[(d1,i)][n] = inv_N * sum_{(d2,j)} grad * right[(d2,j)][n],
+    //                        gright[(d2,j)][n] = inv_N * sum_{(d1,i)} grad * left[(d1,i)][n]:
+    // two contractions whose first operand has a compound row index and a compound contraction index.
+    const auto launch = [&](const float* other, float* out, int64_t mo, int64_t mi, int64_t ko, int64_t ki) {
+        stats_record(D * L, D * L, N);
+        GemmParams p = plain_params();
+        p.A = grad; p.B = other; p.C = out;
+        p.M = static_cast<int>(D * L); p.N = static_cast<int>(N); p.K = static_cast<int>(D * L);
+        p.a_lm = p.a_lk = static_cast<int>(L);
+        p.a_mo = mo * B; p.a_mi = mi * B; p.a_ko = ko * B; p.a_ki = ki * B;
+        p.b_rs = B; p.b_ks = N * B;                     // other[(k*N + n)*B + b]
+        p.c_mi = N * B; p.c_ni = B;                     // out[(m*N + n)*B + b]
+        p.np2 = static_cast<int>(B);
+        p.a_p2 = 1; p.b_p2 = 1; p.c_p2 = 1;
+        p.alpha = inv_N;
+        return launch_gemm(p, static_cast<hipStream_t>(stream), "outer_prod_mean_back_hip");
+    };
+    int rc = RC_OK;
+    if (gleft)  rc = launch(right, gleft, D * L * L, L, L * L, 1);          // m = (d1,i), k = (d2,j)
+    if (rc == RC_OK && gright) rc = launch(left, gright, L * L, 1, D * L * L, L);   // m = (d2,j), k = (d1,i)
     return rc;
 }

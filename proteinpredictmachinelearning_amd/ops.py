@@ -144,6 +144,22 @@ def outer_product_mean(left: torch.Tensor, right: torch.Tensor, D: int, L: int, 
     return out
 
 
+def outer_prod_mean_back(grad: torch.Tensor, left: torch.Tensor, right: torch.Tensor, D: int, L: int, N: int, B: int,
+                         want_left: bool = True, want_right: bool = True):
+    """Gradients of outer_prod_mean's operands (src/backend/CPUKernels.cpp:1034-1105); flat tensors."""
+    grad, left, right = _dev_f32(grad, "grad"), _dev_f32(left, "left"), _dev_f32(right, "right")
+    if grad.numel() != D * D * L * L * B or left.numel() != D * L * N * B or right.numel() != D * L * N * B:
+        raise ValueError("outer_prod_mean_back: operand size does not match D, L, N, B")
+    if not (want_left or want_right):
+        raise ValueError("outer_prod_mean_back: at least one gradient must be wanted")
+    gl = torch.empty(D * L * N * B, dtype=torch.float32, device=grad.device) if want_left else None
+    gr = torch.empty(D * L * N * B, dtype=torch.float32, device=grad.device) if want_right else None
+    cabi.check("outer_prod_mean_back_hip",
+               _lib().outer_prod_mean_back_hip(_ptr(grad), _ptr(left), _ptr(right), _ptr(gl) if gl is not None else None,
+                                               _ptr(gr) if gr is not None else None, D, L, N, B, 1.0 / float(N), _stream()))
+    return gl, gr
+
+
 def outer_product_mean_value(left: torch.Tensor, right: torch.Tensor) -> torch.Tensor:
     """Value form (src/ops/MathUtils.cpp:387-437): (B,N,L,D) x (B,N,L,D) -> (B,L,L,D*D)."""
     left, right = _dev_f32(left, "left"), _dev_f32(right, "right")

@@ -289,6 +289,23 @@ def test_tri_mul_back_node(be, oracle):
         assert np.abs(be.download(gr) - want_r).max() <= 1e-4 * np.abs(want_r).max()
 
 
+def test_outer_prod_mean_back_node(be, oracle):
+    # src/backend/CUDAKernels.cpp:1223-1245
+    rng = np.random.default_rng(15)
+    D, L, N, Bt = 3, 6, 8, 2
+    left = rng.standard_normal(D * L * N * Bt).astype(np.float32)
+    right = rng.standard_normal(D * L * N * Bt).astype(np.float32)
+    grad = rng.standard_normal(D * D * L * L * Bt).astype(np.float32)
+    gl, gr = B.Tensor((D, L, N, Bt)), B.Tensor((D, L, N, Bt))
+    node = B.Tensor((1,), B.F32, B.OP_OUTER_PROD_MEAN_BACK,
+                    [_leaf(be, grad, dims=(D * D, L, L, Bt)), _leaf(be, left, dims=(D, L, N, Bt)), _leaf(be, right, dims=(D, L, N, Bt)), gl, gr])
+    assert be.supports_op(node)
+    assert be.graph_compute([node]) == B.SUCCESS, be.last_error
+    want_l, want_r = oracle.outer_prod_mean_back(grad, left, right, D, L, N, Bt)
+    assert np.abs(be.download(gl) - want_l).max() <= 1e-4 * np.abs(want_l).max()
+    assert np.abs(be.download(gr) - want_r).max() <= 1e-4 * np.abs(want_r).max()
+
+
 def test_backward_gemms_of_mul_mat_as_the_reference_builds_them(be, oracle):
     """ComputeGraph.cpp:708-741: for y = mul_mat(A, W) (A dims [K,M], W dims [K,N], y dims [N,M]) the gradients are
     dA = mul_mat(grad, mat_transpose(W)) and dW = mul_mat(mat_transpose(grad), mat_transpose(A)), where

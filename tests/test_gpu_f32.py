@@ -277,3 +277,24 @@ def test_tri_mul_back(ops, oracle, D, I, J, K, Bt, outgoing):
     assert none is None and np.array_equal(gl.cpu().numpy(), wl)
     none, gr = ops.tri_mul_back(_dev(gi), _dev(li), _dev(ri), D, I, J, K, Bt, 4.0, outgoing, want_left=False)
     assert none is None and np.array_equal(gr.cpu().numpy(), wr)
+
+
+@pytest.mark.parametrize("D,L,N,Bt", [(3, 4, 8, 2), (16, 40, 64, 1), (4, 103, 37, 1)])
+def test_outer_prod_mean_back(ops, oracle, D, L, N, Bt):
+    rng = np.random.default_rng(D + L)
+    left = rng.standard_normal(D * L * N * Bt).astype(np.float32)
+    right = rng.standard_normal(D * L * N * Bt).astype(np.float32)
+    grad = rng.standard_normal(D * D * L * L * Bt).astype(np.float32)
+    want_l, want_r = oracle.outer_prod_mean_back(grad, left, right, D, L, N, Bt)
+    gl, gr = ops.outer_prod_mean_back(_dev(grad), _dev(left), _dev(right), D, L, N, Bt)
+    _check(gl.cpu().numpy(), want_l)
+    _check(gr.cpu().numpy(), want_r)
+    gi = rng.integers(-2, 3, size=grad.size).astype(np.float32)
+    li = rng.integers(-2, 3, size=left.size).astype(np.float32)
+    ri = rng.integers(-2, 3, size=right.size).astype(np.float32)
+    if (N & (N - 1)) == 0:                              # 1/N exact: integers stay exact in any summation order
+        wl, wr = oracle.outer_prod_mean_back(gi, li, ri, D, L, N, Bt)
+        gl, none = ops.outer_prod_mean_back(_dev(gi), _dev(li), _dev(ri), D, L, N, Bt, want_right=False)
+        assert none is None and np.array_equal(gl.cpu().numpy(), wl)
+        none, gr = ops.outer_prod_mean_back(_dev(gi), _dev(li), _dev(ri), D, L, N, Bt, want_left=False)
+        assert none is None and np.array_equal(gr.cpu().numpy(), wr)

@@ -650,3 +650,19 @@ def test_tri_mul_back_against_einsum_and_the_adjoint_identity(oracle):
         assert np.array_equal(fwd.reshape(D, I, J, Bt), np.einsum(f_eq, l64, r64) / L)
         lhs = float((g64.reshape(-1) * fwd).sum())
         assert lhs == float((gl.astype(np.float64) * l64.reshape(-1)).sum()) == float((gr.astype(np.float64) * r64.reshape(-1)).sum())
+
+
+def test_outer_prod_mean_back_against_einsum_and_the_adjoint_identity(oracle):
+    rng = np.random.default_rng(23)
+    D, L, N, Bt = 3, 4, 8, 2                           # 1/N exact
+    left = rng.integers(-3, 4, size=(D, L, N, Bt)).astype(np.float32)
+    right = rng.integers(-3, 4, size=(D, L, N, Bt)).astype(np.float32)
+    grad = rng.integers(-3, 4, size=(D, D, L, L, Bt)).astype(np.float32)      # [d1][d2][i][j][b]
+    gl, gr = oracle.outer_prod_mean_back(grad, left, right, D, L, N, Bt)
+    g64, l64, r64 = grad.astype(np.float64), left.astype(np.float64), right.astype(np.float64)
+    assert np.array_equal(gl.reshape(D, L, N, Bt), np.einsum("deijb,ejnb->dinb", g64, r64) / N)
+    assert np.array_equal(gr.reshape(D, L, N, Bt), np.einsum("deijb,dinb->ejnb", g64, l64) / N)
+    # adjoint of the forward kernel itself: <grad, opm(l, r)> = <gleft, l> = <gright, r>
+    fwd = oracle.outer_prod_mean(left.reshape(-1), right.reshape(-1), D, L, N, Bt).astype(np.float64)
+    lhs = float((g64.reshape(-1) * fwd).sum())
+    assert lhs == float((gl.astype(np.float64) * l64.reshape(-1)).sum()) == float((gr.astype(np.float64) * r64.reshape(-1)).sum())
