@@ -84,6 +84,8 @@ def _load() -> C.CDLL:
     lib.orc_tri_mul_back.argtypes = [f32p] * 5 + [i64] * 5 + [C.c_float, C.c_int, C.c_int]
     lib.orc_permute.restype = C.c_int
     lib.orc_permute.argtypes = [f32p, f32p, C.c_int, C.POINTER(C.c_int32), C.POINTER(i64), C.POINTER(i64)]
+    lib.orc_flash_attn_backward.restype = C.c_int
+    lib.orc_flash_attn_backward.argtypes = [C.c_int] * 5 + [C.c_float] + [f32p] * 11
     lib.orc_max_threads.restype = C.c_int
     return lib
 
@@ -339,6 +341,8 @@ def ref_flash_lib():
     ref.ref_flash_attn_forward.argtypes = [C.c_int] * 5 + [C.c_float, C.c_float, C.c_int] + [f32p] * 6
     ref.ref_flash_attn_forward_plain.restype = C.c_int
     ref.ref_flash_attn_forward_plain.argtypes = [C.c_int] * 5 + [C.c_float] + [f32p] * 6
+    ref.ref_flash_attn_backward.restype = C.c_int
+    ref.ref_flash_attn_backward.argtypes = [C.c_int] * 5 + [C.c_float] + [f32p] * 11
     return ref
 
 
@@ -404,3 +408,29 @@ def outer_prod_mean_back(grad, left, right, D, L, N, B, nthreads=0):
     gr = np.empty(D * L * N * B, dtype=np.float32)
     lib().orc_outer_prod_mean_back(_fp(grad), _fp(left), _fp(right), _fp(gl), _fp(gr), D, L, N, B, nthreads or max_threads())
     return gl, gr
+
+
+def _flash_backward(fn, q, k, v, bias, o, do, lse, causal, scale, want_dbias):
+    q, k, v, o, do, lse = _f32(q), _f32(k), _f32(v), _f32(o), _f32(do), _f32(lse)
+    B, h, L, d = q.shape
+    bias = _f32(bias) if bias is not None else None
+    dq, dk, dv = np.empty_like(q), np.empty_like(q), np.empty_like(q)
+    db = np.empty((B, h, L, L), dtype=np.float32) if want_dbias else None
+    rc = fn(B, h, L, d, int(causal), scale, _fp(q), _fp(k), _fp(v), _opt_fp(bias), _fp(o), _fp(do), _fp(lse),
+            _fp(dq), _fp(dk), _fp(dv), _opt_fp(db))
+    if rc:
+        raise ValueError(f"flash attention backward refused the arguments (rc={rc})")
+    return dq, dk, dv, db
+
+
+def flash_attn_backward(q, k, v, bias, o, do, lse, causal=False, scale=0.0, want_dbias=True):
+    """FlashAttn.cpp:140-210: (dQ, dK, dV, dbias) from dO and the forward's O and LSE."""
+    return _flash_backward(lib().orc_flash_attn_backward, q, k, v, bias, o, do, lse, causal, scale, want_dbias)
+
+
+def ref_flash_attn_backward(q, k, v, bias, o, do, lse, causal=False, scale=0.0, want_dbias=True):
+    """The same through the compiled reference, or None when it was never built."""
+    ref = ref_flash_lib()
+    if ref is None:
+        return None
+    return _flash_backward(ref.ref_flash_attn_backward, q, k, v, bias, o, do, lse, causal, scale, want_dbias)

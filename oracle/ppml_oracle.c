@@ -41,6 +41,8 @@
  *       softmax attention, closed forms (equal scores -> mean of V, one dominant key -> that
  *       row of V, shift invariance in the bias, fully masked rows) where the reference build
  *       is absent.
+ *   orc_flash_attn_backward : the compiled reference routine bit for bit; central finite differences of
+ *       the float64 softmax attention; rows of dbias sum to 0; masked rows give zero gradients.
  */
 #include "ppml_oracle.h"
 
@@ -257,6 +259,52 @@ int orc_permute(const float *src, float *dst, int ndim, const int32_t axes[4], c
         int64_t i[4] = {0, 0, 0, 0};
         for (int p = 0; p < ndim && p < 4; ++p) i[dims[p]] = jv[p];
         dst[idx] = src[((i[3] * sd[2] + i[2]) * sd[1] + i[1]) * sd[0] + i[0]];
+    }
+    return 0;
+}
+
+/* src/ops/FlashAttn.cpp:140-210, same loop nest: rows i ascending, keys j ascending, every accumulation in
+ * that order (dK and dV rows therefore receive their terms in ascending i).  Planes run on threads; nothing
+ * inside a plane is reordered. */
+int orc_flash_attn_backward(int B, int h, int L, int d, int causal, float scale,
+                            const float *Q, const float *K, const float *V, const float *bias,
+                            const float *O, const float *dO, const float *LSE,
+                            float *dQ, float *dK, float *dV, float *dbias) {
+    if (!Q || !K || !V || !O || !dO || !LSE) return 1;
+    if (B <= 0 || h <= 0 || L <= 0 || d <= 0) return 1;
+    if (!dQ && !dK && !dV && !dbias) return 1;
+    const float sc = scale > 0.0f ? scale : 1.0f / sqrtf((float)d);
+    const int64_t planes = (int64_t)B * h, nq = planes * L * d, nb = planes * L * L;
+    if (dQ) memset(dQ, 0, sizeof(float) * (size_t)nq);
+    if (dK) memset(dK, 0, sizeof(float) * (size_t)nq);
+    if (dV) memset(dV, 0, sizeof(float) * (size_t)nq);
+    if (dbias) memset(dbias, 0, sizeof(float) * (size_t)nb);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int64_t pl = 0; pl < planes; ++pl) {
+        const int64_t po = pl * (int64_t)L * d;
+        for (int i = 0; i < L; ++i) {
+            const float lse = LSE[pl * L + i];
+            if (!(lse > -INFINITY)) continue;
+            const float *q = Q + po + (int64_t)i * d, *o_row = O + po + (int64_t)i * d, *do_row = dO + po + (int64_t)i * d;
+            float Dsum = 0.0f;
+            for (int dd = 0; dd < d; ++dd) Dsum += do_row[dd] * o_row[dd];
+            const int jmax = causal ? i + 1 : L;
+            for (int j = 0; j < jmax; ++j) {
+                const float *k = K + po + (int64_t)j * d;
+                float s = 0.0f;
+                for (int dd = 0; dd < d; ++dd) s += q[dd] * k[dd];
+                s *= sc;
+                if (bias) s += bias[(pl * L + i) * (int64_t)L + j];
+                const float p = expf(s - lse);
+                float dp = 0.0f;
+                for (int dd = 0; dd < d; ++dd) dp += do_row[dd] * V[po + (int64_t)j * d + dd];
+                const float ds = p * (dp - Dsum);
+                if (dbias) dbias[(pl * L + i) * (int64_t)L + j] = ds;
+                if (dQ) for (int dd = 0; dd < d; ++dd) dQ[po + (int64_t)i * d + dd] += sc * ds * k[dd];
+                if (dK) for (int dd = 0; dd < d; ++dd) dK[po + (int64_t)j * d + dd] += sc * ds * q[dd];
+                if (dV) for (int dd = 0; dd < d; ++dd) dV[po + (int64_t)j * d + dd] += p * do_row[dd];
+            }
+        }
     }
     return 0;
 }

@@ -111,6 +111,15 @@ void orc_tri_mul_back(const float *grad, const float *left, const float *right, 
  * returns 0 ok, 1 when an axis is outside [0, ndim) -- the reference prints and leaves dst untouched. */
 int orc_permute(const float *src, float *dst, int ndim, const int32_t axes[4], const int64_t sd[4], const int64_t dd[4]);
 
+/* src/ops/FlashAttn.cpp:140-210 (flash_attn_backward_cpu): gradients of orc_flash_attn_forward's inputs from
+ * dO, with P = exp(S - LSE) recomputed.  dQ, dK, dV [B][h][L][d], dbias [B][h][L][L]; any of them may be NULL
+ * (not all).  Outputs are zeroed first; rows with LSE = -inf and masked positions contribute nothing.
+ * returns 0 ok, 1 bad arguments. */
+int orc_flash_attn_backward(int B, int h, int L, int d, int causal, float scale,
+                            const float *Q, const float *K, const float *V, const float *bias,
+                            const float *O, const float *dO, const float *LSE,
+                            float *dQ, float *dK, float *dV, float *dbias);
+
 int orc_max_threads(void);
 
 #ifdef __cplusplus

@@ -27,3 +27,11 @@ extern "C" int ref_flash_attn_forward_plain(int B, int h, int L, int d, int caus
                                             float* O, float* LSE) {
     return ppml::flash_attn_forward_ref_cpu(config_of(B, h, L, d, causal, scale, 0.0f, 0), Q, K, V, bias, O, LSE) ? 0 : 1;
 }
+
+extern "C" int ref_flash_attn_backward(int B, int h, int L, int d, int causal, float scale,
+                                       const float* Q, const float* K, const float* V, const float* bias,
+                                       const float* O, const float* dO, const float* LSE,
+                                       float* dQ, float* dK, float* dV, float* dbias) {
+    return ppml::flash_attn_backward_cpu(config_of(B, h, L, d, causal, scale, 0.0f, 0), Q, K, V, bias, O, dO, LSE,
+                                         dQ, dK, dV, dbias) ? 0 : 1;
+}

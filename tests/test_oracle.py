@@ -666,3 +666,58 @@ def test_outer_prod_mean_back_against_einsum_and_the_adjoint_identity(oracle):
     fwd = oracle.outer_prod_mean(left.reshape(-1), right.reshape(-1), D, L, N, Bt).astype(np.float64)
     lhs = float((g64.reshape(-1) * fwd).sum())
     assert lhs == float((gl.astype(np.float64) * l64.reshape(-1)).sum()) == float((gr.astype(np.float64) * r64.reshape(-1)).sum())
+
+
+# ----------------------------------------------------------------------------- fused attention backward
+@pytest.mark.parametrize("B,h,L,d,causal,use_bias", [(2, 2, 19, 8, False, True), (1, 3, 40, 16, True, True), (1, 1, 70, 32, False, False)])
+def test_flash_attn_backward_against_the_compiled_reference(oracle, B, h, L, d, causal, use_bias):
+    if oracle.ref_flash_lib() is None:
+        pytest.skip("oracle/_ref/libppml_ref_flash.so not built (reference tree absent)")
+    rng = np.random.default_rng(L + d)
+    q, k, v, do = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(4)]
+    bias = rng.standard_normal((B, h, L, L)).astype(np.float32) if use_bias else None
+    if bias is not None and not causal:
+        bias[0, 0, 3, :] = -np.inf                      # a masked row: LSE = -inf, no gradient
+    o, lse = oracle.flash_attn_forward(q, k, v, bias, causal=causal)
+    got = oracle.flash_attn_backward(q, k, v, bias, o, do, lse, causal=causal)
+    want = oracle.ref_flash_attn_backward(q, k, v, bias, o, do, lse, causal=causal)
+    for g, w in zip(got, want):
+        assert (g.view(np.uint32) == w.view(np.uint32)).all()
+
+
+def test_flash_attn_backward_against_finite_differences(oracle):
+    rng = np.random.default_rng(31)
+    B, h, L, d = 1, 2, 9, 4
+    q, k, v, do = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(4)]
+    bias = rng.standard_normal((B, h, L, L)).astype(np.float32)
+    for causal in (False, True):
+        o, lse = oracle.flash_attn_forward(q, k, v, bias, causal=causal, eps=0.0)
+        dq, dk, dv, db = oracle.flash_attn_backward(q, k, v, bias, o, do, lse, causal=causal)
+
+        def loss(q_, k_, v_, b_):
+            o64, _ = _attention_f64(q_, k_, v_, b_, causal, 0.0, 0.0)
+            return float((o64 * do.astype(np.float64)).sum())
+
+        def numeric(which):
+            arrs = [q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), bias.astype(np.float64)]
+            g = np.zeros_like(arrs[which])
+            it = np.nditer(arrs[which], flags=["multi_index"])
+            for _ in it:
+                idx = it.multi_index
+                old = arrs[which][idx]
+                arrs[which][idx] = old + 1e-5
+                up = loss(*arrs)
+                arrs[which][idx] = old - 1e-5
+                dn = loss(*arrs)
+                arrs[which][idx] = old
+                g[idx] = (up - dn) / 2e-5
+            return g
+        for got, which in ((dq, 0), (dk, 1), (dv, 2), (db, 3)):
+            want = numeric(which)
+            assert np.abs(got - want).max() <= 2e-4 * max(1.0, np.abs(want).max()), (causal, which)
+        # softmax rows: the gradient with respect to the scores sums to zero over the keys
+        assert np.abs(db.sum(axis=-1)).max() <= 1e-5
+        if causal:
+            assert (np.triu(db[0, 0], 1) == 0).all()
+    # nothing to compute is refused
+    assert oracle.lib().orc_flash_attn_backward(1, 1, 2, 4, 0, 0.0, *([q.ctypes.data_as(__import__("ctypes").POINTER(__import__("ctypes").c_float))] * 7), None, None, None, None) == 1
