@@ -211,6 +211,32 @@ def main() -> int:
             f32_case(attention(planes, L, D, wb, lay), (4 * planes * L * D + planes * L + (planes * L * L if wb else 0)) * 4,
                      4.0 * planes * L * L * D, "fused_attention_" + tag)
 
+        def attention_back(planes, L, D):
+            def make():
+                import ctypes as C
+                nb = (8 * planes * L * D + planes * L + 2 * planes * L * L) * 4
+                ns = max(2, int(640e6 // nb) + 1)
+                t = lambda *shape: torch.randn(*shape, device=dev, generator=gen)      # noqa: E731
+                sets = []
+                for _ in range(ns):
+                    q, k, v, do, b = t(1, planes, L, D), t(1, planes, L, D), t(1, planes, L, D), t(1, planes, L, D), t(1, planes, L, L)
+                    o, lse = ops.flash_attn_forward(q, k, v, b)
+                    sets.append((q, k, v, b, o, do, lse, torch.empty_like(q), torch.empty_like(q), torch.empty_like(q), torch.empty_like(b)))
+                lib, cabi = ops._lib(), ops.cabi
+                stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+                argsets = [(1, planes, L, D, 0, 0.0) + tuple(C.c_void_p(x.data_ptr()) for x in s_) + (stream,) for s_ in sets]
+
+                def fn(i):
+                    rc = lib.flash_attn_backward_hip(*argsets[i])
+                    if rc:
+                        cabi.check("flash_attn_backward_hip", rc)
+                keep.append(sets)
+                return fn, ns
+            return make
+        # flops: five 2*L*L*D contractions per plane in exact terms (S, dP, dQ, dK, dV); S and dP are computed twice
+        f32_case(attention_back(824, 256, 32), (8 * 824 * 256 * 32 + 824 * 256 + 2 * 824 * 256 * 256) * 4,
+                 10.0 * 824 * 256 * 256 * 32, "fused_attention_backward_msa_824x256x32_bias")
+
         def bridge():
             # the [L, D, h, B] -> [D, L, h, B] copy in front of the fused attention node, MSA-track size
             import ctypes as C

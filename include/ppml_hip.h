@@ -187,6 +187,20 @@ int flash_attn_forward_ex_hip(int B, int h, int L, int d, int causal, float scal
                               const float *Q, const float *K, const float *V, const float *bias,
                               float *O, float *LSE, int layout, ppml_hip_stream_t stream);
 
+/* replaces flash_attn_backward_cuda (declared src/backend/CUDAKernels.cpp:176-179, contract
+ * include/ppml/FlashAttn.h:67-101, called from kernel_flash_attn_back_cuda, CUDAKernels.cpp:905-924), the
+ * mathematics of flash_attn_backward_cpu (src/ops/FlashAttn.cpp:140-210): from dO and the forward's O and LSE,
+ *     P = exp(S - LSE),  D_i = sum_d dO_id O_id,  dS = P (dO V^T - D),
+ *     dQ = scale dS K,   dK = scale dS^T Q,   dV = P^T dO,   dbias = dS  (0 at masked positions)
+ * Layouts as in flash_attn_forward_hip; dQ, dK, dV, dbias may each be NULL (not all).  Every output element is
+ * written (rows with LSE = -inf as zeros), nothing needs clearing beforehand, and there are no atomics: results
+ * do not depend on scheduling.  d <= 64 and a multiple of 4 (the reference's CUDA path stops at 32).
+ * returns 0 = ran, 1 = refused, 6 = launch error. */
+int flash_attn_backward_hip(int B, int h, int L, int d, int causal, float scale,
+                            const float *Q, const float *K, const float *V, const float *bias,
+                            const float *O, const float *dO, const float *LSE,
+                            float *dQ, float *dK, float *dV, float *dbias, ppml_hip_stream_t stream);
+
 /* ---- dimension permutation (a real copy) ------------------------------------------------------ */
 /* replaces permute_cuda and transpose_cuda (declared src/backend/CUDAKernels.cpp:137-143, called from
  * kernel_permute_cuda / kernel_transpose_cuda, 1344-1390); semantics of CPUBackend::kernel_permute

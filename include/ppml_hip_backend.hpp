@@ -38,6 +38,7 @@ enum TensorOp : int {
     OP_PERMUTE = 39,
     OP_TRANSPOSE = 40,
     OP_FLASH_ATTN_EXT = 75,
+    OP_FLASH_ATTN_BACK = 76,
     OP_TRI_MUL = 100,
     OP_TRI_MUL_BACK = 101,
     OP_OUTER_PROD_MEAN = 102,
@@ -114,7 +115,7 @@ private:
 using ComputeGraph = std::vector<Tensor*>;   // nodes in evaluation order
 
 // src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-421 (OP_OUTER_PROD_MEAN, OP_OUTER_PROD_MEAN_BACK),
-// 113-119 (OP_PERMUTE, OP_TRANSPOSE), 395-409 (OP_TRI_MUL, OP_TRI_MUL_BACK), 457-463 (OP_FLASH_ATTN_EXT); a function of the node alone, so it can be asked without a device
+// 113-119 (OP_PERMUTE, OP_TRANSPOSE), 395-409 (OP_TRI_MUL, OP_TRI_MUL_BACK), 457-471 (OP_FLASH_ATTN_EXT, OP_FLASH_ATTN_BACK); a function of the node alone, so it can be asked without a device
 bool node_supported(const Tensor* node);
 
 // include/ppml/Backend.h:550-605; executor obligations of src/backend/CUDABackend.cpp:708-1086
@@ -154,6 +155,7 @@ private:
     Status kernel_out_prod(Tensor* node);
     Status kernel_outer_prod_mean(Tensor* node);
     Status kernel_flash_attn_ext(Tensor* node);
+    Status kernel_flash_attn_back(Tensor* node);
     Status kernel_permute(Tensor* node);
     Status kernel_tri_mul(Tensor* node);
     Status kernel_tri_mul_back(Tensor* node);

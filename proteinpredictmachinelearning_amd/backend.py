@@ -18,7 +18,8 @@ from . import cabi
 F32, F16, Q8_0, Q8_1, Q8_0R, Q8_0M = 0, 1, 8, 9, 19, 64
 # tensor_op
 OP_NONE, OP_MUL_MAT, OP_OUT_PROD, OP_SCALE, OP_RESHAPE, OP_VIEW, OP_PERMUTE, OP_TRANSPOSE, OP_SOFT_MAX = 0, 30, 32, 33, 37, 38, 39, 40, 47
-OP_FLASH_ATTN_EXT, OP_TRI_MUL, OP_TRI_MUL_BACK, OP_OUTER_PROD_MEAN, OP_OUTER_PROD_MEAN_BACK = 75, 100, 101, 102, 103
+OP_FLASH_ATTN_EXT, OP_FLASH_ATTN_BACK, OP_TRI_MUL, OP_TRI_MUL_BACK, OP_OUTER_PROD_MEAN, OP_OUTER_PROD_MEAN_BACK = \
+    75, 76, 100, 101, 102, 103
 # Status
 SUCCESS, ALLOC_FAILED, NOT_SUPPORTED, ABORTED = 0, 1, 2, 3
 

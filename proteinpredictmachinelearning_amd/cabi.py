@@ -38,6 +38,7 @@ SIGNATURES = {
     "tri_mul_hip": (_i, [_vp, _vp, _vp] + [_i64] * 5 + [_f, _i, _vp]),
     "tri_mul_back_hip": (_i, [_vp] * 5 + [_i64] * 5 + [_f, _i, _vp]),
     "flash_attn_forward_hip": (_i, [_i] * 5 + [_f, _f, _i] + [_vp] * 7),
+    "flash_attn_backward_hip": (_i, [_i] * 5 + [_f] + [_vp] * 12),
     "flash_attn_forward_ex_hip": (_i, [_i] * 5 + [_f, _f, _i] + [_vp] * 6 + [_i, _vp]),
     "permute_hip": (_i, [_vp, _vp, _i64, _i] + [_i] * 4 + [_i64] * 8 + [_vp]),
     "ppml_hip_mulmat_stats": (_i, [C.POINTER(_i64), _i]),

@@ -157,6 +157,12 @@ bool node_supported(const Tensor* node) {
             if (!src0 || !src1) return false;
             if (src0->type != TENSOR_TYPE_F32 || src1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32) return false;
             return src0->ndim == 4 && src1->ndim == 4 && node->ndim == 4;
+        case OP_FLASH_ATTN_BACK: {
+            // src/backend/CUDABackend.cpp:465-471 (there: d <= 32; this kernel takes the forward's range)
+            if (!src0 || src0->type != TENSOR_TYPE_F32) return false;
+            const int64_t d = src0->dims[0];
+            return d > 0 && d <= 64 && (d % 4) == 0;
+        }
         case OP_OUTER_PROD_MEAN_BACK:           // src/backend/CUDABackend.cpp:418-421, the same rule
         case OP_TRI_MUL_BACK:
             // src/backend/CUDABackend.cpp:404-409: grad, left, right present, at least one of the two outputs
@@ -422,12 +428,45 @@ Status HipBackend::kernel_outer_prod_mean_back(Tensor* node) {
     return Status::SUCCESS;
 }
 
+// src/backend/CUDAKernels.cpp:905-924: src 0..2 Q, K, V ([d, L, h, B]), 3 bias or null, 4 O, 5 dO, 6 LSE,
+// 7..9 dQ, dK, dV (each may be null); the node itself receives dbias when op_params[5] != 0.
+Status HipBackend::kernel_flash_attn_back(Tensor* node) {
+    const Tensor* q = node->src[0];
+    const Tensor* k = node->src[1];
+    const Tensor* v = node->src[2];
+    const Tensor* bias = node->src[3];
+    const Tensor* o = node->src[4];
+    const Tensor* dout = node->src[5];
+    const Tensor* lse = node->src[6];
+    Tensor* dq = node->src[7];
+    Tensor* dk = node->src[8];
+    Tensor* dv = node->src[9];
+    if (!q || !k || !v || !o || !dout || !lse || !q->data || !k->data || !v->data || !o->data || !dout->data || !lse->data)
+        return fail(Status::NOT_SUPPORTED, "flash_attn_back: unbound tensor");
+    const bool want_dbias = node->op_params[5] != 0;
+    if ((dq && !dq->data) || (dk && !dk->data) || (dv && !dv->data) || (want_dbias && !node->data) || (bias && !bias->data))
+        return fail(Status::NOT_SUPPORTED, "flash_attn_back: unbound output");
+    const int64_t d = q->dims[0], L = q->dims[1], h = dim_or_1(q, 2), B = dim_or_1(q, 3);
+    const int64_t n = q->numel();
+    if (k->numel() != n || v->numel() != n || o->numel() != n || dout->numel() != n || lse->numel() != B * h * L ||
+        (dq && dq->numel() != n) || (dk && dk->numel() != n) || (dv && dv->numel() != n) ||
+        (bias && bias->numel() != B * h * L * L) || (want_dbias && node->numel() != B * h * L * L))
+        return fail(Status::NOT_SUPPORTED, "flash_attn_back: tensor sizes do not match each other");
+    const auto f = [](const Tensor* t) { return t ? static_cast<float*>(t->data) : nullptr; };
+    const int rc = flash_attn_backward_hip(static_cast<int>(B), static_cast<int>(h), static_cast<int>(L), static_cast<int>(d),
+                                           node->op_params[1] != 0, node->param_f32(0), f(q), f(k), f(v), f(bias), f(o), f(dout), f(lse),
+                                           f(dq), f(dk), f(dv), want_dbias ? static_cast<float*>(node->data) : nullptr, nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("flash_attn_back: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
 Status HipBackend::dispatch_node(Tensor* node) {
     switch (node->op) {
         case OP_MUL_MAT: return kernel_mul_mat(node);
         case OP_OUT_PROD: return kernel_out_prod(node);
         case OP_OUTER_PROD_MEAN: return kernel_outer_prod_mean(node);
         case OP_FLASH_ATTN_EXT: return kernel_flash_attn_ext(node);
+        case OP_FLASH_ATTN_BACK: return kernel_flash_attn_back(node);
         case OP_PERMUTE:
         case OP_TRANSPOSE: return kernel_permute(node);
         case OP_TRI_MUL: return kernel_tri_mul(node);
@@ -520,10 +559,14 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         // single-backend mode: outputs nobody allocated get their own device buffer -- the node itself
         // and the second output the fused attention node carries in src[4] (its LSE buffer)
         // (the backward nodes of the triangle multiplication and of outer-product-mean carry both of their
-        // outputs in src[3] and src[4])
+        // outputs in src[3] and src[4]; the attention backward carries dQ, dK, dV in src[7..9] and uses its own
+        // storage for dbias only when op_params[5] asks for it)
         const bool two_outputs = node->op == OP_TRI_MUL_BACK || node->op == OP_OUTER_PROD_MEAN_BACK;
-        Tensor* outputs[3] = {storage, node->op == OP_FLASH_ATTN_EXT || two_outputs ? node->src[4] : nullptr,
-                              two_outputs ? node->src[3] : nullptr};
+        const bool attn_back = node->op == OP_FLASH_ATTN_BACK;
+        Tensor* outputs[5] = {attn_back && node->op_params[5] == 0 ? nullptr : storage,
+                              node->op == OP_FLASH_ATTN_EXT || two_outputs ? node->src[4] : nullptr,
+                              two_outputs ? node->src[3] : nullptr, nullptr, nullptr};
+        if (attn_back) { outputs[1] = node->src[7]; outputs[2] = node->src[8]; outputs[3] = node->src[9]; }
         for (Tensor* out : outputs) {
             if (!out || skip_alloc_ || out->data) continue;
             const size_t need = out->nbytes();
@@ -540,7 +583,7 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
             rewired.buffer_offs = storage->buffer_offs;
         }
 
-        if (!device_pointer_ok(exec))
+        if (!(attn_back && node->op_params[5] == 0) && !device_pointer_ok(exec))
             return fail(Status::NOT_SUPPORTED, "node " + std::to_string(index) + ": output is not device memory inside its buffer");
         for (int j = 0; j < 10; ++j) {
             if (exec->src[j] && !device_pointer_ok(exec->src[j]))

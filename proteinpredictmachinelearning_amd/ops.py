@@ -232,6 +232,25 @@ def flash_attn_forward(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, bias: 
     return o, lse
 
 
+def flash_attn_backward(q, k, v, bias, o, do, lse, causal: bool = False, scale: float = 0.0,
+                        want=("dq", "dk", "dv", "dbias")):
+    """Fused attention backward (include/ppml/FlashAttn.h:67-101): returns (dQ, dK, dV, dbias), None for the
+    gradients not named in `want`."""
+    q, k, v, o, do, lse = (_dev_f32(t, n) for t, n in ((q, "q"), (k, "k"), (v, "v"), (o, "o"), (do, "do"), (lse, "lse")))
+    B, h, L, d = q.shape
+    if bias is not None:
+        bias = _dev_f32(bias, "bias")
+    dq = torch.empty_like(q) if "dq" in want else None
+    dk = torch.empty_like(q) if "dk" in want else None
+    dv = torch.empty_like(q) if "dv" in want else None
+    db = torch.empty((B, h, L, L), dtype=torch.float32, device=q.device) if "dbias" in want else None
+    opt = lambda t: _ptr(t) if t is not None else None      # noqa: E731
+    cabi.check("flash_attn_backward_hip",
+               _lib().flash_attn_backward_hip(B, h, L, d, int(causal), scale, _ptr(q), _ptr(k), _ptr(v), opt(bias), _ptr(o),
+                                              _ptr(do), _ptr(lse), opt(dq), opt(dk), opt(dv), opt(db), _stream()))
+    return dq, dk, dv, db
+
+
 def permute(x: torch.Tensor, axes) -> torch.Tensor:
     """The reference's permute as a copy (src/backend/CPUKernels.cpp:1669-1717).  `x` is a dense tensor whose
     LAST torch dimension is the reference's dims[0]; `axes` is in the reference's numbering: dimension p of

@@ -44,10 +44,24 @@ def main():
         out.append({"B": B, "h": h, "L": L, "d": d, "causal": causal, "Bc": Bc, "scale": scale, "eps": eps,
                     "q": bits(q), "k": bits(k), "v": bits(v), "bias": bits(bias) if bias is not None else None,
                     "o": bits(o), "lse": bits(lse)})
+    back = []
+    for B, h, L, d, causal, use_bias, seed in [(1, 2, 9, 4, False, True, 21), (1, 1, 17, 8, True, True, 22)]:
+        rng = np.random.default_rng(seed)
+        q, k, v, do = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(4)]
+        bias = rng.standard_normal((B, h, L, L)).astype(np.float32) if use_bias else None
+        if bias is not None and not causal:
+            bias[0, 1, 2, :] = -np.inf
+        o, lse = oracle.ref_flash_attn_forward(q, k, v, bias, causal=causal)
+        dq, dk, dv, db = oracle.ref_flash_attn_backward(q, k, v, bias, o, do, lse, causal=causal)
+        back.append({"B": B, "h": h, "L": L, "d": d, "causal": causal, "q": bits(q), "k": bits(k), "v": bits(v),
+                     "bias": bits(bias) if bias is not None else None, "o": bits(o), "lse": bits(lse), "do": bits(do),
+                     "dq": bits(dq), "dk": bits(dk), "dv": bits(dv), "dbias": bits(db)})
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "flash_attn_forward.json")
     with open(path, "w") as f:
         json.dump({"source": "flash_attn_forward_cpu, src/ops/FlashAttn.cpp:55-135, compiled from the reference tree",
-                   "encoding": "binary32 bit patterns, C order", "cases": out}, f)
+                   "encoding": "binary32 bit patterns, C order", "cases": out,
+                   "backward_source": "flash_attn_backward_cpu, src/ops/FlashAttn.cpp:140-210, same build",
+                   "backward_cases": back}, f)
     print("wrote", path, os.path.getsize(path), "bytes")
 
 

@@ -119,3 +119,12 @@ def test_supports_op_tri_mul_back():
     assert B.supports_op(B.Tensor((1,), B.F32, B.OP_TRI_MUL_BACK, [g, l, r, None, gr]))
     assert not B.supports_op(B.Tensor((1,), B.F32, B.OP_TRI_MUL_BACK, [g, l, r]))
     assert not B.supports_op(B.Tensor((1,), B.F32, B.OP_TRI_MUL_BACK, [g, l, None, gl, gr]))
+
+
+def test_supports_op_fused_attention_backward():
+    # src/backend/CUDABackend.cpp:465-471 (the reference's CUDA kernel stops at d = 32; this one at 64)
+    for d, want in [(4, True), (32, True), (64, True), (68, False), (6, False)]:
+        q = B.Tensor((d, 10, 2, 1))
+        assert B.supports_op(B.Tensor((10, 10, 2, 1), B.F32, B.OP_FLASH_ATTN_BACK, [q])) == want, d
+    assert not B.supports_op(B.Tensor((10, 10, 2, 1), B.F32, B.OP_FLASH_ATTN_BACK, []))
+    assert not B.supports_op(B.Tensor((10, 10, 2, 1), B.F32, B.OP_FLASH_ATTN_BACK, [B.Tensor((32, 10, 2, 1), B.F16)]))

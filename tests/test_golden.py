@@ -91,3 +91,18 @@ def test_flash_attn_forward_matches_the_reference_vectors_bit_for_bit(oracle):
     # the vectors do contain the special row: fully masked -> O = 0, LSE = -inf
     first = next(flash_cases())
     assert np.isneginf(first["lse"][0, 0, 1]) and (first["o"][0, 0, 1] == 0).all()
+
+
+def test_flash_attn_backward_matches_the_reference_vectors_bit_for_bit(oracle):
+    with open(FLASH) as f:
+        cases = json.load(f)["backward_cases"]
+    assert len(cases) == 2
+    for c in cases:
+        shape = (c["B"], c["h"], c["L"], c["d"])
+        f32 = lambda bits, shp: np.array(bits, dtype=np.uint32).view(np.float32).reshape(shp)  # noqa: E731
+        sq = (c["B"], c["h"], c["L"], c["L"])
+        bias = f32(c["bias"], sq) if c["bias"] is not None else None
+        got = oracle.flash_attn_backward(f32(c["q"], shape), f32(c["k"], shape), f32(c["v"], shape), bias, f32(c["o"], shape),
+                                         f32(c["do"], shape), f32(c["lse"], shape[:3]), causal=c["causal"])
+        for g, key, shp in zip(got, ("dq", "dk", "dv", "dbias"), (shape, shape, shape, sq)):
+            assert (g.view(np.uint32) == f32(c[key], shp).view(np.uint32)).all(), key

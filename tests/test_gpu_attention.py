@@ -179,3 +179,78 @@ def test_layouts_without_the_bridges(ops, oracle, B, h, L, d, causal, use_bias, 
     if out_ld:
         got_o = got_o.transpose(0, 1, 3, 2)
     _check(got_o, lse.cpu().numpy(), want_o, want_lse)
+
+
+# ----------------------------------------------------------------------------- backward
+def _check_grad(got, want, name):
+    # inputs are O(1); a gradient that is exactly zero in exact arithmetic (a single key: dS = dP - D = 0) comes
+    # out as rounding noise of size 1e-8, hence the floor of the scale
+    scale = max(np.abs(want).max(), 1e-3)
+    err = np.abs(got.astype(np.float64) - want).max() / scale
+    assert err <= RTOL, f"{name} normwise {err:.3e}"
+
+
+@pytest.mark.parametrize("B,h,L,d,causal,use_bias", [
+    (1, 1, 1, 4, False, False), (2, 2, 37, 8, False, True), (1, 4, 103, 32, False, True), (1, 2, 128, 32, True, False),
+    (1, 2, 160, 32, True, True),       # more rows than one LDS stage (128), causal: skipped chunks and tiles
+    (2, 2, 256, 32, False, True), (1, 2, 70, 64, False, True), (1, 1, 150, 64, True, True), (1, 2, 45, 20, False, True),
+])
+def test_flash_attn_backward_matches_oracle(ops, oracle, B, h, L, d, causal, use_bias):
+    rng = np.random.default_rng(7000 + 10 * L + d)
+    q, k, v, do = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(4)]
+    bias = rng.standard_normal((B, h, L, L)).astype(np.float32) if use_bias else None
+    if bias is not None and not causal and L > 4:
+        bias[0, 0, 3, :] = -np.inf                  # a masked row: no gradient from it, zeros in its dbias row
+    o, lse = oracle.flash_attn_forward(q, k, v, bias, causal=causal)
+    want = oracle.flash_attn_backward(q, k, v, bias, o, do, lse, causal=causal)
+    got = ops.flash_attn_backward(_dev(q), _dev(k), _dev(v), _dev(bias), _dev(o), _dev(do), _dev(lse), causal=causal)
+    ops.synchronize()
+    for g, w, name in zip(got, want, ("dQ", "dK", "dV", "dbias")):
+        _check_grad(g.cpu().numpy(), w, name)
+    db = got[3].cpu().numpy()
+    assert (db[np.isneginf(lse)] == 0).all()        # rows without a visible key: exact zeros
+    if bias is not None:
+        assert (db[np.isneginf(bias) & ~np.isneginf(lse)[..., None]] == 0).all()    # masked keys of live rows
+    if causal:
+        assert (np.triu(db[0, 0], 1) == 0).all()
+
+
+def test_flash_attn_backward_subsets_and_determinism(ops, oracle):
+    rng = np.random.default_rng(77)
+    B, h, L, d = 1, 3, 90, 32
+    q, k, v, do = [rng.standard_normal((B, h, L, d)).astype(np.float32) for _ in range(4)]
+    bias = rng.standard_normal((B, h, L, L)).astype(np.float32)
+    o, lse = oracle.flash_attn_forward(q, k, v, bias)
+    args = [_dev(x) for x in (q, k, v, bias, o, do, lse)]
+    full = [t.cpu().numpy() for t in ops.flash_attn_backward(*args)]
+    again = [t.cpu().numpy() for t in ops.flash_attn_backward(*args)]
+    for a, b in zip(full, again):
+        assert np.array_equal(a, b)                 # one owner per output element: no atomics, bit-stable
+    dq, dk, dv, db = ops.flash_attn_backward(*args, want=("dk",))
+    assert dq is None and dv is None and db is None and np.array_equal(dk.cpu().numpy(), full[1])
+    dq, dk, dv, db = ops.flash_attn_backward(*args, want=("dq", "dv"))
+    assert dk is None and db is None and np.array_equal(dq.cpu().numpy(), full[0]) and np.array_equal(dv.cpu().numpy(), full[2])
+    dq, dk, dv, db = ops.flash_attn_backward(*args, want=("dbias",))
+    assert np.array_equal(db.cpu().numpy(), full[3])
+    # the scale argument: caller's head dimension instead of d
+    o2, lse2 = oracle.flash_attn_forward(q, k, v, bias, scale=0.5)
+    want = oracle.flash_attn_backward(q, k, v, bias, o2, do, lse2, scale=0.5)
+    got = ops.flash_attn_backward(*args[:4], _dev(o2), args[5], _dev(lse2), scale=0.5)
+    for g, w, name in zip(got, want, ("dQ", "dK", "dV", "dbias")):
+        _check_grad(g.cpu().numpy(), w, name)
+
+
+def test_backward_reference_golden_vectors(ops):
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "flash_attn_forward.json")
+    with open(path) as f:
+        cases = json.load(f)["backward_cases"]
+    for c in cases:
+        shape = (c["B"], c["h"], c["L"], c["d"])
+        sq = (c["B"], c["h"], c["L"], c["L"])
+        f32 = lambda bits, shp: np.array(bits, dtype=np.uint32).view(np.float32).reshape(shp)  # noqa: E731
+        bias = f32(c["bias"], sq) if c["bias"] is not None else None
+        got = ops.flash_attn_backward(_dev(f32(c["q"], shape)), _dev(f32(c["k"], shape)), _dev(f32(c["v"], shape)), _dev(bias),
+                                      _dev(f32(c["o"], shape)), _dev(f32(c["do"], shape)), _dev(f32(c["lse"], shape[:3])), causal=c["causal"])
+        ops.synchronize()
+        for g, key, shp in zip(got, ("dq", "dk", "dv", "dbias"), (shape, shape, shape, sq)):
+            _check_grad(g.cpu().numpy(), f32(c[key], shp), key)

@@ -289,6 +289,31 @@ def test_tri_mul_back_node(be, oracle):
         assert np.abs(be.download(gr) - want_r).max() <= 1e-4 * np.abs(want_r).max()
 
 
+def test_fused_attention_backward_node(be, oracle):
+    # src/backend/CUDAKernels.cpp:905-924: src 0..2 Q K V, 3 bias, 4 O, 5 dO, 6 LSE, 7..9 dQ dK dV; dbias in the
+    # node itself when op_params[5] != 0
+    rng = np.random.default_rng(16)
+    Bt, h, L, d = 1, 2, 50, 16
+    q, k, v, do = [rng.standard_normal((Bt, h, L, d)).astype(np.float32) for _ in range(4)]
+    bias = rng.standard_normal((Bt, h, L, L)).astype(np.float32)
+    o, lse = oracle.flash_attn_forward(q, k, v, bias)
+    want = oracle.flash_attn_backward(q, k, v, bias, o, do, lse)
+    for want_dbias in (1, 0):
+        dq, dk, dv = B.Tensor((d, L, h, Bt)), B.Tensor((d, L, h, Bt)), B.Tensor((d, L, h, Bt))
+        node = B.Tensor((L, L, h, Bt), B.F32, B.OP_FLASH_ATTN_BACK,
+                        [_leaf(be, q), _leaf(be, k), _leaf(be, v), _leaf(be, bias), _leaf(be, o), _leaf(be, do), _leaf(be, lse), dq, dk, dv])
+        node.set_param(0, float(1.0 / np.sqrt(d))).set_param(1, 0).set_param(5, want_dbias)
+        assert be.supports_op(node)
+        assert be.graph_compute([node]) == B.SUCCESS, be.last_error
+        for t, w in ((dq, want[0]), (dk, want[1]), (dv, want[2])):
+            assert np.abs(be.download(t).reshape(w.shape) - w).max() <= 1e-4 * np.abs(w).max()
+        if want_dbias:
+            assert np.abs(be.download(node).reshape(want[3].shape) - want[3]).max() <= 1e-4 * np.abs(want[3]).max()
+        else:
+            with pytest.raises(RuntimeError):
+                be.download(node)                       # not asked for: not even allocated
+
+
 def test_outer_prod_mean_back_node(be, oracle):
     # src/backend/CUDAKernels.cpp:1223-1245
     rng = np.random.default_rng(15)
