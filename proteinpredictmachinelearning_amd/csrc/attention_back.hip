@@ -153,13 +153,28 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_back_rows_kernel(const Att
         for (int kt = 0; kt < rows / 32; ++kt) {
             const int key0 = c0 + kt * 32;
             // ---- probabilities of this lane's query for its 16 keys of the tile
+            // bias of this lane's 16 keys, requested before the matrix work (16 bytes at a time)
+            float bv[16];
+            if (bias_row) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int key = key0 + 8 * g + 4 * half;
+                    if (key + 3 < L) {
+                        const v4f x = *reinterpret_cast<const v4f_u*>(bias_row + key);
+                        bv[4 * g] = x[0]; bv[4 * g + 1] = x[1]; bv[4 * g + 2] = x[2]; bv[4 * g + 3] = x[3];
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) bv[4 * g + i] = key + i < L ? bias_row[key + i] : 0.0f;
+                    }
+                }
+            }
             v16f st = tile_times_slice<DP>(lds_k + (kt * 32 + j) * KS + half * (DP / 2), qreg);
             v16f dp = tile_times_slice<DP>(lds_v + (kt * 32 + j) * KS + half * (DP / 2), doreg);
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int key = key0 + 8 * (r >> 2) + 4 * half + (r & 3);
                 float s2 = st[r];
-                if (bias_row && key < L) s2 = __builtin_fmaf(bias_row[key], LOG2E, s2);
+                if (bias_row) s2 = __builtin_fmaf(bv[r], LOG2E, s2);
                 const float pr = key < row_keys ? __builtin_amdgcn_exp2f(s2 - lse2) : 0.0f;
                 st[r] = pr * (dp[r] - D_i);            // dS
             }
@@ -260,6 +275,16 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_back_cols_kernel(const Att
         for (int qt = 0; qt < rows / 32; ++qt) {
             const int qbase = c0 + qt * 32;
             if (p.causal && qbase + 32 <= k0w) continue;           // every query of the tile precedes every key of the wave
+            // bias of this lane's key for its 16 queries of the tile, requested before the matrix work
+            float bv[16];
+            if (bias_plane) {
+                const float* bcol = bias_plane + (key < L ? key : L - 1);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int qq = qbase + 8 * (r >> 2) + 4 * half + (r & 3);
+                    bv[r] = bcol[static_cast<int64_t>(qq < L ? qq : L - 1) * L];
+                }
+            }
             // ---- S[query][key] and dO V^T, un-transposed: this lane's key, 16 of the tile's queries
             v16f st = tile_times_slice<DP>(lds_q + (qt * 32 + j) * KS + half * (DP / 2), kreg);
             v16f dp = tile_times_slice<DP>(lds_do + (qt * 32 + j) * KS + half * (DP / 2), vreg);
@@ -273,7 +298,7 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_back_cols_kernel(const Att
                     const int r = 4 * g + i;
                     const int qq = qbase + 8 * g + 4 * half + i;
                     float s2 = st[r];
-                    if (bias_plane && qq < L && key < L) s2 = __builtin_fmaf(bias_plane[static_cast<int64_t>(qq) * L + key], LOG2E, s2);
+                    if (bias_plane) s2 = __builtin_fmaf(bv[r], LOG2E, s2);
                     const bool seen = qq < L && (!p.causal || key <= qq);
                     const float pr = seen ? __builtin_amdgcn_exp2f(s2 - lse4[i]) : 0.0f;
                     st[r] = pr;                                    // P
