@@ -653,13 +653,14 @@ __device__ __forceinline__ void q8_linear_ws_body(
     extern __shared__ __attribute__((aligned(16))) uint8_t ws_lds[];
     v4i (*lds_a)[NBLK * 64] = reinterpret_cast<v4i (*)[NBLK * 64]>(ws_lds);
     constexpr size_t OFF_D = static_cast<size_t>(WS_NBUF) * NBLK * 1024;
-    constexpr size_t OFF_WD = OFF_D + static_cast<size_t>(WS_NBUF) * NBLK * 128;
-    constexpr size_t OFF_READY = OFF_WD + static_cast<size_t>(NW) * TPW * NBLK * 128;
+    constexpr size_t OFF_WD = OFF_D + static_cast<size_t>(WS_NBUF) * NBLK * 256;
+    constexpr size_t OFF_READY = OFF_WD + static_cast<size_t>(NW) * TPW * NBLK * 256;
     constexpr size_t OFF_WQ = OFF_READY + 16;
-    // activation scales [buffer][block][32 rows] and weight scales [wave][column tile][block][32 columns]:
-    // 64 consecutive floats are the operand of one scale MFMA over a pair of blocks
-    float (*lds_d)[NBLK * 32] = reinterpret_cast<float (*)[NBLK * 32]>(ws_lds + OFF_D);
-    float* lds_wd = reinterpret_cast<float*>(ws_lds + OFF_WD);
+    // activation scales [buffer][block][32 rows] and weight scales [wave][column tile][block][32 columns],
+    // kept as the bits of the halves they are, each followed by three zero halves: an entry is a lane's
+    // whole operand of the scale MFMA, and 64 consecutive entries serve one such MFMA over a pair of blocks
+    uint2 (*lds_d)[NBLK * 32] = reinterpret_cast<uint2 (*)[NBLK * 32]>(ws_lds + OFF_D);
+    uint2* lds_wd = reinterpret_cast<uint2*>(ws_lds + OFF_WD);
     // ready[b]: how many waves have written their share of the tile currently being put in buffer b
     // (counts up for the life of the kernel; the k-th filling of a buffer is complete at k * NW)
     unsigned* lds_ready = reinterpret_cast<unsigned*>(ws_lds + OFF_READY);
@@ -709,8 +710,10 @@ __device__ __forceinline__ void q8_linear_ws_body(
     constexpr bool LEAN = STAGE >= 64;
     auto load_tile_async = [&](int tile) {
         if constexpr (!ASYNC) return;
+        // the lane's part of the address is rebuilt here once per tile (a few instructions) from a copy of
+        // the lane number the optimizer cannot trace, rather than kept in registers across the loop
         int ln = lane;
-        if (LEAN) asm volatile("" : "+v"(ln));
+        asm volatile("" : "+v"(ln));
         const int grp = ln >> 2, c4 = ln & 3;
         const int urow = grp & 7, ublk = grp >> 3;
 #pragma unroll
@@ -777,7 +780,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
     static_assert(WL >= 0 && WL < TPW, "at least one column tile stays in registers");
     v4i wq[TPW - WL][NBLK];
     v4i* my_wq = lds_wq + static_cast<size_t>(wave) * WL * NBLK * 64 + lane;
-    float* my_wd = lds_wd + static_cast<size_t>(wave) * TPW * NBLK * 32 + lane;
+    uint2* my_wd = lds_wd + static_cast<size_t>(wave) * TPW * NBLK * 32 + lane;
     auto col_tile_of = [&](int t) {
         const int ct = t * NW + wave;                  // round t of the waves covers NW adjacent column tiles
         return ct < mct_pad ? ct : mct_pad - 1;        // tiles past the end repeat the last one; never stored
@@ -826,7 +829,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
             const BlockQuant bq = quantize_block_lane<false>(x0, x1);
             uint2* dst = reinterpret_cast<uint2*>(lds_a[buf]) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
             *dst = uint2{bq.q_lo, bq.q_hi};
-            if (c4 == 0) lds_d[buf][bl * 32 + row] = half_bits_to_float(bq.d_bits);
+            if (c4 == 0) lds_d[buf][bl * 32 + row] = uint2{bq.d_bits, 0u};
             if (DUMP && xq_dump) {
                 const int t = tok0 + row;
                 if (t < N) store_block_part(xq_dump + (static_cast<int64_t>(t) * NBLK + bl) * Q8_0_BYTES, c4, bq);
@@ -860,9 +863,9 @@ __device__ __forceinline__ void q8_linear_ws_body(
             const int ci = lane + 64 * r;
             if (ci < DCHUNKS) {
                 const uint2 h4 = draw[t][r];
-                const v4f d4{half_bits_to_float(static_cast<uint16_t>(h4.x & 0xffffu)), half_bits_to_float(static_cast<uint16_t>(h4.x >> 16)),
-                             half_bits_to_float(static_cast<uint16_t>(h4.y & 0xffffu)), half_bits_to_float(static_cast<uint16_t>(h4.y >> 16))};
-                *reinterpret_cast<v4f*>(my_wd - lane + t * NBLK * 32 + ci * 4) = d4;
+                v4i* dst = reinterpret_cast<v4i*>(my_wd - lane + t * NBLK * 32 + ci * 4);
+                dst[0] = v4i{static_cast<int>(h4.x & 0xffffu), 0, static_cast<int>(h4.x >> 16), 0};
+                dst[1] = v4i{static_cast<int>(h4.y & 0xffffu), 0, static_cast<int>(h4.y >> 16), 0};
             }
         }
     }
@@ -915,8 +918,11 @@ __device__ __forceinline__ void q8_linear_ws_body(
 #pragma unroll
         for (int r = 0; r < 16; ++r) { zero_i[r] = 0; zero_f[r] = 0.0f; }
         // Per pair of blocks: two int8 MFMAs (exact block sums, one result buffer per parity) and one
-        // v_mfma_f32_32x32x1_2b_f32 whose two 32x32 outer products are the scale tables
-        // d_a[row] * d_w[col] of both blocks (each the exact product of two halves).
+        // v_mfma_f32_32x32x4_2b_f16 whose two 32x32 outer products are the scale tables
+        // d_a[row] * d_w[col] of both blocks: the scale sits in the first of a lane's four k slots and
+        // the others hold zero, so each entry is the exact binary32 product of two halves.  (The
+        // half-precision form shares the matrix pipe with the int8 MFMAs and runs beside vector
+        // instructions; the single-precision form would hold up the vector pipe.)
         v16i sum_a, sum_b;
         v32f scl;
         v32f zero_f2;
@@ -924,7 +930,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
         for (int r = 0; r < 32; ++r) zero_f2[r] = 0.0f;
         v16f acc;
         // LDS operands of one pair of steps, fetched a pair ahead of the MFMAs that consume them
-        struct PairOps { v4i a0, a1, w0, w1; float da, dw; };
+        struct PairOps { v4i a0, a1, w0, w1; uint2 da, dw; };
         auto fetch_pair = [&](int st, PairOps& o) {
             const int t = st / NBLK, b = st % NBLK;
             o.a0 = lds_a[buf][b * 64 + lane];
@@ -935,6 +941,10 @@ __device__ __forceinline__ void q8_linear_ws_body(
                 o.w0 = my_wq[((t - (TPW - WL)) * NBLK + b) * 64];
                 o.w1 = my_wq[((t - (TPW - WL)) * NBLK + b + 1) * 64];
             }
+        };
+        auto scale_tables = [&](const uint2& da, const uint2& dw) {
+            typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+            return __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, da), __builtin_bit_cast(v4h, dw), zero_f2, 0, 0, 0);
         };
         auto block_sum = [&](int st, const v4i& a, const v4i& w_lds) {
             const int t = st / NBLK, b = st % NBLK;
@@ -1026,7 +1036,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
                 if constexpr (TWO_SETS) {
                     PairOps& cur = (pr & 1) ? po : pe;
                     PairOps& nxt = (pr & 1) ? pe : po;
-                    scl = __builtin_amdgcn_mfma_f32_32x32x1f32(cur.da, cur.dw, zero_f2, 0, 0, 0);
+                    scl = scale_tables(cur.da, cur.dw);
                     sum_b = block_sum(st + 1, cur.a1, cur.w1);
                     __builtin_amdgcn_sched_barrier(0);
                     settle(st, sum_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
@@ -1038,7 +1048,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
                     __builtin_amdgcn_sched_barrier(0);
                 } else {
                     // one block sum alive at a time; the other wave of the SIMD fills the waits
-                    scl = __builtin_amdgcn_mfma_f32_32x32x1f32(pe.da, pe.dw, zero_f2, 0, 0, 0);
+                    scl = scale_tables(pe.da, pe.dw);
                     sum_a = block_sum(st, pe.a0, pe.w0);
                     __builtin_amdgcn_sched_barrier(0);
                     settle(st, sum_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
@@ -1127,7 +1137,7 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
         wgs = (all_tiles + rounds - 1) / rounds;
     }
     const dim3 grid(wgs), block(NW * 64);
-    constexpr size_t lds = static_cast<size_t>(WS_NBUF) * NBLK * (1024 + 128) + static_cast<size_t>(NW) * TPW * NBLK * 128 + 16 +
+    constexpr size_t lds = static_cast<size_t>(WS_NBUF) * NBLK * (1024 + 256) + static_cast<size_t>(NW) * TPW * NBLK * 256 + 16 +
                            static_cast<size_t>(NW) * WL * NBLK * 1024;
     using KernelFn = void (*)(const uint8_t*, const float*, float*, int, int, int, int, int, uint8_t*, int32_t*);
     KernelFn fast, dump;
