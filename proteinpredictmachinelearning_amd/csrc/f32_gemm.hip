@@ -1,16 +1,22 @@
-// True-fp32 MFMA contractions for gfx950: dense GEMM with bias (mul_mat), batched transposed
-// GEMM with plane broadcast (out_prod, attention logits) and outer-product-mean in both of the
-// reference's layouts.  One kernel, three operand-access modes.
+// Binary32 contractions for gfx950: dense GEMM with bias (mul_mat), batched transposed GEMM with
+// plane broadcast (out_prod, attention logits), outer-product-mean in both of the reference's layouts,
+// triangle multiplication and the backward contractions of the last two.
 //
 // Reference behaviour restated here (paths relative to the reference tree):
 //   mul_mat          src/backend/CPUKernels.cpp:763-771   (bias first, k ascending)
 //   out_prod         src/backend/CPUKernels.cpp:787-887
 //   outer_prod_mean  src/backend/CPUKernels.cpp:982-1032, src/ops/MathUtils.cpp:387-437
 //
-// Reduction order: every output is accumulated in fp32 by v_mfma_f32_32x32x2_f32, k ascending in
-// steps of 2 (the instruction adds a[k]*b[k] + a[k+1]*b[k+1] to the accumulator), starting from
-// bias[n] (or 0); alpha multiplies the finished sum.
+// Arithmetic.  Binary32 operands are multiplied on the bf16 matrix pipe through an exact three-way
+// split (gemm_bf16x3_kernel, and gemm_planes_kernel for large problems, which splits ahead of the
+// matrix work): products to within 2^-23 of |a||b|, sums in binary32, sixteen k per accumulation step,
+// starting from bias[n] (or 0); alpha multiplies the finished sum.  Half operands go to the f16 matrix
+// pipe unchanged (gemm_f16_kernel).  The clamped contraction of the triangle multiplication, whose
+// result depends on how infinities propagate, stays on the fp32 pipe (gemm_f32_kernel:
+// v_mfma_f32_32x32x2_f32, k ascending two at a time).
 #include "common.hpp"
+
+#include <mutex>
 
 namespace ppmlhip {
 namespace {
@@ -18,7 +24,7 @@ namespace {
 constexpr int BM = 128, BN = 128, BK = 16;
 constexpr int LDS_LD = BM + 4;        // row pitch of the k-major LDS tiles (floats)
 
-enum LoadMode { LOAD_K_CONTIG = 0, LOAD_ROW_CONTIG = 1, LOAD_STRIDED = 2, LOAD_K_CONTIG_F16 = 3, LOAD_SPLIT_A = 4 };
+enum LoadMode { LOAD_K_CONTIG = 0, LOAD_ROW_CONTIG = 1, LOAD_STRIDED = 2, LOAD_SPLIT_A = 4 };
 
 struct GemmParams {
     const float* A;       // rows m: A(m,k) = A[m*a_rs + k*a_ks]
@@ -61,22 +67,6 @@ __device__ __forceinline__ void load_tile(const float* __restrict__ base, int64_
                 else {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) if (k + c < K) v[c] = p[c];
-                }
-            }
-        } else if (MODE == LOAD_K_CONTIG_F16) {
-            // the same tile shape read from halves: 4 of them (8 bytes) per thread and pass
-            const int r = (tid >> 2) + it * 64;
-            const int k = k0 + (tid & 3) * 4;
-            const int row = row0 + r;
-            if (row < nrows) {
-                const __half* p = reinterpret_cast<const __half*>(base) + static_cast<int64_t>(row) * rs + k;
-                if (k + 3 < K && (reinterpret_cast<uintptr_t>(p) & 7) == 0) {
-                    const uint2 raw = *reinterpret_cast<const uint2*>(p);
-                    const __half2 lo = *reinterpret_cast<const __half2*>(&raw.x), hi = *reinterpret_cast<const __half2*>(&raw.y);
-                    v[0] = __low2float(lo); v[1] = __high2float(lo); v[2] = __low2float(hi); v[3] = __high2float(hi);
-                } else {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) if (k + c < K) v[c] = __half2float(p[c]);
                 }
             }
         } else if (MODE == LOAD_ROW_CONTIG) {
@@ -141,9 +131,75 @@ __device__ __forceinline__ void store_tile(float* __restrict__ lds, int tid, con
     }
 }
 
+// work-group -> (plane, tile row, tile col); bands of 8 tile rows keep operand panels in one L2
+template <int TILE_M = BM>
+__device__ __forceinline__ void tile_of_group(const GemmParams& p, int& plane, int& m0, int& n0) {
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int total = tiles * p.np2 * p.np3;
+    const int idx = xcd_contiguous_index(blockIdx.x, total);
+    plane = idx / tiles;
+    int t = idx - plane * tiles;
+    const int band_rows = 8;
+    const int band = t / (band_rows * p.tiles_n);
+    t -= band * band_rows * p.tiles_n;
+    const int rows_here = (p.tiles_m - band * band_rows) < band_rows ? (p.tiles_m - band * band_rows) : band_rows;
+    const int tm = band * band_rows + t % rows_here;
+    const int tn = t / rows_here;
+    m0 = tm * TILE_M;
+    n0 = tn * BN;
+}
+
+// The finished accumulators of one wave (TI x 2 tiles of 32 x 32) (rows from m_base, columns from n_base) go to C.
 // CLAMP: the finite guard of the triangle multiplication (src/backend/CPUKernels.cpp:957-962): NaN -> 0,
 // values beyond +-1e4 -> +-1e4.  A compile-time property: a run-time test in this store loop costs the
 // other contractions a quarter of their speed.
+template <bool SPLIT_C, bool STREAM_C, bool BIAS_LAST, bool CLAMP, int TI = 2>
+__device__ __forceinline__ void store_acc(const GemmParams& p, float* __restrict__ C, const v16f (&acc)[TI][2],
+                                          int m_base, int n_base, int lane) {
+    const int j = lane & 31;
+    const bool scale = p.alpha != 1.0f;
+#pragma unroll
+    for (int ti = 0; ti < TI; ++ti) {
+        // The lane's sixteen rows of this tile are first + 8 * (r / 4) + r % 4.  With a compound row
+        // index the quotient and remainder are formed once, for `first`, and stepped from there: a
+        // division per element would cost more than the contraction itself on large outputs.
+        const int first = m_base + ti * 32 + 4 * (lane >> 5);
+        const int q0 = SPLIT_C ? first / p.c_lm : 0;
+        const int r0 = SPLIT_C ? first - q0 * p.c_lm : 0;
+        const bool one_wrap = p.c_lm >= 32;            // the sixteen rows span 28: at most one carry
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj) {
+            const int n = n_base + tj * 32 + j;
+            if (n >= p.N) continue;
+            const float tail_bias = (BIAS_LAST && p.bias) ? p.bias[n] : 0.0f;
+            int64_t coff;
+            if (SPLIT_C) coff = static_cast<int64_t>(n / p.c_ln) * p.c_no + static_cast<int64_t>(n % p.c_ln) * p.c_ni;
+            else         coff = static_cast<int64_t>(n) * p.c_ni;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int step = 8 * (r >> 2) + (r & 3);
+                const int m = first + step;
+                if (m >= p.M) continue;
+                int64_t roff;
+                if (SPLIT_C) {
+                    int q = q0, rem = r0 + step;
+                    if (one_wrap) { if (rem >= p.c_lm) { rem -= p.c_lm; ++q; } }
+                    else { q += rem / p.c_lm; rem %= p.c_lm; }
+                    roff = static_cast<int64_t>(q) * p.c_mo + static_cast<int64_t>(rem) * p.c_mi;
+                } else {
+                    roff = static_cast<int64_t>(m) * p.c_mi;
+                }
+                float v = acc[ti][tj][r];
+                if (scale) v *= p.alpha;
+                if (BIAS_LAST) v += tail_bias;
+                if (CLAMP) v = (v != v) ? 0.0f : (v > 1e4f ? 1e4f : (v < -1e4f ? -1e4f : v));
+                if (STREAM_C) __builtin_nontemporal_store(v, &C[roff + coff]);
+                else C[roff + coff] = v;
+            }
+        }
+    }
+}
+
 template <int MODE, bool SPLIT_C, bool STREAM_C, bool CLAMP = false>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
     __shared__ __attribute__((aligned(16))) float lds_a[BK * LDS_LD];
@@ -154,32 +210,19 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
     const int j = lane & 31, hh = lane >> 5;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
 
-    // work-group -> (plane, tile row, tile col); bands of 8 tile rows keep operand panels in one L2
-    const int tiles = p.tiles_m * p.tiles_n;
-    const int total = tiles * p.np2 * p.np3;
-    const int idx = xcd_contiguous_index(blockIdx.x, total);
-    const int plane = idx / tiles;
-    int t = idx - plane * tiles;
-    const int band_rows = 8;
-    const int band = t / (band_rows * p.tiles_n);
-    t -= band * band_rows * p.tiles_n;
-    const int rows_here = (p.tiles_m - band * band_rows) < band_rows ? (p.tiles_m - band * band_rows) : band_rows;
-    const int tm = band * band_rows + t % rows_here;
-    const int tn = t / rows_here;
-    const int m0 = tm * BM, n0 = tn * BN;
+    int plane, m0, n0;
+    tile_of_group(p, plane, m0, n0);
 
     const int p2 = plane % p.np2, p3 = plane / p.np2;
     const float* A = p.A + p2 * p.a_p2 + p3 * p.a_p3;
     const float* B = p.B + (p2 / p.b_div2) * p.b_p2 + (p3 / p.b_div3) * p.b_p3;
     float* C = p.C + p2 * p.c_p2 + p3 * p.c_p3;
 
-    // halves in: the bias joins the finished sum (the CPU branch of the reference adds it last)
-    constexpr bool BIAS_LAST = MODE == LOAD_K_CONTIG_F16;
     v16f acc[2][2];
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj) {
         const int n = n0 + wn + tj * 32 + j;
-        const float b0 = (p.bias && !BIAS_LAST && n < p.N) ? p.bias[n] : 0.0f;
+        const float b0 = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
 #pragma unroll
         for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
@@ -215,32 +258,409 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
         __syncthreads();
     }
 
-    const bool scale = p.alpha != 1.0f;
+    store_acc<SPLIT_C, STREAM_C, false, CLAMP>(p, C, acc, m0 + wm, n0 + wn, lane);
+}
+
+// ------------------------------------------------------------------------------------------
+// The same contraction on the bf16 matrix pipe, sixteen times as fast as the fp32 one and able to run
+// beside vector instructions.  A binary32 number is the exact sum of three bf16 numbers
+// (x = x1 + x2 + x3: 8 + 8 + 8 significant bits, taken off the top by truncation), so a product is
+// the exact sum of nine bf16 x bf16 products, each of which the matrix pipe forms exactly and adds
+// into a binary32 accumulator.  Six of them are kept -- (1,1) (1,2) (2,1) (1,3) (3,1) (2,2) -- and the
+// three dropped ones are below 2^-23 of |a||b| together, i.e. about one rounding of a binary32
+// product; the accumulation itself is binary32 as before.  What differs from the fp32 pipe is the
+// order of the roundings inside a group of 16 k, not their size.
+// Non-finite inputs: x - x1 is NaN for an infinite x, so +-inf in an operand gives NaN where the fp32
+// pipe gives +-inf or NaN; the clamped instances (whose result depends on that) stay on the fp32 pipe.
+constexpr int SPLIT_PITCH = 48;                   // bytes per tile row in a plane: 16 bf16, then 16 bytes of padding
+constexpr int SPLIT_PLANE = BM * SPLIT_PITCH;     // one of the three bf16 planes of a 128 x 16 operand tile
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+// four consecutive k of one tile row -> four bf16 (8 bytes) in each of the three planes, returned packed
+__device__ __forceinline__ void split4(const v4f& v, uint2 (&out)[3]) {
+    uint32_t t1[4], t2[4], t3[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t b1 = __float_as_uint(v[c]) & 0xffff0000u;
+        const float r1 = v[c] - __uint_as_float(b1);              // exact: at most 16 significant bits left
+        const uint32_t b2 = __float_as_uint(r1) & 0xffff0000u;
+        const float r2 = r1 - __uint_as_float(b2);                // exact: at most 8 significant bits left
+        t1[c] = b1; t2[c] = b2; t3[c] = __float_as_uint(r2);
+    }
+    // the upper halves of two words side by side
+    const auto pack = [](uint32_t lo, uint32_t hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); };
+    out[0] = uint2{pack(t1[0], t1[1]), pack(t1[2], t1[3])};
+    out[1] = uint2{pack(t2[0], t2[1]), pack(t2[2], t2[3])};
+    out[2] = uint2{pack(t3[0], t3[1]), pack(t3[2], t3[3])};
+}
+
+// A thread's share of a 128 x 16 operand tile goes to the planes.  Operands with contiguous rows are
+// read one row and eight consecutive k per thread (eight loads, each contiguous across the lanes), the
+// others two rows and four consecutive k each.
+template <int MODE>
+__device__ __forceinline__ void split_store(uint8_t* __restrict__ planes, int tid, const v4f (&reg)[2]) {
+    uint2 lo[3], hi[3];
+    split4(reg[0], lo);
+    split4(reg[1], hi);
+    if (MODE == LOAD_ROW_CONTIG) {
+        uint8_t* dst = planes + (tid & 127) * SPLIT_PITCH + (tid >> 7) * 16;
+#pragma unroll
+        for (int s = 0; s < 3; ++s) *reinterpret_cast<uint4*>(dst + s * SPLIT_PLANE) = uint4{lo[s].x, lo[s].y, hi[s].x, hi[s].y};
+    } else {
+        uint8_t* dst = planes + (tid >> 2) * SPLIT_PITCH + (tid & 3) * 8;
+#pragma unroll
+        for (int s = 0; s < 3; ++s) {
+            *reinterpret_cast<uint2*>(dst + s * SPLIT_PLANE) = lo[s];
+            *reinterpret_cast<uint2*>(dst + s * SPLIT_PLANE + 64 * SPLIT_PITCH) = hi[s];
+        }
+    }
+}
+
+// one row, eight consecutive k of an operand whose rows are contiguous in memory: A(row, k) = base[k * ks + row]
+__device__ __forceinline__ void load_rows8(const float* __restrict__ base, int64_t ks, int row0, int nrows, int k0, int K,
+                                           int tid, v4f (&reg)[2]) {
+    const int row = row0 + (tid & 127);
+    const int kb = k0 + (tid >> 7) * 8;
+    const float* src = base + static_cast<int64_t>(kb) * ks + row;
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+        reg[c >> 2][c & 3] = (row < nrows && kb + c < K) ? src[static_cast<int64_t>(c) * ks] : 0.0f;
+}
+
+template <int MODE, bool SPLIT_C, bool STREAM_C>
+__global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * SPLIT_PLANE];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[3 * SPLIT_PLANE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 31, hh = lane >> 5;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+
+    int plane, m0, n0;
+    tile_of_group(p, plane, m0, n0);
+    const int p2 = plane % p.np2, p3 = plane / p.np2;
+    const float* A = p.A + p2 * p.a_p2 + p3 * p.a_p3;
+    const float* B = p.B + (p2 / p.b_div2) * p.b_p2 + (p3 / p.b_div3) * p.b_p3;
+    float* C = p.C + p2 * p.c_p2 + p3 * p.c_p3;
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+        const int n = n0 + wn + tj * 32 + j;
+        const float b0 = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+#pragma unroll
+        for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = b0;
+    }
+
+    v4f ra[2], rb[2];
+    constexpr int MODE_B = MODE == LOAD_SPLIT_A ? LOAD_STRIDED : MODE;
+    const auto load_both = [&](int k0) {
+        if (MODE == LOAD_ROW_CONTIG) {
+            load_rows8(A, p.a_ks, m0, p.M, k0, p.K, tid, ra);
+            load_rows8(B, p.b_ks, n0, p.N, k0, p.K, tid, rb);
+        } else {
+            if (MODE == LOAD_SPLIT_A) load_tile_split(A, p, m0, p.M, k0, p.K, tid, ra);
+            else load_tile<MODE>(A, p.a_rs, p.a_ks, m0, p.M, k0, p.K, tid, ra);
+            load_tile<MODE_B>(B, p.b_rs, p.b_ks, n0, p.N, k0, p.K, tid, rb);
+        }
+    };
+    load_both(0);
+
+    // a lane's fragment of a plane: its row's k = 8 * hh .. 8 * hh + 7, sixteen bytes
+    const uint8_t* frag_a = lds_a + (wm + j) * SPLIT_PITCH + hh * 16;
+    const uint8_t* frag_b = lds_b + (wn + j) * SPLIT_PITCH + hh * 16;
+
+    for (int k0 = 0; k0 < p.K; k0 += BK) {
+        split_store<MODE>(lds_a, tid, ra);
+        split_store<MODE>(lds_b, tid, rb);
+        __syncthreads();
+        if (k0 + BK < p.K) load_both(k0 + BK);
+        v8bf fa[2][3], fb[2][3];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s = 0; s < 3; ++s) {
+                fa[t][s] = *reinterpret_cast<const v8bf*>(frag_a + s * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
+                fb[t][s] = *reinterpret_cast<const v8bf*>(frag_b + s * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
+            }
+        // smallest products first; the four accumulators take turns, so no MFMA waits for the one before it
+        constexpr int TERMS[6][2] = {{1, 1}, {2, 0}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};
+#pragma unroll
+        for (int q = 0; q < 6; ++q)
+#pragma unroll
+            for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < 2; ++tj)
+                    acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][TERMS[q][0]], fb[tj][TERMS[q][1]], acc[ti][tj], 0, 0, 0);
+        __syncthreads();
+    }
+
+    store_acc<SPLIT_C, STREAM_C, false, false>(p, C, acc, m0 + wm, n0 + wn, lane);
+}
+
+// ------------------------------------------------------------------------------------------
+// F16 x F16 -> F32 (mul_mat with both operands in halves, k contiguous): the halves go to the matrix
+// pipe as they are.  v_mfma_f32_32x32x16_f16 forms each product exactly (22 significant bits) and adds
+// into a binary32 accumulator, which is the reference's arithmetic (src/backend/CPUKernels.cpp:763-771
+// with half operands converted on load) up to the order of the additions; the bias joins the finished
+// sum, as the CPU branch of the reference does.
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ uint2 load_halves4(const uint16_t* __restrict__ base, int64_t rs, int row, int nrows, int k, int K) {
+    uint2 v{0u, 0u};
+    if (row < nrows) {
+        const uint16_t* p = base + static_cast<int64_t>(row) * rs + k;
+        if (k + 3 < K && (reinterpret_cast<uintptr_t>(p) & 7) == 0) {
+            v = *reinterpret_cast<const uint2*>(p);
+        } else {
+            uint32_t h[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) if (k + c < K) h[c] = p[c];
+            v = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+        }
+    }
+    return v;
+}
+
+template <bool STREAM_C>
+__global__ __launch_bounds__(256) void gemm_f16_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[SPLIT_PLANE];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[SPLIT_PLANE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 31, hh = lane >> 5;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    int plane, m0, n0;
+    tile_of_group(p, plane, m0, n0);                  // the launcher passes a single plane
+    const uint16_t* A = reinterpret_cast<const uint16_t*>(p.A);
+    const uint16_t* B = reinterpret_cast<const uint16_t*>(p.B);
+
+    v16f acc[2][2];
 #pragma unroll
     for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
-        for (int tj = 0; tj < 2; ++tj) {
-            const int n = n0 + wn + tj * 32 + j;
-            if (n >= p.N) continue;
-            const float tail_bias = (BIAS_LAST && p.bias) ? p.bias[n] : 0.0f;
-            int64_t coff;
-            if (SPLIT_C) coff = static_cast<int64_t>(n / p.c_ln) * p.c_no + static_cast<int64_t>(n % p.c_ln) * p.c_ni;
-            else         coff = static_cast<int64_t>(n) * p.c_ni;
+        for (int tj = 0; tj < 2; ++tj)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm + ti * 32 + mfma32_row(r, lane);
-                if (m >= p.M) continue;
-                int64_t roff;
-                if (SPLIT_C) roff = static_cast<int64_t>(m / p.c_lm) * p.c_mo + static_cast<int64_t>(m % p.c_lm) * p.c_mi;
-                else         roff = static_cast<int64_t>(m) * p.c_mi;
-                float v = acc[ti][tj][r];
-                if (scale) v *= p.alpha;
-                if (BIAS_LAST) v += tail_bias;
-                if (CLAMP) v = (v != v) ? 0.0f : (v > 1e4f ? 1e4f : (v < -1e4f ? -1e4f : v));
-                if (STREAM_C) __builtin_nontemporal_store(v, &C[roff + coff]);
-                else C[roff + coff] = v;
-            }
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
+
+    // a thread's share of a 128 x 16 tile: rows tid / 4 and tid / 4 + 64, four consecutive k each
+    uint2 ra[2], rb[2];
+    const auto load_both = [&](int k0) {
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            ra[it] = load_halves4(A, p.a_rs, m0 + (tid >> 2) + it * 64, p.M, k0 + (tid & 3) * 4, p.K);
+            rb[it] = load_halves4(B, p.b_rs, n0 + (tid >> 2) + it * 64, p.N, k0 + (tid & 3) * 4, p.K);
         }
+    };
+    load_both(0);
+    const int put = (tid >> 2) * SPLIT_PITCH + (tid & 3) * 8;
+    const uint8_t* frag_a = lds_a + (wm + j) * SPLIT_PITCH + hh * 16;
+    const uint8_t* frag_b = lds_b + (wn + j) * SPLIT_PITCH + hh * 16;
+
+    for (int k0 = 0; k0 < p.K; k0 += BK) {
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            *reinterpret_cast<uint2*>(lds_a + put + it * 64 * SPLIT_PITCH) = ra[it];
+            *reinterpret_cast<uint2*>(lds_b + put + it * 64 * SPLIT_PITCH) = rb[it];
+        }
+        __syncthreads();
+        if (k0 + BK < p.K) load_both(k0 + BK);
+        v8h fa[2], fb[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            fa[t] = *reinterpret_cast<const v8h*>(frag_a + t * 32 * SPLIT_PITCH);
+            fb[t] = *reinterpret_cast<const v8h*>(frag_b + t * 32 * SPLIT_PITCH);
+        }
+#pragma unroll
+        for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < 2; ++tj)
+                acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[ti], fb[tj], acc[ti][tj], 0, 0, 0);
+        __syncthreads();
+    }
+    store_acc<false, STREAM_C, true, false>(p, p.C, acc, m0 + wm, n0 + wn, lane);
+}
+
+// ------------------------------------------------------------------------------------------
+// Large contractions split their operands once, ahead of the matrix work, instead of in every
+// work-group that reads them (a 128-row panel of A is read by every tile column): the planes go to a
+// workspace in the order the contraction consumes them,
+//     [plane s][chunk of 16 k][row, padded to whole tiles][16 bf16]   (32 bytes per row and chunk)
+// so a work-group's share of one chunk is 4 KB of contiguous memory per plane, and its main loop is
+// loads, LDS traffic and MFMAs only.
+struct SplitJob {
+    const float* src;
+    uint8_t* dst;
+    int rows, rows_pad, K, chunks;
+    int64_t rs, ks;                                   // element (row, k) at src[row * rs + k * ks] ...
+    int lm, lk;                                       // ... or, with lm > 0, at the compound address of LOAD_SPLIT_A
+    int64_t mo, mi, ko, ki;
+};
+
+template <bool KS1, bool COMPOUND>
+__global__ __launch_bounds__(256) void split_operand_kernel(const SplitJob jb) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int kq = static_cast<int>(idx & 1);
+    const int64_t rc = idx >> 1;
+    const int row = static_cast<int>(rc % jb.rows_pad);
+    const int c = static_cast<int>(rc / jb.rows_pad);
+    if (c >= jb.chunks) return;
+    const int kb = c * BK + kq * 8;
+    v4f v[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    if (row < jb.rows) {
+        if (COMPOUND) {
+            const int64_t roff = static_cast<int64_t>(row / jb.lm) * jb.mo + static_cast<int64_t>(row % jb.lm) * jb.mi;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int k = kb + i;
+                if (k < jb.K) v[i >> 2][i & 3] = jb.src[roff + static_cast<int64_t>(k / jb.lk) * jb.ko + static_cast<int64_t>(k % jb.lk) * jb.ki];
+            }
+        } else if (KS1) {
+            const float* src = jb.src + static_cast<int64_t>(row) * jb.rs + kb;
+            if (kb + 7 < jb.K) {
+                v[0] = *reinterpret_cast<const v4f_u*>(src);
+                v[1] = *reinterpret_cast<const v4f_u*>(src + 4);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) if (kb + i < jb.K) v[i >> 2][i & 3] = src[i];
+            }
+        } else {
+            const float* src = jb.src + static_cast<int64_t>(row) * jb.rs + static_cast<int64_t>(kb) * jb.ks;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) if (kb + i < jb.K) v[i >> 2][i & 3] = src[static_cast<int64_t>(i) * jb.ks];
+        }
+    }
+    uint2 lo[3], hi[3];
+    split4(v[0], lo);
+    split4(v[1], hi);
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+        uint8_t* dst = jb.dst + ((static_cast<int64_t>(s) * jb.chunks + c) * jb.rows_pad + row) * 32 + kq * 16;
+        *reinterpret_cast<uint4*>(dst) = uint4{lo[s].x, lo[s].y, hi[s].x, hi[s].y};
+    }
+}
+
+// Work-group tile 256 x 128, four waves of 128 x 64 each (eight accumulator tiles): a fragment read from
+// LDS feeds twice as many MFMAs as in the 64 x 64 arrangement, and it is LDS bandwidth that bounds this loop.
+constexpr int PBM = 256;
+constexpr int PLANES_MIN_TILES = 8;              // 128-wide tiles per side from which the operands are split ahead
+template <bool SPLIT_C, bool STREAM_C>
+__global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p, const uint8_t* __restrict__ wa,
+                                                             const uint8_t* __restrict__ wb, int chunks, int ma_pad, int nb_pad) {
+    constexpr int A_PLANE = PBM * SPLIT_PITCH;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * A_PLANE];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[3 * SPLIT_PLANE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 31, hh = lane >> 5;
+    const int wm = (wave >> 1) * 128, wn = (wave & 1) * 64;
+
+    int plane, m0, n0;
+    tile_of_group<PBM>(p, plane, m0, n0);             // single plane: the launcher takes this path for np2 = np3 = 1 only
+
+    v16f acc[4][2];
+#pragma unroll
+    for (int tj = 0; tj < 2; ++tj) {
+        const int n = n0 + wn + tj * 32 + j;
+        const float b0 = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = b0;
+    }
+
+    const size_t a_chunk = static_cast<size_t>(ma_pad) * 32, b_chunk = static_cast<size_t>(nb_pad) * 32;
+    const size_t a_plane = a_chunk * chunks, b_plane = b_chunk * chunks;
+    const uint8_t* ga = wa + static_cast<size_t>(m0) * 32 + tid * 16;
+    const uint8_t* gb = wb + static_cast<size_t>(n0) * 32 + tid * 16;
+    v4i ra[3][2], rb[3];
+    const auto load_both = [&](int c) {
+#pragma unroll
+        for (int s = 0; s < 3; ++s) {
+            ra[s][0] = *reinterpret_cast<const v4i*>(ga + s * a_plane + c * a_chunk);
+            ra[s][1] = *reinterpret_cast<const v4i*>(ga + s * a_plane + c * a_chunk + 128 * 32);
+            rb[s] = *reinterpret_cast<const v4i*>(gb + s * b_plane + c * b_chunk);
+        }
+    };
+    load_both(0);
+    const int put = (tid >> 1) * SPLIT_PITCH + (tid & 1) * 16;
+    const uint8_t* frag_a = lds_a + (wm + j) * SPLIT_PITCH + hh * 16;
+    const uint8_t* frag_b = lds_b + (wn + j) * SPLIT_PITCH + hh * 16;
+
+    for (int c = 0; c < chunks; ++c) {
+#pragma unroll
+        for (int s = 0; s < 3; ++s) {
+            *reinterpret_cast<v4i*>(lds_a + s * A_PLANE + put) = ra[s][0];
+            *reinterpret_cast<v4i*>(lds_a + s * A_PLANE + 128 * SPLIT_PITCH + put) = ra[s][1];
+            *reinterpret_cast<v4i*>(lds_b + s * SPLIT_PLANE + put) = rb[s];
+        }
+        __syncthreads();
+        if (c + 1 < chunks) load_both(c + 1);
+        v8bf fb[2][3];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s = 0; s < 3; ++s) fb[t][s] = *reinterpret_cast<const v8bf*>(frag_b + s * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
+        constexpr int TERMS[6][2] = {{1, 1}, {2, 0}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti) {
+            v8bf fa[3];
+#pragma unroll
+            for (int s = 0; s < 3; ++s) fa[s] = *reinterpret_cast<const v8bf*>(frag_a + s * A_PLANE + ti * 32 * SPLIT_PITCH);
+#pragma unroll
+            for (int q = 0; q < 6; ++q)
+#pragma unroll
+                for (int tj = 0; tj < 2; ++tj)
+                    acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[TERMS[q][0]], fb[tj][TERMS[q][1]], acc[ti][tj], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    store_acc<SPLIT_C, STREAM_C, false, false, 4>(p, p.C, acc, m0 + wm, n0 + wn, lane);
+}
+
+// Stream-ordered workspace for the planes: a pool of this library's own per device, which keeps what it
+// has allocated (release threshold at the maximum), so after the first call an allocation is a list
+// operation ordered on the caller's stream; freeing is ordered on that stream as well, which makes reuse
+// from other streams safe without the library tracking anything.  Returns null when the device has no pool.
+hipMemPool_t workspace_pool() {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static hipMemPool_t pools[MAX_DEVICES];
+    static bool tried[MAX_DEVICES];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) { (void)hipGetLastError(); return nullptr; }
+    std::lock_guard<std::mutex> guard(mu);
+    if (!tried[dev]) {
+        tried[dev] = true;
+        hipMemPoolProps props{};
+        props.allocType = hipMemAllocationTypePinned;
+        props.handleTypes = hipMemHandleTypeNone;
+        props.location.type = hipMemLocationTypeDevice;
+        props.location.id = dev;
+        if (hipMemPoolCreate(&pools[dev], &props) != hipSuccess) {
+            (void)hipGetLastError();
+            pools[dev] = nullptr;
+        } else {
+            uint64_t keep = ~0ull;
+            (void)hipMemPoolSetAttribute(pools[dev], hipMemPoolAttrReleaseThreshold, &keep);
+        }
+    }
+    return pools[dev];
+}
+
+int launch_split(const SplitJob& jb, hipStream_t stream) {
+    const int64_t threads = static_cast<int64_t>(jb.chunks) * jb.rows_pad * 2;
+    const dim3 grid(static_cast<unsigned>((threads + 255) / 256)), block(256);
+    if (jb.lm > 0)       hipLaunchKernelGGL((split_operand_kernel<false, true>), grid, block, 0, stream, jb);
+    else if (jb.ks == 1) hipLaunchKernelGGL((split_operand_kernel<true, false>), grid, block, 0, stream, jb);
+    else                 hipLaunchKernelGGL((split_operand_kernel<false, false>), grid, block, 0, stream, jb);
+    return check_launch("split_operand_kernel");
 }
 
 int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
@@ -257,14 +677,53 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
     int mode = LOAD_STRIDED;
     if (p.a_ks == 1 && p.b_ks == 1) mode = LOAD_K_CONTIG;
     else if (p.a_rs == 1 && p.b_rs == 1) mode = LOAD_ROW_CONTIG;
-#define PPML_LAUNCH(MODE, SPLIT)                                                                      \
+    // Large single-plane contractions split their operands ahead of the matrix work (every element would
+    // otherwise be split by each work-group that reads it); when no workspace is to be had they take the
+    // same path as the small ones.
+    if (!p.clamp && !p.f16_in && p.np2 * p.np3 == 1 && p.tiles_m >= PLANES_MIN_TILES && p.tiles_n >= PLANES_MIN_TILES) {
+        const int chunks = (p.K + BK - 1) / BK;
+        const int tiles_m = (p.M + PBM - 1) / PBM;
+        const int ma_pad = tiles_m * PBM, nb_pad = p.tiles_n * BN;
+        const size_t a_bytes = static_cast<size_t>(3) * chunks * ma_pad * 32, b_bytes = static_cast<size_t>(3) * chunks * nb_pad * 32;
+        uint8_t* ws = nullptr;
+        hipMemPool_t pool = workspace_pool();
+        if (pool && hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), a_bytes + b_bytes, pool, stream) != hipSuccess) {
+            (void)hipGetLastError();
+            ws = nullptr;
+        }
+        if (ws) {
+            GemmParams q = p;
+            q.tiles_m = tiles_m;
+            const dim3 pgrid(static_cast<unsigned>(q.tiles_m * q.tiles_n));
+            const SplitJob ja{p.A, ws, p.M, ma_pad, p.K, chunks, p.a_rs, p.a_ks, p.a_lm, p.a_lk, p.a_mo, p.a_mi, p.a_ko, p.a_ki};
+            const SplitJob jb{p.B, ws + a_bytes, p.N, nb_pad, p.K, chunks, p.b_rs, p.b_ks, 0, 0, 0, 0, 0, 0};
+            int rc = launch_split(ja, stream);
+            if (rc == RC_OK) rc = launch_split(jb, stream);
+            if (rc == RC_OK) {
+                if (split) { if (p.stream_c) hipLaunchKernelGGL((gemm_planes_kernel<true, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad);
+                             else hipLaunchKernelGGL((gemm_planes_kernel<true, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad); }
+                else       { if (p.stream_c) hipLaunchKernelGGL((gemm_planes_kernel<false, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad);
+                             else hipLaunchKernelGGL((gemm_planes_kernel<false, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad); }
+                rc = check_launch(what);
+            }
+            if (hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();
+            return rc;
+        }
+    }
+#define PPML_LAUNCH_BF16(MODE, SPLIT)                                                                 \
     do {                                                                                              \
-        if (p.stream_c) hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, true>), grid, block, 0, stream, p);  \
-        else hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, false>), grid, block, 0, stream, p);    \
+        if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_kernel<MODE, SPLIT, true>), grid, block, 0, stream, p);  \
+        else hipLaunchKernelGGL((gemm_bf16x3_kernel<MODE, SPLIT, false>), grid, block, 0, stream, p); \
     } while (0)
     if (p.a_lm > 0) {
         if (split || p.f16_in || p.clamp) { set_error("%s: no split-operand instance for this addressing", what); return RC_BAD_ARGS; }
-        PPML_LAUNCH(LOAD_SPLIT_A, false);
+        PPML_LAUNCH_BF16(LOAD_SPLIT_A, false);
+    }
+    else if (!p.clamp && !p.f16_in) {
+        // binary32 operands without the finite guard: the contraction runs on the bf16 matrix pipe
+        if (mode == LOAD_K_CONTIG)        { if (split) PPML_LAUNCH_BF16(LOAD_K_CONTIG, true);   else PPML_LAUNCH_BF16(LOAD_K_CONTIG, false); }
+        else if (mode == LOAD_ROW_CONTIG) { if (split) PPML_LAUNCH_BF16(LOAD_ROW_CONTIG, true); else PPML_LAUNCH_BF16(LOAD_ROW_CONTIG, false); }
+        else                              { if (split) PPML_LAUNCH_BF16(LOAD_STRIDED, true);    else PPML_LAUNCH_BF16(LOAD_STRIDED, false); }
     }
     else if (p.clamp) {
         if (split || p.stream_c || p.f16_in) { set_error("%s: no clamped instance for this addressing", what); return RC_BAD_ARGS; }
@@ -272,11 +731,12 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
         else if (mode == LOAD_ROW_CONTIG) hipLaunchKernelGGL((gemm_f32_kernel<LOAD_ROW_CONTIG, false, false, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((gemm_f32_kernel<LOAD_STRIDED, false, false, true>), grid, block, 0, stream, p);
     }
-    else if (p.f16_in)                { PPML_LAUNCH(LOAD_K_CONTIG_F16, false); }
-    else if (mode == LOAD_K_CONTIG)   { if (split) PPML_LAUNCH(LOAD_K_CONTIG, true);   else PPML_LAUNCH(LOAD_K_CONTIG, false); }
-    else if (mode == LOAD_ROW_CONTIG) { if (split) PPML_LAUNCH(LOAD_ROW_CONTIG, true); else PPML_LAUNCH(LOAD_ROW_CONTIG, false); }
-    else                              { if (split) PPML_LAUNCH(LOAD_STRIDED, true);    else PPML_LAUNCH(LOAD_STRIDED, false); }
-#undef PPML_LAUNCH
+    else {
+        if (split || p.np2 * p.np3 != 1 || p.a_ks != 1 || p.b_ks != 1) { set_error("%s: no F16 instance for this addressing", what); return RC_BAD_ARGS; }
+        if (p.stream_c) hipLaunchKernelGGL((gemm_f16_kernel<true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((gemm_f16_kernel<false>), grid, block, 0, stream, p);
+    }
+#undef PPML_LAUNCH_BF16
     return check_launch(what);
 }
 

@@ -1,10 +1,14 @@
 """GPU parity of the f32 contractions (mul_mat, out_prod, outer-product-mean) against the CPU oracle.
 
 Bar: 1e-4 relative.  Two measures are checked: normwise (max |diff| / max |want|) and the sharper
-elementwise bound |diff| <= 1e-4 * sum_k |a_k b_k|.  Reduction order on the GPU: fp32 MFMA
-accumulation, k ascending two at a time, starting from the bias; the oracle adds one product at a
-time.  On inputs whose products and partial sums are exact in binary32 (the reference's own test
-inputs) the two orders agree exactly, and the tests require equality there.
+elementwise bound |diff| <= 1e-4 * sum_k |a_k b_k|.  Arithmetic on the GPU: every binary32 operand is
+the exact sum of three bf16 numbers; six of the nine partial products (all but the three smallest,
+together below 2^-23 of |a||b|) go through the bf16 matrix pipe, which forms them exactly and adds them
+into a binary32 accumulator that starts from the bias, sixteen k at a time; the oracle adds one product
+at a time.  On inputs whose products and partial sums are exact in binary32 (the reference's own test
+inputs) the results agree exactly, and the tests require equality there.  The clamped contraction
+(triangle multiplication) and the F16 one use the fp32 matrix pipe, k ascending two at a time.
+test_split_contraction_is_binary32_grade pins the error of the split arithmetic against float64.
 """
 import math
 
@@ -210,13 +214,69 @@ def test_dense_outer_product_mean_stress_shape_properties(ops):
     b = torch.randn(N, LD, device="cuda", generator=g) * 0.1
     o = ops.mul_mat_tn(a, b, 1.0 / N)
     o_t = ops.mul_mat_tn(b, a, 1.0 / N)
-    assert torch.equal(o.t(), o_t)          # same products, same order along k
+    # the same products; the two mixed-size partial products of a pair enter the accumulator in the other
+    # order when the operands swap, which moves the last bit
+    assert (o.t() - o_t).abs().max().item() <= 1e-6 * o.abs().max().item()
     o2 = ops.mul_mat_tn(a * 2.0, b, 1.0 / N)
     assert torch.equal(o2, o * 2.0)
     rows = torch.tensor([0, 1, 127, 128, 5000, 12287], device="cuda")
     want = (a[:, rows].double().t() @ b.double()) / N
     err = (o[rows].double() - want).abs().max().item()
     assert err <= RTOL * want.abs().max().item()
+
+
+def _f64_error(got, a64, b64, want64):
+    """max |got - want| relative to max_ij sum_k |a_ik||b_jk| (the scale rounding errors are measured in)"""
+    scale = (a64.abs() @ b64.abs().t()).max().item()
+    return (got.double() - want64).abs().max().item() / scale
+
+
+@pytest.mark.parametrize("M,K,N", [(1100, 77, 1030), (1024, 256, 1280), (1300, 16, 1025), (2048, 1000, 1100)])
+def test_split_contraction_is_binary32_grade(ops, M, K, N):
+    # Large enough for the path that splits the operands ahead of the matrix work (at least eight 128-wide
+    # tiles a side), ragged in every dimension.  float64 is the judge: the error must stay within what a
+    # binary32 dot product of this length may commit, (K + 2) * 2^-24 * sum |a||b|, and in practice sits
+    # near 2^-22 of the largest such sum; a bf16-only product (no split) would be off by 2^-9.
+    g = torch.Generator(device="cuda").manual_seed(M + K + N)
+    a = torch.randn(M, K, device="cuda", generator=g)
+    b = torch.randn(N, K, device="cuda", generator=g) * 3.0
+    bias = torch.randn(N, device="cuda", generator=g)
+    a64, b64 = a.double(), b.double()
+    bound = (K + 2) * 2.0 ** -24
+    got = ops.mul_mat(a, b, bias)
+    assert _f64_error(got, a64, b64, a64 @ b64.t() + bias.double()) <= min(bound, 2e-6)
+    # rows of both operands contiguous in k-major memory (the dense outer-product-mean form)
+    got = ops.mul_mat_tn(a.t().contiguous(), b.t().contiguous(), 0.5)
+    assert _f64_error(got, a64, b64, 0.5 * (a64 @ b64.t())) <= min(bound, 2e-6)
+    # values across the binary32 range: the split keeps every exponent (bf16 has binary32's range)
+    scale_a = torch.exp2(torch.randint(-40, 40, (M, 1), device="cuda", generator=g).float())
+    scale_b = torch.exp2(torch.randint(-40, 40, (N, 1), device="cuda", generator=g).float())
+    got = ops.mul_mat(a * scale_a, b * scale_b)
+    want = (a64 @ b64.t()) * scale_a.double() * scale_b.double().t()
+    rel = ((got.double() - want).abs() / ((a64.abs() @ b64.abs().t()) * scale_a.double() * scale_b.double().t())).max().item()
+    assert rel <= min(bound, 2e-6)
+
+
+def test_split_contraction_matches_small_path(ops):
+    # The path with operands split ahead and the one that splits inside the work-groups multiply the same
+    # bf16 parts in the same order: a large problem's top-left corner equals the small problem bit for bit.
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = torch.randn(1200, 100, device="cuda", generator=g)
+    b = torch.randn(1100, 100, device="cuda", generator=g)
+    big = ops.mul_mat(a, b)
+    small = ops.mul_mat(a[:300].contiguous(), b[:200].contiguous())
+    assert torch.equal(big[:300, :200], small)
+
+
+def test_outer_product_mean_graph_form_large(ops, oracle):
+    # D * L = 1280 rows a side: the graph form through the split-ahead path, compound output index
+    D, L, N, B = 32, 40, 24, 1
+    rng = np.random.default_rng(11)
+    left = (rng.standard_normal(D * L * N * B) * 0.1).astype(np.float32)
+    right = (rng.standard_normal(D * L * N * B) * 0.1).astype(np.float32)
+    got = ops.outer_product_mean(_dev(left), _dev(right), D, L, N, B).cpu().numpy()
+    want = oracle.outer_prod_mean(left, right, D, L, N, B)
+    _check(got, want)
 
 
 # ----------------------------------------------------------------------------- triangle multiplication
