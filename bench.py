@@ -24,6 +24,7 @@ METRIC = "Q8_0 mul_mat TOPS + GB/s (% of int8 MFMA / HBM roofline), 1 MI355X"
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA, published
 FP32_MFMA_PEAK_TFLOPS = 157.3
+BF16_MFMA_PEAK_TFLOPS = 2500.0
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE
 # scaled by the same counters on a 1 GiB copy: factors 2.000 and 1.000).
@@ -162,12 +163,17 @@ def main() -> int:
             extra[name] = {"us": round(e_ * 1e6, 2), "TOPS": round(no / e_ / 1e12, 2), "GBps": round(nb / e_ / 1e9, 1),
                            "hbm_frac": round(nb / e_ / 1e9 / HBM_PEAK_GBS, 4)}
 
-        def f32_case(make, nbytes, flops, name):
+        def f32_case(make, nbytes, flops, name, pipe="fp32"):
+            # pipe: "fp32" = fp32 MFMA; "bf16x3" = binary32 operands split three ways, six bf16 MFMA
+            # products per binary32 product (TFLOPS counts binary32 products, the fraction bf16 ones)
             fn_, ns = make()
             w_, e_ = time_op(fn_, ns, steps, warm)
             extra[name] = {"us": round(e_ * 1e6, 2), "TFLOPS": round(flops / e_ / 1e12, 2),
-                           "GBps": round(nbytes / e_ / 1e9, 1), "hbm_frac": round(nbytes / e_ / 1e9 / HBM_PEAK_GBS, 4),
-                           "fp32_mfma_frac": round(flops / e_ / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4)}
+                           "GBps": round(nbytes / e_ / 1e9, 1), "hbm_frac": round(nbytes / e_ / 1e9 / HBM_PEAK_GBS, 4)}
+            if pipe == "bf16x3":
+                extra[name]["bf16_mfma_frac"] = round(6.0 * flops / e_ / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4)
+            else:
+                extra[name]["fp32_mfma_frac"] = round(flops / e_ / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4)
 
         def logits(planes, L, D):
             def make():
@@ -178,9 +184,9 @@ def main() -> int:
                 return (lambda i: ops.attention_logits(ks[i], qs[i])), ns
             return make
         f32_case(logits(412, 103, 32), (2 * 412 * 32 * 103 + 412 * 103 * 103) * 4, 2.0 * 412 * 103 * 103 * 32,
-                 "attn_logits_pair_412x103x103x32")
+                 "attn_logits_pair_412x103x103x32", pipe="bf16x3")
         f32_case(logits(824, 256, 32), (2 * 824 * 32 * 256 + 824 * 256 * 256) * 4, 2.0 * 824 * 256 * 256 * 32,
-                 "attn_logits_msa_824x256x256x32")
+                 "attn_logits_msa_824x256x256x32", pipe="bf16x3")
 
         def attention(planes, L, D, with_bias, layout=0):
             def make():
@@ -282,7 +288,13 @@ def main() -> int:
             b = torch.randn(256, 12288, device=dev, generator=gen) * 0.1
             return (lambda i: ops.mul_mat_tn(a, b, 1.0 / 256)), 1
         steps, warm = 50, 10
-        f32_case(opm, (2 * 256 * 12288 + 12288 * 12288) * 4, 2.0 * 12288 * 12288 * 256, "opm_dense_12288x256x12288")
+        f32_case(opm, (2 * 256 * 12288 + 12288 * 12288) * 4, 2.0 * 12288 * 12288 * 256, "opm_dense_12288x256x12288", pipe="bf16x3")
+
+        def dense():
+            a = torch.randn(4096, 4096, device=dev, generator=gen)
+            b = torch.randn(4096, 4096, device=dev, generator=gen)
+            return (lambda i: ops.mul_mat(a, b)), 1
+        f32_case(dense, 3 * 4096 * 4096 * 4, 2.0 * 4096 ** 3, "mul_mat_f32_4096x4096x4096", pipe="bf16x3")
         out["extra"] = extra
 
     if args.copy_calibration:

@@ -51,7 +51,12 @@ const char *ppml_hip_last_error(void);
 
 /* ---- f32 GEMM ------------------------------------------------------------------------------ */
 /* replaces mul_mat_cuda (src/cuda/CUDAKernels.cu:1174-1182):
- * C[m*N+n] = (bias ? bias[n] : 0) + sum_k A[m*K+k] * B[n*K+k].  bias may be NULL. */
+ * C[m*N+n] = (bias ? bias[n] : 0) + sum_k A[m*K+k] * B[n*K+k].  bias may be NULL.
+ * Arithmetic of this and the other f32 contractions below: each binary32 operand is the exact sum of
+ * three bf16 numbers; six of the nine partial products (all but 2^-23 of |a||b|) are formed exactly on
+ * the bf16 matrix pipe and summed in binary32.  An infinite operand yields NaN.  Contractions of at
+ * least 512 work-groups of 256 x 128 outputs take a workspace of 6 bytes per operand element from a
+ * stream-ordered pool (allocated and freed on `stream`); no other launcher allocates. */
 int mul_mat_hip(const float *A, const float *B, float *C, int M, int K, int N,
                 const float *bias, ppml_hip_stream_t stream);
 

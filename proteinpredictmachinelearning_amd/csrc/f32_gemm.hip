@@ -489,9 +489,11 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const GemmParams p) {
 // Large contractions split their operands once, ahead of the matrix work, instead of in every
 // work-group that reads them (a 128-row panel of A is read by every tile column): the planes go to a
 // workspace in the order the contraction consumes them,
-//     [plane s][chunk of 16 k][row, padded to whole tiles][16 bf16]   (32 bytes per row and chunk)
-// so a work-group's share of one chunk is 4 KB of contiguous memory per plane, and its main loop is
-// loads, LDS traffic and MFMAs only.
+//     [plane s][chunk of 16 k][tile of 32 rows][k half][row][8 bf16]   (1 KB per MFMA operand fragment)
+// i.e. a fragment is stored lane by lane as the MFMA wants it (lane = 32 * (k half) + row, 16 bytes each).
+// A work-group's share of one chunk is contiguous per plane, goes to LDS as it lies, and comes out of LDS
+// with every lane reading its own 16 bytes of a 1 KB block: no bank conflicts either way, and a main loop
+// of loads, LDS traffic and MFMAs only.
 struct SplitJob {
     const float* src;
     uint8_t* dst;
@@ -539,7 +541,7 @@ __global__ __launch_bounds__(256) void split_operand_kernel(const SplitJob jb) {
     split4(v[1], hi);
 #pragma unroll
     for (int s = 0; s < 3; ++s) {
-        uint8_t* dst = jb.dst + ((static_cast<int64_t>(s) * jb.chunks + c) * jb.rows_pad + row) * 32 + kq * 16;
+        uint8_t* dst = jb.dst + ((static_cast<int64_t>(s) * jb.chunks + c) * jb.rows_pad + (row & ~31)) * 32 + kq * 512 + (row & 31) * 16;
         *reinterpret_cast<uint4*>(dst) = uint4{lo[s].x, lo[s].y, hi[s].x, hi[s].y};
     }
 }
@@ -547,17 +549,18 @@ __global__ __launch_bounds__(256) void split_operand_kernel(const SplitJob jb) {
 // Work-group tile 256 x 128, four waves of 128 x 64 each (eight accumulator tiles): a fragment read from
 // LDS feeds twice as many MFMAs as in the 64 x 64 arrangement, and it is LDS bandwidth that bounds this loop.
 constexpr int PBM = 256;
-constexpr int PLANES_MIN_TILES = 8;              // 128-wide tiles per side from which the operands are split ahead
+constexpr int PLANES_MIN_TILES = 8;              // 128-wide tiles per side from which the operands are split ahead ...
+constexpr int PLANES_MIN_GROUPS = 512;           // ... if that leaves two 256 x 128 work-groups for every CU
 template <bool SPLIT_C, bool STREAM_C>
 __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p, const uint8_t* __restrict__ wa,
                                                              const uint8_t* __restrict__ wb, int chunks, int ma_pad, int nb_pad) {
-    constexpr int A_PLANE = PBM * SPLIT_PITCH;
+    constexpr int A_PLANE = PBM * 32, B_PLANE = BN * 32;      // fragments of 1 KB, no padding
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * A_PLANE];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_b[3 * SPLIT_PLANE];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[3 * B_PLANE];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int j = lane & 31, hh = lane >> 5;
+    const int j = lane & 31;
     const int wm = (wave >> 1) * 128, wn = (wave & 1) * 64;
 
     int plane, m0, n0;
@@ -588,16 +591,16 @@ __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p,
         }
     };
     load_both(0);
-    const int put = (tid >> 1) * SPLIT_PITCH + (tid & 1) * 16;
-    const uint8_t* frag_a = lds_a + (wm + j) * SPLIT_PITCH + hh * 16;
-    const uint8_t* frag_b = lds_b + (wn + j) * SPLIT_PITCH + hh * 16;
+    const int put = tid * 16;
+    const uint8_t* frag_a = lds_a + wm * 32 + lane * 16;
+    const uint8_t* frag_b = lds_b + wn * 32 + lane * 16;
 
     for (int c = 0; c < chunks; ++c) {
 #pragma unroll
         for (int s = 0; s < 3; ++s) {
             *reinterpret_cast<v4i*>(lds_a + s * A_PLANE + put) = ra[s][0];
-            *reinterpret_cast<v4i*>(lds_a + s * A_PLANE + 128 * SPLIT_PITCH + put) = ra[s][1];
-            *reinterpret_cast<v4i*>(lds_b + s * SPLIT_PLANE + put) = rb[s];
+            *reinterpret_cast<v4i*>(lds_a + s * A_PLANE + 128 * 32 + put) = ra[s][1];
+            *reinterpret_cast<v4i*>(lds_b + s * B_PLANE + put) = rb[s];
         }
         __syncthreads();
         if (c + 1 < chunks) load_both(c + 1);
@@ -605,13 +608,13 @@ __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p,
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int s = 0; s < 3; ++s) fb[t][s] = *reinterpret_cast<const v8bf*>(frag_b + s * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
+            for (int s = 0; s < 3; ++s) fb[t][s] = *reinterpret_cast<const v8bf*>(frag_b + s * B_PLANE + t * 1024);
         constexpr int TERMS[6][2] = {{1, 1}, {2, 0}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};
 #pragma unroll
         for (int ti = 0; ti < 4; ++ti) {
             v8bf fa[3];
 #pragma unroll
-            for (int s = 0; s < 3; ++s) fa[s] = *reinterpret_cast<const v8bf*>(frag_a + s * A_PLANE + ti * 32 * SPLIT_PITCH);
+            for (int s = 0; s < 3; ++s) fa[s] = *reinterpret_cast<const v8bf*>(frag_a + s * A_PLANE + ti * 1024);
 #pragma unroll
             for (int q = 0; q < 6; ++q)
 #pragma unroll
@@ -680,7 +683,8 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
     // Large single-plane contractions split their operands ahead of the matrix work (every element would
     // otherwise be split by each work-group that reads it); when no workspace is to be had they take the
     // same path as the small ones.
-    if (!p.clamp && !p.f16_in && p.np2 * p.np3 == 1 && p.tiles_m >= PLANES_MIN_TILES && p.tiles_n >= PLANES_MIN_TILES) {
+    if (!p.clamp && !p.f16_in && p.np2 * p.np3 == 1 && p.tiles_m >= PLANES_MIN_TILES && p.tiles_n >= PLANES_MIN_TILES &&
+        static_cast<int64_t>((p.M + PBM - 1) / PBM) * p.tiles_n >= PLANES_MIN_GROUPS) {
         const int chunks = (p.K + BK - 1) / BK;
         const int tiles_m = (p.M + PBM - 1) / PBM;
         const int ma_pad = tiles_m * PBM, nb_pad = p.tiles_n * BN;

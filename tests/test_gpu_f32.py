@@ -231,10 +231,11 @@ def _f64_error(got, a64, b64, want64):
     return (got.double() - want64).abs().max().item() / scale
 
 
-@pytest.mark.parametrize("M,K,N", [(1100, 77, 1030), (1024, 256, 1280), (1300, 16, 1025), (2048, 1000, 1100)])
+@pytest.mark.parametrize("M,K,N", [(4100, 77, 3900), (8192, 16, 2048), (1100, 77, 1030), (2048, 1000, 1100)])
 def test_split_contraction_is_binary32_grade(ops, M, K, N):
-    # Large enough for the path that splits the operands ahead of the matrix work (at least eight 128-wide
-    # tiles a side), ragged in every dimension.  float64 is the judge: the error must stay within what a
+    # The first two shapes are large enough for the path that splits the operands ahead of the matrix work
+    # (at least 512 work-groups of 256 x 128), the others split inside the work-groups; ragged in every
+    # dimension.  float64 is the judge: the error must stay within what a
     # binary32 dot product of this length may commit, (K + 2) * 2^-24 * sum |a||b|, and in practice sits
     # near 2^-22 of the largest such sum; a bf16-only product (no split) would be off by 2^-9.
     g = torch.Generator(device="cuda").manual_seed(M + K + N)
@@ -261,16 +262,16 @@ def test_split_contraction_matches_small_path(ops):
     # The path with operands split ahead and the one that splits inside the work-groups multiply the same
     # bf16 parts in the same order: a large problem's top-left corner equals the small problem bit for bit.
     g = torch.Generator(device="cuda").manual_seed(5)
-    a = torch.randn(1200, 100, device="cuda", generator=g)
-    b = torch.randn(1100, 100, device="cuda", generator=g)
+    a = torch.randn(5000, 100, device="cuda", generator=g)
+    b = torch.randn(3400, 100, device="cuda", generator=g)
     big = ops.mul_mat(a, b)
     small = ops.mul_mat(a[:300].contiguous(), b[:200].contiguous())
     assert torch.equal(big[:300, :200], small)
 
 
 def test_outer_product_mean_graph_form_large(ops, oracle):
-    # D * L = 1280 rows a side: the graph form through the split-ahead path, compound output index
-    D, L, N, B = 32, 40, 24, 1
+    # D * L = 5888 rows a side: the graph form through the split-ahead path, compound output index
+    D, L, N, B = 32, 184, 8, 1
     rng = np.random.default_rng(11)
     left = (rng.standard_normal(D * L * N * B) * 0.1).astype(np.float32)
     right = (rng.standard_normal(D * L * N * B) * 0.1).astype(np.float32)
