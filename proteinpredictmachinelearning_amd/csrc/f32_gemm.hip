@@ -516,10 +516,18 @@ __global__ __launch_bounds__(256) void split_operand_kernel(const SplitJob jb) {
     if (row < jb.rows) {
         if (COMPOUND) {
             const int64_t roff = static_cast<int64_t>(row / jb.lm) * jb.mo + static_cast<int64_t>(row % jb.lm) * jb.mi;
+            const int kd = kb / jb.lk, kr = kb - kd * jb.lk;
+            if (kr + 7 < jb.lk && kb + 7 < jb.K) {
+                // the eight k share their outer index: one division for all of them
+                const float* src = jb.src + roff + static_cast<int64_t>(kd) * jb.ko + static_cast<int64_t>(kr) * jb.ki;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int k = kb + i;
-                if (k < jb.K) v[i >> 2][i & 3] = jb.src[roff + static_cast<int64_t>(k / jb.lk) * jb.ko + static_cast<int64_t>(k % jb.lk) * jb.ki];
+                for (int i = 0; i < 8; ++i) v[i >> 2][i & 3] = src[static_cast<int64_t>(i) * jb.ki];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int k = kb + i;
+                    if (k < jb.K) v[i >> 2][i & 3] = jb.src[roff + static_cast<int64_t>(k / jb.lk) * jb.ko + static_cast<int64_t>(k % jb.lk) * jb.ki];
+                }
             }
         } else if (KS1) {
             const float* src = jb.src + static_cast<int64_t>(row) * jb.rs + kb;
@@ -551,9 +559,11 @@ __global__ __launch_bounds__(256) void split_operand_kernel(const SplitJob jb) {
 constexpr int PBM = 256;
 constexpr int PLANES_MIN_TILES = 8;              // 128-wide tiles per side from which the operands are split ahead ...
 constexpr int PLANES_MIN_GROUPS = 512;           // ... if that leaves two 256 x 128 work-groups for every CU
+constexpr int PLANES_MIN_SLICE_CHUNKS = 16;      // a K slice is at least 256 long
 template <bool SPLIT_C, bool STREAM_C>
 __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p, const uint8_t* __restrict__ wa,
-                                                             const uint8_t* __restrict__ wb, int chunks, int ma_pad, int nb_pad) {
+                                                             const uint8_t* __restrict__ wb, int chunks, int ma_pad, int nb_pad,
+                                                             int slice_chunks, float* __restrict__ partial) {
     constexpr int A_PLANE = PBM * 32, B_PLANE = BN * 32;      // fragments of 1 KB, no padding
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * A_PLANE];
     __shared__ __attribute__((aligned(16))) uint8_t lds_b[3 * B_PLANE];
@@ -563,14 +573,19 @@ __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p,
     const int j = lane & 31;
     const int wm = (wave >> 1) * 128, wn = (wave & 1) * 64;
 
-    int plane, m0, n0;
-    tile_of_group<PBM>(p, plane, m0, n0);             // single plane: the launcher takes this path for np2 = np3 = 1 only
+    // One plane only (the launcher's rule); the plane index of the tile numbering is the K slice: with
+    // `partial` set, slice s contracts chunks [s * slice_chunks, (s + 1) * slice_chunks) and leaves its raw
+    // sums in partial[s][m][n] for reduce_slices_kernel, so that skinny problems still fill the chip.
+    int slice, m0, n0;
+    tile_of_group<PBM>(p, slice, m0, n0);
+    const int c_begin = slice * slice_chunks;
+    const int c_end = c_begin + slice_chunks < chunks ? c_begin + slice_chunks : chunks;
 
     v16f acc[4][2];
 #pragma unroll
     for (int tj = 0; tj < 2; ++tj) {
         const int n = n0 + wn + tj * 32 + j;
-        const float b0 = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+        const float b0 = (!partial && p.bias && n < p.N) ? p.bias[n] : 0.0f;
 #pragma unroll
         for (int ti = 0; ti < 4; ++ti)
 #pragma unroll
@@ -590,12 +605,12 @@ __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p,
             rb[s] = *reinterpret_cast<const v4i*>(gb + s * b_plane + c * b_chunk);
         }
     };
-    load_both(0);
+    load_both(c_begin);
     const int put = tid * 16;
     const uint8_t* frag_a = lds_a + wm * 32 + lane * 16;
     const uint8_t* frag_b = lds_b + wn * 32 + lane * 16;
 
-    for (int c = 0; c < chunks; ++c) {
+    for (int c = c_begin; c < c_end; ++c) {
 #pragma unroll
         for (int s = 0; s < 3; ++s) {
             *reinterpret_cast<v4i*>(lds_a + s * A_PLANE + put) = ra[s][0];
@@ -603,7 +618,7 @@ __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p,
             *reinterpret_cast<v4i*>(lds_b + s * B_PLANE + put) = rb[s];
         }
         __syncthreads();
-        if (c + 1 < chunks) load_both(c + 1);
+        if (c + 1 < c_end) load_both(c + 1);
         v8bf fb[2][3];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -624,7 +639,49 @@ __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p,
         __syncthreads();
     }
 
+    if (partial) {
+        // raw sums, rows and columns padded to whole tiles: no bounds to check, 128 contiguous bytes per half-wave
+        float* dst = partial + (static_cast<size_t>(slice) * ma_pad + m0 + wm) * nb_pad + n0 + wn + j;
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    __builtin_nontemporal_store(acc[ti][tj][r], dst + static_cast<size_t>(ti * 32 + mfma32_row(r, lane)) * nb_pad + tj * 32);
+        return;
+    }
     store_acc<SPLIT_C, STREAM_C, false, false, 4>(p, p.C, acc, m0 + wm, n0 + wn, lane);
+}
+
+// C = alpha * (bias + sum over the K slices, in slice order) with the contraction's own output addressing
+template <bool SPLIT_C>
+__global__ __launch_bounds__(256) void reduce_slices_kernel(const GemmParams p, const float* __restrict__ partial,
+                                                            int slices, int ma_pad, int nb_pad) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int nq = (p.N + 3) / 4;
+    const int m = static_cast<int>(idx / nq);
+    const int n4 = static_cast<int>(idx - static_cast<int64_t>(m) * nq) * 4;
+    if (m >= p.M) return;
+    v4f sum = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) if (n4 + c < p.N) sum[c] = p.bias[n4 + c];
+    }
+    const float* src = partial + static_cast<size_t>(m) * nb_pad + n4;          // nb_pad is a multiple of 128
+    for (int s = 0; s < slices; ++s) sum += *reinterpret_cast<const v4f*>(src + static_cast<size_t>(s) * ma_pad * nb_pad);
+    int64_t roff;
+    if (SPLIT_C) roff = static_cast<int64_t>(m / p.c_lm) * p.c_mo + static_cast<int64_t>(m % p.c_lm) * p.c_mi;
+    else         roff = static_cast<int64_t>(m) * p.c_mi;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int n = n4 + c;
+        if (n >= p.N) break;
+        int64_t coff;
+        if (SPLIT_C) coff = static_cast<int64_t>(n / p.c_ln) * p.c_no + static_cast<int64_t>(n % p.c_ln) * p.c_ni;
+        else         coff = static_cast<int64_t>(n) * p.c_ni;
+        p.C[roff + coff] = sum[c] * p.alpha;
+    }
 }
 
 // Stream-ordered workspace for the planes: a pool of this library's own per device, which keeps what it
@@ -681,33 +738,57 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
     if (p.a_ks == 1 && p.b_ks == 1) mode = LOAD_K_CONTIG;
     else if (p.a_rs == 1 && p.b_rs == 1) mode = LOAD_ROW_CONTIG;
     // Large single-plane contractions split their operands ahead of the matrix work (every element would
-    // otherwise be split by each work-group that reads it); when no workspace is to be had they take the
-    // same path as the small ones.
-    if (!p.clamp && !p.f16_in && p.np2 * p.np3 == 1 && p.tiles_m >= PLANES_MIN_TILES && p.tiles_n >= PLANES_MIN_TILES &&
-        static_cast<int64_t>((p.M + PBM - 1) / PBM) * p.tiles_n >= PLANES_MIN_GROUPS) {
-        const int chunks = (p.K + BK - 1) / BK;
+    // otherwise be split by each work-group that reads it).  Problems with few output tiles and a long K are
+    // cut into K slices until two work-groups per CU have work; their partial sums are added in slice order
+    // by a second kernel, so the result does not depend on scheduling.  When no workspace is to be had, the
+    // call takes the same path as the small ones.
+    const int64_t planes_groups = static_cast<int64_t>((p.M + PBM - 1) / PBM) * p.tiles_n;
+    const int chunks = (p.K + BK - 1) / BK;
+    int slices = 1;
+    if (planes_groups < PLANES_MIN_GROUPS) {
+        const int64_t want = (PLANES_MIN_GROUPS + planes_groups - 1) / planes_groups;
+        const int64_t most = chunks / PLANES_MIN_SLICE_CHUNKS;
+        slices = static_cast<int>(want < most ? want : most);
+        if (slices < 1) slices = 1;
+    }
+    const bool planes_fit = slices > 1 ? planes_groups * slices >= PLANES_MIN_GROUPS / 2 && static_cast<int64_t>(p.M) * p.N >= (1 << 20)
+                                       : p.tiles_m >= PLANES_MIN_TILES && p.tiles_n >= PLANES_MIN_TILES && planes_groups >= PLANES_MIN_GROUPS;
+    if (!p.clamp && !p.f16_in && p.np2 * p.np3 == 1 && planes_fit) {
         const int tiles_m = (p.M + PBM - 1) / PBM;
         const int ma_pad = tiles_m * PBM, nb_pad = p.tiles_n * BN;
+        const int slice_chunks = (chunks + slices - 1) / slices;
+        slices = (chunks + slice_chunks - 1) / slice_chunks;
         const size_t a_bytes = static_cast<size_t>(3) * chunks * ma_pad * 32, b_bytes = static_cast<size_t>(3) * chunks * nb_pad * 32;
+        const size_t part_bytes = slices > 1 ? static_cast<size_t>(slices) * ma_pad * nb_pad * 4 : 0;
         uint8_t* ws = nullptr;
         hipMemPool_t pool = workspace_pool();
-        if (pool && hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), a_bytes + b_bytes, pool, stream) != hipSuccess) {
+        if (pool && hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), a_bytes + b_bytes + part_bytes, pool, stream) != hipSuccess) {
             (void)hipGetLastError();
             ws = nullptr;
         }
         if (ws) {
             GemmParams q = p;
             q.tiles_m = tiles_m;
-            const dim3 pgrid(static_cast<unsigned>(q.tiles_m * q.tiles_n));
+            q.np2 = slices;                              // the tile numbering walks the slices as planes
+            float* partial = slices > 1 ? reinterpret_cast<float*>(ws + a_bytes + b_bytes) : nullptr;
+            const dim3 pgrid(static_cast<unsigned>(q.tiles_m * q.tiles_n * slices));
             const SplitJob ja{p.A, ws, p.M, ma_pad, p.K, chunks, p.a_rs, p.a_ks, p.a_lm, p.a_lk, p.a_mo, p.a_mi, p.a_ko, p.a_ki};
             const SplitJob jb{p.B, ws + a_bytes, p.N, nb_pad, p.K, chunks, p.b_rs, p.b_ks, 0, 0, 0, 0, 0, 0};
             int rc = launch_split(ja, stream);
             if (rc == RC_OK) rc = launch_split(jb, stream);
             if (rc == RC_OK) {
-                if (split) { if (p.stream_c) hipLaunchKernelGGL((gemm_planes_kernel<true, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad);
-                             else hipLaunchKernelGGL((gemm_planes_kernel<true, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad); }
-                else       { if (p.stream_c) hipLaunchKernelGGL((gemm_planes_kernel<false, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad);
-                             else hipLaunchKernelGGL((gemm_planes_kernel<false, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad); }
+                const bool stream_c = p.stream_c && !partial;
+                if (split && !partial) { if (stream_c) hipLaunchKernelGGL((gemm_planes_kernel<true, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial);
+                                         else hipLaunchKernelGGL((gemm_planes_kernel<true, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial); }
+                else                   { if (stream_c) hipLaunchKernelGGL((gemm_planes_kernel<false, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial);
+                                         else hipLaunchKernelGGL((gemm_planes_kernel<false, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial); }
+                rc = check_launch(what);
+            }
+            if (rc == RC_OK && partial) {
+                const int64_t threads = static_cast<int64_t>(p.M) * ((p.N + 3) / 4);
+                const dim3 rgrid(static_cast<unsigned>((threads + 255) / 256));
+                if (split) hipLaunchKernelGGL((reduce_slices_kernel<true>), rgrid, block, 0, stream, p, partial, slices, ma_pad, nb_pad);
+                else       hipLaunchKernelGGL((reduce_slices_kernel<false>), rgrid, block, 0, stream, p, partial, slices, ma_pad, nb_pad);
                 rc = check_launch(what);
             }
             if (hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();

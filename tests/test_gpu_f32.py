@@ -231,10 +231,11 @@ def _f64_error(got, a64, b64, want64):
     return (got.double() - want64).abs().max().item() / scale
 
 
-@pytest.mark.parametrize("M,K,N", [(4100, 77, 3900), (8192, 16, 2048), (1100, 77, 1030), (2048, 1000, 1100)])
+@pytest.mark.parametrize("M,K,N", [(4100, 77, 3900), (8192, 16, 2048), (1024, 4100, 1030), (1100, 77, 1030), (2048, 1000, 1100)])
 def test_split_contraction_is_binary32_grade(ops, M, K, N):
     # The first two shapes are large enough for the path that splits the operands ahead of the matrix work
-    # (at least 512 work-groups of 256 x 128), the others split inside the work-groups; ragged in every
+    # (at least 512 work-groups of 256 x 128), the third gets there in 15 slices of its long K (partial sums
+    # added in slice order by a second kernel), the others split inside the work-groups; ragged in every
     # dimension.  float64 is the judge: the error must stay within what a
     # binary32 dot product of this length may commit, (K + 2) * 2^-24 * sum |a||b|, and in practice sits
     # near 2^-22 of the largest such sum; a bf16-only product (no split) would be off by 2^-9.
@@ -340,7 +341,7 @@ def test_tri_mul_back(ops, oracle, D, I, J, K, Bt, outgoing):
     assert none is None and np.array_equal(gr.cpu().numpy(), wr)
 
 
-@pytest.mark.parametrize("D,L,N,Bt", [(3, 4, 8, 2), (16, 40, 64, 1), (4, 103, 37, 1)])
+@pytest.mark.parametrize("D,L,N,Bt", [(3, 4, 8, 2), (16, 40, 64, 1), (4, 103, 37, 1), (32, 64, 512, 1)])   # the last: K slices
 def test_outer_prod_mean_back(ops, oracle, D, L, N, Bt):
     rng = np.random.default_rng(D + L)
     left = rng.standard_normal(D * L * N * Bt).astype(np.float32)
