@@ -8,21 +8,23 @@
 //
 // One work-group per (plane, block of 32*NW queries); wave w owns 32 queries.  K and V of the plane
 // are staged in LDS (up to CH keys at a time, the whole plane for L <= CH) and shared by the waves.
-// All matrix work is fp32 MFMA (v_mfma_f32_32x32x2_f32), arranged so that nothing has to move
-// between lanes:
+// The matrix work is arranged so that nothing has to move between lanes:
 //
 //   scores, transposed:  S^T[key][query] = K_tile (32 keys x d) . Q^T (d x 32 queries)
+//       on the bf16 matrix pipe at binary32 accuracy: Q (times scale * log2 e) and K are split into three
+//       bf16 parts each (exactly), six partial products per 16 features (see common.hpp); K lies in LDS
+//       as ready MFMA fragments, Q in registers.  2.7 times less matrix-pipe time than the fp32 MFMA,
+//       which would moreover keep the vector pipe from running beside it;
 //       lane (query j = lane % 32, half = lane / 32) ends up with 16 of the 32 keys of ITS query in its
 //       accumulator registers -> the softmax row maximum and sum are 16 in-register steps plus one
 //       exchange with lane j + 32;
 //   output, transposed:  O^T[dd][query] += V^T (d x 32 keys) . P (32 keys x 32 queries)
+//       fp32 MFMA (v_mfma_f32_32x32x2_f32; splitting P would cost more vector work than it saves);
 //       the B operand of step kk is accumulator register kk of the scores -- the key order of the
 //       contraction is simply the order in which the score registers hold them (key(kk, half) =
 //       8*(kk/4) + 4*half + kk%4), and the V operand is read from LDS in that order;
 //       the running rescale factor alpha and the final 1/(l + eps) are per-lane scalars.
 //
-// The contraction over d likewise runs in the order that lets one 16-byte LDS read feed four MFMA
-// steps (slot `half` of step s takes element half*DP/2 + s).
 #include "common.hpp"
 
 #include <cmath>
@@ -37,9 +39,11 @@ template <int DP, int NW> struct AttnTiling {
     // keys staged in LDS at a time: about 35 KB per four-wave work-group (four of them share a CU and its
     // 160 KB), 69 KB per eight-wave one (two per CU)
     static constexpr int CH = (DP <= 32 ? 256 : 128) / (NW == 4 ? 2 : 1);
-    static constexpr int KS = DP + 4;                 // row pitch of K in LDS (floats): 16-byte reads, rows 4 banks apart
-    static constexpr int VS = DP;                     // row pitch of V
-    static constexpr size_t lds_bytes = static_cast<size_t>(CH) * (KS + VS) * sizeof(float);
+    static constexpr int NC = DP / 16;                // 16-feature chunks of the score contraction
+    // a 32-key tile of K in LDS: one 1 KB MFMA operand fragment per (chunk, bf16 part), [half][key][8 bf16]
+    static constexpr int KT_BYTES = NC * 3 * 1024;
+    static constexpr int VS = DP;                     // row pitch of V (floats)
+    static constexpr size_t lds_bytes = static_cast<size_t>(CH / 32) * KT_BYTES + static_cast<size_t>(CH) * VS * sizeof(float);
 };
 
 struct AttnParams {
@@ -63,13 +67,14 @@ __device__ __forceinline__ float lane_xor32(float x) {
 // the instance for short sequences uses it: there a work-group is a chain of memory latencies and the
 // machine is far from full anyway.
 template <int DP, int NW, bool PF>
-__global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnParams p) {
+// (the instance for long sequences is held to 128 registers: four waves per SIMD)
+__global__ __launch_bounds__(NW * 64, (DP <= 32 && !PF) ? 4 : 1) void flash_attn_forward_kernel(const AttnParams p) {
     using T = AttnTiling<DP, NW>;
-    constexpr int KS = T::KS, VS = T::VS;
+    constexpr int VS = T::VS, NC = T::NC, KT_BYTES = T::KT_BYTES;
     constexpr int NB = DP / 32;                       // 32-row blocks of the transposed output
     extern __shared__ __attribute__((aligned(16))) float attn_lds[];
-    float* lds_k = attn_lds;
-    float* lds_v = attn_lds + p.stage_rows * KS;
+    uint8_t* lds_k = reinterpret_cast<uint8_t*>(attn_lds);
+    float* lds_v = attn_lds + (p.stage_rows / 32) * (KT_BYTES / 4);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -83,23 +88,34 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
 
     constexpr float LOG2E = 1.44269504088896340736f, LN2 = 0.69314718055994530942f;
     const float sc2 = p.scale * LOG2E;                // scores are kept in the base-2 domain
-    // ---- this lane's slice of its query row, times scale * log2(e): elements half*DP/2 + s, s = 0 .. DP/2-1 (zero past d / past L)
-    float qreg[DP / 2];
-    if (p.in_ld) {
-        // [d][L]: one element per feature row, lanes along the queries (whole 128-byte runs)
+    // ---- this lane's slice of its query row, times scale * log2(e), as the B operand of the score MFMAs:
+    // chunk c holds features 16 c + 8 half .. + 7 (zero past d / past L), split into three bf16 parts
+    v8bf qb[NC][3];
 #pragma unroll
-        for (int s = 0; s < DP / 2; ++s) {
-            const int e = half * (DP / 2) + s;
-            qreg[s] = (q < L && e < d) ? p.Q[plane_off + static_cast<int64_t>(e) * L + q] * sc2 : 0.0f;
-        }
-    } else {
+    for (int c = 0; c < NC; ++c) {
+        const int e0 = 16 * c + 8 * half;
+        v4f x0 = {0.0f, 0.0f, 0.0f, 0.0f}, x1 = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (p.in_ld) {
+            // [d][L]: one element per feature row, lanes along the queries (whole 128-byte runs)
 #pragma unroll
-        for (int s = 0; s < DP / 2; s += 4) {
-            const int e = half * (DP / 2) + s;
-            v4f x = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (q < L && e < d) x = *reinterpret_cast<const v4f*>(p.Q + plane_off + static_cast<int64_t>(q) * d + e);
-            qreg[s] = x[0] * sc2; qreg[s + 1] = x[1] * sc2; qreg[s + 2] = x[2] * sc2; qreg[s + 3] = x[3] * sc2;
+            for (int i = 0; i < 4; ++i) {
+                if (q < L && e0 + i < d) x0[i] = p.Q[plane_off + static_cast<int64_t>(e0 + i) * L + q];
+                if (q < L && e0 + 4 + i < d) x1[i] = p.Q[plane_off + static_cast<int64_t>(e0 + 4 + i) * L + q];
+            }
+        } else {
+            const float* qrow = p.Q + plane_off + static_cast<int64_t>(q) * d;
+            if (q < L && e0 < d) x0 = *reinterpret_cast<const v4f*>(qrow + e0);
+            if (q < L && e0 + 4 < d) x1 = *reinterpret_cast<const v4f*>(qrow + e0 + 4);
         }
+        x0 *= sc2;
+        x1 *= sc2;
+        uint2 lo[3], hi[3];
+        split4(x0, lo);
+        split4(x1, hi);
+#pragma unroll
+        for (int part = 0; part < 3; ++part)
+            qb[c][part] = __builtin_bit_cast(v8bf, v4i{static_cast<int>(lo[part].x), static_cast<int>(lo[part].y),
+                                                      static_cast<int>(hi[part].x), static_cast<int>(hi[part].y)});
     }
 
     v16f acc_o[NB];
@@ -151,14 +167,15 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
         v16f st;
 #pragma unroll
         for (int r = 0; r < 16; ++r) st[r] = 0.0f;
-        const float* krow = lds_k + (kt * 32 + j) * KS + half * (DP / 2);
+        const uint8_t* kfrag = lds_k + kt * KT_BYTES + lane * 16;     // each lane its 16 bytes of a fragment
 #pragma unroll
-        for (int s = 0; s < DP / 2; s += 4) {
-            const v4f kx = *reinterpret_cast<const v4f*>(krow + s);
-            st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[0], qreg[s], st, 0, 0, 0);
-            st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[1], qreg[s + 1], st, 0, 0, 0);
-            st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[2], qreg[s + 2], st, 0, 0, 0);
-            st = __builtin_amdgcn_mfma_f32_32x32x2f32(kx[3], qreg[s + 3], st, 0, 0, 0);
+        for (int c = 0; c < NC; ++c) {
+            v8bf ka[3];
+#pragma unroll
+            for (int part = 0; part < 3; ++part) ka[part] = *reinterpret_cast<const v8bf*>(kfrag + (c * 3 + part) * 1024);
+#pragma unroll
+            for (int t = 0; t < 6; ++t)
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[SPLIT_TERMS[t][0]], qb[c][SPLIT_TERMS[t][1]], st, 0, 0, 0);
         }
         // ---- scores of this lane's query: bias, masks; tile maximum
         float m_tile = -INFINITY;
@@ -233,10 +250,19 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
                             if (kq + i < ckeys) { kx[i] = p.K[off + i]; vx[i] = p.V[off + i]; }
                     }
                 }
+                // four keys of feature dd: two bytes per key and part
+                uint2 parts[3];
+                split4(kx, parts);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    lds_k[(kq + i) * KS + dd] = kx[i];
-                    lds_v[(kq + i) * VS + dd] = vx[i];
+                    const int key = kq + i;
+                    uint8_t* dst = lds_k + (key >> 5) * KT_BYTES + (dd >> 4) * 3072 + ((dd >> 3) & 1) * 512 + (key & 31) * 16 + (dd & 7) * 2;
+#pragma unroll
+                    for (int part = 0; part < 3; ++part) {
+                        const uint32_t w = (i < 2 ? parts[part].x : parts[part].y) >> (16 * (i & 1));
+                        *reinterpret_cast<uint16_t*>(dst + part * 1024) = static_cast<uint16_t>(w);
+                    }
+                    lds_v[key * VS + dd] = vx[i];
                 }
             }
         } else {
@@ -248,7 +274,12 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_forward_kernel(const AttnP
                     kx = *reinterpret_cast<const v4f*>(p.K + off);
                     vx = *reinterpret_cast<const v4f*>(p.V + off);
                 }
-                *reinterpret_cast<v4f*>(lds_k + key * KS + c) = kx;
+                // features c .. c+3 of one key: eight bytes of each part's fragment
+                uint2 parts[3];
+                split4(kx, parts);
+                uint8_t* dst = lds_k + (key >> 5) * KT_BYTES + (c >> 4) * 3072 + ((c >> 3) & 1) * 512 + (key & 31) * 16 + ((c >> 2) & 1) * 8;
+#pragma unroll
+                for (int part = 0; part < 3; ++part) *reinterpret_cast<uint2*>(dst + part * 1024) = parts[part];
                 *reinterpret_cast<v4f*>(lds_v + key * VS + c) = vx;
             }
         }
@@ -305,7 +336,7 @@ int launch_flash(AttnParams p, hipStream_t stream) {
     auto kernel = &flash_attn_forward_kernel<DP, NW, PF>;
     const int l32 = (p.L + 31) / 32 * 32;
     p.stage_rows = l32 < T::CH ? l32 : T::CH;
-    const size_t lds = static_cast<size_t>(p.stage_rows) * (T::KS + T::VS) * sizeof(float);
+    const size_t lds = static_cast<size_t>(p.stage_rows / 32) * T::KT_BYTES + static_cast<size_t>(p.stage_rows) * T::VS * sizeof(float);
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(T::lds_bytes));
     if (attr != hipSuccess) {

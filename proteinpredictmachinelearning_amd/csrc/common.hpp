@@ -32,6 +32,32 @@ __device__ __forceinline__ int mfma32_row(int r, int lane) {
     return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
 }
 
+// ---- binary32 on the bf16 matrix pipe.  x = x1 + x2 + x3 exactly, each part a bf16 number (8 significant
+// bits taken off the top by truncation; the subtractions are exact), so a product of two binary32 numbers
+// is the exact sum of nine bf16 x bf16 products; v_mfma_f32_32x32x16_bf16 forms each exactly and adds it
+// into a binary32 accumulator.  Six are kept, in this order (smallest first); the other three are below
+// 2^-23 of |a||b| together.
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+constexpr int SPLIT_TERMS[6][2] = {{1, 1}, {2, 0}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};   // (part of a, part of b), zero-based
+
+// four consecutive elements -> four bf16 (8 bytes, element order) of each of the three parts
+__device__ __forceinline__ void split4(const v4f& v, uint2 (&out)[3]) {
+    uint32_t t1[4], t2[4], t3[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t b1 = __float_as_uint(v[c]) & 0xffff0000u;
+        const float r1 = v[c] - __uint_as_float(b1);              // exact: at most 16 significant bits left
+        const uint32_t b2 = __float_as_uint(r1) & 0xffff0000u;
+        const float r2 = r1 - __uint_as_float(b2);                // exact: at most 8 significant bits left
+        t1[c] = b1; t2[c] = b2; t3[c] = __float_as_uint(r2);
+    }
+    // the upper halves of two words side by side
+    const auto pack = [](uint32_t lo, uint32_t hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); };
+    out[0] = uint2{pack(t1[0], t1[1]), pack(t1[2], t1[3])};
+    out[1] = uint2{pack(t2[0], t2[1]), pack(t2[2], t2[3])};
+    out[2] = uint2{pack(t3[0], t3[1]), pack(t3[2], t3[3])};
+}
+
 // XCD-aware work-group numbering.  Consecutive work-group ids go round-robin over the 8 XCDs, each
 // with its own L2.  This maps id -> a logical index such that every XCD walks one contiguous
 // eighth of the logical range, so neighbouring tiles (which share operand panels) meet in one L2.

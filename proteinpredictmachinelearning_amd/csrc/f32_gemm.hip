@@ -274,25 +274,6 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
 // pipe gives +-inf or NaN; the clamped instances (whose result depends on that) stay on the fp32 pipe.
 constexpr int SPLIT_PITCH = 48;                   // bytes per tile row in a plane: 16 bf16, then 16 bytes of padding
 constexpr int SPLIT_PLANE = BM * SPLIT_PITCH;     // one of the three bf16 planes of a 128 x 16 operand tile
-typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
-
-// four consecutive k of one tile row -> four bf16 (8 bytes) in each of the three planes, returned packed
-__device__ __forceinline__ void split4(const v4f& v, uint2 (&out)[3]) {
-    uint32_t t1[4], t2[4], t3[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const uint32_t b1 = __float_as_uint(v[c]) & 0xffff0000u;
-        const float r1 = v[c] - __uint_as_float(b1);              // exact: at most 16 significant bits left
-        const uint32_t b2 = __float_as_uint(r1) & 0xffff0000u;
-        const float r2 = r1 - __uint_as_float(b2);                // exact: at most 8 significant bits left
-        t1[c] = b1; t2[c] = b2; t3[c] = __float_as_uint(r2);
-    }
-    // the upper halves of two words side by side
-    const auto pack = [](uint32_t lo, uint32_t hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); };
-    out[0] = uint2{pack(t1[0], t1[1]), pack(t1[2], t1[3])};
-    out[1] = uint2{pack(t2[0], t2[1]), pack(t2[2], t2[3])};
-    out[2] = uint2{pack(t3[0], t3[1]), pack(t3[2], t3[3])};
-}
 
 // A thread's share of a 128 x 16 operand tile goes to the planes.  Operands with contiguous rows are
 // read one row and eight consecutive k per thread (eight loads, each contiguous across the lanes), the
@@ -386,15 +367,13 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
                 fa[t][s] = *reinterpret_cast<const v8bf*>(frag_a + s * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
                 fb[t][s] = *reinterpret_cast<const v8bf*>(frag_b + s * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
             }
-        // smallest products first; the four accumulators take turns, so no MFMA waits for the one before it
-        constexpr int TERMS[6][2] = {{1, 1}, {2, 0}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};
 #pragma unroll
         for (int q = 0; q < 6; ++q)
 #pragma unroll
             for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
                 for (int tj = 0; tj < 2; ++tj)
-                    acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][TERMS[q][0]], fb[tj][TERMS[q][1]], acc[ti][tj], 0, 0, 0);
+                    acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][SPLIT_TERMS[q][0]], fb[tj][SPLIT_TERMS[q][1]], acc[ti][tj], 0, 0, 0);
         __syncthreads();
     }
 
@@ -624,7 +603,6 @@ __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p,
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int s = 0; s < 3; ++s) fb[t][s] = *reinterpret_cast<const v8bf*>(frag_b + s * B_PLANE + t * 1024);
-        constexpr int TERMS[6][2] = {{1, 1}, {2, 0}, {0, 2}, {1, 0}, {0, 1}, {0, 0}};
 #pragma unroll
         for (int ti = 0; ti < 4; ++ti) {
             v8bf fa[3];
@@ -634,7 +612,7 @@ __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p,
             for (int q = 0; q < 6; ++q)
 #pragma unroll
                 for (int tj = 0; tj < 2; ++tj)
-                    acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[TERMS[q][0]], fb[tj][TERMS[q][1]], acc[ti][tj], 0, 0, 0);
+                    acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SPLIT_TERMS[q][0]], fb[tj][SPLIT_TERMS[q][1]], acc[ti][tj], 0, 0, 0);
         }
         __syncthreads();
     }
