@@ -19,10 +19,10 @@
 //       accumulator registers -> the softmax row maximum and sum are 16 in-register steps plus one
 //       exchange with lane j + 32;
 //   output, transposed:  O^T[dd][query] += V^T (d x 32 keys) . P (32 keys x 32 queries)
-//       fp32 MFMA (v_mfma_f32_32x32x2_f32; splitting P would cost more vector work than it saves);
-//       the B operand of step kk is accumulator register kk of the scores -- the key order of the
-//       contraction is simply the order in which the score registers hold them (key(kk, half) =
-//       8*(kk/4) + 4*half + kk%4), and the V operand is read from LDS in that order;
+//       the same arithmetic: the probabilities are split in registers where they were computed, eight
+//       score registers making one B operand of 16 keys -- the key order of the contraction is simply
+//       the order in which the score registers hold them (key(kk, half) = 8*(kk/4) + 4*half + kk%4) --
+//       and V lies in LDS as fragments of V^T in that key order;
 //       the running rescale factor alpha and the final 1/(l + eps) are per-lane scalars.
 //
 #include "common.hpp"
@@ -36,14 +36,16 @@ namespace {
 typedef float v2f __attribute__((ext_vector_type(2)));
 
 template <int DP, int NW> struct AttnTiling {
-    // keys staged in LDS at a time: about 35 KB per four-wave work-group (four of them share a CU and its
-    // 160 KB), 69 KB per eight-wave one (two per CU)
-    static constexpr int CH = (DP <= 32 ? 256 : 128) / (NW == 4 ? 2 : 1);
+    // keys staged in LDS at a time: 36 KB per four-wave work-group (four of them share a CU and its
+    // 160 KB; 128 keys would leave room for three, measured 64.7 against 61.2 us at the MSA shape)
+    static constexpr int CH = DP <= 32 ? (NW == 4 ? 96 : 192) : (NW == 4 ? 64 : 128);
     static constexpr int NC = DP / 16;                // 16-feature chunks of the score contraction
     // a 32-key tile of K in LDS: one 1 KB MFMA operand fragment per (chunk, bf16 part), [half][key][8 bf16]
     static constexpr int KT_BYTES = NC * 3 * 1024;
-    static constexpr int VS = DP;                     // row pitch of V (floats)
-    static constexpr size_t lds_bytes = static_cast<size_t>(CH / 32) * KT_BYTES + static_cast<size_t>(CH) * VS * sizeof(float);
+    // a 32-key tile of V in LDS: fragments of V^T per (32 features, 16 keys, bf16 part); slot i of lane
+    // (feature, half) holds key 16 ch + 8 (i / 4) + 4 half + i % 4 of the tile
+    static constexpr int VT_BYTES = (DP / 32) * 2 * 3 * 1024;
+    static constexpr size_t lds_bytes = static_cast<size_t>(CH / 32) * (KT_BYTES + VT_BYTES);
 };
 
 struct AttnParams {
@@ -70,11 +72,11 @@ template <int DP, int NW, bool PF>
 // (the instance for long sequences is held to 128 registers: four waves per SIMD)
 __global__ __launch_bounds__(NW * 64, (DP <= 32 && !PF) ? 4 : 1) void flash_attn_forward_kernel(const AttnParams p) {
     using T = AttnTiling<DP, NW>;
-    constexpr int VS = T::VS, NC = T::NC, KT_BYTES = T::KT_BYTES;
+    constexpr int NC = T::NC, KT_BYTES = T::KT_BYTES, VT_BYTES = T::VT_BYTES;
     constexpr int NB = DP / 32;                       // 32-row blocks of the transposed output
     extern __shared__ __attribute__((aligned(16))) float attn_lds[];
     uint8_t* lds_k = reinterpret_cast<uint8_t*>(attn_lds);
-    float* lds_v = attn_lds + (p.stage_rows / 32) * (KT_BYTES / 4);
+    uint8_t* lds_v = lds_k + (p.stage_rows / 32) * KT_BYTES;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -208,17 +210,32 @@ __global__ __launch_bounds__(NW * 64, (DP <= 32 && !PF) ? 4 : 1) void flash_attn
         m_run = m_new;
         // ---- O^T = alpha * O^T + V^T . P   (the rescale is skipped while no maximum of the wave moves)
         const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0;
-        const float* vbase = lds_v + (kt * 32 + 4 * half) * VS + j;
+        if (rescale) {
 #pragma unroll
-        for (int b = 0; b < NB; ++b) {
-            if (rescale) {
+            for (int b = 0; b < NB; ++b)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc_o[b][r] *= alpha;
-            }
+        }
+        const uint8_t* vfrag = lds_v + kt * VT_BYTES + lane * 16;
 #pragma unroll
-            for (int kk = 0; kk < 16; ++kk) {
-                const float vx = vbase[(8 * (kk >> 2) + (kk & 3)) * VS + b * 32];
-                acc_o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vx, st[kk], acc_o[b], 0, 0, 0);
+        for (int ch = 0; ch < 2; ++ch) {
+            // the probabilities of 16 keys as three bf16 parts: score registers 8 ch .. 8 ch + 7 of this lane
+            uint2 lo[3], hi[3];
+            split4(v4f{st[8 * ch], st[8 * ch + 1], st[8 * ch + 2], st[8 * ch + 3]}, lo);
+            split4(v4f{st[8 * ch + 4], st[8 * ch + 5], st[8 * ch + 6], st[8 * ch + 7]}, hi);
+            v8bf pb[3];
+#pragma unroll
+            for (int part = 0; part < 3; ++part)
+                pb[part] = __builtin_bit_cast(v8bf, v4i{static_cast<int>(lo[part].x), static_cast<int>(lo[part].y),
+                                                        static_cast<int>(hi[part].x), static_cast<int>(hi[part].y)});
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                v8bf va[3];
+#pragma unroll
+                for (int part = 0; part < 3; ++part) va[part] = *reinterpret_cast<const v8bf*>(vfrag + ((b * 2 + ch) * 3 + part) * 1024);
+#pragma unroll
+                for (int t = 0; t < 6; ++t)
+                    acc_o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[SPLIT_TERMS[t][0]], pb[SPLIT_TERMS[t][1]], acc_o[b], 0, 0, 0);
             }
         }
     };
@@ -250,7 +267,8 @@ __global__ __launch_bounds__(NW * 64, (DP <= 32 && !PF) ? 4 : 1) void flash_attn
                             if (kq + i < ckeys) { kx[i] = p.K[off + i]; vx[i] = p.V[off + i]; }
                     }
                 }
-                // four keys of feature dd: two bytes per key and part
+                // four keys of feature dd.  K: two bytes per key and part; V: the four keys are neighbours in
+                // the lane slot of their feature (kq is a multiple of 4), eight bytes per part
                 uint2 parts[3];
                 split4(kx, parts);
 #pragma unroll
@@ -262,7 +280,14 @@ __global__ __launch_bounds__(NW * 64, (DP <= 32 && !PF) ? 4 : 1) void flash_attn
                         const uint32_t w = (i < 2 ? parts[part].x : parts[part].y) >> (16 * (i & 1));
                         *reinterpret_cast<uint16_t*>(dst + part * 1024) = static_cast<uint16_t>(w);
                     }
-                    lds_v[key * VS + dd] = vx[i];
+                }
+                split4(vx, parts);
+                {
+                    const int kc = kq & 15;            // place of the first key in its chunk of 16
+                    uint8_t* dst = lds_v + (kq >> 5) * VT_BYTES + (((dd >> 5) * 2 + ((kq >> 4) & 1)) * 3) * 1024 +
+                                   (((kc >> 2) & 1) * 32 + (dd & 31)) * 16 + (kc >> 3) * 8;
+#pragma unroll
+                    for (int part = 0; part < 3; ++part) *reinterpret_cast<uint2*>(dst + part * 1024) = parts[part];
                 }
             }
         } else {
@@ -280,7 +305,21 @@ __global__ __launch_bounds__(NW * 64, (DP <= 32 && !PF) ? 4 : 1) void flash_attn
                 uint8_t* dst = lds_k + (key >> 5) * KT_BYTES + (c >> 4) * 3072 + ((c >> 3) & 1) * 512 + (key & 31) * 16 + ((c >> 2) & 1) * 8;
 #pragma unroll
                 for (int part = 0; part < 3; ++part) *reinterpret_cast<uint2*>(dst + part * 1024) = parts[part];
-                *reinterpret_cast<v4f*>(lds_v + key * VS + c) = vx;
+                // V: features c .. c+3 of one key go to four lane slots of the fragments of V^T, two bytes each
+                split4(vx, parts);
+                {
+                    const int kc = key & 15;
+                    const int slot = 4 * (kc >> 3) + (kc & 3);
+                    uint8_t* vdst = lds_v + (key >> 5) * VT_BYTES + (((c >> 5) * 2 + ((key >> 4) & 1)) * 3) * 1024 +
+                                    (((kc >> 2) & 1) * 32 + (c & 31)) * 16 + slot * 2;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int part = 0; part < 3; ++part) {
+                            const uint32_t w = (i < 2 ? parts[part].x : parts[part].y) >> (16 * (i & 1));
+                            *reinterpret_cast<uint16_t*>(vdst + part * 1024 + i * 16) = static_cast<uint16_t>(w);
+                        }
+                }
             }
         }
         __syncthreads();
@@ -336,7 +375,7 @@ int launch_flash(AttnParams p, hipStream_t stream) {
     auto kernel = &flash_attn_forward_kernel<DP, NW, PF>;
     const int l32 = (p.L + 31) / 32 * 32;
     p.stage_rows = l32 < T::CH ? l32 : T::CH;
-    const size_t lds = static_cast<size_t>(p.stage_rows / 32) * T::KT_BYTES + static_cast<size_t>(p.stage_rows) * T::VS * sizeof(float);
+    const size_t lds = static_cast<size_t>(p.stage_rows / 32) * (T::KT_BYTES + T::VT_BYTES);
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(T::lds_bytes));
     if (attr != hipSuccess) {
