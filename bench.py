@@ -215,7 +215,7 @@ def main() -> int:
                                            (824, 256, 32, False, 0, "msa_824x256x32"),
                                            (824, 256, 32, True, 3, "msa_824x256x32_bias_graph_layout")]:
             f32_case(attention(planes, L, D, wb, lay), (4 * planes * L * D + planes * L + (planes * L * L if wb else 0)) * 4,
-                     4.0 * planes * L * L * D, "fused_attention_" + tag)
+                     4.0 * planes * L * L * D, "fused_attention_" + tag, pipe="bf16x3")
 
         def attention_back(planes, L, D):
             def make():
@@ -241,7 +241,7 @@ def main() -> int:
             return make
         # flops: five 2*L*L*D contractions per plane in exact terms (S, dP, dQ, dK, dV); S and dP are computed twice
         f32_case(attention_back(824, 256, 32), (8 * 824 * 256 * 32 + 824 * 256 + 2 * 824 * 256 * 256) * 4,
-                 10.0 * 824 * 256 * 256 * 32, "fused_attention_backward_msa_824x256x32_bias")
+                 10.0 * 824 * 256 * 256 * 32, "fused_attention_backward_msa_824x256x32_bias", pipe="bf16x3")
 
         def bridge():
             # the [L, D, h, B] -> [D, L, h, B] copy in front of the fused attention node, MSA-track size

@@ -2,8 +2,8 @@
 itself checked bit for bit against the reference's compiled src/ops/FlashAttn.cpp.
 
 Bar: 1e-4 relative on O (normwise per case, the f32 bar of this backend) and 1e-5 + 1e-5 * |LSE| on
-LSE.  The GPU sums in another order (fp32 MFMA, keys 32 at a time, hardware exp/log), so equality is
-not expected; special rows (fully masked, masked first block) must match exactly: O = 0, LSE = -inf.
+LSE.  The GPU sums in another order (exact bf16 split products on the matrix pipe, binary32 sums, keys 32 at a
+time, hardware exp/log), so equality is not expected; special rows (fully masked, masked first block) must match exactly: O = 0, LSE = -inf.
 """
 import json
 import os
