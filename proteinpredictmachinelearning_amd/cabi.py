@@ -82,6 +82,35 @@ class BackendError(RuntimeError):
         self.rc = rc
 
 
+class GgufTensor(C.Structure):
+    """``ppml_gguf_tensor`` of include/ppml_hip_weights.h."""
+    _fields_ = [("name", C.c_char_p), ("ndim", C.c_uint32), ("dims", C.c_uint64 * 4), ("type", C.c_uint32),
+                ("data", C.c_void_p)]
+
+
+_u32, _u64, _sz, _cp = C.c_uint32, C.c_uint64, C.c_size_t, C.c_char_p
+_strs = C.POINTER(C.c_char_p)
+
+# every symbol include/ppml_hip_weights.h declares (weight selection and the checkpoint file; host code only)
+WEIGHTS_SIGNATURES = {
+    "ppml_int8_bigop_default_list": (_cp, []),
+    "ppml_int8_bigop_selected": (_i, [_cp, _cp]),
+    "ppml_int8_bigop_shape_ok": (_i, [_u32, C.POINTER(_u64)]),
+    "ppml_gguf_layout_hash": (_u64, [_sz, _strs, C.POINTER(_u32), C.POINTER(_u64)]),
+    "ppml_gguf_save": (_i, [_cp, C.POINTER(GgufTensor), _sz, _sz, _strs, C.POINTER(_f), _sz, _strs, _strs, _sz]),
+    "ppml_gguf_open": (_vp, [_cp]),
+    "ppml_gguf_close": (None, [_vp]),
+    "ppml_gguf_tensor_count": (_sz, [_vp]),
+    "ppml_gguf_tensor_info": (_i, [_vp, _sz, C.POINTER(_cp), C.POINTER(_u32), C.POINTER(_u64), C.POINTER(_u32),
+                                   C.POINTER(_u64), C.POINTER(_u64)]),
+    "ppml_gguf_find_tensor": (_i64, [_vp, _cp]),
+    "ppml_gguf_read_tensor": (_i, [_vp, _sz, _vp, _sz]),
+    "ppml_gguf_meta_float": (_i, [_vp, _cp, C.POINTER(_f)]),
+    "ppml_gguf_meta_string": (_cp, [_vp, _cp]),
+    "ppml_gguf_check_layout": (_i, [_vp, _sz, _strs, C.POINTER(_u32), C.POINTER(_u64)]),
+}
+
+
 def load() -> C.CDLL:
     global _lib
     if _lib is not None:
@@ -91,7 +120,7 @@ def load() -> C.CDLL:
             f"{LIB_PATH} is missing: build it with `make -C proteinpredictmachinelearning_amd/csrc` "
             "(or __graft_entry__.build()); this backend has no CPU fallback")
     lib = C.CDLL(LIB_PATH)
-    for name, (res, args) in list(SIGNATURES.items()) + list(BACKEND_SIGNATURES.items()):
+    for name, (res, args) in list(SIGNATURES.items()) + list(BACKEND_SIGNATURES.items()) + list(WEIGHTS_SIGNATURES.items()):
         fn = getattr(lib, name)          # AttributeError if the library lacks a declared symbol
         fn.restype = res
         fn.argtypes = args

@@ -36,6 +36,19 @@ def test_backend_header_symbols_are_exported_and_bound():
     assert set(names) == set(cabi.BACKEND_SIGNATURES), set(names) ^ set(cabi.BACKEND_SIGNATURES)
 
 
+def test_weights_header_symbols_are_exported_and_bound():
+    from proteinpredictmachinelearning_amd import cabi
+
+    text = open(os.path.join(ROOT, "include", "ppml_hip_weights.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = sorted(set(re.findall(r"\b(ppml_(?:gguf|int8)_\w+)\s*\(", text)))
+    assert len(names) == 14, names
+    lib = cabi.load()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/ppml_hip_weights.h but not exported"
+    assert set(names) == set(cabi.WEIGHTS_SIGNATURES), set(names) ^ set(cabi.WEIGHTS_SIGNATURES)
+
+
 def test_host_side_argument_checks_need_no_gpu():
     from proteinpredictmachinelearning_amd import cabi
 
