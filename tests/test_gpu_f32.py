@@ -270,6 +270,29 @@ def test_split_contraction_matches_small_path(ops):
     assert torch.equal(big[:300, :200], small)
 
 
+def test_split_ahead_workspace_on_two_streams(ops):
+    # The split-ahead path takes its workspace from a stream-ordered pool: calls on different streams may run at
+    # the same time and must not share planes.  Interleaved launches on two streams equal the results of the same
+    # calls made one after the other.
+    g = torch.Generator(device="cuda").manual_seed(9)
+    a1 = torch.randn(4100, 64, device="cuda", generator=g)
+    b1 = torch.randn(3900, 64, device="cuda", generator=g)
+    a2 = torch.randn(4100, 96, device="cuda", generator=g)
+    b2 = torch.randn(3900, 96, device="cuda", generator=g)
+    want1, want2 = ops.mul_mat(a1, b1), ops.mul_mat(a2, b2)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = []
+    for _ in range(4):
+        with torch.cuda.stream(s1):
+            outs.append((1, ops.mul_mat(a1, b1)))
+        with torch.cuda.stream(s2):
+            outs.append((2, ops.mul_mat(a2, b2)))
+    torch.cuda.synchronize()
+    for which, o in outs:
+        assert torch.equal(o, want1 if which == 1 else want2)
+
+
 def test_outer_product_mean_graph_form_large(ops, oracle):
     # D * L = 5888 rows a side: the graph form through the split-ahead path, compound output index
     D, L, N, B = 32, 184, 8, 1
