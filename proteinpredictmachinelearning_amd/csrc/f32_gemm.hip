@@ -262,8 +262,8 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
 }
 
 // ------------------------------------------------------------------------------------------
-// The same contraction on the bf16 matrix pipe, sixteen times as fast as the fp32 one and able to run
-// beside vector instructions.  A binary32 number is the exact sum of three bf16 numbers
+// The same contraction on the bf16 matrix pipe, whose rate is sixteen times that of the fp32 one (which,
+// moreover, never runs beside vector instructions on this chip).  A binary32 number is the exact sum of three bf16 numbers
 // (x = x1 + x2 + x3: 8 + 8 + 8 significant bits, taken off the top by truncation), so a product is
 // the exact sum of nine bf16 x bf16 products, each of which the matrix pipe forms exactly and adds
 // into a binary32 accumulator.  Six of them are kept -- (1,1) (1,2) (2,1) (1,3) (3,1) (2,2) -- and the
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(256) void split_operand_kernel(const SplitJob jb) {
 }
 
 // Work-group tile 256 x 128, four waves of 128 x 64 each (eight accumulator tiles): a fragment read from
-// LDS feeds twice as many MFMAs as in the 64 x 64 arrangement, and it is LDS bandwidth that bounds this loop.
+// LDS feeds twice as many MFMAs as in the 64 x 64 arrangement, which had the LDS at three quarters of its bandwidth.
 constexpr int PBM = 256;
 constexpr int PLANES_MIN_TILES = 8;              // 128-wide tiles per side from which the operands are split ahead ...
 constexpr int PLANES_MIN_GROUPS = 512;           // ... if that leaves two 256 x 128 work-groups for every CU
