@@ -149,6 +149,7 @@ class GgufFile:
         self._h = self._lib.ppml_gguf_open(path.encode())
         if not self._h:
             raise RuntimeError(cabi.last_error())
+        self._size = os.path.getsize(path)
 
     def close(self) -> None:
         if self._h:
@@ -169,7 +170,7 @@ class GgufFile:
         dims, off, nb = (C.c_uint64 * 4)(), C.c_uint64(), C.c_uint64()
         if self._lib.ppml_gguf_tensor_info(self._h, i, C.byref(name), C.byref(ndim), dims, C.byref(typ), C.byref(off), C.byref(nb)):
             raise IndexError(cabi.last_error())
-        return {"name": name.value.decode(), "dims": tuple(dims[d] for d in range(ndim.value)), "type": typ.value,
+        return {"name": name.value.decode(errors="replace"), "dims": tuple(dims[d] for d in range(ndim.value)), "type": typ.value,
                 "offset": off.value, "nbytes": nb.value}
 
     def find(self, name: str) -> int:
@@ -178,12 +179,17 @@ class GgufFile:
     def read(self, i: int):
         """Tensor i: a float32 array of numpy shape ``reversed(dims)`` or a ``QuantizedWeight`` with host blocks."""
         inf = self.info(i)
+        if inf["nbytes"] == 0 or inf["offset"] > self._size or inf["nbytes"] > self._size - inf["offset"]:
+            raise RuntimeError(f"tensor {inf['name']!r} has an unknown type or lies outside the file")
         buf = np.empty(inf["nbytes"], dtype=np.uint8)
         if self._lib.ppml_gguf_read_tensor(self._h, i, buf.ctypes.data, buf.size):
             raise RuntimeError(cabi.last_error())
         if inf["type"] == TYPE_Q8_0:
             return QuantizedWeight(buf, inf["dims"])
-        return buf.view(np.float32).reshape(tuple(reversed(inf["dims"])))
+        try:
+            return buf.view(np.float32).reshape(tuple(reversed(inf["dims"])))
+        except ValueError as e:                      # dimensions whose product does not fit the stored size
+            raise RuntimeError(f"tensor {inf['name']!r}: {e}") from None
 
     def meta_float(self, key: str) -> Optional[float]:
         v = C.c_float()

@@ -201,6 +201,49 @@ def test_open_rejects_what_the_reference_rejects(W, tmp_path):
         W.GgufFile(str(p))
 
 
+def test_truncated_and_damaged_files_fail_cleanly(W, tmp_path):
+    # every prefix of a good file and a few hundred files with bytes overwritten either open and read, or raise:
+    # no tensor is ever read from outside the file
+    import random
+
+    rng = np.random.default_rng(1)
+    params = [rng.standard_normal((3, 5)).astype(np.float32), rng.standard_normal(7).astype(np.float32)]
+    good = str(tmp_path / "good.gguf")
+    W.save_gguf(params, good, [("epoch", 2.0)], [("arch", "v1")], ["a", "b"], [("opt.m.a", np.ones(4, np.float32))])
+    blob = open(good, "rb").read()
+    p = tmp_path / "damaged.gguf"
+
+    def exercise():
+        try:
+            with W.GgufFile(str(p)) as f:
+                for i in range(len(f)):
+                    try:
+                        f.info(i)
+                        f.read(i)
+                    except (RuntimeError, IndexError):
+                        pass
+                try:
+                    f.check_layout([[5, 3], [7]], ["a", "b"])
+                except RuntimeError:
+                    pass
+            return True
+        except RuntimeError:
+            return False
+
+    opened = 0
+    for n in range(0, len(blob), 3):
+        p.write_bytes(blob[:n])
+        opened += exercise()
+    assert 0 < opened < len(blob) // 3                    # short prefixes are rejected, long ones open
+    random.seed(1)
+    for _ in range(300):
+        b = bytearray(blob)
+        for _ in range(random.randint(1, 4)):
+            b[random.randrange(len(b))] = random.randrange(256)
+        p.write_bytes(bytes(b))
+        exercise()
+
+
 def test_metadata_of_every_type_is_read_or_skipped_like_the_reference(W, tmp_path):
     # src/model/GGUF.cpp:347-390: numbers of all widths become floats, small integers and arrays are skipped
     def kv(key, vtype, payload):
