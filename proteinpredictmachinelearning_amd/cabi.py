@@ -129,7 +129,7 @@ def load() -> C.CDLL:
 
 
 def last_error() -> str:
-    return load().ppml_hip_last_error().decode()
+    return load().ppml_hip_last_error().decode(errors="replace")
 
 
 def check(name: str, rc: int) -> None:
