@@ -295,6 +295,18 @@ def main() -> int:
             b = torch.randn(4096, 4096, device=dev, generator=gen)
             return (lambda i: ops.mul_mat(a, b)), 1
         f32_case(dense, 3 * 4096 * 4096 * 4, 2.0 * 4096 ** 3, "mul_mat_f32_4096x4096x4096", pipe="bf16x3")
+
+        def opm_back():
+            # both gradients of the graph-form outer-product-mean at D = 32, L = 384, N = 256: two contractions
+            # 12288 x 12288 -> 256 over a compound index of the 604 MB gradient tensor, cut into K slices
+            Dc, Lc, Nc = 32, 384, 256
+            left = torch.randn(Dc * Lc * Nc, device=dev, generator=gen) * 0.1
+            right = torch.randn(Dc * Lc * Nc, device=dev, generator=gen) * 0.1
+            grad = torch.randn(Dc * Dc * Lc * Lc, device=dev, generator=gen) * 0.1
+            return (lambda i: ops.outer_prod_mean_back(grad, left, right, Dc, Lc, Nc, 1)), 1
+        steps, warm = 20, 5
+        f32_case(opm_back, (2 * 12288 * 12288 + 4 * 12288 * 256) * 4, 4.0 * 12288 * 12288 * 256,
+                 "opm_backward_D32_L384_N256", pipe="bf16x3")
         out["extra"] = extra
 
     if args.copy_calibration:
