@@ -296,6 +296,16 @@ def main() -> int:
             return (lambda i: ops.mul_mat(a, b)), 1
         f32_case(dense, 3 * 4096 * 4096 * 4, 2.0 * 4096 ** 3, "mul_mat_f32_4096x4096x4096", pipe="bf16x3")
 
+        # the same two contractions on the fp32 matrix pipe (the library's other arithmetic for binary32 operands)
+        ops.set_f32_arithmetic("fp32")
+        try:
+            steps, warm = 20, 5
+            f32_case(opm, (2 * 256 * 12288 + 12288 * 12288) * 4, 2.0 * 12288 * 12288 * 256,
+                     "opm_dense_12288x256x12288_fp32_pipe", pipe="fp32")
+            f32_case(dense, 3 * 4096 * 4096 * 4, 2.0 * 4096 ** 3, "mul_mat_f32_4096x4096x4096_fp32_pipe", pipe="fp32")
+        finally:
+            ops.set_f32_arithmetic("split")
+
         def opm_back():
             # both gradients of the graph-form outer-product-mean at D = 32, L = 384, N = 256: two contractions
             # 12288 x 12288 -> 256 over a compound index of the 604 MB gradient tensor, cut into K slices

@@ -50,6 +50,13 @@ int ppml_hip_synchronize(void);
 const char *ppml_hip_last_error(void);
 
 /* ---- f32 GEMM ------------------------------------------------------------------------------ */
+/* Which matrix pipe multiplies binary32 operands in the f32 contractions below: 0 (default) = the bf16 pipe
+ * through an exact three-way split of every operand (binary32-grade results, about 1.5 times the speed),
+ * 1 = the fp32 pipe (v_mfma_f32_32x32x2_f32, k ascending two at a time).  The environment variable
+ * PPML_HIP_F32_ARITH=fp32 selects 1 before the first call.  Returns the previous setting; other values of
+ * `mode` only query.  No counterpart in the reference (its tf32 switch PPML_MUL_MAT_TC trades accuracy,
+ * this one does not). */
+int ppml_hip_set_f32_arithmetic(int mode);
 /* replaces mul_mat_cuda (src/cuda/CUDAKernels.cu:1174-1182):
  * C[m*N+n] = (bias ? bias[n] : 0) + sum_k A[m*K+k] * B[n*K+k].  bias may be NULL.
  * Arithmetic of this and the other f32 contractions below: each binary32 operand is the exact sum of

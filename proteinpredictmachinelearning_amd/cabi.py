@@ -19,6 +19,7 @@ SIGNATURES = {
     "ppml_hip_init": (_i, [_i]),
     "ppml_hip_synchronize": (_i, []),
     "ppml_hip_last_error": (C.c_char_p, []),
+    "ppml_hip_set_f32_arithmetic": (_i, [_i]),
     "mul_mat_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "mul_mat_f16_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp]),
     "quantize_rows_q8_0_hip": (_i, [_vp, _vp, _i64, _vp]),

@@ -16,6 +16,9 @@
 // v_mfma_f32_32x32x2_f32, k ascending two at a time).
 #include "common.hpp"
 
+#include <atomic>
+#include <cstdlib>
+#include <cstring>
 #include <mutex>
 
 namespace ppmlhip {
@@ -701,6 +704,21 @@ int launch_split(const SplitJob& jb, hipStream_t stream) {
     return check_launch("split_operand_kernel");
 }
 
+// Which matrix pipe multiplies binary32 operands: 0 = the bf16 pipe through the exact three-way split (the
+// default), 1 = the fp32 pipe (v_mfma_f32_32x32x2_f32, k ascending two at a time).  Set through
+// ppml_hip_set_f32_arithmetic or, before the first contraction, by PPML_HIP_F32_ARITH=fp32 in the environment.
+std::atomic<int> g_f32_arithmetic{-1};
+
+int f32_arithmetic() {
+    int mode = g_f32_arithmetic.load(std::memory_order_relaxed);
+    if (mode < 0) {
+        const char* env = std::getenv("PPML_HIP_F32_ARITH");
+        mode = (env && std::strcmp(env, "fp32") == 0) ? 1 : 0;
+        g_f32_arithmetic.store(mode, std::memory_order_relaxed);
+    }
+    return mode;
+}
+
 int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
@@ -720,6 +738,7 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
     // cut into K slices until two work-groups per CU have work; their partial sums are added in slice order
     // by a second kernel, so the result does not depend on scheduling.  When no workspace is to be had, the
     // call takes the same path as the small ones.
+    const bool fp32_pipe = f32_arithmetic() == 1;
     const int64_t planes_groups = static_cast<int64_t>((p.M + PBM - 1) / PBM) * p.tiles_n;
     const int chunks = (p.K + BK - 1) / BK;
     int slices = 1;
@@ -731,7 +750,7 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
     }
     const bool planes_fit = slices > 1 ? planes_groups * slices >= PLANES_MIN_GROUPS / 2 && static_cast<int64_t>(p.M) * p.N >= (1 << 20)
                                        : p.tiles_m >= PLANES_MIN_TILES && p.tiles_n >= PLANES_MIN_TILES && planes_groups >= PLANES_MIN_GROUPS;
-    if (!p.clamp && !p.f16_in && p.np2 * p.np3 == 1 && planes_fit) {
+    if (!fp32_pipe && !p.clamp && !p.f16_in && p.np2 * p.np3 == 1 && planes_fit) {
         const int tiles_m = (p.M + PBM - 1) / PBM;
         const int ma_pad = tiles_m * PBM, nb_pad = p.tiles_n * BN;
         const int slice_chunks = (chunks + slices - 1) / slices;
@@ -778,9 +797,20 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
         if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_kernel<MODE, SPLIT, true>), grid, block, 0, stream, p);  \
         else hipLaunchKernelGGL((gemm_bf16x3_kernel<MODE, SPLIT, false>), grid, block, 0, stream, p); \
     } while (0)
+#define PPML_LAUNCH_F32(MODE, SPLIT)                                                                  \
+    do {                                                                                              \
+        if (p.stream_c) hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, true>), grid, block, 0, stream, p);  \
+        else hipLaunchKernelGGL((gemm_f32_kernel<MODE, SPLIT, false>), grid, block, 0, stream, p);    \
+    } while (0)
     if (p.a_lm > 0) {
         if (split || p.f16_in || p.clamp) { set_error("%s: no split-operand instance for this addressing", what); return RC_BAD_ARGS; }
-        PPML_LAUNCH_BF16(LOAD_SPLIT_A, false);
+        if (fp32_pipe) PPML_LAUNCH_F32(LOAD_SPLIT_A, false);
+        else PPML_LAUNCH_BF16(LOAD_SPLIT_A, false);
+    }
+    else if (!p.clamp && !p.f16_in && fp32_pipe) {
+        if (mode == LOAD_K_CONTIG)        { if (split) PPML_LAUNCH_F32(LOAD_K_CONTIG, true);   else PPML_LAUNCH_F32(LOAD_K_CONTIG, false); }
+        else if (mode == LOAD_ROW_CONTIG) { if (split) PPML_LAUNCH_F32(LOAD_ROW_CONTIG, true); else PPML_LAUNCH_F32(LOAD_ROW_CONTIG, false); }
+        else                              { if (split) PPML_LAUNCH_F32(LOAD_STRIDED, true);    else PPML_LAUNCH_F32(LOAD_STRIDED, false); }
     }
     else if (!p.clamp && !p.f16_in) {
         // binary32 operands without the finite guard: the contraction runs on the bf16 matrix pipe
@@ -800,6 +830,7 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
         else hipLaunchKernelGGL((gemm_f16_kernel<false>), grid, block, 0, stream, p);
     }
 #undef PPML_LAUNCH_BF16
+#undef PPML_LAUNCH_F32
     return check_launch(what);
 }
 
@@ -816,6 +847,12 @@ GemmParams plain_params() {
 }  // namespace ppmlhip
 
 using namespace ppmlhip;
+
+extern "C" int ppml_hip_set_f32_arithmetic(int mode) {
+    const int before = f32_arithmetic();
+    if (mode == 0 || mode == 1) g_f32_arithmetic.store(mode, std::memory_order_relaxed);
+    return before;
+}
 
 extern "C" int mul_mat_hip(const float* A, const float* B, float* C, int M, int K, int N,
                            const float* bias, ppml_hip_stream_t stream) {

@@ -52,6 +52,13 @@ def synchronize() -> None:
 
 
 # ----------------------------------------------------------------------------- f32
+def set_f32_arithmetic(mode: str) -> str:
+    """Matrix pipe of the f32 contractions: "split" (default: bf16 pipe, exact three-way split) or "fp32"
+    (fp32 MFMA).  Returns the previous setting."""
+    before = _lib().ppml_hip_set_f32_arithmetic({"split": 0, "fp32": 1}[mode])
+    return "fp32" if before == 1 else "split"
+
+
 def mul_mat(a: torch.Tensor, b: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
     """a [M,K], b [N,K] -> [M,N] = a @ b.T (+ bias[N]); src/core/ComputeGraphHelper.cpp:262-314."""
     a, b = _dev_f32(a, "a"), _dev_f32(b, "b")

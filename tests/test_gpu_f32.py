@@ -225,6 +225,34 @@ def test_dense_outer_product_mean_stress_shape_properties(ops):
     assert err <= RTOL * want.abs().max().item()
 
 
+@pytest.fixture
+def fp32_pipe(ops):
+    before = ops.set_f32_arithmetic("fp32")
+    yield
+    ops.set_f32_arithmetic(before)
+
+
+def test_fp32_pipe_arithmetic_is_selectable_and_within_the_same_bar(ops, oracle, fp32_pipe):
+    # the other arithmetic of the library for binary32 operands: fp32 MFMA, k ascending two at a time
+    rng = np.random.default_rng(17)
+    A = rng.standard_normal((300, 70)).astype(np.float32)
+    B = (rng.standard_normal((260, 70)) * 0.02).astype(np.float32)
+    bias = rng.standard_normal(260).astype(np.float32)
+    _check(ops.mul_mat(_dev(A), _dev(B), _dev(bias)).cpu().numpy(), oracle.mul_mat_f32(A, B, bias))
+    Ai = ((np.arange(17 * 9) % 11) * 0.5 - 2.0).astype(np.float32).reshape(17, 9)     # tests/test_cuda.cpp:133-167
+    Bi = ((np.arange(23 * 9) % 13) * 0.25 + 0.5).astype(np.float32).reshape(23, 9)
+    assert (ops.mul_mat(_dev(Ai), _dev(Bi)).cpu().numpy() == oracle.mul_mat_f32(Ai, Bi)).all()
+    g = torch.Generator(device="cuda").manual_seed(4)
+    a = torch.randn(4100, 77, device="cuda", generator=g)                              # large: no split-ahead path here
+    b = torch.randn(3900, 77, device="cuda", generator=g)
+    got = ops.mul_mat(a, b)
+    assert _f64_error(got, a.double(), b.double(), a.double() @ b.double().t()) <= 2e-6
+    assert ops.set_f32_arithmetic("fp32") == "fp32"
+    k = rng.standard_normal((1, 6, 32, 50)).astype(np.float32)
+    q = rng.standard_normal((1, 6, 32, 40)).astype(np.float32)
+    _check(ops.out_prod(_dev(k), _dev(q)).cpu().numpy(), oracle.out_prod(k, q))
+
+
 def _f64_error(got, a64, b64, want64):
     """max |got - want| relative to max_ij sum_k |a_ik||b_jk| (the scale rounding errors are measured in)"""
     scale = (a64.abs() @ b64.abs().t()).max().item()
