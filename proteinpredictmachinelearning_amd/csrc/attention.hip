@@ -167,8 +167,6 @@ __global__ __launch_bounds__(NW * 64, (DP <= 32 && !PF) ? 4 : 1) void flash_attn
         }
         // ---- S^T = K_tile . Q^T
         v16f st;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) st[r] = 0.0f;
         const uint8_t* kfrag = lds_k + kt * KT_BYTES + lane * 16;     // each lane its 16 bytes of a fragment
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
@@ -176,8 +174,11 @@ __global__ __launch_bounds__(NW * 64, (DP <= 32 && !PF) ? 4 : 1) void flash_attn
 #pragma unroll
             for (int part = 0; part < 3; ++part) ka[part] = *reinterpret_cast<const v8bf*>(kfrag + (c * 3 + part) * 1024);
 #pragma unroll
-            for (int t = 0; t < 6; ++t)
-                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[SPLIT_TERMS[t][0]], qb[c][SPLIT_TERMS[t][1]], st, 0, 0, 0);
+            for (int t = 0; t < 6; ++t) {
+                // the first product starts from the constant zero: no registers to clear
+                const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[SPLIT_TERMS[t][0]], qb[c][SPLIT_TERMS[t][1]], (c == 0 && t == 0) ? zero : st, 0, 0, 0);
+            }
         }
         // ---- scores of this lane's query: bias, masks; tile maximum
         float m_tile = -INFINITY;

@@ -148,15 +148,16 @@ template <int DP>
 __device__ __forceinline__ v16f tile_times_slice(const uint8_t* frags, const v8bf (&slice)[DP / 16][3]) {
     v16f acc;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-#pragma unroll
     for (int c = 0; c < DP / 16; ++c) {
         v8bf a[3];
 #pragma unroll
         for (int part = 0; part < 3; ++part) a[part] = *reinterpret_cast<const v8bf*>(frags + (c * 3 + part) * 1024);
 #pragma unroll
-        for (int t = 0; t < 6; ++t)
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[SPLIT_TERMS[t][0]], slice[c][SPLIT_TERMS[t][1]], acc, 0, 0, 0);
+        for (int t = 0; t < 6; ++t) {
+            // the first product starts from the constant zero: no registers to clear
+            const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[SPLIT_TERMS[t][0]], slice[c][SPLIT_TERMS[t][1]], (c == 0 && t == 0) ? zero : acc, 0, 0, 0);
+        }
     }
     return acc;
 }
