@@ -236,6 +236,24 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_back_rows_kernel(const Att
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc_q[b][r] = 0.0f;
 
+    // Bias of this lane's 16 keys of the tile that starts at key0 (zeros past L), 16 bytes at a time.
+    float bv[16];
+    const auto load_bias = [&](int key0) {
+        if (!bias_row) return;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int key = key0 + 8 * g + 4 * half;
+            if (key + 3 < L) {
+                const v4f x = *reinterpret_cast<const v4f_u*>(bias_row + key);
+                bv[4 * g] = x[0]; bv[4 * g + 1] = x[1]; bv[4 * g + 2] = x[2]; bv[4 * g + 3] = x[3];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) bv[4 * g + i] = key + i < L ? bias_row[key + i] : 0.0f;
+            }
+        }
+    };
+    if (wave_active) load_bias(0);
+
     const int stage = p.stage_rows;
     for (int c0 = 0; c0 < L; c0 += stage) {
         __syncthreads();
@@ -246,22 +264,8 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_back_rows_kernel(const Att
         if (!wave_active) continue;
         for (int kt = 0; kt < rows / 32; ++kt) {
             const int key0 = c0 + kt * 32;
-            // ---- probabilities of this lane's query for its 16 keys of the tile
-            // bias of this lane's 16 keys, requested before the matrix work (16 bytes at a time)
-            float bv[16];
-            if (bias_row) {
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int key = key0 + 8 * g + 4 * half;
-                    if (key + 3 < L) {
-                        const v4f x = *reinterpret_cast<const v4f_u*>(bias_row + key);
-                        bv[4 * g] = x[0]; bv[4 * g + 1] = x[1]; bv[4 * g + 2] = x[2]; bv[4 * g + 3] = x[3];
-                    } else {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) bv[4 * g + i] = key + i < L ? bias_row[key + i] : 0.0f;
-                    }
-                }
-            }
+            // ---- probabilities of this lane's query for its 16 keys of the tile (their bias was requested a
+            // tile ago, see below)
             v16f st = tile_times_slice<DP>(lds_k_row + kt * T::ROW_BYTES + lane * 16, qb);
             v16f dp = tile_times_slice<DP>(lds_v_row + kt * T::ROW_BYTES + lane * 16, dob);
 #pragma unroll
@@ -272,6 +276,9 @@ __global__ __launch_bounds__(NW * 64) void flash_attn_back_rows_kernel(const Att
                 const float pr = key < row_keys ? __builtin_amdgcn_exp2f(s2 - lse2) : 0.0f;
                 st[r] = pr * (dp[r] - D_i);            // dS
             }
+            // the bias registers are free again: the next tile's values travel during the rest of this tile
+            // and the first contractions of the next (the tiles follow each other across the stages)
+            if (key0 + 32 < L) load_bias(key0 + 32);
             // ---- dbias = dS (zeros where the key is masked; every position of a valid row is written)
             if (dbias_row && q < L) {
 #pragma unroll
