@@ -391,26 +391,33 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
 // sum, as the CPU branch of the reference does.
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
-__device__ __forceinline__ uint2 load_halves4(const uint16_t* __restrict__ base, int64_t rs, int row, int nrows, int k, int K) {
-    uint2 v{0u, 0u};
-    if (row < nrows) {
+// eight consecutive halves (16 bytes) of row `row`, zeros past the matrix
+__device__ __forceinline__ v4i load_halves8(const uint16_t* __restrict__ base, int64_t rs, int row, int nrows, int k, int K) {
+    v4i v = {0, 0, 0, 0};
+    if (row < nrows && k < K) {
         const uint16_t* p = base + static_cast<int64_t>(row) * rs + k;
-        if (k + 3 < K && (reinterpret_cast<uintptr_t>(p) & 7) == 0) {
-            v = *reinterpret_cast<const uint2*>(p);
+        if (k + 7 < K && (reinterpret_cast<uintptr_t>(p) & 15) == 0) {
+            v = *reinterpret_cast<const v4i*>(p);
         } else {
-            uint32_t h[4] = {0u, 0u, 0u, 0u};
+            uint32_t h[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
 #pragma unroll
-            for (int c = 0; c < 4; ++c) if (k + c < K) h[c] = p[c];
-            v = uint2{h[0] | (h[1] << 16), h[2] | (h[3] << 16)};
+            for (int c = 0; c < 8; ++c) if (k + c < K) h[c] = p[c];
+            v = v4i{static_cast<int>(h[0] | (h[1] << 16)), static_cast<int>(h[2] | (h[3] << 16)),
+                    static_cast<int>(h[4] | (h[5] << 16)), static_cast<int>(h[6] | (h[7] << 16))};
         }
     }
     return v;
 }
 
+// A stage is 64 k deep (four MFMA steps): with so little matrix work per element the loop is a chain of
+// memory round trips, and a deeper stage makes it four times shorter.
+constexpr int F16_BK = 64;
+constexpr int F16_PITCH = F16_BK * 2 + 16;            // bytes per tile row: 16-byte fragment reads without bank conflicts
+
 template <bool STREAM_C>
 __global__ __launch_bounds__(256) void gemm_f16_kernel(const GemmParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[SPLIT_PLANE];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_b[SPLIT_PLANE];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[BM * F16_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[BN * F16_PITCH];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -429,39 +436,43 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const GemmParams p) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
 
-    // a thread's share of a 128 x 16 tile: rows tid / 4 and tid / 4 + 64, four consecutive k each
-    uint2 ra[2], rb[2];
+    // a thread's share of a 128 x 64 tile: row tid / 2, 32 consecutive k (four loads of 16 bytes)
+    v4i ra[4], rb[4];
+    const int srow = tid >> 1, sk = (tid & 1) * 32;
     const auto load_both = [&](int k0) {
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            ra[it] = load_halves4(A, p.a_rs, m0 + (tid >> 2) + it * 64, p.M, k0 + (tid & 3) * 4, p.K);
-            rb[it] = load_halves4(B, p.b_rs, n0 + (tid >> 2) + it * 64, p.N, k0 + (tid & 3) * 4, p.K);
+        for (int i = 0; i < 4; ++i) {
+            ra[i] = load_halves8(A, p.a_rs, m0 + srow, p.M, k0 + sk + 8 * i, p.K);
+            rb[i] = load_halves8(B, p.b_rs, n0 + srow, p.N, k0 + sk + 8 * i, p.K);
         }
     };
     load_both(0);
-    const int put = (tid >> 2) * SPLIT_PITCH + (tid & 3) * 8;
-    const uint8_t* frag_a = lds_a + (wm + j) * SPLIT_PITCH + hh * 16;
-    const uint8_t* frag_b = lds_b + (wn + j) * SPLIT_PITCH + hh * 16;
+    const int put = srow * F16_PITCH + sk * 2;
+    const uint8_t* frag_a = lds_a + (wm + j) * F16_PITCH + hh * 16;
+    const uint8_t* frag_b = lds_b + (wn + j) * F16_PITCH + hh * 16;
 
-    for (int k0 = 0; k0 < p.K; k0 += BK) {
+    for (int k0 = 0; k0 < p.K; k0 += F16_BK) {
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            *reinterpret_cast<uint2*>(lds_a + put + it * 64 * SPLIT_PITCH) = ra[it];
-            *reinterpret_cast<uint2*>(lds_b + put + it * 64 * SPLIT_PITCH) = rb[it];
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<v4i*>(lds_a + put + 16 * i) = ra[i];
+            *reinterpret_cast<v4i*>(lds_b + put + 16 * i) = rb[i];
         }
         __syncthreads();
-        if (k0 + BK < p.K) load_both(k0 + BK);
-        v8h fa[2], fb[2];
+        if (k0 + F16_BK < p.K) load_both(k0 + F16_BK);
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            fa[t] = *reinterpret_cast<const v8h*>(frag_a + t * 32 * SPLIT_PITCH);
-            fb[t] = *reinterpret_cast<const v8h*>(frag_b + t * 32 * SPLIT_PITCH);
+        for (int s = 0; s < F16_BK / 16; ++s) {
+            v8h fa[2], fb[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                fa[t] = *reinterpret_cast<const v8h*>(frag_a + t * 32 * F16_PITCH + s * 32);
+                fb[t] = *reinterpret_cast<const v8h*>(frag_b + t * 32 * F16_PITCH + s * 32);
+            }
+#pragma unroll
+            for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < 2; ++tj)
+                    acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[ti], fb[tj], acc[ti][tj], 0, 0, 0);
         }
-#pragma unroll
-        for (int ti = 0; ti < 2; ++ti)
-#pragma unroll
-            for (int tj = 0; tj < 2; ++tj)
-                acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[ti], fb[tj], acc[ti][tj], 0, 0, 0);
         __syncthreads();
     }
     store_acc<false, STREAM_C, true, false>(p, p.C, acc, m0 + wm, n0 + wn, lane);
