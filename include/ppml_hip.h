@@ -54,7 +54,8 @@ const char *ppml_hip_last_error(void);
  * through an exact three-way split of every operand (binary32-grade results, about 1.5 times the speed),
  * 1 = the fp32 pipe (v_mfma_f32_32x32x2_f32, k ascending two at a time).  The environment variable
  * PPML_HIP_F32_ARITH=fp32 selects 1 before the first call.  Returns the previous setting; other values of
- * `mode` only query.  No counterpart in the reference (its tf32 switch PPML_MUL_MAT_TC trades accuracy,
+ * `mode` only query.  The setting belongs to the calling thread (threads that want different arithmetic do
+ * not disturb each other; a new thread starts from the environment's choice).  No counterpart in the reference (its tf32 switch PPML_MUL_MAT_TC trades accuracy,
  * this one does not). */
 int ppml_hip_set_f32_arithmetic(int mode);
 /* replaces mul_mat_cuda (src/cuda/CUDAKernels.cu:1174-1182):
@@ -110,8 +111,7 @@ int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K,
  *                src/modules/Attention.cpp:1097-1104)
  *   flags bit 1: quantize X with the Q8_1 rule of quantize_rows_q8_1_hip instead of the Q8_0 rule:
  *                the numbers mul_mat_q8_cuda itself produces (src/cuda/MulMatQ8Kernel.cu:520-527
- *                quantizes activations to Q8_1 and settles with their d).  Served by the general
- *                kernel, not by the weight-stationary one.
+ *                quantizes activations to Q8_1 and settles with their d).
  *   xq_dump  (may be NULL): receives the Q8_0 blocks the kernel made of X, [N][K/32] block_q8_0
  *   sums_dump(may be NULL): receives the per-block int32 sums, [(n*M+m)*(K/32)+ib]            */
 int mul_mat_q8_ex_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
@@ -227,11 +227,58 @@ int permute_hip(const float *src, float *dst, int64_t total, int ndim,
                 int64_t s0, int64_t s1, int64_t s2, int64_t s3,
                 int64_t dd0, int64_t dd1, int64_t dd2, int64_t dd3, ppml_hip_stream_t stream);
 
-/* ---- observability (include/ppml/MulMatStats.h:154-169) -------------------------------------- */
-/* Per-shape call counters keyed like the reference (M<<40 | K<<20 | N); enabled by the
- * environment variable PPML_MULMAT_STATS=1.  Writes up to `cap` rows of
- * {M, K, N, calls} (int64 each) and returns the number of distinct shapes. */
+/* ---- sum over the copies of a broadcast (the bias gradient of mul_mat) ------------------------- */
+/* replaces repeat_back4_cuda (declared src/backend/CUDAKernels.cpp:336-339, called from
+ * kernel_repeat_back_cross_cuda, 1290-1320); semantics of CPUBackend::kernel_repeat_back
+ * (src/backend/CPUKernels.cpp:2091-2148):
+ *   dst[j0,j1,j2,j3] = sum_{k0<r0, k1<r1, k2<r2, k3<r3} src[j0+k0*d0, j1+k1*d1, j2+k2*d2, j3+k3*d3]
+ * s0..s3 source sizes, d0..d3 destination sizes (dimension 0 innermost), r0..r3 copies per dimension as the
+ * caller derives them (integer quotient of the sizes, dimension d of dst against dimension d of src).  This
+ * is the node the backward of a biased mul_mat emits for the bias: grad [N, M] -> dbias [N]
+ * (src/core/ComputeGraph.cpp:742).  The reference adds the copies one at a time, k3 fastest; here that
+ * sequence is cut into consecutive runs summed side by side and added in run order (a fixed bracketing,
+ * no atomics).  With few destination elements and many copies the partial sums take a workspace from the
+ * library's stream-ordered pool.  returns 0 ok, 1 bad arguments (a copy outside the source), 6 launch error. */
+int repeat_back_hip(const float *src, float *dst,
+                    int64_t s0, int64_t s1, int64_t s2, int64_t s3,
+                    int64_t d0, int64_t d1, int64_t d2, int64_t d3,
+                    int64_t r0, int64_t r1, int64_t r2, int64_t r3, ppml_hip_stream_t stream);
+
+/* ---- observability (include/ppml/MulMatStats.h:39-169, src/cuda/CUDAKernels.cu:1693-1732) ------ */
+/* MUL_MAT statistics: per (path, M, K, N) the number of launcher calls and the device time of their
+ * launches, measured with a pair of events recorded on the launcher's stream (nothing waits; inside a
+ * stream capture only the call is counted).  Enabled by the environment variable PPML_MULMAT_STATS (set and
+ * not "0", the reference's rule) or by ppml_hip_mulmat_stats_enable(1); while enabled, the table is also
+ * printed to stderr when the process exits, as the reference does.  Shapes are kept whole (the reference's
+ * key holds 20 bits per dimension). */
+typedef struct ppml_hip_mulmat_stat {
+    char path[32];   /* "hip/<kernel family>", the reference's "<where>/<path>" bucket name */
+    int64_t M, K, N; /* output rows, contracted length, output columns, as the reference prints them */
+    int64_t calls;
+    double ms;       /* accumulated device time of the calls whose launches have finished */
+} ppml_hip_mulmat_stat;
+/* Switches the statistics on (1) or off (0); other values only query.  Returns the previous state. */
+int ppml_hip_mulmat_stats_enable(int on);
+/* Writes up to `cap` rows of {M, K, N, calls} (int64 each), summed over the paths, ordered by shape;
+ * returns the number of distinct shapes. */
 int ppml_hip_mulmat_stats(int64_t *rows, int cap);
+/* Waits for the recorded launches, then writes up to `cap` rows ordered by (path, M, K, N); returns the
+ * number of rows the table holds.  mulmat_stats_record's table (MulMatStats.h:154-169) read back. */
+int ppml_hip_mulmat_stats_rows(ppml_hip_mulmat_stat *rows, int cap);
+/* mulmat_stats_dump (MulMatStats.h:86-145): totals, per-path lines and the top 12 shapes, to stderr. */
+void ppml_hip_mulmat_stats_dump(void);
+/* Empties the table (recorded launches are waited for first). */
+void ppml_hip_mulmat_stats_reset(void);
+
+/* Which kernel family served the calling thread's last mul_mat_q8_hip / mul_mat_q8_ex_hip call: the
+ * counterpart of mul_mat_q8_cuda's *path_out (src/cuda/MulMatQ8Kernel.cu:476, 1 = MMQ, 0 = MMVQ), whose
+ * two values do not describe this library's kernels. */
+enum {
+    PPML_Q8_PATH_GENERAL = 0,           /* one token tile per work-group, any shape and weight layout */
+    PPML_Q8_PATH_WEIGHT_STATIONARY = 1, /* persistent work-groups, weight fragments resident in registers */
+    PPML_Q8_PATH_LOW_LATENCY = 2        /* few token tiles per CU: many small work-groups, weights through L2 */
+};
+int ppml_hip_q8_last_path(void);
 
 #ifdef __cplusplus
 }

@@ -58,6 +58,15 @@ void ppml_hip_backend_set_q8_1_activations(ppml_hip_backend *b, int on);
  * reader / they are its only reader; the attention kernel takes the other layout itself and the skipped
  * tensors are never written.  0 (default): every node is executed as it stands. */
 void ppml_hip_backend_set_fuse_attention_bridges(ppml_hip_backend *b, int on);
+/* Matrix pipe of this backend's f32 contractions for the length of each graph_compute: 0 = bf16 pipe through
+ * the exact three-way split, 1 = fp32 pipe, anything else = the calling thread's ppml_hip_set_f32_arithmetic
+ * choice (default).  A field of the backend object, so backends with different settings do not interfere. */
+void ppml_hip_backend_set_f32_arithmetic(ppml_hip_backend *b, int mode);
+/* graph_compute in single-backend mode (skip_alloc off) copies sources bound to HOST memory to the device for
+ * the duration of the call and puts the tensors' fields back afterwards (ensure_host_shadow /
+ * release_host_shadows, src/backend/CUDABackend.cpp:521-577, 824-830); ppml_hip_tensor_set_data accepts such a
+ * host pointer.  Returns how many sources the last graph_compute covered this way. */
+int ppml_hip_backend_host_shadows_made(const ppml_hip_backend *b);
 int ppml_hip_backend_graph_compute(ppml_hip_backend *b, ppml_hip_tensor **nodes, int n);
 int ppml_hip_backend_pack_weight(ppml_hip_backend *b, ppml_hip_tensor *weight);
 

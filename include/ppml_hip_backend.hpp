@@ -30,6 +30,7 @@ enum TensorType : int {
 
 enum TensorOp : int {
     OP_NONE = 0,
+    OP_REPEAT_BACK = 21,
     OP_MUL_MAT = 30,
     OP_OUT_PROD = 32,
     OP_SCALE = 33,
@@ -145,6 +146,16 @@ public:
     void set_fuse_attention_bridges(bool v) { fuse_attention_bridges_ = v; }
     bool fuse_attention_bridges() const { return fuse_attention_bridges_; }
 
+    // Matrix pipe of this backend's f32 contractions: 0 = bf16 pipe through the exact three-way split, 1 = fp32
+    // pipe, -1 (default) = whatever the calling thread has chosen with ppml_hip_set_f32_arithmetic.  Applied
+    // for the length of each graph_compute and put back afterwards, so two backends (or threads) with different
+    // settings do not disturb each other.
+    void set_f32_arithmetic(int mode) { f32_arithmetic_ = (mode == 0 || mode == 1) ? mode : -1; }
+    int f32_arithmetic() const { return f32_arithmetic_; }
+    // Host-resident sources the last graph_compute copied to the device for its duration
+    // (src/backend/CUDABackend.cpp:521-577; single-backend mode only, i.e. not under skip_alloc).
+    size_t host_shadows_made() const { return host_shadows_made_; }
+
     // Once-per-weight step of src/model/PPML.cpp:4504-4528: turns a Q8_0 / Q8_1 / Q8_0R weight node
     // into the MFMA-fragment layout in a buffer owned by this backend.
     Status pack_weight(Tensor* weight);
@@ -157,6 +168,7 @@ private:
     Status kernel_flash_attn_ext(Tensor* node);
     Status kernel_flash_attn_back(Tensor* node);
     Status kernel_permute(Tensor* node);
+    Status kernel_repeat_back(Tensor* node);
     Status kernel_tri_mul(Tensor* node);
     Status kernel_tri_mul_back(Tensor* node);
     Status kernel_outer_prod_mean_back(Tensor* node);
@@ -168,6 +180,8 @@ private:
     bool skip_alloc_ = false;
     bool q8_1_activations_ = false;
     bool fuse_attention_bridges_ = false;
+    int f32_arithmetic_ = -1;
+    size_t host_shadows_made_ = 0;
     int attn_layout_ = 0;                                // layout bits of the attention node being dispatched
     std::string error_;
     std::vector<std::unique_ptr<Buffer>> owned_;         // node outputs allocated here, packed weights

@@ -86,6 +86,8 @@ def _load() -> C.CDLL:
     lib.orc_permute.argtypes = [f32p, f32p, C.c_int, C.POINTER(C.c_int32), C.POINTER(i64), C.POINTER(i64)]
     lib.orc_flash_attn_backward.restype = C.c_int
     lib.orc_flash_attn_backward.argtypes = [C.c_int] * 5 + [C.c_float] + [f32p] * 11
+    lib.orc_repeat_back.restype = None
+    lib.orc_repeat_back.argtypes = [f32p, f32p, C.c_int, C.POINTER(i64), C.c_int, C.POINTER(i64)]
     lib.orc_max_threads.restype = C.c_int
     return lib
 
@@ -434,3 +436,15 @@ def ref_flash_attn_backward(q, k, v, bias, o, do, lse, causal=False, scale=0.0, 
     if ref is None:
         return None
     return _flash_backward(ref.ref_flash_attn_backward, q, k, v, bias, o, do, lse, causal, scale, want_dbias)
+
+
+def repeat_back(src, dst_shape) -> np.ndarray:
+    """kernel_repeat_back (CPUKernels.cpp:2091-2148).  `src` is a numpy array whose LAST axis is the reference's
+    dims[0]; `dst_shape` is the result's shape in the same (numpy) order."""
+    src = _f32(src)
+    dst_shape = tuple(int(d) for d in dst_shape)
+    sd = list(src.shape[::-1]) + [1] * (4 - src.ndim)
+    dd = list(dst_shape[::-1]) + [1] * (4 - len(dst_shape))
+    out = np.empty(dst_shape, dtype=np.float32)
+    lib().orc_repeat_back(_fp(src), _fp(out), src.ndim, (C.c_int64 * 4)(*sd), len(dst_shape), (C.c_int64 * 4)(*dd))
+    return out

@@ -35,6 +35,11 @@
  *       <grad, tri_mul(l, r)> = <gleft, l> = <gright, r> against orc_tri_mul, both forms.
  *   orc_permute : numpy.transpose with the axes translated (dst dim p = src dim axes[p], dims[0]
  *       innermost), identity and inverse permutations, hand-checked 2 x 3 case.
+ *   orc_repeat_back : numpy sums over the broadcast axes on small integers (exact in any order), the
+ *       bias-gradient case against a column sum, the mixed case where a dimension is both kept and
+ *       repeated, the summation order probed with 2^24 + 1 + 1 (sequential from the left gives 2^24,
+ *       any pairing of the two ones gives 2^24 + 2), and the dimension alignment of
+ *       src/backend/CPUKernels.cpp:2099-2109 (dimension d of dst meets dimension d of src).
  *   orc_flash_attn_forward : the reference's own src/ops/FlashAttn.cpp compiled as-is
  *       (oracle/_ref/libppml_ref_flash.so: it needs nothing but its header) -- bit-for-bit on
  *       random inputs, with and without bias, causal and not, ragged block sizes; plus float64
@@ -714,4 +719,37 @@ void orc_attention_scores(const float *Q, const float *K, float *scores,
                     for (int64_t d = 0; d < D; ++d) s += qp[d * Lq] * kp[d * Lk];
                     scores[((b * H + h) * Lq + i) * Lk + j] = s * inv_scale;
                 }
+}
+
+/* src/backend/CPUKernels.cpp:2091-2148 (kernel_repeat_back).  nd_src / nd_dst are the tensors' ranks, sd_in /
+ * dd_in their sizes (dims[0] innermost; entries past the rank ignored).  Dimension d of dst meets dimension
+ * d of src (2108); the number of copies per dimension is the integer quotient of the sizes (2117-2122); every
+ * destination element is the sum of its copies added one at a time, k0 outermost, k3 innermost (2139-2151). */
+void orc_repeat_back(const float *src, float *dst, int nd_src, const int64_t sd_in[4], int nd_dst, const int64_t dd_in[4]) {
+    const int off = (nd_src >= nd_dst) ? 0 : (nd_src - nd_dst);
+    int64_t dd[4] = {1, 1, 1, 1}, sd[4] = {1, 1, 1, 1}, rd[4] = {1, 1, 1, 1};
+    for (int d = 0; d < nd_dst && d < 4; ++d) dd[d] = dd_in[d];
+    for (int d = 0; d < nd_src && d < 4; ++d) sd[d] = sd_in[d];
+    for (int d = 0; d < 4; ++d) {
+        const int s_idx = d + off;
+        const int64_t sdim = (s_idx >= 0 && s_idx < 4) ? sd[s_idx] : 1;
+        rd[d] = dd[d] > 0 ? sdim / dd[d] : 1;
+    }
+    const int64_t total = dd[0] * dd[1] * dd[2] * dd[3];
+    for (int64_t idx = 0; idx < total; ++idx) {
+        int64_t t = idx;
+        const int64_t j0 = t % dd[0]; t /= dd[0];
+        const int64_t j1 = t % dd[1]; t /= dd[1];
+        const int64_t j2 = t % dd[2]; t /= dd[2];
+        const int64_t j3 = t;
+        float sum = 0.0f;
+        for (int64_t k0 = 0; k0 < rd[0]; ++k0)
+            for (int64_t k1 = 0; k1 < rd[1]; ++k1)
+                for (int64_t k2 = 0; k2 < rd[2]; ++k2)
+                    for (int64_t k3 = 0; k3 < rd[3]; ++k3) {
+                        const int64_t s0 = j0 + k0 * dd[0], s1 = j1 + k1 * dd[1], s2 = j2 + k2 * dd[2], s3 = j3 + k3 * dd[3];
+                        sum += src[((s3 * sd[2] + s2) * sd[1] + s1) * sd[0] + s0];
+                    }
+        dst[idx] = sum;
+    }
 }

@@ -120,6 +120,10 @@ int orc_flash_attn_backward(int B, int h, int L, int d, int causal, float scale,
                             const float *O, const float *dO, const float *LSE,
                             float *dQ, float *dK, float *dV, float *dbias);
 
+/* src/backend/CPUKernels.cpp:2091-2148 (kernel_repeat_back): dst = src summed over its copies; nd_* are the
+ * ranks, sd / dd the sizes (dims[0] innermost), dimension d of dst meets dimension d of src. */
+void orc_repeat_back(const float *src, float *dst, int nd_src, const int64_t sd[4], int nd_dst, const int64_t dd[4]);
+
 int orc_max_threads(void);
 
 #ifdef __cplusplus

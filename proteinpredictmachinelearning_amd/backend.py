@@ -17,6 +17,7 @@ from . import cabi
 # tensor_type
 F32, F16, Q8_0, Q8_1, Q8_0R, Q8_0M = 0, 1, 8, 9, 19, 64
 # tensor_op
+OP_REPEAT_BACK = 21
 OP_NONE, OP_MUL_MAT, OP_OUT_PROD, OP_SCALE, OP_RESHAPE, OP_VIEW, OP_PERMUTE, OP_TRANSPOSE, OP_SOFT_MAX = 0, 30, 32, 33, 37, 38, 39, 40, 47
 OP_FLASH_ATTN_EXT, OP_FLASH_ATTN_BACK, OP_TRI_MUL, OP_TRI_MUL_BACK, OP_OUTER_PROD_MEAN, OP_OUTER_PROD_MEAN_BACK = \
     75, 76, 100, 101, 102, 103
@@ -102,6 +103,15 @@ class Backend:
 
     def set_fuse_attention_bridges(self, on: bool) -> None:
         self._lib.ppml_hip_backend_set_fuse_attention_bridges(self.handle, int(on))
+
+    def set_f32_arithmetic(self, mode) -> None:
+        """"split", "fp32", or None for the calling thread's own choice (ppml_hip_backend_set_f32_arithmetic)."""
+        self._lib.ppml_hip_backend_set_f32_arithmetic(self.handle, {"split": 0, "fp32": 1, None: -1}[mode])
+
+    @property
+    def host_shadows_made(self) -> int:
+        """Host-resident sources the last graph_compute copied to the device for its duration."""
+        return self._lib.ppml_hip_backend_host_shadows_made(self.handle)
 
     def upload(self, t: Tensor, host: np.ndarray) -> Tensor:
         host = np.ascontiguousarray(host)

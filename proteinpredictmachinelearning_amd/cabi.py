@@ -42,8 +42,21 @@ SIGNATURES = {
     "flash_attn_backward_hip": (_i, [_i] * 5 + [_f] + [_vp] * 12),
     "flash_attn_forward_ex_hip": (_i, [_i] * 5 + [_f, _f, _i] + [_vp] * 6 + [_i, _vp]),
     "permute_hip": (_i, [_vp, _vp, _i64, _i] + [_i] * 4 + [_i64] * 8 + [_vp]),
+    "repeat_back_hip": (_i, [_vp, _vp] + [_i64] * 12 + [_vp]),
     "ppml_hip_mulmat_stats": (_i, [C.POINTER(_i64), _i]),
+    "ppml_hip_mulmat_stats_enable": (_i, [_i]),
+    "ppml_hip_mulmat_stats_rows": (_i, [_vp, _i]),
+    "ppml_hip_mulmat_stats_dump": (None, []),
+    "ppml_hip_mulmat_stats_reset": (None, []),
+    "ppml_hip_q8_last_path": (_i, []),
 }
+
+
+class MulMatStat(C.Structure):
+    """``ppml_hip_mulmat_stat`` of include/ppml_hip.h."""
+    _fields_ = [("path", C.c_char * 32), ("M", C.c_int64), ("K", C.c_int64), ("N", C.c_int64),
+                ("calls", C.c_int64), ("ms", C.c_double)]
+
 
 # every symbol include/ppml_hip_backend.h declares (the executor driver above the launchers)
 BACKEND_SIGNATURES = {
@@ -68,6 +81,8 @@ BACKEND_SIGNATURES = {
     "ppml_hip_backend_set_skip_alloc": (None, [_vp, _i]),
     "ppml_hip_backend_set_q8_1_activations": (None, [_vp, _i]),
     "ppml_hip_backend_set_fuse_attention_bridges": (None, [_vp, _i]),
+    "ppml_hip_backend_set_f32_arithmetic": (None, [_vp, _i]),
+    "ppml_hip_backend_host_shadows_made": (_i, [_vp]),
     "ppml_hip_backend_graph_compute": (_i, [_vp, C.POINTER(_vp), _i]),
     "ppml_hip_backend_pack_weight": (_i, [_vp, _vp]),
 }

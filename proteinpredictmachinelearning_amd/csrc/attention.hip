@@ -426,7 +426,7 @@ extern "C" int flash_attn_forward_ex_hip(int B, int h, int L, int d, int causal,
     p.stage_rows = 0;                                 // set per instance
     p.in_ld = layout & 1;
     p.out_ld = (layout >> 1) & 1;
-    stats_record(static_cast<int64_t>(planes) * L, d, L);
+    StatsScope stat("hip/flash_attn", static_cast<int64_t>(planes) * L, d, L, static_cast<hipStream_t>(stream));
     hipStream_t s = static_cast<hipStream_t>(stream);
     // Four-wave work-groups (128 queries): 824 planes of 256 queries make 1648 of them, which spread over
     // 256 CUs more evenly than 824 eight-wave ones (6.4 per CU against 3.2, each rounded up).

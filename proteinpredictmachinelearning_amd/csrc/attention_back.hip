@@ -519,7 +519,7 @@ extern "C" int flash_attn_backward_hip(int B, int h, int L, int d, int causal, f
     p.causal = causal ? 1 : 0;
     p.scale = scale > 0.0f ? scale : 1.0f / std::sqrt(static_cast<float>(d));   // FlashAttn.cpp:153
     p.stage_rows = 0;
-    stats_record(static_cast<int64_t>(planes) * L, d, L);
+    StatsScope stat("hip/flash_attn_back", static_cast<int64_t>(planes) * L, d, L, static_cast<hipStream_t>(stream));
     hipStream_t s = static_cast<hipStream_t>(stream);
     return d <= 32 ? launch_back<32>(p, s) : launch_back<64>(p, s);
 }

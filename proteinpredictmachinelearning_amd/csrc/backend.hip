@@ -16,6 +16,7 @@
 //     views beforehand.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstring>
 #include <new>
 #include <unordered_map>
@@ -123,6 +124,23 @@ void HipBackend::synchronize() {
     (void)hipDeviceSynchronize();
 }
 
+// The operand combinations OP_MUL_MAT takes (src/backend/CUDABackend.cpp:121-157), one row each: the result
+// is always F32, a bias (src[2]) rides along on the all-F32 row only, and a quantized operand is the weight of
+// a product whose other side is F32 activations.
+enum OperandClass { OPERAND_F32, OPERAND_F16, OPERAND_Q8, OPERAND_OTHER };
+static OperandClass operand_class(int type) {
+    if (type == TENSOR_TYPE_F32) return OPERAND_F32;
+    if (type == TENSOR_TYPE_F16) return OPERAND_F16;
+    return is_quantized_type(type) ? OPERAND_Q8 : OPERAND_OTHER;
+}
+struct MulMatCombo { OperandClass src0, src1; bool bias; };
+static const MulMatCombo MUL_MAT_COMBOS[] = {
+    {OPERAND_F32, OPERAND_F32, true},
+    {OPERAND_F16, OPERAND_F16, false},
+    {OPERAND_Q8, OPERAND_F32, false},
+    {OPERAND_F32, OPERAND_Q8, false},
+};
+
 bool node_supported(const Tensor* node) {
     if (!node) return false;
     const Tensor* src0 = node->src[0];
@@ -133,21 +151,16 @@ bool node_supported(const Tensor* node) {
         case OP_RESHAPE:
             return true;
         case OP_MUL_MAT: {
-            if (!src1) return true;
-            // the bias epilogue exists on the f32 path only
-            if (node->src[2] && ((src0 && src0->type != TENSOR_TYPE_F32) || src1->type != TENSOR_TYPE_F32)) return false;
-            if (is_quantized_type(src1->type) || (src0 && is_quantized_type(src0->type))) {
-                if (!src0) return false;
-                const bool q0 = is_quantized_type(src0->type), q1 = is_quantized_type(src1->type);
-                if (q0 == q1) return false;     // exactly one side is the quantized weight
-                const Tensor* w = q0 ? src0 : src1;
-                const Tensor* a = q0 ? src1 : src0;
-                return w->quant_shape_valid() && is_quantized_type_supported(w->type) &&
-                       a->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32;
+            if (!src1) return true;              // nothing to multiply with yet: the reference lets such a node pass
+            if (!src0 || node->type != TENSOR_TYPE_F32) return false;
+            const OperandClass c0 = operand_class(src0->type), c1 = operand_class(src1->type);
+            for (const MulMatCombo& combo : MUL_MAT_COMBOS) {
+                if (combo.src0 != c0 || combo.src1 != c1) continue;
+                if (node->src[2] && !combo.bias) return false;
+                const Tensor* w = c0 == OPERAND_Q8 ? src0 : c1 == OPERAND_Q8 ? src1 : nullptr;
+                return !w || (w->quant_shape_valid() && is_quantized_type_supported(w->type));
             }
-            const bool ok_f32 = src0 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32;
-            const bool ok_f16 = src0 && src0->type == TENSOR_TYPE_F16 && src1->type == TENSOR_TYPE_F16;
-            return (ok_f32 || ok_f16) && node->type == TENSOR_TYPE_F32;
+            return false;
         }
         case OP_OUT_PROD:
             return src0 && src1 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
@@ -169,6 +182,10 @@ bool node_supported(const Tensor* node) {
             if (!src0 || !src1 || !node->src[2]) return false;
             if (!node->src[3] && !node->src[4]) return false;
             return src0->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32;
+        case OP_REPEAT_BACK:
+            // src/backend/CUDABackend.cpp:317-330: F32 in and out, at most four dimensions either side
+            return src0 && src0->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32 &&
+                   src0->ndim >= 1 && src0->ndim <= 4 && node->ndim >= 1 && node->ndim <= 4;
         case OP_PERMUTE:
         case OP_TRANSPOSE:
             // src/backend/CUDABackend.cpp:113-119
@@ -226,6 +243,73 @@ bool HipBackend::device_pointer_ok(const Tensor* t) const {
     }
     return true;
 }
+
+// Single-backend mode has no scheduler to copy host-resident leaves (embedding tables, constant masks, any
+// tensor bound to host memory) to the device, so the executor does it: every such source gets a device copy
+// for the duration of graph_compute, and the tensor's own fields are put back afterwards
+// (src/backend/CUDABackend.cpp:521-577, 824-830).
+namespace {
+bool is_device_memory(const void* p) {
+    hipPointerAttribute_t attr{};
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError();                        // an ordinary host pointer: not an error to report later
+        return false;
+    }
+    return attr.type == hipMemoryTypeDevice || attr.type == hipMemoryTypeManaged;
+}
+}  // namespace
+
+class HostShadows {
+public:
+    ~HostShadows() {
+        for (const Saved& s : saved_) {
+            s.t->data = s.data;
+            s.t->buffer = s.buffer;
+            s.t->buffer_offs = s.offs;
+        }
+        // views that were bound to a copy while it existed go back to unbound (only unbound sources get bound)
+        for (Tensor* t : borrowed_) {
+            t->data = nullptr;
+            t->buffer = nullptr;
+            t->buffer_offs = 0;
+        }
+        for (const Saved& s : saved_) (void)hipFree(s.dev);      // waits for the kernels that read it
+    }
+    // Leaves `t` bound to device memory if that can be arranged; a tensor it cannot help is left as it is,
+    // and the executor's pointer check names it.
+    void cover(Tensor* t) {
+        if (!t || !t->data) return;
+        for (const Saved& s : saved_) {
+            if (s.t == t) return;
+            const char* p = static_cast<const char*>(t->data);
+            if (p >= static_cast<const char*>(s.dev) && p < static_cast<const char*>(s.dev) + s.bytes) {
+                // a view of a covered leaf, resolved while the copy is the leaf's storage
+                if (std::find(borrowed_.begin(), borrowed_.end(), t) == borrowed_.end()) borrowed_.push_back(t);
+                return;
+            }
+        }
+        if (t->buffer ? !t->buffer->is_host() : is_device_memory(t->data)) return;
+        size_t bytes = t->nbytes();
+        if (bytes == 0) return;
+        void* dev = nullptr;
+        if (hipMalloc(&dev, bytes) != hipSuccess) { (void)hipGetLastError(); return; }
+        if (hipMemcpy(dev, t->data, bytes, hipMemcpyHostToDevice) != hipSuccess) {
+            (void)hipGetLastError();
+            (void)hipFree(dev);
+            return;
+        }
+        saved_.push_back(Saved{t, t->data, t->buffer, t->buffer_offs, dev, bytes});
+        t->data = dev;
+        t->buffer = nullptr;                            // the copy belongs to no Buffer
+        t->buffer_offs = 0;
+    }
+    size_t count() const { return saved_.size(); }
+
+private:
+    struct Saved { Tensor* t; void* data; Buffer* buffer; size_t offs; void* dev; size_t bytes; };
+    std::vector<Saved> saved_;
+    std::vector<Tensor*> borrowed_;
+};
 
 static Status status_of_rc(int rc) {
     if (rc == 0) return Status::SUCCESS;
@@ -460,6 +544,26 @@ Status HipBackend::kernel_flash_attn_back(Tensor* node) {
     return Status::SUCCESS;
 }
 
+// src/backend/CUDAKernels.cpp:1290-1320 (kernel_repeat_back_cross_cuda): dimension d of the node meets
+// dimension d of src[0] (only a node of higher rank is right-aligned), copies = integer quotient of the sizes.
+Status HipBackend::kernel_repeat_back(Tensor* node) {
+    const Tensor* a = node->src[0];
+    if (!a || !a->data || !node->data) return fail(Status::NOT_SUPPORTED, "repeat_back: unbound tensor");
+    const int off = a->ndim >= node->ndim ? 0 : a->ndim - node->ndim;
+    int64_t sd[4] = {1, 1, 1, 1}, dd[4] = {1, 1, 1, 1}, rd[4] = {1, 1, 1, 1};
+    for (int d = 0; d < node->ndim && d < 4; ++d) dd[d] = node->dims[d];
+    for (int d = 0; d < a->ndim && d < 4; ++d) sd[d] = a->dims[d];
+    for (int d = 0; d < 4; ++d) {
+        const int si = d + off;
+        const int64_t sdim = (si >= 0 && si < 4) ? sd[si] : 1;
+        rd[d] = dd[d] > 0 ? sdim / dd[d] : 1;
+    }
+    const int rc = repeat_back_hip(static_cast<const float*>(a->data), static_cast<float*>(node->data),
+                                   sd[0], sd[1], sd[2], sd[3], dd[0], dd[1], dd[2], dd[3], rd[0], rd[1], rd[2], rd[3], nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("repeat_back: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
 Status HipBackend::dispatch_node(Tensor* node) {
     switch (node->op) {
         case OP_MUL_MAT: return kernel_mul_mat(node);
@@ -469,6 +573,7 @@ Status HipBackend::dispatch_node(Tensor* node) {
         case OP_FLASH_ATTN_BACK: return kernel_flash_attn_back(node);
         case OP_PERMUTE:
         case OP_TRANSPOSE: return kernel_permute(node);
+        case OP_REPEAT_BACK: return kernel_repeat_back(node);
         case OP_TRI_MUL: return kernel_tri_mul(node);
         case OP_TRI_MUL_BACK: return kernel_tri_mul_back(node);
         case OP_OUTER_PROD_MEAN_BACK: return kernel_outer_prod_mean_back(node);
@@ -524,6 +629,15 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         }
     }
 
+    // the arithmetic this backend's f32 contractions were configured with, for the length of this call
+    struct ArithmeticScope {
+        int before = -1;
+        explicit ArithmeticScope(int mode) { if (mode == 0 || mode == 1) before = ppml_hip_set_f32_arithmetic(mode); }
+        ~ArithmeticScope() { if (before >= 0) ppml_hip_set_f32_arithmetic(before); }
+    } arithmetic(f32_arithmetic_);
+
+    HostShadows shadows;                                // restored and freed on every way out of this function
+    host_shadows_made_ = 0;
     int index = -1;
     for (Tensor* node : *graph) {
         ++index;
@@ -555,6 +669,11 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
             }
         }
         resolve_views(exec);
+        if (!skip_alloc_) {
+            // under a scheduler the copies across backends are nodes of the graph; here nobody else makes them
+            for (Tensor* src : exec->src) shadows.cover(src);
+            host_shadows_made_ = shadows.count();
+        }
 
         // single-backend mode: outputs nobody allocated get their own device buffer -- the node itself
         // and the second output the fused attention node carries in src[4] (its LSE buffer)
@@ -737,6 +856,12 @@ void ppml_hip_backend_set_fuse_attention_bridges(ppml_hip_backend* b, int on) {
 }
 void ppml_hip_backend_set_skip_alloc(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_skip_alloc(on != 0);
+}
+void ppml_hip_backend_set_f32_arithmetic(ppml_hip_backend* b, int mode) {
+    if (b) b->impl.set_f32_arithmetic(mode);
+}
+int ppml_hip_backend_host_shadows_made(const ppml_hip_backend* b) {
+    return b ? static_cast<int>(b->impl.host_shadows_made()) : 0;
 }
 
 }  // extern "C"

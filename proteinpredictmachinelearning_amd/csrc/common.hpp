@@ -18,7 +18,27 @@ enum Rc { RC_OK = 0, RC_BAD_ARGS = 1, RC_K_NOT_32 = 2, RC_ALLOC = 3, RC_WTYPE = 
 
 void set_error(const char* fmt, ...);
 int  check_launch(const char* what);     // hipGetLastError -> RC_LAUNCH with message
-void stats_record(int64_t M, int64_t K, int64_t N);
+
+// One launcher call in the MUL_MAT statistics (include/ppml/MulMatStats.h:154-169; the event pair of
+// src/cuda/CUDAKernels.cu:1713-1732): counts the call and, outside stream capture, brackets the work
+// issued on `stream` during its lifetime with two events.  Costs one relaxed load when statistics are off.
+bool stats_enabled();
+class StatsScope {
+public:
+    StatsScope(const char* path, int64_t M, int64_t K, int64_t N, hipStream_t stream);
+    ~StatsScope();
+    void set_path(const char* path) { path_ = path; }     // a string literal: kept by pointer until the scope ends
+    StatsScope(const StatsScope&) = delete;
+    StatsScope& operator=(const StatsScope&) = delete;
+private:
+    const char* path_;
+    int64_t M_, K_, N_;
+    hipStream_t stream_;
+    hipEvent_t e0_ = nullptr, e1_ = nullptr;
+    bool on_ = false, timed_ = false;
+};
+hipMemPool_t workspace_pool();         // the library's stream-ordered pool on the current device, or null
+void set_q8_path(int path);              // what ppml_hip_q8_last_path() reports for the calling thread
 
 typedef int   v4i  __attribute__((ext_vector_type(4)));
 typedef int   v16i __attribute__((ext_vector_type(16)));

@@ -676,36 +676,6 @@ __global__ __launch_bounds__(256) void reduce_slices_kernel(const GemmParams p, 
     }
 }
 
-// Stream-ordered workspace for the planes: a pool of this library's own per device, which keeps what it
-// has allocated (release threshold at the maximum), so after the first call an allocation is a list
-// operation ordered on the caller's stream; freeing is ordered on that stream as well, which makes reuse
-// from other streams safe without the library tracking anything.  Returns null when the device has no pool.
-hipMemPool_t workspace_pool() {
-    constexpr int MAX_DEVICES = 64;
-    static std::mutex mu;
-    static hipMemPool_t pools[MAX_DEVICES];
-    static bool tried[MAX_DEVICES];
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) { (void)hipGetLastError(); return nullptr; }
-    std::lock_guard<std::mutex> guard(mu);
-    if (!tried[dev]) {
-        tried[dev] = true;
-        hipMemPoolProps props{};
-        props.allocType = hipMemAllocationTypePinned;
-        props.handleTypes = hipMemHandleTypeNone;
-        props.location.type = hipMemLocationTypeDevice;
-        props.location.id = dev;
-        if (hipMemPoolCreate(&pools[dev], &props) != hipSuccess) {
-            (void)hipGetLastError();
-            pools[dev] = nullptr;
-        } else {
-            uint64_t keep = ~0ull;
-            (void)hipMemPoolSetAttribute(pools[dev], hipMemPoolAttrReleaseThreshold, &keep);
-        }
-    }
-    return pools[dev];
-}
-
 int launch_split(const SplitJob& jb, hipStream_t stream) {
     const int64_t threads = static_cast<int64_t>(jb.chunks) * jb.rows_pad * 2;
     const dim3 grid(static_cast<unsigned>((threads + 255) / 256)), block(256);
@@ -718,16 +688,14 @@ int launch_split(const SplitJob& jb, hipStream_t stream) {
 // Which matrix pipe multiplies binary32 operands: 0 = the bf16 pipe through the exact three-way split (the
 // default), 1 = the fp32 pipe (v_mfma_f32_32x32x2_f32, k ascending two at a time).  Set through
 // ppml_hip_set_f32_arithmetic or, before the first contraction, by PPML_HIP_F32_ARITH=fp32 in the environment.
-std::atomic<int> g_f32_arithmetic{-1};
+thread_local int t_f32_arithmetic = -1;            // per thread: callers with different wishes do not race
 
 int f32_arithmetic() {
-    int mode = g_f32_arithmetic.load(std::memory_order_relaxed);
-    if (mode < 0) {
+    if (t_f32_arithmetic < 0) {
         const char* env = std::getenv("PPML_HIP_F32_ARITH");
-        mode = (env && std::strcmp(env, "fp32") == 0) ? 1 : 0;
-        g_f32_arithmetic.store(mode, std::memory_order_relaxed);
+        t_f32_arithmetic = (env && std::strcmp(env, "fp32") == 0) ? 1 : 0;
     }
-    return mode;
+    return t_f32_arithmetic;
 }
 
 int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
@@ -861,14 +829,14 @@ using namespace ppmlhip;
 
 extern "C" int ppml_hip_set_f32_arithmetic(int mode) {
     const int before = f32_arithmetic();
-    if (mode == 0 || mode == 1) g_f32_arithmetic.store(mode, std::memory_order_relaxed);
+    if (mode == 0 || mode == 1) t_f32_arithmetic = mode;
     return before;
 }
 
 extern "C" int mul_mat_hip(const float* A, const float* B, float* C, int M, int K, int N,
                            const float* bias, ppml_hip_stream_t stream) {
     if (!A || !B || !C || M <= 0 || K <= 0 || N <= 0) { set_error("mul_mat_hip: bad arguments (M=%d K=%d N=%d)", M, K, N); return RC_BAD_ARGS; }
-    stats_record(M, K, N);
+    StatsScope stat("hip/mul_mat", M, K, N, static_cast<hipStream_t>(stream));
     GemmParams p = plain_params();
     p.A = A; p.B = B; p.C = C; p.bias = bias;
     p.M = M; p.N = N; p.K = K;
@@ -880,7 +848,7 @@ extern "C" int mul_mat_hip(const float* A, const float* B, float* C, int M, int 
 extern "C" int mul_mat_f16_hip(const void* A16, const void* B16, float* C, int M, int K, int N,
                                const float* bias, ppml_hip_stream_t stream) {
     if (!A16 || !B16 || !C || M <= 0 || K <= 0 || N <= 0) { set_error("mul_mat_f16_hip: bad arguments (M=%d K=%d N=%d)", M, K, N); return RC_BAD_ARGS; }
-    stats_record(M, K, N);
+    StatsScope stat("hip/mul_mat-f16", M, K, N, static_cast<hipStream_t>(stream));
     GemmParams p = plain_params();
     p.A = static_cast<const float*>(A16); p.B = static_cast<const float*>(B16); p.C = C; p.bias = bias;
     p.M = M; p.N = N; p.K = K;
@@ -893,7 +861,7 @@ extern "C" int mul_mat_f16_hip(const void* A16, const void* B16, float* C, int M
 extern "C" int mul_mat_tn_hip(const float* A, const float* Bm, float* O, int M, int K, int Nc, float alpha,
                               ppml_hip_stream_t stream) {
     if (!A || !Bm || !O || M <= 0 || K <= 0 || Nc <= 0) { set_error("mul_mat_tn_hip: bad arguments"); return RC_BAD_ARGS; }
-    stats_record(M, K, Nc);
+    StatsScope stat("hip/mul_mat-tn", M, K, Nc, static_cast<hipStream_t>(stream));
     GemmParams p = plain_params();
     p.A = A; p.B = Bm; p.C = O;
     p.M = M; p.N = Nc; p.K = K;
@@ -920,7 +888,7 @@ extern "C" int out_prod_scaled_hip(const float* src0, const float* src1, float* 
                   (long long)ne0, (long long)ne1, (long long)ne2, (long long)ne3);
         return RC_BAD_ARGS;
     }
-    stats_record(ne1, ne01, ne0);
+    StatsScope stat("hip/out_prod", ne1, ne01, ne0, static_cast<hipStream_t>(stream));
     GemmParams p = plain_params();
     p.A = src1; p.B = src0; p.C = dst;                 // rows = i1 (src1), cols = i0 (src0)
     p.M = static_cast<int>(ne1); p.N = static_cast<int>(ne0); p.K = static_cast<int>(ne01);
@@ -950,7 +918,7 @@ extern "C" int outer_prod_mean_hip(const float* left, const float* right, float*
     if (!left || !right || !dst || D <= 0 || L <= 0 || N <= 0 || B <= 0 || D * L > 0x7fffffff || N > 0x7fffffff) {
         set_error("outer_prod_mean_hip: bad arguments"); return RC_BAD_ARGS;
     }
-    stats_record(D * L, N, D * L);
+    StatsScope stat("hip/outer_prod_mean", D * L, N, D * L, static_cast<hipStream_t>(stream));
     GemmParams p = plain_params();
     p.A = left; p.B = right; p.C = dst;               // rows = (d1,i), cols = (d2,j), k = n
     p.M = p.N = static_cast<int>(D * L); p.K = static_cast<int>(N);
@@ -969,7 +937,7 @@ extern "C" int outer_product_mean_value_hip(const float* left, const float* righ
     if (!left || !right || !dst || D <= 0 || L <= 0 || N <= 0 || B <= 0 || D * L > 0x7fffffff || N > 0x7fffffff) {
         set_error("outer_product_mean_value_hip: bad arguments"); return RC_BAD_ARGS;
     }
-    stats_record(D * L, N, D * L);
+    StatsScope stat("hip/outer_product_mean-value", D * L, N, D * L, static_cast<hipStream_t>(stream));
     GemmParams p = plain_params();
     p.A = left; p.B = right; p.C = dst;               // rows = (i,d1), cols = (j,d2), k = n
     p.M = p.N = static_cast<int>(L * D); p.K = static_cast<int>(N);
@@ -989,7 +957,7 @@ extern "C" int tri_mul_hip(const float* left, const float* right, float* dst,
         I > 0x7fffffff || J > 0x7fffffff || K > 0x7fffffff || D > 0x7fffffff || B > 0x7fffffff) {
         set_error("tri_mul_hip: bad arguments"); return RC_BAD_ARGS;
     }
-    stats_record(I, K, J);
+    StatsScope stat("hip/tri_mul", I, K, J, static_cast<hipStream_t>(stream));
     GemmParams p = plain_params();
     p.A = left; p.B = right; p.C = dst;                // rows = i, cols = j, planes = (d, b)
     p.M = static_cast<int>(I); p.N = static_cast<int>(J); p.K = static_cast<int>(K);
@@ -1021,7 +989,7 @@ extern "C" int tri_mul_back_hip(const float* grad, const float* left, const floa
     const auto launch = [&](const float* a, int64_t a_rs, int64_t a_ks, const float* b, int64_t b_rs, int64_t b_ks,
                             float* c, int64_t c_mi, int64_t c_ni, int64_t M, int64_t N, int64_t Kc,
                             int64_t a_p3, int64_t b_p3, int64_t c_p3) {
-        stats_record(M, Kc, N);
+        StatsScope stat("hip/tri_mul_back", M, Kc, N, static_cast<hipStream_t>(stream));
         GemmParams p = plain_params();
         p.A = a; p.B = b; p.C = c;
         p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(Kc);
@@ -1054,7 +1022,7 @@ extern "C" int outer_prod_mean_back_hip(const float* grad, const float* left, co
     //                        gright[(d2,j)][n] = inv_N * sum_{(d1,i)} grad * left[(d1,i)][n]:
     // two contractions whose first operand has a compound row index and a compound contraction index.
     const auto launch = [&](const float* other, float* out, int64_t mo, int64_t mi, int64_t ko, int64_t ki) {
-        stats_record(D * L, D * L, N);
+        StatsScope stat("hip/outer_prod_mean_back", D * L, D * L, N, static_cast<hipStream_t>(stream));
         GemmParams p = plain_params();
         p.A = grad; p.B = other; p.C = out;
         p.M = static_cast<int>(D * L); p.N = static_cast<int>(N); p.K = static_cast<int>(D * L);

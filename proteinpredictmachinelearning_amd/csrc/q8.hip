@@ -307,19 +307,6 @@ __global__ __launch_bounds__(64) void q8_weight_pack_kernel(const uint8_t* __res
 // rows K is walked in chunks and the partial result of every output is carried in C itself, which
 // keeps the per-output block order intact.
 // ------------------------------------------------------------------------------------------
-#ifdef PPML_Q8_TRACE
-// Development aid, compiled out of the library: per-wave timestamps of the kernel's phases.
-__device__ unsigned long long* g_q8_trace = nullptr;
-__device__ int g_q8_dbg[4] = {0, 0, 0, 0};
-#define PPML_TRACE_MARK(slot)                                                                      \
-    do {                                                                                           \
-        if ((PPML_Q8_TRACE == 1 || (slot) == 0 || (slot) >= 60) && g_q8_trace && (threadIdx.x & 63) == 0) \
-            g_q8_trace[(static_cast<size_t>(blockIdx.x) * NW + (threadIdx.x >> 6)) * 64 + (slot)] = \
-                __builtin_amdgcn_s_memrealtime();   /* 100 MHz, common to the whole device */      \
-    } while (0)
-#else
-#define PPML_TRACE_MARK(slot) do {} while (0)
-#endif
 
 constexpr int TILE_TOK = 32;
 // Cache policy of the output stores of the weight-stationary kernel: sc0 | nt.  The output is
@@ -431,7 +418,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
     const WGeom g{W, M, nblk, packed_tiles(M)};
     const COut out{C, M, N, c_trans};
     const int tok = tok0 + j;                          // this lane's activation row in every MFMA result
-    PPML_TRACE_MARK(0);
 
     for (int b0 = 0; b0 < nblk; b0 += kc) {
         const int nb = (nblk - b0) < kc ? (nblk - b0) : kc;
@@ -493,9 +479,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
                 wp.load(W);
             }
         }
-        PPML_TRACE_MARK(1);
         __syncthreads();
-        PPML_TRACE_MARK(2);
 
         // ---------------- phase 2 + 3: one pair of column tiles at a time
         for (int pr = wave; pr < npairs; pr += NW) {
@@ -580,9 +564,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
                 }
             }
         }
-        PPML_TRACE_MARK(3);
     }
-    PPML_TRACE_MARK(4);
 }
 
 template <int NW, int WT>
@@ -639,7 +621,7 @@ constexpr int ws_staging_regs(int nblk, int nw = 8) {   // 8 registers per unit 
 }
 constexpr int ws_compiler_vgprs(int nblk, int nw = 8) { return 256 - ws_staging_regs(nblk, nw); }
 
-template <int NW, int TPW, int NBLK, int WL, bool DUMP>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81>
 __device__ __forceinline__ void q8_linear_ws_body(
     const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
     int M, int N, int ntiles, int npart, int relu,
@@ -769,7 +751,6 @@ __device__ __forceinline__ void q8_linear_ws_body(
     const int part_col = wg % TPW;
     auto tile_of = [&](int i) { return i < n_full ? wg + i * grid : ntiles + wg / TPW; };
     int tile = tile_of(0);
-    PPML_TRACE_MARK(0);
     if (tid < WS_NBUF) lds_ready[tid] = 0u;
     __syncthreads();                                   // the only barrier of the kernel
     if (n_iter > 0) load_tile(tile, xv);
@@ -807,7 +788,6 @@ __device__ __forceinline__ void q8_linear_ws_body(
             }
         }
     }
-    PPML_TRACE_MARK(42);
 
     // quantizes the tile held in xv into LDS buffer `buf`
     auto quantize_tile = [&](int buf, int tok0, v4f (&xv)[UPW][2]) {
@@ -826,7 +806,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
 #pragma unroll
                 for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
             }
-            const BlockQuant bq = quantize_block_lane<false>(x0, x1);
+            const BlockQuant bq = quantize_block_lane<Q81>(x0, x1);
             uint2* dst = reinterpret_cast<uint2*>(lds_a[buf]) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
             *dst = uint2{bq.q_lo, bq.q_hi};
             if (c4 == 0) lds_d[buf][bl * 32 + row] = uint2{bq.d_bits, 0u};
@@ -854,7 +834,6 @@ __device__ __forceinline__ void q8_linear_ws_body(
         quantize_tile(0, tile * TILE_TOK, xv);
         announce(0);
     }
-    PPML_TRACE_MARK(43);
     // weight scales and the fragments that live in LDS: written and read by this wave only
 #pragma unroll
     for (int t = 0; t < TPW; ++t) {
@@ -876,13 +855,11 @@ __device__ __forceinline__ void q8_linear_ws_body(
             my_wq[((t - (TPW - WL)) * NBLK + b) * 64] =
                 *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(col_tile_of(t) * NBLK + b) * 64 + lane) * 16);
     }
-    PPML_TRACE_MARK(44);
     // Every weight fragment has arrived before the loop starts: a load still pending here would make
     // its first use inside the loop wait for vmcnt(0), i.e. for all output stores, on every iteration.
     __builtin_amdgcn_s_waitcnt(0x0f70);                // vmcnt(0), other counters untouched
     // the second tile is requested now and quantized two thirds into the first one
     if (n_iter > 1) load_tile_async(tile_of(1));
-    PPML_TRACE_MARK(1);
 
     // Step at which the next tile is quantized.  Its loads were issued one full round of column tiles
     // earlier (right after the previous quantization freed the staging registers), so they have
@@ -897,11 +874,6 @@ __device__ __forceinline__ void q8_linear_ws_body(
     // No barrier inside the loop.  A wave may start tile `it` once all waves have announced it, which
     // also means all of them are past two thirds of tile it-1; the tile quantized during tile `it`
     // goes to buffer (it+1) % 3, last read for tile it-2, which every wave has left by then.
-#ifdef PPML_Q8_TRACE
-    if (g_q8_dbg[0] > 0 && wave >= 4) {
-        for (int i = 0; i < g_q8_dbg[0]; ++i) __builtin_amdgcn_s_sleep(8);   // 512 cycles each
-    }
-#endif
     for (int it = 0; it < n_iter; ++it) {
         tile = tile_of(it);
         const int buf = it % WS_NBUF;
@@ -910,7 +882,6 @@ __device__ __forceinline__ void q8_linear_ws_body(
         const int next = has_next ? tile_of(it + 1) : tile;
         const bool partial = it >= n_full;             // compute column tile part_col only
         await_tile(buf, static_cast<unsigned>(NW) * static_cast<unsigned>(it / WS_NBUF + 1));
-        PPML_TRACE_MARK(2 + 10 * it);
 
         // ---------------- MFMA one block ahead of the settle; tiles in turn, blocks ascending
         v16i zero_i;
@@ -1004,7 +975,6 @@ __device__ __forceinline__ void q8_linear_ws_body(
             if (!opaque_one()) continue;
             if (partial && t0 != part_col) continue;
             if (t0 * NBLK == QSTEP_TILE * NBLK && has_next) {
-                PPML_TRACE_MARK(2 + 10 * it + 7);
                 {
                     v4f xn[UPW][2];
                     if (it == 0) take_tile(std::integral_constant<int, NEWER_FIRST>{}, next, xn);
@@ -1013,7 +983,6 @@ __device__ __forceinline__ void q8_linear_ws_body(
                     quantize_tile((it + 1) % WS_NBUF, next * TILE_TOK, xn);
                     announce((it + 1) % WS_NBUF);
                 }
-                PPML_TRACE_MARK(2 + 10 * it + 8);
             }
             // Pairs of steps use the operand sets pe / po alternately, so they swap roles by name.  A
             // pair starts by issuing its scale MFMA and the block sum of its second step; the block
@@ -1060,18 +1029,8 @@ __device__ __forceinline__ void q8_linear_ws_body(
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
-            PPML_TRACE_MARK(2 + 10 * it + 1 + t0);
         }
-        PPML_TRACE_MARK(2 + 10 * it + 9);
     }
-#ifdef PPML_Q8_TRACE
-    // shader clock under this kernel's load: 1024 x 16 x s_nop 15 = 262144 cycles plus loop overhead
-    PPML_TRACE_MARK(60);
-    for (int i = 0; g_q8_trace && i < 1024; ++i)
-        asm volatile("s_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\n"
-                     "s_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15\ns_nop 15" ::: "memory");
-    PPML_TRACE_MARK(61);
-#endif
 }
 
 // The attribute takes a literal, hence one kernel per staging size (16 registers up to K = 256, 32 or
@@ -1079,30 +1038,30 @@ __device__ __forceinline__ void q8_linear_ws_body(
 // value counts architectural and accumulation registers separately): 120 keeps it below v240.  A
 // value the compiler does not honour would go unnoticed until its registers and the staged tile
 // collide, so the build checks the generated code (check_ws_isa.py).
-template <int NW, int TPW, int NBLK, int WL, bool DUMP>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(120)))
 void q8_linear_ws_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                          int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                          int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 120, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
-template <int NW, int TPW, int NBLK, int WL, bool DUMP>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(112)))
 void q8_linear_ws32_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 112, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
-template <int NW, int TPW, int NBLK, int WL, bool DUMP>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(96)))
 void q8_linear_ws64_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 96, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
 int device_cu_count() {
@@ -1117,7 +1076,7 @@ int device_cu_count() {
     return cus;
 }
 
-template <int TPW, int NBLK, int WL, int NW = 8>
+template <int TPW, int NBLK, int WL, int NW, bool Q81>
 int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int relu,
                         void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
     // Eight waves fill a CU (256 registers each): one resident work-group of 8 waves per CU, or two
@@ -1142,15 +1101,15 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
     using KernelFn = void (*)(const uint8_t*, const float*, float*, int, int, int, int, int, uint8_t*, int32_t*);
     KernelFn fast, dump;
     if constexpr (ws_staging_regs(NBLK, NW) == 16) {
-        fast = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false>;
-        dump = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true>;
+        fast = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81>;
+        dump = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true, Q81>;
     } else if constexpr (ws_staging_regs(NBLK, NW) == 32) {
-        fast = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, false>;
-        dump = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, true>;
+        fast = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, false, Q81>;
+        dump = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, true, Q81>;
     } else {
         static_assert(ws_staging_regs(NBLK, NW) == 64, "no kernel for this staging size");
-        fast = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, false>;
-        dump = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, true>;
+        fast = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, false, Q81>;
+        dump = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, true, Q81>;
     }
     if (lds > 64 * 1024) {
         static const hipError_t attr_fast = hipFuncSetAttribute(
@@ -1172,24 +1131,34 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
 }
 
 // returns -1 when the shape has no weight-stationary instance
+template <bool Q81>
 int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
                      int relu, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
     if (!c_trans) return -1;
     if (static_cast<int64_t>(N) * M * 4 >= 0x7fff0000LL) return -1;   // the kernel addresses C with 32-bit byte offsets
     const int mct = (M + 31) / 32;
     const int tpw = (mct + 7) / 8;
+#define PPML_WS(TPW, NBLK, WL, NW) return launch_q8_linear_ws<TPW, NBLK, WL, NW, Q81>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
     // Up to four column tiles: work-groups of four waves, one column tile each and two per CU, so no
     // wave idles (with eight waves half of them would have no column tile).
     if (mct <= 4) {
-        if (nblk == 4) return launch_q8_linear_ws<1, 4, 0, 4>(W, X, C, M, N, relu, xq_dump, sums_dump, stream);
-        if (nblk == 8) return launch_q8_linear_ws<1, 8, 0, 4>(W, X, C, M, N, relu, xq_dump, sums_dump, stream);
-        if (nblk == 16) return launch_q8_linear_ws<1, 16, 0, 4>(W, X, C, M, N, relu, xq_dump, sums_dump, stream);
+        if (nblk == 4) PPML_WS(1, 4, 0, 4);
+        if (nblk == 8) PPML_WS(1, 8, 0, 4);
+        if (nblk == 16) PPML_WS(1, 16, 0, 4);
     }
-#define PPML_WS(TPW, NBLK, WL) if (tpw == TPW && nblk == NBLK) return launch_q8_linear_ws<TPW, NBLK, WL>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
     // (column tiles per wave, blocks of K, column tiles whose fragments live in LDS instead of registers)
-    PPML_WS(1, 4, 0);  PPML_WS(2, 4, 0);  PPML_WS(3, 4, 0);  PPML_WS(4, 4, 0);
-    PPML_WS(1, 8, 0);  PPML_WS(2, 8, 0);  PPML_WS(3, 8, 1);
-    PPML_WS(1, 16, 0);
+    if (nblk == 4) {
+        if (tpw == 1) PPML_WS(1, 4, 0, 8);
+        if (tpw == 2) PPML_WS(2, 4, 0, 8);
+        if (tpw == 3) PPML_WS(3, 4, 0, 8);
+        if (tpw == 4) PPML_WS(4, 4, 0, 8);
+    } else if (nblk == 8) {
+        if (tpw == 1) PPML_WS(1, 8, 0, 8);
+        if (tpw == 2) PPML_WS(2, 8, 0, 8);
+        if (tpw == 3) PPML_WS(3, 8, 1, 8);
+    } else if (nblk == 16) {
+        if (tpw == 1) PPML_WS(1, 16, 0, 8);
+    }
 #undef PPML_WS
     return -1;
 }
@@ -1272,18 +1241,18 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
     if ((K % QK) != 0) { set_error("mul_mat_q8_hip: K=%d is not a multiple of 32", K); return RC_K_NOT_32; }
     const int nblk = K / QK;
     const int relu = flags & 1;                        // bit 0: ReLU on X
-    const int act = flags & 3;                         // bit 1: Q8_1 rule for the activations (general kernel only)
+    const int act = flags & 3;                         // bit 1: Q8_1 rule for the activations
     hipStream_t s = static_cast<hipStream_t>(stream);
-    stats_record(M, K, N);
+    StatsScope stat("hip/q8-general", M, K, N, s);
+    set_q8_path(PPML_Q8_PATH_GENERAL);
     switch (wtype) {
         case PPML_WTYPE_Q8_0:  return dispatch_q8_linear<PPML_WTYPE_Q8_0>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_1:  return dispatch_q8_linear<PPML_WTYPE_Q8_1>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0R: return dispatch_q8_linear<PPML_WTYPE_Q8_0R>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0M: {
-            if (!(act & 2)) {
-                const int rc = try_q8_linear_ws(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
-                if (rc >= 0) return rc;
-            }
+            const int rc = (act & 2) ? try_q8_linear_ws<true>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s)
+                                     : try_q8_linear_ws<false>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
+            if (rc >= 0) { set_q8_path(PPML_Q8_PATH_WEIGHT_STATIONARY); stat.set_path("hip/q8-weight-stationary"); return rc; }
             return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         }
         default: set_error("mul_mat_q8_hip: unsupported wtype %d", wtype); return RC_WTYPE;

@@ -1,10 +1,16 @@
 // Device selection, error text and the per-shape call statistics of the backend.
 #include "common.hpp"
 
+#include <algorithm>
+#include <atomic>
+#include <chrono>
 #include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <string>
+#include <tuple>
+#include <vector>
 
 namespace ppmlhip {
 
@@ -24,25 +30,172 @@ int check_launch(const char* what) {
     return RC_LAUNCH;
 }
 
-// Mirrors mulmat_stats_record (include/ppml/MulMatStats.h:154-169): a histogram keyed by shape,
-// switched on by PPML_MULMAT_STATS=1.  Only call counts are kept; kernel times come from rocprof.
-static std::mutex g_stats_mtx;
-static std::map<uint64_t, int64_t> g_stats;
+// Mirrors the reference's MUL_MAT statistics (include/ppml/MulMatStats.h:39-169 and the event
+// fold-in of src/cuda/CUDAKernels.cu:1693-1732): a histogram keyed by (path, M, K, N) with a call
+// count and the accumulated milliseconds of the launches, measured with a pair of events recorded on
+// the launcher's stream so that nothing waits.  The elapsed times are folded in when the table is
+// read or dumped (and at exit).  Switched on by PPML_MULMAT_STATS=1 or ppml_hip_mulmat_stats_enable.
+// Unlike the reference's key (20 bits per dimension, MulMatStats.h:70-74) the key keeps whole values.
+namespace {
 
-static bool stats_enabled() {
-    static const bool on = [] {
+struct StatKey {
+    std::string path;
+    int64_t M, K, N;
+    bool operator<(const StatKey& o) const { return std::tie(path, M, K, N) < std::tie(o.path, o.M, o.K, o.N); }
+};
+struct StatVal { int64_t calls = 0; double ms = 0.0; };
+struct Pending { StatKey key; hipEvent_t e0, e1; };
+
+struct Stats {
+    std::mutex mu;
+    std::map<StatKey, StatVal> table;
+    std::vector<Pending> pending;
+    std::vector<hipEvent_t> spare;                     // events to use again
+    std::chrono::steady_clock::time_point t_first{};
+    bool started = false;
+};
+Stats& stats() {
+    static Stats* s = new Stats();                     // never destroyed: the exit handler still reads it
+    return *s;
+}
+std::atomic<int> g_stats_on{-1};
+
+// Elapsed times of finished launches go into the table; with `wait` the unfinished ones are waited for.
+void fold_pending_locked(Stats& s, bool wait) {
+    size_t keep = 0;
+    for (size_t i = 0; i < s.pending.size(); ++i) {
+        Pending& p = s.pending[i];
+        hipError_t e = wait ? hipEventSynchronize(p.e1) : hipEventQuery(p.e1);
+        if (e == hipErrorNotReady) { s.pending[keep++] = p; continue; }
+        float ms = 0.0f;
+        if (e == hipSuccess && hipEventElapsedTime(&ms, p.e0, p.e1) == hipSuccess) s.table[p.key].ms += ms;
+        else (void)hipGetLastError();
+        s.spare.push_back(p.e0);
+        s.spare.push_back(p.e1);
+    }
+    s.pending.resize(keep);
+}
+
+void dump_locked(Stats& s) {
+    const double wall_ms = s.started
+        ? std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - s.t_first).count() : 0.0;
+    int64_t calls = 0;
+    double ms = 0.0;
+    std::map<std::string, StatVal> by_path;
+    std::vector<std::pair<StatKey, StatVal>> rows(s.table.begin(), s.table.end());
+    for (const auto& kv : rows) {
+        calls += kv.second.calls; ms += kv.second.ms;
+        by_path[kv.first.path].calls += kv.second.calls;
+        by_path[kv.first.path].ms += kv.second.ms;
+    }
+    std::fprintf(stderr, "\n[MULMAT-STAT] ===== MUL_MAT shapes and times (PPML_MULMAT_STATS=1) =====\n");
+    std::fprintf(stderr, "[MULMAT-STAT] total calls=%lld device time=%.3f ms | wall since the first call=%.0f ms (%.1f%%)\n",
+                 (long long)calls, ms, wall_ms, wall_ms > 0.0 ? 100.0 * ms / wall_ms : 0.0);
+    for (const auto& kv : by_path)
+        std::fprintf(stderr, "[MULMAT-STAT]   %-24s calls=%-7lld time=%10.3f ms\n", kv.first.c_str(), (long long)kv.second.calls, kv.second.ms);
+    std::sort(rows.begin(), rows.end(), [](const auto& a, const auto& b) { return a.second.ms > b.second.ms; });
+    std::fprintf(stderr, "[MULMAT-STAT] top shapes by accumulated time (M = output rows, K = contracted, N = output columns):\n");
+    for (size_t i = 0; i < rows.size() && i < 12; ++i)
+        std::fprintf(stderr, "[MULMAT-STAT]   #%-2zu %-24s M=%-8lld K=%-8lld N=%-8lld calls=%-7lld time=%10.3f ms\n", i + 1,
+                     rows[i].first.path.c_str(), (long long)rows[i].first.M, (long long)rows[i].first.K, (long long)rows[i].first.N,
+                     (long long)rows[i].second.calls, rows[i].second.ms);
+    std::fprintf(stderr, "[MULMAT-STAT] ===== end =====\n");
+}
+
+void stats_at_exit() {
+    Stats& s = stats();
+    std::lock_guard<std::mutex> lock(s.mu);
+    if (s.table.empty()) return;
+    fold_pending_locked(s, true);
+    dump_locked(s);
+}
+
+}  // namespace
+
+bool stats_enabled() {
+    int on = g_stats_on.load(std::memory_order_relaxed);
+    if (on < 0) {
         const char* e = std::getenv("PPML_MULMAT_STATS");
-        return e && e[0] && e[0] != '0';
-    }();
-    return on;
+        on = (e && e[0] && std::strcmp(e, "0") != 0) ? 1 : 0;      // the reference's rule, MulMatStats.h:39-45
+        g_stats_on.store(on, std::memory_order_relaxed);
+    }
+    return on == 1;
 }
 
-void stats_record(int64_t M, int64_t K, int64_t N) {
+StatsScope::StatsScope(const char* path, int64_t M, int64_t K, int64_t N, hipStream_t stream)
+    : path_(path), M_(M), K_(K), N_(N), stream_(stream) {
     if (!stats_enabled()) return;
-    const uint64_t key = (static_cast<uint64_t>(M) << 40) | (static_cast<uint64_t>(K) << 20) | static_cast<uint64_t>(N);
-    std::lock_guard<std::mutex> lock(g_stats_mtx);
-    ++g_stats[key];
+    on_ = true;
+    // events cannot be recorded into a stream that is being captured: count the call only
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) { (void)hipGetLastError(); cap = hipStreamCaptureStatusNone; }
+    if (cap != hipStreamCaptureStatusNone) return;
+    Stats& s = stats();
+    {
+        std::lock_guard<std::mutex> lock(s.mu);
+        for (hipEvent_t* e : {&e0_, &e1_}) {
+            if (!s.spare.empty()) { *e = s.spare.back(); s.spare.pop_back(); }
+        }
+    }
+    if (!e0_ && hipEventCreate(&e0_) != hipSuccess) { (void)hipGetLastError(); e0_ = nullptr; }
+    if (!e1_ && hipEventCreate(&e1_) != hipSuccess) { (void)hipGetLastError(); e1_ = nullptr; }
+    timed_ = e0_ && e1_ && hipEventRecord(e0_, stream) == hipSuccess;
+    if (!timed_) (void)hipGetLastError();
 }
+
+StatsScope::~StatsScope() {
+    if (!on_) return;
+    if (timed_ && hipEventRecord(e1_, stream_) != hipSuccess) { (void)hipGetLastError(); timed_ = false; }
+    Stats& s = stats();
+    std::lock_guard<std::mutex> lock(s.mu);
+    static const bool registered = [] { std::atexit(stats_at_exit); return true; }();
+    (void)registered;
+    if (!s.started) { s.t_first = std::chrono::steady_clock::now(); s.started = true; }
+    StatKey key{path_ ? path_ : "unknown", M_, K_, N_};
+    ++s.table[key].calls;
+    if (timed_) {
+        s.pending.push_back(Pending{key, e0_, e1_});
+        if (s.pending.size() >= 4096) fold_pending_locked(s, false);
+    } else {
+        if (e0_) s.spare.push_back(e0_);
+        if (e1_) s.spare.push_back(e1_);
+    }
+}
+
+// Stream-ordered workspace of the launchers that need one (the split planes of the large f32 contractions,
+// the partial sums of repeat_back): a pool of this library's own per device, which keeps what it
+// has allocated (release threshold at the maximum), so after the first call an allocation is a list
+// operation ordered on the caller's stream; freeing is ordered on that stream as well, which makes reuse
+// from other streams safe without the library tracking anything.  Returns null when the device has no pool.
+hipMemPool_t workspace_pool() {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static hipMemPool_t pools[MAX_DEVICES];
+    static bool tried[MAX_DEVICES];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) { (void)hipGetLastError(); return nullptr; }
+    std::lock_guard<std::mutex> guard(mu);
+    if (!tried[dev]) {
+        tried[dev] = true;
+        hipMemPoolProps props{};
+        props.allocType = hipMemAllocationTypePinned;
+        props.handleTypes = hipMemHandleTypeNone;
+        props.location.type = hipMemLocationTypeDevice;
+        props.location.id = dev;
+        if (hipMemPoolCreate(&pools[dev], &props) != hipSuccess) {
+            (void)hipGetLastError();
+            pools[dev] = nullptr;
+        } else {
+            uint64_t keep = ~0ull;
+            (void)hipMemPoolSetAttribute(pools[dev], hipMemPoolAttrReleaseThreshold, &keep);
+        }
+    }
+    return pools[dev];
+}
+
+// which kernel family served the calling thread's last mul_mat_q8 call
+static thread_local int g_q8_path = 0;
+void set_q8_path(int path) { g_q8_path = path; }
 
 }  // namespace ppmlhip
 
@@ -76,17 +229,60 @@ extern "C" int ppml_hip_synchronize(void) {
     return RC_OK;
 }
 
+extern "C" int ppml_hip_mulmat_stats_enable(int on) {
+    const int before = stats_enabled() ? 1 : 0;
+    if (on == 0 || on == 1) g_stats_on.store(on, std::memory_order_relaxed);
+    return before;
+}
+
 extern "C" int ppml_hip_mulmat_stats(int64_t* rows, int cap) {
-    std::lock_guard<std::mutex> lock(g_stats_mtx);
+    Stats& s = stats();
+    std::lock_guard<std::mutex> lock(s.mu);
+    std::map<std::tuple<int64_t, int64_t, int64_t>, int64_t> shapes;      // summed over the paths
+    for (const auto& kv : s.table) shapes[std::make_tuple(kv.first.M, kv.first.K, kv.first.N)] += kv.second.calls;
     int i = 0;
-    for (const auto& kv : g_stats) {
+    for (const auto& kv : shapes) {
         if (rows && i < cap) {
-            rows[4 * i + 0] = static_cast<int64_t>(kv.first >> 40);
-            rows[4 * i + 1] = static_cast<int64_t>((kv.first >> 20) & 0xfffff);
-            rows[4 * i + 2] = static_cast<int64_t>(kv.first & 0xfffff);
+            rows[4 * i + 0] = std::get<0>(kv.first);
+            rows[4 * i + 1] = std::get<1>(kv.first);
+            rows[4 * i + 2] = std::get<2>(kv.first);
             rows[4 * i + 3] = kv.second;
         }
         ++i;
     }
     return i;
 }
+
+extern "C" int ppml_hip_mulmat_stats_rows(ppml_hip_mulmat_stat* rows, int cap) {
+    Stats& s = stats();
+    std::lock_guard<std::mutex> lock(s.mu);
+    fold_pending_locked(s, true);
+    int i = 0;
+    for (const auto& kv : s.table) {
+        if (rows && i < cap) {
+            std::snprintf(rows[i].path, sizeof rows[i].path, "%s", kv.first.path.c_str());
+            rows[i].M = kv.first.M; rows[i].K = kv.first.K; rows[i].N = kv.first.N;
+            rows[i].calls = kv.second.calls;
+            rows[i].ms = kv.second.ms;
+        }
+        ++i;
+    }
+    return i;
+}
+
+extern "C" void ppml_hip_mulmat_stats_dump(void) {
+    Stats& s = stats();
+    std::lock_guard<std::mutex> lock(s.mu);
+    fold_pending_locked(s, true);
+    dump_locked(s);
+}
+
+extern "C" void ppml_hip_mulmat_stats_reset(void) {
+    Stats& s = stats();
+    std::lock_guard<std::mutex> lock(s.mu);
+    fold_pending_locked(s, true);
+    s.table.clear();
+    s.started = false;
+}
+
+extern "C" int ppml_hip_q8_last_path(void) { return g_q8_path; }

@@ -47,6 +47,29 @@ def _ptr(t) -> C.c_void_p:
     return C.c_void_p(0 if t is None else t.data_ptr())
 
 
+Q8_PATH_NAMES = {0: "general", 1: "weight-stationary", 2: "low-latency"}
+
+
+def last_q8_path() -> str:
+    """Kernel family that served this thread's last mul_mat_q8 call (``ppml_hip_q8_last_path``)."""
+    return Q8_PATH_NAMES[_lib().ppml_hip_q8_last_path()]
+
+
+def mulmat_stats_enable(on: bool) -> bool:
+    """Switches the MUL_MAT statistics (include/ppml/MulMatStats.h) on or off; returns the previous state."""
+    return bool(cabi.load().ppml_hip_mulmat_stats_enable(1 if on else 0))
+
+
+def mulmat_stats_rows():
+    """The statistics table as a list of dicts {path, M, K, N, calls, ms}, ordered by (path, M, K, N)."""
+    lib = cabi.load()
+    n = lib.ppml_hip_mulmat_stats_rows(None, 0)
+    rows = (cabi.MulMatStat * max(n, 1))()
+    n = min(lib.ppml_hip_mulmat_stats_rows(C.cast(rows, C.c_void_p), n), n)
+    return [{"path": rows[i].path.decode(), "M": rows[i].M, "K": rows[i].K, "N": rows[i].N, "calls": rows[i].calls,
+             "ms": rows[i].ms} for i in range(n)]
+
+
 def synchronize() -> None:
     cabi.check("ppml_hip_synchronize", _lib().ppml_hip_synchronize())
 
@@ -272,6 +295,27 @@ def permute(x: torch.Tensor, axes) -> torch.Tensor:
     ax = axes + list(range(nd, 4))
     out = torch.empty(tuple(dd[:nd][::-1]), dtype=torch.float32, device=x.device)
     cabi.check("permute_hip", _lib().permute_hip(_ptr(x), _ptr(out), x.numel(), nd, *ax, *sd, *dd, _stream()))
+    return out
+
+
+def repeat_back(a: torch.Tensor, b_shape) -> torch.Tensor:
+    """The builder's ``repeat_back(a, b)`` (src/core/ComputeGraphHelper.cpp:114-133) with the kernel's index rule
+    (src/backend/CPUKernels.cpp:2091-2148): `a` summed over the copies that a broadcast of a tensor of shape
+    `b_shape` made.  Shapes are torch order (LAST dimension = the reference's dims[0]); dimension d of the
+    result meets dimension d of `a` counted from dims[0], missing dimensions count as 1."""
+    a = _dev_f32(a, "a")
+    b_shape = tuple(int(d) for d in b_shape)
+    if a.dim() < 1 or a.dim() > 4 or len(b_shape) < 1 or len(b_shape) > 4:
+        raise ValueError("repeat_back: tensors have 1 to 4 dimensions")
+    sd = list(a.shape[::-1]) + [1] * (4 - a.dim())
+    dd = list(b_shape[::-1]) + [1] * (4 - len(b_shape))
+    off = 0 if a.dim() >= len(b_shape) else a.dim() - len(b_shape)
+    rd = []
+    for d in range(4):
+        sdim = sd[d + off] if 0 <= d + off < 4 else 1
+        rd.append(sdim // dd[d] if dd[d] > 0 else 1)
+    out = torch.empty(b_shape, dtype=torch.float32, device=a.device)
+    cabi.check("repeat_back_hip", _lib().repeat_back_hip(_ptr(a), _ptr(out), *sd, *dd, *rd, _stream()))
     return out
 
 

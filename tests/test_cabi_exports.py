@@ -66,3 +66,21 @@ def test_host_side_argument_checks_need_no_gpu():
     assert lib.mul_mat_hip(None, one, one, 1, 1, 1, None, None) == 1
     dims = [4, 3, 1, 1, 5, 2, 1, 1, 4, 5, 1, 1]        # contraction lengths differ
     assert lib.out_prod_hip(one, one, one, *dims, None) == 1
+
+
+def test_mulmat_stats_switch_and_empty_table_need_no_gpu():
+    from proteinpredictmachinelearning_amd import cabi, ops
+
+    lib = cabi.load()
+    before = lib.ppml_hip_mulmat_stats_enable(1)
+    try:
+        assert lib.ppml_hip_mulmat_stats_enable(-1) == 1            # other values only query
+        lib.ppml_hip_mulmat_stats_reset()
+        assert ops.mulmat_stats_rows() == []
+        assert lib.ppml_hip_mulmat_stats(None, 0) == 0
+        # refused calls are not counted: the reference records after its own argument checks as well
+        assert lib.mul_mat_hip(None, None, None, 1, 1, 1, None, None) == 1
+        assert ops.mulmat_stats_rows() == []
+    finally:
+        lib.ppml_hip_mulmat_stats_enable(before)
+    assert ctypes.sizeof(cabi.MulMatStat) == 32 + 4 * 8 + 8

@@ -379,10 +379,23 @@ def test_failure_statuses(be):
     ghost = B.Tensor((4, 5))
     assert be.graph_compute([B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, ghost])]) == B.NOT_SUPPORTED
     assert "src1" in be.last_error
-    # a host pointer passed off as device memory (src/backend/CUDABackend.cpp:894-973)
+    # a host pointer under a scheduler (skip_alloc): the copies across backends are the scheduler's nodes, so
+    # the executor refuses it (src/backend/CUDABackend.cpp:824-830, 894-973)
     host = np.ones((5, 4), np.float32)
     fake = B.Tensor((4, 5)).bind(host.ctypes.data)
-    assert be.graph_compute([B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, fake])]) == B.NOT_SUPPORTED
+    import torch
+    out = torch.zeros(15, device="cuda")
+    be.set_skip_alloc(True)
+    try:
+        assert be.graph_compute([B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, fake]).bind(out.data_ptr())]) == B.NOT_SUPPORTED
+        assert "src1" in be.last_error
+        assert be.graph_compute([B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, b]).bind(out.data_ptr())]) == B.SUCCESS
+    finally:
+        be.set_skip_alloc(False)
+    assert (out.cpu().numpy() == 4.0).all()
+    # a host pointer as the OUTPUT is never covered
+    res = np.zeros((3, 5), np.float32)
+    assert be.graph_compute([B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, b]).bind(res.ctypes.data)]) == B.NOT_SUPPORTED
     # shapes that do not match the node
     assert be.graph_compute([B.Tensor((6, 3), B.F32, B.OP_MUL_MAT, [a, b])]) == B.NOT_SUPPORTED
     # with a scheduler in charge of allocation the executor allocates nothing
@@ -395,3 +408,106 @@ def test_failure_statuses(be):
     node = B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, b])
     assert be.graph_compute([node]) == B.SUCCESS
     assert (be.download(node) == 4.0).all()
+
+
+def test_host_resident_leaves_get_device_shadows(be, oracle):
+    # single-backend mode: sources bound to host memory (leaves nobody uploaded) are copied to the device for
+    # the length of graph_compute and the tensors' own fields are put back afterwards
+    # (src/backend/CUDABackend.cpp:521-577, 824-830)
+    M, K, N = 29, 40, 21
+    rng = np.random.default_rng(21)
+    A = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    Wm = rng.integers(-4, 5, size=(N, K)).astype(np.float32)
+    bias = rng.integers(-4, 5, size=N).astype(np.float32)
+    a = B.Tensor((K, M)).bind(A.ctypes.data)                      # host
+    w = _leaf(be, Wm)                                             # device
+    c = B.Tensor((N,)).bind(bias.ctypes.data)                     # host
+    node = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [a, w, c])
+    # a second node reads the same host leaf, and a view of it: one shadow per tensor, views follow their root
+    half = B.Tensor((K, M // 2), B.F32, B.OP_VIEW).view_of(a, 0)
+    node2 = B.Tensor((N, M // 2), B.F32, B.OP_MUL_MAT, [half, w])
+    assert be.graph_compute([node, half, node2]) == B.SUCCESS, be.last_error
+    assert be.host_shadows_made == 2                              # a and bias; the view borrowed a's copy
+    assert (be.download(node).reshape(M, N) == oracle.mul_mat_f32(A, Wm, bias)).all()
+    assert (be.download(node2).reshape(M // 2, N) == oracle.mul_mat_f32(A[:M // 2], Wm)).all()
+    # the host tensors are host tensors again (and the view unbound again): a second run uploads the (changed)
+    # contents anew, whichever of the two comes first
+    A[:] = A[::-1].copy()
+    node4 = B.Tensor((N, M // 2), B.F32, B.OP_MUL_MAT, [half, w])
+    assert be.graph_compute([half, node4]) == B.SUCCESS, be.last_error
+    assert (be.download(node4).reshape(M // 2, N) == oracle.mul_mat_f32(A[:M // 2], Wm)).all()
+    node3 = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [a, w])
+    assert be.graph_compute([node3]) == B.SUCCESS, be.last_error
+    assert be.host_shadows_made == 1
+    assert (be.download(node3).reshape(M, N) == oracle.mul_mat_f32(A, Wm)).all()
+    # a quantized host weight is sized by its blocks
+    wq = oracle.quantize_q8_0((rng.standard_normal((N, 64)) * 0.02).astype(np.float32))
+    raw = np.frombuffer(wq.tobytes(), np.uint8).copy()
+    x = rng.standard_normal((M, 64)).astype(np.float32)
+    wt = B.Tensor((64, N), B.Q8_0).bind(raw.ctypes.data)
+    qn = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [_leaf(be, x), wt])
+    assert be.graph_compute([qn]) == B.SUCCESS, be.last_error
+    assert (be.download(qn).reshape(M, N) == oracle.mul_mat_q8(wq, x, wtype=0, c_trans=1, fma=1)).all()
+
+
+@pytest.mark.parametrize("src_dims,dst_dims", [((19, 37), (19,)), ((5, 3, 4, 2), (5, 1, 4, 1)), ((6, 4), (3, 4)),
+                                               ((768, 2000), (768,)), ((8, 51, 6), (8, 1, 6))])
+def test_repeat_back_node(be, oracle, src_dims, dst_dims):
+    # OP_REPEAT_BACK, the bias gradient of a mul_mat (src/core/ComputeGraph.cpp:742): dims innermost first
+    rng = np.random.default_rng(len(src_dims) * 100 + src_dims[0])
+    g = rng.integers(-6, 7, size=src_dims[::-1]).astype(np.float32)
+    node = B.Tensor(dst_dims, B.F32, B.OP_REPEAT_BACK, [_leaf(be, g)])
+    assert be.supports_op(node)
+    got = be_run(be, node).reshape(dst_dims[::-1])
+    assert (got == oracle.repeat_back(g, dst_dims[::-1])).all()      # small integers: exact in any order
+
+
+def test_backward_of_a_biased_linear_stays_on_the_device(be, oracle):
+    """ComputeGraph.cpp:708-742 for y = mul_mat(A, W, bias): dA, dW as above and dbias = repeat_back(grad, bias);
+    six nodes, none of which leaves this backend."""
+    rng = np.random.default_rng(16)
+    M, K, N = 45, 32, 27
+    A = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    W = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+    G = rng.integers(-3, 4, size=(M, N)).astype(np.float32)
+    a, w, g = _leaf(be, A), _leaf(be, W), _leaf(be, G)
+
+    def mat_t(t, dims):
+        n = B.Tensor(dims, B.F32, B.OP_PERMUTE, [t])
+        n.set_param(0, 1).set_param(1, 0)
+        return n
+    wt, gt, at = mat_t(w, (N, K)), mat_t(g, (M, N)), mat_t(a, (M, K))
+    dA = B.Tensor((K, M), B.F32, B.OP_MUL_MAT, [g, wt])
+    dW = B.Tensor((K, N), B.F32, B.OP_MUL_MAT, [gt, at])
+    db = B.Tensor((N,), B.F32, B.OP_REPEAT_BACK, [g])
+    nodes = [wt, dA, gt, at, dW, db]
+    assert all(be.supports_op(n) for n in nodes)
+    assert be.graph_compute(nodes) == B.SUCCESS, be.last_error
+    assert np.array_equal(be.download(dA).reshape(M, K), G @ W)
+    assert np.array_equal(be.download(dW).reshape(N, K), G.T @ A)
+    assert np.array_equal(be.download(db), G.sum(axis=0))
+    assert np.array_equal(be.download(db), oracle.repeat_back(G, (N,)))
+
+
+def test_f32_arithmetic_is_a_field_of_the_backend(be, oracle):
+    # two backends with different pipes do not disturb each other or the calling thread's own setting
+    from proteinpredictmachinelearning_amd import ops
+    M, K, N = 70, 40, 50
+    rng = np.random.default_rng(3)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    Wm = rng.standard_normal((N, K)).astype(np.float32)
+    A[3, 5] = np.inf                                              # tells the pipes apart: NaN (split) or inf (fp32)
+    want = oracle.mul_mat_f32(A, Wm)
+    other = B.Backend(0)
+    other.set_f32_arithmetic("fp32")
+    assert ops.set_f32_arithmetic("split") in ("split", "fp32")
+    try:
+        for _ in range(2):
+            n1 = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [_leaf(be, A), _leaf(be, Wm)])
+            n2 = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [_leaf(other, A), _leaf(other, Wm)])
+            assert be.graph_compute([n1]) == B.SUCCESS and other.graph_compute([n2]) == B.SUCCESS
+            assert np.isnan(be.download(n1).reshape(M, N)[3]).all()
+            assert (other.download(n2).reshape(M, N)[3] == want[3]).all()
+        assert ops.set_f32_arithmetic("split") == "split"        # the thread's setting came back after each call
+    finally:
+        other.set_f32_arithmetic(None)

@@ -159,6 +159,90 @@ def test_attention_logits_shapes(ops, oracle, planes, L, D):
     _check(got.reshape(planes, 1, L, L), scores)
 
 
+def test_attention_logits_msa_row_attention_full_size(ops, oracle):
+    # The configured MSA form: 824 planes (8 heads x 103 residues) of 256 x 256 logits over a head dimension of
+    # 32.  The 216 MB result is past the size where the launcher switches to the streaming-store instances, so
+    # this is the one test that runs them.  (a) sampled planes against the oracle; (b) planes are independent:
+    # a 64-plane slice launched alone (17 MB, the ordinary-store instance) must give the same bits as the same
+    # planes of the full launch; (c) every plane of the full result is covered by a checksum against a second
+    # full launch on the same inputs and by the slice-wise comparison of (b) walked over all planes.
+    planes, L, D = 824, 256, 32
+    g = torch.Generator(device="cuda").manual_seed(824)
+    k = torch.randn(1, planes, D, L, device="cuda", generator=g)
+    q = torch.randn(1, planes, D, L, device="cuda", generator=g)
+    full = ops.attention_logits(k, q)
+    assert full.shape == (1, planes, L, L)
+    sel = [0, 1, 63, 64, 411, 412, 700, 822, 823]
+    kh, qh = k[:, sel].cpu().numpy(), q[:, sel].cpu().numpy()
+    want = oracle.out_prod(kh, qh) * np.float32(1.0 / math.sqrt(D))
+    absprod = np.einsum("pqki,pqkj->pqji", np.abs(kh).astype(np.float64), np.abs(qh).astype(np.float64)) / math.sqrt(D)
+    _check(full[:, sel].cpu().numpy(), want, absprod)
+    for p0 in range(0, planes, 64):
+        p1 = min(p0 + 64, planes)
+        part = ops.attention_logits(k[:, p0:p1].contiguous(), q[:, p0:p1].contiguous())
+        assert torch.equal(part, full[:, p0:p1]), f"planes {p0}..{p1} differ between the two store forms"
+    again = ops.attention_logits(k, q)
+    assert torch.equal(again, full)
+
+
+# ----------------------------------------------------------------------------- non-finite and subnormal operands
+def test_infinite_operand_gives_nan_on_the_split_pipe_and_inf_on_the_fp32_pipe(ops, oracle):
+    # The reference's loop (src/backend/CPUKernels.cpp:763-771) carries an infinite operand through: inf * b
+    # summed with finite terms is +-inf.  The default arithmetic here splits every operand into three bf16
+    # parts by subtraction, and inf - inf is NaN: an output whose sum touches an infinite operand is NaN
+    # instead of +-inf.  Outputs that do not touch it are unaffected, NaN operands give NaN either way, and
+    # the fp32 pipe (ppml_hip_set_f32_arithmetic(1)) gives the reference's +-inf.  This test pins all four.
+    M, K, N = 70, 40, 50
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    b = rng.standard_normal((N, K)).astype(np.float32)
+    b[b == 0] = 1.0
+    a[3, 5] = np.inf
+    a[9, 0] = -np.inf
+    a[20, 7] = np.nan
+    want = oracle.mul_mat_f32(a, b)
+    assert np.isinf(want[3]).all() and np.isinf(want[9]).all() and np.isnan(want[20]).all()
+    got = ops.mul_mat(_dev(a), _dev(b)).cpu().numpy()
+    clean = np.ones(M, bool)
+    clean[[3, 9, 20]] = False
+    _check(got[clean], want[clean])
+    assert np.isnan(got[[3, 9, 20]]).all()                  # the documented difference: NaN where the reference has +-inf
+    before = ops.set_f32_arithmetic("fp32")
+    try:
+        got32 = ops.mul_mat(_dev(a), _dev(b)).cpu().numpy()
+    finally:
+        ops.set_f32_arithmetic(before)
+    _check(got32[clean], want[clean])
+    assert (got32[[3, 9]] == want[[3, 9]]).all() and np.isnan(got32[20]).all()
+
+
+def test_subnormal_operands(ops, oracle):
+    # operands below 2^-126 against large ones: the products are ordinary numbers, so flushing the small
+    # operand to zero would lose the whole result
+    M, K, N = 64, 48, 40
+    rng = np.random.default_rng(5)
+    a = (rng.standard_normal((M, K)) * 2.0 ** -130).astype(np.float32)          # all subnormal
+    assert (np.abs(a) < 2.0 ** -126).all() and (a != 0).mean() > 0.9
+    b = (rng.standard_normal((N, K)) * 2.0 ** 100).astype(np.float32)
+    want = oracle.mul_mat_f32(a, b)
+    assert np.abs(want).max() > 2.0 ** -32
+    absprod = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64).T
+    for mode in ("split", "fp32"):
+        before = ops.set_f32_arithmetic(mode)
+        try:
+            got = ops.mul_mat(_dev(a), _dev(b)).cpu().numpy()
+        finally:
+            ops.set_f32_arithmetic(before)
+        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        assert (err <= 1e-4 * absprod + 1e-45).all(), f"{mode}: elementwise {np.max(err / (absprod + 1e-300)):.3e}"
+    # a subnormal RESULT: products of ordinary numbers that underflow
+    a2 = (rng.standard_normal((M, K)) * 2.0 ** -70).astype(np.float32)
+    b2 = (rng.standard_normal((N, K)) * 2.0 ** -70).astype(np.float32)
+    want2 = oracle.mul_mat_f32(a2, b2)
+    got2 = ops.mul_mat(_dev(a2), _dev(b2)).cpu().numpy()
+    assert np.abs(got2.astype(np.float64) - want2.astype(np.float64)).max() <= 2.0 ** -149 * (K + 2)
+
+
 # ----------------------------------------------------------------------------- outer product mean
 @pytest.mark.parametrize("D,L,N,B", [(3, 4, 8, 2), (16, 51, 8, 1), (5, 40, 33, 3), (32, 24, 256, 1)])
 def test_outer_prod_mean_graph_form(ops, oracle, D, L, N, B):

@@ -111,12 +111,35 @@ SHAPES = [
 
 SHAPES += [
     # shapes with a weight-stationary instance when the weight is packed (K/32 in {4,8,16})
+    (300, 128, 100),      # four-wave work-groups, four blocks
     (300, 128, 512),      # pair feed-forward up-projection, ragged last token tile
     (200, 512, 128),      # pair feed-forward down-projection
     (1000, 256, 768),     # MSA QKV projection: more token tiles than one pass of work-groups on a small grid
     (77, 256, 700),       # output features not a multiple of 32 (and not of 4 at the edge tile)
     (9000, 128, 100),     # more token tiles than CUs: the persistent loop and its double buffer
 ]
+
+# one shape per remaining weight-stationary instance (column tiles per wave, K/32, waves per work-group), each
+# with a ragged last token tile; WS_INSTANCE_SHAPES below lists every instance with a shape that reaches it
+SHAPES += [
+    (200, 128, 200),      # (1, 4) eight waves: 7 column tiles
+    (150, 128, 700),      # (3, 4): 22 column tiles
+    (300, 256, 400),      # (2, 8): 13 column tiles
+    (300, 512, 200),      # (1, 16) eight waves: 7 column tiles
+    (300, 256, 100),      # (1, 8) four waves: 4 column tiles
+    (9000, 256, 400),     # (2, 8) with several token tiles per work-group (staged loads, three LDS buffers in turn)
+    (9000, 512, 200),     # (1, 16) likewise: the 64-register staging range
+    (17000, 128, 700),    # (3, 4) likewise, with leftover tiles shared between work-groups
+]
+
+# (column tiles of 32 outputs) -> instance: up to 4 tiles the four-wave kernels, beyond that ceil(tiles / 8) per wave
+WS_INSTANCE_SHAPES = {
+    # (TPW, NBLK, waves): (N, K, M)
+    (1, 4, 4): (300, 128, 100), (1, 8, 4): (300, 256, 100), (1, 16, 4): (200, 512, 128),
+    (1, 4, 8): (200, 128, 200), (2, 4, 8): (300, 128, 512), (3, 4, 8): (150, 128, 700), (4, 4, 8): (70, 128, 800),
+    (1, 8, 8): (408, 256, 256), (2, 8, 8): (300, 256, 400), (3, 8, 8): (1000, 256, 768),
+    (1, 16, 8): (300, 512, 200),
+}
 
 
 @pytest.mark.parametrize("packed", [False, True])
@@ -138,6 +161,30 @@ def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packe
     # the undumped fast path gives the same bits
     fast = ops.mul_mat_q8(W, _dev(x), c_trans=1).cpu().numpy()
     assert (fast == out).all()
+    # packed weights of K / 32 in {4, 8, 16} and at most 256 Ki elements are served by the resident-weight kernels
+    if packed and _has_resident_weight_instance(K, M):
+        assert ops.last_q8_path() != "general"
+    elif not packed:
+        assert ops.last_q8_path() == "general"
+
+
+def _has_resident_weight_instance(K, M):
+    tiles, nblk = (M + 31) // 32, K // 32
+    tpw = (tiles + 7) // 8
+    return K % 32 == 0 and nblk in (4, 8, 16) and (tiles <= 4 or tpw <= {4: 4, 8: 3, 16: 1}[nblk])
+
+
+def test_every_weight_stationary_instance_has_a_shape_in_the_suite():
+    # the dispatch rule restated: up to four column tiles -> four-wave work-groups, one tile per wave; beyond
+    # that eight waves with ceil(tiles / 8) tiles each.  Every instance the library builds is listed, and each
+    # listed shape is one of SHAPES, so the parametrized test above runs it (dump and fast form).
+    for (tpw, nblk, waves), (N, K, M) in WS_INSTANCE_SHAPES.items():
+        tiles = (M + 31) // 32
+        assert K // 32 == nblk
+        assert (waves == 4) == (tiles <= 4)
+        assert tpw == (1 if waves == 4 else (tiles + 7) // 8)
+        assert (N, K, M) in SHAPES, (N, K, M)
+    assert len(WS_INSTANCE_SHAPES) == 11
 
 
 @pytest.mark.parametrize("N,K,M", [(408, 256, 256), (100, 96, 100), (70, 128, 800)])
@@ -282,4 +329,6 @@ def test_fused_linear_with_q8_1_activations(ops, oracle, wname, N, K, M, c_trans
     # without the dump, and the two rules really differ
     y2 = ops.mul_mat_q8(W, _dev(x), c_trans=c_trans, act="q8_1").cpu().numpy()
     assert (y2 == want).all()
+    # a packed weight in the LinearLayer orientation gets the resident-weight kernels under this rule too
+    assert (ops.last_q8_path() != "general") == (wname == "packed" and c_trans == 1)
     assert (ops.mul_mat_q8(W, _dev(x), c_trans=c_trans).cpu().numpy() != want).any()

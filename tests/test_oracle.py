@@ -721,3 +721,40 @@ def test_flash_attn_backward_against_finite_differences(oracle):
             assert (np.triu(db[0, 0], 1) == 0).all()
     # nothing to compute is refused
     assert oracle.lib().orc_flash_attn_backward(1, 1, 2, 4, 0, 0.0, *([q.ctypes.data_as(__import__("ctypes").POINTER(__import__("ctypes").c_float))] * 7), None, None, None, None) == 1
+
+
+# ----------------------------------------------------------------------------- repeat_back
+def test_repeat_back_bias_gradient_and_broadcast_axes(oracle):
+    # the gradient of a mul_mat bias: grad [N, M] (dims[0] = N) -> dbias [N] = sum over the M rows
+    # (src/core/ComputeGraph.cpp:742); numpy shapes are outermost first
+    rng = np.random.default_rng(31)
+    g = rng.integers(-8, 9, size=(23, 17)).astype(np.float32)          # M = 23 rows of N = 17
+    assert (oracle.repeat_back(g, (17,)) == g.sum(axis=0)).all()
+    # a wrong (right-aligned) pairing of the dimensions would sum 17 // 23 = 0 copies or read one element
+    assert not (oracle.repeat_back(g, (17,)) == g[0]).all()
+    # same rank, broadcast over dims[1] and dims[3]: [5,1,4,1] from [5,3,4,2]
+    x = rng.integers(-5, 6, size=(2, 4, 3, 5)).astype(np.float32)
+    assert (oracle.repeat_back(x, (1, 4, 1, 5)) == x.sum(axis=(0, 2), keepdims=True)).all()
+    # a dimension that is kept and repeated at once: dst dims[0] = 3 from src dims[0] = 6, copies j0 and j0 + 3
+    y = rng.integers(-5, 6, size=(4, 6)).astype(np.float32)
+    want = y[:, :3] + y[:, 3:]
+    assert (oracle.repeat_back(y, (4, 3)) == want).all()
+    # no repetition at all is a copy
+    assert (oracle.repeat_back(y, (4, 6)) == y).all()
+
+
+def test_repeat_back_adds_its_terms_one_at_a_time(oracle):
+    # 2^24 + 1 + 1: adding from the left rounds each 1 away (2^24); pairing the ones first gives 2^24 + 2
+    col = np.array([[2.0 ** 24], [1.0], [1.0]], dtype=np.float32)       # three rows of one element
+    assert oracle.repeat_back(col, (1,))[0] == np.float32(2.0 ** 24)
+    col2 = np.array([[1.0], [1.0], [2.0 ** 24]], dtype=np.float32)
+    assert oracle.repeat_back(col2, (1,))[0] == np.float32(2.0 ** 24 + 2)
+    # with two repeated dimensions the innermost loop is the OUTER dimension (k3 fastest, k0 slowest):
+    # src dims [2, 2] -> dst [1, 1]; order of the four terms is (k0,k1) = (0,0), (0,1), (1,0), (1,1)
+    m = np.array([[2.0 ** 24, 1.0], [1.0, 1.0]], dtype=np.float32)      # m[i1][i0]
+    # (0,0) = 2^24, (0,1) = m[1][0] = 1 -> lost, (1,0) = m[0][1] = 1 -> lost, (1,1) = 1 -> lost
+    assert oracle.repeat_back(m, (1, 1))[0, 0] == np.float32(2.0 ** 24)
+    m2 = np.array([[1.0, 2.0 ** 24], [1.0, 1.0]], dtype=np.float32)
+    # 1 + 1 = 2, + 2^24 = 2^24 + 2, + 1 -> tie, rounds to even: 2^24 + 4?  (2^24 + 3 lies between 2^24+2 and 2^24+4)
+    got = oracle.repeat_back(m2, (1, 1))[0, 0]
+    assert got == np.float32(np.float32(np.float32(1.0 + 1.0) + np.float32(2.0 ** 24)) + np.float32(1.0))
