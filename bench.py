@@ -17,6 +17,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -26,9 +27,21 @@ INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA, published
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 
-# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE
-# scaled by the same counters on a 1 GiB copy: factors 2.000 and 1.000).
-MEASURED_TRAFFIC_BYTES = 113_570_000   # 28.89 MB read + 81.00 MB written per launch
+PREHEAT_MS = 3.0             # untimed load ahead of every event-timed region: the shader clock needs 1-2 ms to settle
+TRAFFIC_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "q8_linear_msa_qkv_hbm_traffic.md")
+
+
+def measured_traffic_bytes():
+    """HBM bytes per launch of the dominant kernel as the committed rocprofv3 --pmc summary states them
+    (FETCH_SIZE + WRITE_SIZE, each scaled by the same counter's reading for a 1 GiB copy): the line
+    ``traffic_bytes_per_launch: <integer>`` of profiles/q8_linear_msa_qkv_hbm_traffic.md.  None when the
+    summary is not there."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", f.read(), flags=re.M)
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def q8_bytes(rows, K, N):
@@ -65,18 +78,28 @@ def main() -> int:
     gen = torch.Generator(device=dev).manual_seed(1)
 
     def time_op(fn, nsets, steps, warmup):
-        """Returns (wall seconds per step, event seconds per step)."""
+        """Two clocks, both reported.  Wall: `warmup` untimed steps, then exactly `steps` steps between two
+        device synchronisations (the whole-job figure; after a synchronisation the GPU starts from idle clocks,
+        so short runs read slower here).  Events: the same `steps` steps again between two HIP events on the
+        launch stream, queued directly behind PREHEAT_MS of untimed launches of the same step, so the region
+        runs at the steady clock whatever `steps` is.  Returns (wall s / step, event s / step)."""
         for i in range(warmup):
             fn(i % nsets)
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        for i in range(steps):
+            fn(i % nsets)
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) / steps
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        heat = max(warmup, min(20000, int(PREHEAT_MS * 1e-3 / max(wall, 1e-7)) + 1))
+        for i in range(heat):
+            fn(i % nsets)
         e0.record()
         for i in range(steps):
             fn(i % nsets)
         e1.record()
         torch.cuda.synchronize()
-        wall = (time.perf_counter() - t0) / steps
         return wall, e0.elapsed_time(e1) * 1e-3 / steps
 
     def q8_case(rows, K, N, relu=False):
@@ -122,10 +145,12 @@ def main() -> int:
         "config": {"workload": "MSA-track QKV Q8_0 linear: X 26368x256 f32 -> Q8_0 on the fly, "
                                "W 768x256 Q8_0, Y 26368x768 f32",
                    "buffer_rotation": nsets, "weight_layout": "Q8_0M (MFMA fragments)"},
+        "preheat_ms": PREHEAT_MS,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic_bytes(),
                      "kernel": "q8_linear_ws_kernel", "algorithmic_bytes_per_launch": nbytes,
-                     "kernel_us": round(ev * 1e6, 2),
+                     "kernel_us": round(ev * 1e6, 2), "clock": "HIP events on the launch stream, region queued behind preheat_ms of load",
+                     "wall_us": round(wall * 1e6, 2), "frac_wall_clock": round(nbytes / wall / 1e9 / HBM_PEAK_GBS, 4),
                      "int8_mfma_frac": round(nops / ev / 1e12 / INT8_PEAK_TOPS, 4)},
     }
 
@@ -137,16 +162,25 @@ def main() -> int:
         threads = min(len(os.sched_getaffinity(0)), 16)
         xq_rows = x0.cpu().numpy()
         wq = oracle.quantize_q8_0(w0.cpu().numpy())
-        reps, t_cpu = 0, 0.0
-        while t_cpu < 10.0 and reps < 50:
-            t0 = time.perf_counter()
-            oracle.mul_mat_q8(wq, xq_rows, wtype=0, c_trans=1, fma=1, nthreads=threads)
-            t_cpu += time.perf_counter() - t0
-            reps += 1
+
+        def cpu_leg(nthreads, budget_s):
+            reps, t_cpu = 0, 0.0
+            while t_cpu < budget_s and reps < 50:
+                t0 = time.perf_counter()
+                oracle.mul_mat_q8(wq, xq_rows, wtype=0, c_trans=1, fma=1, nthreads=nthreads)
+                t_cpu += time.perf_counter() - t0
+                reps += 1
+            return reps, t_cpu
+        reps, t_cpu = cpu_leg(threads, 10.0)
+        # the reference's own default is PPML_N_THREADS = 4 (src/model/PPML.cpp:3828-3833)
+        reps4, t_cpu4 = cpu_leg(min(4, threads), 8.0)
         out["cpu_baseline"] = {"value": round(nops * reps / t_cpu / 1e12, 5), "unit": "TOPS", "cores": threads,
                                "kind": "port",
                                "sample": f"{reps} full passes of the same 26368x256->768 workload "
-                                         f"(quantize rows + block dot), {t_cpu:.1f} s of CPU time"}
+                                         f"(quantize rows + block dot), {t_cpu:.1f} s of CPU time",
+                               "reference_default_threads": {"value": round(nops * reps4 / t_cpu4 / 1e12, 5), "unit": "TOPS",
+                                                             "cores": min(4, threads),
+                                                             "sample": f"{reps4} full passes, {t_cpu4:.1f} s of CPU time"}}
         del np
 
     # ------------------------------------------------------------------ the other configured shapes

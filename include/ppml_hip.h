@@ -62,7 +62,11 @@ int ppml_hip_set_f32_arithmetic(int mode);
  * C[m*N+n] = (bias ? bias[n] : 0) + sum_k A[m*K+k] * B[n*K+k].  bias may be NULL.
  * Arithmetic of this and the other f32 contractions below: each binary32 operand is the exact sum of
  * three bf16 numbers; six of the nine partial products (all but 2^-23 of |a||b|) are formed exactly on
- * the bf16 matrix pipe and summed in binary32.  An infinite operand yields NaN.  Contractions of at
+ * the bf16 matrix pipe and summed in binary32.  Two kinds of operand fall outside that: an infinite operand
+ * yields NaN where the reference's loop yields +-inf, and a subnormal operand (below 2^-126) is cut to a
+ * multiple of 2^-133, bf16's smallest step (the reference keeps its bits down to 2^-149).  Callers that must
+ * have the reference's results on such operands select the fp32 pipe (ppml_hip_set_f32_arithmetic(1)), which
+ * carries both through.  Contractions of at
  * least 512 work-groups of 256 x 128 outputs take a workspace of 6 bytes per operand element from a
  * stream-ordered pool (allocated and freed on `stream`); no other launcher allocates. */
 int mul_mat_hip(const float *A, const float *B, float *C, int M, int K, int N,
