@@ -161,6 +161,20 @@ int outer_product_mean_value_hip(const float *left, const float *right, float *d
 int mul_mat_tn_hip(const float *A, const float *Bm, float *O, int M, int K, int Nc, float alpha,
                    ppml_hip_stream_t stream);
 
+/* mul_mat_tn_hip for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc): the same contraction with the same kernels and the same bits, but the workspace the
+ * large cases need (the bf16 planes of both operands, 6 bytes per padded operand element, plus the partial sums
+ * of K slices) is a static 64 MiB device array of the library instead of a pool allocation.  It has no
+ * counterpart in the reference.  The call allocates and frees nothing and records no statistics.  A contraction
+ * whose workspace exceeds 64 MiB is refused with status 1 and a message that names both sizes (for two square
+ * operands without K slices that is (M_pad + N_pad) * K_pad * 6 bytes, M padded to 256, N to 128, K to 16:
+ * e.g. 12288 x 256 x 12288 takes 36 MiB); contractions that need no workspace run whatever their size.  The
+ * array's address on a device is looked up by ppml_hip_init(device) -- or by the first call on a device that
+ * was never initialised, so call ppml_hip_init first where even that lookup is unwelcome.  All calls on one GPU
+ * share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race; order them. */
+int mul_mat_tn_noalloc_hip(const float *A, const float *Bm, float *O, int M, int K, int Nc, float alpha,
+                           ppml_hip_stream_t stream);
+
 /* replaces tri_mul_cuda (src/cuda/PairKernels.cu:514-523, declared src/backend/CUDAKernels.cpp:316-318),
  * indexing and finite guard of CPUBackend::kernel_tri_mul (src/backend/CPUKernels.cpp:907-968):
  *   outgoing: dst[((d*I+i)*J+j)*B+b] = inv_L * sum_k left[((d*I+i)*K+k)*B+b] * right[((d*J+j)*K+k)*B+b]

@@ -36,6 +36,7 @@ SIGNATURES = {
     "outer_prod_mean_back_hip": (_i, [_vp] * 5 + [_i64] * 4 + [_f, _vp]),
     "outer_product_mean_value_hip": (_i, [_vp, _vp, _vp] + [_i64] * 4 + [_vp]),
     "mul_mat_tn_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _f, _vp]),
+    "mul_mat_tn_noalloc_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _f, _vp]),
     "tri_mul_hip": (_i, [_vp, _vp, _vp] + [_i64] * 5 + [_f, _i, _vp]),
     "tri_mul_back_hip": (_i, [_vp] * 5 + [_i64] * 5 + [_f, _i, _vp]),
     "flash_attn_forward_hip": (_i, [_i] * 5 + [_f, _f, _i] + [_vp] * 7),

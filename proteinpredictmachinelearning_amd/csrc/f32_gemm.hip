@@ -698,7 +698,10 @@ int f32_arithmetic() {
     return t_f32_arithmetic;
 }
 
-int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
+// `fixed_ws` / `fixed_cap`: a workspace the caller brings (the static array of the entry point that allocates
+// nothing).  With one, the pool is never touched: a contraction that wants more workspace than `fixed_cap`
+// is refused, one that wants none runs as it always does.
+int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fixed_ws = nullptr, size_t fixed_cap = 0) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
     // An output that fits the 256 MB last-level cache is likely read next by the consumer node (the
@@ -737,10 +740,19 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
         const size_t a_bytes = static_cast<size_t>(3) * chunks * ma_pad * 32, b_bytes = static_cast<size_t>(3) * chunks * nb_pad * 32;
         const size_t part_bytes = slices > 1 ? static_cast<size_t>(slices) * ma_pad * nb_pad * 4 : 0;
         uint8_t* ws = nullptr;
-        hipMemPool_t pool = workspace_pool();
-        if (pool && hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), a_bytes + b_bytes + part_bytes, pool, stream) != hipSuccess) {
-            (void)hipGetLastError();
-            ws = nullptr;
+        if (fixed_ws) {
+            if (a_bytes + b_bytes + part_bytes > fixed_cap) {
+                set_error("%s: this contraction needs %zu bytes of workspace, the static one holds %zu", what,
+                          a_bytes + b_bytes + part_bytes, fixed_cap);
+                return RC_BAD_ARGS;
+            }
+            ws = fixed_ws;
+        } else {
+            hipMemPool_t pool = workspace_pool();
+            if (pool && hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), a_bytes + b_bytes + part_bytes, pool, stream) != hipSuccess) {
+                (void)hipGetLastError();
+                ws = nullptr;
+            }
         }
         if (ws) {
             GemmParams q = p;
@@ -767,7 +779,7 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what) {
                 else       hipLaunchKernelGGL((reduce_slices_kernel<false>), rgrid, block, 0, stream, p, partial, slices, ma_pad, nb_pad);
                 rc = check_launch(what);
             }
-            if (hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();
+            if (!fixed_ws && hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();
             return rc;
         }
     }
@@ -869,6 +881,65 @@ extern "C" int mul_mat_tn_hip(const float* A, const float* Bm, float* O, int M, 
     p.c_mi = Nc; p.c_ni = 1;
     p.alpha = alpha;
     return launch_gemm(p, static_cast<hipStream_t>(stream), "mul_mat_tn_hip");
+}
+
+// ---- the entry point that allocates nothing -------------------------------------------------------------
+// Workspace of mul_mat_tn_noalloc_hip: the split planes (and K-slice partial sums) that mul_mat_tn_hip takes
+// from the stream-ordered pool live here instead, for callers that may not allocate (HIP graph capture, tight
+// serving loops).  Every device the library runs on holds its own copy until the process ends.  The name below
+// is a host-side stand-in for the symbol, not a device address: host code uses the per-device pointer that
+// hipGetSymbolAddress returned, never the name.
+constexpr size_t NOALLOC_SCRATCH_BYTES = static_cast<size_t>(64) << 20;
+static __device__ __align__(256) uint8_t scratch[NOALLOC_SCRATCH_BYTES];
+
+namespace ppmlhip {
+namespace {
+constexpr int NOALLOC_MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+uint8_t* g_scratch_ptr[NOALLOC_MAX_DEVICES];          // per device: each GPU has the array at its own address
+}  // namespace
+
+// Looks the array's address up on the current device (once per device); called by ppml_hip_init with the
+// device it has just selected, and by the entry point for a device nobody initialised.
+int noalloc_scratch_setup(uint8_t** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= NOALLOC_MAX_DEVICES) {
+        (void)hipGetLastError();
+        set_error("mul_mat_tn_noalloc_hip: no current device below %d", NOALLOC_MAX_DEVICES);
+        return RC_NO_DEVICE;
+    }
+    std::lock_guard<std::mutex> guard(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            set_error("mul_mat_tn_noalloc_hip: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return RC_NO_DEVICE;
+        }
+        g_scratch_ptr[dev] = static_cast<uint8_t*>(ptr);
+    }
+    if (out) *out = g_scratch_ptr[dev];
+    return RC_OK;
+}
+}  // namespace ppmlhip
+
+extern "C" int mul_mat_tn_noalloc_hip(const float* A, const float* Bm, float* O, int M, int K, int Nc, float alpha,
+                                      ppml_hip_stream_t stream) {
+    if (!A || !Bm || !O || M <= 0 || K <= 0 || Nc <= 0) { set_error("mul_mat_tn_noalloc_hip: bad arguments"); return RC_BAD_ARGS; }
+    uint8_t* ws = nullptr;
+    const int rc = noalloc_scratch_setup(&ws);
+    if (rc != RC_OK) return rc;
+    GemmParams p = plain_params();
+    p.A = A; p.B = Bm; p.C = O;
+    p.M = M; p.N = Nc; p.K = K;
+    p.a_rs = 1; p.a_ks = M; p.b_rs = 1; p.b_ks = Nc;
+    p.c_mi = Nc; p.c_ni = 1;
+    p.alpha = alpha;
+    // No statistics scope here: its events would be created on the way.  Nothing in the workspace has to start
+    // at zero: the split kernels write every byte of the planes they hand on (padding rows and k included) and
+    // every K slice writes its whole padded block of partial sums before they are added.
+    return launch_gemm(p, static_cast<hipStream_t>(stream), "mul_mat_tn_noalloc_hip", ws, NOALLOC_SCRATCH_BYTES);
 }
 
 extern "C" int out_prod_scaled_hip(const float* src0, const float* src1, float* dst,

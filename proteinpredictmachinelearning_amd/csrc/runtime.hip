@@ -220,7 +220,8 @@ extern "C" int ppml_hip_init(int device) {
         set_error("ppml_hip_init: device %d is %s, this library holds gfx950 code only", device, prop.gcnArchName);
         return RC_NO_DEVICE;
     }
-    return RC_OK;
+    // set-up of the entry point that allocates nothing: the address of its static workspace on this device
+    return noalloc_scratch_setup(nullptr);
 }
 
 extern "C" int ppml_hip_synchronize(void) {
