@@ -8,6 +8,7 @@
 #include "common.hpp"
 #include <type_traits>
 #include <cstdlib>
+#include <cstring>
 
 namespace ppmlhip {
 namespace {
@@ -1163,6 +1164,215 @@ int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int 
     return -1;
 }
 
+// ------------------------------------------------------------------------------------------
+// Low-latency form of the same linear, for Q8_0M weights of at most 64 Ki elements and so few tokens that
+// a work-group of the weight-stationary kernel gets one or two token tiles: there is nothing to amortise
+// resident weights over, and one tile per work-group is a chain of load -> quantize -> block steps ->
+// store in which nothing overlaps (measured at 10609 x 512 -> 128: 12.4 us against about 8 us for a copy
+// of the same bytes).  Here the tokens are cut into units of TOK = 8 or 16 rows, one four-wave work-group
+// each, three of them resident per CU at different stages:
+//
+//   * every lane requests its whole share of the unit's activations at once (with all work-groups
+//     resident the whole of X is in flight within the first microsecond), and right behind them ALL the
+//     weight fragments and scales of its wave's CPW column tiles (wave, wave + 4, ...): at most 64 + 8
+//     registers, served by L2 (the weight is a few tens of KB shared by every work-group) while the
+//     activations are still on their way from HBM;
+//   * the unit is quantized into LDS in MFMA-fragment order as its loads land; one barrier;
+//   * per column tile and pair of blocks: two v_mfma_i32_32x32x32_i8 and one v_mfma_f32_32x32x4_2b_f16 for
+//     the two scale tables, no memory operation but the LDS reads.  The activations are the A operand, so
+//     the TOK tokens occupy the first TOK / 2 accumulator registers of every lane and only those are
+//     settled and stored: the matrix pipe does 32 / TOK times the useful work (it has the slack: these
+//     shapes are bound by memory and latency), the vector pipe none extra.
+//
+// Blocks ascend per output and every settlement is the same fma as everywhere else: same bits.
+// ------------------------------------------------------------------------------------------
+template <int TOK, int NBLK, int CPW, bool DUMP, bool Q81>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void q8_linear_ll_kernel(
+    const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
+    int M, int N, int relu, uint8_t* __restrict__ xq_dump, int32_t* __restrict__ sums_dump) {
+    static_assert(TOK == 8 || TOK == 16, "token rows per work-group");
+    static_assert(NBLK % 2 == 0, "blocks are taken in pairs");
+    static_assert(CPW * NBLK <= 16, "the wave's weight fragments stay in 64 registers");
+    constexpr int NW = 4;
+    constexpr int K = NBLK * QK;
+    constexpr int NUNITS = (TOK / 8) * (NBLK / 2);     // (8 rows) x (2 blocks) each: one wave-wide load pair
+    constexpr int UPW = (NUNITS + NW - 1) / NW;
+    constexpr int RV = TOK / 2;                        // accumulator registers that hold real tokens
+    __shared__ __attribute__((aligned(16))) v4i lds_a[NBLK * 64];     // [block][k half][row][16 quants]
+    __shared__ __attribute__((aligned(8))) uint2 lds_d[NBLK * 32];    // [block][row] {fp16 scale, 0, 0, 0}
+    __shared__ uint16_t lds_wd[NW * CPW * (NBLK / 2) * 64];           // [wave][column tile][pair][lane] fp16 weight scales
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 31;
+    const int tok0 = blockIdx.x * TOK;
+    const int mct = (M + 31) / 32;
+    const int mct_pad = packed_tiles(M);
+    const int grp = lane >> 2, c4 = lane & 3;
+    const int urow = grp & 7, ublk = grp >> 3;
+
+    // ---- all of this lane's activations at once
+    v4f xv[UPW][2];
+#pragma unroll
+    for (int s = 0; s < UPW; ++s) {
+        int u = wave + s * NW;
+        u = u < NUNITS ? u : NUNITS - 1;               // surplus slots repeat the last unit
+        const int bl = (u / (TOK / 8)) * 2 + ublk;
+        int t = tok0 + (u % (TOK / 8)) * 8 + urow;
+        t = t < N ? t : N - 1;                         // rows past the end repeat the last row; never stored
+        const float* src = X + static_cast<int64_t>(t) * K + bl * QK + c4 * 8;
+        xv[s][0] = *reinterpret_cast<const v4f_u*>(src);
+        xv[s][1] = *reinterpret_cast<const v4f_u*>(src + 4);
+    }
+    // ---- all weight fragments and scales of this wave's column tiles, behind them
+    v4i wq[CPW][NBLK];
+    uint16_t wd[CPW][NBLK / 2];                        // parked in LDS once they have arrived: read back pair by pair
+    {
+        const uint16_t* dplane = reinterpret_cast<const uint16_t*>(W + static_cast<size_t>(mct_pad) * NBLK * 1024);
+#pragma unroll
+        for (int t = 0; t < CPW; ++t) {
+            int ct = wave + t * NW;
+            ct = ct < mct_pad ? ct : mct_pad - 1;      // tiles past the end repeat the last one; never stored
+            const size_t frag = static_cast<size_t>(ct) * NBLK;
+#pragma unroll
+            for (int b = 0; b < NBLK; ++b) wq[t][b] = *reinterpret_cast<const v4i*>(W + ((frag + b) * 64 + lane) * 16);
+#pragma unroll
+            for (int pr = 0; pr < NBLK / 2; ++pr)      // lanes 0..31: columns of block 2 pr, 32..63: of block 2 pr + 1
+                wd[t][pr] = dplane[(frag + 2 * pr) * 32 + lane];
+        }
+    }
+
+    // ---- quantize into LDS
+#pragma unroll
+    for (int s = 0; s < UPW; ++s) {
+        const int u = wave + s * NW;
+        if (u >= NUNITS) break;                        // wave-uniform
+        const int row = (u % (TOK / 8)) * 8 + urow;
+        const int bl = (u / (TOK / 8)) * 2 + ublk;
+        v4f x0 = xv[s][0], x1 = xv[s][1];
+        if (relu) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
+        }
+        const BlockQuant bq = quantize_block_lane<Q81>(x0, x1);
+        uint2* dst = reinterpret_cast<uint2*>(lds_a) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
+        *dst = uint2{bq.q_lo, bq.q_hi};
+        if (c4 == 0) lds_d[bl * 32 + row] = uint2{bq.d_bits, 0u};
+        if (DUMP && xq_dump) {
+            const int t = tok0 + row;
+            if (t < N) store_block_part(xq_dump + (static_cast<int64_t>(t) * NBLK + bl) * Q8_0_BYTES, c4, bq);
+        }
+    }
+    uint16_t* my_wd = lds_wd + wave * (CPW * (NBLK / 2) * 64) + lane;
+#pragma unroll
+    for (int t = 0; t < CPW; ++t)
+#pragma unroll
+        for (int pr = 0; pr < NBLK / 2; ++pr) my_wd[(t * (NBLK / 2) + pr) * 64] = wd[t][pr];   // written and read by this wave only
+    __syncthreads();
+
+    // ---- column tiles of this wave, blocks ascending
+    v16i zero_i;
+    v32f zero_f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) zero_i[r] = 0;
+#pragma unroll
+    for (int r = 0; r < 32; ++r) zero_f[r] = 0.0f;
+    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+#pragma unroll
+    for (int t = 0; t < CPW; ++t) {
+        // one basic block per column tile (see opaque_one()), and scheduling fences between the pairs inside
+        // it: left alone, the compiler issues every MFMA of the unrolled code up front and keeps all of
+        // their results alive at once
+        if (!opaque_one()) continue;
+        const int ct = wave + t * NW;
+        if (ct >= mct) break;                          // wave-uniform
+        const int m = ct * 32 + j;                     // this lane's output feature
+        float acc[RV];
+#pragma unroll
+        for (int pr = 0; pr < NBLK / 2; ++pr) {
+            // a basic block per pair: instruction selection orders a block's pure arithmetic as it likes, and
+            // under register pressure it has put every MFMA first and spilled their results
+            if (!opaque_one()) continue;
+            const int b = 2 * pr;
+            const v4i a0 = lds_a[b * 64 + lane];
+            const v4i a1 = lds_a[(b + 1) * 64 + lane];
+            const uint2 da = lds_d[b * 32 + lane];     // lanes 0..31: rows of block b, 32..63: of block b + 1
+            const uint2 dw = uint2{my_wd[(t * (NBLK / 2) + pr) * 64], 0u};
+            // one block sum alive at a time (the waves sharing the SIMD fill the waits): scale tables and the
+            // first sum, settle it, second sum, settle it
+            const v32f scl = __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, da), __builtin_bit_cast(v4h, dw), zero_f, 0, 0, 0);
+            const v16i s0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, wq[t][b], zero_i, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(static_cast<float>(s0[r]), scl[r], pr == 0 ? 0.0f : acc[r]);
+            const v16i s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, wq[t][b + 1], zero_i, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(static_cast<float>(s1[r]), scl[16 + r], acc[r]);
+            if (DUMP && sums_dump) {
+#pragma unroll
+                for (int r = 0; r < RV; ++r) {
+                    const int tok = tok0 + mfma32_row(r, lane);
+                    if (tok < N && m < M) {
+                        sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b] = s0[r];
+                        sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b + 1] = s1[r];
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // each half-wave writes one full 128-byte line of a C row per register
+        if (m < M) {
+#pragma unroll
+            for (int r = 0; r < RV; ++r) {
+                const int tok = tok0 + mfma32_row(r, lane);
+                if (tok < N) __builtin_nontemporal_store(acc[r], C + static_cast<int64_t>(tok) * M + m);
+            }
+        }
+    }
+}
+
+template <int TOK, int NBLK, int CPW, bool Q81>
+int launch_q8_linear_ll(const void* W, const float* X, float* C, int M, int N, int relu,
+                        void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
+    const dim3 grid((N + TOK - 1) / TOK), block(256);
+    if (xq_dump || sums_dump)
+        hipLaunchKernelGGL((q8_linear_ll_kernel<TOK, NBLK, CPW, true, Q81>), grid, block, 0, stream, static_cast<const uint8_t*>(W), X, C,
+                           M, N, relu, static_cast<uint8_t*>(xq_dump), sums_dump);
+    else
+        hipLaunchKernelGGL((q8_linear_ll_kernel<TOK, NBLK, CPW, false, Q81>), grid, block, 0, stream, static_cast<const uint8_t*>(W), X, C,
+                           M, N, relu, static_cast<uint8_t*>(nullptr), static_cast<int32_t*>(nullptr));
+    return check_launch("q8_linear_ll_kernel");
+}
+
+// Shape gate of the low-latency kernel; returns -1 when the weight-stationary kernel (or the general one)
+// should take the call.  `force` = 8 or 16 picks that unit size whatever the gate says (measurements).
+template <bool Q81>
+int try_q8_linear_ll(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
+                     int relu, int force, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
+    if (!c_trans) return -1;
+    const int mct = (M + 31) / 32;
+    const int cpw = nblk == 16 ? 1 : nblk == 8 ? 2 : nblk == 4 ? 4 : 0;
+    if (cpw == 0 || mct > 4 * cpw) return -1;          // the wave's share of the weight must fit 64 registers
+    int tok = force;
+    if (tok == 0) {
+        // Measured crossover against the weight-stationary kernel (us, low-latency / weight-stationary):
+        //   408 x 256 -> 256   4.4 (TOK 8) / 5.2       2601 x 128 -> 128   4.3 (16) / 5.1      2601 x 256 -> 256  5.5 (16) / 5.6
+        //   10609 x 512 -> 128 10.2 (16) / 12.4        10609 x 128 -> 512  7.9 (16) / 7.1      26368 x 256 -> 768  no instance / 24
+        // i.e. it wins while all its work-groups are resident at once (three per CU) and the output is narrow.
+        const int resident = 3 * device_cu_count();
+        if (N <= 2048) tok = 8;
+        else if (N <= 4096 || (nblk == 16 && (N + 15) / 16 <= resident)) tok = 16;
+        else return -1;
+    }
+#define PPML_LL(TOK, NBLK, CPW) if (tok == TOK && nblk == NBLK) return launch_q8_linear_ll<TOK, NBLK, CPW, Q81>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
+    PPML_LL(8, 4, 4);  PPML_LL(8, 8, 2);  PPML_LL(8, 16, 1);
+    PPML_LL(16, 4, 4); PPML_LL(16, 8, 2); PPML_LL(16, 16, 1);
+#undef PPML_LL
+    return -1;
+}
+
 template <int WT>
 int dispatch_q8_linear(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
                        int relu, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
@@ -1250,7 +1460,13 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
         case PPML_WTYPE_Q8_1:  return dispatch_q8_linear<PPML_WTYPE_Q8_1>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0R: return dispatch_q8_linear<PPML_WTYPE_Q8_0R>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0M: {
-            const int rc = (act & 2) ? try_q8_linear_ws<true>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s)
+            const int force_ll = (flags & PPML_Q8_FLAG_LOW_LATENCY_8) ? 8 : (flags & PPML_Q8_FLAG_LOW_LATENCY_16) ? 16 : 0;
+            const int rl = (flags & PPML_Q8_FLAG_NO_LOW_LATENCY) ? -1
+                         : (act & 2) ? try_q8_linear_ll<true>(W, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s)
+                                     : try_q8_linear_ll<false>(W, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s);
+            if (rl >= 0) { set_q8_path(PPML_Q8_PATH_LOW_LATENCY); stat.set_path("hip/q8-low-latency"); return rl; }
+            const int rc = (flags & PPML_Q8_FLAG_NO_WEIGHT_STATIONARY) ? -1
+                         : (act & 2) ? try_q8_linear_ws<true>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s)
                                      : try_q8_linear_ws<false>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
             if (rc >= 0) { set_q8_path(PPML_Q8_PATH_WEIGHT_STATIONARY); stat.set_path("hip/q8-weight-stationary"); return rc; }
             return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);

@@ -392,13 +392,19 @@ class Q8Weight:
         return Q8Weight(out, self.M, self.K, WTYPE_Q8_0M)
 
 
+_Q8_PATH_FLAGS = {"auto": 0, "weight-stationary": 4, "general": 4 | 8, "low-latency": 0, "low-latency-8": 16, "low-latency-16": 32}
+
+
 def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = False,
-               dump: bool = False, act: str = "q8_0"):
+               dump: bool = False, act: str = "q8_0", path: str = "auto"):
     """Q8_0 linear: x f32 [N,K] (rows = tokens) times quantized w [M,K] -> [N,M] (c_trans=1, the
     LinearLayer orientation) or [M,N] (c_trans=0); src/backend/CUDAKernels.cpp:740-789.
     With ``dump`` also returns the kernel's own Q8_0 blocks of x and its per-block int32 sums.
     ``act`` selects the rule the activations are quantized with: "q8_0" (the CPU contract) or
-    "q8_1" (what the reference's CUDA launcher does, src/cuda/MulMatQ8Kernel.cu:483-527)."""
+    "q8_1" (what the reference's CUDA launcher does, src/cuda/MulMatQ8Kernel.cu:483-527).
+    ``path`` restricts the kernel choice for a packed weight ("weight-stationary": not the low-latency kernel;
+    "general": neither of the two; "low-latency-8" / "-16": that unit size wherever an instance exists); every
+    choice gives the same bits."""
     if act not in ("q8_0", "q8_1"):
         raise ValueError("mul_mat_q8: act must be 'q8_0' or 'q8_1'")
     x = _dev_f32(x, "x")
@@ -408,7 +414,7 @@ def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = Fals
     M = w.M
     out = torch.empty((N, M) if c_trans else (M, N), dtype=torch.float32, device=x.device)
     lib = _lib()
-    if not dump and not relu and act == "q8_0":
+    if not dump and not relu and act == "q8_0" and path == "auto":
         path = C.c_int(0)
         cabi.check("mul_mat_q8_hip", lib.mul_mat_q8_hip(_ptr(w.data), _ptr(x), _ptr(out), M, N, K, w.wtype,
                                                          c_trans, C.byref(path), _stream()))
@@ -418,6 +424,6 @@ def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = Fals
         xq = torch.empty((N, K // QK, BLOCK_BYTES), dtype=torch.uint8, device=x.device)
         sums = torch.empty((N, M, K // QK), dtype=torch.int32, device=x.device)
     cabi.check("mul_mat_q8_ex_hip", lib.mul_mat_q8_ex_hip(_ptr(w.data), _ptr(x), _ptr(out), M, N, K, w.wtype,
-                                                           c_trans, (1 if relu else 0) | (2 if act == "q8_1" else 0),
+                                                           c_trans, (1 if relu else 0) | (2 if act == "q8_1" else 0) | _Q8_PATH_FLAGS[path],
                                                            _ptr(xq), _ptr(sums), _stream()))
     return (out, xq, sums) if dump else out

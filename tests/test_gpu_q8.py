@@ -130,6 +130,9 @@ SHAPES += [
     (9000, 256, 400),     # (2, 8) with several token tiles per work-group (staged loads, three LDS buffers in turn)
     (9000, 512, 200),     # (1, 16) likewise: the 64-register staging range
     (17000, 128, 700),    # (3, 4) likewise, with leftover tiles shared between work-groups
+    (3001, 512, 128),     # more than 2048 tokens: the library itself picks the low-latency kernel with 16-token units
+    (3001, 128, 500),
+    (3001, 256, 250),
 ]
 
 # (column tiles of 32 outputs) -> instance: up to 4 tiles the four-wave kernels, beyond that ceil(tiles / 8) per wave
@@ -161,10 +164,27 @@ def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packe
     # the undumped fast path gives the same bits
     fast = ops.mul_mat_q8(W, _dev(x), c_trans=1).cpu().numpy()
     assert (fast == out).all()
-    # packed weights of K / 32 in {4, 8, 16} and at most 256 Ki elements are served by the resident-weight kernels
-    if packed and _has_resident_weight_instance(K, M):
-        assert ops.last_q8_path() != "general"
-    elif not packed:
+    if not packed:
+        assert ops.last_q8_path() == "general"
+        return
+    # a packed weight: every kernel family that has an instance for the shape, dump form and fast form
+    families = ["general"]
+    if _has_resident_weight_instance(K, M):
+        families.append("weight-stationary")
+    if _has_low_latency_instance(K, M):
+        families += ["low-latency-8", "low-latency-16"]
+    for fam in families:
+        o2, xq2, sums2 = ops.mul_mat_q8(W, _dev(x), c_trans=1, dump=True, path=fam)
+        assert ops.last_q8_path() == fam.rsplit("-", 1)[0] if fam.startswith("low") else ops.last_q8_path() == fam, fam
+        assert (o2.cpu().numpy() == want).all() and (xq2.cpu().numpy() == xq_want).all() and (sums2.cpu().numpy() == sums).all(), fam
+        assert (ops.mul_mat_q8(W, _dev(x), c_trans=1, path=fam).cpu().numpy() == want).all(), fam
+    # the library's own choice: low-latency for few tokens, else weight-stationary, else general
+    ops.mul_mat_q8(W, _dev(x), c_trans=1)
+    if _has_low_latency_instance(K, M) and N <= 4096:
+        assert ops.last_q8_path() == "low-latency"
+    elif _has_resident_weight_instance(K, M):
+        assert ops.last_q8_path() == "weight-stationary"
+    else:
         assert ops.last_q8_path() == "general"
 
 
@@ -172,6 +192,12 @@ def _has_resident_weight_instance(K, M):
     tiles, nblk = (M + 31) // 32, K // 32
     tpw = (tiles + 7) // 8
     return K % 32 == 0 and nblk in (4, 8, 16) and (tiles <= 4 or tpw <= {4: 4, 8: 3, 16: 1}[nblk])
+
+
+def _has_low_latency_instance(K, M):
+    # the wave's share of the weight (column tiles wave, wave + 4, ...) must fit 64 registers
+    tiles, nblk = (M + 31) // 32, K // 32
+    return K % 32 == 0 and nblk in (4, 8, 16) and tiles <= 4 * (16 // nblk)
 
 
 def test_every_weight_stationary_instance_has_a_shape_in_the_suite():
@@ -217,9 +243,10 @@ def test_relu_fused_into_the_quantizer(ops, oracle):
     x, w = _inputs(21, 200, 512, 128)
     wq = oracle.quantize_q8_0(w)
     W = ops.Q8Weight(_dev(wq.reshape(-1)), 128, 512, ops.WTYPE_Q8_0).pack()
-    got = ops.mul_mat_q8(W, _dev(x), relu=True).cpu().numpy()
     want = oracle.mul_mat_q8(wq, np.maximum(x, 0.0), wtype=0, c_trans=1, fma=1)
-    assert (got == want).all()
+    for fam in ("auto", "general", "weight-stationary", "low-latency-8", "low-latency-16"):
+        got = ops.mul_mat_q8(W, _dev(x), relu=True, path=fam).cpu().numpy()
+        assert (got == want).all(), fam
 
 
 def test_status_codes(ops):
@@ -331,4 +358,11 @@ def test_fused_linear_with_q8_1_activations(ops, oracle, wname, N, K, M, c_trans
     assert (y2 == want).all()
     # a packed weight in the LinearLayer orientation gets the resident-weight kernels under this rule too
     assert (ops.last_q8_path() != "general") == (wname == "packed" and c_trans == 1)
+    if wname == "packed" and c_trans == 1:
+        for fam in ("weight-stationary", "low-latency-8", "low-latency-16"):
+            if fam.startswith("low") and not _has_low_latency_instance(K, M):
+                continue
+            y3 = ops.mul_mat_q8(W, _dev(x), c_trans=1, act="q8_1", path=fam).cpu().numpy()
+            assert ops.last_q8_path() == fam.rsplit("-", 1)[0] if fam.startswith("low") else ops.last_q8_path() == fam
+            assert (y3 == want).all(), fam
     assert (ops.mul_mat_q8(W, _dev(x), c_trans=c_trans).cpu().numpy() != want).any()
