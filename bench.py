@@ -102,6 +102,36 @@ def main() -> int:
         torch.cuda.synchronize()
         return wall, e0.elapsed_time(e1) * 1e-3 / steps
 
+    # ------------------------------------------------------------------ what the bytes alone cost
+    import ctypes as C
+    probe_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "proteinpredictmachinelearning_amd", "lib", "libppml_probe.so")
+    probe = C.CDLL(probe_path) if os.path.exists(probe_path) else None
+    if probe is not None:
+        probe.ppml_probe_stream.restype = C.c_int
+        probe.ppml_probe_stream.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_void_p]
+
+    def bytes_only_us(read_bytes, write_bytes, steps, warmup):
+        """Time per launch of a kernel that only reads `read_bytes` and writes `write_bytes` (16 bytes per lane,
+        coalesced, buffers rotated past the last-level cache), measured in the same loop as everything else: the
+        practical floor of a launch with that HBM traffic on this box, launch latency included.  The best of
+        streaming / ordinary stores and of a one-pass / persistent grid."""
+        if probe is None:
+            return None
+        read_bytes, write_bytes = (int(read_bytes) + 15) // 16 * 16, (int(write_bytes) + 15) // 16 * 16
+        ns = max(2, int(640e6 // (read_bytes + write_bytes)) + 1)
+        srcs = [torch.randn(max(read_bytes, 16) // 4, device=dev, generator=gen) for _ in range(ns)]
+        dsts = [torch.empty(max(write_bytes, 16) // 4, device=dev) for _ in range(ns)]
+        stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+        best = None
+        for nt in (1, 0):
+            for groups in (0, 2048):
+                def fn(i, nt=nt, groups=groups):
+                    probe.ppml_probe_stream(C.c_void_p(srcs[i].data_ptr()), C.c_void_p(dsts[i].data_ptr()), read_bytes, write_bytes,
+                                            nt, groups, stream)
+                _, ev_ = time_op(fn, ns, steps, warmup)
+                best = ev_ if best is None else min(best, ev_)
+        return round(best * 1e6, 2)
+
     def q8_case(rows, K, N, relu=False):
         nbytes = q8_bytes(rows, K, N)
         nsets = max(2, int(640e6 // nbytes) + 1)
@@ -110,7 +140,6 @@ def main() -> int:
         xs = [torch.randn(rows, K, device=dev, generator=gen) for _ in range(nsets)]
         ys = [torch.empty(rows, N, device=dev) for _ in range(nsets)]
         lib, cabi = ops._lib(), ops.cabi
-        import ctypes as C
         stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
         wp = C.c_void_p(W.data.data_ptr())
         xp = [C.c_void_p(x.data_ptr()) for x in xs]
@@ -151,7 +180,8 @@ def main() -> int:
                      "kernel": "q8_linear_ws_kernel", "algorithmic_bytes_per_launch": nbytes,
                      "kernel_us": round(ev * 1e6, 2), "clock": "HIP events on the launch stream, region queued behind preheat_ms of load",
                      "wall_us": round(wall * 1e6, 2), "frac_wall_clock": round(nbytes / wall / 1e9 / HBM_PEAK_GBS, 4),
-                     "int8_mfma_frac": round(nops / ev / 1e12 / INT8_PEAK_TOPS, 4)},
+                     "int8_mfma_frac": round(nops / ev / 1e12 / INT8_PEAK_TOPS, 4),
+                     "bytes_only_us": bytes_only_us(rows * K * 4 + N * K * 34 // 32, rows * N * 4, max(20, args.steps // 4), 5)},
     }
 
     # ------------------------------------------------------------------ CPU baseline (oracle, rank 0)
@@ -195,9 +225,10 @@ def main() -> int:
             f, ns, nb, no, _ = q8_case(r, k, n, relu)
             w_, e_ = time_op(f, ns, steps, warm)
             extra[name] = {"us": round(e_ * 1e6, 2), "TOPS": round(no / e_ / 1e12, 2), "GBps": round(nb / e_ / 1e9, 1),
-                           "hbm_frac": round(nb / e_ / 1e9 / HBM_PEAK_GBS, 4)}
+                           "hbm_frac": round(nb / e_ / 1e9 / HBM_PEAK_GBS, 4), "kernel": ops.last_q8_path(),
+                           "bytes_only_us": bytes_only_us(r * k * 4 + n * k * 34 // 32, r * n * 4, steps, warm)}
 
-        def f32_case(make, nbytes, flops, name, pipe="fp32"):
+        def f32_case(make, nbytes, flops, name, pipe="fp32", rw=None):
             # pipe: "fp32" = fp32 MFMA; "bf16x3" = binary32 operands split three ways, six bf16 MFMA
             # products per binary32 product (TFLOPS counts binary32 products, the fraction bf16 ones)
             fn_, ns = make()
@@ -208,6 +239,10 @@ def main() -> int:
                 extra[name]["bf16_mfma_frac"] = round(6.0 * flops / e_ / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4)
             else:
                 extra[name]["fp32_mfma_frac"] = round(flops / e_ / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4)
+            if rw is not None:                          # (bytes read, bytes written) of an HBM-bound shape
+                extra[name]["bytes_only_us"] = bytes_only_us(rw[0], rw[1], steps, warm)
+
+        keep = []
 
         def logits(planes, L, D):
             def make():
@@ -215,12 +250,26 @@ def main() -> int:
                 ns = max(2, int(640e6 // nb) + 1)
                 ks = [torch.randn(1, planes, D, L, device=dev, generator=gen) for _ in range(ns)]
                 qs = [torch.randn(1, planes, D, L, device=dev, generator=gen) for _ in range(ns)]
-                return (lambda i: ops.attention_logits(ks[i], qs[i])), ns
+                outs = [torch.empty(1, planes, L, L, device=dev) for _ in range(ns)]
+                # straight through the C ABI on preallocated outputs: the Python operator's own bookkeeping
+                # (shape checks, output allocation) costs more host time per call than the small shape takes on the GPU
+                lib, cabi = ops._lib(), ops.cabi
+                stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+                dims = [L, D, planes, 1, L, D, planes, 1, L, L, planes, 1]
+                argsets = [(C.c_void_p(ks[i].data_ptr()), C.c_void_p(qs[i].data_ptr()), C.c_void_p(outs[i].data_ptr()), *dims,
+                            1.0 / D ** 0.5, stream) for i in range(ns)]
+
+                def fn(i):
+                    rc = lib.out_prod_scaled_hip(*argsets[i])
+                    if rc:
+                        cabi.check("out_prod_scaled_hip", rc)
+                keep.append((ks, qs, outs))
+                return fn, ns
             return make
         f32_case(logits(412, 103, 32), (2 * 412 * 32 * 103 + 412 * 103 * 103) * 4, 2.0 * 412 * 103 * 103 * 32,
-                 "attn_logits_pair_412x103x103x32", pipe="bf16x3")
+                 "attn_logits_pair_412x103x103x32", pipe="bf16x3", rw=(2 * 412 * 32 * 103 * 4, 412 * 103 * 103 * 4))
         f32_case(logits(824, 256, 32), (2 * 824 * 32 * 256 + 824 * 256 * 256) * 4, 2.0 * 824 * 256 * 256 * 32,
-                 "attn_logits_msa_824x256x256x32", pipe="bf16x3")
+                 "attn_logits_msa_824x256x256x32", pipe="bf16x3", rw=(2 * 824 * 32 * 256 * 4, 824 * 256 * 256 * 4))
 
         def attention(planes, L, D, with_bias, layout=0):
             def make():
@@ -243,7 +292,6 @@ def main() -> int:
                 keep.append((qkv, bs, outs))
                 return fn, ns
             return make
-        keep = []
         # layout 3: Q, K, V and O in the graph's [L, D, h, B] layout, i.e. without the four permutation copies
         for planes, L, D, wb, lay, tag in [(412, 103, 32, True, 0, "pair_412x103x32_bias"), (824, 256, 32, True, 0, "msa_824x256x32_bias"),
                                            (824, 256, 32, False, 0, "msa_824x256x32"),
@@ -294,7 +342,7 @@ def main() -> int:
                     cabi.check("permute_hip", rc)
             keep.append((xs, ys))
             return fn, ns
-        f32_case(bridge, 2 * 824 * 32 * 256 * 4, 0.0, "permute_attention_bridge_824x256x32")
+        f32_case(bridge, 2 * 824 * 32 * 256 * 4, 0.0, "permute_attention_bridge_824x256x32", rw=(824 * 32 * 256 * 4, 824 * 32 * 256 * 4))
 
         def trimul():
             # triangle multiplication (outgoing) of the pair track: 128 channels x 103 x 103, contracted length 103

@@ -39,6 +39,7 @@ private:
 };
 hipMemPool_t workspace_pool();         // the library's stream-ordered pool on the current device, or null
 int noalloc_scratch_setup(uint8_t** out);   // address of the no-allocation entry point's static workspace on the current device
+int device_cu_count();
 void set_q8_path(int path);              // what ppml_hip_q8_last_path() reports for the calling thread
 
 typedef int   v4i  __attribute__((ext_vector_type(4)));

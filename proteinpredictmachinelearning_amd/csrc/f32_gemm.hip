@@ -311,8 +311,54 @@ __device__ __forceinline__ void load_rows8(const float* __restrict__ base, int64
         reg[c >> 2][c & 3] = (row < nrows && kb + c < K) ? src[static_cast<int64_t>(c) * ks] : 0.0f;
 }
 
-template <int MODE, bool SPLIT_C, bool STREAM_C>
+// ---- buffer-addressed forms for planes below 2 GiB (FAST_IO).  The generic paths above spend most of the
+// kernel's vector instructions on 64-bit address arithmetic and bounds tests (counters at the attention-logit
+// shapes: about 1150 vector instructions per wave, of which the split is 180); a buffer resource per plane
+// takes both over: the address is one 32-bit add per access, and an access whose offset is not inside the
+// plane is dropped (stores) or returns zero (loads) in hardware.  Lanes whose row or column lies outside the
+// matrix carry an offset of 2^31, which no plane reaches.
+constexpr uint32_t OUTSIDE = 0x80000000u;
+
+// one row, eight consecutive k of an operand plane [K][ks] whose rows are contiguous: A(row, k) = plane[k * ks + row]
+__device__ __forceinline__ void load_rows8_buffer(const __amdgpu_buffer_rsrc_t rsrc, uint32_t ks_bytes, int row0, int nrows, int k0,
+                                                  int tid, v4f (&reg)[2]) {
+    const int row = row0 + (tid & 127);
+    const uint32_t lane_off = row < nrows ? static_cast<uint32_t>(row) * 4u : OUTSIDE;
+    // k is the same for the whole wave: its part of the offset is scalar arithmetic
+    const uint32_t kb = static_cast<uint32_t>(k0 + __builtin_amdgcn_readfirstlane(tid >> 7) * 8);
+#pragma unroll
+    for (int c = 0; c < 8; ++c)
+        reg[c >> 2][c & 3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, lane_off + (kb + c) * ks_bytes, 0, 0));
+}
+
+// The finished accumulators of one wave to a dense plane C[m * ld + n] through a buffer resource over the plane.
+template <bool STREAM_C>
+__device__ __forceinline__ void store_acc_buffer(const __amdgpu_buffer_rsrc_t rsrc, uint32_t ld_bytes, int N, float alpha,
+                                                 const v16f (&acc)[2][2], int m_base, int n_base, int lane) {
+    const int j = lane & 31;
+    const bool scale = alpha != 1.0f;
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti) {
+        const uint32_t first = static_cast<uint32_t>(m_base + ti * 32 + 4 * (lane >> 5));
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj) {
+            const int n = n_base + tj * 32 + j;
+            // rows past the matrix fall outside the plane by themselves (offset >= M * ld bytes)
+            const uint32_t base = n < N ? first * ld_bytes + static_cast<uint32_t>(n) * 4u : OUTSIDE;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = acc[ti][tj][r];
+                if (scale) v *= alpha;
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rsrc, base + (8 * (r >> 2) + (r & 3)) * ld_bytes, 0,
+                                                      STREAM_C ? 3 : 0);
+            }
+        }
+    }
+}
+
+template <int MODE, bool SPLIT_C, bool STREAM_C, bool FAST_IO = false>
 __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
+    static_assert(!FAST_IO || (MODE == LOAD_ROW_CONTIG && !SPLIT_C), "buffer addressing: contiguous rows, dense output");
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * SPLIT_PLANE];
     __shared__ __attribute__((aligned(16))) uint8_t lds_b[3 * SPLIT_PLANE];
 
@@ -341,8 +387,18 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
 
     v4f ra[2], rb[2];
     constexpr int MODE_B = MODE == LOAD_SPLIT_A ? LOAD_STRIDED : MODE;
+    // FAST_IO: one buffer resource per operand plane and for the output plane (sizes checked by the launcher)
+    __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_c;
+    if (FAST_IO) {
+        rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, static_cast<int>(p.K * p.a_ks * 4), 0x00020000);
+        rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, static_cast<int>(p.K * p.b_ks * 4), 0x00020000);
+        rsrc_c = __builtin_amdgcn_make_buffer_rsrc(C, 0, static_cast<int>(p.M * p.c_mi * 4), 0x00020000);
+    }
     const auto load_both = [&](int k0) {
-        if (MODE == LOAD_ROW_CONTIG) {
+        if (FAST_IO) {
+            load_rows8_buffer(rsrc_a, static_cast<uint32_t>(p.a_ks) * 4u, m0, p.M, k0, tid, ra);
+            load_rows8_buffer(rsrc_b, static_cast<uint32_t>(p.b_ks) * 4u, n0, p.N, k0, tid, rb);
+        } else if (MODE == LOAD_ROW_CONTIG) {
             load_rows8(A, p.a_ks, m0, p.M, k0, p.K, tid, ra);
             load_rows8(B, p.b_ks, n0, p.N, k0, p.K, tid, rb);
         } else {
@@ -380,7 +436,176 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
         __syncthreads();
     }
 
-    store_acc<SPLIT_C, STREAM_C, false, false>(p, C, acc, m0 + wm, n0 + wn, lane);
+    if (FAST_IO) store_acc_buffer<STREAM_C>(rsrc_c, static_cast<uint32_t>(p.c_mi) * 4u, p.N, p.alpha, acc, m0 + wm, n0 + wn, lane);
+    else store_acc<SPLIT_C, STREAM_C, false, false>(p, C, acc, m0 + wm, n0 + wn, lane);
+}
+
+// ------------------------------------------------------------------------------------------
+// Batched contractions with a short K (at most 32: the attention logits, K = head dimension) on operands whose
+// rows are contiguous, into dense output planes.  Per output tile there are two 16-k chunks of matrix work and
+// TM x TM x 4 bytes to write, so a work-group that does one tile is a chain load -> split -> MFMA -> store
+// whose stages wait for each other, and the kernel above ran at 0.45 (pair shape) and 0.75 (MSA shape) of what
+// its bytes alone take.  This form is persistent and staged the other way round:
+//
+//   * two work-groups per CU walk the tile list; the tiles of one XCD are consecutive ones, so the two or
+//     four tiles that share an operand panel meet in one L2;
+//   * the whole K of a tile is loaded at once (every lane: one row, eight k, per operand and 16-k chunk), and
+//     the loads of tile i + 1 are issued before the matrix work of tile i; they are older than tile i's stores,
+//     so waiting for them at the top of the next iteration does not wait for those stores;
+//   * both chunks are split into LDS together: two barriers per tile, no load inside the matrix work;
+//   * addresses through one buffer resource per plane (rows and columns outside the matrix: zero on the way
+//     in, dropped on the way out).
+//
+// Arithmetic and order of the sums are those of gemm_bf16x3_kernel: same bits.
+template <int TM, bool STREAM_C>
+__global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmParams p, int total_tiles) {
+    static_assert(TM == 64 || TM == 128, "tile side");
+    constexpr int WT = TM / 2;                        // a wave's square of the tile
+    constexpr int NT = WT / 32;                       // 32 x 32 accumulator tiles per side of it
+    constexpr int CHUNK_PLANE = TM * SPLIT_PITCH;     // one bf16 plane of one 16-k chunk of one operand
+    constexpr int OPERAND = 2 * 3 * CHUNK_PLANE;      // [chunk][plane][row][48 bytes]
+    constexpr int LOADS = TM == 128 ? 2 : 1;          // 16-k chunks a thread loads separately (at 64 rows one pass covers K = 32)
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[OPERAND];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_b[OPERAND];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const int wm = (wave >> 1) * WT, wn = (wave & 1) * WT;
+    const int tiles_m = (p.M + TM - 1) / TM, tiles_n = (p.N + TM - 1) / TM;
+    const int per_plane = tiles_m * tiles_n;
+
+    // this work-group's tiles: the list is cut into eight consecutive parts, one per XCD (work-group ids go
+    // round the XCDs), and the work-groups of an XCD take the tiles of its part in turn
+    constexpr int XCDS = 8;
+    const int groups = static_cast<int>(gridDim.x) / XCDS;                 // work-groups per XCD (the grid is a multiple of 8)
+    const int xcd = static_cast<int>(blockIdx.x) % XCDS, slot = static_cast<int>(blockIdx.x) / XCDS;
+    const int part = (total_tiles + XCDS - 1) / XCDS;
+    const int part_begin = xcd * part;
+    const int part_end = part_begin + part < total_tiles ? part_begin + part : total_tiles;
+
+    // thread -> (row of the tile, octet of k) for the loads and the split
+    const int lrow = TM == 128 ? (tid & 127) : (tid & 63);
+    const int loct = TM == 128 ? (tid >> 7) : (tid >> 6);                  // uniform within a wave
+    v4f ra[LOADS][2], rb[LOADS][2];
+
+    struct Tile { const float* A; const float* B; float* C; int m0, n0; };
+    const auto tile_at = [&](int t) {
+        const int plane = t / per_plane;
+        const int r = t - plane * per_plane;
+        const int p2 = plane % p.np2, p3 = plane / p.np2;
+        Tile tl;
+        tl.A = p.A + p2 * p.a_p2 + p3 * p.a_p3;
+        tl.B = p.B + (p2 / p.b_div2) * p.b_p2 + (p3 / p.b_div3) * p.b_p3;
+        tl.C = p.C + p2 * p.c_p2 + p3 * p.c_p3;
+        tl.m0 = (r / tiles_n) * TM;
+        tl.n0 = (r % tiles_n) * TM;
+        return tl;
+    };
+    const uint32_t a_ks = static_cast<uint32_t>(p.a_ks) * 4u, b_ks = static_cast<uint32_t>(p.b_ks) * 4u;
+    const int a_bytes = static_cast<int>(p.K * p.a_ks * 4), b_bytes = static_cast<int>(p.K * p.b_ks * 4);
+    const auto load_tile_regs = [&](const Tile& tl) {
+        const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(tl.A), 0, a_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(tl.B), 0, b_bytes, 0x00020000);
+        const uint32_t off_a = tl.m0 + lrow < p.M ? static_cast<uint32_t>(tl.m0 + lrow) * 4u : OUTSIDE;
+        const uint32_t off_b = tl.n0 + lrow < p.N ? static_cast<uint32_t>(tl.n0 + lrow) * 4u : OUTSIDE;
+#pragma unroll
+        for (int l = 0; l < LOADS; ++l) {
+            const uint32_t kb = static_cast<uint32_t>((TM == 128 ? l * 16 : 0) + __builtin_amdgcn_readfirstlane(loct) * 8);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                // k >= K lies behind the end of the plane: zero
+                ra[l][c >> 2][c & 3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_a, off_a + (kb + c) * a_ks, 0, 0));
+                rb[l][c >> 2][c & 3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_b, off_b + (kb + c) * b_ks, 0, 0));
+            }
+        }
+    };
+    // a lane's share goes to the three planes of its chunk: row lrow, bytes 16 * (octet % 2) of the row's 32
+    const auto split_to_lds = [&]() {
+#pragma unroll
+        for (int l = 0; l < LOADS; ++l) {
+            const int oct = (TM == 128 ? 2 * l : 0) + loct;                 // octet of k, 0..3
+            const int at = (oct >> 1) * 3 * CHUNK_PLANE + lrow * SPLIT_PITCH + (oct & 1) * 16;
+            uint2 lo[3], hi[3];
+            split4(ra[l][0], lo);
+            split4(ra[l][1], hi);
+#pragma unroll
+            for (int q = 0; q < 3; ++q) *reinterpret_cast<uint4*>(lds_a + at + q * CHUNK_PLANE) = uint4{lo[q].x, lo[q].y, hi[q].x, hi[q].y};
+            split4(rb[l][0], lo);
+            split4(rb[l][1], hi);
+#pragma unroll
+            for (int q = 0; q < 3; ++q) *reinterpret_cast<uint4*>(lds_b + at + q * CHUNK_PLANE) = uint4{lo[q].x, lo[q].y, hi[q].x, hi[q].y};
+        }
+    };
+
+    int t = part_begin + slot;
+    if (t >= part_end) return;                          // whole work-group: no barrier is left behind
+    Tile cur = tile_at(t);
+    load_tile_regs(cur);
+    const uint8_t* frag_a = lds_a + (wm + j) * SPLIT_PITCH + hh * 16;
+    const uint8_t* frag_b = lds_b + (wn + j) * SPLIT_PITCH + hh * 16;
+    const bool scale = p.alpha != 1.0f;
+    const uint32_t ld_bytes = static_cast<uint32_t>(p.c_mi) * 4u;
+    const int c_bytes = static_cast<int>(p.M * p.c_mi * 4);
+
+    while (true) {
+        split_to_lds();
+        __syncthreads();
+        const int t_next = t + groups;
+        const bool more = t_next < part_end;
+        Tile nxt = cur;
+        if (more) {
+            nxt = tile_at(t_next);
+            load_tile_regs(nxt);
+        }
+        v16f acc[NT][NT];
+#pragma unroll
+        for (int ti = 0; ti < NT; ++ti)
+#pragma unroll
+            for (int tj = 0; tj < NT; ++tj)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            v8bf fa[NT][3], fb[NT][3];
+#pragma unroll
+            for (int ti = 0; ti < NT; ++ti)
+#pragma unroll
+                for (int q = 0; q < 3; ++q) {
+                    fa[ti][q] = *reinterpret_cast<const v8bf*>(frag_a + (c * 3 + q) * CHUNK_PLANE + ti * 32 * SPLIT_PITCH);
+                    fb[ti][q] = *reinterpret_cast<const v8bf*>(frag_b + (c * 3 + q) * CHUNK_PLANE + ti * 32 * SPLIT_PITCH);
+                }
+#pragma unroll
+            for (int q = 0; q < 6; ++q)
+#pragma unroll
+                for (int ti = 0; ti < NT; ++ti)
+#pragma unroll
+                    for (int tj = 0; tj < NT; ++tj)
+                        acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][SPLIT_TERMS[q][0]], fb[tj][SPLIT_TERMS[q][1]], acc[ti][tj], 0, 0, 0);
+        }
+        __syncthreads();                                // the planes may be overwritten
+        // ---- stores of this tile: younger than the next tile's loads
+        const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(cur.C, 0, c_bytes, 0x00020000);
+#pragma unroll
+        for (int ti = 0; ti < NT; ++ti) {
+            const uint32_t first = static_cast<uint32_t>(cur.m0 + wm + ti * 32 + 4 * hh);
+#pragma unroll
+            for (int tj = 0; tj < NT; ++tj) {
+                const int n = cur.n0 + wn + tj * 32 + j;
+                const uint32_t base = n < p.N ? first * ld_bytes + static_cast<uint32_t>(n) * 4u : OUTSIDE;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float v = acc[ti][tj][r];
+                    if (scale) v *= p.alpha;
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rsrc_c, base + (8 * (r >> 2) + (r & 3)) * ld_bytes, 0,
+                                                          STREAM_C ? 3 : 0);
+                }
+            }
+        }
+        if (!more) break;
+        t = t_next;
+        cur = nxt;
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -802,6 +1027,32 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
         if (mode == LOAD_K_CONTIG)        { if (split) PPML_LAUNCH_F32(LOAD_K_CONTIG, true);   else PPML_LAUNCH_F32(LOAD_K_CONTIG, false); }
         else if (mode == LOAD_ROW_CONTIG) { if (split) PPML_LAUNCH_F32(LOAD_ROW_CONTIG, true); else PPML_LAUNCH_F32(LOAD_ROW_CONTIG, false); }
         else                              { if (split) PPML_LAUNCH_F32(LOAD_STRIDED, true);    else PPML_LAUNCH_F32(LOAD_STRIDED, false); }
+    }
+    else if (!p.clamp && !p.f16_in && mode == LOAD_ROW_CONTIG && !split && p.c_ni == 1 && !p.bias &&
+             p.K * p.a_ks * 4 < (1LL << 31) && p.K * p.b_ks * 4 < (1LL << 31) && p.M * p.c_mi * 4 < (1LL << 31) &&
+             p.a_ks < (1 << 24) && p.b_ks < (1 << 24) && p.c_mi < (1 << 22)) {
+        // (the last three keep "offset of a lane outside the matrix + up to 32 k steps / 128 rows" below 2^32)
+        // contiguous rows, dense output planes below 2 GiB each: buffer addressing
+        if (p.K <= 32) {
+            // a short K: the persistent, single-stage form; two work-groups per CU, a multiple of eight in all
+            // 128-wide tiles from about 100 rows a side (measured at the logit shapes: 103 rows 10.2 us against 10.6
+            // with 64-wide tiles, 256 rows 43 against 47)
+            const bool big = (p.M < p.N ? p.M : p.N) >= 96;
+            const int tm = big ? 128 : 64;
+            const int64_t tiles = static_cast<int64_t>((p.M + tm - 1) / tm) * ((p.N + tm - 1) / tm) * p.np2 * p.np3;
+            if (tiles <= 0x7fffffffLL) {
+                int wgs = (big ? 2 : 4) * device_cu_count();      // resident work-groups: 72 KB / 36 KB of LDS each
+                if (tiles < wgs) wgs = static_cast<int>((tiles + 7) / 8 * 8);
+                const dim3 pgrid(static_cast<unsigned>(wgs));
+                if (big) { if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<128, true>), pgrid, block, 0, stream, p, static_cast<int>(tiles));
+                           else hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<128, false>), pgrid, block, 0, stream, p, static_cast<int>(tiles)); }
+                else     { if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<64, true>), pgrid, block, 0, stream, p, static_cast<int>(tiles));
+                           else hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<64, false>), pgrid, block, 0, stream, p, static_cast<int>(tiles)); }
+                return check_launch(what);
+            }
+        }
+        if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_kernel<LOAD_ROW_CONTIG, false, true, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((gemm_bf16x3_kernel<LOAD_ROW_CONTIG, false, false, true>), grid, block, 0, stream, p);
     }
     else if (!p.clamp && !p.f16_in) {
         // binary32 operands without the finite guard: the contraction runs on the bf16 matrix pipe

@@ -773,6 +773,16 @@ __device__ __forceinline__ void q8_linear_ws_body(
         for (int b = 0; b < NBLK; ++b)
             wq[t][b] = *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(col_tile_of(t) * NBLK + b) * 64 + lane) * 16);
     }
+    // fragments of the column tiles that live in LDS: requested now with the rest, parked in registers that
+    // are free until the loop starts, and written to LDS once the first tile has been quantized (requested
+    // only then, their whole way from L2 would lie between the quantizer and the first block step)
+    v4i wl[WL > 0 ? WL : 1][NBLK];
+#pragma unroll
+    for (int t = TPW - WL; t < TPW; ++t) {
+#pragma unroll
+        for (int b = 0; b < NBLK; ++b)
+            wl[t - (TPW - WL)][b] = *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(col_tile_of(t) * NBLK + b) * 64 + lane) * 16);
+    }
     // scales of one column tile: NBLK x 32 halves, contiguous; a lane takes four at a time
     constexpr int DCHUNKS = NBLK * 8;                  // groups of four halves per column tile
     constexpr int DREP = (DCHUNKS + 63) / 64;
@@ -853,8 +863,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
     for (int t = TPW - WL; t < TPW; ++t) {
 #pragma unroll
         for (int b = 0; b < NBLK; ++b)
-            my_wq[((t - (TPW - WL)) * NBLK + b) * 64] =
-                *reinterpret_cast<const v4i*>(W + (static_cast<size_t>(col_tile_of(t) * NBLK + b) * 64 + lane) * 16);
+            my_wq[((t - (TPW - WL)) * NBLK + b) * 64] = wl[t - (TPW - WL)][b];
     }
     // Every weight fragment has arrived before the loop starts: a load still pending here would make
     // its first use inside the loop wait for vmcnt(0), i.e. for all output stores, on every iteration.
@@ -1063,18 +1072,6 @@ void q8_linear_ws64_kernel(const uint8_t* __restrict__ W, const float* __restric
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 96, "staging size");
     q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
-}
-
-int device_cu_count() {
-    static const int cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
-            (void)hipGetLastError();
-            n = 256;
-        }
-        return n;
-    }();
-    return cus;
 }
 
 template <int TPW, int NBLK, int WL, int NW, bool Q81>

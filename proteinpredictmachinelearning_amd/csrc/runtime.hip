@@ -193,6 +193,19 @@ hipMemPool_t workspace_pool() {
     return pools[dev];
 }
 
+// compute units of the device the library first ran on (256 on the part this library is built for)
+int device_cu_count() {
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = 256;
+        }
+        return n;
+    }();
+    return cus;
+}
+
 // which kernel family served the calling thread's last mul_mat_q8 call
 static thread_local int g_q8_path = 0;
 void set_q8_path(int path) { g_q8_path = path; }
