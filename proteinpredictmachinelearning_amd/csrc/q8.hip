@@ -954,26 +954,19 @@ __device__ __forceinline__ void q8_linear_ws_body(
                 // row.  Buffer stores with a bounds-checked offset: lanes past the edge of C pass an
                 // offset beyond the buffer and are dropped by the hardware, so every wave issues
                 // exactly 16 stores here and the memory counter stays predictable.
-                const uint32_t base = (static_cast<uint32_t>(tok0 + 4 * hh) * M + m) * 4u;
-                const uint32_t out_of_range = 0xfffffff0u;
-                // Row pitch through a copy the optimizer cannot trace: the sixteen scalar row offsets are
-                // then rebuilt here (a handful of scalar operations) instead of occupying sixteen
-                // scalar registers for the whole kernel, which has none to spare.
+                // The whole byte offset of a store sits in the vector operand, which is what the hardware checks
+                // against the size of C: rows past the last token lie behind the end of the buffer and drop out
+                // by themselves (the ragged last tile needs no predicates), columns past M start from an offset of
+                // 2^31, which stays outside whatever is added to it (C is below 2^31 bytes, see the launcher).
+                // Stepping the offset costs one add per store; a scalar offset per row would cost none but is not
+                // range-checked, and its sixteen predicates per column tile ran for every tile, ragged or not.
+                uint32_t off = m < M ? (static_cast<uint32_t>(tok0 + 4 * hh) * M + m) * 4u : 0x80000000u;
                 int pitch = M * 4;
-                asm volatile("" : "+s"(pitch));
-                if (tok0 + TILE_TOK <= N) {
-                    const uint32_t b0 = m < M ? base : out_of_range;
+                asm volatile("" : "+s"(pitch));          // one scalar, not sixteen folded row offsets
 #pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[r]), c_rsrc, b0,
-                                                              (8 * (r >> 2) + (r & 3)) * pitch, WS_STORE_AUX);
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const bool ok = m < M && tok0 + mfma32_row(r, lane) < N;
-                        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[r]), c_rsrc, ok ? base : out_of_range,
-                                                              (8 * (r >> 2) + (r & 3)) * pitch, WS_STORE_AUX);
-                    }
+                for (int r = 0; r < 16; ++r) {
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[r]), c_rsrc, off, 0, WS_STORE_AUX);
+                    off += ((r & 3) == 3 ? 5 : 1) * pitch;   // rows 8 * (r / 4) + r % 4 (+ 4 in the upper half-wave)
                 }
             }
         };
