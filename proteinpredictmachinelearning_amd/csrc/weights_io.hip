@@ -16,6 +16,8 @@
 #include <cstring>
 #include <fstream>
 #include <map>
+#include <exception>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -231,13 +233,26 @@ extern "C" int ppml_gguf_save(const char* path, const ppml_gguf_tensor* tensors,
     return RC_OK;
 }
 
+static ppml_gguf_file* gguf_open_checked(const char* path);
+
+// No exception may leave an extern "C" function: a damaged file that asks for more memory than there is
+// ends in a null handle and a message like every other refusal.
 extern "C" ppml_gguf_file* ppml_gguf_open(const char* path) {
+    try {
+        return gguf_open_checked(path);
+    } catch (const std::exception& e) {
+        set_error("ppml_gguf_open: %s: %s", path ? path : "(null)", e.what());
+        return nullptr;
+    }
+}
+
+static ppml_gguf_file* gguf_open_checked(const char* path) {
     if (!path) { set_error("ppml_gguf_open: no path"); return nullptr; }
-    ppml_gguf_file* f = new (std::nothrow) ppml_gguf_file;
+    std::unique_ptr<ppml_gguf_file> owner(new (std::nothrow) ppml_gguf_file);
+    ppml_gguf_file* f = owner.get();                   // released to the caller on success only
     if (!f) { set_error("ppml_gguf_open: out of memory"); return nullptr; }
     const auto fail = [&](const char* why) -> ppml_gguf_file* {
         set_error("ppml_gguf_open: %s: %s", path, why);
-        delete f;
         return nullptr;
     };
     f->in.open(path, std::ios::binary);
@@ -259,7 +274,9 @@ extern "C" ppml_gguf_file* ppml_gguf_open(const char* path) {
     if (r32() != GGUF_MAGIC) return fail("Not a GGUF file");
     if (r32() != GGUF_VERSION) return fail("Wrong version");
     const uint64_t tensor_count = r64(), kv_count = r64();
-    if (!in || tensor_count > f->file_size || kv_count > f->file_size) return fail("truncated header");
+    // a tensor info takes at least 24 bytes (name length, rank, type, offset), a metadata entry at least 13:
+    // counts a file of this size cannot hold are refused before anything is sized by them
+    if (!in || tensor_count > f->file_size / 24 || kv_count > f->file_size / 13) return fail("truncated header");
     for (uint64_t i = 0; i < kv_count; ++i) {
         const std::string key = rstr();
         const uint32_t vtype = r32();
@@ -289,13 +306,18 @@ extern "C" ppml_gguf_file* ppml_gguf_open(const char* path) {
         if (!in || bad_string || nd > 4) return fail("bad tensor info");
         t.dims.resize(nd);
         uint64_t numel = 1;
-        for (uint32_t d = 0; d < nd; ++d) { t.dims[d] = r64(); numel *= t.dims[d]; }
+        bool wrapped = false;
+        for (uint32_t d = 0; d < nd; ++d) {
+            t.dims[d] = r64();
+            wrapped = __builtin_mul_overflow(numel, t.dims[d], &numel) || wrapped;
+        }
+        if (wrapped) return fail("bad tensor info");   // a wrapped element count would pass for a small tensor
         t.type = r32();
         t.offset = r64();
         t.nbytes = tensor_bytes(t.type, numel);
         if (!in) return fail("truncated tensor infos");
     }
-    return f;
+    return owner.release();
 }
 
 extern "C" void ppml_gguf_close(ppml_gguf_file* f) { delete f; }

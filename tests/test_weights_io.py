@@ -294,3 +294,33 @@ def test_q8_0_parameter_is_stored_as_ggml_blocks(W, oracle, tmp_path):
     # rows may not split blocks, and the element count must fill whole blocks
     with pytest.raises(RuntimeError, match="cannot be stored"):
         W.save_gguf([W.QuantizedWeight(raw[:34 * 3], (48, 2))], str(tmp_path / "bad.gguf"))
+
+
+def test_counts_and_dimensions_a_file_cannot_hold_are_refused(W, tmp_path):
+    # a header that claims more tensors than the file could describe, and dimensions whose product wraps around
+    # 2^64 to a small number: both must end in an ordinary refusal (no allocation by the claimed count, no
+    # "small" tensor read from a shape that is not small)
+    import struct
+
+    good = str(tmp_path / "good.gguf")
+    W.save_gguf([np.arange(15, dtype=np.float32).reshape(3, 5)], good, [], [], ["a"], [])
+    blob = bytearray(open(good, "rb").read())
+    assert struct.unpack_from("<Q", blob, 8)[0] == 1               # tensor count sits behind magic and version
+    p = tmp_path / "bad.gguf"
+    huge = bytearray(blob)
+    struct.pack_into("<Q", huge, 8, len(blob) // 8)                # fits "count <= file size", not 24 bytes per tensor
+    p.write_bytes(huge)
+    with pytest.raises(RuntimeError, match="truncated header"):
+        W.GgufFile(str(p))
+    kv = bytearray(blob)
+    struct.pack_into("<Q", kv, 16, len(blob) // 8)
+    p.write_bytes(kv)
+    with pytest.raises(RuntimeError, match="truncated"):
+        W.GgufFile(str(p))
+    # dims [5, 3] -> [2^63, 2]: the element count wraps to 0
+    at = bytes(blob).index(struct.pack("<QQ", 5, 3))
+    wrap = bytearray(blob)
+    struct.pack_into("<QQ", wrap, at, 1 << 63, 2)
+    p.write_bytes(wrap)
+    with pytest.raises(RuntimeError, match="bad tensor info"):
+        W.GgufFile(str(p))
