@@ -116,7 +116,7 @@ int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K,
  *   flags bit 1: quantize X with the Q8_1 rule of quantize_rows_q8_1_hip instead of the Q8_0 rule:
  *                the numbers mul_mat_q8_cuda itself produces (src/cuda/MulMatQ8Kernel.cu:520-527
  *                quantizes activations to Q8_1 and settles with their d).
- *   flags bits 2..5 (PPML_Q8_FLAG_*): restrict the choice among the kernels that serve a Q8_0M weight with
+ *   flags bits 2..7 (PPML_Q8_FLAG_*): restrict the choice among the kernels that serve a Q8_0M weight with
  *                c_trans = 1, all of which give the same bits; for tests and measurements.
  *   xq_dump  (may be NULL): receives the Q8_0 blocks the kernel made of X, [N][K/32] block_q8_0
  *   sums_dump(may be NULL): receives the per-block int32 sums, [(n*M+m)*(K/32)+ib]            */
@@ -126,7 +126,9 @@ enum {
     PPML_Q8_FLAG_NO_LOW_LATENCY = 4,       /* do not take the low-latency kernel */
     PPML_Q8_FLAG_NO_WEIGHT_STATIONARY = 8, /* do not take the weight-stationary kernel */
     PPML_Q8_FLAG_LOW_LATENCY_8 = 16,       /* low-latency kernel with units of 8 tokens wherever it has an instance */
-    PPML_Q8_FLAG_LOW_LATENCY_16 = 32       /* ... of 16 tokens */
+    PPML_Q8_FLAG_LOW_LATENCY_16 = 32,      /* ... of 16 tokens */
+    PPML_Q8_FLAG_COLUMN_PARTS = 64,        /* weight-stationary kernel: work-groups share a token tile, a part of the columns each, wherever there is an instance */
+    PPML_Q8_FLAG_NO_COLUMN_PARTS = 128     /* ... never */
 };
 int mul_mat_q8_ex_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
                       int c_trans, int flags, void *xq_dump, int32_t *sums_dump,

@@ -17,14 +17,17 @@ namespace {
 // Quantizer arithmetic shared by the standalone and the fused kernel.
 // ------------------------------------------------------------------------------------------
 
-// max over each aligned group of 4 lanes (one Q8 block when every lane holds 8 elements)
+// max over each aligned group of 4 lanes (one Q8 block when every lane holds 8 elements) of a value that is
+// not negative and not NaN: such floats order like their bit patterns, and an integer max has no signalling
+// NaN to quiet, so each step is a single v_max_u32 that takes its other operand through DPP
 __device__ __forceinline__ float group4_max(float v) {
-    float o;
-    o = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));  // lane ^ 1
-    v = fmaxf(v, o);
-    o = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));  // lane ^ 2
-    v = fmaxf(v, o);
-    return v;
+    uint32_t b = __float_as_uint(v);
+    uint32_t o;
+    o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b), 0xB1, 0xf, 0xf, false));  // lane ^ 1
+    b = b > o ? b : o;
+    o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b), 0x4E, 0xf, 0xf, false));  // lane ^ 2
+    b = b > o ? b : o;
+    return __uint_as_float(b);
 }
 
 struct BlockQuant {
@@ -71,16 +74,51 @@ __device__ __forceinline__ void group4_first_max(float& a, float& v) {
     }
 }
 
+// amax / 127 in three operations: q0 = a * c with c = RN(1 / 127), the exact remainder r = a - 127 q0 from one
+// fma, q0 + r * c.  Equal to the IEEE quotient for every finite a >= 0, subnormals included (all 2^31 - 2^23
+// values compared on the device); a = +inf gives NaN here and takes the caller's slow path.
+__device__ __forceinline__ float div_by_127(float a) {
+    const float c = 0x1.020408p-7f;
+    const float q0 = a * c;
+    const float r = __builtin_fmaf(-127.0f, q0, a);
+    return __builtin_fmaf(r, c, q0);
+}
+
+// 1 / d in three operations: the hardware's approximation and one Newton step.  Equal to the IEEE reciprocal
+// whenever d and 1 / d are both normal numbers, 2^-126 <= |d| <= 2^126 (all values compared on the device;
+// outside that range the step's own arithmetic underflows).
+__device__ __forceinline__ float rcp_normal(float d) {
+    const float y0 = __builtin_amdgcn_rcpf(d);
+    const float e = __builtin_fmaf(-d, y0, 1.0f);
+    return __builtin_fmaf(e, y0, y0);
+}
+__device__ __forceinline__ bool rcp_normal_ok(float d) {
+    return ((__float_as_uint(d) & 0x7fffffffu) - 0x00800000u) <= (0x7e800000u - 0x00800000u);
+}
+
 // x0,x1 hold elements 8*c4 .. 8*c4+7 of one 32-element block, the 4 lanes of an aligned group hold
 // the whole block.  IEEE division for the scale and its reciprocal, round half away from zero.
 //   Q81 = false: d = amax / 127, clamp to +-127             (include/ppml/QuantBlocks.h:62-79)
 //   Q81 = true : d = vmax / -128 with vmax the signed element of largest magnitude, clamp to
 //                [-128, 127]; *qsum receives this lane's share of the sum of the quants
 //                                                            (include/ppml/QuantBlocks.h:81-111)
-template <bool Q81>
+//   RELU       : the block is max(x, 0).  Nothing is spent on forming it: its largest magnitude is the
+//                signed maximum of x and zero, and the quants of its zeros are made zero by the clamp
+//                (x < 0 lands on the side of zero opposite to the kept elements; NaN converts to 0 either
+//                way, like the 0 that max(NaN, 0) is).
+// The two divisions take the short forms above whenever every block of the wave is in their proven range
+// (an all-zero block counts: its reciprocal is replaced by 0 below), else the compiler's IEEE expansion.
+template <bool Q81, bool RELU = false>
 __device__ __forceinline__ BlockQuant quantize_block_lane(v4f x0, v4f x1, int* qsum = nullptr) {
     float amax = 0.0f, vmax = 0.0f;
-    if (Q81) {
+    if (RELU) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) amax = fmaxf(amax, x0[c]);          // fmaxf drops NaN like std::fmax
+#pragma unroll
+        for (int c = 0; c < 4; ++c) amax = fmaxf(amax, x1[c]);
+        amax = group4_max(amax);
+        vmax = amax;
+    } else if (Q81) {
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
             const float x = c < 4 ? x0[c & 3] : x1[c & 3];
@@ -96,20 +134,51 @@ __device__ __forceinline__ BlockQuant quantize_block_lane(v4f x0, v4f x1, int* q
         for (int c = 0; c < 4; ++c) amax = fmaxf(amax, fabsf(x1[c]));
         amax = group4_max(amax);
     }
-    const float d = Q81 ? ((amax == 0.0f) ? 0.0f : vmax / -128.0f) : amax / 127.0f;
-    const float inv = (Q81 ? d == 0.0f : amax == 0.0f) ? 0.0f : 1.0f / d;
+    float d = Q81 ? vmax * -0x1p-7f : div_by_127(amax);                // the division by -128 is an exact scaling, or a subnormal rounded once either way
+    float inv;
+    const bool zero = amax == 0.0f;
+    const bool fast = __builtin_amdgcn_ballot_w64(!(zero || rcp_normal_ok(d))) == 0;   // wave-uniform
+    if (__builtin_expect(fast, 1)) {
+        inv = rcp_normal(d);
+    } else {
+        d = Q81 ? vmax / -128.0f : amax / 127.0f;
+        inv = 1.0f / d;
+    }
+    if (Q81) {
+        if (zero) d = 0.0f;
+        if (d == 0.0f) inv = 0.0f;
+    } else if (zero) {
+        inv = 0.0f;
+    }
     BlockQuant out;
     out.d_bits = __half_as_ushort(__float2half_rn(d));
     out.d = d;
     int q[8];
+    constexpr int QMIN = Q81 ? -128 : (RELU ? 0 : -127);
+    constexpr int QMAX = (Q81 && RELU) ? 0 : 127;
+    if (!Q81 && fast) {
+        // With d and 1 / d normal, |x * inv| <= 127 (1 + 2^-23)(1 + 2^-24) for every element of the block, which
+        // rounds to at most 127: the clamp has nothing to do.  Under RELU the kept elements are positive, so the
+        // rounding offset needs no sign, and the unsigned conversion turns the others (and NaN) into the 0 they are.
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        q[c] = round_half_away_to_int(x0[c] * inv);
-        q[4 + c] = round_half_away_to_int(x1[c] * inv);
+        for (int c = 0; c < 8; ++c) {
+            const float t = (c < 4 ? x0[c & 3] : x1[c & 3]) * inv;
+            if (RELU) {
+                const float u = t + 0x1.fffffep-2f;
+                unsigned qu;
+                asm("v_cvt_u32_f32 %0, %1" : "=v"(qu) : "v"(u));
+                q[c] = static_cast<int>(qu);
+            } else {
+                q[c] = round_half_away_to_int(t);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            q[c] = round_half_away_to_int((c < 4 ? x0[c & 3] : x1[c & 3]) * inv);
+            q[c] = q[c] > QMAX ? QMAX : (q[c] < QMIN ? QMIN : q[c]);
+        }
     }
-    constexpr int QMIN = Q81 ? -128 : -127;
-#pragma unroll
-    for (int c = 0; c < 8; ++c) q[c] = q[c] > 127 ? 127 : (q[c] < QMIN ? QMIN : q[c]);
     if (Q81 && qsum) *qsum = q[0] + q[1] + q[2] + q[3] + q[4] + q[5] + q[6] + q[7];
     out.q_lo = pack4(q[0], q[1], q[2], q[3]);
     out.q_hi = pack4(q[4], q[5], q[6], q[7]);
@@ -314,6 +383,7 @@ constexpr int TILE_TOK = 32;
 // written once and not read again by this kernel; streaming stores measured 15 % faster end to
 // end than default ones at the MSA QKV shape (the same hint on the activation loads costs 4 %).
 constexpr int WS_STORE_AUX = 3;
+constexpr int WS_MAGIC_BITS = 0x4B400000;   // binary32 1.5 * 2^23: accumulator start of the int8 MFMAs whose sums are read as floats
 constexpr int WS_NBUF = 3;          // quantized activation tiles the weight-stationary kernel keeps in LDS
 constexpr int KC_MAX = 56;          // blocks of K staged in LDS at once (63 KiB)
 constexpr int UB = 4;               // quantizer units (8 rows x 2 blocks) a wave keeps in flight
@@ -456,12 +526,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
                     if (u >= units) break;             // wave-uniform
                     const int row = (u & 3) * 8 + urow;
                     const int bl = (u >> 2) * 2 + ublk;
-                    v4f x0 = xv[s][0], x1 = xv[s][1];
-                    if (relu & 1) {
-#pragma unroll
-                        for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
-                    }
-                    const BlockQuant bq = (relu & 2) ? quantize_block_lane<true>(x0, x1) : quantize_block_lane<false>(x0, x1);
+                    const v4f x0 = xv[s][0], x1 = xv[s][1];
+                    const BlockQuant bq = (relu & 2) ? ((relu & 1) ? quantize_block_lane<true, true>(x0, x1) : quantize_block_lane<true, false>(x0, x1))
+                                                     : ((relu & 1) ? quantize_block_lane<false, true>(x0, x1) : quantize_block_lane<false, false>(x0, x1));
                     if (bl < nb) {
                         // fragment order: block bl, k-half c4/2, row, dword pair c4%2
                         uint2* dst = reinterpret_cast<uint2*>(lds_a) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
@@ -622,7 +689,7 @@ constexpr int ws_staging_regs(int nblk, int nw = 8) {   // 8 registers per unit 
 }
 constexpr int ws_compiler_vgprs(int nblk, int nw = 8) { return 256 - ws_staging_regs(nblk, nw); }
 
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT>
 __device__ __forceinline__ void q8_linear_ws_body(
     const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
     int M, int N, int ntiles, int npart, int relu,
@@ -744,10 +811,23 @@ __device__ __forceinline__ void q8_linear_ws_body(
     // tiles left over by whole rounds are few enough -- one more tile of which it computes a single
     // column tile per wave (tile ntiles + blockIdx / TPW, column part blockIdx % TPW), so that TPW
     // work-groups share each leftover tile instead of a few work-groups running a whole extra round.
-    const int grid = static_cast<int>(gridDim.x);
-    const int wg = static_cast<int>(blockIdx.x);
+    // CSPLIT: the columns are cut into `npart` parts of NW * TPW column tiles and `npart` work-groups share each
+    // token tile, one part each.  A work-group then keeps a fraction of the weight (a start-up that is as
+    // much shorter) and reads every tile of its group; the members of a group run on one XCD wherever the
+    // grid allows (work-groups go to the XCDs in turn), so the tile comes from memory once and from that
+    // XCD's L2 for the others.
+    int grid = static_cast<int>(gridDim.x);
+    int wg = static_cast<int>(blockIdx.x);
+    int ct0 = 0;                                       // first column tile of this work-group's part
+    if (CSPLIT) {
+        const int vid = (grid & 7) == 0 ? (wg & 7) * (grid >> 3) + (wg >> 3) : wg;
+        const int group = vid / npart;
+        ct0 = (vid - group * npart) * (NW * TPW);
+        grid = grid / npart;
+        wg = group < grid ? group : ntiles;            // work-groups beyond the last whole group have no tile
+    }
     const int n_full = wg < ntiles ? (ntiles - wg + grid - 1) / grid : 0;
-    const bool has_part = wg < npart;
+    const bool has_part = !CSPLIT && wg < npart;
     const int n_iter = n_full + (has_part ? 1 : 0);
     const int part_col = wg % TPW;
     auto tile_of = [&](int i) { return i < n_full ? wg + i * grid : ntiles + wg / TPW; };
@@ -764,7 +844,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
     v4i* my_wq = lds_wq + static_cast<size_t>(wave) * WL * NBLK * 64 + lane;
     uint2* my_wd = lds_wd + static_cast<size_t>(wave) * TPW * NBLK * 32 + lane;
     auto col_tile_of = [&](int t) {
-        const int ct = t * NW + wave;                  // round t of the waves covers NW adjacent column tiles
+        const int ct = ct0 + t * NW + wave;            // round t of the waves covers NW adjacent column tiles
         return ct < mct_pad ? ct : mct_pad - 1;        // tiles past the end repeat the last one; never stored
     };
 #pragma unroll
@@ -812,12 +892,8 @@ __device__ __forceinline__ void q8_linear_ws_body(
             if (u >= NUNITS) break;                    // wave-uniform
             const int row = (u & 3) * 8 + urow;
             const int bl = (u >> 2) * 2 + ublk;
-            v4f x0 = xv[s][0], x1 = xv[s][1];
-            if (relu & 1) {
-#pragma unroll
-                for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
-            }
-            const BlockQuant bq = quantize_block_lane<Q81>(x0, x1);
+            const v4f x0 = xv[s][0], x1 = xv[s][1];
+            const BlockQuant bq = (relu & 1) ? quantize_block_lane<Q81, true>(x0, x1) : quantize_block_lane<Q81, false>(x0, x1);
             uint2* dst = reinterpret_cast<uint2*>(lds_a[buf]) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
             *dst = uint2{bq.q_lo, bq.q_hi};
             if (c4 == 0) lds_d[buf][bl * 32 + row] = uint2{bq.d_bits, 0u};
@@ -881,6 +957,23 @@ __device__ __forceinline__ void q8_linear_ws_body(
     constexpr int NEWER_FIRST = 16 * (QSTEP / NBLK) < 63 ? 16 * (QSTEP / NBLK) : 63;
     constexpr int NEWER = 16 * TPW < 63 ? 16 * TPW : 63;
 
+    // Block sums leave the matrix pipe as floats.  An int8 MFMA that starts from the bit pattern of
+    // 1.5 * 2^23 instead of zero returns, read as binary32, exactly 1.5 * 2^23 + sum (|sum| <= 32 * 128 * 128
+    // stays inside that binade, where one unit in the last place is one); a bf16 MFMA whose only non-zero
+    // products are (-0.75 * 2^23) * 1 in k slots 0 and 4 then takes the offset off again, exactly, since
+    // float(sum) is representable.  This replaces one v_cvt_f32_i32 per output and block on the vector
+    // pipe, which is what bounds this kernel, by 8 passes of the matrix pipe, which has the slack.
+    // The constants are hidden from the optimizer so that they stay in registers instead of being
+    // rebuilt in front of every MFMA.
+    v16i magic_i;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) magic_i[r] = WS_MAGIC_BITS;
+    asm volatile("" : "+v"(magic_i));
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    v4s unbias_a = {static_cast<short>(0xCAC0), 0, 0, 0};   // bf16 -0.75 * 2^23
+    v4s unbias_b = {static_cast<short>(0x3F80), 0, 0, 0};   // bf16 1
+    asm volatile("" : "+v"(unbias_a), "+v"(unbias_b));
+
     // No barrier inside the loop.  A wave may start tile `it` once all waves have announced it, which
     // also means all of them are past two thirds of tile it-1; the tile quantized during tile `it`
     // goes to buffer (it+1) % 3, last read for tile it-2, which every wave has left by then.
@@ -894,10 +987,6 @@ __device__ __forceinline__ void q8_linear_ws_body(
         await_tile(buf, static_cast<unsigned>(NW) * static_cast<unsigned>(it / WS_NBUF + 1));
 
         // ---------------- MFMA one block ahead of the settle; tiles in turn, blocks ascending
-        v16i zero_i;
-        v16f zero_f;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) { zero_i[r] = 0; zero_f[r] = 0.0f; }
         // Per pair of blocks: two int8 MFMAs (exact block sums, one result buffer per parity) and one
         // v_mfma_f32_32x32x4_2b_f16 whose two 32x32 outer products are the scale tables
         // d_a[row] * d_w[col] of both blocks: the scale sits in the first of a lane's four k slots and
@@ -930,23 +1019,27 @@ __device__ __forceinline__ void q8_linear_ws_body(
         auto block_sum = [&](int st, const v4i& a, const v4i& w_lds) {
             const int t = st / NBLK, b = st % NBLK;
             const v4i w = t < TPW - WL ? wq[t < TPW - WL ? t : 0][b] : w_lds;
-            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, w, zero_i, 0, 0, 0);
+            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, w, magic_i, 0, 0, 0);
         };
-        auto settle = [&](int st, const v16i& sum, const v16f scl) {
+        // 1.5 * 2^23 + sum -> float(sum), on the matrix pipe
+        auto to_float = [&](const v16i& biased) {
+            return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(unbias_a, unbias_b, __builtin_bit_cast(v16f, biased), 0, 0, 0);
+        };
+        auto settle = [&](int st, const v16f& sum, const v16f scl) {
             const int t = st / NBLK, b = st % NBLK;
             if (b == 0) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(static_cast<float>(sum[r]), scl[r], 0.0f);
+                for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(sum[r], scl[r], 0.0f);
             } else {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(static_cast<float>(sum[r]), scl[r], acc[r]);
+                for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(sum[r], scl[r], acc[r]);
             }
-            const int m = (t * NW + wave) * 32 + j;    // this lane's output feature
+            const int m = (ct0 + t * NW + wave) * 32 + j;   // this lane's output feature
             if (DUMP && sums_dump) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int tok = tok0 + mfma32_row(r, lane);
-                    if (tok < N && m < M) sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b] = sum[r];
+                    if (tok < N && m < M) sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b] = static_cast<int>(sum[r]);
                 }
             }
             if (b == NBLK - 1) {
@@ -1008,27 +1101,31 @@ __device__ __forceinline__ void q8_linear_ws_body(
                 if constexpr (TWO_SETS) {
                     PairOps& cur = (pr & 1) ? po : pe;
                     PairOps& nxt = (pr & 1) ? pe : po;
+                    const v16f flt_a = to_float(sum_a);
                     scl = scale_tables(cur.da, cur.dw);
                     sum_b = block_sum(st + 1, cur.a1, cur.w1);
                     __builtin_amdgcn_sched_barrier(0);
-                    settle(st, sum_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
+                    settle(st, flt_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
                     __builtin_amdgcn_sched_barrier(0);
+                    const v16f flt_b = to_float(sum_b);
                     if (2 * pr + 2 < NBLK) sum_a = block_sum(st + 2, nxt.a0, nxt.w0);
                     if (2 * pr + 4 < NBLK) fetch_pair(st + 4, cur);
                     __builtin_amdgcn_sched_barrier(0);
-                    settle(st + 1, sum_b, __builtin_shufflevector(scl, scl, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31));
+                    settle(st + 1, flt_b, __builtin_shufflevector(scl, scl, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31));
                     __builtin_amdgcn_sched_barrier(0);
                 } else {
                     // one block sum alive at a time; the other wave of the SIMD fills the waits
-                    scl = scale_tables(pe.da, pe.dw);
                     sum_a = block_sum(st, pe.a0, pe.w0);
+                    scl = scale_tables(pe.da, pe.dw);
+                    const v16f flt_a = to_float(sum_a);
                     __builtin_amdgcn_sched_barrier(0);
-                    settle(st, sum_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
+                    settle(st, flt_a, __builtin_shufflevector(scl, scl, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15));
                     __builtin_amdgcn_sched_barrier(0);
                     sum_a = block_sum(st + 1, pe.a1, pe.w1);
                     if (2 * pr + 2 < NBLK) fetch_pair(st + 2, pe);
+                    const v16f flt_b = to_float(sum_a);
                     __builtin_amdgcn_sched_barrier(0);
-                    settle(st + 1, sum_a, __builtin_shufflevector(scl, scl, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31));
+                    settle(st + 1, flt_b, __builtin_shufflevector(scl, scl, 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31));
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -1041,35 +1138,35 @@ __device__ __forceinline__ void q8_linear_ws_body(
 // value counts architectural and accumulation registers separately): 120 keeps it below v240.  A
 // value the compiler does not honour would go unnoticed until its registers and the staged tile
 // collide, so the build checks the generated code (check_ws_isa.py).
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(120)))
 void q8_linear_ws_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                          int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                          int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 120, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(112)))
 void q8_linear_ws32_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 112, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(96)))
 void q8_linear_ws64_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 96, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
-template <int TPW, int NBLK, int WL, int NW, bool Q81>
+template <int TPW, int NBLK, int WL, int NW, bool Q81, bool CSPLIT = false>
 int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int relu,
-                        void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
+                        void* xq_dump, int32_t* sums_dump, hipStream_t stream, int cparts = 1) {
     // Eight waves fill a CU (256 registers each): one resident work-group of 8 waves per CU, or two
     // of 4.  With more tiles than resident work-groups every work-group takes the same number of
     // tiles (824 tiles on 256 CUs: 206 work-groups x 4 rather than 256 x 3 + 56 x 1).
@@ -1077,7 +1174,11 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
     const int all_tiles = (N + TILE_TOK - 1) / TILE_TOK;
     int wgs, ntiles = all_tiles, npart = 0;
     const int left = all_tiles % cus;
-    if (all_tiles > cus && left > 0 && left * TPW <= cus && TPW > 1) {
+    if (CSPLIT) {
+        // one work-group per CU; `cparts` of them share a token tile, a column part each
+        wgs = cus;
+        npart = cparts;
+    } else if (all_tiles > cus && left > 0 && left * TPW <= cus && TPW > 1) {
         // whole rounds on every CU, then the leftover tiles shared by TPW work-groups each
         wgs = cus;
         ntiles = all_tiles - left;
@@ -1092,15 +1193,15 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
     using KernelFn = void (*)(const uint8_t*, const float*, float*, int, int, int, int, int, uint8_t*, int32_t*);
     KernelFn fast, dump;
     if constexpr (ws_staging_regs(NBLK, NW) == 16) {
-        fast = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81>;
-        dump = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true, Q81>;
+        fast = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81, CSPLIT>;
+        dump = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true, Q81, CSPLIT>;
     } else if constexpr (ws_staging_regs(NBLK, NW) == 32) {
-        fast = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, false, Q81>;
-        dump = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, true, Q81>;
+        fast = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, false, Q81, CSPLIT>;
+        dump = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, true, Q81, CSPLIT>;
     } else {
         static_assert(ws_staging_regs(NBLK, NW) == 64, "no kernel for this staging size");
-        fast = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, false, Q81>;
-        dump = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, true, Q81>;
+        fast = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, false, Q81, CSPLIT>;
+        dump = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, true, Q81, CSPLIT>;
     }
     if (lds > 64 * 1024) {
         static const hipError_t attr_fast = hipFuncSetAttribute(
@@ -1122,13 +1223,29 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
 }
 
 // returns -1 when the shape has no weight-stationary instance
+// `csplit`: -1 never, 1 wherever there is an instance, 0 by the gate below
 template <bool Q81>
 int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
-                     int relu, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
+                     int relu, int csplit, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
     if (!c_trans) return -1;
     if (static_cast<int64_t>(N) * M * 4 >= 0x7fff0000LL) return -1;   // the kernel addresses C with 32-bit byte offsets
     const int mct = (M + 31) / 32;
     const int tpw = (mct + 7) / 8;
+    // Column parts: `tpw` work-groups of the one-column-tile-per-wave instance share each token tile.  Every
+    // work-group then quantizes the whole tile for a `tpw`-th of the columns, which costs more than the shorter
+    // start-up saves except where the whole-width instance is short of registers and LDS (measured, us, parts /
+    // whole: 26368 x 256 -> 768  23.8 / 22.2;  10609 x 128 -> 512  6.8 / 6.3;  26368 x 128 -> 1024  20.1 / 25.1).
+    if (tpw > 1 && csplit >= 0) {
+        const int cus = device_cu_count();
+        const int tiles = (N + TILE_TOK - 1) / TILE_TOK;
+        const bool take = csplit > 0 || (tpw == 4 && tiles >= 3 * cus);
+        if (take && cus >= tpw) {
+#define PPML_WSC(NBLK) return launch_q8_linear_ws<1, NBLK, 0, 8, Q81, true>(W, X, C, M, N, relu, xq_dump, sums_dump, stream, tpw)
+            if (nblk == 4) PPML_WSC(4);
+            if (nblk == 8) PPML_WSC(8);
+#undef PPML_WSC
+        }
+    }
 #define PPML_WS(TPW, NBLK, WL, NW) return launch_q8_linear_ws<TPW, NBLK, WL, NW, Q81>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
     // Up to four column tiles: work-groups of four waves, one column tile each and two per CU, so no
     // wave idles (with eight waves half of them would have no column tile).
@@ -1240,12 +1357,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         if (u >= NUNITS) break;                        // wave-uniform
         const int row = (u % (TOK / 8)) * 8 + urow;
         const int bl = (u / (TOK / 8)) * 2 + ublk;
-        v4f x0 = xv[s][0], x1 = xv[s][1];
-        if (relu) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) { x0[c] = fmaxf(x0[c], 0.0f); x1[c] = fmaxf(x1[c], 0.0f); }
-        }
-        const BlockQuant bq = quantize_block_lane<Q81>(x0, x1);
+        const v4f x0 = xv[s][0], x1 = xv[s][1];
+        const BlockQuant bq = relu ? quantize_block_lane<Q81, true>(x0, x1) : quantize_block_lane<Q81, false>(x0, x1);
         uint2* dst = reinterpret_cast<uint2*>(lds_a) + ((bl * 64 + (c4 >> 1) * 32 + row) * 2 + (c4 & 1));
         *dst = uint2{bq.q_lo, bq.q_hi};
         if (c4 == 0) lds_d[bl * 32 + row] = uint2{bq.d_bits, 0u};
@@ -1261,11 +1374,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         for (int pr = 0; pr < NBLK / 2; ++pr) my_wd[(t * (NBLK / 2) + pr) * 64] = wd[t][pr];   // written and read by this wave only
     __syncthreads();
 
-    // ---- column tiles of this wave, blocks ascending
-    v16i zero_i;
+    // ---- column tiles of this wave, blocks ascending.  The block sums come out of the matrix pipe as floats
+    // (see the weight-stationary kernel: int8 MFMA started from 1.5 * 2^23, offset taken off by a bf16 MFMA).
+    v16i magic_i;
     v32f zero_f;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) zero_i[r] = 0;
+    for (int r = 0; r < 16; ++r) magic_i[r] = WS_MAGIC_BITS;
+    asm volatile("" : "+v"(magic_i));
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    v4s unbias_a = {static_cast<short>(0xCAC0), 0, 0, 0};   // bf16 -0.75 * 2^23, in k slots 0 and 4
+    v4s unbias_b = {static_cast<short>(0x3F80), 0, 0, 0};   // bf16 1
+    asm volatile("" : "+v"(unbias_a), "+v"(unbias_b));
 #pragma unroll
     for (int r = 0; r < 32; ++r) zero_f[r] = 0.0f;
     typedef _Float16 v4h __attribute__((ext_vector_type(4)));
@@ -1289,24 +1408,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             const v4i a1 = lds_a[(b + 1) * 64 + lane];
             const uint2 da = lds_d[b * 32 + lane];     // lanes 0..31: rows of block b, 32..63: of block b + 1
             const uint2 dw = uint2{my_wd[(t * (NBLK / 2) + pr) * 64], 0u};
-            // one block sum alive at a time (the waves sharing the SIMD fill the waits): scale tables and the
-            // first sum, settle it, second sum, settle it
+            // scale tables, both block sums and their conversions at once (the waves sharing the SIMD fill the
+            // wait), then both settlements
             const v32f scl = __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, da), __builtin_bit_cast(v4h, dw), zero_f, 0, 0, 0);
-            const v16i s0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, wq[t][b], zero_i, 0, 0, 0);
+            const v16i b0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, wq[t][b], magic_i, 0, 0, 0);
+            const v16i b1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, wq[t][b + 1], magic_i, 0, 0, 0);
+            const v16f s0 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(unbias_a, unbias_b, __builtin_bit_cast(v16f, b0), 0, 0, 0);
+            const v16f s1 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(unbias_a, unbias_b, __builtin_bit_cast(v16f, b1), 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(static_cast<float>(s0[r]), scl[r], pr == 0 ? 0.0f : acc[r]);
-            const v16i s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, wq[t][b + 1], zero_i, 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
+            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(s0[r], scl[r], pr == 0 ? 0.0f : acc[r]);
 #pragma unroll
-            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(static_cast<float>(s1[r]), scl[16 + r], acc[r]);
+            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(s1[r], scl[16 + r], acc[r]);
             if (DUMP && sums_dump) {
 #pragma unroll
                 for (int r = 0; r < RV; ++r) {
                     const int tok = tok0 + mfma32_row(r, lane);
                     if (tok < N && m < M) {
-                        sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b] = s0[r];
-                        sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b + 1] = s1[r];
+                        sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b] = static_cast<int>(s0[r]);
+                        sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b + 1] = static_cast<int>(s1[r]);
                     }
                 }
             }
@@ -1455,9 +1575,10 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
                          : (act & 2) ? try_q8_linear_ll<true>(W, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s)
                                      : try_q8_linear_ll<false>(W, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s);
             if (rl >= 0) { set_q8_path(PPML_Q8_PATH_LOW_LATENCY); stat.set_path("hip/q8-low-latency"); return rl; }
+            const int csplit = (flags & PPML_Q8_FLAG_COLUMN_PARTS) ? 1 : (flags & PPML_Q8_FLAG_NO_COLUMN_PARTS) ? -1 : 0;
             const int rc = (flags & PPML_Q8_FLAG_NO_WEIGHT_STATIONARY) ? -1
-                         : (act & 2) ? try_q8_linear_ws<true>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s)
-                                     : try_q8_linear_ws<false>(W, X, C, M, N, nblk, c_trans, relu, xq_dump, sums_dump, s);
+                         : (act & 2) ? try_q8_linear_ws<true>(W, X, C, M, N, nblk, c_trans, relu, csplit, xq_dump, sums_dump, s)
+                                     : try_q8_linear_ws<false>(W, X, C, M, N, nblk, c_trans, relu, csplit, xq_dump, sums_dump, s);
             if (rc >= 0) { set_q8_path(PPML_Q8_PATH_WEIGHT_STATIONARY); stat.set_path("hip/q8-weight-stationary"); return rc; }
             return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         }

@@ -80,6 +80,58 @@ def test_quantize_ties_and_nan_block(ops, oracle):
     assert list(got[0, 0, 2:11].view(np.int8)) == [127, 1, -1, 2, -2, 3, -3, 0, 0]
 
 
+def _exponent_sweep_blocks(seed):
+    """One 32-element block per (largest-magnitude exponent, mantissa draw): every binary32 exponent from the
+    subnormals to the top, so that the scale d = amax / 127 and its reciprocal pass through their subnormal,
+    normal and overflowing ranges; the other elements are random fractions of the largest one, of either sign."""
+    rng = np.random.default_rng(seed)
+    exps = np.arange(0, 255, dtype=np.uint32)
+    mant = rng.integers(0, 1 << 23, size=(exps.size, 24), dtype=np.uint32)
+    mant[:, 0], mant[:, 1] = 0, (1 << 23) - 1
+    top = ((exps[:, None] << 23) | mant).view(np.float32).reshape(-1)              # 255 * 24 largest magnitudes
+    frac = rng.uniform(-1.0, 1.0, size=(top.size, 32)).astype(np.float32)
+    x = (frac.astype(np.float64) * top[:, None].astype(np.float64)).astype(np.float32)
+    pos = rng.integers(0, 32, size=top.size)
+    x[np.arange(top.size), pos] = top * rng.choice(np.array([-1.0, 1.0], dtype=np.float32), size=top.size)
+    x[5] = 0.0                                                                      # an all-zero block among them
+    return x
+
+
+def test_quantizers_over_the_whole_exponent_range(ops, oracle):
+    # the scale and its reciprocal take a short exact form where both are normal numbers and the IEEE expansion
+    # elsewhere: bytes and scales of both rules over every exponent the largest element can have
+    x = _exponent_sweep_blocks(77)
+    rows = x.shape[0]
+    got0 = ops.quantize_rows_q8_0(_dev(x)).cpu().numpy()
+    want0 = oracle.quantize_q8_0(x)
+    assert (got0 == want0).all(), f"{(got0 != want0).any(axis=(1, 2)).sum()} of {rows} blocks differ (Q8_0 rule)"
+    got1 = ops.quantize_rows_q8_1(_dev(x)).cpu().numpy()
+    want1 = oracle.quantize_q8_1(x)
+    assert (got1 == want1).all(), f"{(got1 != want1).any(axis=(1, 2)).sum()} of {rows} blocks differ (Q8_1 rule)"
+
+
+@pytest.mark.parametrize("act", ["q8_0", "q8_1"])
+@pytest.mark.parametrize("fam", ["general", "weight-stationary", "low-latency-8", "low-latency-16"])
+def test_relu_quantizer_over_the_whole_exponent_range(ops, oracle, act, fam):
+    # ReLU in front of the quantizer costs nothing in the kernels (signed maximum, clamp at zero): the blocks they
+    # make of x must be the blocks of max(x, 0) under both rules, over every exponent, in every kernel family
+    blocks = _exponent_sweep_blocks(78)
+    K = 128
+    x = blocks[: (blocks.shape[0] // 4) * 4].reshape(-1, K)
+    _, w = _inputs(5, 1, K, 64)
+    W = ops.Q8Weight.from_f32(_dev(w)).pack()
+    for relu in (True, False):
+        _, xq, _ = ops.mul_mat_q8(W, _dev(x), relu=relu, dump=True, act=act, path=fam)
+        xr = np.maximum(x, 0.0) if relu else x
+        if act == "q8_0":
+            want = oracle.quantize_q8_0(xr)
+        else:
+            x1 = oracle.quantize_q8_1(xr)
+            want = np.ascontiguousarray(np.concatenate([x1[..., 0:2], x1[..., 4:]], axis=-1))
+        got = xq.cpu().numpy()
+        assert (got == want).all(), f"relu={relu}: {(got != want).any(axis=2).sum()} of {want.shape[0] * want.shape[1]} blocks differ"
+
+
 def test_dequantize_matches_oracle(ops, oracle):
     x, _ = _inputs(3, 17, 96, 1)
     blk = oracle.quantize_q8_0(x)
@@ -170,12 +222,14 @@ def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packe
     # a packed weight: every kernel family that has an instance for the shape, dump form and fast form
     families = ["general"]
     if _has_resident_weight_instance(K, M):
-        families.append("weight-stationary")
+        families += ["weight-stationary", "weight-stationary-whole"]
+    if _has_column_parts_instance(K, M):
+        families.append("weight-stationary-column-parts")
     if _has_low_latency_instance(K, M):
         families += ["low-latency-8", "low-latency-16"]
     for fam in families:
         o2, xq2, sums2 = ops.mul_mat_q8(W, _dev(x), c_trans=1, dump=True, path=fam)
-        assert ops.last_q8_path() == fam.rsplit("-", 1)[0] if fam.startswith("low") else ops.last_q8_path() == fam, fam
+        assert ops.last_q8_path() == _FAMILY_PATH[fam], fam
         assert (o2.cpu().numpy() == want).all() and (xq2.cpu().numpy() == xq_want).all() and (sums2.cpu().numpy() == sums).all(), fam
         assert (ops.mul_mat_q8(W, _dev(x), c_trans=1, path=fam).cpu().numpy() == want).all(), fam
     # the library's own choice: low-latency for few tokens, else weight-stationary, else general
@@ -192,6 +246,17 @@ def _has_resident_weight_instance(K, M):
     tiles, nblk = (M + 31) // 32, K // 32
     tpw = (tiles + 7) // 8
     return K % 32 == 0 and nblk in (4, 8, 16) and (tiles <= 4 or tpw <= {4: 4, 8: 3, 16: 1}[nblk])
+
+
+_FAMILY_PATH = {"general": "general", "weight-stationary": "weight-stationary", "weight-stationary-whole": "weight-stationary",
+                "weight-stationary-column-parts": "weight-stationary", "low-latency-8": "low-latency", "low-latency-16": "low-latency"}
+
+
+def _has_column_parts_instance(K, M):
+    # several column tiles per wave, K of 128 or 256: that many work-groups can share a token tile, a part of
+    # the columns each
+    tiles, nblk = (M + 31) // 32, K // 32
+    return K % 32 == 0 and nblk in (4, 8) and tiles > 8 and _has_resident_weight_instance(K, M)
 
 
 def _has_low_latency_instance(K, M):
@@ -359,10 +424,12 @@ def test_fused_linear_with_q8_1_activations(ops, oracle, wname, N, K, M, c_trans
     # a packed weight in the LinearLayer orientation gets the resident-weight kernels under this rule too
     assert (ops.last_q8_path() != "general") == (wname == "packed" and c_trans == 1)
     if wname == "packed" and c_trans == 1:
-        for fam in ("weight-stationary", "low-latency-8", "low-latency-16"):
+        for fam in ("weight-stationary", "weight-stationary-column-parts", "low-latency-8", "low-latency-16"):
             if fam.startswith("low") and not _has_low_latency_instance(K, M):
                 continue
+            if fam.endswith("parts") and not _has_column_parts_instance(K, M):
+                continue
             y3 = ops.mul_mat_q8(W, _dev(x), c_trans=1, act="q8_1", path=fam).cpu().numpy()
-            assert ops.last_q8_path() == fam.rsplit("-", 1)[0] if fam.startswith("low") else ops.last_q8_path() == fam
+            assert ops.last_q8_path() == _FAMILY_PATH[fam]
             assert (y3 == want).all(), fam
     assert (ops.mul_mat_q8(W, _dev(x), c_trans=c_trans).cpu().numpy() != want).any()
