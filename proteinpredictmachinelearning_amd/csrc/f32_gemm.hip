@@ -1061,7 +1061,8 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
         else                              { if (split) PPML_LAUNCH_BF16(LOAD_STRIDED, true);    else PPML_LAUNCH_BF16(LOAD_STRIDED, false); }
     }
     else if (p.clamp) {
-        if (split || p.stream_c || p.f16_in) { set_error("%s: no clamped instance for this addressing", what); return RC_BAD_ARGS; }
+        if (split || p.f16_in) { set_error("%s: no clamped instance for this addressing", what); return RC_BAD_ARGS; }
+        p.stream_c = 0;                                // (the clamped instances store the ordinary way, whatever the size)
         if (mode == LOAD_K_CONTIG) hipLaunchKernelGGL((gemm_f32_kernel<LOAD_K_CONTIG, false, false, true>), grid, block, 0, stream, p);
         else if (mode == LOAD_ROW_CONTIG) hipLaunchKernelGGL((gemm_f32_kernel<LOAD_ROW_CONTIG, false, false, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((gemm_f32_kernel<LOAD_STRIDED, false, false, true>), grid, block, 0, stream, p);

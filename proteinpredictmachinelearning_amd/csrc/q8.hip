@@ -1374,20 +1374,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         for (int pr = 0; pr < NBLK / 2; ++pr) my_wd[(t * (NBLK / 2) + pr) * 64] = wd[t][pr];   // written and read by this wave only
     __syncthreads();
 
-    // ---- column tiles of this wave, blocks ascending.  The block sums come out of the matrix pipe as floats
-    // (see the weight-stationary kernel: int8 MFMA started from 1.5 * 2^23, offset taken off by a bf16 MFMA).
-    v16i magic_i;
+    // ---- column tiles of this wave, blocks ascending.  (The block sums are converted on the vector pipe here: the
+    // matrix-pipe conversion of the weight-stationary kernel costs twenty registers, which this kernel, at three
+    // waves per SIMD, spends on the operands fetched ahead instead; measured equal at 10609 x 512 -> 128 and
+    // better on the few-token shapes.)
     v32f zero_f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) magic_i[r] = WS_MAGIC_BITS;
-    asm volatile("" : "+v"(magic_i));
-    typedef short v4s __attribute__((ext_vector_type(4)));
-    v4s unbias_a = {static_cast<short>(0xCAC0), 0, 0, 0};   // bf16 -0.75 * 2^23, in k slots 0 and 4
-    v4s unbias_b = {static_cast<short>(0x3F80), 0, 0, 0};   // bf16 1
-    asm volatile("" : "+v"(unbias_a), "+v"(unbias_b));
 #pragma unroll
     for (int r = 0; r < 32; ++r) zero_f[r] = 0.0f;
     typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    // LDS operands of one pair of blocks.  They are fetched a pair ahead, under the matrix work of the pair in hand:
+    // with the work-groups of a CU at different stages the LDS round trip used to be covered by other waves, but the
+    // work-groups whose activations arrive last run alone, and their chain of pairs is what the kernel ends on
+    // (per-wave time stamps: 2.1 us for the sixteen blocks of the pair feed-forward down-projection).
+    struct PairOps { v4i a0, a1; uint2 da, dw; };
+    const auto fetch = [&](int t, int pr, PairOps& o) {
+        const int b = 2 * pr;
+        o.a0 = lds_a[b * 64 + lane];
+        o.a1 = lds_a[(b + 1) * 64 + lane];
+        o.da = lds_d[b * 32 + lane];                   // lanes 0..31: rows of block b, 32..63: of block b + 1
+        o.dw = uint2{my_wd[(t * (NBLK / 2) + pr) * 64], 0u};
+    };
+    PairOps ops_even, ops_odd;                          // pairs take them in turn, by name
+    fetch(0, 0, ops_even);
 #pragma unroll
     for (int t = 0; t < CPW; ++t) {
         // one basic block per column tile (see opaque_one()), and scheduling fences between the pairs inside
@@ -1404,22 +1412,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             // under register pressure it has put every MFMA first and spilled their results
             if (!opaque_one()) continue;
             const int b = 2 * pr;
-            const v4i a0 = lds_a[b * 64 + lane];
-            const v4i a1 = lds_a[(b + 1) * 64 + lane];
-            const uint2 da = lds_d[b * 32 + lane];     // lanes 0..31: rows of block b, 32..63: of block b + 1
-            const uint2 dw = uint2{my_wd[(t * (NBLK / 2) + pr) * 64], 0u};
-            // scale tables, both block sums and their conversions at once (the waves sharing the SIMD fill the
-            // wait), then both settlements
-            const v32f scl = __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, da), __builtin_bit_cast(v4h, dw), zero_f, 0, 0, 0);
-            const v16i b0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, wq[t][b], magic_i, 0, 0, 0);
-            const v16i b1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, wq[t][b + 1], magic_i, 0, 0, 0);
-            const v16f s0 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(unbias_a, unbias_b, __builtin_bit_cast(v16f, b0), 0, 0, 0);
-            const v16f s1 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(unbias_a, unbias_b, __builtin_bit_cast(v16f, b1), 0, 0, 0);
+            const int q = t * (NBLK / 2) + pr;          // pairs in the order they are taken
+            PairOps& cur = (q & 1) ? ops_odd : ops_even;
+            PairOps& nxt = (q & 1) ? ops_even : ops_odd;
+            if (pr + 1 < NBLK / 2) fetch(t, pr + 1, nxt);
+            else if (t + 1 < CPW) fetch(t + 1, 0, nxt);
+            // both block sums and the scale tables at once; the settlements follow as their operands complete
+            v16i zero_i;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) zero_i[r] = 0;
+            v16i s0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.a0, wq[t][b], zero_i, 0, 0, 0);
+            v32f scl = __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, cur.da), __builtin_bit_cast(v4h, cur.dw), zero_f, 0, 0, 0);
+            v16i s1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(cur.a1, wq[t][b + 1], zero_i, 0, 0, 0);
+            // all three are issued before the first settlement: the empty statement needs their results, and
+            // instruction selection, which places pure arithmetic where it likes, cannot move it
+            asm volatile("" : "+v"(s0), "+v"(scl), "+v"(s1));
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(s0[r], scl[r], pr == 0 ? 0.0f : acc[r]);
+            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(static_cast<float>(s0[r]), scl[r], pr == 0 ? 0.0f : acc[r]);
 #pragma unroll
-            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(s1[r], scl[16 + r], acc[r]);
+            for (int r = 0; r < RV; ++r) acc[r] = __builtin_fmaf(static_cast<float>(s1[r]), scl[16 + r], acc[r]);
             if (DUMP && sums_dump) {
 #pragma unroll
                 for (int r = 0; r < RV; ++r) {

@@ -469,6 +469,41 @@ def test_tri_mul_finite_guard(ops, oracle):
     assert got.tolist() == oracle.tri_mul(left, right, 1, 4, 1, 2, 1, 2.0, True).tolist()
 
 
+@pytest.mark.parametrize("arith", ["split", "fp32"])
+@pytest.mark.parametrize("D,I,J,K,Bt,outgoing", [
+    (4, 103, 103, 103, 1, True), (4, 103, 103, 103, 1, False), (3, 40, 150, 70, 2, True), (3, 40, 150, 70, 2, False),
+])
+def test_tri_mul_non_finite_operands_anywhere(ops, oracle, D, I, J, K, Bt, outgoing, arith):
+    # The guard's result depends on how infinities travel through the sum (inf * b + finite terms = +-inf -> +-1e4,
+    # inf - inf and inf * 0 = NaN -> 0), which is why this contraction runs on the fp32 pipe whatever arithmetic is
+    # selected (the split of the bf16 pipe would turn an infinite operand into NaN): infinities, NaNs and huge
+    # finite values (whose products overflow) scattered over both operands, several per plane, must give the
+    # reference's class for every output (0, +-1e4) and its value everywhere else.
+    rng = np.random.default_rng(D * 31 + K + (7 if outgoing else 0))
+    left = rng.standard_normal(D * I * K * Bt).astype(np.float32)
+    right = rng.standard_normal(D * J * K * Bt).astype(np.float32)
+    for arr in (left, right):
+        pos = rng.choice(arr.size, size=24, replace=False)
+        arr[pos[:6]] = np.inf
+        arr[pos[6:12]] = -np.inf
+        arr[pos[12:16]] = np.nan
+        arr[pos[16:20]] = 3e30            # finite, but its products with a like value overflow
+        arr[pos[20:24]] = 0.0             # inf * 0 where they meet
+    L = float(K)
+    want = oracle.tri_mul(left, right, D, I, J, K, Bt, L, outgoing)
+    before = ops.set_f32_arithmetic(arith)
+    try:
+        got = ops.tri_mul(_dev(left), _dev(right), D, I, J, K, Bt, L, outgoing).cpu().numpy()
+    finally:
+        ops.set_f32_arithmetic(before)
+    assert np.isfinite(got).all()
+    touched = (np.abs(want) == 1e4) | (want == 0.0)
+    assert touched.sum() > 100 and (~touched).sum() > 100
+    # outputs whose sum met a non-finite or overflowing term: the same value exactly (0, +1e4 or -1e4)
+    assert np.array_equal(got[touched], want[touched])
+    _check(got[~touched], want[~touched])
+
+
 @pytest.mark.parametrize("D,I,J,K,Bt,outgoing", [
     (3, 5, 4, 6, 2, True), (3, 5, 4, 6, 2, False),
     (8, 103, 103, 103, 1, True), (8, 103, 103, 103, 1, False),
