@@ -106,7 +106,10 @@ int q8_weight_pack_hip(const void *W, int wtype, int M, int K, void *packed,
  * contracted with int8 MFMA into an exact int32 and settled as
  *     acc = fma(float(sumi), d_w * d_a, acc)        blocks ascending
  * (src/cuda/MulMatQ8Kernel.cu:120-142).  c_trans 0 -> C[m*N+n], 1 -> C[n*M+m].
- * *path_out (may be NULL) is set to 1: there is only the MFMA path. */
+ * *path_out (may be NULL) receives what the reference would report for the call (MulMatQ8Kernel.cu:493-496):
+ * 1 when PPML_MMQ is not 0 and N reaches PPML_MMQ_MIN_N (default 16) or the weight is repacked (wtype 2, 3),
+ * else 0; 0 on every error.  It names the reference's kernels, not this library's (ppml_hip_q8_last_path
+ * does that): every path gives the same numbers. */
 int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
                    int c_trans, int *path_out, ppml_hip_stream_t stream);
 

@@ -1598,10 +1598,27 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
     }
 }
 
+// What mul_mat_q8_cuda would report in *path_out for this call (src/cuda/MulMatQ8Kernel.cu:493-496): 1 (its
+// MMQ kernels) when PPML_MMQ is not 0 and the token count reaches PPML_MMQ_MIN_N (default 16) or the weight is
+// repacked, else 0 (its MMVQ kernels).  Both of its paths give the same numbers and so does this library, whose
+// own choice of kernel ppml_hip_q8_last_path() reports; the value is kept for callers that log or count it.
+static int reference_path_value(int N, int wtype) {
+    const auto env_int = [](const char* name, int fallback) {
+        const char* v = std::getenv(name);
+        if (!v || !*v) return fallback;
+        char* end = nullptr;
+        const long x = std::strtol(v, &end, 10);
+        return end == v ? fallback : static_cast<int>(x);
+    };
+    const int min_n = env_int("PPML_MMQ_MIN_N", 16);
+    const bool mmq_on = env_int("PPML_MMQ", 1) != 0;
+    return (mmq_on && (N >= min_n || wtype == PPML_WTYPE_Q8_0R || wtype == PPML_WTYPE_Q8_0M)) ? 1 : 0;
+}
+
 extern "C" int mul_mat_q8_hip(const void* W, const float* X, float* C, int M, int N, int K, int wtype,
                               int c_trans, int* path_out, ppml_hip_stream_t stream) {
     if (path_out) *path_out = 0;
     const int rc = mul_mat_q8_ex_hip(W, X, C, M, N, K, wtype, c_trans, 0, nullptr, nullptr, stream);
-    if (rc == RC_OK && path_out) *path_out = 1;
+    if (rc == RC_OK && path_out) *path_out = reference_path_value(N, wtype);
     return rc;
 }

@@ -323,7 +323,23 @@ def test_status_codes(ops):
     assert lib.mul_mat_q8_hip(p, p, p, 4, 4, 48, 0, 1, C.byref(path), None) == 2 and path.value == 0
     assert lib.mul_mat_q8_hip(p, p, p, 4, 4, 32, 4, 1, C.byref(path), None) == 5
     assert lib.mul_mat_q8_hip(None, p, p, 4, 4, 32, 0, 1, None, None) == 1
-    assert lib.mul_mat_q8_hip(p, p, p, 4, 4, 32, 0, 1, C.byref(path), None) == 0 and path.value == 1
+    # *path_out: the reference's own rule (src/cuda/MulMatQ8Kernel.cu:493-496): its MMQ kernels (1) from 16 tokens
+    # on or for a repacked weight, unless PPML_MMQ=0; the threshold is PPML_MMQ_MIN_N
+    import os
+    saved = {k: os.environ.pop(k, None) for k in ("PPML_MMQ", "PPML_MMQ_MIN_N")}
+    try:
+        assert lib.mul_mat_q8_hip(p, p, p, 4, 4, 32, 0, 1, C.byref(path), None) == 0 and path.value == 0
+        assert lib.mul_mat_q8_hip(p, p, p, 4, 16, 32, 0, 1, C.byref(path), None) == 0 and path.value == 1
+        assert lib.mul_mat_q8_hip(p, p, p, 4, 4, 32, 2, 1, C.byref(path), None) == 0 and path.value == 1
+        os.environ["PPML_MMQ_MIN_N"] = "4"
+        assert lib.mul_mat_q8_hip(p, p, p, 4, 4, 32, 0, 1, C.byref(path), None) == 0 and path.value == 1
+        os.environ["PPML_MMQ"] = "0"
+        assert lib.mul_mat_q8_hip(p, p, p, 4, 16, 32, 2, 1, C.byref(path), None) == 0 and path.value == 0
+    finally:
+        for k, v in saved.items():
+            os.environ.pop(k, None)
+            if v is not None:
+                os.environ[k] = v
     with pytest.raises(ValueError):
         ops.mul_mat_q8(ops.Q8Weight(buf.view(torch.uint8)[:34 * 4], 4, 32, 0), torch.zeros(3, 64, device="cuda"))
 
