@@ -21,7 +21,7 @@ namespace {
 // not negative and not NaN: such floats order like their bit patterns, and an integer max has no signalling
 // NaN to quiet, so each step is a single v_max_u32 that takes its other operand through DPP
 __device__ __forceinline__ float group4_max(float v) {
-    uint32_t b = __float_as_uint(v);
+    uint32_t b = __float_as_uint(v) & 0x7fffffffu;     // (a maximum of +0 and -0 may come out as -0: not the largest pattern)
     uint32_t o;
     o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b), 0xB1, 0xf, 0xf, false));  // lane ^ 1
     b = b > o ? b : o;

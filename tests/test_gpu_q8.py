@@ -94,6 +94,11 @@ def _exponent_sweep_blocks(seed):
     pos = rng.integers(0, 32, size=top.size)
     x[np.arange(top.size), pos] = top * rng.choice(np.array([-1.0, 1.0], dtype=np.float32), size=top.size)
     x[5] = 0.0                                                                      # an all-zero block among them
+    x[6] = -0.0                                                                     # ... of negative zeros
+    x[7] = -np.abs(x[7])                                                            # nothing above zero, and
+    x[7, 3] = -0.0                                                                  # a negative zero as the largest value
+    x[8] = -np.abs(x[8])
+    x[8, 0], x[8, 31] = -0.0, 0.0
     return x
 
 
