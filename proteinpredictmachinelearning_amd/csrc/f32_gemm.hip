@@ -929,10 +929,21 @@ int f32_arithmetic() {
 int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fixed_ws = nullptr, size_t fixed_cap = 0) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
-    // An output that fits the 256 MB last-level cache is likely read next by the consumer node (the
-    // logits by their softmax); a larger one only evicts useful lines on its way to HBM.  Measured:
-    // streaming stores 72 -> 63 us on the 216 MB MSA logits, 14 -> 16 us on the 17 MB pair logits.
-    p.stream_c = static_cast<int64_t>(p.M) * p.N * p.np2 * p.np3 * 4 >= (128LL << 20);
+    // Streaming (non-temporal) stores where every store instruction writes whole 128-byte lines: dense rows of a
+    // multiple of 32 floats, on a 128-byte boundary, in every plane.  Ordinary stores leave the output dirty in the
+    // XCDs' L2s, which are written back when the kernel ends; streaming ones go out as they are issued.  Measured
+    // on the attention-logit kernels (us, streaming / ordinary): 100 planes of 128 x 128  4.8 / 6.1, 400 of them
+    // 8.0 / 10.9, 2000 of them 30.5 / 42.7, 824 planes of 256 x 256  49 / 54.  With rows that are not whole lines
+    // it is the other way round at every size (412 planes of 103 x 103  12.3 / 10.0, 3200 of them 100 / 49:
+    // partial lines are merged in L2 only by ordinary stores).  Outputs with compound addressing keep the older
+    // rule (streaming from 128 MB on: 72 -> 63 us on the 216 MB logits at the time).
+    {
+        const bool compound = !(p.c_lm >= p.M && p.c_ln >= p.N);
+        const bool planes_ok = (p.np2 == 1 || p.c_p2 % 32 == 0) && (p.np3 == 1 || p.c_p3 % 32 == 0);
+        const bool whole_lines = !compound && p.c_ni == 1 && p.c_mi % 32 == 0 && p.N % 32 == 0 && planes_ok &&
+                                 (reinterpret_cast<uintptr_t>(p.C) & 127) == 0;
+        p.stream_c = compound ? static_cast<int64_t>(p.M) * p.N * p.np2 * p.np3 * 4 >= (128LL << 20) : whole_lines;
+    }
     const int64_t total = static_cast<int64_t>(p.tiles_m) * p.tiles_n * p.np2 * p.np3;
     if (total <= 0 || total > 0x7fffffffLL) { set_error("%s: grid of %lld work-groups is out of range", what, (long long)total); return RC_BAD_ARGS; }
     const dim3 grid(static_cast<unsigned>(total)), block(256);
