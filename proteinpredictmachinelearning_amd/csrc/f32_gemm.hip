@@ -457,7 +457,15 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
 //     in, dropped on the way out).
 //
 // Arithmetic and order of the sums are those of gemm_bf16x3_kernel: same bits.
-template <int TM, bool STREAM_C>
+//
+// C_FORM says how a tile leaves: C_ORDINARY / C_STREAM store the accumulator registers as they lie (a store
+// instruction writes 32 consecutive floats of two rows: whole 128-byte lines only when the rows are), C_FLAT is for
+// dense planes whose rows are NOT whole lines and a tile that spans all columns (N <= TM): the rows of the tile are then
+// one contiguous range of memory, which goes through LDS (free once the matrix work is done) and leaves as whole,
+// aligned lines by streaming stores -- rows that end anywhere inside a line no longer leave partly written lines
+// behind in L2 -- except for the first and last line of the range, which it shares with its neighbours.
+constexpr int C_ORDINARY = 0, C_STREAM = 1, C_FLAT = 2;
+template <int TM, int C_FORM>
 __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmParams p, int total_tiles) {
     static_assert(TM == 64 || TM == 128, "tile side");
     constexpr int WT = TM / 2;                        // a wave's square of the tile
@@ -465,8 +473,10 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
     constexpr int CHUNK_PLANE = TM * SPLIT_PITCH;     // one bf16 plane of one 16-k chunk of one operand
     constexpr int OPERAND = 2 * 3 * CHUNK_PLANE;      // [chunk][plane][row][48 bytes]
     constexpr int LOADS = TM == 128 ? 2 : 1;          // 16-k chunks a thread loads separately (at 64 rows one pass covers K = 32)
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[OPERAND];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_b[OPERAND];
+    static_assert(2 * OPERAND >= (TM * TM + 32) * 4, "a whole tile of C, shifted by up to a line, fits the operands' LDS");
+    __shared__ __attribute__((aligned(128))) uint8_t lds_ab[2 * OPERAND];
+    uint8_t* const lds_a = lds_ab;
+    uint8_t* const lds_b = lds_ab + OPERAND;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -585,6 +595,57 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
         }
         __syncthreads();                                // the planes may be overwritten
         // ---- stores of this tile: younger than the next tile's loads
+        if (C_FORM == C_FLAT) {
+            // The tile's rows m0 .. m0 + rows - 1 are the floats [0, total) behind row_base.  In LDS float e of that
+            // range sits at shift + e, shift = floats between the start of row_base's 128-byte line and row_base: a
+            // 16-byte piece of LDS then is an aligned 16-byte piece of memory.
+            float* const stage = reinterpret_cast<float*>(lds_ab);
+            float* const row_base = cur.C + static_cast<int64_t>(cur.m0) * p.N;
+            const int shift = static_cast<int>((reinterpret_cast<uintptr_t>(row_base) & 127) >> 2);
+            const int rows = p.M - cur.m0 < TM ? static_cast<int>(p.M) - cur.m0 : TM;
+            const int total = rows * static_cast<int>(p.N);
+#pragma unroll
+            for (int ti = 0; ti < NT; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < NT; ++tj) {
+                    const int n = wn + tj * 32 + j;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int row = wm + ti * 32 + 4 * hh + 8 * (r >> 2) + (r & 3);
+                        float v = acc[ti][tj][r];
+                        if (scale) v *= p.alpha;
+                        // (rows past the matrix land behind the range that is stored: no test)
+                        if (n < p.N) stage[shift + row * static_cast<int>(p.N) + n] = v;
+                    }
+                }
+            __syncthreads();
+            float* const line_base = row_base - shift;            // 128-byte aligned
+            const int end = shift + total;
+            const int whole_begin = shift ? 32 : 0;               // floats of LDS that lie in lines this tile owns alone
+            const int whole_end = end & ~31;
+            // every piece is read before the first is stored: one LDS round trip per tile, not one per piece
+            constexpr int PIECES = (TM * TM + 32 + 1023) / 1024;
+            static_assert(PIECES * 1024 * 4 <= 2 * OPERAND, "the pieces past the tile still lie in the operands' LDS");
+            v4f piece[PIECES];
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i) piece[i] = *reinterpret_cast<const v4f*>(stage + (tid + 256 * i) * 4);
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i) {
+                const int q = (tid + 256 * i) * 4;
+                if (q >= whole_begin && q + 4 <= whole_end) {
+                    __builtin_nontemporal_store(piece[i], reinterpret_cast<v4f*>(line_base + q));
+                } else if (q + 4 > shift && q < end) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        if (q + c >= shift && q + c < end) line_base[q + c] = piece[i][c];
+                }
+            }
+            if (!more) break;
+            __syncthreads();                            // the staged tile has been read: the next split may overwrite it
+            t = t_next;
+            cur = nxt;
+            continue;
+        }
         const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(cur.C, 0, c_bytes, 0x00020000);
 #pragma unroll
         for (int ti = 0; ti < NT; ++ti) {
@@ -598,7 +659,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
                     float v = acc[ti][tj][r];
                     if (scale) v *= p.alpha;
                     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rsrc_c, base + (8 * (r >> 2) + (r & 3)) * ld_bytes, 0,
-                                                          STREAM_C ? 3 : 0);
+                                                          C_FORM == C_STREAM ? 3 : 0);
                 }
             }
         }
@@ -1055,10 +1116,17 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
                 int wgs = (big ? 2 : 4) * device_cu_count();      // resident work-groups: 72 KB / 36 KB of LDS each
                 if (tiles < wgs) wgs = static_cast<int>((tiles + 7) / 8 * 8);
                 const dim3 pgrid(static_cast<unsigned>(wgs));
-                if (big) { if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<128, true>), pgrid, block, 0, stream, p, static_cast<int>(tiles));
-                           else hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<128, false>), pgrid, block, 0, stream, p, static_cast<int>(tiles)); }
-                else     { if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<64, true>), pgrid, block, 0, stream, p, static_cast<int>(tiles));
-                           else hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<64, false>), pgrid, block, 0, stream, p, static_cast<int>(tiles)); }
+                // Rows that are not whole lines, dense, and one tile across: the tile leaves as one contiguous range.  It
+                // costs an LDS round trip per tile, which pays once the output no longer stays in L2 anyway (us, ordinary
+                // / contiguous: 100 planes of 103 x 103 4.9 / 6.1, 200 6.9 / 6.4, 412 10.0 / 8.0, 3200 50.7 / 43.9; 1200
+                // planes of 50 x 50 9.5 / 9.7, 3000 18.6 / 17.8).
+                const int64_t c_total = static_cast<int64_t>(p.M) * p.N * p.np2 * p.np3 * 4;
+                const bool flat = !p.stream_c && p.c_mi == p.N && p.N <= tm && c_total >= (big ? 8LL << 20 : 24LL << 20);
+                const int form = p.stream_c ? C_STREAM : flat ? C_FLAT : C_ORDINARY;
+#define PPML_SHORTK(TM_, FORM_) hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<TM_, FORM_>), pgrid, block, 0, stream, p, static_cast<int>(tiles))
+                if (big) { if (form == C_STREAM) PPML_SHORTK(128, C_STREAM); else if (form == C_FLAT) PPML_SHORTK(128, C_FLAT); else PPML_SHORTK(128, C_ORDINARY); }
+                else     { if (form == C_STREAM) PPML_SHORTK(64, C_STREAM);  else if (form == C_FLAT) PPML_SHORTK(64, C_FLAT);  else PPML_SHORTK(64, C_ORDINARY); }
+#undef PPML_SHORTK
                 return check_launch(what);
             }
         }

@@ -131,10 +131,11 @@ def mul_mat_tn(a: torch.Tensor, b: torch.Tensor, alpha: float = 1.0) -> torch.Te
     return out
 
 
-def out_prod(a: torch.Tensor, b: torch.Tensor, scale: float | None = None) -> torch.Tensor:
+def out_prod(a: torch.Tensor, b: torch.Tensor, scale: float | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
     """a [ne03,ne02,K,ne00], b [ne13,ne12,K,ne10] -> [ne13,ne12,ne10,ne00];
     src/core/ComputeGraphHelper.cpp:318-345, broadcast of src/backend/CPUKernels.cpp:836-858.
-    ``scale`` fuses the OP_SCALE node that follows in the attention path."""
+    ``scale`` fuses the OP_SCALE node that follows in the attention path.  ``out``: a contiguous float32
+    device tensor of the result's size to write into (any 4-byte alignment) instead of a new one."""
     a, b = _dev_f32(a, "a"), _dev_f32(b, "b")
     while a.dim() < 4:
         a = a.unsqueeze(0)
@@ -145,7 +146,12 @@ def out_prod(a: torch.Tensor, b: torch.Tensor, scale: float | None = None) -> to
     if ne01 != ne11:
         raise ValueError(f"out_prod: contraction dims differ ({ne01} vs {ne11})")
     ne0, ne1, ne2, ne3 = ne00, ne10, max(ne02, ne12), max(ne03, ne13)
-    out = torch.empty((ne3, ne2, ne1, ne0), dtype=torch.float32, device=a.device)
+    if out is None:
+        out = torch.empty((ne3, ne2, ne1, ne0), dtype=torch.float32, device=a.device)
+    elif out.dtype != torch.float32 or out.device != a.device or not out.is_contiguous() or out.numel() != ne0 * ne1 * ne2 * ne3:
+        raise ValueError("out_prod: `out` must be a contiguous float32 tensor of the result's size on the operands' device")
+    else:
+        out = out.view(ne3, ne2, ne1, ne0)
     dims = [ne00, ne01, ne02, ne03, ne10, ne11, ne12, ne13, ne0, ne1, ne2, ne3]
     lib = _lib()
     if scale is None:
@@ -156,10 +162,10 @@ def out_prod(a: torch.Tensor, b: torch.Tensor, scale: float | None = None) -> to
     return out
 
 
-def attention_logits(k: torch.Tensor, q: torch.Tensor, head_dim: int | None = None) -> torch.Tensor:
+def attention_logits(k: torch.Tensor, q: torch.Tensor, head_dim: int | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
     """out_prod(K, Q) * 1/sqrt(head_dim), steps 1-2 of src/modules/Attention.cpp:264-270."""
     d = k.shape[-2] if head_dim is None else head_dim
-    return out_prod(k, q, scale=1.0 / math.sqrt(float(d)))
+    return out_prod(k, q, scale=1.0 / math.sqrt(float(d)), out=out)
 
 
 def outer_product_mean(left: torch.Tensor, right: torch.Tensor, D: int, L: int, N: int, B: int) -> torch.Tensor:

@@ -161,11 +161,10 @@ def test_attention_logits_shapes(ops, oracle, planes, L, D):
 
 def test_attention_logits_msa_row_attention_full_size(ops, oracle):
     # The configured MSA form: 824 planes (8 heads x 103 residues) of 256 x 256 logits over a head dimension of
-    # 32.  The 216 MB result is past the size where the launcher switches to the streaming-store instances, so
-    # this is the one test that runs them.  (a) sampled planes against the oracle; (b) planes are independent:
-    # a 64-plane slice launched alone (17 MB, the ordinary-store instance) must give the same bits as the same
-    # planes of the full launch; (c) every plane of the full result is covered by a checksum against a second
-    # full launch on the same inputs and by the slice-wise comparison of (b) walked over all planes.
+    # 32.  Rows of whole 128-byte lines on a 128-byte boundary leave by streaming stores.  (a) sampled planes against
+    # the oracle; (b) planes are independent: a 64-plane slice written to an address that is NOT on a line boundary
+    # (the ordinary-store instance) must give the same bits as the same planes of the full launch, walked over all
+    # planes; (c) a second full launch on the same inputs gives the same bits.
     planes, L, D = 824, 256, 32
     g = torch.Generator(device="cuda").manual_seed(824)
     k = torch.randn(1, planes, D, L, device="cuda", generator=g)
@@ -177,11 +176,51 @@ def test_attention_logits_msa_row_attention_full_size(ops, oracle):
     want = oracle.out_prod(kh, qh) * np.float32(1.0 / math.sqrt(D))
     absprod = np.einsum("pqki,pqkj->pqji", np.abs(kh).astype(np.float64), np.abs(qh).astype(np.float64)) / math.sqrt(D)
     _check(full[:, sel].cpu().numpy(), want, absprod)
+    room = torch.empty(64 * L * L + 32, device="cuda")
     for p0 in range(0, planes, 64):
         p1 = min(p0 + 64, planes)
-        part = ops.attention_logits(k[:, p0:p1].contiguous(), q[:, p0:p1].contiguous())
+        out = room[3:3 + (p1 - p0) * L * L]
+        assert out.data_ptr() % 128 != 0
+        part = ops.attention_logits(k[:, p0:p1].contiguous(), q[:, p0:p1].contiguous(), out=out)
         assert torch.equal(part, full[:, p0:p1]), f"planes {p0}..{p1} differ between the two store forms"
     again = ops.attention_logits(k, q)
+    assert torch.equal(again, full)
+
+
+@pytest.mark.parametrize("planes,rows,cols,D,lead", [
+    (412, 103, 103, 32, 0),     # the pair-track logits: one 128-wide tile per plane
+    (412, 103, 103, 32, 5),     # ... on an output that starts 20 bytes into a line
+    (3200, 103, 103, 32, 1),    # six or seven tiles per work-group
+    (90, 300, 103, 32, 2),      # three row tiles per plane, the last one ragged
+    (3300, 50, 50, 32, 3),      # 64-wide tiles
+    (700, 127, 127, 8, 31),     # rows of 127 floats, K below a 16-k chunk
+])
+def test_attention_logits_ragged_rows_leave_as_contiguous_ranges(ops, oracle, planes, rows, cols, D, lead):
+    # Dense planes whose rows are not whole 128-byte lines: from a few MB on, a tile that spans all columns is staged
+    # through LDS and stored as one contiguous range of whole lines.  Same bits as the instance that stores the
+    # accumulator registers directly (what small launches of the same planes use), for every plane; nothing outside
+    # the output is written (it starts and ends inside lines it shares with its surroundings); sampled planes against
+    # the oracle.
+    g = torch.Generator(device="cuda").manual_seed(planes + rows)
+    a = torch.randn(1, planes, D, cols, device="cuda", generator=g)
+    b = torch.randn(1, planes, D, rows, device="cuda", generator=g)
+    n = planes * rows * cols
+    room = torch.full((n + 96,), -7.5, device="cuda")
+    full = ops.out_prod(a, b, scale=0.25, out=room[lead:lead + n])
+    assert full.shape == (1, planes, rows, cols)
+    assert torch.all(room[:lead] == -7.5) and torch.all(room[lead + n:] == -7.5), "stores outside the output"
+    sel = [0, 1, planes // 2, planes - 1]
+    ah, bh = a[:, sel].cpu().numpy(), b[:, sel].cpu().numpy()
+    want = oracle.out_prod(ah, bh) * np.float32(0.25)
+    absprod = np.einsum("pqki,pqkj->pqji", np.abs(ah).astype(np.float64), np.abs(bh).astype(np.float64)) * 0.25
+    _check(full[:, sel].cpu().numpy(), want, absprod)
+    step = max(1, (1 << 20) // (rows * cols * 4))      # 1 MB at a time: the ordinary-store instance
+    for p0 in list(range(0, planes, step))[:: max(1, planes // step // 40)]:
+        p1 = min(p0 + step, planes)
+        part = ops.out_prod(a[:, p0:p1].contiguous(), b[:, p0:p1].contiguous(), scale=0.25)
+        assert torch.equal(part, full[:, p0:p1]), f"planes {p0}..{p1} differ between the two store forms"
+    room.fill_(-7.5)
+    again = ops.out_prod(a, b, scale=0.25, out=room[lead:lead + n])
     assert torch.equal(again, full)
 
 
