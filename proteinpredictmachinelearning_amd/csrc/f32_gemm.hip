@@ -463,8 +463,10 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
 // dense planes whose rows are NOT whole lines and a tile that spans all columns (N <= TM): the rows of the tile are then
 // one contiguous range of memory, which goes through LDS (free once the matrix work is done) and leaves as whole,
 // aligned lines by streaming stores -- rows that end anywhere inside a line no longer leave partly written lines
-// behind in L2 -- except for the first and last line of the range, which it shares with its neighbours.
-constexpr int C_ORDINARY = 0, C_STREAM = 1, C_FLAT = 2;
+// behind in L2 -- except for the first and last line of the range, which it shares with its neighbours.  C_ROWS is
+// for rows of whole lines that are longer than the tile is wide: the tile goes through LDS as well and leaves
+// sixteen bytes per lane, a store instruction writing two 512-byte runs instead of two lines.
+constexpr int C_ORDINARY = 0, C_STREAM = 1, C_FLAT = 2, C_ROWS = 3;
 template <int TM, int C_FORM>
 __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmParams p, int total_tiles) {
     static_assert(TM == 64 || TM == 128, "tile side");
@@ -642,6 +644,39 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
             }
             if (!more) break;
             __syncthreads();                            // the staged tile has been read: the next split may overwrite it
+            t = t_next;
+            cur = nxt;
+            continue;
+        }
+        if (C_FORM == C_ROWS) {
+            // rows of whole lines: the tile goes to LDS as [row][TM] and leaves sixteen bytes per lane
+            float* const stage = reinterpret_cast<float*>(lds_ab);
+#pragma unroll
+            for (int ti = 0; ti < NT; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < NT; ++tj)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int row = wm + ti * 32 + 4 * hh + 8 * (r >> 2) + (r & 3);
+                        float v = acc[ti][tj][r];
+                        if (scale) v *= p.alpha;
+                        stage[row * TM + wn + tj * 32 + j] = v;
+                    }
+            __syncthreads();
+            constexpr int PIECES = TM * TM / 1024;
+            v4f piece[PIECES];
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i) piece[i] = *reinterpret_cast<const v4f*>(stage + (tid + 256 * i) * 4);
+            float* const tile_base = cur.C + static_cast<int64_t>(cur.m0) * p.c_mi + cur.n0;
+#pragma unroll
+            for (int i = 0; i < PIECES; ++i) {
+                const int q = tid + 256 * i;
+                const int row = q / (TM / 4), c4 = (q % (TM / 4)) * 4;
+                if (cur.m0 + row < p.M && cur.n0 + c4 < p.N)
+                    __builtin_nontemporal_store(piece[i], reinterpret_cast<v4f*>(tile_base + static_cast<int64_t>(row) * p.c_mi + c4));
+            }
+            if (!more) break;
+            __syncthreads();
             t = t_next;
             cur = nxt;
             continue;
@@ -1122,9 +1157,14 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
                 // planes of 50 x 50 9.5 / 9.7, 3000 18.6 / 17.8).
                 const int64_t c_total = static_cast<int64_t>(p.M) * p.N * p.np2 * p.np3 * 4;
                 const bool flat = !p.stream_c && p.c_mi == p.N && p.N <= tm && c_total >= (big ? 8LL << 20 : 24LL << 20);
-                const int form = p.stream_c ? C_STREAM : flat ? C_FLAT : C_ORDINARY;
+                // Rows of whole lines that are longer than a tile is wide: through LDS too, sixteen bytes per lane (us,
+                // registers as they lie / through LDS: 824 planes of 256 x 256 46-48 / 44.5, 200 of 512 x 512 45.4 / 41.5;
+                // rows that one tile spans lose the round trip: 2000 planes of 128 x 128 30.2 / 31.4, 100 of them 4.8 / 5.5).
+                const bool rows = p.stream_c && big && p.N > tm;
+                const int form = rows ? C_ROWS : p.stream_c ? C_STREAM : flat ? C_FLAT : C_ORDINARY;
 #define PPML_SHORTK(TM_, FORM_) hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<TM_, FORM_>), pgrid, block, 0, stream, p, static_cast<int>(tiles))
-                if (big) { if (form == C_STREAM) PPML_SHORTK(128, C_STREAM); else if (form == C_FLAT) PPML_SHORTK(128, C_FLAT); else PPML_SHORTK(128, C_ORDINARY); }
+                if (form == C_ROWS) PPML_SHORTK(128, C_ROWS);
+                else if (big) { if (form == C_STREAM) PPML_SHORTK(128, C_STREAM); else if (form == C_FLAT) PPML_SHORTK(128, C_FLAT); else PPML_SHORTK(128, C_ORDINARY); }
                 else     { if (form == C_STREAM) PPML_SHORTK(64, C_STREAM);  else if (form == C_FLAT) PPML_SHORTK(64, C_FLAT);  else PPML_SHORTK(64, C_ORDINARY); }
 #undef PPML_SHORTK
                 return check_launch(what);

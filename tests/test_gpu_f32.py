@@ -224,6 +224,29 @@ def test_attention_logits_ragged_rows_leave_as_contiguous_ranges(ops, oracle, pl
     assert torch.equal(again, full)
 
 
+@pytest.mark.parametrize("planes,rows,cols,D", [(40, 300, 384, 32), (9, 130, 256, 20), (3, 128, 160, 32)])
+def test_attention_logits_long_rows_of_whole_lines(ops, oracle, planes, rows, cols, D):
+    # Rows of whole 128-byte lines that are longer than a tile is wide leave through LDS, sixteen bytes per lane;
+    # the same call on an output that does not start on a line boundary takes the instance that stores the
+    # accumulator registers directly: same bits; ragged last row tile, ragged last column tile; against the oracle.
+    g = torch.Generator(device="cuda").manual_seed(rows + cols)
+    a = torch.randn(1, planes, D, cols, device="cuda", generator=g)
+    b = torch.randn(1, planes, D, rows, device="cuda", generator=g)
+    n = planes * rows * cols
+    room = torch.full((n + 64,), -7.5, device="cuda")
+    assert room.data_ptr() % 128 == 0
+    aligned = ops.out_prod(a, b, scale=0.5, out=room[32:32 + n]).clone()
+    assert torch.all(room[:32] == -7.5) and torch.all(room[32 + n:] == -7.5), "stores outside the output"
+    room.fill_(-7.5)
+    shifted = ops.out_prod(a, b, scale=0.5, out=room[7:7 + n])
+    assert torch.all(room[:7] == -7.5) and torch.all(room[7 + n:] == -7.5), "stores outside the output"
+    assert torch.equal(aligned, shifted)
+    ah, bh = a.cpu().numpy(), b.cpu().numpy()
+    want = oracle.out_prod(ah[:, :3], bh[:, :3]) * np.float32(0.5)
+    absprod = np.einsum("pqki,pqkj->pqji", np.abs(ah[:, :3]).astype(np.float64), np.abs(bh[:, :3]).astype(np.float64)) * 0.5
+    _check(aligned[:, :3].cpu().numpy(), want, absprod)
+
+
 # ----------------------------------------------------------------------------- non-finite and subnormal operands
 def test_infinite_operand_gives_nan_on_the_split_pipe_and_inf_on_the_fp32_pipe(ops, oracle):
     # The reference's loop (src/backend/CPUKernels.cpp:763-771) carries an infinite operand through: inf * b
