@@ -265,6 +265,148 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmParams p) {
 }
 
 // ------------------------------------------------------------------------------------------
+// Many planes of small contractions with K <= 128 on the fp32 pipe (the triangle multiplication: 128 channel
+// planes of 103 x 103 over K = 103).  With 128 x 128 tiles that is one work-group per plane, half the CUs idle, each
+// walking seven 16-k stages of load -> LDS -> 32 MFMAs per wave -> barrier one after the other.  Here a work-group
+// takes a 64 x 64 tile (four per plane: every CU has two), loads the whole K of both panels at once -- one memory
+// round trip -- and then runs its K / 2 MFMAs per wave out of LDS without a barrier in between.  Products and sums are
+// those of gemm_f32_kernel in the same order (k ascending two at a time from the bias): same bits.
+constexpr int MIDK_MAX = 128;
+template <int MODE> struct MidK { static constexpr int LD = MODE == LOAD_ROW_CONTIG ? 68 : 65; };   // floats per k row of a panel
+
+template <int MODE, bool CLAMP>
+__global__ __launch_bounds__(256) void gemm_f32_midk_kernel(const GemmParams p, int kp) {
+    static_assert(MODE == LOAD_K_CONTIG || MODE == LOAD_ROW_CONTIG, "contiguous operands only");
+    constexpr int T = 64, LD = MidK<MODE>::LD;
+    extern __shared__ __attribute__((aligned(16))) float lds_midk[];
+    float* const lds_a = lds_midk;                      // [kp][LD]: k-major, rows contiguous
+    float* const lds_b = lds_midk + kp * LD;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 31, hh = lane >> 5;
+    const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+    const int tiles_m = (p.M + T - 1) / T, tiles_n = (p.N + T - 1) / T;
+    const int tiles = tiles_m * tiles_n;
+    const int idx = xcd_contiguous_index(blockIdx.x, tiles * p.np2 * p.np3);
+    const int plane = idx / tiles;
+    const int t = idx - plane * tiles;
+    const int m0 = (t / tiles_n) * T, n0 = (t % tiles_n) * T;
+    const int p2 = plane % p.np2, p3 = plane / p.np2;
+    const float* A = p.A + p2 * p.a_p2 + p3 * p.a_p3;
+    const float* B = p.B + (p2 / p.b_div2) * p.b_p2 + (p3 / p.b_div3) * p.b_p3;
+    float* C = p.C + p2 * p.c_p2 + p3 * p.c_p3;
+
+    // ---- both panels, all of K, in flight at once
+    v4f ra[8], rb[8];
+    const auto load_panel = [&](const float* __restrict__ base, int64_t rs, int64_t ks, int row0, int nrows, v4f (&reg)[8]) {
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            v4f v = {0.f, 0.f, 0.f, 0.f};
+            if (MODE == LOAD_K_CONTIG) {
+                // sixteen lanes along 64 k of a row, four rows per wave instruction
+                const int row = row0 + (tid >> 4) + 16 * (it & 3);
+                const int k = (tid & 15) * 4 + 64 * (it >> 2);
+                if (row < nrows && k < p.K) {
+                    const float* src = base + static_cast<int64_t>(row) * rs + k;
+                    if (k + 3 < p.K) v = *reinterpret_cast<const v4f_u*>(src);
+                    else {
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) if (k + c < p.K) v[c] = src[c];
+                    }
+                }
+            } else {
+                // sixteen lanes along the 64 rows of one k, four k per wave instruction
+                const int k = (tid >> 4) + 16 * it;
+                const int row = row0 + (tid & 15) * 4;
+                if (k < p.K && row < nrows) {
+                    const float* src = base + static_cast<int64_t>(k) * ks + row;
+                    if (row + 3 < nrows) v = *reinterpret_cast<const v4f_u*>(src);
+                    else {
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) if (row + c < nrows) v[c] = src[c];
+                    }
+                }
+            }
+            reg[it] = v;
+        }
+    };
+    const auto park_panel = [&](float* __restrict__ lds, const v4f (&reg)[8]) {
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            if (MODE == LOAD_K_CONTIG) {
+                const int row = (tid >> 4) + 16 * (it & 3);
+                const int k = (tid & 15) * 4 + 64 * (it >> 2);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) if (k + c < kp) lds[(k + c) * LD + row] = reg[it][c];
+            } else {
+                const int k = (tid >> 4) + 16 * it;
+                if (k < kp) *reinterpret_cast<v4f*>(lds + k * LD + (tid & 15) * 4) = reg[it];
+            }
+        }
+    };
+    load_panel(A, p.a_rs, p.a_ks, m0, p.M, ra);
+    load_panel(B, p.b_rs, p.b_ks, n0, p.N, rb);
+
+    v16f acc;
+    {
+        const int n = n0 + wn + j;
+        const float b0 = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = b0;
+    }
+    park_panel(lds_a, ra);
+    park_panel(lds_b, rb);
+    __syncthreads();
+
+    const float* fa = lds_a + hh * LD + wm + j;
+    const float* fb = lds_b + hh * LD + wn + j;
+    int kk = 0;
+    for (; kk + 16 <= kp; kk += 16) {                   // eight steps' operands are read ahead of their MFMAs
+        float a[8], b[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { a[u] = fa[(kk + 2 * u) * LD]; b[u] = fb[(kk + 2 * u) * LD]; }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc, 0, 0, 0);
+    }
+    for (; kk < kp; kk += 2) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[kk * LD], fb[kk * LD], acc, 0, 0, 0);
+
+    const int n = n0 + wn + j;
+    if (n >= p.N) return;
+    const bool scale = p.alpha != 1.0f;
+    float* out = C + static_cast<int64_t>(n) * p.c_ni;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + 4 * hh + 8 * (r >> 2) + (r & 3);
+        if (m >= p.M) continue;
+        float v = acc[r];
+        if (scale) v *= p.alpha;
+        if (CLAMP) v = (v != v) ? 0.0f : (v > 1e4f ? 1e4f : (v < -1e4f ? -1e4f : v));
+        out[static_cast<int64_t>(m) * p.c_mi] = v;
+    }
+}
+
+template <int MODE, bool CLAMP>
+int launch_f32_midk(const GemmParams& p, hipStream_t stream, const char* what) {
+    const int kp = (p.K + 1) & ~1;
+    const size_t lds = static_cast<size_t>(2) * kp * MidK<MODE>::LD * sizeof(float);
+    auto kernel = &gemm_f32_midk_kernel<MODE, CLAMP>;
+    static std::atomic<bool> sized{false};              // per instance: more than 64 KB of dynamic LDS has to be asked for
+    if (!sized.load(std::memory_order_acquire)) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                2 * MIDK_MAX * MidK<MODE>::LD * static_cast<int>(sizeof(float))) != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("%s: cannot size the LDS of the mid-K kernel", what);
+            return RC_LAUNCH;
+        }
+        sized.store(true, std::memory_order_release);
+    }
+    const int64_t tiles = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * p.np2 * p.np3;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(256), lds, stream, p, kp);
+    return check_launch(what);
+}
+
+// ------------------------------------------------------------------------------------------
 // The same contraction on the bf16 matrix pipe, whose rate is sixteen times that of the fp32 one (which,
 // moreover, never runs beside vector instructions on this chip).  A binary32 number is the exact sum of three bf16 numbers
 // (x = x1 + x2 + x3: 8 + 8 + 8 significant bits, taken off the top by truncation), so a product is
@@ -1182,6 +1324,12 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
     else if (p.clamp) {
         if (split || p.f16_in) { set_error("%s: no clamped instance for this addressing", what); return RC_BAD_ARGS; }
         p.stream_c = 0;                                // (the clamped instances store the ordinary way, whatever the size)
+        // planes of small contractions that leave most CUs without a 128 x 128 tile: 64 x 64 tiles, whole K at once
+        const int64_t tiles64 = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * p.np2 * p.np3;
+        if (p.K <= MIDK_MAX && !p.bias && static_cast<int64_t>(grid.x) < 2 * device_cu_count() && tiles64 <= 0x7fffffffLL) {
+            if (mode == LOAD_K_CONTIG) return launch_f32_midk<LOAD_K_CONTIG, true>(p, stream, what);
+            if (mode == LOAD_ROW_CONTIG) return launch_f32_midk<LOAD_ROW_CONTIG, true>(p, stream, what);
+        }
         if (mode == LOAD_K_CONTIG) hipLaunchKernelGGL((gemm_f32_kernel<LOAD_K_CONTIG, false, false, true>), grid, block, 0, stream, p);
         else if (mode == LOAD_ROW_CONTIG) hipLaunchKernelGGL((gemm_f32_kernel<LOAD_ROW_CONTIG, false, false, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((gemm_f32_kernel<LOAD_STRIDED, false, false, true>), grid, block, 0, stream, p);
