@@ -502,6 +502,10 @@ def test_outer_product_mean_graph_form_large(ops, oracle):
     (3, 5, 4, 6, 2, True), (3, 5, 4, 6, 2, False),            # batch innermost: strided operands
     (16, 103, 103, 103, 1, True), (16, 103, 103, 103, 1, False),   # pair-track shape, a slice of the channels
     (2, 130, 70, 33, 1, True), (2, 130, 70, 33, 1, False),    # two row tiles, ragged everywhere
+    (5, 64, 65, 128, 1, True), (5, 64, 65, 128, 1, False),    # the longest K the whole-K kernel takes
+    (3, 40, 90, 127, 1, True), (3, 40, 90, 127, 1, False),    # ... an odd one
+    (4, 33, 31, 1, 1, True), (4, 33, 31, 2, 1, False),        # the shortest
+    (3, 70, 66, 129, 1, True), (3, 70, 66, 129, 1, False),    # one past: the staged kernel
 ])
 def test_tri_mul(ops, oracle, D, I, J, K, Bt, outgoing):
     rng = np.random.default_rng(D * 1000 + I)
@@ -516,6 +520,21 @@ def test_tri_mul(ops, oracle, D, I, J, K, Bt, outgoing):
     ri = rng.integers(-4, 5, size=right.size).astype(np.float32)
     got = ops.tri_mul(_dev(li), _dev(ri), D, I, J, K, Bt, 8.0, outgoing).cpu().numpy()
     assert np.array_equal(got, oracle.tri_mul(li, ri, D, I, J, K, Bt, 8.0, outgoing))
+
+
+@pytest.mark.parametrize("outgoing", [True, False])
+def test_tri_mul_whole_k_kernel_gives_the_staged_kernel_bits(ops, outgoing):
+    # 600 planes of 103 x 103 x 103 fill the chip with 128 x 128 tiles (the staged fp32 kernel); 100 of them do not
+    # and take 64 x 64 tiles with the whole K at once.  Planes are independent: same bits, plane by plane.
+    D, I, J, K = 600, 103, 103, 103
+    g = torch.Generator(device="cuda").manual_seed(600 + int(outgoing))
+    left = torch.randn(D * I * K, device="cuda", generator=g)
+    right = torch.randn(D * J * K, device="cuda", generator=g)
+    full = ops.tri_mul(left, right, D, I, J, K, 1, float(K), outgoing).reshape(D, I * J)
+    for d0 in range(0, D, 100):
+        part = ops.tri_mul(left[d0 * I * K:(d0 + 100) * I * K].contiguous(), right[d0 * J * K:(d0 + 100) * J * K].contiguous(),
+                           100, I, J, K, 1, float(K), outgoing).reshape(100, I * J)
+        assert torch.equal(part, full[d0:d0 + 100]), f"planes {d0}..{d0 + 100}"
 
 
 def test_tri_mul_finite_guard(ops, oracle):
