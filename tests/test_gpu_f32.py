@@ -224,6 +224,17 @@ def test_attention_logits_ragged_rows_leave_as_contiguous_ranges(ops, oracle, pl
     assert torch.equal(again, full)
 
 
+def test_out_prod_refuses_an_unfit_output_tensor(ops):
+    a = torch.randn(1, 2, 8, 5, device="cuda")
+    b = torch.randn(1, 2, 8, 7, device="cuda")
+    good = torch.empty(2 * 7 * 5, device="cuda")
+    assert ops.out_prod(a, b, out=good).shape == (1, 2, 7, 5)
+    for bad in (torch.empty(2 * 7 * 5 + 1, device="cuda"), torch.empty(2 * 7 * 5, device="cuda", dtype=torch.float64),
+                torch.empty(2 * 7 * 5 * 2, device="cuda")[::2], torch.empty(2 * 7 * 5)):
+        with pytest.raises(ValueError):
+            ops.out_prod(a, b, out=bad)
+
+
 @pytest.mark.parametrize("planes,rows,cols,D", [(40, 300, 384, 32), (9, 130, 256, 20), (3, 128, 160, 32)])
 def test_attention_logits_long_rows_of_whole_lines(ops, oracle, planes, rows, cols, D):
     # Rows of whole 128-byte lines that are longer than a tile is wide leave through LDS, sixteen bytes per lane;
