@@ -391,15 +391,20 @@ int launch_f32_midk(const GemmParams& p, hipStream_t stream, const char* what) {
     const int kp = (p.K + 1) & ~1;
     const size_t lds = static_cast<size_t>(2) * kp * MidK<MODE>::LD * sizeof(float);
     auto kernel = &gemm_f32_midk_kernel<MODE, CLAMP>;
-    static std::atomic<bool> sized{false};              // per instance: more than 64 KB of dynamic LDS has to be asked for
-    if (!sized.load(std::memory_order_acquire)) {
+    // more than 64 KB of dynamic LDS has to be asked for, once per instance and device
+    constexpr int MAX_DEVICES = 64;
+    static std::atomic<bool> sized[MAX_DEVICES];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); dev = -1; }
+    const bool known = dev >= 0 && dev < MAX_DEVICES;
+    if (!known || !sized[dev].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 2 * MIDK_MAX * MidK<MODE>::LD * static_cast<int>(sizeof(float))) != hipSuccess) {
             (void)hipGetLastError();
-            set_error("%s: cannot size the LDS of the mid-K kernel", what);
+            set_error("%s: cannot size the LDS of the whole-K kernel", what);
             return RC_LAUNCH;
         }
-        sized.store(true, std::memory_order_release);
+        if (known) sized[dev].store(true, std::memory_order_release);
     }
     const int64_t tiles = static_cast<int64_t>((p.M + 63) / 64) * ((p.N + 63) / 64) * p.np2 * p.np3;
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(tiles)), dim3(256), lds, stream, p, kp);
