@@ -8,6 +8,7 @@
 #include "common.hpp"
 #include <type_traits>
 #include <cstdlib>
+#include <mutex>
 #include <cstring>
 
 namespace ppmlhip {
@@ -689,7 +690,7 @@ constexpr int ws_staging_regs(int nblk, int nw = 8) {   // 8 registers per unit 
 }
 constexpr int ws_compiler_vgprs(int nblk, int nw = 8) { return 256 - ws_staging_regs(nblk, nw); }
 
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY>
 __device__ __forceinline__ void q8_linear_ws_body(
     const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
     int M, int N, int ntiles, int npart, int relu,
@@ -944,13 +945,19 @@ __device__ __forceinline__ void q8_linear_ws_body(
     // Every weight fragment has arrived before the loop starts: a load still pending here would make
     // its first use inside the loop wait for vmcnt(0), i.e. for all output stores, on every iteration.
     __builtin_amdgcn_s_waitcnt(0x0f70);                // vmcnt(0), other counters untouched
-    // the second tile is requested now and quantized two thirds into the first one
+    // the second tile is requested now and quantized during the first one (at QSTEP_TILE, below)
     if (n_iter > 1) load_tile_async(tile_of(1));
 
     // Step at which the next tile is quantized.  Its loads were issued one full round of column tiles
     // earlier (right after the previous quantization freed the staging registers), so they have
     // long arrived; the tile after it is requested as soon as this one is in LDS.
-    constexpr int QSTEP_TILE = (2 * TPW) / 3;            // column tile in front of which the next tile is quantized
+    // QEARLY: at the very start of the tile instead.  The sooner the next tile is announced, the less the waves wait for
+    // each other where one tile ends and the next begins; but in the first iteration the next tile's loads have only
+    // just been issued, and waiting for them there costs a work-group with one or two tiles more than it gains later
+    // (us, two thirds in / at the start: 26368 x 256 -> 768  22.7 / 21.8, 52736 rows 40.6 / 40.1, 13184 rows 12.8 / 13.1;
+    // 26368 x 128 -> 768  17.7 / 18.3): the launcher picks it for K = 256 with three column tiles per wave from three
+    // whole rounds of tiles on.
+    constexpr int QSTEP_TILE = QEARLY ? 0 : (2 * TPW) / 3;   // column tile in front of which the next tile is quantized
     constexpr int QSTEP = QSTEP_TILE * NBLK;
     // Vector-memory operations issued between a tile's loads and the wait in front of its
     // quantization: 16 stores per column tile, one round of column tiles (fewer before the first wait).
@@ -975,7 +982,7 @@ __device__ __forceinline__ void q8_linear_ws_body(
     asm volatile("" : "+v"(unbias_a), "+v"(unbias_b));
 
     // No barrier inside the loop.  A wave may start tile `it` once all waves have announced it, which
-    // also means all of them are past two thirds of tile it-1; the tile quantized during tile `it`
+    // also means all of them have reached the quantization point of tile it-1, i.e. have left tile it-2; the tile quantized during tile `it`
     // goes to buffer (it+1) % 3, last read for tile it-2, which every wave has left by then.
     for (int it = 0; it < n_iter; ++it) {
         tile = tile_of(it);
@@ -1138,30 +1145,30 @@ __device__ __forceinline__ void q8_linear_ws_body(
 // value counts architectural and accumulation registers separately): 120 keeps it below v240.  A
 // value the compiler does not honour would go unnoticed until its registers and the staged tile
 // collide, so the build checks the generated code (check_ws_isa.py).
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(120)))
 void q8_linear_ws_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                          int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                          int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 120, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT, QEARLY>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(112)))
 void q8_linear_ws32_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 112, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT, QEARLY>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(96)))
 void q8_linear_ws64_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 96, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT, QEARLY>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
 template <int TPW, int NBLK, int WL, int NW, bool Q81, bool CSPLIT = false>
@@ -1192,7 +1199,14 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
                            static_cast<size_t>(NW) * WL * NBLK * 1024;
     using KernelFn = void (*)(const uint8_t*, const float*, float*, int, int, int, int, int, uint8_t*, int32_t*);
     KernelFn fast, dump;
-    if constexpr (ws_staging_regs(NBLK, NW) == 16) {
+    // the next tile quantized at the start of a tile rather than two thirds in (see QEARLY in the kernel)
+    constexpr bool CAN_EARLY = TPW == 3 && NBLK == 8 && NW == 8 && !CSPLIT;
+    const bool early = CAN_EARLY && all_tiles / cus >= 3;
+    if constexpr (CAN_EARLY) {
+        static_assert(ws_staging_regs(NBLK, NW) == 16, "the instance with the early quantization");
+        fast = early ? &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81, CSPLIT, true> : &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81, CSPLIT>;
+        dump = early ? &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true, Q81, CSPLIT, true> : &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true, Q81, CSPLIT>;
+    } else if constexpr (ws_staging_regs(NBLK, NW) == 16) {
         fast = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81, CSPLIT>;
         dump = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true, Q81, CSPLIT>;
     } else if constexpr (ws_staging_regs(NBLK, NW) == 32) {
@@ -1204,11 +1218,17 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
         dump = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, true, Q81, CSPLIT>;
     }
     if (lds > 64 * 1024) {
-        static const hipError_t attr_fast = hipFuncSetAttribute(
-            reinterpret_cast<const void*>(fast), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-        static const hipError_t attr_dump = hipFuncSetAttribute(
-            reinterpret_cast<const void*>(dump), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-        if (attr_fast != hipSuccess || attr_dump != hipSuccess) {
+        // (once per instance; where the launcher chooses between two forms of the kernel, once per form)
+        static hipError_t attr_fast[2] = {hipErrorNotReady, hipErrorNotReady}, attr_dump[2] = {hipErrorNotReady, hipErrorNotReady};
+        static std::mutex attr_lock;
+        {
+            std::lock_guard<std::mutex> hold(attr_lock);
+            if (attr_fast[early] == hipErrorNotReady) {
+                attr_fast[early] = hipFuncSetAttribute(reinterpret_cast<const void*>(fast), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+                attr_dump[early] = hipFuncSetAttribute(reinterpret_cast<const void*>(dump), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+            }
+        }
+        if (attr_fast[early] != hipSuccess || attr_dump[early] != hipSuccess) {
             (void)hipGetLastError();
             return -1;                                  // fall back to the general kernel
         }

@@ -388,6 +388,26 @@ def test_msa_qkv_shape_full_size_properties(ops, oracle):
     # and the result approximates the unquantized product to quantization accuracy
     full = x[idx].astype(np.float64) @ w.astype(np.float64).T
     assert np.abs(got[idx] - full).max() <= 0.03 * np.abs(full).max()
+    # From three whole rounds of tiles on, this shape's instance quantizes the next tile at the start of a tile
+    # instead of two thirds in (another compiled form).  Rows are independent: a slice of 4096 rows launched alone
+    # runs the other form and must give the same bits; so must the diagnostic form of the early kernel, whose dumped
+    # blocks and sums are compared with the oracle on the sampled rows; and the same under the Q8_1 activation rule.
+    part = ops.mul_mat_q8(W, xd[8192:12288].contiguous())
+    assert torch.equal(part, y[8192:12288])
+    yd, xq, sums = ops.mul_mat_q8(W, xd, dump=True)
+    assert torch.equal(yd, y)
+    want_q = oracle.quantize_q8_0(x[idx])
+    xq_np = xq.cpu().numpy()
+    assert (xq_np.reshape((N,) + want_q.shape[1:])[idx] == want_q).all()
+    want_sums = oracle.q8_block_sums(wq, want_q[:80])
+    sums_np = sums.cpu().numpy()
+    assert (sums_np.reshape((N,) + want_sums.shape[1:])[idx[:80]] == want_sums).all()
+    del xq_np, sums_np
+    del yd, xq, sums
+    y1 = ops.mul_mat_q8(W, xd, act="q8_1")
+    part1 = ops.mul_mat_q8(W, xd[8192:12288].contiguous(), act="q8_1")
+    assert torch.equal(part1, y1[8192:12288])
+    assert not torch.equal(y1, y)
 
 
 # ----------------------------------------------------------------------------- Q8_1 activation rule
