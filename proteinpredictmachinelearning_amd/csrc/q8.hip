@@ -1077,10 +1077,18 @@ __device__ __forceinline__ void q8_linear_ws_body(
             // inside it, so nothing but loop state crosses the boundary.
             if (!opaque_one()) continue;
             if (partial && t0 != part_col) continue;
-            if (t0 * NBLK == QSTEP_TILE * NBLK && has_next) {
+            // QEARLY: the waves that share a SIMD (w and w + 4) take turns -- one quantizes at the start of the tile while
+            // the other is at its block steps, and the other way round one column tile later (another 1 to 2 % at
+            // 26368 x 256 -> 768; two column tiles later: nothing).  Sixteen stores lie between the loads and the first
+            // wait of the second group.
+            const bool q_here = QEARLY ? ((t0 == 0 && wave < NW / 2) || (t0 == 1 && wave >= NW / 2)) : t0 == QSTEP_TILE;
+            if (q_here && has_next) {
                 {
                     v4f xn[UPW][2];
-                    if (it == 0) take_tile(std::integral_constant<int, NEWER_FIRST>{}, next, xn);
+                    if (it == 0) {
+                        if (QEARLY && t0 == 1) take_tile(std::integral_constant<int, 16>{}, next, xn);
+                        else take_tile(std::integral_constant<int, NEWER_FIRST>{}, next, xn);
+                    }
                     else take_tile(std::integral_constant<int, NEWER>{}, next, xn);
                     if (it + 2 < n_iter) load_tile_async(tile_of(it + 2));
                     quantize_tile((it + 1) % WS_NBUF, next * TILE_TOK, xn);
