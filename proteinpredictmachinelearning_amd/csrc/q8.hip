@@ -1077,10 +1077,10 @@ __device__ __forceinline__ void q8_linear_ws_body(
             // inside it, so nothing but loop state crosses the boundary.
             if (!opaque_one()) continue;
             if (partial && t0 != part_col) continue;
-            // QEARLY: the waves that share a SIMD (w and w + 4) take turns -- one quantizes at the start of the tile while
-            // the other is at its block steps, and the other way round one column tile later (another 1 to 2 % at
-            // 26368 x 256 -> 768; two column tiles later: nothing).  Sixteen stores lie between the loads and the first
-            // wait of the second group.
+            // QEARLY: half of the waves quantize at the start of the tile, the other half one column tile later, so
+            // that not all eight are at their vector work at once (another 1 to 2 % at 26368 x 256 -> 768; which waves
+            // form a half makes no difference, two column tiles later gains nothing).  Sixteen stores lie between the
+            // loads and the first wait of the second half.
             const bool q_here = QEARLY ? ((t0 == 0 && wave < NW / 2) || (t0 == 1 && wave >= NW / 2)) : t0 == QSTEP_TILE;
             if (q_here && has_next) {
                 {
