@@ -130,6 +130,7 @@ enum {
     PPML_Q8_FLAG_NO_WEIGHT_STATIONARY = 8, /* do not take the weight-stationary kernel */
     PPML_Q8_FLAG_LOW_LATENCY_8 = 16,       /* low-latency kernel with units of 8 tokens wherever it has an instance */
     PPML_Q8_FLAG_LOW_LATENCY_16 = 32,      /* ... of 16 tokens */
+    PPML_Q8_FLAG_LOW_LATENCY_32 = 48,      /* ... of 32 tokens (both bits; K = 512 only) */
     PPML_Q8_FLAG_COLUMN_PARTS = 64,        /* weight-stationary kernel: work-groups share a token tile, a part of the columns each, wherever there is an instance */
     PPML_Q8_FLAG_NO_COLUMN_PARTS = 128     /* ... never */
 };

@@ -1304,7 +1304,7 @@ int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int 
 // a work-group of the weight-stationary kernel gets one or two token tiles: there is nothing to amortise
 // resident weights over, and one tile per work-group is a chain of load -> quantize -> block steps ->
 // store in which nothing overlaps (measured at 10609 x 512 -> 128: 12.4 us against about 8 us for a copy
-// of the same bytes).  Here the tokens are cut into units of TOK = 8 or 16 rows, one four-wave work-group
+// of the same bytes).  Here the tokens are cut into units of TOK = 8 or 16 rows (32 at two per CU), one four-wave work-group
 // each, three of them resident per CU at different stages:
 //
 //   * every lane requests its whole share of the unit's activations at once (with all work-groups
@@ -1322,10 +1322,10 @@ int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int 
 // Blocks ascend per output and every settlement is the same fma as everywhere else: same bits.
 // ------------------------------------------------------------------------------------------
 template <int TOK, int NBLK, int CPW, bool DUMP, bool Q81>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void q8_linear_ll_kernel(
+__device__ __forceinline__ void q8_linear_ll_body(
     const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
     int M, int N, int relu, uint8_t* __restrict__ xq_dump, int32_t* __restrict__ sums_dump) {
-    static_assert(TOK == 8 || TOK == 16, "token rows per work-group");
+    static_assert(TOK == 8 || TOK == 16 || TOK == 32, "token rows per work-group");
     static_assert(NBLK % 2 == 0, "blocks are taken in pairs");
     static_assert(CPW * NBLK <= 16, "the wave's weight fragments stay in 64 registers");
     constexpr int NW = 4;
@@ -1483,11 +1483,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     }
 }
 
+template <int TOK, int NBLK, int CPW, bool DUMP, bool Q81>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void q8_linear_ll_kernel(
+    const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
+    int M, int N, int relu, uint8_t* __restrict__ xq_dump, int32_t* __restrict__ sums_dump) {
+    q8_linear_ll_body<TOK, NBLK, CPW, DUMP, Q81>(W, X, C, M, N, relu, xq_dump, sums_dump);
+}
+template <int TOK, int NBLK, int CPW, bool DUMP, bool Q81>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void q8_linear_ll2_kernel(
+    const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
+    int M, int N, int relu, uint8_t* __restrict__ xq_dump, int32_t* __restrict__ sums_dump) {
+    q8_linear_ll_body<TOK, NBLK, CPW, DUMP, Q81>(W, X, C, M, N, relu, xq_dump, sums_dump);
+}
+
 template <int TOK, int NBLK, int CPW, bool Q81>
 int launch_q8_linear_ll(const void* W, const float* X, float* C, int M, int N, int relu,
                         void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
     const dim3 grid((N + TOK - 1) / TOK), block(256);
-    if (xq_dump || sums_dump)
+    if constexpr (TOK == 32) {
+        if (xq_dump || sums_dump)
+            hipLaunchKernelGGL((q8_linear_ll2_kernel<TOK, NBLK, CPW, true, Q81>), grid, block, 0, stream, static_cast<const uint8_t*>(W), X, C,
+                               M, N, relu, static_cast<uint8_t*>(xq_dump), sums_dump);
+        else
+            hipLaunchKernelGGL((q8_linear_ll2_kernel<TOK, NBLK, CPW, false, Q81>), grid, block, 0, stream, static_cast<const uint8_t*>(W), X, C,
+                               M, N, relu, static_cast<uint8_t*>(nullptr), static_cast<int32_t*>(nullptr));
+    } else if (xq_dump || sums_dump)
         hipLaunchKernelGGL((q8_linear_ll_kernel<TOK, NBLK, CPW, true, Q81>), grid, block, 0, stream, static_cast<const uint8_t*>(W), X, C,
                            M, N, relu, static_cast<uint8_t*>(xq_dump), sums_dump);
     else
@@ -1514,11 +1534,16 @@ int try_q8_linear_ll(const void* W, const float* X, float* C, int M, int N, int 
         const int resident = 3 * device_cu_count();
         if (N <= 2048) tok = 8;
         else if (N <= 4096 || (nblk == 16 && (N + 15) / 16 <= resident)) tok = 16;
+        // K = 512 beyond that, while units of 32 tokens are all resident at two work-groups per CU (they need the
+        // registers of two waves per SIMD): 16000 x 512 -> 128 11.2 us against 12.0 weight-stationary (at 10609 rows,
+        // where units of 16 are all resident, 10.6 against their 9.7)
+        else if (nblk == 16 && (N + 31) / 32 <= 2 * device_cu_count()) tok = 32;
         else return -1;
     }
 #define PPML_LL(TOK, NBLK, CPW) if (tok == TOK && nblk == NBLK) return launch_q8_linear_ll<TOK, NBLK, CPW, Q81>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
     PPML_LL(8, 4, 4);  PPML_LL(8, 8, 2);  PPML_LL(8, 16, 1);
     PPML_LL(16, 4, 4); PPML_LL(16, 8, 2); PPML_LL(16, 16, 1);
+    PPML_LL(32, 16, 1);
 #undef PPML_LL
     return -1;
 }
@@ -1610,7 +1635,9 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
         case PPML_WTYPE_Q8_1:  return dispatch_q8_linear<PPML_WTYPE_Q8_1>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0R: return dispatch_q8_linear<PPML_WTYPE_Q8_0R>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0M: {
-            const int force_ll = (flags & PPML_Q8_FLAG_LOW_LATENCY_8) ? 8 : (flags & PPML_Q8_FLAG_LOW_LATENCY_16) ? 16 : 0;
+            const int ll_bits = flags & (PPML_Q8_FLAG_LOW_LATENCY_8 | PPML_Q8_FLAG_LOW_LATENCY_16);
+            const int force_ll = ll_bits == PPML_Q8_FLAG_LOW_LATENCY_32 ? 32 : ll_bits == PPML_Q8_FLAG_LOW_LATENCY_8 ? 8 :
+                                 ll_bits == PPML_Q8_FLAG_LOW_LATENCY_16 ? 16 : 0;
             const int rl = (flags & PPML_Q8_FLAG_NO_LOW_LATENCY) ? -1
                          : (act & 2) ? try_q8_linear_ll<true>(W, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s)
                                      : try_q8_linear_ll<false>(W, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s);

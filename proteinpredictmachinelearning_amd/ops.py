@@ -398,7 +398,7 @@ class Q8Weight:
         return Q8Weight(out, self.M, self.K, WTYPE_Q8_0M)
 
 
-_Q8_PATH_FLAGS = {"auto": 0, "weight-stationary": 4, "general": 4 | 8, "low-latency": 0, "low-latency-8": 16, "low-latency-16": 32,
+_Q8_PATH_FLAGS = {"auto": 0, "weight-stationary": 4, "general": 4 | 8, "low-latency": 0, "low-latency-8": 16, "low-latency-16": 32, "low-latency-32": 48,
                   "weight-stationary-column-parts": 4 | 64, "weight-stationary-whole": 4 | 128}
 
 
@@ -410,7 +410,7 @@ def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = Fals
     ``act`` selects the rule the activations are quantized with: "q8_0" (the CPU contract) or
     "q8_1" (what the reference's CUDA launcher does, src/cuda/MulMatQ8Kernel.cu:483-527).
     ``path`` restricts the kernel choice for a packed weight ("weight-stationary": not the low-latency kernel;
-    "general": neither of the two; "low-latency-8" / "-16": that unit size wherever an instance exists;
+    "general": neither of the two; "low-latency-8" / "-16" / "-32": that unit size wherever an instance exists (32: K = 512 only);
     "weight-stationary-column-parts" / "-whole": that kernel with the columns shared out between work-groups
     wherever an instance exists / never); every choice gives the same bits."""
     if act not in ("q8_0", "q8_1"):

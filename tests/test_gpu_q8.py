@@ -232,6 +232,8 @@ def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packe
         families.append("weight-stationary-column-parts")
     if _has_low_latency_instance(K, M):
         families += ["low-latency-8", "low-latency-16"]
+        if K == 512:
+            families.append("low-latency-32")          # units of 32 tokens: K = 512 only
     for fam in families:
         o2, xq2, sums2 = ops.mul_mat_q8(W, _dev(x), c_trans=1, dump=True, path=fam)
         assert ops.last_q8_path() == _FAMILY_PATH[fam], fam
@@ -254,7 +256,8 @@ def _has_resident_weight_instance(K, M):
 
 
 _FAMILY_PATH = {"general": "general", "weight-stationary": "weight-stationary", "weight-stationary-whole": "weight-stationary",
-                "weight-stationary-column-parts": "weight-stationary", "low-latency-8": "low-latency", "low-latency-16": "low-latency"}
+                "weight-stationary-column-parts": "weight-stationary", "low-latency-8": "low-latency", "low-latency-16": "low-latency",
+                "low-latency-32": "low-latency"}
 
 
 def _has_column_parts_instance(K, M):
@@ -314,7 +317,7 @@ def test_relu_fused_into_the_quantizer(ops, oracle):
     wq = oracle.quantize_q8_0(w)
     W = ops.Q8Weight(_dev(wq.reshape(-1)), 128, 512, ops.WTYPE_Q8_0).pack()
     want = oracle.mul_mat_q8(wq, np.maximum(x, 0.0), wtype=0, c_trans=1, fma=1)
-    for fam in ("auto", "general", "weight-stationary", "low-latency-8", "low-latency-16"):
+    for fam in ("auto", "general", "weight-stationary", "low-latency-8", "low-latency-16", "low-latency-32"):
         got = ops.mul_mat_q8(W, _dev(x), relu=True, path=fam).cpu().numpy()
         assert (got == want).all(), fam
 
@@ -365,6 +368,28 @@ def test_pair_feed_forward_shapes_full(ops, oracle):
     assert _rel_err(y, y_want) <= 1e-5 and (y == y_want).all()
     z_want = oracle.mul_mat_q8(w2q, np.maximum(y_want, 0.0), fma=1)
     assert _rel_err(z, z_want) <= 1e-5 and (z == z_want).all()
+
+
+def test_down_projection_beyond_the_pair_length_takes_units_of_32_tokens(ops, oracle):
+    # K = 512 with more tokens than units of 16 can hold resident (a pair tensor of L = 126: 15876 rows): the
+    # low-latency kernel with units of 32 tokens, two work-groups per CU.  Sampled rows against the oracle, bit for bit;
+    # rows are independent, so slices of 4000 rows (units of 16) must give the same bits; ReLU in front, ragged end.
+    N, K, M = 15876, 512, 128
+    x, w = _inputs(126, N, K, M)
+    wq = oracle.quantize_q8_0(w)
+    W = ops.Q8Weight(_dev(wq.reshape(-1)), M, K, 0).pack()
+    xd = _dev(x)
+    y = ops.mul_mat_q8(W, xd, relu=True)
+    assert ops.last_q8_path() == "low-latency"
+    idx = np.r_[0:40, N - 40:N, np.arange(13, N, 499)]
+    want = oracle.mul_mat_q8(wq, np.maximum(x[idx], 0.0), fma=1)
+    assert (y.cpu().numpy()[idx] == want).all()
+    for r0 in range(0, N, 4000):
+        part = ops.mul_mat_q8(W, xd[r0:r0 + 4000].contiguous(), relu=True)
+        assert torch.equal(part, y[r0:r0 + 4000]), r0
+    y1 = ops.mul_mat_q8(W, xd, relu=True, act="q8_1")
+    part1 = ops.mul_mat_q8(W, xd[:4000].contiguous(), relu=True, act="q8_1")
+    assert torch.equal(part1, y1[:4000])
 
 
 def test_msa_qkv_shape_full_size_properties(ops, oracle):
@@ -465,8 +490,8 @@ def test_fused_linear_with_q8_1_activations(ops, oracle, wname, N, K, M, c_trans
     # a packed weight in the LinearLayer orientation gets the resident-weight kernels under this rule too
     assert (ops.last_q8_path() != "general") == (wname == "packed" and c_trans == 1)
     if wname == "packed" and c_trans == 1:
-        for fam in ("weight-stationary", "weight-stationary-column-parts", "low-latency-8", "low-latency-16"):
-            if fam.startswith("low") and not _has_low_latency_instance(K, M):
+        for fam in ("weight-stationary", "weight-stationary-column-parts", "low-latency-8", "low-latency-16", "low-latency-32"):
+            if fam.startswith("low") and (not _has_low_latency_instance(K, M) or (fam.endswith("32") and K != 512)):
                 continue
             if fam.endswith("parts") and not _has_column_parts_instance(K, M):
                 continue
