@@ -27,18 +27,24 @@ INT8_PEAK_TOPS = 5000.0      # dense int8 MFMA, published
 FP32_MFMA_PEAK_TFLOPS = 157.3
 BF16_MFMA_PEAK_TFLOPS = 2500.0
 
-PREHEAT_MS = 3.0             # untimed load ahead of every event-timed region: the shader clock needs 1-2 ms to settle
-TRAFFIC_PROFILE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "q8_linear_msa_qkv_hbm_traffic.md")
+PREHEAT_MS = 40.0            # untimed load ahead of every timed region: the chip needs 25-30 ms of continuous load to settle
+EVENT_REGION_MS = 5.0        # least length of each of the three event-timed regions
+PROFILES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
+TRAFFIC_PROFILE = os.path.join(PROFILES, "q8_linear_msa_qkv_hbm_traffic.md")
+TRAFFIC_PROFILE_OTHERS = os.path.join(PROFILES, "hbm_traffic_other_configured_shapes.md")
 
 
-def measured_traffic_bytes():
-    """HBM bytes per launch of the dominant kernel as the committed rocprofv3 --pmc summary states them
-    (FETCH_SIZE + WRITE_SIZE, each scaled by the same counter's reading for a 1 GiB copy): the line
-    ``traffic_bytes_per_launch: <integer>`` of profiles/q8_linear_msa_qkv_hbm_traffic.md.  None when the
-    summary is not there."""
+def measured_traffic_bytes(name=None):
+    """HBM bytes per launch as the committed rocprofv3 --pmc summaries state them (FETCH_SIZE + WRITE_SIZE, each
+    scaled by the same counter's reading for a 1 GiB copy).  The dominant kernel: the line
+    ``traffic_bytes_per_launch: <integer>`` of profiles/q8_linear_msa_qkv_hbm_traffic.md; another configured
+    shape: the line ``traffic_bytes_per_launch[<name>]: <integer>`` of
+    profiles/hbm_traffic_other_configured_shapes.md.  None when the summary or the line is not there."""
+    path = TRAFFIC_PROFILE if name is None else TRAFFIC_PROFILE_OTHERS
+    key = r"traffic_bytes_per_launch" + ("" if name is None else r"\[" + re.escape(name) + r"\]")
     try:
-        with open(TRAFFIC_PROFILE) as f:
-            m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", f.read(), flags=re.M)
+        with open(path) as f:
+            m = re.search(r"^" + key + r":\s*(\d+)", f.read(), flags=re.M)
         return int(m.group(1)) if m else None
     except OSError:
         return None
@@ -78,11 +84,28 @@ def main() -> int:
     gen = torch.Generator(device=dev).manual_seed(1)
 
     def time_op(fn, nsets, steps, warmup):
-        """Two clocks, both reported.  Wall: `warmup` untimed steps, then exactly `steps` steps between two
-        device synchronisations (the whole-job figure; after a synchronisation the GPU starts from idle clocks,
-        so short runs read slower here).  Events: the same `steps` steps again between two HIP events on the
-        launch stream, queued directly behind PREHEAT_MS of untimed launches of the same step, so the region
-        runs at the steady clock whatever `steps` is.  Returns (wall s / step, event s / step)."""
+        """Two clocks, both reported; neither depends on the other's length.
+        Pre-heat: PREHEAT_MS of untimed launches of the same step.  After any pause of 10 ms or more the chip runs
+        a load at full speed for about a millisecond, then 15-50 % slower for some 15 ms, and is back at its steady
+        rate after 25-30 ms of continuous load; both clocks below start behind that.
+        Wall: `warmup` untimed steps, one device synchronisation, then exactly `steps` steps up to the next
+        synchronisation (the whole-job figure: it contains the launch latency of the first step).
+        Events: three consecutive regions of `event_steps` launches each between HIP events on the launch stream,
+        event_steps = max(steps, EVENT_REGION_MS / step time) -- a region of fixed length in time, whatever `steps`
+        is -- queued directly behind more untimed launches so that the queue is deep when the first event is
+        reached; the figure is the median region.  Returns (wall s / step, event s / step); details in
+        time_op.last."""
+        for i in range(3):
+            fn(i % nsets)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(5):
+            fn(i % nsets)
+        torch.cuda.synchronize()
+        est = max((time.perf_counter() - t0) / 5, 1e-6)
+        heat = min(40000, int(PREHEAT_MS * 1e-3 / est) + 1)
+        for i in range(heat):
+            fn(i % nsets)
         for i in range(warmup):
             fn(i % nsets)
         torch.cuda.synchronize()
@@ -91,20 +114,31 @@ def main() -> int:
             fn(i % nsets)
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) / steps
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        heat = max(warmup, min(20000, int(PREHEAT_MS * 1e-3 / max(wall, 1e-7)) + 1))
-        for i in range(heat):
+        event_steps = max(steps, min(40000, int(EVENT_REGION_MS * 1e-3 / max(wall, 1e-7)) + 1))
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        for i in range(max(warmup, min(heat, event_steps))):
             fn(i % nsets)
-        e0.record()
-        for i in range(steps):
-            fn(i % nsets)
-        e1.record()
+        marks[0].record()
+        for r in range(3):
+            for i in range(event_steps):
+                fn(i % nsets)
+            marks[r + 1].record()
         torch.cuda.synchronize()
-        return wall, e0.elapsed_time(e1) * 1e-3 / steps
+        regions = sorted(marks[r].elapsed_time(marks[r + 1]) * 1e-3 / event_steps for r in range(3))
+        time_op.last = {"event_steps": event_steps, "event_regions_us": [round(t * 1e6, 2) for t in regions],
+                        "preheat_launches": heat}
+        return wall, regions[1]
+
+    # the event machinery's first use in a process costs some 150 us inside the region that contains it
+    first = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    first[0].record()
+    first[1].record()
+    torch.cuda.synchronize()
+    first[0].elapsed_time(first[1])
 
     # ------------------------------------------------------------------ what the bytes alone cost
     import ctypes as C
-    probe_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "proteinpredictmachinelearning_amd", "lib", "libppml_probe.so")
+    probe_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bench_probe", "libppml_probe.so")
     probe = C.CDLL(probe_path) if os.path.exists(probe_path) else None
     if probe is not None:
         probe.ppml_probe_stream.restype = C.c_int
@@ -178,40 +212,54 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic_bytes(),
                      "kernel": "q8_linear_ws_kernel", "algorithmic_bytes_per_launch": nbytes,
-                     "kernel_us": round(ev * 1e6, 2), "clock": "HIP events on the launch stream, region queued behind preheat_ms of load",
+                     "kernel_us": round(ev * 1e6, 2),
+                     "clock": "HIP events on the launch stream: median of three consecutive regions of event_steps launches, "
+                              "queued behind preheat_ms of load",
+                     "event_steps": time_op.last["event_steps"], "event_regions_us": time_op.last["event_regions_us"],
                      "wall_us": round(wall * 1e6, 2), "frac_wall_clock": round(nbytes / wall / 1e9 / HBM_PEAK_GBS, 4),
+                     "clocks_differ_by_more_than_10_percent": bool(abs(ev - wall) > 0.1 * min(ev, wall)),
                      "int8_mfma_frac": round(nops / ev / 1e12 / INT8_PEAK_TOPS, 4),
                      "bytes_only_us": bytes_only_us(rows * K * 4 + N * K * 34 // 32, rows * N * 4, max(20, args.steps // 4), 5)},
     }
 
     # ------------------------------------------------------------------ CPU baseline (oracle, rank 0)
+    cpu_pair = None
     if not args.no_cpu:
         import numpy as np
         import oracle   # the checker, timed here as a reported baseline only
 
         threads = min(len(os.sched_getaffinity(0)), 16)
-        xq_rows = x0.cpu().numpy()
-        wq = oracle.quantize_q8_0(w0.cpu().numpy())
 
-        def cpu_leg(nthreads, budget_s):
+        def cpu_leg(run, nthreads, budget_s):
             reps, t_cpu = 0, 0.0
             while t_cpu < budget_s and reps < 50:
                 t0 = time.perf_counter()
-                oracle.mul_mat_q8(wq, xq_rows, wtype=0, c_trans=1, fma=1, nthreads=nthreads)
+                run(nthreads)
                 t_cpu += time.perf_counter() - t0
                 reps += 1
             return reps, t_cpu
-        reps, t_cpu = cpu_leg(threads, 10.0)
-        # the reference's own default is PPML_N_THREADS = 4 (src/model/PPML.cpp:3828-3833)
-        reps4, t_cpu4 = cpu_leg(min(4, threads), 8.0)
-        out["cpu_baseline"] = {"value": round(nops * reps / t_cpu / 1e12, 5), "unit": "TOPS", "cores": threads,
-                               "kind": "port",
-                               "sample": f"{reps} full passes of the same 26368x256->768 workload "
-                                         f"(quantize rows + block dot), {t_cpu:.1f} s of CPU time",
-                               "reference_default_threads": {"value": round(nops * reps4 / t_cpu4 / 1e12, 5), "unit": "TOPS",
-                                                             "cores": min(4, threads),
-                                                             "sample": f"{reps4} full passes, {t_cpu4:.1f} s of CPU time"}}
-        del np
+
+        def cpu_pair(run, work, unit, what, budget_all=3.0, budget_ref=2.5):
+            """The CPU oracle on `threads` host threads and on the reference's own default of 4
+            (PPML_N_THREADS, src/model/PPML.cpp:3828-3833); `work` = operations of one pass of `run`."""
+            reps, t_cpu = cpu_leg(run, threads, budget_all)
+            reps4, t_cpu4 = cpu_leg(run, min(4, threads), budget_ref)
+            return {"value": round(work * reps / t_cpu / 1e12, 5), "unit": unit, "cores": threads, "kind": "port",
+                    "sample": f"{reps} passes of {what}, {t_cpu:.1f} s of CPU time",
+                    "reference_default_threads": {"value": round(work * reps4 / t_cpu4 / 1e12, 5), "unit": unit,
+                                                  "cores": min(4, threads),
+                                                  "sample": f"{reps4} passes, {t_cpu4:.1f} s of CPU time"}}
+
+        def q8_cpu(w_dev, x_dev, relu, work, what, **budgets):
+            xh = x_dev.cpu().numpy()
+            wq = oracle.quantize_q8_0(w_dev.cpu().numpy())
+            if relu:
+                return cpu_pair(lambda nt: oracle.mul_mat_q8(wq, np.maximum(xh, 0.0), wtype=0, c_trans=1, fma=1, nthreads=nt),
+                                work, "TOPS", what + " (ReLU + quantize rows + block dot)", **budgets)
+            return cpu_pair(lambda nt: oracle.mul_mat_q8(wq, xh, wtype=0, c_trans=1, fma=1, nthreads=nt),
+                            work, "TOPS", what + " (quantize rows + block dot)", **budgets)
+
+        out["cpu_baseline"] = q8_cpu(w0, x0, False, nops, "the whole 26368x256->768 workload", budget_all=10.0, budget_ref=8.0)
 
     # ------------------------------------------------------------------ the other configured shapes
     if not args.no_extra:
@@ -222,13 +270,17 @@ def main() -> int:
             "pair_ff_up_10609x128_512": (10609, 128, 512, False),
             "pair_ff_down_relu_10609x512_128": (10609, 512, 128, True),
         }.items():
-            f, ns, nb, no, _ = q8_case(r, k, n, relu)
+            f, ns, nb, no, (w_dev, x_dev) = q8_case(r, k, n, relu)
             w_, e_ = time_op(f, ns, steps, warm)
             extra[name] = {"us": round(e_ * 1e6, 2), "TOPS": round(no / e_ / 1e12, 2), "GBps": round(nb / e_ / 1e9, 1),
                            "hbm_frac": round(nb / e_ / 1e9 / HBM_PEAK_GBS, 4), "kernel": ops.last_q8_path(),
+                           "event_steps": time_op.last["event_steps"], "algorithmic_bytes_per_launch": nb,
+                           "traffic": measured_traffic_bytes(name),
                            "bytes_only_us": bytes_only_us(r * k * 4 + n * k * 34 // 32, r * n * 4, steps, warm)}
+            if cpu_pair is not None:
+                extra[name]["cpu_baseline"] = q8_cpu(w_dev, x_dev, relu, no, f"the whole {r}x{k}->{n} workload")
 
-        def f32_case(make, nbytes, flops, name, pipe="fp32", rw=None):
+        def f32_case(make, nbytes, flops, name, pipe="fp32", rw=None, cpu=None):
             # pipe: "fp32" = fp32 MFMA; "bf16x3" = binary32 operands split three ways, six bf16 MFMA
             # products per binary32 product (TFLOPS counts binary32 products, the fraction bf16 ones)
             fn_, ns = make()
@@ -241,6 +293,11 @@ def main() -> int:
                 extra[name]["fp32_mfma_frac"] = round(flops / e_ / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4)
             if rw is not None:                          # (bytes read, bytes written) of an HBM-bound shape
                 extra[name]["bytes_only_us"] = bytes_only_us(rw[0], rw[1], steps, warm)
+                extra[name]["algorithmic_bytes_per_launch"] = nbytes
+                extra[name]["traffic"] = measured_traffic_bytes(name)
+            extra[name]["event_steps"] = time_op.last["event_steps"]
+            if cpu is not None and cpu_pair is not None:
+                extra[name]["cpu_baseline"] = cpu()
 
         keep = []
 

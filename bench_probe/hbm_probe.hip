@@ -1,4 +1,4 @@
-// Measurement aid of bench.py, built into its own small library (lib/libppml_probe.so) and never loaded by the
+// Measurement aid of bench.py, built into its own small library (libppml_probe.so beside this file) and never loaded by the
 // backend: a kernel that only moves bytes -- reads `read_bytes` from src and writes `write_bytes` to dst, 16
 // bytes per lane, fully coalesced, in one pass of a grid sized like the backend's own kernels.  Timed in the
 // same loop as a contraction, it says what a launch that does nothing but that contraction's HBM traffic

@@ -278,6 +278,40 @@ int repeat_back_hip(const float *src, float *dst,
                     int64_t d0, int64_t d1, int64_t d2, int64_t d3,
                     int64_t r0, int64_t r1, int64_t r2, int64_t r3, ppml_hip_stream_t stream);
 
+/* ---- element-wise nodes between the contractions ------------------------------------------------ */
+/* The nodes the reference's graphs put between two matrix multiplications, so that such a graph stays on the
+ * device: FeedForward is linear -> relu -> linear (src/modules/Attention.cpp:1097-1104), the attention logits are
+ * out_prod -> scale -> add(bias) -> softmax (Attention.cpp:264-273).  All are HBM-bound streaming kernels. */
+
+/* replaces scale_cuda (declared src/backend/CUDAKernels.cpp:257, called from kernel_scale_cuda, 992-1004);
+ * semantics of CPUBackend::kernel_scale (src/backend/CPUKernels.cpp:1737-1754): dst[i] = x[i] * scale.
+ * returns 0 ok, 1 bad arguments, 6 launch error. */
+int scale_hip(const float *x, float *dst, float scale, int64_t nelements, ppml_hip_stream_t stream);
+
+/* replaces unary_cuda (declared src/backend/CUDAKernels.cpp:208, called from kernel_unary_cuda, 666-672; its
+ * block_size argument is a launch detail and has no counterpart).  uop is the reference's unary_op value
+ * (include/ppml/ComputeGraph.h:20-39); this backend serves UNARY_OP_RELU = 4, the one between the configured
+ * matrix multiplications: dst[i] = src[i] > 0 ? src[i] : 0 (compute_forward_relu, src/backend/CPUKernels.cpp:
+ * 2649-2657: NaN and -0 give +0).  returns 0 ok, 1 bad arguments or another uop, 6 launch error. */
+int unary_hip(const float *src, float *dst, int64_t n, int uop, ppml_hip_stream_t stream);
+
+/* replaces bcast_elemwise_cuda (declared src/backend/CUDAKernels.cpp:114-118, called from
+ * kernel_elemwise_{add,sub,mul,div}_cuda, 678-712); semantics of CPUBackend::kernel_elemwise
+ * (src/backend/CPUKernels.cpp:446-596): dst[i] = a[i % an] op b[i % bn] for i < n, eop 0 add, 1 sub, 2 mul,
+ * 3 div (IEEE division) -- an operand shorter than dst repeats along dst's flat order, i.e. it covers dst's
+ * innermost dimensions.  an and bn must divide n (the reference reads on through an operand that does not and
+ * only warns, CPUKernels.cpp:507-514; here that is status 1).  returns 0 ok, 1 bad arguments, 6 launch error. */
+int bcast_elemwise_hip(const float *a, const float *b, float *dst, int64_t n, int64_t an, int64_t bn, int eop,
+                       ppml_hip_stream_t stream);
+
+/* replaces softmax_cuda (declared src/backend/CUDAKernels.cpp:153, called from kernel_softmax_cuda, 849-857;
+ * block_size dropped); semantics of CPUBackend::kernel_softmax (src/backend/CPUKernels.cpp:1446-1467): M rows of
+ * N values, output[r][d] = exp(x[r][d] - max_r) * (1 / (sum_d exp(x[r][d] - max_r) + 1e-9)).  The maximum starts
+ * from the row's first element and moves on `>` only (a NaN there makes the whole row NaN, as in the reference).
+ * The sum is formed across a wavefront, not d ascending: results agree with the reference's to rounding
+ * (a few units in the last place), not bit for bit.  returns 0 ok, 1 bad arguments, 6 launch error. */
+int softmax_hip(const float *input, float *output, int M, int N, ppml_hip_stream_t stream);
+
 /* ---- observability (include/ppml/MulMatStats.h:39-169, src/cuda/CUDAKernels.cu:1693-1732) ------ */
 /* MUL_MAT statistics: per (path, M, K, N) the number of launcher calls and the device time of their
  * launches, measured with a pair of events recorded on the launcher's stream (nothing waits; inside a

@@ -39,6 +39,9 @@ void ppml_hip_tensor_set_view(ppml_hip_tensor *t, ppml_hip_tensor *view_src, siz
 /* op_params as in the reference's node (include/ppml/Tensor.h:449-450): 32-bit integers, floats stored by bit pattern */
 void ppml_hip_tensor_set_param(ppml_hip_tensor *t, int index, float value);
 void ppml_hip_tensor_set_param_i32(ppml_hip_tensor *t, int index, int value);
+/* the node's flag bits (include/ppml/Tensor.h:19-22: INPUT = 1, OUTPUT = 2); a tensor marked OUTPUT is never
+ * folded into a neighbouring node by graph_compute */
+void ppml_hip_tensor_set_flag(ppml_hip_tensor *t, int flag);
 size_t ppml_hip_tensor_nbytes(const ppml_hip_tensor *t);
 int ppml_hip_tensor_type(const ppml_hip_tensor *t);
 /* allocate device storage through the backend's BufferType and copy host data in / out */
@@ -58,6 +61,23 @@ void ppml_hip_backend_set_q8_1_activations(ppml_hip_backend *b, int on);
  * reader / they are its only reader; the attention kernel takes the other layout itself and the skipped
  * tensors are never written.  0 (default): every node is executed as it stands. */
 void ppml_hip_backend_set_fuse_attention_bridges(ppml_hip_backend *b, int on);
+/* Folding of element-wise nodes into the contraction beside them.  The rule is the reference's own for eliminating
+ * an intermediate (exactly one reader in the graph, include/ppml/ComputeGraph.h:73-87), plus "not marked OUTPUT";
+ * a folded tensor is never written.
+ *   relu_into_q8 (default 1): an OP_UNARY/RELU read only -- directly or through whole OP_VIEW / OP_RESHAPE nodes --
+ *     by the activation side of a quantized OP_MUL_MAT is applied by that matmul's quantizer
+ *     (src/modules/Attention.cpp:1097-1104); same bits as the two nodes run one after the other.
+ *   scale_into_out_prod (default 1): an OP_SCALE whose source is an OP_OUT_PROD nobody else reads runs as one
+ *     scaled contraction (src/modules/Attention.cpp:264-270); same bits.
+ *   attention_chain (default 0): out_prod(K,Q) -> scale -> [add bias] -> softmax -> permute / permute(V) ->
+ *     out_prod (src/modules/Attention.cpp:264-281) runs as one fused attention launch when no intermediate has
+ *     another reader -- what the reference does itself under PPML_FLASH_ATTN (Attention.cpp:232-262); agrees with
+ *     the node-by-node chain to rounding, not bit for bit. */
+void ppml_hip_backend_set_fuse_relu_into_q8(ppml_hip_backend *b, int on);
+void ppml_hip_backend_set_fuse_scale_into_out_prod(ppml_hip_backend *b, int on);
+void ppml_hip_backend_set_fuse_attention_chain(ppml_hip_backend *b, int on);
+/* how many nodes the last graph_compute folded into a neighbour and did not execute */
+int ppml_hip_backend_nodes_fused_away(const ppml_hip_backend *b);
 /* Matrix pipe of this backend's f32 contractions for the length of each graph_compute: 0 = bf16 pipe through
  * the exact three-way split, 1 = fp32 pipe, anything else = the calling thread's ppml_hip_set_f32_arithmetic
  * choice (default).  A field of the backend object, so backends with different settings do not interfere. */

@@ -30,6 +30,10 @@ enum TensorType : int {
 
 enum TensorOp : int {
     OP_NONE = 0,
+    OP_ADD = 2,
+    OP_SUB = 6,
+    OP_MUL = 7,
+    OP_DIV = 8,
     OP_REPEAT_BACK = 21,
     OP_MUL_MAT = 30,
     OP_OUT_PROD = 32,
@@ -38,13 +42,21 @@ enum TensorOp : int {
     OP_VIEW = 38,
     OP_PERMUTE = 39,
     OP_TRANSPOSE = 40,
+    OP_SOFT_MAX = 47,
     OP_FLASH_ATTN_EXT = 75,
     OP_FLASH_ATTN_BACK = 76,
+    OP_UNARY = 88,
     OP_TRI_MUL = 100,
     OP_TRI_MUL_BACK = 101,
     OP_OUTER_PROD_MEAN = 102,
     OP_OUTER_PROD_MEAN_BACK = 103,
 };
+
+// include/ppml/ComputeGraph.h:20-39: the sub-type of an OP_UNARY node, kept in op_params[0]
+enum UnaryOp : int { UNARY_OP_RELU = 4 };
+
+// include/ppml/Tensor.h:19-22
+enum TensorFlag : int { TENSOR_FLAG_INPUT = 1, TENSOR_FLAG_OUTPUT = 2 };
 
 // include/ppml/Backend.h:168-173
 enum class Status : int { SUCCESS = 0, ALLOC_FAILED, NOT_SUPPORTED, ABORTED };
@@ -70,6 +82,7 @@ struct Tensor {
     Tensor* view_src = nullptr;           // OP_VIEW / OP_RESHAPE share their source's storage
     size_t view_offs = 0;
     int32_t op_params[16] = {0};          // as in the reference: integers, or the bit pattern of a float
+    int32_t flag = 0;                     // TensorFlag bits; a tensor marked OUTPUT is never fused away
 
     float param_f32(int i) const { float f; std::memcpy(&f, &op_params[i], sizeof f); return f; }
     void set_param_f32(int i, float f) { std::memcpy(&op_params[i], &f, sizeof f); }
@@ -116,7 +129,9 @@ private:
 using ComputeGraph = std::vector<Tensor*>;   // nodes in evaluation order
 
 // src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-421 (OP_OUTER_PROD_MEAN, OP_OUTER_PROD_MEAN_BACK),
-// 113-119 (OP_PERMUTE, OP_TRANSPOSE), 395-409 (OP_TRI_MUL, OP_TRI_MUL_BACK), 457-471 (OP_FLASH_ATTN_EXT, OP_FLASH_ATTN_BACK); a function of the node alone, so it can be asked without a device
+// 113-119 (OP_PERMUTE, OP_TRANSPOSE), 395-409 (OP_TRI_MUL, OP_TRI_MUL_BACK), 457-471 (OP_FLASH_ATTN_EXT, OP_FLASH_ATTN_BACK),
+// 94-98 (OP_ADD, OP_SUB, OP_MUL, OP_DIV), 236-237 (OP_SOFT_MAX), 340-344 (OP_SCALE), 470-493 (OP_UNARY); a function of
+// the node alone, so it can be asked without a device
 bool node_supported(const Tensor* node);
 
 // include/ppml/Backend.h:550-605; executor obligations of src/backend/CUDABackend.cpp:708-1086
@@ -146,6 +161,29 @@ public:
     void set_fuse_attention_bridges(bool v) { fuse_attention_bridges_ = v; }
     bool fuse_attention_bridges() const { return fuse_attention_bridges_; }
 
+    // Fusion of the element-wise nodes into the contraction beside them.  The legality rule is the reference's own
+    // for eliminating an intermediate (include/ppml/ComputeGraph.h:73-87): the tensor has exactly one reader in the
+    // graph handed to graph_compute; here it must also not be marked TENSOR_FLAG_OUTPUT.  A fused-away tensor is
+    // never written.  Both are ON by default and give the same bits as the nodes run one by one:
+    //   relu   -- an OP_UNARY/RELU node read only (directly or through whole OP_VIEW / OP_RESHAPE nodes) by the
+    //             activation side of a quantized OP_MUL_MAT is not executed; the matmul's quantizer applies it
+    //             (src/modules/Attention.cpp:1097-1104: linear1 -> relu -> linear2 of the pair feed-forward);
+    //   scale  -- an OP_SCALE whose source is an OP_OUT_PROD nobody else reads runs as one scaled contraction
+    //             (src/modules/Attention.cpp:264-270: the attention logits and their 1/sqrt(D)).
+    void set_fuse_relu_into_q8(bool v) { fuse_relu_into_q8_ = v; }
+    bool fuse_relu_into_q8() const { return fuse_relu_into_q8_; }
+    void set_fuse_scale_into_out_prod(bool v) { fuse_scale_into_out_prod_ = v; }
+    bool fuse_scale_into_out_prod() const { return fuse_scale_into_out_prod_; }
+    // Off by default.  On: the reference's default attention chain (src/modules/Attention.cpp:264-281)
+    //   out_prod(K, Q) -> scale -> [add bias] -> softmax -> permute{1,0,2,3} ; permute{1,0,2,3}(V) -> out_prod
+    // whose intermediates have no other reader runs as one fused attention launch on the graph's own layouts
+    // (what the reference does itself under PPML_FLASH_ATTN, Attention.cpp:232-262).  Results then agree with the
+    // node-by-node chain to rounding, not bit for bit (the softmax sums are formed in another order).
+    void set_fuse_attention_chain(bool v) { fuse_attention_chain_ = v; }
+    bool fuse_attention_chain() const { return fuse_attention_chain_; }
+    // How many nodes the last graph_compute folded into a neighbour and did not execute.
+    size_t nodes_fused_away() const { return nodes_fused_away_; }
+
     // Matrix pipe of this backend's f32 contractions: 0 = bf16 pipe through the exact three-way split, 1 = fp32
     // pipe, -1 (default) = whatever the calling thread has chosen with ppml_hip_set_f32_arithmetic.  Applied
     // for the length of each graph_compute and put back afterwards, so two backends (or threads) with different
@@ -172,6 +210,10 @@ private:
     Status kernel_tri_mul(Tensor* node);
     Status kernel_tri_mul_back(Tensor* node);
     Status kernel_outer_prod_mean_back(Tensor* node);
+    Status kernel_scale(Tensor* node);
+    Status kernel_unary(Tensor* node);
+    Status kernel_elemwise(Tensor* node);
+    Status kernel_soft_max(Tensor* node);
     bool resolve_views(Tensor* node);                    // src/backend/CUDABackend.cpp:800-819
     bool device_pointer_ok(const Tensor* t) const;       // src/backend/CUDABackend.cpp:894-973
     Status fail(Status s, const std::string& why);
@@ -182,7 +224,14 @@ private:
     bool fuse_attention_bridges_ = false;
     int f32_arithmetic_ = -1;
     size_t host_shadows_made_ = 0;
+    bool fuse_relu_into_q8_ = true;
+    bool fuse_scale_into_out_prod_ = true;
+    bool fuse_attention_chain_ = false;
+    size_t nodes_fused_away_ = 0;
     int attn_layout_ = 0;                                // layout bits of the attention node being dispatched
+    bool relu_in_quantizer_ = false;                     // the matmul being dispatched applies a fused-away ReLU
+    float out_prod_alpha_ = 1.0f;                        // scale of a fused-away OP_SCALE behind the out_prod being dispatched
+    bool out_prod_scaled_ = false;
     std::string error_;
     std::vector<std::unique_ptr<Buffer>> owned_;         // node outputs allocated here, packed weights
 };

@@ -88,6 +88,14 @@ def _load() -> C.CDLL:
     lib.orc_flash_attn_backward.argtypes = [C.c_int] * 5 + [C.c_float] + [f32p] * 11
     lib.orc_repeat_back.restype = None
     lib.orc_repeat_back.argtypes = [f32p, f32p, C.c_int, C.POINTER(i64), C.c_int, C.POINTER(i64)]
+    lib.orc_scale.restype = None
+    lib.orc_scale.argtypes = [f32p, f32p, i64, C.c_float, C.c_int]
+    lib.orc_relu.restype = None
+    lib.orc_relu.argtypes = [f32p, f32p, i64, C.c_int]
+    lib.orc_bcast_elemwise.restype = C.c_int
+    lib.orc_bcast_elemwise.argtypes = [f32p, f32p, f32p, i64, i64, i64, C.c_int, C.c_int]
+    lib.orc_softmax.restype = None
+    lib.orc_softmax.argtypes = [f32p, f32p, i64, i64, C.c_int]
     lib.orc_max_threads.restype = C.c_int
     return lib
 
@@ -447,4 +455,44 @@ def repeat_back(src, dst_shape) -> np.ndarray:
     dd = list(dst_shape[::-1]) + [1] * (4 - len(dst_shape))
     out = np.empty(dst_shape, dtype=np.float32)
     lib().orc_repeat_back(_fp(src), _fp(out), src.ndim, (C.c_int64 * 4)(*sd), len(dst_shape), (C.c_int64 * 4)(*dd))
+    return out
+
+
+def scale(x, s, nthreads=0) -> np.ndarray:
+    """kernel_scale (CPUKernels.cpp:1737-1754): x * s element by element."""
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().orc_scale(_fp(x), _fp(out), x.size, float(np.float32(s)), nthreads)
+    return out
+
+
+def relu(x, nthreads=0) -> np.ndarray:
+    """compute_forward_relu (CPUKernels.cpp:2649-2657): (x > 0) ? x : 0."""
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().orc_relu(_fp(x), _fp(out), x.size, nthreads)
+    return out
+
+
+ELEMWISE_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+
+def bcast_elemwise(a, b, op="add", nthreads=0) -> np.ndarray:
+    """kernel_elemwise (CPUKernels.cpp:446-596).  The result has the shape of the larger operand (the reference's
+    dst is a copy of src[0]'s shape); the other one repeats along the flat order, i % numel."""
+    a, b = _f32(a), _f32(b)
+    big = a if a.size >= b.size else b
+    out = np.empty_like(big)
+    rc = lib().orc_bcast_elemwise(_fp(a), _fp(b), _fp(out), big.size, a.size, b.size, ELEMWISE_OPS[op], nthreads)
+    if rc:
+        raise ValueError("orc_bcast_elemwise: bad arguments")
+    return out
+
+
+def softmax(x, nthreads=0) -> np.ndarray:
+    """kernel_softmax (CPUKernels.cpp:1446-1467) over the LAST numpy axis (the reference's dims[0])."""
+    x = _f32(x)
+    out = np.empty_like(x)
+    D = x.shape[-1]
+    lib().orc_softmax(_fp(x), _fp(out), x.size // D, D, nthreads)
     return out

@@ -40,6 +40,16 @@
  *       repeated, the summation order probed with 2^24 + 1 + 1 (sequential from the left gives 2^24,
  *       any pairing of the two ones gives 2^24 + 2), and the dimension alignment of
  *       src/backend/CPUKernels.cpp:2099-2109 (dimension d of dst meets dimension d of src).
+ *   orc_scale, orc_relu, orc_bcast_elemwise : one IEEE operation per element -- numpy's float32 operations
+ *       bit for bit (np.float32 multiply, maximum-with-zero incl. NaN and -0 -> +0, add/sub/mul/div on
+ *       np.resize'd operands, which is the flat-modulo broadcast); the prefix-broadcast case against numpy's
+ *       own dimension-wise broadcasting.  No reference-held vector.
+ *   orc_softmax : float64 softmax within 1e-6 (rows of equal values -> 1/(D + 1e-9 e^0 ...), i.e. the
+ *       closed form 1 / (D + 1e-9) exactly where D is small; a dominant entry -> 1; shift invariance bit for
+ *       bit for shifts that are exact; the 1e-9 in the denominator probed with a one-element row: 1/(1 + 1e-9)
+ *       rounds to 1 in binary32 and exp(0) = 1, while a row of -inf gives NaN), and the composed chain
+ *       scale -> add -> softmax -> second contraction against orc_flash_attn_forward on the golden vectors
+ *       (tests/golden/flash_attn_forward.json).  No reference-held vector of the node itself.
  *   orc_flash_attn_forward : the reference's own src/ops/FlashAttn.cpp compiled as-is
  *       (oracle/_ref/libppml_ref_flash.so: it needs nothing but its header) -- bit-for-bit on
  *       random inputs, with and without bias, causal and not, ragged block sizes; plus float64
@@ -751,5 +761,56 @@ void orc_repeat_back(const float *src, float *dst, int nd_src, const int64_t sd_
                         sum += src[((s3 * sd[2] + s2) * sd[1] + s1) * sd[0] + s0];
                     }
         dst[idx] = sum;
+    }
+}
+
+/* src/backend/CPUKernels.cpp:1737-1754 (kernel_scale): dst[i] = src[i] * s, s from op_params[0]. */
+void orc_scale(const float *src, float *dst, int64_t n, float s, int nthreads) {
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(static) num_threads(nt)
+    for (int64_t i = 0; i < n; ++i) dst[i] = src[i] * s;
+}
+
+/* src/backend/CPUKernels.cpp:2649-2657 (compute_forward_relu): d = (s > 0) ? s : 0 -- NaN and -0 give +0. */
+void orc_relu(const float *src, float *dst, int64_t n, int nthreads) {
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(static) num_threads(nt)
+    for (int64_t i = 0; i < n; ++i) dst[i] = (src[i] > 0.0f) ? src[i] : 0.0f;
+}
+
+/* src/backend/CPUKernels.cpp:446-596 (kernel_elemwise): d[i] = a[a_full ? i : i % an] op b[b_full ? i : i % bn]
+ * (549-592); eop 0 add, 1 sub, 2 mul, 3 div as the CUDA wrapper numbers them (src/backend/CUDAKernels.cpp:678-712).
+ * The AVX2 branch of OP_ADD (542-548) adds the same pairs.  returns 0 ok, 1 bad arguments. */
+int orc_bcast_elemwise(const float *a, const float *b, float *d, int64_t n, int64_t an, int64_t bn, int eop, int nthreads) {
+    if (!a || !b || !d || n < 0 || an <= 0 || bn <= 0 || eop < 0 || eop > 3) return 1;
+    const int a_full = an == n, b_full = bn == n;
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(static) num_threads(nt)
+    for (int64_t i = 0; i < n; ++i) {
+        const float x = a[a_full ? i : i % an], y = b[b_full ? i : i % bn];
+        d[i] = eop == 0 ? x + y : eop == 1 ? x - y : eop == 2 ? x * y : x / y;
+    }
+    return 0;
+}
+
+/* src/backend/CPUKernels.cpp:1446-1467 (kernel_softmax): rows of D = dims[0] values; maximum from the first
+ * element moved by `>` (1459-1460), sum of expf(x - mx) d ascending (1461-1462), inv = 1 / (sum + 1e-9f) (1463),
+ * expf recomputed for the output (1464). */
+void orc_softmax(const float *src, float *dst, int64_t rows, int64_t D, int nthreads) {
+    const int nt = pick_threads(nthreads);
+    (void)nt;
+#pragma omp parallel for schedule(static) num_threads(nt)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float *sr = src + r * D;
+        float *dr = dst + r * D;
+        float mx = sr[0];
+        for (int64_t d = 1; d < D; ++d) if (sr[d] > mx) mx = sr[d];
+        float sum = 0;
+        for (int64_t d = 0; d < D; ++d) sum += expf(sr[d] - mx);
+        const float inv = 1.0f / (sum + 1e-9f);
+        for (int64_t d = 0; d < D; ++d) dr[d] = expf(sr[d] - mx) * inv;
     }
 }

@@ -124,6 +124,14 @@ int orc_flash_attn_backward(int B, int h, int L, int d, int causal, float scale,
  * ranks, sd / dd the sizes (dims[0] innermost), dimension d of dst meets dimension d of src. */
 void orc_repeat_back(const float *src, float *dst, int nd_src, const int64_t sd[4], int nd_dst, const int64_t dd[4]);
 
+/* The element-wise nodes between the contractions (one IEEE operation per element, so thread counts change
+ * nothing): src/backend/CPUKernels.cpp:1737-1754 (kernel_scale), 2649-2657 (compute_forward_relu), 446-596
+ * (kernel_elemwise: flat-modulo broadcast, eop 0 add 1 sub 2 mul 3 div), 1446-1467 (kernel_softmax over dims[0]). */
+void orc_scale(const float *src, float *dst, int64_t n, float s, int nthreads);
+void orc_relu(const float *src, float *dst, int64_t n, int nthreads);
+int orc_bcast_elemwise(const float *a, const float *b, float *d, int64_t n, int64_t an, int64_t bn, int eop, int nthreads);
+void orc_softmax(const float *src, float *dst, int64_t rows, int64_t D, int nthreads);
+
 int orc_max_threads(void);
 
 #ifdef __cplusplus

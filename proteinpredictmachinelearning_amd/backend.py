@@ -17,7 +17,11 @@ from . import cabi
 # tensor_type
 F32, F16, Q8_0, Q8_1, Q8_0R, Q8_0M = 0, 1, 8, 9, 19, 64
 # tensor_op
+OP_ADD, OP_SUB, OP_MUL, OP_DIV = 2, 6, 7, 8
 OP_REPEAT_BACK = 21
+OP_UNARY = 88
+UNARY_OP_RELU = 4                      # include/ppml/ComputeGraph.h:20-25, kept in op_params[0]
+FLAG_INPUT, FLAG_OUTPUT = 1, 2         # include/ppml/Tensor.h:19-22
 OP_NONE, OP_MUL_MAT, OP_OUT_PROD, OP_SCALE, OP_RESHAPE, OP_VIEW, OP_PERMUTE, OP_TRANSPOSE, OP_SOFT_MAX = 0, 30, 32, 33, 37, 38, 39, 40, 47
 OP_FLASH_ATTN_EXT, OP_FLASH_ATTN_BACK, OP_TRI_MUL, OP_TRI_MUL_BACK, OP_OUTER_PROD_MEAN, OP_OUTER_PROD_MEAN_BACK = \
     75, 76, 100, 101, 102, 103
@@ -65,6 +69,11 @@ class Tensor:
             self._lib.ppml_hip_tensor_set_param_i32(self.handle, index, int(value))
         return self
 
+    def set_flag(self, flag: int) -> "Tensor":
+        """The node's flag bits; a tensor marked FLAG_OUTPUT is never folded into a neighbour."""
+        self._lib.ppml_hip_tensor_set_flag(self.handle, int(flag))
+        return self
+
     def view_of(self, base: "Tensor", byte_offset: int = 0) -> "Tensor":
         self._base = base
         self._lib.ppml_hip_tensor_set_view(self.handle, base.handle, byte_offset)
@@ -103,6 +112,20 @@ class Backend:
 
     def set_fuse_attention_bridges(self, on: bool) -> None:
         self._lib.ppml_hip_backend_set_fuse_attention_bridges(self.handle, int(on))
+
+    def set_fuse_relu_into_q8(self, on: bool) -> None:
+        self._lib.ppml_hip_backend_set_fuse_relu_into_q8(self.handle, int(on))
+
+    def set_fuse_scale_into_out_prod(self, on: bool) -> None:
+        self._lib.ppml_hip_backend_set_fuse_scale_into_out_prod(self.handle, int(on))
+
+    def set_fuse_attention_chain(self, on: bool) -> None:
+        self._lib.ppml_hip_backend_set_fuse_attention_chain(self.handle, int(on))
+
+    @property
+    def nodes_fused_away(self) -> int:
+        """Nodes the last graph_compute folded into a neighbour and did not execute."""
+        return self._lib.ppml_hip_backend_nodes_fused_away(self.handle)
 
     def set_f32_arithmetic(self, mode) -> None:
         """"split", "fp32", or None for the calling thread's own choice (ppml_hip_backend_set_f32_arithmetic)."""

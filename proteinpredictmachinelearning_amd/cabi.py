@@ -44,6 +44,10 @@ SIGNATURES = {
     "flash_attn_forward_ex_hip": (_i, [_i] * 5 + [_f, _f, _i] + [_vp] * 6 + [_i, _vp]),
     "permute_hip": (_i, [_vp, _vp, _i64, _i] + [_i] * 4 + [_i64] * 8 + [_vp]),
     "repeat_back_hip": (_i, [_vp, _vp] + [_i64] * 12 + [_vp]),
+    "scale_hip": (_i, [_vp, _vp, _f, _i64, _vp]),
+    "unary_hip": (_i, [_vp, _vp, _i64, _i, _vp]),
+    "bcast_elemwise_hip": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i, _vp]),
+    "softmax_hip": (_i, [_vp, _vp, _i, _i, _vp]),
     "ppml_hip_mulmat_stats": (_i, [C.POINTER(_i64), _i]),
     "ppml_hip_mulmat_stats_enable": (_i, [_i]),
     "ppml_hip_mulmat_stats_rows": (_i, [_vp, _i]),
@@ -74,6 +78,7 @@ BACKEND_SIGNATURES = {
     "ppml_hip_tensor_set_view": (None, [_vp, _vp, C.c_size_t]),
     "ppml_hip_tensor_set_param": (None, [_vp, _i, _f]),
     "ppml_hip_tensor_set_param_i32": (None, [_vp, _i, _i]),
+    "ppml_hip_tensor_set_flag": (None, [_vp, _i]),
     "ppml_hip_tensor_nbytes": (C.c_size_t, [_vp]),
     "ppml_hip_tensor_type": (_i, [_vp]),
     "ppml_hip_tensor_upload": (_i, [_vp, _vp, _vp, C.c_size_t]),
@@ -82,6 +87,10 @@ BACKEND_SIGNATURES = {
     "ppml_hip_backend_set_skip_alloc": (None, [_vp, _i]),
     "ppml_hip_backend_set_q8_1_activations": (None, [_vp, _i]),
     "ppml_hip_backend_set_fuse_attention_bridges": (None, [_vp, _i]),
+    "ppml_hip_backend_set_fuse_relu_into_q8": (None, [_vp, _i]),
+    "ppml_hip_backend_set_fuse_scale_into_out_prod": (None, [_vp, _i]),
+    "ppml_hip_backend_set_fuse_attention_chain": (None, [_vp, _i]),
+    "ppml_hip_backend_nodes_fused_away": (_i, [_vp]),
     "ppml_hip_backend_set_f32_arithmetic": (None, [_vp, _i]),
     "ppml_hip_backend_host_shadows_made": (_i, [_vp]),
     "ppml_hip_backend_graph_compute": (_i, [_vp, C.POINTER(_vp), _i]),

@@ -5,7 +5,8 @@
 //   supports_op      src/backend/CUDABackend.cpp:121-163 (OP_MUL_MAT, OP_OUT_PROD), 410-416 (OP_OUTER_PROD_MEAN)
 //   graph_compute    src/backend/CUDABackend.cpp:708-1086 (skip no-op nodes, resolve view sources,
 //                    refuse host / out-of-buffer pointers, dispatch, launch error -> ABORTED)
-//   node -> launcher src/backend/CUDAKernels.cpp:717-847 (mul_mat), 1537-1565 (out_prod), 1204-1221 (outer_prod_mean)
+//   node -> launcher src/backend/CUDAKernels.cpp:717-847 (mul_mat), 1537-1565 (out_prod), 1204-1221 (outer_prod_mean),
+//                    666-712 (unary, element-wise binary ops), 849-857 (softmax), 992-1004 (scale)
 //
 // Two deliberate differences, both on failure paths only:
 //   * the reference's quantized mul_mat prints and returns normally when the launcher fails, so the
@@ -165,6 +166,25 @@ bool node_supported(const Tensor* node) {
         case OP_OUT_PROD:
             return src0 && src1 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
                    node->type == TENSOR_TYPE_F32;
+        case OP_SCALE:
+            // src/backend/CUDABackend.cpp:340-344
+            return src0 && src0->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32;
+        case OP_UNARY:
+            // src/backend/CUDABackend.cpp:470-493 lists the sub-types its unary kernel has; of those, this
+            // backend has the one that sits between two matrix multiplications
+            return src0 && src0->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32 &&
+                   node->op_params[0] == UNARY_OP_RELU;
+        case OP_ADD:
+        case OP_SUB:
+        case OP_MUL:
+        case OP_DIV:
+            // src/backend/CUDABackend.cpp:94-98 says yes to all four without looking; the kernel behind them is
+            // f32 with operands that repeat along the result's flat order (CUDAKernels.cpp:678-712)
+            return src0 && src1 && src0->type == TENSOR_TYPE_F32 && src1->type == TENSOR_TYPE_F32 &&
+                   node->type == TENSOR_TYPE_F32;
+        case OP_SOFT_MAX:
+            // src/backend/CUDABackend.cpp:236-237 (unconditional there)
+            return src0 && src0->type == TENSOR_TYPE_F32 && node->type == TENSOR_TYPE_F32 && node->dims[0] > 0;
         case OP_TRI_MUL:
             // src/backend/CUDABackend.cpp:395-402: left, right and the result all 4-D f32
             if (!src0 || !src1) return false;
@@ -346,7 +366,10 @@ Status HipBackend::kernel_mul_mat(Tensor* node) {
         const int c_trans = q0 ? 0 : 1;
         rc = mul_mat_q8_ex_hip(w->data, static_cast<const float*>(a->data), static_cast<float*>(node->data),
                                static_cast<int>(Mq), static_cast<int>(Nq), static_cast<int>(K), wtype, c_trans,
-                               q8_1_activations_ ? 2 : 0, nullptr, nullptr, nullptr);
+                               (q8_1_activations_ ? PPML_Q8_FLAG_Q8_1_ACTIVATIONS : 0) | (relu_in_quantizer_ ? PPML_Q8_FLAG_RELU : 0),
+                               nullptr, nullptr, nullptr);
+    } else if (relu_in_quantizer_) {
+        return fail(Status::ABORTED, "mul_mat: a ReLU was folded into a matmul that has no quantizer");
     } else if (s0->type == TENSOR_TYPE_F16 && s1->type == TENSOR_TYPE_F16) {
         // src/backend/CUDAKernels.cpp:794-821: F16 x F16 -> F32, no bias epilogue on this path
         if (bias) return fail(Status::NOT_SUPPORTED, "mul_mat: the F16 path has no bias epilogue");
@@ -371,7 +394,12 @@ Status HipBackend::kernel_out_prod(Tensor* node) {
     const Tensor* b = node->src[1];
     if (!a || !b) return fail(Status::NOT_SUPPORTED, "out_prod: missing source");
     // the reference clears dst first and accumulates; the launcher overwrites dst instead
-    const int rc = out_prod_hip(static_cast<const float*>(a->data), static_cast<const float*>(b->data),
+    const int rc = out_prod_scaled_ ? out_prod_scaled_hip(static_cast<const float*>(a->data), static_cast<const float*>(b->data),
+                                static_cast<float*>(node->data),
+                                a->dims[0], a->dims[1], dim_or_1(a, 2), dim_or_1(a, 3),
+                                b->dims[0], b->dims[1], dim_or_1(b, 2), dim_or_1(b, 3),
+                                node->dims[0], node->dims[1], dim_or_1(node, 2), dim_or_1(node, 3), out_prod_alpha_, nullptr)
+                                    : out_prod_hip(static_cast<const float*>(a->data), static_cast<const float*>(b->data),
                                 static_cast<float*>(node->data),
                                 a->dims[0], a->dims[1], dim_or_1(a, 2), dim_or_1(a, 3),
                                 b->dims[0], b->dims[1], dim_or_1(b, 2), dim_or_1(b, 3),
@@ -564,6 +592,50 @@ Status HipBackend::kernel_repeat_back(Tensor* node) {
     return Status::SUCCESS;
 }
 
+// src/backend/CUDAKernels.cpp:992-1004: dst = src * s, s the float in op_params[0]
+Status HipBackend::kernel_scale(Tensor* node) {
+    const Tensor* a = node->src[0];
+    if (!a || !a->data || !node->data) return fail(Status::NOT_SUPPORTED, "scale: unbound tensor");
+    if (a->numel() != node->numel()) return fail(Status::NOT_SUPPORTED, "scale: source and result differ in size");
+    const int rc = scale_hip(static_cast<const float*>(a->data), static_cast<float*>(node->data), node->param_f32(0), node->numel(), nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("scale: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
+// src/backend/CUDAKernels.cpp:666-672: the sub-type rides in op_params[0]
+Status HipBackend::kernel_unary(Tensor* node) {
+    const Tensor* a = node->src[0];
+    if (!a || !a->data || !node->data) return fail(Status::NOT_SUPPORTED, "unary: unbound tensor");
+    if (a->numel() != node->numel()) return fail(Status::NOT_SUPPORTED, "unary: source and result differ in size");
+    const int rc = unary_hip(static_cast<const float*>(a->data), static_cast<float*>(node->data), node->numel(), node->op_params[0], nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("unary: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
+// src/backend/CUDAKernels.cpp:678-712: n, an, bn are the element counts of the node and of its two sources
+Status HipBackend::kernel_elemwise(Tensor* node) {
+    const Tensor* a = node->src[0];
+    const Tensor* b = node->src[1];
+    if (!a || !b || !a->data || !b->data || !node->data) return fail(Status::NOT_SUPPORTED, "elemwise: unbound tensor");
+    const int eop = node->op == OP_ADD ? 0 : node->op == OP_SUB ? 1 : node->op == OP_MUL ? 2 : 3;
+    const int rc = bcast_elemwise_hip(static_cast<const float*>(a->data), static_cast<const float*>(b->data),
+                                      static_cast<float*>(node->data), node->numel(), a->numel(), b->numel(), eop, nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("elemwise: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
+// src/backend/CUDAKernels.cpp:849-857: rows of dims[0] values
+Status HipBackend::kernel_soft_max(Tensor* node) {
+    const Tensor* a = node->src[0];
+    if (!a || !a->data || !node->data) return fail(Status::NOT_SUPPORTED, "soft_max: unbound tensor");
+    const int64_t N = node->dims[0], M = N > 0 ? node->numel() / N : 0;
+    if (a->numel() != node->numel() || N <= 0 || N > 0x7fffffffLL || M > 0x7fffffffLL)
+        return fail(Status::NOT_SUPPORTED, "soft_max: sizes outside what one launch takes");
+    const int rc = softmax_hip(static_cast<const float*>(a->data), static_cast<float*>(node->data), static_cast<int>(M), static_cast<int>(N), nullptr);
+    if (rc != 0) return fail(status_of_rc(rc), std::string("soft_max: ") + ppml_hip_last_error());
+    return Status::SUCCESS;
+}
+
 Status HipBackend::dispatch_node(Tensor* node) {
     switch (node->op) {
         case OP_MUL_MAT: return kernel_mul_mat(node);
@@ -577,6 +649,13 @@ Status HipBackend::dispatch_node(Tensor* node) {
         case OP_TRI_MUL: return kernel_tri_mul(node);
         case OP_TRI_MUL_BACK: return kernel_tri_mul_back(node);
         case OP_OUTER_PROD_MEAN_BACK: return kernel_outer_prod_mean_back(node);
+        case OP_SCALE: return kernel_scale(node);
+        case OP_UNARY: return kernel_unary(node);
+        case OP_ADD:
+        case OP_SUB:
+        case OP_MUL:
+        case OP_DIV: return kernel_elemwise(node);
+        case OP_SOFT_MAX: return kernel_soft_max(node);
         default: return fail(Status::NOT_SUPPORTED, "no kernel for op " + std::to_string(node->op));
     }
 }
@@ -589,44 +668,152 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
     }
     error_.clear();
 
-    // Optional fusion of the layout bridges around fused attention nodes (ComputeGraphHelper.cpp:456-458,
-    // 483): a permutation {1,0,2,3} that feeds only the attention node, or is the only reader of its result,
-    // is not executed; the attention kernel reads / writes that layout itself.  All three inputs fuse
-    // together or not at all.
-    struct Bridges { bool in = false; Tensor* out = nullptr; };
-    std::unordered_map<const Tensor*, Bridges> fused;
+    // ---- fusion plan.  Legality is the reference's own rule for eliminating an intermediate: exactly one reader
+    // in this graph (include/ppml/ComputeGraph.h:73-87), and here also no TENSOR_FLAG_OUTPUT.  A tensor fused away
+    // is never written.
+    struct Plan {
+        bool bridges_in = false;            // fused attention node: the three leading {1,0,2,3} permutations are skipped
+        Tensor* bridge_out = nullptr;       // ... and this trailing one, whose storage the node writes
+        int relu_slot = -1;                 // quantized mul_mat: activation slot whose chain ends in a skipped ReLU
+        Tensor* relu = nullptr;
+        Tensor* out_prod = nullptr;         // OP_SCALE node that runs as the (skipped) out_prod it reads, scaled
+        bool chain = false;                 // out_prod(attn_t, V_t) that runs as the whole attention chain
+        Tensor *q = nullptr, *k = nullptr, *v = nullptr, *bias = nullptr;
+        float scale = 1.0f;
+    };
+    std::unordered_map<const Tensor*, Plan> plans;
     std::unordered_set<const Tensor*> skipped;
-    if (fuse_attention_bridges_) {
+    nodes_fused_away_ = 0;
+    if (fuse_attention_bridges_ || fuse_relu_into_q8_ || fuse_scale_into_out_prod_ || fuse_attention_chain_) {
         std::unordered_map<const Tensor*, int> uses, position;
         std::unordered_map<const Tensor*, Tensor*> single_user;
         int pos = 0;
         for (Tensor* n : *graph) {
             if (!n) continue;
             position[n] = pos++;
-            for (Tensor* s : n->src) if (s) { ++uses[s]; single_user[s] = n; }
+            bool view_counted = false;
+            for (Tensor* s : n->src) if (s) { ++uses[s]; single_user[s] = n; view_counted = view_counted || s == n->view_src; }
+            if (n->view_src && !view_counted) { ++uses[n->view_src]; single_user[n->view_src] = n; }
         }
+        const auto before = [&](const Tensor* a, const Tensor* b) {
+            const auto ia = position.find(a), ib = position.find(b);
+            return ia != position.end() && ib != position.end() && ia->second < ib->second;
+        };
+        // an intermediate this graph computes that only `reader` reads and nobody outside is promised
+        const auto private_to = [&](const Tensor* t, const Tensor* reader) {
+            return t && !(t->flag & TENSOR_FLAG_OUTPUT) && !t->view_src && t->type == TENSOR_TYPE_F32 && uses[t] == 1 &&
+                   before(t, reader) && !skipped.count(t);
+        };
         const auto is_bridge = [](const Tensor* t) {
             if (!t || (t->op != OP_PERMUTE && t->op != OP_TRANSPOSE) || t->ndim != 4 || t->type != TENSOR_TYPE_F32) return false;
             return t->op_params[0] == 1 && t->op_params[1] == 0 && t->op_params[2] == 2 && t->op_params[3] == 3 &&
                    t->src[0] && t->src[0]->type == TENSOR_TYPE_F32 && t->src[0]->ndim == 4 && !t->view_src;
         };
-        for (Tensor* n : *graph) {
-            if (!n || n->op != OP_FLASH_ATTN_EXT || !node_supported(n)) continue;
-            Bridges b;
-            b.in = true;
-            for (int s = 0; s < 3; ++s) {
-                const Tensor* pq = n->src[s];
-                b.in = b.in && is_bridge(pq) && uses[pq] == 1 && position.count(pq) && position[pq] < position[n];
+
+        // (1) the layout bridges around fused attention nodes (ComputeGraphHelper.cpp:456-458, 483): a permutation
+        // {1,0,2,3} that feeds only the attention node, or is the only reader of its result, is not executed; the
+        // attention kernel reads / writes that layout itself.  All three inputs fuse together or not at all.
+        if (fuse_attention_bridges_) {
+            for (Tensor* n : *graph) {
+                if (!n || n->op != OP_FLASH_ATTN_EXT || !node_supported(n)) continue;
+                Plan b;
+                b.bridges_in = true;
+                for (int s = 0; s < 3; ++s) {
+                    const Tensor* pq = n->src[s];
+                    b.bridges_in = b.bridges_in && is_bridge(pq) && uses[pq] == 1 && before(pq, n);
+                }
+                // a tensor that feeds two of the three slots (self-attention on one projection) has uses == 2: not fused
+                Tensor* user = uses[n] == 1 ? single_user[n] : nullptr;
+                if (user && is_bridge(user) && user->src[0] == n && before(n, user)) b.bridge_out = user;
+                if (!b.bridges_in && !b.bridge_out) continue;
+                plans[n] = b;
+                if (b.bridges_in) for (int s = 0; s < 3; ++s) skipped.insert(n->src[s]);
+                if (b.bridge_out) skipped.insert(b.bridge_out);
             }
-            // a tensor that feeds two of the three slots (self-attention on one projection) has uses == 2: not fused
-            Tensor* user = uses[n] == 1 ? single_user[n] : nullptr;
-            if (user && is_bridge(user) && user->src[0] == n && position.count(user) && position[user] > position[n])
-                b.out = user;
-            if (!b.in && !b.out) continue;
-            fused[n] = b;
-            if (b.in) for (int s = 0; s < 3; ++s) skipped.insert(n->src[s]);
-            if (b.out) skipped.insert(b.out);
         }
+
+        // (2) the reference's default attention chain (src/modules/Attention.cpp:264-281) as one fused launch
+        if (fuse_attention_chain_) {
+            for (Tensor* n : *graph) {
+                if (!n || n->op != OP_OUT_PROD || n->type != TENSOR_TYPE_F32 || n->ndim != 4) continue;
+                Tensor* attn_t = n->src[0];
+                Tensor* v_t = n->src[1];
+                if (!is_bridge(attn_t) || !is_bridge(v_t) || !private_to(attn_t, n) || !private_to(v_t, n)) continue;
+                Tensor* attn = attn_t->src[0];
+                if (!attn || attn->op != OP_SOFT_MAX || !private_to(attn, attn_t)) continue;
+                Tensor* x = attn->src[0];
+                Tensor* bias = nullptr;
+                Tensor* added = nullptr;
+                if (x && x->op == OP_ADD) {
+                    if (!private_to(x, attn) || !x->src[0] || !x->src[1] || x->src[1]->numel() != x->numel() ||
+                        x->src[1]->type != TENSOR_TYPE_F32) continue;
+                    added = x;
+                    bias = x->src[1];
+                    x = x->src[0];
+                }
+                if (!x || x->op != OP_SCALE || !private_to(x, added ? added : attn)) continue;
+                Tensor* scores = x->src[0];
+                if (!scores || scores->op != OP_OUT_PROD || !private_to(scores, x)) continue;
+                Tensor* k = scores->src[0];
+                Tensor* q = scores->src[1];
+                Tensor* v = v_t->src[0];
+                const auto plain4 = [](const Tensor* t) { return t && t->type == TENSOR_TYPE_F32 && t->ndim == 4; };
+                if (!plain4(k) || !plain4(q) || !plain4(v)) continue;
+                const int64_t L = q->dims[0], D = q->dims[1];
+                bool same = true;
+                for (int d = 0; d < 4; ++d) same = same && k->dims[d] == q->dims[d] && v->dims[d] == q->dims[d];
+                if (!same || D <= 0 || D > 64 || (D % 4) != 0) continue;           // the fused kernel's own range
+                if (n->numel() != q->numel() || scores->numel() != L * L * q->dims[2] * q->dims[3]) continue;
+                Plan c;
+                c.chain = true;
+                c.q = q; c.k = k; c.v = v; c.bias = bias;
+                c.scale = x->param_f32(0);
+                plans[n] = c;
+                for (const Tensor* t : {static_cast<const Tensor*>(attn_t), static_cast<const Tensor*>(v_t),
+                                        static_cast<const Tensor*>(attn), static_cast<const Tensor*>(added),
+                                        static_cast<const Tensor*>(x), static_cast<const Tensor*>(scores)})
+                    if (t) skipped.insert(t);
+            }
+        }
+
+        // (3) ReLU in front of a quantized matmul (src/modules/Attention.cpp:1097-1104; in evaluation the dropout
+        // between them is the identity, src/ops/Dropout.cpp:87-91): the matmul's quantizer applies it
+        if (fuse_relu_into_q8_) {
+            for (Tensor* n : *graph) {
+                if (!n || n->op != OP_MUL_MAT || !node_supported(n) || !n->src[0] || !n->src[1]) continue;
+                const bool q0 = is_quantized_type(n->src[0]->type), q1 = is_quantized_type(n->src[1]->type);
+                if (q0 == q1) continue;
+                const int slot = q0 ? 1 : 0;
+                const Tensor* reader = n;
+                Tensor* t = n->src[slot];
+                // through whole views: same element count, no offset, nobody else looking
+                for (int guard = 0; guard < 16 && t && (t->op == OP_VIEW || t->op == OP_RESHAPE); ++guard) {
+                    Tensor* from = t->view_src ? t->view_src : t->src[0];
+                    if (!from || (t->flag & TENSOR_FLAG_OUTPUT) || uses[t] != 1 || t->view_offs != 0 || from->numel() != t->numel() ||
+                        !before(t, reader)) { t = nullptr; break; }
+                    reader = t;
+                    t = from;
+                }
+                if (!t || t->op != OP_UNARY || t->op_params[0] != UNARY_OP_RELU || !private_to(t, reader)) continue;
+                if (!t->src[0] || t->src[0]->type != TENSOR_TYPE_F32 || t->src[0]->numel() != t->numel()) continue;
+                Plan& r = plans[n];
+                r.relu_slot = slot;
+                r.relu = t;
+                skipped.insert(t);
+            }
+        }
+
+        // (4) the 1/sqrt(D) behind the attention logits (src/modules/Attention.cpp:264-270)
+        if (fuse_scale_into_out_prod_) {
+            for (Tensor* n : *graph) {
+                if (!n || n->op != OP_SCALE || skipped.count(n) || !node_supported(n)) continue;
+                Tensor* p = n->src[0];
+                if (!p || p->op != OP_OUT_PROD || !node_supported(p) || !private_to(p, n) || p->numel() != n->numel()) continue;
+                plans[n].out_prod = p;
+                skipped.insert(p);
+            }
+        }
+        nodes_fused_away_ = skipped.size();
     }
 
     // the arithmetic this backend's f32 contractions were configured with, for the length of this call
@@ -649,23 +836,58 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         if (!supports_op(node))
             return fail(Status::NOT_SUPPORTED, "op " + std::to_string(node->op) + " (node " + std::to_string(index) + ") is not supported");
 
-        // the node as it is executed: for a fused attention node a copy whose sources are the bridges'
-        // sources and whose storage is the trailing bridge's
+        // the node as it is executed: a copy with other sources / storage where the plan folded neighbours into it
         Tensor rewired;
+        Tensor alias;                                   // a folded ReLU's input, seen through the matmul's own view of it
         Tensor* exec = node;
         Tensor* storage = node;
         attn_layout_ = 0;
-        const auto plan = fused.find(node);
-        if (plan != fused.end()) {
+        relu_in_quantizer_ = false;
+        out_prod_scaled_ = false;
+        const auto plan = plans.find(node);
+        if (plan != plans.end()) {
+            const Plan& pl = plan->second;
             rewired = *node;
             exec = &rewired;
-            if (plan->second.in) {
+            if (pl.bridges_in) {
                 for (int s = 0; s < 3; ++s) rewired.src[s] = node->src[s]->src[0];
                 attn_layout_ |= 1;
             }
-            if (plan->second.out) {
-                storage = plan->second.out;
+            if (pl.bridge_out) {
+                storage = pl.bridge_out;
                 attn_layout_ |= 2;
+            }
+            if (pl.relu) {
+                resolve_views(pl.relu);                 // binds the ReLU's own source if it is a view
+                Tensor* in = pl.relu->src[0];
+                if (!skip_alloc_) shadows.cover(in);
+                alias = *node->src[pl.relu_slot];
+                alias.op = OP_NONE;
+                alias.view_src = nullptr;
+                alias.view_offs = 0;
+                alias.src[0] = nullptr;
+                alias.data = in->data;
+                alias.buffer = in->buffer;
+                alias.buffer_offs = in->buffer_offs;
+                rewired.src[pl.relu_slot] = &alias;
+                relu_in_quantizer_ = true;
+            }
+            if (pl.out_prod) {
+                rewired.op = OP_OUT_PROD;
+                for (int s = 0; s < 10; ++s) rewired.src[s] = pl.out_prod->src[s];
+                out_prod_scaled_ = true;
+                out_prod_alpha_ = node->param_f32(0);
+            }
+            if (pl.chain) {
+                // src/core/ComputeGraphHelper.cpp:450-484: Q, K, V, bias in src 0..3; scale, causal, eps, Br, Bc
+                rewired.op = OP_FLASH_ATTN_EXT;
+                for (int s = 0; s < 10; ++s) rewired.src[s] = nullptr;
+                rewired.src[0] = pl.q; rewired.src[1] = pl.k; rewired.src[2] = pl.v; rewired.src[3] = pl.bias;
+                for (int32_t& w : rewired.op_params) w = 0;
+                rewired.set_param_f32(0, pl.scale);
+                rewired.set_param_f32(2, 1e-9f);        // kernel_softmax's 1 / (sum + 1e-9), CPUKernels.cpp:1463
+                rewired.op_params[4] = 64;
+                attn_layout_ = 3;                       // inputs [L, D, h, B] as they are, result [L, D, h, B]
             }
         }
         resolve_views(exec);
@@ -696,7 +918,7 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
             out->buffer_offs = 0;
             owned_.push_back(std::move(buf));
         }
-        if (storage != node) {
+        if (exec != node) {                             // the copy was taken before its storage was settled
             rewired.data = storage->data;
             rewired.buffer = storage->buffer;
             rewired.buffer_offs = storage->buffer_offs;
@@ -712,6 +934,8 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
 
         const Status st = dispatch_node(exec);
         attn_layout_ = 0;
+        relu_in_quantizer_ = false;
+        out_prod_scaled_ = false;
         if (st != Status::SUCCESS) return st;
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess)
@@ -808,6 +1032,9 @@ void ppml_hip_tensor_set_param(ppml_hip_tensor* t, int index, float value) {
 void ppml_hip_tensor_set_param_i32(ppml_hip_tensor* t, int index, int value) {
     if (t && index >= 0 && index < 16) t->t.op_params[index] = value;
 }
+void ppml_hip_tensor_set_flag(ppml_hip_tensor* t, int flag) {
+    if (t) t->t.flag = flag;
+}
 size_t ppml_hip_tensor_nbytes(const ppml_hip_tensor* t) { return t ? t->t.nbytes() : 0; }
 int ppml_hip_tensor_type(const ppml_hip_tensor* t) { return t ? t->t.type : -1; }
 
@@ -853,6 +1080,18 @@ void ppml_hip_backend_set_q8_1_activations(ppml_hip_backend* b, int on) {
 }
 void ppml_hip_backend_set_fuse_attention_bridges(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_fuse_attention_bridges(on != 0);
+}
+void ppml_hip_backend_set_fuse_relu_into_q8(ppml_hip_backend* b, int on) {
+    if (b) b->impl.set_fuse_relu_into_q8(on != 0);
+}
+void ppml_hip_backend_set_fuse_scale_into_out_prod(ppml_hip_backend* b, int on) {
+    if (b) b->impl.set_fuse_scale_into_out_prod(on != 0);
+}
+void ppml_hip_backend_set_fuse_attention_chain(ppml_hip_backend* b, int on) {
+    if (b) b->impl.set_fuse_attention_chain(on != 0);
+}
+int ppml_hip_backend_nodes_fused_away(const ppml_hip_backend* b) {
+    return b ? static_cast<int>(b->impl.nodes_fused_away()) : 0;
 }
 void ppml_hip_backend_set_skip_alloc(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_skip_alloc(on != 0);

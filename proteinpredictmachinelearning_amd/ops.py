@@ -326,6 +326,55 @@ def repeat_back(a: torch.Tensor, b_shape) -> torch.Tensor:
 
 
 # ----------------------------------------------------------------------------- Q8_0
+def scale(x: torch.Tensor, s: float) -> torch.Tensor:
+    """The reference's scale() node (src/core/ComputeGraphHelper.cpp:235-243; kernel src/backend/CPUKernels.cpp:1737-1754)."""
+    x = _dev_f32(x, "x")
+    out = torch.empty_like(x)
+    cabi.check("scale_hip", _lib().scale_hip(_ptr(x), _ptr(out), float(s), x.numel(), _stream()))
+    return out
+
+
+UNARY_OP_RELU = 4
+
+
+def relu(x: torch.Tensor) -> torch.Tensor:
+    """The reference's relu() node (src/core/ComputeGraphHelper.cpp:513-520; kernel src/backend/CPUKernels.cpp:2649-2657)."""
+    x = _dev_f32(x, "x")
+    out = torch.empty_like(x)
+    cabi.check("unary_hip", _lib().unary_hip(_ptr(x), _ptr(out), x.numel(), UNARY_OP_RELU, _stream()))
+    return out
+
+
+ELEMWISE_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+
+def bcast_elemwise(a: torch.Tensor, b: torch.Tensor, op: str = "add") -> torch.Tensor:
+    """add / sub / mul / div with the reference's broadcast (src/backend/CPUKernels.cpp:446-596): the result has
+    the shape of `a` (the reference's dst is a copy of src[0]'s shape, ComputeGraphHelper.cpp:61-124) and an operand
+    with fewer elements repeats along the flat order, so it must cover the innermost dimensions."""
+    a, b = _dev_f32(a, "a"), _dev_f32(b, "b")
+    if op not in ELEMWISE_OPS:
+        raise ValueError(f"bcast_elemwise: op must be one of {sorted(ELEMWISE_OPS)}")
+    n = a.numel()
+    if b.numel() == 0 or b.numel() > n or n % b.numel() != 0:
+        raise ValueError(f"bcast_elemwise: {b.numel()} elements do not repeat into {n}")
+    out = torch.empty_like(a)
+    cabi.check("bcast_elemwise_hip", _lib().bcast_elemwise_hip(_ptr(a), _ptr(b), _ptr(out), n, n, b.numel(), ELEMWISE_OPS[op], _stream()))
+    return out
+
+
+def softmax(x: torch.Tensor) -> torch.Tensor:
+    """The reference's softmax() node over dims[0], the LAST torch dimension (src/core/ComputeGraphHelper.cpp:420-425;
+    kernel src/backend/CPUKernels.cpp:1446-1467, incl. its 1 / (sum + 1e-9))."""
+    x = _dev_f32(x, "x")
+    if x.dim() < 1 or x.shape[-1] == 0:
+        raise ValueError("softmax: needs a non-empty innermost dimension")
+    out = torch.empty_like(x)
+    N = x.shape[-1]
+    cabi.check("softmax_hip", _lib().softmax_hip(_ptr(x), _ptr(out), x.numel() // N, N, _stream()))
+    return out
+
+
 def quantize_rows_q8_0(x: torch.Tensor) -> torch.Tensor:
     """f32 [..., K] -> uint8 [..., K/32, 34] block_q8_0 records (include/ppml/QuantBlocks.h:62-79)."""
     x = _dev_f32(x, "x")

@@ -56,8 +56,28 @@ def test_supports_op_other_ops():
     # no-op nodes are accepted (and skipped by the executor); everything else belongs to other backends
     assert B.supports_op(B.Tensor((4,), B.F32, B.OP_VIEW, [a]))
     assert B.supports_op(B.Tensor((4,), B.F32, B.OP_RESHAPE, [a]))
-    assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_SCALE, [a]))
-    assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_SOFT_MAX, [a]))
+    assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, 24, [a]))          # OP_NORM: not on this path
+
+
+def test_supports_op_elementwise_nodes_between_the_contractions():
+    # src/backend/CUDABackend.cpp:340-344 OP_SCALE, 470-493 OP_UNARY (sub-type in op_params[0]),
+    # 94-98 OP_ADD..OP_DIV, 236-237 OP_SOFT_MAX -- all f32 here
+    a = B.Tensor((4, 3, 2, 2))
+    h = B.Tensor((4, 3, 2, 2), B.F16)
+    assert B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_SCALE, [a]))
+    assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_SCALE, []))
+    assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_SCALE, [h]))
+    assert B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_SOFT_MAX, [a]))
+    assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F16, B.OP_SOFT_MAX, [a]))
+    relu = B.Tensor((4, 3, 2, 2), B.F32, B.OP_UNARY, [a]).set_param(0, B.UNARY_OP_RELU)
+    assert B.supports_op(relu)
+    for other in (0, 5, 7, 10, 13):              # ABS, GELU, SILU, SIGMOID, EXP: the CUDA backend's, not this path's
+        assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, B.OP_UNARY, [a]).set_param(0, other))
+    bias = B.Tensor((4, 3))
+    for op in (B.OP_ADD, B.OP_SUB, B.OP_MUL, B.OP_DIV):
+        assert B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, op, [a, bias]))
+        assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, op, [a]))
+        assert not B.supports_op(B.Tensor((4, 3, 2, 2), B.F32, op, [a, h]))
 
 
 def test_supports_op_fused_attention():

@@ -374,7 +374,9 @@ def test_failure_statuses(be):
     a = _leaf(be, np.ones((3, 4), np.float32))
     b = _leaf(be, np.ones((5, 4), np.float32))
     # an op without a kernel here: NOT_SUPPORTED, nothing launched
-    assert be.graph_compute([B.Tensor((4, 3), B.F32, B.OP_SCALE, [a])]) == B.NOT_SUPPORTED
+    assert be.graph_compute([B.Tensor((4, 3), B.F32, 24, [a])]) == B.NOT_SUPPORTED          # OP_NORM
+    # a unary sub-type this path does not carry (op_params[0] = 7, SILU)
+    assert be.graph_compute([B.Tensor((4, 3), B.F32, B.OP_UNARY, [a]).set_param(0, 7)]) == B.NOT_SUPPORTED
     # a source nobody bound
     ghost = B.Tensor((4, 5))
     assert be.graph_compute([B.Tensor((5, 3), B.F32, B.OP_MUL_MAT, [a, ghost])]) == B.NOT_SUPPORTED
@@ -511,3 +513,219 @@ def test_f32_arithmetic_is_a_field_of_the_backend(be, oracle):
         assert ops.set_f32_arithmetic("split") == "split"        # the thread's setting came back after each call
     finally:
         other.set_f32_arithmetic(None)
+
+
+# ----------------------------------------------------------------------------- element-wise nodes and their folding
+def _q8_leaf(be, oracle, w, layout):
+    """A quantized weight leaf [K, F] in one of the layouts the reference's loader produces (PPML.cpp:4504-4528)."""
+    F, K = w.shape
+    wq = oracle.quantize_q8_0(w)
+    if layout == "Q8_0R":
+        t = _leaf(be, np.frombuffer(oracle.repack_q8_0(wq).tobytes(), np.uint8), B.Q8_0R, (K, F))
+    else:
+        t = _leaf(be, np.frombuffer(wq.tobytes(), np.uint8), B.Q8_0, (K, F))
+        if layout == "packed":
+            assert be.pack_weight(t) == B.SUCCESS, be.last_error
+    return t, wq
+
+
+def _feed_forward_graph(be, x_leaf, w1, w2, L, D, H):
+    """FeedForward::forward_graph without its layer norm (src/modules/Attention.cpp:1097-1104; dropout is the identity
+    in evaluation, src/ops/Dropout.cpp:87-91), each linear as LinearLayer::forward_graph builds it
+    (src/model/Embedding.cpp:120-153): view to [D_in, tokens] -> mul_mat -> view back."""
+    tok = L * L
+    x_flat = B.Tensor((D, tok), B.F32, B.OP_VIEW).view_of(x_leaf)
+    h_flat = B.Tensor((H, tok), B.F32, B.OP_MUL_MAT, [x_flat, w1])
+    h = B.Tensor((H, L, L, 1), B.F32, B.OP_VIEW).view_of(h_flat)
+    r = B.Tensor((H, L, L, 1), B.F32, B.OP_UNARY, [h]).set_param(0, B.UNARY_OP_RELU)
+    r_flat = B.Tensor((H, tok), B.F32, B.OP_VIEW).view_of(r)
+    y_flat = B.Tensor((D, tok), B.F32, B.OP_MUL_MAT, [r_flat, w2])
+    y = B.Tensor((D, L, L, 1), B.F32, B.OP_VIEW).view_of(y_flat)
+    return [x_flat, h_flat, h, r, r_flat, y_flat, y], r, y_flat
+
+
+@pytest.mark.parametrize("layout", ["Q8_0R", "packed"])
+@pytest.mark.parametrize("L", [19, 103])
+def test_pair_feed_forward_graph_fused_and_node_by_node(be, oracle, layout, L):
+    """linear1 128 -> 512, relu, linear2 512 -> 128 on the pair track (L = 103: the configured 10609 tokens): the ReLU
+    node folded into the second matmul's quantizer, and executed as a node of its own -- the same bits both ways, and
+    the oracle's."""
+    D, H = 128, 512
+    rng = np.random.default_rng(L)
+    x = rng.standard_normal((L * L, D)).astype(np.float32)
+    w1 = (rng.standard_normal((H, D)) * 0.02).astype(np.float32)
+    w2 = (rng.standard_normal((D, H)) * 0.02).astype(np.float32)
+    w1t, w1q = _q8_leaf(be, oracle, w1, layout)
+    w2t, w2q = _q8_leaf(be, oracle, w2, layout)
+    hidden = oracle.mul_mat_q8(w1q, x, wtype=0, c_trans=1, fma=1)
+    want = oracle.mul_mat_q8(w2q, oracle.relu(hidden), wtype=0, c_trans=1, fma=1)
+    xl = _leaf(be, x, dims=(D, L, L, 1))
+    results = []
+    for fuse in (True, False):
+        be.set_fuse_relu_into_q8(fuse)
+        try:
+            graph, relu, y_flat = _feed_forward_graph(be, xl, w1t, w2t, L, D, H)
+            assert be.graph_compute(graph) == B.SUCCESS, be.last_error
+            assert be.nodes_fused_away == (1 if fuse else 0)
+            got = be.download(y_flat).reshape(L * L, D)
+            if not fuse:                                        # the node ran: its own tensor holds relu(hidden)
+                assert np.array_equal(be.download(relu).reshape(L * L, H), oracle.relu(hidden))
+        finally:
+            be.set_fuse_relu_into_q8(True)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), fuse
+        results.append(got)
+    assert np.array_equal(results[0], results[1])
+
+
+def test_relu_is_not_folded_when_somebody_else_needs_it(be, oracle):
+    D, H, L = 64, 96, 9
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((L * L, D)).astype(np.float32)
+    w1 = (rng.standard_normal((H, D)) * 0.05).astype(np.float32)
+    w2 = (rng.standard_normal((D, H)) * 0.05).astype(np.float32)
+    w1t, w1q = _q8_leaf(be, oracle, w1, "Q8_0")
+    w2t, w2q = _q8_leaf(be, oracle, w2, "Q8_0")
+    hidden = oracle.mul_mat_q8(w1q, x)
+    want = oracle.mul_mat_q8(w2q, oracle.relu(hidden))
+    xl = _leaf(be, x, dims=(D, L, L, 1))
+    # marked as an output of the graph (include/ppml/Tensor.h:21): it has to be written
+    graph, relu, y_flat = _feed_forward_graph(be, xl, w1t, w2t, L, D, H)
+    relu.set_flag(B.FLAG_OUTPUT)
+    assert be.graph_compute(graph) == B.SUCCESS, be.last_error
+    assert be.nodes_fused_away == 0
+    assert np.array_equal(be.download(relu).reshape(L * L, H), oracle.relu(hidden))
+    assert np.array_equal(be.download(y_flat).reshape(L * L, D), want)
+    # a second reader of the ReLU (here a scale node)
+    graph, relu, y_flat = _feed_forward_graph(be, xl, w1t, w2t, L, D, H)
+    other = B.Tensor((H, L, L, 1), B.F32, B.OP_SCALE, [relu]).set_param(0, 2.0)
+    assert be.graph_compute(graph + [other]) == B.SUCCESS, be.last_error
+    assert be.nodes_fused_away == 0
+    assert np.array_equal(be.download(other).reshape(L * L, H), oracle.relu(hidden) * np.float32(2))
+    assert np.array_equal(be.download(y_flat).reshape(L * L, D), want)
+    # a ReLU in front of an f32 matmul stays a node (there is no quantizer to fold it into)
+    wf = _leaf(be, w2)
+    h = _leaf(be, hidden)
+    r = B.Tensor((H, L * L), B.F32, B.OP_UNARY, [h]).set_param(0, B.UNARY_OP_RELU)
+    y = B.Tensor((D, L * L), B.F32, B.OP_MUL_MAT, [r, wf])
+    assert be.graph_compute([r, y]) == B.SUCCESS, be.last_error
+    assert be.nodes_fused_away == 0
+    ref = oracle.mul_mat_f32(oracle.relu(hidden), w2)
+    np.testing.assert_allclose(be.download(y).reshape(L * L, D), ref, rtol=0, atol=1e-4 * np.abs(ref).max())
+
+
+def _logits_graph(k_leaf, q_leaf, L, H, planes, scale):
+    scores = B.Tensor((L, L, H, planes), B.F32, B.OP_OUT_PROD, [k_leaf, q_leaf])
+    scaled = B.Tensor((L, L, H, planes), B.F32, B.OP_SCALE, [scores]).set_param(0, float(scale))
+    return scores, scaled
+
+
+def test_attention_logits_graph_fused_and_node_by_node(be, oracle):
+    """out_prod(K, Q) -> scale(1/sqrt(D)) as src/modules/Attention.cpp:264-270 builds it, at the pair-track shape
+    (103 x 4 heads planes of 103 x 103 over D = 32): one scaled contraction, and two nodes -- the same bits."""
+    L, D, H, Bt = 103, 32, 4, 103
+    rng = np.random.default_rng(12)
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(D)))
+    for exact in (True, False):
+        if exact:       # small integers: every product and sum is exact, so one rounding (the scale) is all there is
+            k = rng.integers(-4, 5, size=(Bt, H, D, L)).astype(np.float32)
+            q = rng.integers(-4, 5, size=(Bt, H, D, L)).astype(np.float32)
+        else:
+            k = rng.standard_normal((Bt, H, D, L)).astype(np.float32)
+            q = rng.standard_normal((Bt, H, D, L)).astype(np.float32)
+        want = oracle.scale(oracle.out_prod(k, q), scale)
+        kl, ql = _leaf(be, k), _leaf(be, q)
+        outs = []
+        for fuse in (True, False):
+            be.set_fuse_scale_into_out_prod(fuse)
+            try:
+                scores, scaled = _logits_graph(kl, ql, L, H, Bt, scale)
+                assert be.graph_compute([scores, scaled]) == B.SUCCESS, be.last_error
+                assert be.nodes_fused_away == (1 if fuse else 0)
+                outs.append(be.download(scaled).reshape(want.shape))
+            finally:
+                be.set_fuse_scale_into_out_prod(True)
+        assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+        if exact:
+            assert np.array_equal(outs[0].view(np.uint32), want.view(np.uint32))
+        else:           # f32 GEMM bar: 1e-4 of the magnitude sum (k ascending on the CPU, matrix pipe here)
+            bound = 1e-4 * scale * float(np.abs(k).max() * np.abs(q).max() * D)
+            assert np.abs(outs[0] - want).max() <= bound
+    # scores that something else reads, or that are an output, stay a node of their own
+    scores, scaled = _logits_graph(kl, ql, L, H, Bt, scale)
+    scores.set_flag(B.FLAG_OUTPUT)
+    assert be.graph_compute([scores, scaled]) == B.SUCCESS and be.nodes_fused_away == 0
+    assert np.array_equal(be.download(scaled).view(np.uint32), outs[0].reshape(-1).view(np.uint32))
+
+
+def _attention_chain_graph(be, kl, ql, vl, bias_leaf, L, D, H, Bt, scale):
+    """SelfAttention::forward_graph, default path (src/modules/Attention.cpp:264-281)."""
+    scores = B.Tensor((L, L, H, Bt), B.F32, B.OP_OUT_PROD, [kl, ql])
+    scaled = B.Tensor((L, L, H, Bt), B.F32, B.OP_SCALE, [scores]).set_param(0, float(scale))
+    nodes = [scores, scaled]
+    x = scaled
+    if bias_leaf is not None:
+        x = B.Tensor((L, L, H, Bt), B.F32, B.OP_ADD, [scaled, bias_leaf])
+        nodes.append(x)
+    attn = B.Tensor((L, L, H, Bt), B.F32, B.OP_SOFT_MAX, [x])
+    attn_t = B.Tensor((L, L, H, Bt), B.F32, B.OP_PERMUTE, [attn])
+    v_t = B.Tensor((D, L, H, Bt), B.F32, B.OP_PERMUTE, [vl])
+    for p in (attn_t, v_t):
+        for i, a in enumerate((1, 0, 2, 3)):
+            p.set_param(i, a)
+    out = B.Tensor((L, D, H, Bt), B.F32, B.OP_OUT_PROD, [attn_t, v_t])
+    return nodes + [attn, attn_t, v_t, out], out
+
+
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_default_attention_chain_stays_on_the_device(be, oracle, with_bias):
+    """The chain the reference builds when PPML_FLASH_ATTN is off, node by node on this backend, against the oracle's
+    restatement of the same nodes; then the same graph with the chain recognised and run as one fused launch."""
+    L, D, H, Bt = 51, 32, 4, 6
+    rng = np.random.default_rng(31 + with_bias)
+    k, q, v = (rng.standard_normal((Bt, H, D, L)).astype(np.float32) for _ in range(3))       # graph layout [L, D, H, B]
+    bias = rng.standard_normal((Bt, H, L, L)).astype(np.float32) if with_bias else None
+    scale = float(np.float32(1.0) / np.sqrt(np.float32(D)))
+    x = oracle.scale(oracle.out_prod(k, q), scale)
+    if with_bias:
+        x = oracle.bcast_elemwise(x, bias, "add")
+    want = oracle.out_prod(oracle.permute(oracle.softmax(x), (1, 0, 2, 3)), oracle.permute(v, (1, 0, 2, 3)))
+    kl, ql, vl = _leaf(be, k), _leaf(be, q), _leaf(be, v)
+    bl = _leaf(be, bias) if with_bias else None
+    graph, out = _attention_chain_graph(be, kl, ql, vl, bl, L, D, H, Bt, scale)
+    assert all(be.supports_op(n) for n in graph)
+    assert be.graph_compute(graph) == B.SUCCESS, be.last_error
+    assert be.nodes_fused_away == 1                                   # the logits and their scale
+    got = be.download(out).reshape(want.shape)
+    np.testing.assert_allclose(got, want, rtol=0, atol=1e-4 * np.abs(want).max())
+    # opt in: the whole chain as one launch
+    be.set_fuse_attention_chain(True)
+    try:
+        graph, out = _attention_chain_graph(be, kl, ql, vl, bl, L, D, H, Bt, scale)
+        assert be.graph_compute(graph) == B.SUCCESS, be.last_error
+        assert be.nodes_fused_away == (6 if with_bias else 5)
+        fused = be.download(out).reshape(want.shape)
+    finally:
+        be.set_fuse_attention_chain(False)
+    np.testing.assert_allclose(fused, want, rtol=0, atol=1e-4 * np.abs(want).max())
+    # and against the reference's fused routine itself (layouts [B][h][L][d])
+    o, _ = oracle.flash_attn_forward(q.transpose(0, 1, 3, 2).copy(), k.transpose(0, 1, 3, 2).copy(), v.transpose(0, 1, 3, 2).copy(),
+                                     bias, scale=scale)
+    np.testing.assert_allclose(fused.transpose(0, 1, 3, 2), o, rtol=0, atol=2e-5 * np.abs(o).max())
+
+
+def test_attention_chain_is_left_alone_when_an_intermediate_is_read_elsewhere(be, oracle):
+    L, D, H, Bt = 20, 16, 2, 3
+    rng = np.random.default_rng(5)
+    k, q, v = (rng.standard_normal((Bt, H, D, L)).astype(np.float32) for _ in range(3))
+    kl, ql, vl = _leaf(be, k), _leaf(be, q), _leaf(be, v)
+    be.set_fuse_attention_chain(True)
+    try:
+        graph, out = _attention_chain_graph(be, kl, ql, vl, None, L, D, H, Bt, 0.25)
+        attn = graph[2]
+        attn.set_flag(B.FLAG_OUTPUT)                                  # the probabilities are wanted (e.g. for a backward pass)
+        assert be.graph_compute(graph) == B.SUCCESS, be.last_error
+        assert be.nodes_fused_away == 1                               # only the scale went into the logits
+        probs = oracle.softmax(oracle.scale(oracle.out_prod(k, q), 0.25))
+        np.testing.assert_allclose(be.download(attn).reshape(probs.shape), probs, rtol=1e-4, atol=1e-7)
+    finally:
+        be.set_fuse_attention_chain(False)

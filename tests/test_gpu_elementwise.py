@@ -1,0 +1,161 @@
+"""GPU parity of the element-wise launchers (scale_hip, unary_hip, bcast_elemwise_hip, softmax_hip) against the CPU
+oracle.  scale, relu and the four binary operations are one IEEE operation per element: equality of bits.
+softmax sums across a wavefront and uses the device's expf: 1e-5 relative, the bar of the path's f32 outputs."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+SOFTMAX_RTOL = 1e-5      # against the oracle's sequential sums and glibc expf, rows up to some hundred values
+
+
+def softmax_rtol(D):
+    """The reference adds a row's D exponentials one after the other in binary32: that sum alone may be off by
+    D * 2^-24 of its value, and the wavefront's tree sum here by far less, so on long rows the two drift apart by
+    the reference's own rounding.  1e-5 up to the attention shapes' row lengths, D * 2^-24 beyond."""
+    return max(SOFTMAX_RTOL, D * 2.0 ** -24)
+
+
+SOFTMAX_ATOL = 1e-37     # outputs down in the subnormal range differ in their last bits only
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "GPU tests need a device"
+    from proteinpredictmachinelearning_amd import ops as _ops
+
+    return _ops
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _same_bits(got, want):
+    nan = np.isnan(want)
+    return np.array_equal(np.isnan(got), nan) and np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 255, 1024, 1027, 103 * 103 * 4 + 1])
+def test_scale_and_relu_bits(ops, oracle, n):
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 50).astype(np.float32)
+    x[: min(n, 6)] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-42][: min(n, 6)]
+    s = float(np.float32(1.0 / np.sqrt(np.float32(32.0))))
+    got = ops.scale(_dev(x), s).cpu().numpy()
+    assert _same_bits(got, oracle.scale(x, s))
+    got = ops.relu(_dev(x)).cpu().numpy()
+    want = oracle.relu(x)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))      # NaN and -0 -> +0: no NaN left to exclude
+
+
+def test_scale_and_relu_on_pointers_that_are_only_4_byte_aligned(ops, oracle):
+    rng = np.random.default_rng(1)
+    base = rng.standard_normal(1000).astype(np.float32)
+    d = _dev(base)
+    for off in (1, 2, 3):
+        got = ops.scale(d[off:], 0.3)
+        assert got.data_ptr() % 16 == 0 and d[off:].data_ptr() % 16 != 0
+        assert _same_bits(got.cpu().numpy(), oracle.scale(base[off:], 0.3))
+        assert np.array_equal(ops.relu(d[off:]).cpu().numpy(), oracle.relu(base[off:]))
+
+
+def test_unary_other_than_relu_is_refused(ops):
+    import ctypes as C
+    x = _dev(np.ones(8, np.float32))
+    lib = ops._lib()
+    for uop in (0, 5, 7, 13, -1):
+        assert lib.unary_hip(C.c_void_p(x.data_ptr()), C.c_void_p(x.data_ptr()), 8, uop, None) == 1
+    assert "UNARY_OP_RELU" in ops.cabi.last_error()
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+def test_bcast_elemwise_bits(ops, oracle, op):
+    rng = np.random.default_rng(7)
+    a = rng.standard_normal((3, 5, 8, 12)).astype(np.float32)
+    for shape in [(3, 5, 8, 12), (8, 12), (12,), (1,), (5, 8, 12), (4,)]:
+        b = (rng.standard_normal(shape) + 3).astype(np.float32)
+        got = ops.bcast_elemwise(_dev(a), _dev(b), op).cpu().numpy()
+        assert _same_bits(got, oracle.bcast_elemwise(a, b, op)), shape
+    # sizes and offsets that take the element-by-element path
+    a = rng.standard_normal((7, 103)).astype(np.float32)
+    for shape in [(7, 103), (103,), (1,)]:
+        b = (rng.standard_normal(shape) + 3).astype(np.float32)
+        assert _same_bits(ops.bcast_elemwise(_dev(a), _dev(b), op).cpu().numpy(), oracle.bcast_elemwise(a, b, op)), shape
+    big = _dev(rng.standard_normal(4 * 64 + 1).astype(np.float32))
+    aa, bb = big[1:], _dev(rng.standard_normal(4 * 64).astype(np.float32) + 3)
+    assert _same_bits(ops.bcast_elemwise(aa, bb, op).cpu().numpy(), oracle.bcast_elemwise(aa.cpu().numpy(), bb.cpu().numpy(), op))
+    # special values
+    sa = np.float32([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, 1e-42, 3e38])
+    sb = np.float32([0.0, 5.0, np.inf, 2.0, 1.0, 0.0, 1e-3, 3e38])
+    assert _same_bits(ops.bcast_elemwise(_dev(sa), _dev(sb), op).cpu().numpy(), oracle.bcast_elemwise(sa, sb, op))
+
+
+def test_bcast_elemwise_refuses_operands_that_do_not_repeat(ops):
+    import ctypes as C
+    a, b = _dev(np.ones(12, np.float32)), _dev(np.ones(5, np.float32))
+    with pytest.raises(ValueError):
+        ops.bcast_elemwise(a, b)
+    lib = ops._lib()
+    p = lambda t: C.c_void_p(t.data_ptr())  # noqa: E731
+    assert lib.bcast_elemwise_hip(p(a), p(b), p(a), 12, 12, 5, 0, None) == 1
+    assert lib.bcast_elemwise_hip(p(a), p(b), p(a), 12, 12, 4, 4, None) == 1       # no such operation
+    assert lib.bcast_elemwise_hip(p(a), p(b), p(a), 12, 24, 4, 0, None) == 1       # an operand longer than the result
+
+
+def test_attention_bias_add_at_the_pair_shape_in_full(ops, oracle):
+    # scaled [Lk, Lq, H, B*L] + bias of the same shape (src/modules/Attention.cpp:271-273)
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((412, 103, 103)).astype(np.float32)
+    b = rng.standard_normal((412, 103, 103)).astype(np.float32)
+    got = ops.bcast_elemwise(_dev(x), _dev(b), "add").cpu().numpy()
+    assert np.array_equal(got, x + b)
+
+
+@pytest.mark.parametrize("D", [1, 2, 3, 31, 64, 65, 103, 128, 256, 257, 512, 513, 1000, 2048, 2049, 5000])
+def test_softmax_rows(ops, oracle, D):
+    rng = np.random.default_rng(D)
+    rows = 37 if D < 1000 else 9
+    x = (4 * rng.standard_normal((rows, D))).astype(np.float32)
+    got = ops.softmax(_dev(x)).cpu().numpy()
+    np.testing.assert_allclose(got, oracle.softmax(x), rtol=softmax_rtol(D), atol=SOFTMAX_ATOL)
+    # against float64 the tree sum is the closer one
+    e = np.exp(x.astype(np.float64) - x.max(-1, keepdims=True))
+    np.testing.assert_allclose(got, e / (e.sum(-1, keepdims=True) + 1e-9), rtol=5e-6, atol=SOFTMAX_ATOL)
+    # a leading dimension changes nothing: rows are dims[0]
+    got3 = ops.softmax(_dev(x.reshape(rows, 1, D))).cpu().numpy().reshape(rows, D)
+    assert np.array_equal(got3, got)
+
+
+def test_softmax_closed_forms_and_special_rows(ops, oracle):
+    for D in (1, 7, 103, 256, 3000):
+        got = ops.softmax(_dev(np.full((5, D), 3.25, np.float32))).cpu().numpy()
+        np.testing.assert_allclose(got, np.float32(1.0) / (np.float32(D) + np.float32(1e-9)), rtol=3e-7)
+    z = np.zeros((5, 70), np.float32)
+    z[0, 0] = np.nan                  # the maximum starts there: the whole row is NaN
+    z[1, 33] = np.nan                 # reaches every entry through the sum
+    z[2, :] = -np.inf                 # inf - inf
+    z[3, 1:40] = -np.inf              # masked keys beside live ones: plain zeros
+    z[4, 5] = 200.0                   # a dominant entry
+    got = ops.softmax(_dev(z)).cpu().numpy()
+    want = oracle.softmax(z)
+    assert np.isnan(got[:3]).all() and np.isnan(want[:3]).all()
+    assert (got[3, 1:40] == 0).all()
+    np.testing.assert_allclose(got[3:], want[3:], rtol=SOFTMAX_RTOL)
+    assert got[4, 5] == 1.0 and got[4].sum() == 1.0
+    # rows on 4-byte boundaries only (odd row length behind an odd offset)
+    rng = np.random.default_rng(3)
+    base = rng.standard_normal(1 + 11 * 103).astype(np.float32)
+    got = ops.softmax(_dev(base)[1:].reshape(11, 103)).cpu().numpy()
+    np.testing.assert_allclose(got, oracle.softmax(base[1:].reshape(11, 103)), rtol=SOFTMAX_RTOL)
+
+
+def test_softmax_at_the_configured_attention_shapes_in_full(ops, oracle):
+    rng = np.random.default_rng(11)
+    for planes, L in [(412, 103), (824, 256)]:
+        x = (2 * rng.standard_normal((planes, L, L))).astype(np.float32)
+        got = ops.softmax(_dev(x)).cpu().numpy()
+        np.testing.assert_allclose(got, oracle.softmax(x), rtol=SOFTMAX_RTOL, atol=SOFTMAX_ATOL)
+        np.testing.assert_allclose(got.sum(-1), 1.0, rtol=2e-6)

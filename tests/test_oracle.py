@@ -758,3 +758,113 @@ def test_repeat_back_adds_its_terms_one_at_a_time(oracle):
     # 1 + 1 = 2, + 2^24 = 2^24 + 2, + 1 -> tie, rounds to even: 2^24 + 4?  (2^24 + 3 lies between 2^24+2 and 2^24+4)
     got = oracle.repeat_back(m2, (1, 1))[0, 0]
     assert got == np.float32(np.float32(np.float32(1.0 + 1.0) + np.float32(2.0 ** 24)) + np.float32(1.0))
+
+
+# ----------------------------------------------------------------------------- element-wise nodes between the contractions
+def test_scale_and_relu_are_one_ieee_operation_per_element(oracle):
+    rng = np.random.default_rng(40)
+    x = rng.standard_normal(1001).astype(np.float32) * np.float32(1e3)
+    x[:6] = [0.0, -0.0, np.inf, -np.inf, np.nan, np.float32(1e-42)]
+    s = np.float32(1.0 / np.sqrt(np.float32(32.0)))
+    got = oracle.scale(x, s)
+    want = x * s                                        # numpy's float32 multiply: one rounding
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.isnan(got[4])
+    assert oracle.scale(np.float32([3.0]), 0.1)[0] == np.float32(3.0) * np.float32(0.1)     # the factor is a binary32
+    r = oracle.relu(x)
+    assert np.array_equal(r[6:], np.maximum(x[6:], 0))
+    # (s > 0) ? s : 0 -- NaN and -0 fail the comparison and give +0; np.maximum would keep both
+    assert r[0] == 0 and not np.signbit(r[0]) and r[1] == 0 and not np.signbit(r[1])
+    assert r[2] == np.inf and r[3] == 0 and r[4] == 0 and not np.signbit(r[4]) and r[5] == np.float32(1e-42)
+
+
+def test_bcast_elemwise_is_the_flat_modulo_broadcast(oracle):
+    rng = np.random.default_rng(41)
+    a = rng.standard_normal((3, 5, 4, 6)).astype(np.float32)
+    for shape in [(3, 5, 4, 6), (4, 6), (6,), (1,), (5, 4, 6)]:
+        b = (rng.standard_normal(shape) + 3).astype(np.float32)
+        tiled = np.resize(b.ravel(), a.size).reshape(a.shape)                    # b[i % bn]
+        for op, f in [("add", np.add), ("sub", np.subtract), ("mul", np.multiply), ("div", np.divide)]:
+            got = oracle.bcast_elemwise(a, b, op)
+            assert got.shape == a.shape
+            assert np.array_equal(got.view(np.uint32), f(a, tiled).view(np.uint32)), (shape, op)
+        # an operand that covers the innermost dimensions: numpy's own dimension-wise broadcast says the same
+        assert np.array_equal(oracle.bcast_elemwise(a, b, "add"), a + b)
+    # ... and one that does not (a middle dimension): the flat rule reads other elements than numpy's broadcast
+    mid = rng.standard_normal((5, 1, 1)).astype(np.float32)
+    assert not np.array_equal(oracle.bcast_elemwise(a, mid, "add"), a + mid)
+    # the smaller operand may come first (dst then has the larger one's shape)
+    b = rng.standard_normal(6).astype(np.float32)
+    assert np.array_equal(oracle.bcast_elemwise(b, a, "sub"), b - a)
+
+
+def test_softmax_closed_forms(oracle):
+    # rows of equal values: expf(0) = 1 exactly, sum = D exactly, so every entry is fl(1 / fl(D + 1e-9))
+    for D in (1, 2, 3, 7, 64, 103, 256, 1000):
+        got = oracle.softmax(np.full((2, D), 3.25, np.float32))
+        want = np.float32(1.0) / (np.float32(D) + np.float32(1e-9))
+        assert (got == want).all(), D
+    # one dominant entry
+    x = np.full((1, 50), -200.0, np.float32)
+    x[0, 17] = 5.0
+    got = oracle.softmax(x)
+    assert got[0, 17] == 1.0 and got.sum() == 1.0
+    # against float64 on random rows
+    rng = np.random.default_rng(42)
+    x = (4 * rng.standard_normal((37, 103))).astype(np.float32)
+    e = np.exp(x.astype(np.float64) - x.max(-1, keepdims=True))
+    want = e / (e.sum(-1, keepdims=True) + 1e-9)
+    np.testing.assert_allclose(oracle.softmax(x), want, rtol=2e-6, atol=1e-12)
+    # over the LAST axis only: rows are independent
+    y = oracle.softmax(x.reshape(37, 1, 103))
+    assert np.array_equal(y.reshape(37, 103), oracle.softmax(x))
+    # exact shifts leave the bits alone (the maximum is subtracted first)
+    xi = rng.integers(-8, 9, size=(5, 40)).astype(np.float32)
+    assert np.array_equal(oracle.softmax(xi), oracle.softmax(xi + 16))
+    # the maximum starts from the first element and moves on `>`: a NaN there poisons the row, elsewhere too
+    # (through the sum); a row of -inf is NaN (inf - inf); -inf entries beside finite ones are plain zeros
+    z = np.zeros((4, 5), np.float32)
+    z[0, 0] = np.nan
+    z[1, 3] = np.nan
+    z[2, :] = -np.inf
+    z[3, 1:3] = -np.inf
+    s = oracle.softmax(z)
+    assert np.isnan(s[0]).all() and np.isnan(s[1]).all() and np.isnan(s[2]).all()
+    assert (s[3, 1:3] == 0).all() and np.allclose(s[3, [0, 3, 4]], 1 / 3)
+
+
+def test_attention_chain_of_nodes_equals_the_fused_reference_on_its_golden_vectors(oracle):
+    """out_prod(K,Q) -> scale -> add(bias) -> softmax -> permute, permute(V) -> out_prod, node by node with the oracle's
+    restatements (src/modules/Attention.cpp:264-281), against the outputs of the reference's own fused
+    flash_attn_forward_cpu held in tests/golden/flash_attn_forward.json (non-causal cases; the fused routine
+    accumulates online, so agreement is to rounding)."""
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "flash_attn_forward.json")
+    with open(path) as f:
+        cases = json.load(f)["cases"]
+    n = 0
+    for c in cases:
+        if c["causal"]:
+            continue
+        shape = (c["B"], c["h"], c["L"], c["d"])
+        f32 = lambda bits, shp: np.array(bits, dtype=np.uint32).view(np.float32).reshape(shp)  # noqa: E731
+        q, k, v = f32(c["q"], shape), f32(c["k"], shape), f32(c["v"], shape)
+        bias = f32(c["bias"], (c["B"], c["h"], c["L"], c["L"])) if c["bias"] is not None else None
+        want = f32(c["o"], shape)
+        # the graph's tensors are [L, D, h, B] (dims[0] first) = numpy (B, h, D, L)
+        kg, qg, vg = (np.ascontiguousarray(t.transpose(0, 1, 3, 2)) for t in (k, q, v))
+        scores = oracle.out_prod(kg, qg)                                   # [Lk, Lq, h, B] = numpy (B, h, Lq, Lk)
+        scale = c["scale"] if c["scale"] > 0 else 1.0 / np.sqrt(np.float32(c["d"]))
+        x = oracle.scale(scores, scale)
+        if bias is not None:
+            x = oracle.bcast_elemwise(x, bias, "add")
+        attn = oracle.softmax(x)
+        attn_t = oracle.permute(attn, (1, 0, 2, 3))                        # [Lq, Lk, h, B]
+        v_t = oracle.permute(vg, (1, 0, 2, 3))                             # [D, Lk, h, B]
+        out = oracle.out_prod(attn_t, v_t)                                 # [Lq, D, h, B] = numpy (B, h, D, Lq)
+        got = out.transpose(0, 1, 3, 2)
+        rows = np.isfinite(f32(c["lse"], shape[:3]))                       # fully masked rows: O = 0 there, NaN here
+        np.testing.assert_allclose(got[rows], want[rows], rtol=2e-5, atol=2e-6)
+        n += 1
+    assert n >= 2
