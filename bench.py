@@ -63,6 +63,9 @@ def main() -> int:
                     help="untimed steps; the shader clock needs 1-2 ms of load to reach its steady value")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configured shapes")
+    ap.add_argument("--configured-shapes-only", action="store_true",
+                    help="of the other shapes, measure only the five HBM-bound configured ones (the short run that the "
+                         "rocprofv3 --pmc traffic passes use)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 1 GiB device copy, the kernel of known size against which the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run are scaled")
@@ -280,7 +283,11 @@ def main() -> int:
             if cpu_pair is not None:
                 extra[name]["cpu_baseline"] = q8_cpu(w_dev, x_dev, relu, no, f"the whole {r}x{k}->{n} workload")
 
+        rest = {"skip": False}
+
         def f32_case(make, nbytes, flops, name, pipe="fp32", rw=None, cpu=None):
+            if rest["skip"]:
+                return
             # pipe: "fp32" = fp32 MFMA; "bf16x3" = binary32 operands split three ways, six bf16 MFMA
             # products per binary32 product (TFLOPS counts binary32 products, the fraction bf16 ones)
             fn_, ns = make()
@@ -323,11 +330,23 @@ def main() -> int:
                 keep.append((ks, qs, outs))
                 return fn, ns
             return make
+        def logits_cpu(planes, L, D):
+            # the reference's two nodes on the CPU: kernel_out_prod then kernel_scale (CPUKernels.cpp:787-887, 1737-1754)
+            def cpu():
+                ks, qs, _ = keep[-1]
+                kh, qh = ks[0].cpu().numpy(), qs[0].cpu().numpy()
+                s = float(np.float32(1.0) / np.sqrt(np.float32(D)))
+                return cpu_pair(lambda nt: oracle.scale(oracle.out_prod(kh, qh, nthreads=nt), s, nthreads=nt),
+                                2.0 * planes * L * L * D, "TFLOPS", f"the whole {planes} x {L} x {L} x {D} workload (out_prod + scale)")
+            return cpu
         f32_case(logits(412, 103, 32), (2 * 412 * 32 * 103 + 412 * 103 * 103) * 4, 2.0 * 412 * 103 * 103 * 32,
-                 "attn_logits_pair_412x103x103x32", pipe="bf16x3", rw=(2 * 412 * 32 * 103 * 4, 412 * 103 * 103 * 4))
+                 "attn_logits_pair_412x103x103x32", pipe="bf16x3", rw=(2 * 412 * 32 * 103 * 4, 412 * 103 * 103 * 4),
+                 cpu=logits_cpu(412, 103, 32))
         f32_case(logits(824, 256, 32), (2 * 824 * 32 * 256 + 824 * 256 * 256) * 4, 2.0 * 824 * 256 * 256 * 32,
-                 "attn_logits_msa_824x256x256x32", pipe="bf16x3", rw=(2 * 824 * 32 * 256 * 4, 824 * 256 * 256 * 4))
+                 "attn_logits_msa_824x256x256x32", pipe="bf16x3", rw=(2 * 824 * 32 * 256 * 4, 824 * 256 * 256 * 4),
+                 cpu=logits_cpu(824, 256, 32))
 
+        rest["skip"] = args.configured_shapes_only         # everything below is beyond the configured shapes
         def attention(planes, L, D, with_bias, layout=0):
             def make():
                 import ctypes as C
@@ -422,12 +441,27 @@ def main() -> int:
             return fn, ns
         f32_case(trimul, 3 * 128 * 103 * 103 * 4, 2.0 * 128 * 103 ** 3, "tri_mul_outgoing_128x103x103x103")
 
+        opm_operands = []
+
         def opm():
             a = torch.randn(256, 12288, device=dev, generator=gen) * 0.1
             b = torch.randn(256, 12288, device=dev, generator=gen) * 0.1
+            opm_operands[:] = [a, b]
             return (lambda i: ops.mul_mat_tn(a, b, 1.0 / 256)), 1
+
+        def opm_cpu():
+            # the reference's CPU mul_mat (CPUKernels.cpp:763-771) on the transposed operands, on a sample of the output
+            # rows: 768 of 12288 (one sixteenth of the 77.3 GFLOP), every column, followed by the 1/N scale
+            rows_sample = 768
+            at = np.ascontiguousarray(opm_operands[0][:, :rows_sample].cpu().numpy().T)
+            bt = np.ascontiguousarray(opm_operands[1].cpu().numpy().T)
+            inv = float(np.float32(1.0) / np.float32(256))
+            return cpu_pair(lambda nt: oracle.scale(oracle.mul_mat_f32(at, bt, nthreads=nt), inv, nthreads=nt),
+                            2.0 * rows_sample * 12288 * 256, "TFLOPS",
+                            f"{rows_sample} of the 12288 output rows x all 12288 columns x K = 256 (1/16 of the workload)")
         steps, warm = 50, 10
-        f32_case(opm, (2 * 256 * 12288 + 12288 * 12288) * 4, 2.0 * 12288 * 12288 * 256, "opm_dense_12288x256x12288", pipe="bf16x3")
+        f32_case(opm, (2 * 256 * 12288 + 12288 * 12288) * 4, 2.0 * 12288 * 12288 * 256, "opm_dense_12288x256x12288", pipe="bf16x3",
+                 cpu=opm_cpu)
 
         def dense():
             a = torch.randn(4096, 4096, device=dev, generator=gen)
