@@ -81,8 +81,14 @@ extern "C" int repeat_back_hip(const float* src, float* dst,
                                int64_t r0, int64_t r1, int64_t r2, int64_t r3, ppml_hip_stream_t stream) {
     const bool pos = s0 > 0 && s1 > 0 && s2 > 0 && s3 > 0 && d0 > 0 && d1 > 0 && d2 > 0 && d3 > 0 &&
                      r0 > 0 && r1 > 0 && r2 > 0 && r3 > 0;
-    // every term must lie inside the source: (d - 1) + (r - 1) * d < s per dimension
-    if (!src || !dst || !pos || r0 * d0 > s0 || r1 * d1 > s1 || r2 * d2 > s2 || r3 * d3 > s3) {
+    // every term must lie inside the source: (d - 1) + (r - 1) * d < s per dimension, i.e. r <= s / d (a quotient,
+    // so that sizes near 2^63 cannot wrap a product past the test)
+    const bool inside = pos && r0 <= s0 / d0 && r1 <= s1 / d1 && r2 <= s2 / d2 && r3 <= s3 / d3;
+    int64_t total = 0, reps = 0, t01 = 0, t23 = 0, q01 = 0, q23 = 0;
+    const bool sized = inside && !__builtin_mul_overflow(d0, d1, &t01) && !__builtin_mul_overflow(d2, d3, &t23) &&
+                       !__builtin_mul_overflow(t01, t23, &total) && !__builtin_mul_overflow(r0, r1, &q01) &&
+                       !__builtin_mul_overflow(r2, r3, &q23) && !__builtin_mul_overflow(q01, q23, &reps);
+    if (!src || !dst || !sized) {
         set_error("repeat_back_hip: bad arguments (src [%lld,%lld,%lld,%lld], dst [%lld,%lld,%lld,%lld], copies [%lld,%lld,%lld,%lld])",
                   (long long)s0, (long long)s1, (long long)s2, (long long)s3, (long long)d0, (long long)d1, (long long)d2,
                   (long long)d3, (long long)r0, (long long)r1, (long long)r2, (long long)r3);
@@ -94,9 +100,8 @@ extern "C" int repeat_back_hip(const float* src, float* dst,
     jb.s0 = s0; jb.s1 = s1; jb.s2 = s2;
     jb.d0 = d0; jb.d1 = d1; jb.d2 = d2; jb.d3 = d3;
     jb.r1 = r1; jb.r2 = r2; jb.r3 = r3;
-    jb.total = d0 * d1 * d2 * d3;
-    jb.reps = r0 * r1 * r2 * r3;
-    StatsScope stat("hip/repeat_back", jb.total, jb.reps, 1, s);
+    jb.total = total;
+    jb.reps = reps;
     const int64_t blocks = (jb.total + 255) / 256;
     if (blocks > 0x7fffffffLL) { set_error("repeat_back_hip: destination too large"); return RC_BAD_ARGS; }
     // Few destination elements and many copies (a bias gradient: 768 sums of 26368 terms) would leave most of

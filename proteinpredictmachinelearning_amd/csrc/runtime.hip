@@ -8,6 +8,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <optional>
 #include <string>
 #include <tuple>
 #include <vector>
@@ -51,8 +52,7 @@ struct Stats {
     std::map<StatKey, StatVal> table;
     std::vector<Pending> pending;
     std::vector<hipEvent_t> spare;                     // events to use again
-    std::chrono::steady_clock::time_point t_first{};
-    bool started = false;
+    std::optional<std::chrono::steady_clock::time_point> first_call;   // the clock the report's wall time runs on
 };
 Stats& stats() {
     static Stats* s = new Stats();                     // never destroyed: the exit handler still reads it
@@ -76,31 +76,48 @@ void fold_pending_locked(Stats& s, bool wait) {
     s.pending.resize(keep);
 }
 
-void dump_locked(Stats& s) {
-    const double wall_ms = s.started
-        ? std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - s.t_first).count() : 0.0;
-    int64_t calls = 0;
-    double ms = 0.0;
-    std::map<std::string, StatVal> by_path;
-    std::vector<std::pair<StatKey, StatVal>> rows(s.table.begin(), s.table.end());
-    for (const auto& kv : rows) {
-        calls += kv.second.calls; ms += kv.second.ms;
-        by_path[kv.first.path].calls += kv.second.calls;
-        by_path[kv.first.path].ms += kv.second.ms;
+// The report in two steps: the table folded three ways (whole, per kernel family, per shape by time), then printed.
+// Only the look of the lines is shared with the reference's report (include/ppml/MulMatStats.h:86-145): tools that
+// grep "[MULMAT-STAT]" keep working.
+struct Report {
+    struct Line { std::string path; int64_t M = 0, K = 0, N = 0, calls = 0; double ms = 0.0; };
+    Line whole;
+    std::vector<Line> families;                        // one per path, by name
+    std::vector<Line> shapes;                          // one per (path, M, K, N), most device time first
+    double wall_ms = 0.0;
+};
+
+Report summarise(const Stats& s) {
+    Report r;
+    if (s.first_call) r.wall_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - *s.first_call).count();
+    for (const auto& [key, val] : s.table) {           // the map is ordered by path first
+        if (r.families.empty() || r.families.back().path != key.path) r.families.push_back(Report::Line{key.path});
+        for (Report::Line* into : {&r.whole, &r.families.back()}) { into->calls += val.calls; into->ms += val.ms; }
+        r.shapes.push_back(Report::Line{key.path, key.M, key.K, key.N, val.calls, val.ms});
     }
-    std::fprintf(stderr, "\n[MULMAT-STAT] ===== MUL_MAT shapes and times (PPML_MULMAT_STATS=1) =====\n");
-    std::fprintf(stderr, "[MULMAT-STAT] total calls=%lld device time=%.3f ms | wall since the first call=%.0f ms (%.1f%%)\n",
-                 (long long)calls, ms, wall_ms, wall_ms > 0.0 ? 100.0 * ms / wall_ms : 0.0);
-    for (const auto& kv : by_path)
-        std::fprintf(stderr, "[MULMAT-STAT]   %-24s calls=%-7lld time=%10.3f ms\n", kv.first.c_str(), (long long)kv.second.calls, kv.second.ms);
-    std::sort(rows.begin(), rows.end(), [](const auto& a, const auto& b) { return a.second.ms > b.second.ms; });
-    std::fprintf(stderr, "[MULMAT-STAT] top shapes by accumulated time (M = output rows, K = contracted, N = output columns):\n");
-    for (size_t i = 0; i < rows.size() && i < 12; ++i)
-        std::fprintf(stderr, "[MULMAT-STAT]   #%-2zu %-24s M=%-8lld K=%-8lld N=%-8lld calls=%-7lld time=%10.3f ms\n", i + 1,
-                     rows[i].first.path.c_str(), (long long)rows[i].first.M, (long long)rows[i].first.K, (long long)rows[i].first.N,
-                     (long long)rows[i].second.calls, rows[i].second.ms);
-    std::fprintf(stderr, "[MULMAT-STAT] ===== end =====\n");
+    std::stable_sort(r.shapes.begin(), r.shapes.end(), [](const Report::Line& a, const Report::Line& b) { return a.ms > b.ms; });
+    return r;
 }
+
+void print_report(const Report& r, std::FILE* to) {
+    constexpr size_t TOP = 12;
+    const double share = r.wall_ms > 0.0 ? 100.0 * r.whole.ms / r.wall_ms : 0.0;
+    std::fprintf(to, "\n[MULMAT-STAT] ===== MUL_MAT shapes and times (PPML_MULMAT_STATS=1) =====\n");
+    std::fprintf(to, "[MULMAT-STAT] total calls=%lld device time=%.3f ms | wall since the first call=%.0f ms (%.1f%%)\n",
+                 (long long)r.whole.calls, r.whole.ms, r.wall_ms, share);
+    for (const Report::Line& f : r.families)
+        std::fprintf(to, "[MULMAT-STAT]   %-24s calls=%-7lld time=%10.3f ms\n", f.path.c_str(), (long long)f.calls, f.ms);
+    std::fprintf(to, "[MULMAT-STAT] top shapes by accumulated time (M = output rows, K = contracted, N = output columns):\n");
+    size_t rank = 0;
+    for (const Report::Line& sh : r.shapes) {
+        if (++rank > TOP) break;
+        std::fprintf(to, "[MULMAT-STAT]   #%-2zu %-24s M=%-8lld K=%-8lld N=%-8lld calls=%-7lld time=%10.3f ms\n", rank, sh.path.c_str(),
+                     (long long)sh.M, (long long)sh.K, (long long)sh.N, (long long)sh.calls, sh.ms);
+    }
+    std::fprintf(to, "[MULMAT-STAT] ===== end =====\n");
+}
+
+void dump_locked(Stats& s) { print_report(summarise(s), stderr); }
 
 void stats_at_exit() {
     Stats& s = stats();
@@ -150,7 +167,7 @@ StatsScope::~StatsScope() {
     std::lock_guard<std::mutex> lock(s.mu);
     static const bool registered = [] { std::atexit(stats_at_exit); return true; }();
     (void)registered;
-    if (!s.started) { s.t_first = std::chrono::steady_clock::now(); s.started = true; }
+    if (!s.first_call) s.first_call = std::chrono::steady_clock::now();
     StatKey key{path_ ? path_ : "unknown", M_, K_, N_};
     ++s.table[key].calls;
     if (timed_) {
@@ -296,7 +313,7 @@ extern "C" void ppml_hip_mulmat_stats_reset(void) {
     std::lock_guard<std::mutex> lock(s.mu);
     fold_pending_locked(s, true);
     s.table.clear();
-    s.started = false;
+    s.first_call.reset();
 }
 
 extern "C" int ppml_hip_q8_last_path(void) { return g_q8_path; }

@@ -401,6 +401,37 @@ def test_dense_outer_product_mean_stress_shape_properties(ops):
     assert err <= RTOL * want.abs().max().item()
 
 
+def test_dense_outer_product_mean_stress_shape_against_the_oracle_on_both_pipes(ops, oracle):
+    """12288 x 256 -> 12288 (the shape bench.py times on both matrix pipes), six rows of the result against the CPU
+    oracle's own sums -- one product at a time, k ascending (src/backend/CPUKernels.cpp:763-771), then the 1/N scale
+    (src/backend/CPUKernels.cpp:1737-1754) -- instead of float64 on the device.  The fp32-pipe instance
+    (gemm_f32_kernel<1, false, true, false>) and the split one (split_operand_kernel + gemm_planes_kernel) both."""
+    N, LD = 256, 12288
+    g = torch.Generator(device="cuda").manual_seed(1)
+    a = torch.randn(N, LD, device="cuda", generator=g) * 0.1
+    b = torch.randn(N, LD, device="cuda", generator=g) * 0.1
+    rows = [0, 1, 127, 128, 5000, 12287]
+    ah, bh = a.cpu().numpy(), b.cpu().numpy()
+    at = np.ascontiguousarray(ah[:, rows].T)                   # [6][256]
+    bt = np.ascontiguousarray(bh.T)                            # [12288][256]
+    want = oracle.scale(oracle.mul_mat_f32(at, bt), float(np.float32(1.0) / np.float32(N)))
+    absprod = (np.abs(at).astype(np.float64) @ np.abs(bt).astype(np.float64).T) / N
+    results = {}
+    for pipe in ("split", "fp32"):
+        before = ops.set_f32_arithmetic(pipe)
+        try:
+            o = ops.mul_mat_tn(a, b, 1.0 / N)
+            ops.synchronize()
+        finally:
+            ops.set_f32_arithmetic(before)
+        got = o[rows].cpu().numpy()
+        _check(got, want, absprod)
+        results[pipe] = o
+    # the two pipes agree with each other to the same bar over the WHOLE output
+    diff = (results["split"] - results["fp32"]).abs().max().item()
+    assert diff <= RTOL * results["fp32"].abs().max().item()
+
+
 @pytest.fixture
 def fp32_pipe(ops):
     before = ops.set_f32_arithmetic("fp32")

@@ -74,3 +74,19 @@ def test_bad_arguments(ops):
     assert b"repeat_back_hip" in lib.ppml_hip_last_error()
     with pytest.raises(ValueError):
         ops.repeat_back(torch.zeros(2, 2, 2, 2, 2, device="cuda"), (2,))
+
+
+def test_sizes_whose_products_would_wrap_are_refused(ops):
+    """r * d computed in 64 bits wraps for sizes near 2^63 and would pass a product test; the launcher compares
+    quotients and refuses (nothing is launched, the operands are never read)."""
+    import ctypes as C
+    lib = ops._lib()
+    x = torch.zeros(16, device="cuda")
+    p = C.c_void_p(x.data_ptr())
+    big = 1 << 62
+    # copies x destination size = 2^62 * 4 = 2^64 -> 0 in 64 bits, "inside" a source of 16
+    assert lib.repeat_back_hip(p, p, 16, 1, 1, 1, 4, 1, 1, 1, big, 1, 1, 1, None) == 1
+    # destination sizes whose product wraps
+    assert lib.repeat_back_hip(p, p, big, big, 4, 1, big, big, 4, 1, 1, 1, 1, 1, None) == 1
+    # a plain case still runs
+    assert lib.repeat_back_hip(p, p, 16, 1, 1, 1, 4, 1, 1, 1, 4, 1, 1, 1, None) == 0

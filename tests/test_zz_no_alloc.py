@@ -65,3 +65,36 @@ def test_no_alloc_entry_point_refuses_what_does_not_fit():
     assert _call(lib.mul_mat_tn_noalloc_hip, one, one, one, 0, 4, 4, 1.0) == 1
     null = C.c_void_p(0)
     assert lib.mul_mat_tn_noalloc_hip(null, null, null, 4, 4, 4, 1.0, None) == 1
+
+
+def test_no_alloc_entry_point_inside_a_captured_graph():
+    """What the entry point is for: two calls recorded into a HIP graph, replayed several times with eager work and
+    synchronisations of the program's own in between, every replay checked against the allocating entry point."""
+    from proteinpredictmachinelearning_amd import cabi, ops
+
+    lib = ops._lib()
+    g = torch.Generator(device="cuda").manual_seed(5)
+    shapes = [(4100, 77, 3900), (1024, 2048, 1030)]          # planes split ahead; K slices with partial sums
+    ops_in = [(M, K, N, torch.randn(K, M, device="cuda", generator=g), torch.randn(K, N, device="cuda", generator=g),
+               torch.full((M, N), float("nan"), device="cuda")) for M, K, N in shapes]
+    # one eager call first: nothing is looked up or created for the first time while the stream is being captured
+    for M, K, N, a, b, out in ops_in:
+        assert _call(lib.mul_mat_tn_noalloc_hip, a, b, out, M, K, N, 0.5) == 0, cabi.last_error()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for M, K, N, a, b, out in ops_in:
+            assert _call(lib.mul_mat_tn_noalloc_hip, a, b, out, M, K, N, 0.5) == 0, cabi.last_error()
+    for replay in range(4):
+        for M, K, N, a, b, out in ops_in:                   # new operands for every replay, written the eager way
+            a.normal_(generator=g)
+            b.normal_(generator=g)
+            out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for M, K, N, a, b, out in ops_in:
+            want = torch.empty_like(out)
+            assert _call(lib.mul_mat_tn_hip, a, b, want, M, K, N, 0.5) == 0, cabi.last_error()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want), (replay, M, K, N)
