@@ -80,6 +80,45 @@ __device__ __forceinline__ void split4(const v4f& v, uint2 (&out)[3]) {
     out[2] = uint2{pack(t3[0], t3[1]), pack(t3[2], t3[3])};
 }
 
+// What the three parts cannot carry.  The split is exact for every binary32 number whose third part is itself a
+// bf16 number; two kinds of operand fall outside that: a non-finite one (x - x1 is NaN, so every product with its
+// lower parts is NaN where binary32 arithmetic gives +-inf), and one so small that its lower parts lie below bf16's
+// smallest step 2^-133 (they are cut off).  A SplitGuard collects both over the elements a thread splits: the bits
+// of the third parts that the packing drops (an OR of the words, looked at once at the end), and the sum of the
+// packed third parts (NaN as soon as one of them is -- they are finite numbers below 2^-16 of their operand otherwise,
+// so the sum cannot overflow; v_dot2_f32_bf16 adds two of them per instruction).  One vector instruction per element.
+// A contraction whose guard fires redoes the affected outputs in plain binary32 arithmetic, one product at a time, k
+// ascending: the reference's own loop.
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+struct SplitGuard {
+    uint32_t low = 0;
+    float sum3 = 0.0f;
+    __device__ __forceinline__ bool fired() const { return (low & 0xffffu) != 0 || sum3 != sum3; }
+};
+
+__device__ __forceinline__ void split4(const v4f& v, uint2 (&out)[3], SplitGuard& g) {
+    uint32_t t1[4], t2[4], t3[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t b1 = __float_as_uint(v[c]) & 0xffff0000u;
+        const float r1 = v[c] - __uint_as_float(b1);
+        const uint32_t b2 = __float_as_uint(r1) & 0xffff0000u;
+        const float r2 = r1 - __uint_as_float(b2);
+        t1[c] = b1; t2[c] = b2; t3[c] = __float_as_uint(r2);
+    }
+    const auto pack = [](uint32_t lo, uint32_t hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); };
+    out[0] = uint2{pack(t1[0], t1[1]), pack(t1[2], t1[3])};
+    out[1] = uint2{pack(t2[0], t2[1]), pack(t2[2], t2[3])};
+    out[2] = uint2{pack(t3[0], t3[1]), pack(t3[2], t3[3])};
+    g.low |= t3[0] | t3[1];
+    g.low |= t3[2] | t3[3];
+#if defined(__HIP_DEVICE_COMPILE__)                     // (the host pass of a .hip file does not know the builtin)
+    const v2bf ones = __builtin_bit_cast(v2bf, 0x3f803f80u);
+    g.sum3 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, out[2].x), ones, g.sum3, false);
+    g.sum3 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, out[2].y), ones, g.sum3, false);
+#endif
+}
+
 // XCD-aware work-group numbering.  Consecutive work-group ids go round-robin over the 8 XCDs, each
 // with its own L2.  This maps id -> a logical index such that every XCD walks one contiguous
 // eighth of the logical range, so neighbouring tiles (which share operand panels) meet in one L2.

@@ -420,19 +420,94 @@ int launch_f32_midk(const GemmParams& p, hipStream_t stream, const char* what) {
 // three dropped ones are below 2^-23 of |a||b| together, i.e. about one rounding of a binary32
 // product; the accumulation itself is binary32 as before.  What differs from the fp32 pipe is the
 // order of the roundings inside a group of 16 k, not their size.
-// Non-finite inputs: x - x1 is NaN for an infinite x, so +-inf in an operand gives NaN where the fp32
-// pipe gives +-inf or NaN; the clamped instances (whose result depends on that) stay on the fp32 pipe.
+// Operands the three parts cannot carry -- non-finite ones (x - x1 is NaN for an infinite x) and ones whose lower
+// parts fall below bf16's smallest step 2^-133 -- are noticed while they are split (SplitGuard, common.hpp), and the
+// outputs they touch are redone by plain_dot() below in plain binary32 arithmetic, the reference's own loop: the
+// split pipe then gives +-inf where the reference does and keeps every bit of a subnormal operand.  The clamped
+// instances stay on the fp32 pipe.
 constexpr int SPLIT_PITCH = 48;                   // bytes per tile row in a plane: 16 bf16, then 16 bytes of padding
 constexpr int SPLIT_PLANE = BM * SPLIT_PITCH;     // one of the three bf16 planes of a 128 x 16 operand tile
+
+// One output the reference's way (src/backend/CPUKernels.cpp:763-771, 836-884, 1006-1028): from the bias (or zero),
+// one product at a time, k ascending, every product and every sum rounded to binary32 on its own (this file is
+// compiled without contraction).  A and B are the plane's bases.
+__device__ __forceinline__ float plain_dot(const GemmParams& p, const float* __restrict__ A, const float* __restrict__ B, int m, int n) {
+    float s = p.bias ? p.bias[n] : 0.0f;
+    const int64_t ra = p.a_lm > 0 ? static_cast<int64_t>(m / p.a_lm) * p.a_mo + static_cast<int64_t>(m % p.a_lm) * p.a_mi
+                                  : static_cast<int64_t>(m) * p.a_rs;
+    const float* b = B + static_cast<int64_t>(n) * p.b_rs;
+    for (int k = 0; k < p.K; ++k) {
+        const float a = p.a_lm > 0 ? A[ra + static_cast<int64_t>(k / p.a_lk) * p.a_ko + static_cast<int64_t>(k % p.a_lk) * p.a_ki]
+                                   : A[ra + static_cast<int64_t>(k) * p.a_ks];
+        const float prod = a * b[static_cast<int64_t>(k) * p.b_ks];
+        s = s + prod;
+    }
+    return s;
+}
+
+// A whole tile of the output (rows x cols from (m0, n0) of the plane whose bases are A, B, C) by plain_dot, written
+// straight to C with the contraction's own output addressing: what a work-group does INSTEAD of storing its
+// accumulators when a SplitGuard fired for the tile.  One loop, no use of the accumulators: the ordinary path pays
+// nothing for it but the test.
+__device__ __forceinline__ void plain_tile(const GemmParams& p, const float* __restrict__ A, const float* __restrict__ B,
+                                           float* __restrict__ C, int m0, int n0, int rows, int cols, int tid) {
+    for (int e = tid; e < rows * cols; e += 256) {
+        const int m = m0 + e / cols, n = n0 + e % cols;
+        if (m >= p.M || n >= p.N) continue;
+        const float v = plain_dot(p, A, B, m, n) * p.alpha;
+        C[static_cast<int64_t>(m / p.c_lm) * p.c_mo + static_cast<int64_t>(m % p.c_lm) * p.c_mi +
+          static_cast<int64_t>(n / p.c_ln) * p.c_no + static_cast<int64_t>(n % p.c_ln) * p.c_ni] = v;
+    }
+}
+
+// The same for the kernels whose operands have contiguous rows (A(m, k) = A[k * a_ks + m]) and whose output plane is
+// dense (C[m * ldc + n]), without bias: it names nothing that those kernels do not hold already.
+__device__ __forceinline__ void plain_tile_rows(const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+                                                int a_ks, int b_ks, int ldc, int K, float alpha, int M, int N,
+                                                int m0, int n0, int side, int tid) {
+    for (int e = tid; e < side * side; e += 256) {
+        const int m = m0 + e / side, n = n0 + e % side;      // (side is a power of two)
+        if (m >= M || n >= N) continue;
+        float s = 0.0f;
+        for (int k = 0; k < K; ++k) {
+            const float prod = A[static_cast<int64_t>(k) * a_ks + m] * B[static_cast<int64_t>(k) * b_ks + n];
+            s = s + prod;
+        }
+        C[static_cast<int64_t>(m) * ldc + n] = s * alpha;
+    }
+}
+
+// Tile `t` of the short-K kernel's tile list (tiles of `side` x `side`, planes laid end to end) by plain_tile_rows, with
+// every parameter read afresh from the kernel-argument segment, where the launch's GemmParams lies first: the ordinary
+// path then holds nothing alive for this one (held in registers across the tile loop, the few pointers and sizes it
+// needs cost that loop a third of a microsecond per launch in scheduling freedom).
+__device__ __forceinline__ void shortk_tile_again_inline(int t, int side, int tid) {
+#if defined(__HIP_DEVICE_COMPILE__)                     // (the host pass of this file knows neither the builtin nor its address space)
+    typedef const __attribute__((address_space(4))) GemmParams* KernargParams;
+    KernargParams q = (KernargParams)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(q));                         // not the same values as the kernel's own copy, as far as the compiler knows
+#else
+    const GemmParams* q = nullptr;
+#endif
+    const int tiles_m = (q->M + side - 1) / side, tiles_n = (q->N + side - 1) / side;
+    const int plane = t / (tiles_m * tiles_n);
+    const int r = t - plane * tiles_m * tiles_n;
+    const int p2 = plane % q->np2, p3 = plane / q->np2;
+    const float* A = q->A + p2 * q->a_p2 + p3 * q->a_p3;
+    const float* B = q->B + (p2 / q->b_div2) * q->b_p2 + (p3 / q->b_div3) * q->b_p3;
+    float* C = q->C + p2 * q->c_p2 + p3 * q->c_p3;
+    plain_tile_rows(A, B, C, static_cast<int>(q->a_ks), static_cast<int>(q->b_ks), static_cast<int>(q->c_mi), q->K, q->alpha, q->M, q->N,
+                    (r / tiles_n) * side, (r % tiles_n) * side, side, tid);
+}
 
 // A thread's share of a 128 x 16 operand tile goes to the planes.  Operands with contiguous rows are
 // read one row and eight consecutive k per thread (eight loads, each contiguous across the lanes), the
 // others two rows and four consecutive k each.
 template <int MODE>
-__device__ __forceinline__ void split_store(uint8_t* __restrict__ planes, int tid, const v4f (&reg)[2]) {
+__device__ __forceinline__ void split_store(uint8_t* __restrict__ planes, int tid, const v4f (&reg)[2], SplitGuard& guard) {
     uint2 lo[3], hi[3];
-    split4(reg[0], lo);
-    split4(reg[1], hi);
+    split4(reg[0], lo, guard);
+    split4(reg[1], hi, guard);
     if (MODE == LOAD_ROW_CONTIG) {
         uint8_t* dst = planes + (tid & 127) * SPLIT_PITCH + (tid >> 7) * 16;
 #pragma unroll
@@ -560,9 +635,10 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
     const uint8_t* frag_a = lds_a + (wm + j) * SPLIT_PITCH + hh * 16;
     const uint8_t* frag_b = lds_b + (wn + j) * SPLIT_PITCH + hh * 16;
 
+    SplitGuard guard;
     for (int k0 = 0; k0 < p.K; k0 += BK) {
-        split_store<MODE>(lds_a, tid, ra);
-        split_store<MODE>(lds_b, tid, rb);
+        split_store<MODE>(lds_a, tid, ra, guard);
+        split_store<MODE>(lds_b, tid, rb, guard);
         __syncthreads();
         if (k0 + BK < p.K) load_both(k0 + BK);
         v8bf fa[2][3], fb[2][3];
@@ -581,6 +657,13 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
                 for (int tj = 0; tj < 2; ++tj)
                     acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][SPLIT_TERMS[q][0]], fb[tj][SPLIT_TERMS[q][1]], acc[ti][tj], 0, 0, 0);
         __syncthreads();
+    }
+
+    // an operand of this tile that the split could not carry (non-finite, or bits below 2^-133): the whole tile again,
+    // the reference's way
+    if (__syncthreads_or(guard.fired() ? 1 : 0)) {
+        plain_tile(p, A, B, C, m0, n0, BM, BN, tid);
+        return;
     }
 
     if (FAST_IO) store_acc_buffer<STREAM_C>(rsrc_c, static_cast<uint32_t>(p.c_mi) * 4u, p.N, p.alpha, acc, m0 + wm, n0 + wn, lane);
@@ -624,6 +707,10 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
     constexpr int LOADS = TM == 128 ? 2 : 1;          // 16-k chunks a thread loads separately (at 64 rows one pass covers K = 32)
     static_assert(2 * OPERAND >= (TM * TM + 32) * 4, "a whole tile of C, shifted by up to a line, fits the operands' LDS");
     __shared__ __attribute__((aligned(128))) uint8_t lds_ab[2 * OPERAND];
+    // "A SplitGuard fired for tile t": a thread whose guard fires writes t + 1 into the word of t's turn, and after the
+    // barrier everybody compares.  Nothing is cleared: a tile number never comes back within a work-group, and a stale
+    // or chance match only sends a tile down the plain path, whose result is right as well.
+    __shared__ int lds_guard[2];
     uint8_t* const lds_a = lds_ab;
     uint8_t* const lds_b = lds_ab + OPERAND;
 
@@ -680,25 +767,28 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
         }
     };
     // a lane's share goes to the three planes of its chunk: row lrow, bytes 16 * (octet % 2) of the row's 32
-    const auto split_to_lds = [&]() {
+    const auto split_to_lds = [&](int* fired, int mark) {
+        SplitGuard guard;
 #pragma unroll
         for (int l = 0; l < LOADS; ++l) {
             const int oct = (TM == 128 ? 2 * l : 0) + loct;                 // octet of k, 0..3
             const int at = (oct >> 1) * 3 * CHUNK_PLANE + lrow * SPLIT_PITCH + (oct & 1) * 16;
             uint2 lo[3], hi[3];
-            split4(ra[l][0], lo);
-            split4(ra[l][1], hi);
+            split4(ra[l][0], lo, guard);
+            split4(ra[l][1], hi, guard);
 #pragma unroll
             for (int q = 0; q < 3; ++q) *reinterpret_cast<uint4*>(lds_a + at + q * CHUNK_PLANE) = uint4{lo[q].x, lo[q].y, hi[q].x, hi[q].y};
-            split4(rb[l][0], lo);
-            split4(rb[l][1], hi);
+            split4(rb[l][0], lo, guard);
+            split4(rb[l][1], hi, guard);
 #pragma unroll
             for (int q = 0; q < 3; ++q) *reinterpret_cast<uint4*>(lds_b + at + q * CHUNK_PLANE) = uint4{lo[q].x, lo[q].y, hi[q].x, hi[q].y};
         }
+        if (guard.fired()) *fired = mark;               // (every writer writes the same value)
     };
 
     int t = part_begin + slot;
     if (t >= part_end) return;                          // whole work-group: no barrier is left behind
+    int turn = 0;
     Tile cur = tile_at(t);
     load_tile_regs(cur);
     const uint8_t* frag_a = lds_a + (wm + j) * SPLIT_PITCH + hh * 16;
@@ -708,8 +798,21 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
     const int c_bytes = static_cast<int>(p.M * p.c_mi * 4);
 
     while (true) {
-        split_to_lds();
+        split_to_lds(&lds_guard[turn], t + 1);
         __syncthreads();
+        // An operand of this tile that the split could not carry: the tile is stored as the matrix pipe leaves it all the
+        // same, and then -- once those stores have been acknowledged -- written again the reference's way.  Looking
+        // only after the stores keeps the test out of the chain load -> split -> MFMA -> store that a work-group
+        // with one tile consists of (decided ahead of the matrix work it cost half a microsecond per launch).
+        const int fired_mark = lds_guard[turn];         // requested with the fragments, looked at where the tile is stored
+        const auto again_if_fired = [&]() {
+            if (__builtin_amdgcn_readfirstlane(fired_mark) == t + 1) {                 // uniform over the work-group
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                shortk_tile_again_inline(t, TM, tid);
+            }
+        };
+        turn ^= 1;
         const int t_next = t + groups;
         const bool more = t_next < part_end;
         Tile nxt = cur;
@@ -778,6 +881,15 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
             v4f piece[PIECES];
 #pragma unroll
             for (int i = 0; i < PIECES; ++i) piece[i] = *reinterpret_cast<const v4f*>(stage + (tid + 256 * i) * 4);
+            // (the staged forms look at the guard here, between reading the pieces and storing them: nothing is out yet)
+            if (__builtin_amdgcn_readfirstlane(fired_mark) == t + 1) {                 // uniform over the work-group
+                shortk_tile_again_inline(t, TM, tid);
+                if (!more) break;
+                __syncthreads();
+                t = t_next;
+                cur = nxt;
+                continue;
+            }
 #pragma unroll
             for (int i = 0; i < PIECES; ++i) {
                 const int q = (tid + 256 * i) * 4;
@@ -814,6 +926,14 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
             v4f piece[PIECES];
 #pragma unroll
             for (int i = 0; i < PIECES; ++i) piece[i] = *reinterpret_cast<const v4f*>(stage + (tid + 256 * i) * 4);
+            if (__builtin_amdgcn_readfirstlane(fired_mark) == t + 1) {                 // uniform over the work-group
+                shortk_tile_again_inline(t, TM, tid);
+                if (!more) break;
+                __syncthreads();
+                t = t_next;
+                cur = nxt;
+                continue;
+            }
             float* const tile_base = cur.C + static_cast<int64_t>(cur.m0) * p.c_mi + cur.n0;
 #pragma unroll
             for (int i = 0; i < PIECES; ++i) {
@@ -845,6 +965,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
                 }
             }
         }
+        again_if_fired();
         if (!more) break;
         t = t_next;
         cur = nxt;
@@ -962,6 +1083,7 @@ struct SplitJob {
     int64_t rs, ks;                                   // element (row, k) at src[row * rs + k * ks] ...
     int lm, lk;                                       // ... or, with lm > 0, at the compound address of LOAD_SPLIT_A
     int64_t mo, mi, ko, ki;
+    int* fired;                                       // [rows_pad / 32]: set where a SplitGuard fired for that tile of 32 rows
 };
 
 template <bool KS1, bool COMPOUND>
@@ -1006,13 +1128,20 @@ __global__ __launch_bounds__(256) void split_operand_kernel(const SplitJob jb) {
         }
     }
     uint2 lo[3], hi[3];
-    split4(v[0], lo);
-    split4(v[1], hi);
+    SplitGuard guard;
+    split4(v[0], lo, guard);
+    split4(v[1], hi, guard);
 #pragma unroll
     for (int s = 0; s < 3; ++s) {
         uint8_t* dst = jb.dst + ((static_cast<int64_t>(s) * jb.chunks + c) * jb.rows_pad + (row & ~31)) * 32 + kq * 512 + (row & 31) * 16;
         *reinterpret_cast<uint4*>(dst) = uint4{lo[s].x, lo[s].y, hi[s].x, hi[s].y};
     }
+    if (guard.fired()) jb.fired[row >> 5] = 1;          // (rare; every writer writes the same value)
+}
+
+__global__ __launch_bounds__(256) void clear_flags_kernel(int* __restrict__ flags, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) flags[i] = 0;
 }
 
 // Work-group tile 256 x 128, four waves of 128 x 64 each (eight accumulator tiles): a fragment read from
@@ -1024,7 +1153,8 @@ constexpr int PLANES_MIN_SLICE_CHUNKS = 16;      // a K slice is at least 256 lo
 template <bool SPLIT_C, bool STREAM_C>
 __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p, const uint8_t* __restrict__ wa,
                                                              const uint8_t* __restrict__ wb, int chunks, int ma_pad, int nb_pad,
-                                                             int slice_chunks, float* __restrict__ partial) {
+                                                             int slice_chunks, float* __restrict__ partial,
+                                                             const int* __restrict__ fired_a, const int* __restrict__ fired_b) {
     constexpr int A_PLANE = PBM * 32, B_PLANE = BN * 32;      // fragments of 1 KB, no padding
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * A_PLANE];
     __shared__ __attribute__((aligned(16))) uint8_t lds_b[3 * B_PLANE];
@@ -1111,13 +1241,25 @@ __global__ __launch_bounds__(256, 2) void gemm_planes_kernel(const GemmParams p,
                     __builtin_nontemporal_store(acc[ti][tj][r], dst + static_cast<size_t>(ti * 32 + mfma32_row(r, lane)) * nb_pad + tj * 32);
         return;
     }
+    // a tile of 32 rows of either operand that the split could not carry: this tile again, the reference's way
+    // (the flags are the same for the whole work-group; with K slices reduce_slices_kernel looks at them instead)
+    int fired = 0;
+#pragma unroll
+    for (int i = 0; i < PBM / 32; ++i) fired |= fired_a[(m0 >> 5) + i];
+#pragma unroll
+    for (int i = 0; i < BN / 32; ++i) fired |= fired_b[(n0 >> 5) + i];
+    if (fired) {
+        plain_tile(p, p.A, p.B, p.C, m0, n0, PBM, BN, tid);
+        return;
+    }
     store_acc<SPLIT_C, STREAM_C, false, false, 4>(p, p.C, acc, m0 + wm, n0 + wn, lane);
 }
 
 // C = alpha * (bias + sum over the K slices, in slice order) with the contraction's own output addressing
 template <bool SPLIT_C>
 __global__ __launch_bounds__(256) void reduce_slices_kernel(const GemmParams p, const float* __restrict__ partial,
-                                                            int slices, int ma_pad, int nb_pad) {
+                                                            int slices, int ma_pad, int nb_pad,
+                                                            const int* __restrict__ fired_a, const int* __restrict__ fired_b) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     const int nq = (p.N + 3) / 4;
     const int m = static_cast<int>(idx / nq);
@@ -1130,6 +1272,10 @@ __global__ __launch_bounds__(256) void reduce_slices_kernel(const GemmParams p, 
     }
     const float* src = partial + static_cast<size_t>(m) * nb_pad + n4;          // nb_pad is a multiple of 128
     for (int s = 0; s < slices; ++s) sum += *reinterpret_cast<const v4f*>(src + static_cast<size_t>(s) * ma_pad * nb_pad);
+    if (fired_a[m >> 5] | fired_b[n4 >> 5]) {           // operands the split could not carry: these four again, the reference's way
+#pragma unroll
+        for (int c = 0; c < 4; ++c) if (n4 + c < p.N) sum[c] = plain_dot(p, p.A, p.B, m, n4 + c);
+    }
     int64_t roff;
     if (SPLIT_C) roff = static_cast<int64_t>(m / p.c_lm) * p.c_mo + static_cast<int64_t>(m % p.c_lm) * p.c_mi;
     else         roff = static_cast<int64_t>(m) * p.c_mi;
@@ -1218,17 +1364,19 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
         slices = (chunks + slice_chunks - 1) / slice_chunks;
         const size_t a_bytes = static_cast<size_t>(3) * chunks * ma_pad * 32, b_bytes = static_cast<size_t>(3) * chunks * nb_pad * 32;
         const size_t part_bytes = slices > 1 ? static_cast<size_t>(slices) * ma_pad * nb_pad * 4 : 0;
+        const int n_flags = ma_pad / 32 + nb_pad / 32;  // one per tile of 32 rows of either operand (see SplitGuard)
+        const size_t flag_bytes = (static_cast<size_t>(n_flags) * 4 + 255) / 256 * 256;
+        const size_t ws_bytes = a_bytes + b_bytes + part_bytes + flag_bytes;
         uint8_t* ws = nullptr;
         if (fixed_ws) {
-            if (a_bytes + b_bytes + part_bytes > fixed_cap) {
-                set_error("%s: this contraction needs %zu bytes of workspace, the static one holds %zu", what,
-                          a_bytes + b_bytes + part_bytes, fixed_cap);
+            if (ws_bytes > fixed_cap) {
+                set_error("%s: this contraction needs %zu bytes of workspace, the static one holds %zu", what, ws_bytes, fixed_cap);
                 return RC_BAD_ARGS;
             }
             ws = fixed_ws;
         } else {
             hipMemPool_t pool = workspace_pool();
-            if (pool && hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), a_bytes + b_bytes + part_bytes, pool, stream) != hipSuccess) {
+            if (pool && hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), ws_bytes, pool, stream) != hipSuccess) {
                 (void)hipGetLastError();
                 ws = nullptr;
             }
@@ -1239,23 +1387,28 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
             q.np2 = slices;                              // the tile numbering walks the slices as planes
             float* partial = slices > 1 ? reinterpret_cast<float*>(ws + a_bytes + b_bytes) : nullptr;
             const dim3 pgrid(static_cast<unsigned>(q.tiles_m * q.tiles_n * slices));
-            const SplitJob ja{p.A, ws, p.M, ma_pad, p.K, chunks, p.a_rs, p.a_ks, p.a_lm, p.a_lk, p.a_mo, p.a_mi, p.a_ko, p.a_ki};
-            const SplitJob jb{p.B, ws + a_bytes, p.N, nb_pad, p.K, chunks, p.b_rs, p.b_ks, 0, 0, 0, 0, 0, 0};
-            int rc = launch_split(ja, stream);
+            int* fired_a = reinterpret_cast<int*>(ws + a_bytes + b_bytes + part_bytes);
+            int* fired_b = fired_a + ma_pad / 32;
+            const SplitJob ja{p.A, ws, p.M, ma_pad, p.K, chunks, p.a_rs, p.a_ks, p.a_lm, p.a_lk, p.a_mo, p.a_mi, p.a_ko, p.a_ki, fired_a};
+            const SplitJob jb{p.B, ws + a_bytes, p.N, nb_pad, p.K, chunks, p.b_rs, p.b_ks, 0, 0, 0, 0, 0, 0, fired_b};
+            // (a small kernel, not a memset: this launcher may be recorded into a graph)
+            hipLaunchKernelGGL(clear_flags_kernel, dim3((n_flags + 255) / 256), block, 0, stream, fired_a, n_flags);
+            int rc = check_launch(what);
+            if (rc == RC_OK) rc = launch_split(ja, stream);
             if (rc == RC_OK) rc = launch_split(jb, stream);
             if (rc == RC_OK) {
                 const bool stream_c = p.stream_c && !partial;
-                if (split && !partial) { if (stream_c) hipLaunchKernelGGL((gemm_planes_kernel<true, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial);
-                                         else hipLaunchKernelGGL((gemm_planes_kernel<true, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial); }
-                else                   { if (stream_c) hipLaunchKernelGGL((gemm_planes_kernel<false, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial);
-                                         else hipLaunchKernelGGL((gemm_planes_kernel<false, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial); }
+                if (split && !partial) { if (stream_c) hipLaunchKernelGGL((gemm_planes_kernel<true, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial, fired_a, fired_b);
+                                         else hipLaunchKernelGGL((gemm_planes_kernel<true, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial, fired_a, fired_b); }
+                else                   { if (stream_c) hipLaunchKernelGGL((gemm_planes_kernel<false, true>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial, fired_a, fired_b);
+                                         else hipLaunchKernelGGL((gemm_planes_kernel<false, false>), pgrid, block, 0, stream, q, ws, ws + a_bytes, chunks, ma_pad, nb_pad, slice_chunks, partial, fired_a, fired_b); }
                 rc = check_launch(what);
             }
             if (rc == RC_OK && partial) {
                 const int64_t threads = static_cast<int64_t>(p.M) * ((p.N + 3) / 4);
                 const dim3 rgrid(static_cast<unsigned>((threads + 255) / 256));
-                if (split) hipLaunchKernelGGL((reduce_slices_kernel<true>), rgrid, block, 0, stream, p, partial, slices, ma_pad, nb_pad);
-                else       hipLaunchKernelGGL((reduce_slices_kernel<false>), rgrid, block, 0, stream, p, partial, slices, ma_pad, nb_pad);
+                if (split) hipLaunchKernelGGL((reduce_slices_kernel<true>), rgrid, block, 0, stream, p, partial, slices, ma_pad, nb_pad, fired_a, fired_b);
+                else       hipLaunchKernelGGL((reduce_slices_kernel<false>), rgrid, block, 0, stream, p, partial, slices, ma_pad, nb_pad, fired_a, fired_b);
                 rc = check_launch(what);
             }
             if (!fixed_ws && hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();

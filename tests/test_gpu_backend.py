@@ -493,26 +493,36 @@ def test_backward_of_a_biased_linear_stays_on_the_device(be, oracle):
 
 def test_f32_arithmetic_is_a_field_of_the_backend(be, oracle):
     # two backends with different pipes do not disturb each other or the calling thread's own setting
+    import torch
     from proteinpredictmachinelearning_amd import ops
     M, K, N = 70, 40, 50
     rng = np.random.default_rng(3)
     A = rng.standard_normal((M, K)).astype(np.float32)
     Wm = rng.standard_normal((N, K)).astype(np.float32)
-    A[3, 5] = np.inf                                              # tells the pipes apart: NaN (split) or inf (fp32)
-    want = oracle.mul_mat_f32(A, Wm)
+    # what each pipe gives through the launcher: the sums differ in their last bits, which tells the pipes apart
+    per_pipe = {}
+    for pipe in ("split", "fp32"):
+        before = ops.set_f32_arithmetic(pipe)
+        try:
+            per_pipe[pipe] = ops.mul_mat(torch.from_numpy(A).cuda(), torch.from_numpy(Wm).cuda()).cpu().numpy()
+        finally:
+            ops.set_f32_arithmetic(before)
+    assert not np.array_equal(per_pipe["split"], per_pipe["fp32"])
     other = B.Backend(0)
     other.set_f32_arithmetic("fp32")
+    be.set_f32_arithmetic("split")
     assert ops.set_f32_arithmetic("split") in ("split", "fp32")
     try:
         for _ in range(2):
             n1 = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [_leaf(be, A), _leaf(be, Wm)])
             n2 = B.Tensor((N, M), B.F32, B.OP_MUL_MAT, [_leaf(other, A), _leaf(other, Wm)])
             assert be.graph_compute([n1]) == B.SUCCESS and other.graph_compute([n2]) == B.SUCCESS
-            assert np.isnan(be.download(n1).reshape(M, N)[3]).all()
-            assert (other.download(n2).reshape(M, N)[3] == want[3]).all()
+            assert np.array_equal(be.download(n1).reshape(M, N), per_pipe["split"])
+            assert np.array_equal(other.download(n2).reshape(M, N), per_pipe["fp32"])
         assert ops.set_f32_arithmetic("split") == "split"        # the thread's setting came back after each call
     finally:
         other.set_f32_arithmetic(None)
+        be.set_f32_arithmetic(None)
 
 
 # ----------------------------------------------------------------------------- element-wise nodes and their folding

@@ -259,13 +259,14 @@ def test_attention_logits_long_rows_of_whole_lines(ops, oracle, planes, rows, co
 
 
 # ----------------------------------------------------------------------------- non-finite and subnormal operands
-def test_infinite_operand_gives_nan_on_the_split_pipe_and_inf_on_the_fp32_pipe(ops, oracle):
+def test_infinite_operands_give_the_references_infinities_on_both_pipes(ops, oracle):
     # The reference's loop (src/backend/CPUKernels.cpp:763-771) carries an infinite operand through: inf * b
-    # summed with finite terms is +-inf.  The default arithmetic here splits every operand into three bf16
-    # parts by subtraction, and inf - inf is NaN: an output whose sum touches an infinite operand is NaN
-    # instead of +-inf.  Outputs that do not touch it are unaffected, NaN operands give NaN either way, and
-    # the fp32 pipe (ppml_hip_set_f32_arithmetic(1)) gives the reference's +-inf.  This test pins all four.
-    M, K, N = 70, 40, 50
+    # summed with finite terms is +-inf.  The default arithmetic splits every operand into three bf16 parts by
+    # subtraction, and inf - inf is NaN -- so the split notices such an operand (the sum of the third parts turns
+    # NaN) and the tile is computed again in plain binary32 arithmetic, one product at a time, k ascending: the
+    # outputs that touch it come out exactly as the reference's do (equal bits: it IS the reference's loop), the
+    # other outputs of that tile too, and tiles it does not touch keep the matrix pipe's sums.
+    M, K, N = 300, 40, 270
     rng = np.random.default_rng(3)
     a = rng.standard_normal((M, K)).astype(np.float32)
     b = rng.standard_normal((N, K)).astype(np.float32)
@@ -273,40 +274,99 @@ def test_infinite_operand_gives_nan_on_the_split_pipe_and_inf_on_the_fp32_pipe(o
     a[3, 5] = np.inf
     a[9, 0] = -np.inf
     a[20, 7] = np.nan
+    b[200, 3] = np.inf                                      # a column of the second tile column
     want = oracle.mul_mat_f32(a, b)
-    assert np.isinf(want[3]).all() and np.isinf(want[9]).all() and np.isnan(want[20]).all()
-    got = ops.mul_mat(_dev(a), _dev(b)).cpu().numpy()
-    clean = np.ones(M, bool)
-    clean[[3, 9, 20]] = False
-    _check(got[clean], want[clean])
-    assert np.isnan(got[[3, 9, 20]]).all()                  # the documented difference: NaN where the reference has +-inf
-    before = ops.set_f32_arithmetic("fp32")
-    try:
-        got32 = ops.mul_mat(_dev(a), _dev(b)).cpu().numpy()
-    finally:
-        ops.set_f32_arithmetic(before)
-    _check(got32[clean], want[clean])
-    assert (got32[[3, 9]] == want[[3, 9]]).all() and np.isnan(got32[20]).all()
+    assert np.isinf(want[3]).all() and np.isinf(want[9]).all() and np.isnan(want[20]).all() and np.isinf(want[100, 200])
+    for pipe in ("split", "fp32"):
+        before = ops.set_f32_arithmetic(pipe)
+        try:
+            got = ops.mul_mat(_dev(a), _dev(b)).cpu().numpy()
+        finally:
+            ops.set_f32_arithmetic(before)
+        special = ~np.isfinite(want)
+        assert np.array_equal(np.isnan(got), np.isnan(want)), pipe
+        assert np.array_equal(got[special & ~np.isnan(want)], want[special & ~np.isnan(want)]), pipe       # the same infinities
+        _check(got[~special], want[~special])
+        if pipe == "split":
+            # the tiles that were redone are the reference's loop bit for bit: rows 0..127 (first tile row) and the
+            # second tile column (columns 128..255)
+            finite = np.isfinite(want)
+            assert np.array_equal(got[:128][finite[:128]], want[:128][finite[:128]])
+            assert np.array_equal(got[:, 128:256][finite[:, 128:256]], want[:, 128:256][finite[:, 128:256]])
+
+
+@pytest.mark.parametrize("kind", ["inf", "tiny"])
+def test_operands_the_split_cannot_carry_in_every_kernel_family(ops, oracle, kind):
+    """The same guard in every kernel that splits: the batched generic one (out_prod with planes), the short-K
+    persistent one in its store forms (attention logits: ordinary, contiguous range, rows through LDS), the
+    split-ahead one (large single plane) and its K-sliced form.  `tiny`: operands around 2^-128 against 2^100 --
+    their lower parts lie below bf16's smallest step, so the split would cut them off."""
+    rng = np.random.default_rng(17)
+
+    def plant(x):
+        flat = x.reshape(-1)
+        idx = rng.choice(flat.size, size=max(1, flat.size // 5000), replace=False)
+        if kind == "inf":
+            flat[idx] = np.where(rng.random(idx.size) < 0.5, np.inf, -np.inf).astype(np.float32)
+        else:
+            flat[idx] = (rng.standard_normal(idx.size) * 2.0 ** -128).astype(np.float32)
+        return x
+
+    def agree(got, want, absprod):
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        inf = np.isinf(want)
+        assert np.array_equal(got[inf], want[inf])
+        ok = np.isfinite(want)
+        err = np.abs(got[ok].astype(np.float64) - want[ok].astype(np.float64))
+        assert (err <= RTOL * absprod[ok] + 1e-45).all(), float(np.max(err / (absprod[ok] + 1e-300)))
+
+    scale_b = np.float32(2.0 ** 100 if kind == "tiny" else 1.0)
+    # attention logits (short K): 103-wide ragged planes (ordinary stores), enough of them for the contiguous-range
+    # form, and 256-wide planes (rows through LDS)
+    for planes, L, D in [(12, 103, 32), (300, 103, 32), (40, 256, 32), (9, 50, 16)]:
+        k = plant(rng.standard_normal((1, planes, D, L)).astype(np.float32))
+        q = rng.standard_normal((1, planes, D, L)).astype(np.float32) * scale_b
+        got = ops.out_prod(_dev(k), _dev(q), scale=0.5).cpu().numpy()
+        with np.errstate(invalid="ignore", over="ignore"):
+            want = oracle.scale(oracle.out_prod(k, q), 0.5)
+            absprod = np.einsum("bpdi,bpdj->bpji", np.abs(k).astype(np.float64), np.abs(q).astype(np.float64)) * 0.5
+        agree(got, want, np.nan_to_num(absprod, nan=0.0, posinf=0.0))
+    # the generic batched kernel (K > 32)
+    k = plant(rng.standard_normal((2, 3, 70, 90)).astype(np.float32))
+    q = rng.standard_normal((2, 3, 70, 140)).astype(np.float32) * scale_b
+    got = ops.out_prod(_dev(k), _dev(q)).cpu().numpy()
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = oracle.out_prod(k, q)
+        absprod = np.einsum("bpdi,bpdj->bpji", np.abs(k).astype(np.float64), np.abs(q).astype(np.float64))
+    agree(got, want, np.nan_to_num(absprod, nan=0.0, posinf=0.0))
+    # split ahead (>= 8 x 8 tiles of 128, >= 512 work-groups), and cut into K slices (few tiles, long K)
+    for M, K, N in [(2100, 48, 4200), (300, 4096, 1030)]:
+        a = plant(rng.standard_normal((M, K)).astype(np.float32))
+        b = rng.standard_normal((N, K)).astype(np.float32) * scale_b
+        if kind == "inf":
+            b = plant(b)
+        got = ops.mul_mat(_dev(a), _dev(b)).cpu().numpy()
+        with np.errstate(invalid="ignore", over="ignore"):
+            want = oracle.mul_mat_f32(a, b)
+            absprod = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64).T
+        agree(got, want, np.nan_to_num(absprod, nan=0.0, posinf=0.0))
 
 
 def test_subnormal_operands(ops, oracle):
     # Operands below 2^-126 against large ones: the products are ordinary numbers, so flushing the small
-    # operand to zero would lose the whole result.  The fp32 pipe keeps subnormal operands whole and meets the
-    # ordinary bar.  The default split arithmetic cannot: its parts are bf16 numbers, whose grid stops at
-    # 2^-133, so a subnormal operand is cut to a multiple of 2^-133 (an ABSOLUTE error below 2^-133 per element,
-    # where the reference's loop, src/backend/CPUKernels.cpp:763-771, keeps all of its bits down to 2^-149).
-    # This test pins both: the bound sum_k 2^-133 |b_k| on the split pipe, and that it is not a flush to zero
-    # down to that grid.
+    # operand to zero would lose the whole result, and so would cutting it to bf16's grid, which stops at 2^-133
+    # (the reference's loop, src/backend/CPUKernels.cpp:763-771, keeps all of its bits down to 2^-149).  The fp32
+    # pipe keeps subnormal operands whole; the split notices the bits its third part drops and computes the tile
+    # again in plain binary32 arithmetic.  Both meet the ordinary bar.
     M, K, N = 64, 48, 40
     rng = np.random.default_rng(5)
-    for shift in (-127, -130):
+    for shift in (-127, -130, -140):
         a = (rng.standard_normal((M, K)) * 2.0 ** shift).astype(np.float32)
         assert (np.abs(a) < 2.0 ** -126).mean() > 0.6 and (a != 0).mean() > 0.9
         b = (rng.standard_normal((N, K)) * 2.0 ** 100).astype(np.float32)
         want = oracle.mul_mat_f32(a, b).astype(np.float64)
-        assert np.abs(want).max() > 2.0 ** -32
+        assert np.abs(want).max() > 2.0 ** -42
         absprod = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64).T
-        grid = 2.0 ** -133 * np.abs(b).astype(np.float64).sum(axis=1)[None, :]
         for mode in ("split", "fp32"):
             before = ops.set_f32_arithmetic(mode)
             try:
@@ -314,13 +374,11 @@ def test_subnormal_operands(ops, oracle):
                 got_t = ops.mul_mat(_dev(b), _dev(a)).cpu().numpy().astype(np.float64)      # subnormal second operand
             finally:
                 ops.set_f32_arithmetic(before)
-            for g, w, ap, gr in ((got, want, absprod, grid), (got_t, want.T, absprod.T, grid.T)):
+            for g, w, ap in ((got, want, absprod), (got_t, want.T, absprod.T)):
                 err = np.abs(g - w)
-                if mode == "fp32":
-                    assert (err <= RTOL * ap).all(), f"fp32 pipe: {np.max(err / ap):.3e}"
-                else:
-                    assert (err <= RTOL * ap + gr).all(), f"split pipe: {np.max(err / (RTOL * ap + gr)):.3e} of its bound"
-                    assert (g != 0).mean() > 0.99                 # cut to the bf16 grid, not flushed
+                assert (err <= RTOL * ap).all(), f"{mode} pipe: {np.max(err / ap):.3e}"
+                if mode == "split":
+                    assert np.array_equal(g, w)           # the reference's own loop
     # a subnormal RESULT from ordinary operands (products that underflow) is kept on either pipe
     a2 = (rng.standard_normal((M, K)) * 2.0 ** -70).astype(np.float32)
     b2 = (rng.standard_normal((N, K)) * 2.0 ** -70).astype(np.float32)

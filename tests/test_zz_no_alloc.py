@@ -58,10 +58,11 @@ def test_no_alloc_entry_point_refuses_what_does_not_fit():
 
     lib = ops._lib()
     one = torch.zeros(16, device="cuda")
-    # 4096^3 wants 192 MiB of planes: refused before anything is launched (the operands are never read)
+    # 4096^3 wants 192 MiB of planes (and 1 KiB of guard flags): refused before anything is launched (the operands
+    # are never read)
     assert _call(lib.mul_mat_tn_noalloc_hip, one, one, one, 4096, 4096, 4096, 1.0) == 1
     msg = cabi.last_error()
-    assert "201326592" in msg and "67108864" in msg, msg
+    assert str(201326592 + 1024) in msg and "67108864" in msg, msg
     assert _call(lib.mul_mat_tn_noalloc_hip, one, one, one, 0, 4, 4, 1.0) == 1
     null = C.c_void_p(0)
     assert lib.mul_mat_tn_noalloc_hip(null, null, null, 4, 4, 4, 1.0, None) == 1
