@@ -62,11 +62,13 @@ int ppml_hip_set_f32_arithmetic(int mode);
  * C[m*N+n] = (bias ? bias[n] : 0) + sum_k A[m*K+k] * B[n*K+k].  bias may be NULL.
  * Arithmetic of this and the other f32 contractions below: each binary32 operand is the exact sum of
  * three bf16 numbers; six of the nine partial products (all but 2^-23 of |a||b|) are formed exactly on
- * the bf16 matrix pipe and summed in binary32.  Two kinds of operand fall outside that: an infinite operand
- * yields NaN where the reference's loop yields +-inf, and a subnormal operand (below 2^-126) is cut to a
- * multiple of 2^-133, bf16's smallest step (the reference keeps its bits down to 2^-149).  Callers that must
- * have the reference's results on such operands select the fp32 pipe (ppml_hip_set_f32_arithmetic(1)), which
- * carries both through.  Contractions of at
+ * the bf16 matrix pipe and summed in binary32.  Two kinds of operand fall outside what three bf16 parts
+ * carry: a non-finite one, and one with bits below 2^-133, bf16's smallest step (subnormal operands and the
+ * smallest normal ones).  The kernels notice both while they split the operands and redo the outputs of the
+ * affected tile in plain binary32 arithmetic, one product at a time with k ascending (the reference's own
+ * loop): +-inf, NaN and the bits down to 2^-149 come out as the reference's.  The fused attention kernels
+ * (flash_attn_*_hip) split without that check; ppml_hip_set_f32_arithmetic(1) selects the fp32 pipe, which
+ * carries every operand, for all of them.  Contractions of at
  * least 512 work-groups of 256 x 128 outputs take a workspace of 6 bytes per operand element from a
  * stream-ordered pool (allocated and freed on `stream`); no other launcher allocates. */
 int mul_mat_hip(const float *A, const float *B, float *C, int M, int K, int N,
@@ -119,8 +121,9 @@ int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K,
  *   flags bit 1: quantize X with the Q8_1 rule of quantize_rows_q8_1_hip instead of the Q8_0 rule:
  *                the numbers mul_mat_q8_cuda itself produces (src/cuda/MulMatQ8Kernel.cu:520-527
  *                quantizes activations to Q8_1 and settles with their d).
- *   flags bits 2..7 (PPML_Q8_FLAG_*): restrict the choice among the kernels that serve a Q8_0M weight with
- *                c_trans = 1, all of which give the same bits; for tests and measurements.
+ *   flags bits 2..7 (PPML_Q8_FLAG_*): restrict the choice among the kernels that serve a Q8_0M weight, all
+ *                of which give the same bits; for tests and measurements.  (With c_trans = 0 the choice is
+ *                between the weight-stationary kernel without column parts and the general one.)
  *   xq_dump  (may be NULL): receives the Q8_0 blocks the kernel made of X, [N][K/32] block_q8_0
  *   sums_dump(may be NULL): receives the per-block int32 sums, [(n*M+m)*(K/32)+ib]            */
 enum {

@@ -690,7 +690,7 @@ constexpr int ws_staging_regs(int nblk, int nw = 8) {   // 8 registers per unit 
 }
 constexpr int ws_compiler_vgprs(int nblk, int nw = 8) { return 256 - ws_staging_regs(nblk, nw); }
 
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY, bool CT0>
 __device__ __forceinline__ void q8_linear_ws_body(
     const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
     int M, int N, int ntiles, int npart, int relu,
@@ -1019,14 +1019,21 @@ __device__ __forceinline__ void q8_linear_ws_body(
                 o.w1 = my_wq[((t - (TPW - WL)) * NBLK + b + 1) * 64];
             }
         };
+        // CT0 (C stored [M][N], features outermost): the operands change places, in the block sums and in the scale
+        // tables alike, so that a lane holds one token and sixteen features instead of one feature and sixteen tokens
+        // and a half-wave store is again one line of a C row.  Both operands of these MFMAs have the same fragment
+        // layout (lane % 32 = row or column, lane / 32 = half of k), the products and their order of addition are the
+        // same: same bits.
         auto scale_tables = [&](const uint2& da, const uint2& dw) {
             typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-            return __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, da), __builtin_bit_cast(v4h, dw), zero_f2, 0, 0, 0);
+            if constexpr (CT0) return __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, dw), __builtin_bit_cast(v4h, da), zero_f2, 0, 0, 0);
+            else return __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, da), __builtin_bit_cast(v4h, dw), zero_f2, 0, 0, 0);
         };
         auto block_sum = [&](int st, const v4i& a, const v4i& w_lds) {
             const int t = st / NBLK, b = st % NBLK;
             const v4i w = t < TPW - WL ? wq[t < TPW - WL ? t : 0][b] : w_lds;
-            return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, w, magic_i, 0, 0, 0);
+            if constexpr (CT0) return __builtin_amdgcn_mfma_i32_32x32x32_i8(w, a, magic_i, 0, 0, 0);
+            else return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, w, magic_i, 0, 0, 0);
         };
         // 1.5 * 2^23 + sum -> float(sum), on the matrix pipe
         auto to_float = [&](const v16i& biased) {
@@ -1041,12 +1048,13 @@ __device__ __forceinline__ void q8_linear_ws_body(
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[r] = __builtin_fmaf(sum[r], scl[r], acc[r]);
             }
-            const int m = (ct0 + t * NW + wave) * 32 + j;   // this lane's output feature
+            const int m = (ct0 + t * NW + wave) * 32 + (CT0 ? 0 : j);   // this lane's output feature (CT0: the first of its column tile)
             if (DUMP && sums_dump) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int tok = tok0 + mfma32_row(r, lane);
-                    if (tok < N && m < M) sums_dump[(static_cast<int64_t>(tok) * M + m) * NBLK + b] = static_cast<int>(sum[r]);
+                    const int tok = CT0 ? tok0 + j : tok0 + mfma32_row(r, lane);
+                    const int mm = CT0 ? m + mfma32_row(r, lane) : m;
+                    if (tok < N && mm < M) sums_dump[(static_cast<int64_t>(tok) * M + mm) * NBLK + b] = static_cast<int>(sum[r]);
                 }
             }
             if (b == NBLK - 1) {
@@ -1060,8 +1068,16 @@ __device__ __forceinline__ void q8_linear_ws_body(
                 // 2^31, which stays outside whatever is added to it (C is below 2^31 bytes, see the launcher).
                 // Stepping the offset costs one add per store; a scalar offset per row would cost none but is not
                 // range-checked, and its sixteen predicates per column tile ran for every tile, ragged or not.
-                uint32_t off = m < M ? (static_cast<uint32_t>(tok0 + 4 * hh) * M + m) * 4u : 0x80000000u;
-                int pitch = M * 4;
+                // CT0: rows of C are features.  The lane's token picks the column, tokens past the end start from 2^31;
+                // feature rows past M lie behind the end of the buffer (the launcher keeps the padded height of C
+                // below 2^31 bytes, so the offsets of live lanes do not wrap), and column tiles past the padded end,
+                // which repeat the last tile's weights, start from 2^31 like the tokens.
+                uint32_t off;
+                if constexpr (CT0)
+                    off = (tok0 + j < N && m < mct_pad * 32) ? (static_cast<uint32_t>(m + 4 * hh) * N + (tok0 + j)) * 4u : 0x80000000u;
+                else
+                    off = m < M ? (static_cast<uint32_t>(tok0 + 4 * hh) * M + m) * 4u : 0x80000000u;
+                int pitch = (CT0 ? N : M) * 4;
                 asm volatile("" : "+s"(pitch));          // one scalar, not sixteen folded row offsets
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
@@ -1153,33 +1169,33 @@ __device__ __forceinline__ void q8_linear_ws_body(
 // value counts architectural and accumulation registers separately): 120 keeps it below v240.  A
 // value the compiler does not honour would go unnoticed until its registers and the staged tile
 // collide, so the build checks the generated code (check_ws_isa.py).
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY = false>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY = false, bool CT0 = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(120)))
 void q8_linear_ws_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                          int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                          int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 120, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT, QEARLY>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT, QEARLY, CT0>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY = false>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY = false, bool CT0 = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(112)))
 void q8_linear_ws32_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 112, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT, QEARLY>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT, QEARLY, CT0>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
-template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY = false>
+template <int NW, int TPW, int NBLK, int WL, bool DUMP, bool Q81, bool CSPLIT, bool QEARLY = false, bool CT0 = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2), amdgpu_num_vgpr(96)))
 void q8_linear_ws64_kernel(const uint8_t* __restrict__ W, const float* __restrict__ X, float* __restrict__ C,
                            int M, int N, int ntiles, int npart, int relu, uint8_t* __restrict__ xq_dump,
                            int32_t* __restrict__ sums_dump) {
     static_assert(ws_compiler_vgprs(NBLK, NW) == 2 * 96, "staging size");
-    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT, QEARLY>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
+    q8_linear_ws_body<NW, TPW, NBLK, WL, DUMP, Q81, CSPLIT, QEARLY, CT0>(W, X, C, M, N, ntiles, npart, relu, xq_dump, sums_dump);
 }
 
-template <int TPW, int NBLK, int WL, int NW, bool Q81, bool CSPLIT = false>
+template <int TPW, int NBLK, int WL, int NW, bool Q81, bool CSPLIT = false, bool CT0 = false>
 int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int relu,
                         void* xq_dump, int32_t* sums_dump, hipStream_t stream, int cparts = 1) {
     // Eight waves fill a CU (256 registers each): one resident work-group of 8 waves per CU, or two
@@ -1210,7 +1226,22 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
     // the next tile quantized at the start of a tile rather than two thirds in (see QEARLY in the kernel)
     constexpr bool CAN_EARLY = TPW == 3 && NBLK == 8 && NW == 8 && !CSPLIT;
     const bool early = CAN_EARLY && all_tiles / cus >= 3;
-    if constexpr (CAN_EARLY) {
+    if constexpr (CT0) {
+        // C with the features outermost: the fast instances only (a call that asks for the diagnostic buffers
+        // takes the general kernel, see try_q8_linear_ws)
+        static_assert(!CSPLIT, "no column parts for this orientation");
+        if constexpr (CAN_EARLY) {
+            fast = early ? &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81, false, true, true> : &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81, false, false, true>;
+        } else if constexpr (ws_staging_regs(NBLK, NW) == 16) {
+            fast = &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81, false, false, true>;
+        } else if constexpr (ws_staging_regs(NBLK, NW) == 32) {
+            fast = &q8_linear_ws32_kernel<NW, TPW, NBLK, WL, false, Q81, false, false, true>;
+        } else {
+            static_assert(ws_staging_regs(NBLK, NW) == 64, "no kernel for this staging size");
+            fast = &q8_linear_ws64_kernel<NW, TPW, NBLK, WL, false, Q81, false, false, true>;
+        }
+        dump = fast;
+    } else if constexpr (CAN_EARLY) {
         static_assert(ws_staging_regs(NBLK, NW) == 16, "the instance with the early quantization");
         fast = early ? &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81, CSPLIT, true> : &q8_linear_ws_kernel<NW, TPW, NBLK, WL, false, Q81, CSPLIT>;
         dump = early ? &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true, Q81, CSPLIT, true> : &q8_linear_ws_kernel<NW, TPW, NBLK, WL, true, Q81, CSPLIT>;
@@ -1252,18 +1283,26 @@ int launch_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, i
 
 // returns -1 when the shape has no weight-stationary instance
 // `csplit`: -1 never, 1 wherever there is an instance, 0 by the gate below
-template <bool Q81>
+template <bool Q81, bool CT0 = false>
 int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans,
                      int relu, int csplit, void* xq_dump, int32_t* sums_dump, hipStream_t stream) {
-    if (!c_trans) return -1;
-    if (static_cast<int64_t>(N) * M * 4 >= 0x7fff0000LL) return -1;   // the kernel addresses C with 32-bit byte offsets
+    if (!c_trans && !CT0) {
+        // C [M][N] (the weight was src[0]): instances of their own, without the diagnostic buffers
+        if (xq_dump || sums_dump) return -1;
+        return try_q8_linear_ws<Q81, true>(W, X, C, M, N, nblk, 0, relu, -1, nullptr, nullptr, stream);
+    }
+    // the kernel addresses C with 32-bit byte offsets; with the features outermost the offsets it forms reach
+    // the padded height of C plus the four rows between the two halves of a wave
+    if (static_cast<int64_t>(N) * M * 4 >= 0x7fff0000LL) return -1;
+    if (CT0 && static_cast<int64_t>(N) * (packed_tiles(M) * 32 + 4) * 4 >= 0x7fff0000LL) return -1;
     const int mct = (M + 31) / 32;
     const int tpw = (mct + 7) / 8;
+    if (CT0) csplit = -1;
     // Column parts: `tpw` work-groups of the one-column-tile-per-wave instance share each token tile.  Every
     // work-group then quantizes the whole tile for a `tpw`-th of the columns, which costs more than the shorter
     // start-up saves except where the whole-width instance is short of registers and LDS (measured, us, parts /
     // whole: 26368 x 256 -> 768  23.8 / 22.2;  10609 x 128 -> 512  6.8 / 6.3;  26368 x 128 -> 1024  20.1 / 25.1).
-    if (tpw > 1 && csplit >= 0) {
+    if (!CT0 && tpw > 1 && csplit >= 0) {
         const int cus = device_cu_count();
         const int tiles = (N + TILE_TOK - 1) / TILE_TOK;
         const bool take = csplit > 0 || (tpw == 4 && tiles >= 3 * cus);
@@ -1274,7 +1313,7 @@ int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int 
 #undef PPML_WSC
         }
     }
-#define PPML_WS(TPW, NBLK, WL, NW) return launch_q8_linear_ws<TPW, NBLK, WL, NW, Q81>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
+#define PPML_WS(TPW, NBLK, WL, NW) return launch_q8_linear_ws<TPW, NBLK, WL, NW, Q81, false, CT0>(W, X, C, M, N, relu, xq_dump, sums_dump, stream)
     // Up to four column tiles: work-groups of four waves, one column tile each and two per CU, so no
     // wave idles (with eight waves half of them would have no column tile).
     if (mct <= 4) {

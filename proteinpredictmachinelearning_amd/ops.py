@@ -452,7 +452,7 @@ _Q8_PATH_FLAGS = {"auto": 0, "weight-stationary": 4, "general": 4 | 8, "low-late
 
 
 def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = False,
-               dump: bool = False, act: str = "q8_0", path: str = "auto"):
+               dump: bool = False, act: str = "q8_0", path: str = "auto", out: torch.Tensor = None):
     """Q8_0 linear: x f32 [N,K] (rows = tokens) times quantized w [M,K] -> [N,M] (c_trans=1, the
     LinearLayer orientation) or [M,N] (c_trans=0); src/backend/CUDAKernels.cpp:740-789.
     With ``dump`` also returns the kernel's own Q8_0 blocks of x and its per-block int32 sums.
@@ -461,7 +461,8 @@ def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = Fals
     ``path`` restricts the kernel choice for a packed weight ("weight-stationary": not the low-latency kernel;
     "general": neither of the two; "low-latency-8" / "-16" / "-32": that unit size wherever an instance exists (32: K = 512 only);
     "weight-stationary-column-parts" / "-whole": that kernel with the columns shared out between work-groups
-    wherever an instance exists / never); every choice gives the same bits."""
+    wherever an instance exists / never); every choice gives the same bits.
+    ``out``: a contiguous f32 device tensor of the result's shape to write into instead of a new one."""
     if act not in ("q8_0", "q8_1"):
         raise ValueError("mul_mat_q8: act must be 'q8_0' or 'q8_1'")
     x = _dev_f32(x, "x")
@@ -469,7 +470,11 @@ def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = Fals
         raise ValueError(f"mul_mat_q8: activations {tuple(x.shape)} do not match weight K={w.K}")
     N, K = x.shape
     M = w.M
-    out = torch.empty((N, M) if c_trans else (M, N), dtype=torch.float32, device=x.device)
+    shape = (N, M) if c_trans else (M, N)
+    if out is None:
+        out = torch.empty(shape, dtype=torch.float32, device=x.device)
+    elif (tuple(out.shape) != shape or out.dtype != torch.float32 or not out.is_contiguous() or out.device != x.device):
+        raise ValueError(f"mul_mat_q8: out must be a contiguous f32 tensor of shape {shape} on {x.device}")
     lib = _lib()
     if not dump and not relu and act == "q8_0" and path == "auto":
         path = C.c_int(0)

@@ -311,6 +311,55 @@ def test_weight_layouts_and_output_orientations_agree(ops, oracle, N, K, M):
     assert (Wd.data.cpu().numpy() == wq.reshape(-1)).all()
 
 
+@pytest.mark.parametrize("key", sorted(WS_INSTANCE_SHAPES))
+def test_features_outermost_output_on_the_weight_stationary_kernel(ops, oracle, key):
+    """c_trans = 0 (the quantized weight was src[0], src/backends/CPUKernels.cpp:1120-1130: C is [M][N]) with a packed
+    weight: every weight-stationary instance has a form that stores this orientation; same bits as the oracle."""
+    N, K, M = WS_INSTANCE_SHAPES[key]
+    x, w = _inputs(5 * N + K + M, N, K, M)
+    wq = oracle.quantize_q8_0(w)
+    W = ops.Q8Weight(_dev(wq.reshape(-1)), M, K, ops.WTYPE_Q8_0).pack()
+    want = oracle.mul_mat_q8(wq, x, wtype=0, c_trans=0, fma=1)
+    assert want.shape == (M, N)
+    got = ops.mul_mat_q8(W, _dev(x), c_trans=0)
+    assert ops.last_q8_path() == "weight-stationary"
+    assert (got.cpu().numpy() == want).all()
+    # ragged token counts around the 32-token tile, and a single token
+    for n in (1, 31, 33, 65):
+        got = ops.mul_mat_q8(W, _dev(x[:n]), c_trans=0).cpu().numpy()
+        assert got.shape == (M, n) and (got == want[:, :n]).all(), n
+    # ReLU in the quantizer and the Q8_1 rule for the activations
+    got = ops.mul_mat_q8(W, _dev(x), c_trans=0, relu=True).cpu().numpy()
+    assert (got == oracle.mul_mat_q8(wq, np.maximum(x, 0.0), wtype=0, c_trans=0, fma=1)).all()
+    got = ops.mul_mat_q8(W, _dev(x), c_trans=0, act="q8_1").cpu().numpy()
+    assert (got == oracle.mul_mat_q8_act(wq, x, act=1, c_trans=0)).all()
+    # the diagnostic buffers come from the general kernel in this orientation
+    out, xq, sums = ops.mul_mat_q8(W, _dev(x), c_trans=0, dump=True)
+    assert ops.last_q8_path() == "general" and (out.cpu().numpy() == want).all()
+    # the general kernel on request
+    assert (ops.mul_mat_q8(W, _dev(x), c_trans=0, path="general").cpu().numpy() == want).all()
+    assert ops.last_q8_path() == "general"
+
+
+@pytest.mark.parametrize("N,K,M", [(26368, 256, 768), (10609, 128, 512), (10609, 512, 128), (8500, 128, 100)])
+def test_features_outermost_output_at_the_configured_sizes(ops, N, K, M):
+    """Several rounds of tiles per work-group, the leftover tiles shared by column parts, the early quantization of
+    the next tile (26368 x 256 -> 768 takes that instance) and rows of C that do not start on a line (10609
+    tokens): the transposed result of the token-outermost call, which the oracle pins at these sizes."""
+    x, w = _inputs(N + M, N, K, M)
+    W = ops.Q8Weight.from_f32(_dev(w)).pack()
+    xd = _dev(x)
+    want = ops.mul_mat_q8(W, xd, c_trans=1, path="weight-stationary")
+    got = ops.mul_mat_q8(W, xd, c_trans=0)
+    assert ops.last_q8_path() == "weight-stationary"
+    assert got.shape == (M, N) and torch.equal(got, want.T.contiguous())
+    # a buffer with sentinels around C: nothing is written outside it
+    buf = torch.full((M * N + 2048,), 7.5, device="cuda")
+    out = buf[1024:1024 + M * N].view(M, N)
+    ops.mul_mat_q8(W, xd, c_trans=0, out=out)
+    assert torch.equal(out, got) and (buf[:1024] == 7.5).all() and (buf[1024 + M * N:] == 7.5).all()
+
+
 def test_relu_fused_into_the_quantizer(ops, oracle):
     # pair-track feed-forward: linear1 -> ReLU -> linear2 (src/modules/Attention.cpp:1097-1104)
     x, w = _inputs(21, 200, 512, 128)
