@@ -110,9 +110,12 @@ __device__ __forceinline__ void split4(const v4f& v, uint2 (&out)[3], SplitGuard
     out[0] = uint2{pack(t1[0], t1[1]), pack(t1[2], t1[3])};
     out[1] = uint2{pack(t2[0], t2[1]), pack(t2[2], t2[3])};
     out[2] = uint2{pack(t3[0], t3[1]), pack(t3[2], t3[3])};
-    g.low |= t3[0] | t3[1];
-    g.low |= t3[2] | t3[3];
-#if defined(__HIP_DEVICE_COMPILE__)                     // (the host pass of a .hip file does not know the builtin)
+#if defined(__HIP_DEVICE_COMPILE__)                     // (the host pass of a .hip file knows neither the instruction nor the builtin)
+    // The ORs as volatile statements: they stay where they are written.  Left to the scheduler they all sink to the end
+    // of a thread's split, with every third part alive until then (the kernels that split in their tile loop are short
+    // of registers there: a tenth of a microsecond per launch on the small attention-logit shapes).
+    asm volatile("v_or3_b32 %0, %0, %1, %2" : "+v"(g.low) : "v"(t3[0]), "v"(t3[1]));
+    asm volatile("v_or3_b32 %0, %0, %1, %2" : "+v"(g.low) : "v"(t3[2]), "v"(t3[3]));
     const v2bf ones = __builtin_bit_cast(v2bf, 0x3f803f80u);
     g.sum3 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, out[2].x), ones, g.sum3, false);
     g.sum3 = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2bf, out[2].y), ones, g.sum3, false);

@@ -17,6 +17,7 @@
 #include "common.hpp"
 
 #include <atomic>
+#include <type_traits>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
@@ -500,6 +501,31 @@ __device__ __forceinline__ void shortk_tile_again_inline(int t, int side, int ti
                     (r / tiles_n) * side, (r % tiles_n) * side, side, tid);
 }
 
+// What a work-group of the short-K kernel does once its tile loop has ended, if a SplitGuard fired in it: bit i of
+// `fired_its` stands for the i-th tile the work-group took (bit 63 for that one and every later one), and those tiles
+// are written again by shortk_tile_again_inline.  The work-group's tile list is rebuilt from the kernel-argument
+// segment (`total_tiles` follows the GemmParams there) and its own number, exactly as the kernel builds it.
+__device__ __forceinline__ void shortk_redo_fired(uint64_t fired_its, int side, int tid) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef const __attribute__((address_space(4))) int* KernargInt;
+    KernargInt words = (KernargInt)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(words));
+    static_assert(sizeof(GemmParams) % 8 == 0, "the next kernel argument follows the structure without padding");
+    const int total_tiles = words[sizeof(GemmParams) / 4];
+#else
+    const int total_tiles = 0;
+#endif
+    constexpr int XCDS = 8;
+    const int groups = static_cast<int>(gridDim.x) / XCDS;
+    const int xcd = static_cast<int>(blockIdx.x) % XCDS, slot = static_cast<int>(blockIdx.x) / XCDS;
+    const int part = (total_tiles + XCDS - 1) / XCDS;
+    const int part_begin = xcd * part;
+    const int part_end = part_begin + part < total_tiles ? part_begin + part : total_tiles;
+    int i = 0;
+    for (int t = part_begin + slot; t < part_end; t += groups, ++i)
+        if ((fired_its >> (i < 63 ? i : 63)) & 1) shortk_tile_again_inline(t, side, tid);
+}
+
 // A thread's share of a 128 x 16 operand tile goes to the planes.  Operands with contiguous rows are
 // read one row and eight consecutive k per thread (eight loads, each contiguous across the lanes), the
 // others two rows and four consecutive k each.
@@ -708,8 +734,12 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
     static_assert(2 * OPERAND >= (TM * TM + 32) * 4, "a whole tile of C, shifted by up to a line, fits the operands' LDS");
     __shared__ __attribute__((aligned(128))) uint8_t lds_ab[2 * OPERAND];
     // "A SplitGuard fired for tile t": a thread whose guard fires writes t + 1 into the word of t's turn, and after the
-    // barrier everybody compares.  Nothing is cleared: a tile number never comes back within a work-group, and a stale
-    // or chance match only sends a tile down the plain path, whose result is right as well.
+    // barrier everybody compares.  Within a launch a tile number never comes back to a work-group.  LDS keeps what
+    // earlier kernels left there, and work-groups land on the same CUs launch after launch: a mark left behind would
+    // match the same tile number in every later launch of the shape and send that tile down the plain path each time
+    // (right results, fifteen times the time).  So a work-group that saw a mark clears both words before it ends; a
+    // word that happens to hold a tile number for any other reason costs one needless pass and is cleared by it.
+    // (Clearing them when the kernel starts takes a barrier in front of the first split: 0.3 us per launch.)
     __shared__ int lds_guard[2];
     uint8_t* const lds_a = lds_ab;
     uint8_t* const lds_b = lds_ab + OPERAND;
@@ -789,6 +819,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
     int t = part_begin + slot;
     if (t >= part_end) return;                          // whole work-group: no barrier is left behind
     int turn = 0;
+    uint64_t fired_its = 0;                             // the tiles of this loop for which a SplitGuard fired (see below)
+    int it = 0;
     Tile cur = tile_at(t);
     load_tile_regs(cur);
     const uint8_t* frag_a = lds_a + (wm + j) * SPLIT_PITCH + hh * 16;
@@ -798,20 +830,15 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
     const int c_bytes = static_cast<int>(p.M * p.c_mi * 4);
 
     while (true) {
-        split_to_lds(&lds_guard[turn], t + 1);
-        __syncthreads();
         // An operand of this tile that the split could not carry: the tile is stored as the matrix pipe leaves it all the
-        // same, and then -- once those stores have been acknowledged -- written again the reference's way.  Looking
-        // only after the stores keeps the test out of the chain load -> split -> MFMA -> store that a work-group
-        // with one tile consists of (decided ahead of the matrix work it cost half a microsecond per launch).
-        const int fired_mark = lds_guard[turn];         // requested with the fragments, looked at where the tile is stored
-        const auto again_if_fired = [&]() {
-            if (__builtin_amdgcn_readfirstlane(fired_mark) == t + 1) {                 // uniform over the work-group
-                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-                __syncthreads();
-                shortk_tile_again_inline(t, TM, tid);
-            }
-        };
+        // same, the loop only notes which of its tiles that was (a mark in the LDS word of the tile's turn, read behind
+        // the matrix work), and the work-group writes those tiles again, the reference's way, when the loop has ended.
+        // That keeps the test and the other path's code out of the chain load -> split -> MFMA -> store that a
+        // work-group with one tile consists of (decided ahead of the matrix work it cost half a microsecond per
+        // launch; with the other path inline behind the stores, a third).
+        int* const mark_word = &lds_guard[turn];
+        split_to_lds(mark_word, t + 1);
+        __syncthreads();
         turn ^= 1;
         const int t_next = t + groups;
         const bool more = t_next < part_end;
@@ -846,6 +873,8 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
                         acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][SPLIT_TERMS[q][0]], fb[tj][SPLIT_TERMS[q][1]], acc[ti][tj], 0, 0, 0);
         }
         __syncthreads();                                // the planes may be overwritten
+        if (__builtin_amdgcn_readfirstlane(*mark_word) == t + 1) fired_its |= 1ull << (it < 63 ? it : 63);   // uniform over the work-group
+        ++it;
         // ---- stores of this tile: younger than the next tile's loads
         if (C_FORM == C_FLAT) {
             // The tile's rows m0 .. m0 + rows - 1 are the floats [0, total) behind row_base.  In LDS float e of that
@@ -881,15 +910,6 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
             v4f piece[PIECES];
 #pragma unroll
             for (int i = 0; i < PIECES; ++i) piece[i] = *reinterpret_cast<const v4f*>(stage + (tid + 256 * i) * 4);
-            // (the staged forms look at the guard here, between reading the pieces and storing them: nothing is out yet)
-            if (__builtin_amdgcn_readfirstlane(fired_mark) == t + 1) {                 // uniform over the work-group
-                shortk_tile_again_inline(t, TM, tid);
-                if (!more) break;
-                __syncthreads();
-                t = t_next;
-                cur = nxt;
-                continue;
-            }
 #pragma unroll
             for (int i = 0; i < PIECES; ++i) {
                 const int q = (tid + 256 * i) * 4;
@@ -926,14 +946,6 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
             v4f piece[PIECES];
 #pragma unroll
             for (int i = 0; i < PIECES; ++i) piece[i] = *reinterpret_cast<const v4f*>(stage + (tid + 256 * i) * 4);
-            if (__builtin_amdgcn_readfirstlane(fired_mark) == t + 1) {                 // uniform over the work-group
-                shortk_tile_again_inline(t, TM, tid);
-                if (!more) break;
-                __syncthreads();
-                t = t_next;
-                cur = nxt;
-                continue;
-            }
             float* const tile_base = cur.C + static_cast<int64_t>(cur.m0) * p.c_mi + cur.n0;
 #pragma unroll
             for (int i = 0; i < PIECES; ++i) {
@@ -965,10 +977,15 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
                 }
             }
         }
-        again_if_fired();
         if (!more) break;
         t = t_next;
         cur = nxt;
+    }
+    if (fired_its != 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's stores have been acknowledged ...
+        __syncthreads();                                    // ... and so have the other waves'
+        if (tid < 2) lds_guard[tid] = 0;                    // (see lds_guard)
+        shortk_redo_fired(fired_its, TM, tid);
     }
 }
 

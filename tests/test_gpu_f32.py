@@ -352,6 +352,36 @@ def test_operands_the_split_cannot_carry_in_every_kernel_family(ops, oracle, kin
         agree(got, want, np.nan_to_num(absprod, nan=0.0, posinf=0.0))
 
 
+@pytest.mark.parametrize("planes,L,D", [(412, 103, 32), (60, 256, 32), (40, 103, 32), (30, 50, 16)])
+def test_a_launch_that_took_the_plain_path_leaves_nothing_behind_for_the_next(ops, planes, L, D):
+    """The persistent short-K kernel notes in LDS which of a work-group's tiles the split could not carry, and LDS keeps
+    its contents from launch to launch while work-groups land on the same CUs: after a launch whose every tile went
+    down the plain path, a launch of the same shape on ordinary operands must take the matrix pipe again for every
+    tile -- the same bits as before (the plain path rounds differently), not merely results within the bar."""
+    rng = np.random.default_rng(planes)
+    k = rng.standard_normal((1, planes, D, L)).astype(np.float32)
+    q = rng.standard_normal((1, planes, D, L)).astype(np.float32)
+    kd, qd = _dev(k), _dev(q)
+    before = ops.out_prod(kd, qd, scale=0.25)
+    # every plane holds an infinite operand: every tile is written again the reference's way
+    k_inf = k.copy()
+    k_inf[:, :, 0, 0] = np.inf
+    hot = ops.out_prod(_dev(k_inf), qd, scale=0.25)
+    assert bool(torch.isinf(hot).any())
+    for _ in range(3):
+        after = ops.out_prod(kd, qd, scale=0.25)
+        assert torch.equal(after.view(torch.int32), before.view(torch.int32))
+    # and the two paths do differ in their bits on such operands, so the comparison above can tell them apart:
+    # with a single infinite operand the other rows of that tile come from the plain path
+    one = k.copy()
+    one[0, 0, 0, 0] = np.inf
+    mixed = ops.out_prod(_dev(one), qd, scale=0.25)
+    same_plane = mixed[0, 0, :, 1:]                 # outputs of plane 0 that do not touch the infinite operand (row 0 of k)
+    assert not torch.equal(same_plane.view(torch.int32), before[0, 0, :, 1:].view(torch.int32))
+    torch.testing.assert_close(same_plane, before[0, 0, :, 1:], rtol=1e-4, atol=1e-5)
+    assert torch.equal(mixed[0, 1:].view(torch.int32), before[0, 1:].view(torch.int32))     # the other planes' tiles: the matrix pipe
+
+
 def test_subnormal_operands(ops, oracle):
     # Operands below 2^-126 against large ones: the products are ordinary numbers, so flushing the small
     # operand to zero would lose the whole result, and so would cutting it to bf16's grid, which stops at 2^-133

@@ -536,8 +536,8 @@ def test_fused_linear_with_q8_1_activations(ops, oracle, wname, N, K, M, c_trans
     # without the dump, and the two rules really differ
     y2 = ops.mul_mat_q8(W, _dev(x), c_trans=c_trans, act="q8_1").cpu().numpy()
     assert (y2 == want).all()
-    # a packed weight in the LinearLayer orientation gets the resident-weight kernels under this rule too
-    assert (ops.last_q8_path() != "general") == (wname == "packed" and c_trans == 1)
+    # a packed weight gets the resident-weight kernels under this rule too, in either orientation
+    assert (ops.last_q8_path() != "general") == (wname == "packed")
     if wname == "packed" and c_trans == 1:
         for fam in ("weight-stationary", "weight-stationary-column-parts", "low-latency-8", "low-latency-16", "low-latency-32"):
             if fam.startswith("low") and (not _has_low_latency_instance(K, M) or (fam.endswith("32") and K != 512)):
