@@ -1305,7 +1305,11 @@ int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int 
     if (!CT0 && tpw > 1 && csplit >= 0) {
         const int cus = device_cu_count();
         const int tiles = (N + TILE_TOK - 1) / TILE_TOK;
-        const bool take = csplit > 0 || (tpw == 4 && tiles >= 3 * cus);
+        // ... and wherever there is no whole-width instance at all (K = 128 beyond 1024 columns, K = 256 beyond 768): the
+        // parts take any width (a work-group holds 256 columns, `tpw` of them share a tile), the alternative is the
+        // general kernel, which streams the weight per tile (10609 x 256 -> 1024: 15.4 us in parts, 31.6 general)
+        const bool no_whole = (nblk == 4 && tpw > 4) || (nblk == 8 && tpw > 3);
+        const bool take = csplit > 0 || (tpw == 4 && tiles >= 3 * cus) || no_whole;
         if (take && cus >= tpw) {
 #define PPML_WSC(NBLK) return launch_q8_linear_ws<1, NBLK, 0, 8, Q81, true>(W, X, C, M, N, relu, xq_dump, sums_dump, stream, tpw)
             if (nblk == 4) PPML_WSC(4);

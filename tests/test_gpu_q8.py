@@ -311,6 +311,37 @@ def test_weight_layouts_and_output_orientations_agree(ops, oracle, N, K, M):
     assert (Wd.data.cpu().numpy() == wq.reshape(-1)).all()
 
 
+@pytest.mark.parametrize("N,K,M", [(300, 256, 1024), (2100, 256, 1024), (500, 128, 1500), (700, 256, 2048), (95, 128, 1100)])
+def test_projections_wider_than_a_work_group_holds_go_in_column_parts(ops, oracle, N, K, M):
+    """K = 256 beyond 768 output features and K = 128 beyond 1024 (the MSA feed-forward 256 -> 1024 if it is
+    quantized) have no instance that keeps the whole weight in one work-group: several work-groups share each token
+    tile, 256 columns each, whatever the token count.  Same bits as the oracle, internals included."""
+    x, w = _inputs(N + M, N, K, M)
+    wq = oracle.quantize_q8_0(w)
+    W = ops.Q8Weight(_dev(wq.reshape(-1)), M, K, ops.WTYPE_Q8_0).pack()
+    want = oracle.mul_mat_q8(wq, x, wtype=0, c_trans=1, fma=1)
+    got = ops.mul_mat_q8(W, _dev(x), c_trans=1)
+    assert ops.last_q8_path() == "weight-stationary"
+    assert (got.cpu().numpy() == want).all()
+    out, xq, sums = ops.mul_mat_q8(W, _dev(x), c_trans=1, dump=True)
+    assert ops.last_q8_path() == "weight-stationary"
+    xq_want = oracle.quantize_q8_0(x)
+    assert (out.cpu().numpy() == want).all() and (xq.cpu().numpy() == xq_want).all()
+    assert (sums.cpu().numpy() == oracle.q8_block_sums(wq, xq_want)).all()
+    got = ops.mul_mat_q8(W, _dev(x), relu=True).cpu().numpy()
+    assert (got == oracle.mul_mat_q8(wq, np.maximum(x, 0.0), wtype=0, c_trans=1, fma=1)).all()
+    got = ops.mul_mat_q8(W, _dev(x), act="q8_1").cpu().numpy()
+    assert (got == oracle.mul_mat_q8_act(wq, x, act=1, c_trans=1)).all()
+    # told not to share the columns out, the call falls to the general kernel: same bits
+    got = ops.mul_mat_q8(W, _dev(x), path="weight-stationary-whole")
+    assert ops.last_q8_path() == "general" and (got.cpu().numpy() == want).all()
+    # sentinels around C
+    buf = torch.full((N * M + 2048,), 7.5, device="cuda")
+    ops.mul_mat_q8(W, _dev(x), out=buf[1024:1024 + N * M].view(N, M))
+    assert (buf[1024:1024 + N * M].view(N, M).cpu().numpy() == want).all()
+    assert (buf[:1024] == 7.5).all() and (buf[1024 + N * M:] == 7.5).all()
+
+
 @pytest.mark.parametrize("key", sorted(WS_INSTANCE_SHAPES))
 def test_features_outermost_output_on_the_weight_stationary_kernel(ops, oracle, key):
     """c_trans = 0 (the quantized weight was src[0], src/backends/CPUKernels.cpp:1120-1130: C is [M][N]) with a packed
