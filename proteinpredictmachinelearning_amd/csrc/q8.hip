@@ -1321,12 +1321,15 @@ int try_q8_linear_ws(const void* W, const float* X, float* C, int M, int N, int 
     // Up to four column tiles: work-groups of four waves, one column tile each and two per CU, so no
     // wave idles (with eight waves half of them would have no column tile).
     if (mct <= 4) {
+        if (nblk == 2) PPML_WS(1, 2, 0, 4);
         if (nblk == 4) PPML_WS(1, 4, 0, 4);
         if (nblk == 8) PPML_WS(1, 8, 0, 4);
         if (nblk == 16) PPML_WS(1, 16, 0, 4);
     }
     // (column tiles per wave, blocks of K, column tiles whose fragments live in LDS instead of registers)
-    if (nblk == 4) {
+    if (nblk == 2) {                                   // K = 64: the 64 -> 64 and 64 -> 256 projections of the full-MSA track
+        if (tpw == 1) PPML_WS(1, 2, 0, 8);
+    } else if (nblk == 4) {
         if (tpw == 1) PPML_WS(1, 4, 0, 8);
         if (tpw == 2) PPML_WS(2, 4, 0, 8);
         if (tpw == 3) PPML_WS(3, 4, 0, 8);

@@ -190,11 +190,15 @@ SHAPES += [
     (3001, 512, 128),     # more than 2048 tokens: the library itself picks the low-latency kernel with 16-token units
     (3001, 128, 500),
     (3001, 256, 250),
+    (300, 64, 64),        # (1, 2) four waves: K = 64, the 64 -> 64 projections of the full-MSA track
+    (300, 64, 256),       # (1, 2) eight waves: its feed-forward 64 -> 256
+    (9000, 64, 64),       # likewise with several token tiles per work-group
 ]
 
 # (column tiles of 32 outputs) -> instance: up to 4 tiles the four-wave kernels, beyond that ceil(tiles / 8) per wave
 WS_INSTANCE_SHAPES = {
     # (TPW, NBLK, waves): (N, K, M)
+    (1, 2, 4): (300, 64, 64), (1, 2, 8): (300, 64, 256),
     (1, 4, 4): (300, 128, 100), (1, 8, 4): (300, 256, 100), (1, 16, 4): (200, 512, 128),
     (1, 4, 8): (200, 128, 200), (2, 4, 8): (300, 128, 512), (3, 4, 8): (150, 128, 700), (4, 4, 8): (70, 128, 800),
     (1, 8, 8): (408, 256, 256), (2, 8, 8): (300, 256, 400), (3, 8, 8): (1000, 256, 768),
@@ -252,7 +256,7 @@ def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packe
 def _has_resident_weight_instance(K, M):
     tiles, nblk = (M + 31) // 32, K // 32
     tpw = (tiles + 7) // 8
-    return K % 32 == 0 and nblk in (4, 8, 16) and (tiles <= 4 or tpw <= {4: 4, 8: 3, 16: 1}[nblk])
+    return K % 32 == 0 and nblk in (2, 4, 8, 16) and (tiles <= 4 or tpw <= {2: 1, 4: 4, 8: 3, 16: 1}[nblk])
 
 
 _FAMILY_PATH = {"general": "general", "weight-stationary": "weight-stationary", "weight-stationary-whole": "weight-stationary",
@@ -283,7 +287,7 @@ def test_every_weight_stationary_instance_has_a_shape_in_the_suite():
         assert (waves == 4) == (tiles <= 4)
         assert tpw == (1 if waves == 4 else (tiles + 7) // 8)
         assert (N, K, M) in SHAPES, (N, K, M)
-    assert len(WS_INSTANCE_SHAPES) == 11
+    assert len(WS_INSTANCE_SHAPES) == 13
 
 
 @pytest.mark.parametrize("N,K,M", [(408, 256, 256), (100, 96, 100), (70, 128, 800)])
