@@ -151,6 +151,17 @@ int out_prod_hip(const float *src0, const float *src1, float *dst,
                  int64_t ne10, int64_t ne11, int64_t ne12, int64_t ne13,
                  int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3,
                  ppml_hip_stream_t stream);
+/* out_prod_hip of the {1,0,2,3} permutations of both operands, without the permutation copies -- the second
+ * contraction of the attention chain as the reference builds it, out_prod(permute(attn), permute(V))
+ * (src/modules/Attention.cpp:277-281; its permute is a copy, src/core/ComputeGraphHelper.cpp:700-729):
+ * dst[i0,i1,i2,i3] = sum_k src0[k,i0,i2/(ne2/ne02),i3/(ne3/ne03)] * src1[k,i1,i2,i3], dimensions of the operands AS
+ * THEY LIE (ne00 = ne10 = the contracted length, ne0 = ne01, ne1 = ne11).  Same kernel, same products in the same
+ * order as out_prod_hip on the permuted copies: same bits.  No counterpart among the reference's launchers. */
+int out_prod_tt_hip(const float *src0, const float *src1, float *dst,
+                    int64_t ne00, int64_t ne01, int64_t ne02, int64_t ne03,
+                    int64_t ne10, int64_t ne11, int64_t ne12, int64_t ne13,
+                    int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3,
+                    ppml_hip_stream_t stream);
 /* out_prod followed by the OP_SCALE node of the attention path in one pass
  * (src/modules/Attention.cpp:264-270): dst = scale * out_prod(src0, src1). */
 int out_prod_scaled_hip(const float *src0, const float *src1, float *dst,
@@ -314,6 +325,14 @@ int bcast_elemwise_hip(const float *a, const float *b, float *dst, int64_t n, in
  * The sum is formed across a wavefront, not d ascending: results agree with the reference's to rounding
  * (a few units in the last place), not bit for bit.  returns 0 ok, 1 bad arguments, 6 launch error. */
 int softmax_hip(const float *input, float *output, int M, int N, ppml_hip_stream_t stream);
+/* softmax_hip on input + bias, without the sum going to memory: the OP_ADD node in front of the attention softmax
+ * (src/modules/Attention.cpp:271-276) folded into it.  Row r of the input is added to row r % bias_rows of `bias`
+ * ([bias_rows][N]; bias_rows must divide M: the flat-modulo rule of bcast_elemwise_hip for an operand of whole
+ * rows), one binary32 addition per element exactly as the node makes it, so the result has the bits of
+ * softmax_hip(bcast_elemwise_hip(input, bias, add)).  It has no counterpart among the reference's launchers (its
+ * graphs run the two nodes).  returns 0 ok, 1 bad arguments, 6 launch error. */
+int softmax_add_hip(const float *input, const float *bias, float *output, int M, int N, int bias_rows,
+                    ppml_hip_stream_t stream);
 
 /* ---- observability (include/ppml/MulMatStats.h:39-169, src/cuda/CUDAKernels.cu:1693-1732) ------ */
 /* MUL_MAT statistics: per (path, M, K, N) the number of launcher calls and the device time of their

@@ -76,6 +76,14 @@ void ppml_hip_backend_set_fuse_attention_bridges(ppml_hip_backend *b, int on);
 void ppml_hip_backend_set_fuse_relu_into_q8(ppml_hip_backend *b, int on);
 void ppml_hip_backend_set_fuse_scale_into_out_prod(ppml_hip_backend *b, int on);
 void ppml_hip_backend_set_fuse_attention_chain(ppml_hip_backend *b, int on);
+/*   add_into_soft_max (default 1): an OP_ADD read only by an OP_SOFT_MAX (first operand of the result's size, second
+ *     operand whole rows of the softmax: the attention bias, src/modules/Attention.cpp:271-276) is added on the
+ *     softmax kernel's way in; same bits.
+ *   permutes_into_out_prod (default 1): an OP_OUT_PROD whose operands are both {1,0,2,3} permutations nobody else
+ *     reads (src/modules/Attention.cpp:277-281) contracts the unpermuted tensors over their innermost dimension;
+ *     same bits, two copies less. */
+void ppml_hip_backend_set_fuse_add_into_soft_max(ppml_hip_backend *b, int on);
+void ppml_hip_backend_set_fuse_permutes_into_out_prod(ppml_hip_backend *b, int on);
 /* how many nodes the last graph_compute folded into a neighbour and did not execute */
 int ppml_hip_backend_nodes_fused_away(const ppml_hip_backend *b);
 /* Matrix pipe of this backend's f32 contractions for the length of each graph_compute: 0 = bf16 pipe through

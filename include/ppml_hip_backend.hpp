@@ -174,6 +174,17 @@ public:
     bool fuse_relu_into_q8() const { return fuse_relu_into_q8_; }
     void set_fuse_scale_into_out_prod(bool v) { fuse_scale_into_out_prod_ = v; }
     bool fuse_scale_into_out_prod() const { return fuse_scale_into_out_prod_; }
+    // Two more of the same kind, ON by default, same bits as the nodes run one by one; together with `scale` they turn
+    // the reference's default attention chain (src/modules/Attention.cpp:264-281) from seven launches into three:
+    //   add      -- an OP_ADD read only by an OP_SOFT_MAX, whose first operand has the result's size and whose second
+    //               is whole rows of the softmax (the attention bias), is added on the softmax kernel's way in;
+    //   permutes -- an OP_OUT_PROD both of whose operands are {1,0,2,3} permutations nobody else reads contracts
+    //               the unpermuted tensors over their innermost dimension instead (the permutation is a copy in the
+    //               reference, src/core/ComputeGraphHelper.cpp:700-729).
+    void set_fuse_add_into_soft_max(bool v) { fuse_add_into_soft_max_ = v; }
+    bool fuse_add_into_soft_max() const { return fuse_add_into_soft_max_; }
+    void set_fuse_permutes_into_out_prod(bool v) { fuse_permutes_into_out_prod_ = v; }
+    bool fuse_permutes_into_out_prod() const { return fuse_permutes_into_out_prod_; }
     // Off by default.  On: the reference's default attention chain (src/modules/Attention.cpp:264-281)
     //   out_prod(K, Q) -> scale -> [add bias] -> softmax -> permute{1,0,2,3} ; permute{1,0,2,3}(V) -> out_prod
     // whose intermediates have no other reader runs as one fused attention launch on the graph's own layouts
@@ -227,11 +238,15 @@ private:
     bool fuse_relu_into_q8_ = true;
     bool fuse_scale_into_out_prod_ = true;
     bool fuse_attention_chain_ = false;
+    bool fuse_add_into_soft_max_ = true;
+    bool fuse_permutes_into_out_prod_ = true;
     size_t nodes_fused_away_ = 0;
     int attn_layout_ = 0;                                // layout bits of the attention node being dispatched
     bool relu_in_quantizer_ = false;                     // the matmul being dispatched applies a fused-away ReLU
     float out_prod_alpha_ = 1.0f;                        // scale of a fused-away OP_SCALE behind the out_prod being dispatched
     bool out_prod_scaled_ = false;
+    bool out_prod_transposed_ = false;                   // the out_prod being dispatched reads the sources of two fused-away permutations
+    const Tensor* soft_max_bias_ = nullptr;              // second operand of a fused-away OP_ADD in front of the softmax being dispatched
     std::string error_;
     std::vector<std::unique_ptr<Buffer>> owned_;         // node outputs allocated here, packed weights
 };

@@ -119,6 +119,14 @@ class Backend:
     def set_fuse_scale_into_out_prod(self, on: bool) -> None:
         self._lib.ppml_hip_backend_set_fuse_scale_into_out_prod(self.handle, int(on))
 
+    def set_fuse_add_into_soft_max(self, on: bool) -> None:
+        """On by default: an OP_ADD read only by an OP_SOFT_MAX (the attention bias) is added inside the softmax kernel."""
+        self._lib.ppml_hip_backend_set_fuse_add_into_soft_max(self.handle, int(on))
+
+    def set_fuse_permutes_into_out_prod(self, on: bool) -> None:
+        """On by default: an OP_OUT_PROD of two {1,0,2,3} permutations nobody else reads contracts the unpermuted tensors."""
+        self._lib.ppml_hip_backend_set_fuse_permutes_into_out_prod(self.handle, int(on))
+
     def set_fuse_attention_chain(self, on: bool) -> None:
         self._lib.ppml_hip_backend_set_fuse_attention_chain(self.handle, int(on))
 

@@ -32,6 +32,7 @@ SIGNATURES = {
     "mul_mat_q8_ex_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "out_prod_hip": (_i, [_vp, _vp, _vp] + [_i64] * 12 + [_vp]),
     "out_prod_scaled_hip": (_i, [_vp, _vp, _vp] + [_i64] * 12 + [_f, _vp]),
+    "out_prod_tt_hip": (_i, [_vp, _vp, _vp] + [_i64] * 12 + [_vp]),
     "outer_prod_mean_hip": (_i, [_vp, _vp, _vp] + [_i64] * 4 + [_f, _vp]),
     "outer_prod_mean_back_hip": (_i, [_vp] * 5 + [_i64] * 4 + [_f, _vp]),
     "outer_product_mean_value_hip": (_i, [_vp, _vp, _vp] + [_i64] * 4 + [_vp]),
@@ -48,6 +49,7 @@ SIGNATURES = {
     "unary_hip": (_i, [_vp, _vp, _i64, _i, _vp]),
     "bcast_elemwise_hip": (_i, [_vp, _vp, _vp, _i64, _i64, _i64, _i, _vp]),
     "softmax_hip": (_i, [_vp, _vp, _i, _i, _vp]),
+    "softmax_add_hip": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "ppml_hip_mulmat_stats": (_i, [C.POINTER(_i64), _i]),
     "ppml_hip_mulmat_stats_enable": (_i, [_i]),
     "ppml_hip_mulmat_stats_rows": (_i, [_vp, _i]),
@@ -89,6 +91,8 @@ BACKEND_SIGNATURES = {
     "ppml_hip_backend_set_fuse_attention_bridges": (None, [_vp, _i]),
     "ppml_hip_backend_set_fuse_relu_into_q8": (None, [_vp, _i]),
     "ppml_hip_backend_set_fuse_scale_into_out_prod": (None, [_vp, _i]),
+    "ppml_hip_backend_set_fuse_add_into_soft_max": (None, [_vp, _i]),
+    "ppml_hip_backend_set_fuse_permutes_into_out_prod": (None, [_vp, _i]),
     "ppml_hip_backend_set_fuse_attention_chain": (None, [_vp, _i]),
     "ppml_hip_backend_nodes_fused_away": (_i, [_vp]),
     "ppml_hip_backend_set_f32_arithmetic": (None, [_vp, _i]),

@@ -394,6 +394,15 @@ Status HipBackend::kernel_out_prod(Tensor* node) {
     const Tensor* b = node->src[1];
     if (!a || !b) return fail(Status::NOT_SUPPORTED, "out_prod: missing source");
     // the reference clears dst first and accumulates; the launcher overwrites dst instead
+    if (out_prod_transposed_) {
+        // a, b are the sources of the two folded permutations: [k, i0, ..] and [k, i1, ..]
+        const int rc = out_prod_tt_hip(static_cast<const float*>(a->data), static_cast<const float*>(b->data), static_cast<float*>(node->data),
+                                       a->dims[0], a->dims[1], dim_or_1(a, 2), dim_or_1(a, 3),
+                                       b->dims[0], b->dims[1], dim_or_1(b, 2), dim_or_1(b, 3),
+                                       node->dims[0], node->dims[1], dim_or_1(node, 2), dim_or_1(node, 3), nullptr);
+        if (rc != 0) return fail(status_of_rc(rc), std::string("out_prod: ") + ppml_hip_last_error());
+        return Status::SUCCESS;
+    }
     const int rc = out_prod_scaled_ ? out_prod_scaled_hip(static_cast<const float*>(a->data), static_cast<const float*>(b->data),
                                 static_cast<float*>(node->data),
                                 a->dims[0], a->dims[1], dim_or_1(a, 2), dim_or_1(a, 3),
@@ -631,7 +640,16 @@ Status HipBackend::kernel_soft_max(Tensor* node) {
     const int64_t N = node->dims[0], M = N > 0 ? node->numel() / N : 0;
     if (a->numel() != node->numel() || N <= 0 || N > 0x7fffffffLL || M > 0x7fffffffLL)
         return fail(Status::NOT_SUPPORTED, "soft_max: sizes outside what one launch takes");
-    const int rc = softmax_hip(static_cast<const float*>(a->data), static_cast<float*>(node->data), static_cast<int>(M), static_cast<int>(N), nullptr);
+    int rc;
+    if (soft_max_bias_) {
+        const Tensor* bias = soft_max_bias_;
+        if (!bias->data || bias->numel() <= 0 || bias->numel() % N != 0 || M % (bias->numel() / N) != 0)
+            return fail(Status::NOT_SUPPORTED, "soft_max: the folded bias is not whole rows of the softmax");
+        rc = softmax_add_hip(static_cast<const float*>(a->data), static_cast<const float*>(bias->data), static_cast<float*>(node->data),
+                             static_cast<int>(M), static_cast<int>(N), static_cast<int>(bias->numel() / N), nullptr);
+    } else {
+        rc = softmax_hip(static_cast<const float*>(a->data), static_cast<float*>(node->data), static_cast<int>(M), static_cast<int>(N), nullptr);
+    }
     if (rc != 0) return fail(status_of_rc(rc), std::string("soft_max: ") + ppml_hip_last_error());
     return Status::SUCCESS;
 }
@@ -677,6 +695,8 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         int relu_slot = -1;                 // quantized mul_mat: activation slot whose chain ends in a skipped ReLU
         Tensor* relu = nullptr;
         Tensor* out_prod = nullptr;         // OP_SCALE node that runs as the (skipped) out_prod it reads, scaled
+        Tensor* added = nullptr;            // OP_SOFT_MAX node that adds the second operand of this (skipped) OP_ADD on its way in
+        bool transposed = false;            // OP_OUT_PROD that reads the sources of its two (skipped) {1,0,2,3} permutations
         bool chain = false;                 // out_prod(attn_t, V_t) that runs as the whole attention chain
         Tensor *q = nullptr, *k = nullptr, *v = nullptr, *bias = nullptr;
         float scale = 1.0f;
@@ -684,7 +704,8 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
     std::unordered_map<const Tensor*, Plan> plans;
     std::unordered_set<const Tensor*> skipped;
     nodes_fused_away_ = 0;
-    if (fuse_attention_bridges_ || fuse_relu_into_q8_ || fuse_scale_into_out_prod_ || fuse_attention_chain_) {
+    if (fuse_attention_bridges_ || fuse_relu_into_q8_ || fuse_scale_into_out_prod_ || fuse_attention_chain_ ||
+        fuse_add_into_soft_max_ || fuse_permutes_into_out_prod_) {
         std::unordered_map<const Tensor*, int> uses, position;
         std::unordered_map<const Tensor*, Tensor*> single_user;
         int pos = 0;
@@ -813,6 +834,39 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
                 skipped.insert(p);
             }
         }
+
+        // (5) the bias add in front of the attention softmax (src/modules/Attention.cpp:271-276)
+        if (fuse_add_into_soft_max_) {
+            for (Tensor* n : *graph) {
+                if (!n || n->op != OP_SOFT_MAX || skipped.count(n) || !node_supported(n)) continue;
+                Tensor* x = n->src[0];
+                if (!x || x->op != OP_ADD || !node_supported(x) || !private_to(x, n) || x->numel() != n->numel()) continue;
+                const Tensor* full = x->src[0];
+                const Tensor* bias = x->src[1];
+                const int64_t row = n->dims[0];
+                if (!full || !bias || full->type != TENSOR_TYPE_F32 || bias->type != TENSOR_TYPE_F32 || full->numel() != x->numel() ||
+                    row <= 0 || bias->numel() <= 0 || bias->numel() % row != 0 || (x->numel() / row) % (bias->numel() / row) != 0) continue;
+                plans[n].added = x;
+                skipped.insert(x);
+            }
+        }
+
+        // (6) the two permutation copies in front of the second contraction of the attention chain
+        // (src/modules/Attention.cpp:277-281)
+        if (fuse_permutes_into_out_prod_) {
+            for (Tensor* n : *graph) {
+                if (!n || n->op != OP_OUT_PROD || n->type != TENSOR_TYPE_F32 || n->ndim != 4 || skipped.count(n) || !node_supported(n)) continue;
+                const auto planned = plans.find(n);
+                if (planned != plans.end() && planned->second.chain) continue;
+                Tensor* p0 = n->src[0];
+                Tensor* p1 = n->src[1];
+                if (p0 == p1 || !is_bridge(p0) || !is_bridge(p1) || !private_to(p0, n) || !private_to(p1, n)) continue;
+                if (p0->src[0]->numel() != p0->numel() || p1->src[0]->numel() != p1->numel()) continue;
+                plans[n].transposed = true;
+                skipped.insert(p0);
+                skipped.insert(p1);
+            }
+        }
         nodes_fused_away_ = skipped.size();
     }
 
@@ -844,6 +898,8 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         attn_layout_ = 0;
         relu_in_quantizer_ = false;
         out_prod_scaled_ = false;
+        out_prod_transposed_ = false;
+        soft_max_bias_ = nullptr;
         const auto plan = plans.find(node);
         if (plan != plans.end()) {
             const Plan& pl = plan->second;
@@ -877,6 +933,17 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
                 for (int s = 0; s < 10; ++s) rewired.src[s] = pl.out_prod->src[s];
                 out_prod_scaled_ = true;
                 out_prod_alpha_ = node->param_f32(0);
+            }
+            if (pl.added) {
+                resolve_views(pl.added);                // binds the add's own sources if they are views
+                rewired.src[0] = pl.added->src[0];
+                rewired.src[1] = pl.added->src[1];      // (covered and checked with the other sources below)
+                soft_max_bias_ = pl.added->src[1];
+            }
+            if (pl.transposed) {
+                rewired.src[0] = node->src[0]->src[0];
+                rewired.src[1] = node->src[1]->src[0];
+                out_prod_transposed_ = true;
             }
             if (pl.chain) {
                 // src/core/ComputeGraphHelper.cpp:450-484: Q, K, V, bias in src 0..3; scale, causal, eps, Br, Bc
@@ -936,6 +1003,8 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         attn_layout_ = 0;
         relu_in_quantizer_ = false;
         out_prod_scaled_ = false;
+        out_prod_transposed_ = false;
+        soft_max_bias_ = nullptr;
         if (st != Status::SUCCESS) return st;
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess)
@@ -1086,6 +1155,12 @@ void ppml_hip_backend_set_fuse_relu_into_q8(ppml_hip_backend* b, int on) {
 }
 void ppml_hip_backend_set_fuse_scale_into_out_prod(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_fuse_scale_into_out_prod(on != 0);
+}
+void ppml_hip_backend_set_fuse_add_into_soft_max(ppml_hip_backend* b, int on) {
+    if (b) b->impl.set_fuse_add_into_soft_max(on != 0);
+}
+void ppml_hip_backend_set_fuse_permutes_into_out_prod(ppml_hip_backend* b, int on) {
+    if (b) b->impl.set_fuse_permutes_into_out_prod(on != 0);
 }
 void ppml_hip_backend_set_fuse_attention_chain(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_fuse_attention_chain(on != 0);

@@ -107,12 +107,17 @@ __device__ __forceinline__ float wave_sum(float v) {
 // it is read once and written once.  PIECES 16-byte pieces (VEC) or single elements per lane.  The reference starts
 // its maximum from the first element and moves it with `>` only, so a NaN there stays the maximum; elsewhere a NaN
 // is skipped by the maximum and reaches every output through the sum.  Both follow here from fmaxf plus one test.
-template <int PIECES, bool VEC>
-__global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t rows, int n) {
+// HAS_BIAS: the OP_ADD node in front of the softmax folded in (src/modules/Attention.cpp:271-276: scores + bias, then
+// softmax): row r of the input plus row r % bias_rows of `bias`, one binary32 addition per element exactly as the node
+// would have made it, on the way into the registers -- the sum never goes to memory.
+template <int PIECES, bool VEC, bool HAS_BIAS>
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int64_t rows, int n,
+                                                           const float* __restrict__ bias, int64_t bias_rows) {
     const int lane = threadIdx.x & 63;
     const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
     const float* x = in + row * n;
+    const float* b = HAS_BIAS ? bias + (row % bias_rows) * n : nullptr;
     float* y = out + row * n;
     constexpr int W = VEC ? 4 : 1;
     float v[PIECES * W];
@@ -122,11 +127,20 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restri
         const int at = (lane + 64 * p) * W;
         if (VEC) {
             v4f t = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-            if (at < n) t = *reinterpret_cast<const v4f*>(x + at);
+            if (at < n) {
+                // (with a bias the inputs need only be 4-byte aligned: see launch_softmax)
+                if (HAS_BIAS) t = *reinterpret_cast<const v4f_u*>(x + at);
+                else t = *reinterpret_cast<const v4f*>(x + at);
+                if (HAS_BIAS) {
+                    const v4f tb = *reinterpret_cast<const v4f_u*>(b + at);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) t[c] = t[c] + tb[c];
+                }
+            }
 #pragma unroll
             for (int c = 0; c < 4; ++c) v[p * 4 + c] = t[c];
         } else {
-            v[p] = at < n ? x[at] : -INFINITY;
+            v[p] = at < n ? (HAS_BIAS ? x[at] + b[at] : x[at]) : -INFINITY;
         }
 #pragma unroll
         for (int c = 0; c < W; ++c) mx = fmaxf(mx, v[p * W + c]);
@@ -164,28 +178,33 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restri
 
 // Rows too long for a wave's registers: one work-group per row, three passes over memory (the second and third
 // come from L2).
-__global__ __launch_bounds__(256) void softmax_long_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int n) {
+template <bool HAS_BIAS>
+__global__ __launch_bounds__(256) void softmax_long_rows_kernel(const float* __restrict__ in, float* __restrict__ out, int n,
+                                                                const float* __restrict__ bias, int64_t bias_rows) {
     __shared__ float part[4];
-    const float* x = in + static_cast<int64_t>(blockIdx.x) * n;
+    const float* xin = in + static_cast<int64_t>(blockIdx.x) * n;
+    const float* b = HAS_BIAS ? bias + (static_cast<int64_t>(blockIdx.x) % bias_rows) * n : nullptr;
+    // (the same addition in each of the three passes gives the same value each time)
+    const auto x = [&](int i) { return HAS_BIAS ? xin[i] + b[i] : xin[i]; };
     float* y = out + static_cast<int64_t>(blockIdx.x) * n;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     float mx = -INFINITY;
-    for (int i = threadIdx.x; i < n; i += 256) mx = fmaxf(mx, x[i]);
+    for (int i = threadIdx.x; i < n; i += 256) mx = fmaxf(mx, x(i));
     mx = wave_max(mx);
     if (lane == 0) part[wave] = mx;
     __syncthreads();
     mx = fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]));
-    const float first = x[0];
+    const float first = x(0);
     if (first != first) mx = first;
     __syncthreads();
     float sum = 0.0f;
-    for (int i = threadIdx.x; i < n; i += 256) sum += expf(x[i] - mx);
+    for (int i = threadIdx.x; i < n; i += 256) sum += expf(x(i) - mx);
     sum = wave_sum(sum);
     if (lane == 0) part[wave] = sum;
     __syncthreads();
     sum = (part[0] + part[1]) + (part[2] + part[3]);
     const float inv = 1.0f / (sum + 1e-9f);
-    for (int i = threadIdx.x; i < n; i += 256) y[i] = expf(x[i] - mx) * inv;
+    for (int i = threadIdx.x; i < n; i += 256) y[i] = expf(x(i) - mx) * inv;
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -218,15 +237,35 @@ int launch_bcast(const float* a, const float* b, float* dst, int64_t n, int64_t 
     return check_launch("bcast_elemwise_kernel");
 }
 
-template <bool VEC>
-void launch_softmax_rows(int pieces, dim3 grid, hipStream_t stream, const float* in, float* out, int64_t rows, int n) {
+template <bool VEC, bool HAS_BIAS>
+void launch_softmax_rows(int pieces, dim3 grid, hipStream_t stream, const float* in, float* out, int64_t rows, int n,
+                         const float* bias, int64_t bias_rows) {
     const dim3 block(256);
     switch (pieces) {
-        case 1: hipLaunchKernelGGL((softmax_rows_kernel<1, VEC>), grid, block, 0, stream, in, out, rows, n); break;
-        case 2: hipLaunchKernelGGL((softmax_rows_kernel<2, VEC>), grid, block, 0, stream, in, out, rows, n); break;
-        case 3: case 4: hipLaunchKernelGGL((softmax_rows_kernel<4, VEC>), grid, block, 0, stream, in, out, rows, n); break;
-        default: hipLaunchKernelGGL((softmax_rows_kernel<8, VEC>), grid, block, 0, stream, in, out, rows, n); break;
+        case 1: hipLaunchKernelGGL((softmax_rows_kernel<1, VEC, HAS_BIAS>), grid, block, 0, stream, in, out, rows, n, bias, bias_rows); break;
+        case 2: hipLaunchKernelGGL((softmax_rows_kernel<2, VEC, HAS_BIAS>), grid, block, 0, stream, in, out, rows, n, bias, bias_rows); break;
+        case 3: case 4: hipLaunchKernelGGL((softmax_rows_kernel<4, VEC, HAS_BIAS>), grid, block, 0, stream, in, out, rows, n, bias, bias_rows); break;
+        default: hipLaunchKernelGGL((softmax_rows_kernel<8, VEC, HAS_BIAS>), grid, block, 0, stream, in, out, rows, n, bias, bias_rows); break;
     }
+}
+
+template <bool HAS_BIAS>
+int launch_softmax(const char* name, const float* input, const float* bias, float* output, int M, int N, int64_t bias_rows, hipStream_t s) {
+    // Which lane holds which element decides the order of the additions in the row's sum, i.e. the last bits of the
+    // result.  The folded form has to make the choice the softmax node would have made on the sum the add node would
+    // have written -- a tensor of its own, aligned like the output -- so it goes by the output alone and reads its two
+    // inputs sixteen bytes at a time wherever they lie.
+    const bool vec = (N % 4 == 0) && aligned16(output) && (HAS_BIAS || aligned16(input));
+    const int per_lane = vec ? 4 : 1;
+    const int pieces = (N + 64 * per_lane - 1) / (64 * per_lane);
+    if (pieces <= 8) {
+        const dim3 grid(static_cast<unsigned>((static_cast<int64_t>(M) + 3) / 4));
+        if (vec) launch_softmax_rows<true, HAS_BIAS>(pieces, grid, s, input, output, M, N, bias, bias_rows);
+        else launch_softmax_rows<false, HAS_BIAS>(pieces, grid, s, input, output, M, N, bias, bias_rows);
+    } else {
+        hipLaunchKernelGGL(softmax_long_rows_kernel<HAS_BIAS>, dim3(static_cast<unsigned>(M)), dim3(256), 0, s, input, output, N, bias, bias_rows);
+    }
+    return check_launch(name);
 }
 
 }  // namespace
@@ -268,16 +307,15 @@ extern "C" int bcast_elemwise_hip(const float* a, const float* b, float* dst, in
 extern "C" int softmax_hip(const float* input, float* output, int M, int N, ppml_hip_stream_t stream) {
     if (!input || !output || M < 0 || N <= 0) { set_error("softmax_hip: bad arguments (M = %d, N = %d)", M, N); return RC_BAD_ARGS; }
     if (M == 0) return RC_OK;
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    const bool vec = (N % 4 == 0) && aligned16(input) && aligned16(output);
-    const int per_lane = vec ? 4 : 1;
-    const int pieces = (N + 64 * per_lane - 1) / (64 * per_lane);
-    if (pieces <= 8) {
-        const dim3 grid(static_cast<unsigned>((static_cast<int64_t>(M) + 3) / 4));
-        if (vec) launch_softmax_rows<true>(pieces, grid, s, input, output, M, N);
-        else launch_softmax_rows<false>(pieces, grid, s, input, output, M, N);
-    } else {
-        hipLaunchKernelGGL(softmax_long_rows_kernel, dim3(static_cast<unsigned>(M)), dim3(256), 0, s, input, output, N);
+    return launch_softmax<false>("softmax_kernel", input, nullptr, output, M, N, 1, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int softmax_add_hip(const float* input, const float* bias, float* output, int M, int N, int bias_rows,
+                               ppml_hip_stream_t stream) {
+    if (!input || !bias || !output || M < 0 || N <= 0 || bias_rows <= 0 || (M % bias_rows) != 0) {
+        set_error("softmax_add_hip: bad arguments (M = %d, N = %d, bias_rows = %d)", M, N, bias_rows);
+        return RC_BAD_ARGS;
     }
-    return check_launch("softmax_kernel");
+    if (M == 0) return RC_OK;
+    return launch_softmax<true>("softmax_add_kernel", input, bias, output, M, N, bias_rows, static_cast<hipStream_t>(stream));
 }

@@ -1677,6 +1677,41 @@ extern "C" int out_prod_hip(const float* src0, const float* src1, float* dst,
                                ne0, ne1, ne2, ne3, 1.0f, stream);
 }
 
+// out_prod of the two {1,0,2,3} permutations of src0 and src1, without the permutations: the contraction runs
+// over the INNERMOST dimension of both operands as they lie,
+//     dst[i0, i1, i2, i3] = sum_k src0[k, i0, i2 / (ne2 / ne02), i3 / (ne3 / ne03)] * src1[k, i1, i2, i3],
+// which is what the second contraction of the attention chain asks for (src/modules/Attention.cpp:277-281:
+// out_prod(permute(attn), permute(V)), attn [Lk, Lq, h, B], V [L, D, h, B]).  The same kernel as out_prod_hip with
+// the operands read k-contiguous instead of row-contiguous: same products, same order, same bits.
+extern "C" int out_prod_tt_hip(const float* src0, const float* src1, float* dst,
+                               int64_t ne00, int64_t ne01, int64_t ne02, int64_t ne03,
+                               int64_t ne10, int64_t ne11, int64_t ne12, int64_t ne13,
+                               int64_t ne0, int64_t ne1, int64_t ne2, int64_t ne3,
+                               ppml_hip_stream_t stream) {
+    if (!src0 || !src1 || !dst) { set_error("out_prod_tt_hip: null pointer"); return RC_BAD_ARGS; }
+    const bool pos = ne00 > 0 && ne01 > 0 && ne02 > 0 && ne03 > 0 && ne10 > 0 && ne11 > 0 && ne12 > 0 && ne13 > 0;
+    if (!pos || ne00 != ne10 || ne0 != ne01 || ne1 != ne11 || ne2 != ne12 || ne3 != ne13 ||
+        ne2 % ne02 != 0 || ne3 % ne03 != 0 || ne0 > 0x7fffffff || ne1 > 0x7fffffff || ne00 > 0x7fffffff) {
+        set_error("out_prod_tt_hip: shape mismatch src0[%lld,%lld,%lld,%lld] src1[%lld,%lld,%lld,%lld] dst[%lld,%lld,%lld,%lld]",
+                  (long long)ne00, (long long)ne01, (long long)ne02, (long long)ne03,
+                  (long long)ne10, (long long)ne11, (long long)ne12, (long long)ne13,
+                  (long long)ne0, (long long)ne1, (long long)ne2, (long long)ne3);
+        return RC_BAD_ARGS;
+    }
+    StatsScope stat("hip/out_prod", ne1, ne00, ne0, static_cast<hipStream_t>(stream));
+    GemmParams p = plain_params();
+    p.A = src1; p.B = src0; p.C = dst;                 // rows = i1 (src1), cols = i0 (src0)
+    p.M = static_cast<int>(ne1); p.N = static_cast<int>(ne0); p.K = static_cast<int>(ne00);
+    p.a_rs = ne10; p.a_ks = 1; p.b_rs = ne00; p.b_ks = 1;
+    p.np2 = static_cast<int>(ne2); p.np3 = static_cast<int>(ne3);
+    p.a_p2 = ne10 * ne11; p.a_p3 = ne10 * ne11 * ne12;
+    p.b_p2 = ne00 * ne01; p.b_p3 = ne00 * ne01 * ne02;
+    p.c_p2 = ne0 * ne1;   p.c_p3 = ne0 * ne1 * ne2;
+    p.b_div2 = static_cast<int>(ne2 / ne02); p.b_div3 = static_cast<int>(ne3 / ne03);
+    p.c_mi = ne0; p.c_ni = 1;
+    return launch_gemm(p, static_cast<hipStream_t>(stream), "out_prod_tt_hip");
+}
+
 extern "C" int outer_prod_mean_hip(const float* left, const float* right, float* dst,
                                    int64_t D, int64_t L, int64_t N, int64_t B, float inv_N,
                                    ppml_hip_stream_t stream) {

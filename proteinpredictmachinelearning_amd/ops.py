@@ -363,15 +363,44 @@ def bcast_elemwise(a: torch.Tensor, b: torch.Tensor, op: str = "add") -> torch.T
     return out
 
 
-def softmax(x: torch.Tensor) -> torch.Tensor:
+def softmax(x: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
     """The reference's softmax() node over dims[0], the LAST torch dimension (src/core/ComputeGraphHelper.cpp:420-425;
-    kernel src/backend/CPUKernels.cpp:1446-1467, incl. its 1 / (sum + 1e-9))."""
+    kernel src/backend/CPUKernels.cpp:1446-1467, incl. its 1 / (sum + 1e-9)).  With ``bias`` (whole rows of x's row
+    length, a count that divides x's): softmax(x + bias) with the add node in front folded in, the same bits as
+    softmax(bcast_elemwise(x, bias, "add"))."""
     x = _dev_f32(x, "x")
     if x.dim() < 1 or x.shape[-1] == 0:
         raise ValueError("softmax: needs a non-empty innermost dimension")
     out = torch.empty_like(x)
     N = x.shape[-1]
-    cabi.check("softmax_hip", _lib().softmax_hip(_ptr(x), _ptr(out), x.numel() // N, N, _stream()))
+    M = x.numel() // N
+    if bias is None:
+        cabi.check("softmax_hip", _lib().softmax_hip(_ptr(x), _ptr(out), M, N, _stream()))
+        return out
+    bias = _dev_f32(bias, "bias")
+    if bias.numel() == 0 or bias.numel() % N or M % (bias.numel() // N):
+        raise ValueError("softmax: the bias must be whole rows of x's row length, a number of them that divides x's")
+    cabi.check("softmax_add_hip", _lib().softmax_add_hip(_ptr(x), _ptr(bias), _ptr(out), M, N, bias.numel() // N, _stream()))
+    return out
+
+
+def out_prod_tt(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """out_prod of the {1,0,2,3} permutations of a and b without the copies: a [ne03,ne02,ne01,K], b [ne13,ne12,ne11,K]
+    -> [ne13,ne12,ne11,ne01], contraction over the LAST torch dimension of both (src/modules/Attention.cpp:277-281:
+    out_prod(permute(attn), permute(V))).  The bits of out_prod on the permuted copies."""
+    a, b = _dev_f32(a, "a"), _dev_f32(b, "b")
+    while a.dim() < 4:
+        a = a.unsqueeze(0)
+    while b.dim() < 4:
+        b = b.unsqueeze(0)
+    ne03, ne02, ne01, ne00 = a.shape
+    ne13, ne12, ne11, ne10 = b.shape
+    if ne00 != ne10:
+        raise ValueError(f"out_prod_tt: contraction dims differ ({ne00} vs {ne10})")
+    ne0, ne1, ne2, ne3 = ne01, ne11, max(ne02, ne12), max(ne03, ne13)
+    out = torch.empty((ne3, ne2, ne1, ne0), dtype=torch.float32, device=a.device)
+    dims = [ne00, ne01, ne02, ne03, ne10, ne11, ne12, ne13, ne0, ne1, ne2, ne3]
+    cabi.check("out_prod_tt_hip", _lib().out_prod_tt_hip(_ptr(a), _ptr(b), _ptr(out), *dims, _stream()))
     return out
 
 

@@ -704,9 +704,34 @@ def test_default_attention_chain_stays_on_the_device(be, oracle, with_bias):
     graph, out = _attention_chain_graph(be, kl, ql, vl, bl, L, D, H, Bt, scale)
     assert all(be.supports_op(n) for n in graph)
     assert be.graph_compute(graph) == B.SUCCESS, be.last_error
-    assert be.nodes_fused_away == 1                                   # the logits and their scale
+    # the scale goes into the logits, the bias add into the softmax, the two permutations into the second contraction:
+    # three launches (out_prod_scaled, softmax_add, out_prod_tt) for the seven (six) nodes
+    assert be.nodes_fused_away == (4 if with_bias else 3)
     got = be.download(out).reshape(want.shape)
     np.testing.assert_allclose(got, want, rtol=0, atol=1e-4 * np.abs(want).max())
+    # every node on its own: the same bits
+    for setter in (be.set_fuse_scale_into_out_prod, be.set_fuse_add_into_soft_max, be.set_fuse_permutes_into_out_prod):
+        setter(False)
+    try:
+        graph, out = _attention_chain_graph(be, kl, ql, vl, bl, L, D, H, Bt, scale)
+        assert be.graph_compute(graph) == B.SUCCESS, be.last_error
+        assert be.nodes_fused_away == 0
+        plain = be.download(out).reshape(want.shape)
+        probs = be.download(graph[-4]).reshape(Bt, H, L, L)              # the softmax node's own tensor
+        np.testing.assert_allclose(probs, oracle.softmax(x), rtol=1e-5, atol=1e-37)
+    finally:
+        for setter in (be.set_fuse_scale_into_out_prod, be.set_fuse_add_into_soft_max, be.set_fuse_permutes_into_out_prod):
+            setter(True)
+    assert np.array_equal(plain.view(np.uint32), got.view(np.uint32))
+    # one pass at a time
+    for setter in (be.set_fuse_add_into_soft_max, be.set_fuse_permutes_into_out_prod):
+        setter(False)
+        try:
+            graph, out = _attention_chain_graph(be, kl, ql, vl, bl, L, D, H, Bt, scale)
+            assert be.graph_compute(graph) == B.SUCCESS, be.last_error
+            assert np.array_equal(be.download(out).reshape(want.shape).view(np.uint32), got.view(np.uint32))
+        finally:
+            setter(True)
     # opt in: the whole chain as one launch
     be.set_fuse_attention_chain(True)
     try:
@@ -734,8 +759,51 @@ def test_attention_chain_is_left_alone_when_an_intermediate_is_read_elsewhere(be
         attn = graph[2]
         attn.set_flag(B.FLAG_OUTPUT)                                  # the probabilities are wanted (e.g. for a backward pass)
         assert be.graph_compute(graph) == B.SUCCESS, be.last_error
-        assert be.nodes_fused_away == 1                               # only the scale went into the logits
+        assert be.nodes_fused_away == 3                               # the scale into the logits, the permutations into the second contraction
         probs = oracle.softmax(oracle.scale(oracle.out_prod(k, q), 0.25))
         np.testing.assert_allclose(be.download(attn).reshape(probs.shape), probs, rtol=1e-4, atol=1e-7)
     finally:
         be.set_fuse_attention_chain(False)
+
+
+def test_bias_add_and_permutations_stay_nodes_when_somebody_else_needs_them(be, oracle):
+    L, D, H, Bt = 20, 16, 2, 3
+    rng = np.random.default_rng(6)
+    k, q, v = (rng.standard_normal((Bt, H, D, L)).astype(np.float32) for _ in range(3))
+    bias = rng.standard_normal((Bt, H, L, L)).astype(np.float32)
+    kl, ql, vl, bl = _leaf(be, k), _leaf(be, q), _leaf(be, v), _leaf(be, bias)
+    x = oracle.bcast_elemwise(oracle.scale(oracle.out_prod(k, q), 0.25), bias, "add")
+    want = oracle.out_prod(oracle.permute(oracle.softmax(x), (1, 0, 2, 3)), oracle.permute(v, (1, 0, 2, 3)))
+    # the sum and the permuted probabilities flagged as outputs of the graph: both are written, nothing is folded
+    # but the scale
+    graph, out = _attention_chain_graph(be, kl, ql, vl, bl, L, D, H, Bt, 0.25)
+    added, attn_t = graph[2], graph[4]                              # the OP_ADD node and permute(softmax)
+    added.set_flag(B.FLAG_OUTPUT)
+    attn_t.set_flag(B.FLAG_OUTPUT)
+    assert be.graph_compute(graph) == B.SUCCESS, be.last_error
+    assert be.nodes_fused_away == 1
+    np.testing.assert_allclose(be.download(added).reshape(x.shape), x, rtol=0, atol=1e-4 * np.abs(x).max())      # (the logits are an f32 contraction)
+    np.testing.assert_allclose(be.download(attn_t).reshape(Bt, H, L, L), oracle.softmax(x).transpose(0, 1, 3, 2), rtol=1e-5, atol=1e-37)
+    np.testing.assert_allclose(be.download(out).reshape(want.shape), want, rtol=0, atol=1e-4 * np.abs(want).max())
+    # a bias that is one plane for all (whole rows, a count that divides the softmax's): folded, same bits as the nodes
+    small = rng.standard_normal((L, L)).astype(np.float32)
+    sl = _leaf(be, small)
+    outs = []
+    for fold in (True, False):
+        be.set_fuse_add_into_soft_max(fold)
+        try:
+            graph, out = _attention_chain_graph(be, kl, ql, vl, sl, L, D, H, Bt, 0.25)
+            assert be.graph_compute(graph) == B.SUCCESS, be.last_error
+            assert be.nodes_fused_away == (4 if fold else 3)
+            outs.append(be.download(out))
+        finally:
+            be.set_fuse_add_into_soft_max(True)
+    assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32))
+    # an add whose FIRST operand is the short one is left alone (the folded form adds whole rows to a full-size input)
+    scores = B.Tensor((L, L, H, Bt), B.F32, B.OP_OUT_PROD, [kl, ql])
+    swapped = B.Tensor((L, L, H, Bt), B.F32, B.OP_ADD, [sl, scores])
+    attn = B.Tensor((L, L, H, Bt), B.F32, B.OP_SOFT_MAX, [swapped])
+    assert be.graph_compute([scores, swapped, attn]) == B.SUCCESS, be.last_error
+    assert be.nodes_fused_away == 0
+    ref = oracle.softmax(oracle.bcast_elemwise(small, oracle.out_prod(k, q), "add"))
+    np.testing.assert_allclose(be.download(attn).reshape(ref.shape), ref, rtol=2e-5, atol=1e-30)

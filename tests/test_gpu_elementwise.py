@@ -159,3 +159,51 @@ def test_softmax_at_the_configured_attention_shapes_in_full(ops, oracle):
         got = ops.softmax(_dev(x)).cpu().numpy()
         np.testing.assert_allclose(got, oracle.softmax(x), rtol=SOFTMAX_RTOL, atol=SOFTMAX_ATOL)
         np.testing.assert_allclose(got.sum(-1), 1.0, rtol=2e-6)
+
+
+@pytest.mark.parametrize("D", [1, 3, 64, 103, 256, 257, 512, 513, 2048, 2049, 5000])
+def test_softmax_with_the_bias_add_folded_in_has_the_bits_of_the_two_nodes(ops, oracle, D):
+    rng = np.random.default_rng(D + 1)
+    rows = 36 if D < 1000 else 8
+    x = (3 * rng.standard_normal((rows, D))).astype(np.float32)
+    for brows in (rows, 4, 1):
+        b = (2 * rng.standard_normal((brows, D))).astype(np.float32)
+        two = ops.softmax(ops.bcast_elemwise(_dev(x), _dev(b), "add"))
+        one = ops.softmax(_dev(x), bias=_dev(b))
+        assert torch.equal(one.view(torch.int32), two.view(torch.int32)), (D, brows)
+        np.testing.assert_allclose(one.cpu().numpy(), oracle.softmax(oracle.bcast_elemwise(x, b, "add")),
+                                   rtol=softmax_rtol(D), atol=SOFTMAX_ATOL)
+    # masked keys in the bias, a NaN in the first element of a row and elsewhere, rows on 4-byte boundaries
+    b = np.zeros((rows, D), np.float32)
+    b[0, :] = -np.inf
+    b[1, D // 2:] = -np.inf
+    b[2, 0] = np.nan
+    b[3, D - 1] = np.nan
+    two = ops.softmax(ops.bcast_elemwise(_dev(x), _dev(b), "add"))
+    one = ops.softmax(_dev(x), bias=_dev(b))
+    assert torch.equal(torch.isnan(one), torch.isnan(two))
+    assert torch.equal(one.nan_to_num(7.0).view(torch.int32), two.nan_to_num(7.0).view(torch.int32))
+    base = _dev(rng.standard_normal(1 + rows * D).astype(np.float32))
+    xb = base[1:].reshape(rows, D)
+    bb = _dev(rng.standard_normal(rows * D + 1).astype(np.float32))[1:].reshape(rows, D)
+    assert torch.equal(ops.softmax(xb, bias=bb).view(torch.int32), ops.softmax(ops.bcast_elemwise(xb, bb, "add")).view(torch.int32))
+
+
+def test_softmax_add_refuses_a_bias_that_is_not_whole_rows(ops):
+    import ctypes as C
+    x, b = _dev(np.ones((6, 8), np.float32)), _dev(np.ones((4, 8), np.float32))
+    with pytest.raises(ValueError):
+        ops.softmax(x, bias=b)                                       # 4 rows do not divide 6
+    with pytest.raises(ValueError):
+        ops.softmax(x, bias=_dev(np.ones(12, np.float32)))           # not whole rows
+    p = lambda t: C.c_void_p(t.data_ptr())  # noqa: E731
+    assert ops._lib().softmax_add_hip(p(x), p(b), p(x), 6, 8, 4, None) == 1
+    assert ops._lib().softmax_add_hip(p(x), p(b), p(x), 6, 8, 0, None) == 1
+
+
+def test_softmax_add_at_the_configured_attention_shapes_in_full(ops, oracle):
+    rng = np.random.default_rng(12)
+    for planes, L in [(412, 103), (824, 256)]:
+        x = _dev((2 * rng.standard_normal((planes, L, L))).astype(np.float32))
+        b = _dev(rng.standard_normal((planes, L, L)).astype(np.float32))
+        assert torch.equal(ops.softmax(x, bias=b).view(torch.int32), ops.softmax(ops.bcast_elemwise(x, b, "add")).view(torch.int32))

@@ -760,3 +760,35 @@ def test_outer_prod_mean_back(ops, oracle, D, L, N, Bt):
         assert none is None and np.array_equal(gl.cpu().numpy(), wl)
         none, gr = ops.outer_prod_mean_back(_dev(gi), _dev(li), _dev(ri), D, L, N, Bt, want_left=False)
         assert none is None and np.array_equal(gr.cpu().numpy(), wr)
+
+
+@pytest.mark.parametrize("planes,Lq,Lk,D", [(3, 20, 20, 16), (7, 51, 51, 32), (412, 103, 103, 32), (60, 256, 256, 32), (5, 70, 33, 8)])
+def test_out_prod_of_the_unpermuted_operands_has_the_bits_of_out_prod_on_the_copies(ops, oracle, planes, Lq, Lk, D):
+    """The second contraction of the attention chain, out_prod(permute(attn), permute(V)) (src/modules/Attention.cpp:
+    277-281), without the two permutation copies: same products in the same order, on both matrix pipes."""
+    rng = np.random.default_rng(planes + Lq)
+    attn = rng.random((1, planes, Lq, Lk)).astype(np.float32)          # graph dims [Lk, Lq, planes, 1]
+    v = rng.standard_normal((1, planes, D, Lk)).astype(np.float32)     # graph dims [Lk, D, planes, 1]
+    ad, vd = _dev(attn), _dev(v)
+    for mode in ("split", "fp32"):
+        before = ops.set_f32_arithmetic(mode)
+        try:
+            copies = ops.out_prod(ops.permute(ad, (1, 0, 2, 3)), ops.permute(vd, (1, 0, 2, 3)))
+            direct = ops.out_prod_tt(ad, vd)
+        finally:
+            ops.set_f32_arithmetic(before)
+        assert direct.shape == copies.shape == (1, planes, D, Lq)
+        assert torch.equal(direct.view(torch.int32), copies.view(torch.int32)), mode
+    want = np.einsum("bpqk,bpdk->bpdq", attn.astype(np.float64), v.astype(np.float64))
+    np.testing.assert_allclose(direct.cpu().numpy(), want, rtol=0, atol=1e-4 * np.abs(want).max())
+    if planes <= 7:
+        ref = oracle.out_prod(oracle.permute(attn, (1, 0, 2, 3)), oracle.permute(v, (1, 0, 2, 3)))
+        np.testing.assert_allclose(direct.cpu().numpy(), ref, rtol=0, atol=1e-4 * np.abs(ref).max())
+    # a plane of src0 shared by several planes of src1 (the broadcast rule of out_prod), and shapes that do not fit
+    if planes % 3 == 0:
+        shared = _dev(attn[:, : planes // 3])
+        got = ops.out_prod_tt(shared, vd)
+        exp = ops.out_prod(ops.permute(shared, (1, 0, 2, 3)), ops.permute(vd, (1, 0, 2, 3)))
+        assert torch.equal(got.view(torch.int32), exp.view(torch.int32))
+    with pytest.raises(ValueError):
+        ops.out_prod_tt(ad, _dev(np.ones((1, planes, D, Lk + 1), np.float32)))
