@@ -348,7 +348,7 @@ def test_projections_wider_than_a_work_group_holds_go_in_column_parts(ops, oracl
 
 @pytest.mark.parametrize("key", sorted(WS_INSTANCE_SHAPES))
 def test_features_outermost_output_on_the_weight_stationary_kernel(ops, oracle, key):
-    """c_trans = 0 (the quantized weight was src[0], src/backends/CPUKernels.cpp:1120-1130: C is [M][N]) with a packed
+    """c_trans = 0 (the quantized weight was src[0], src/backend/CUDAKernels.cpp:761-777: C is [M][N]) with a packed
     weight: every weight-stationary instance has a form that stores this orientation; same bits as the oracle."""
     N, K, M = WS_INSTANCE_SHAPES[key]
     x, w = _inputs(5 * N + K + M, N, K, M)
