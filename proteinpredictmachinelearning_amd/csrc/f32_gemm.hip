@@ -579,6 +579,30 @@ __device__ __forceinline__ void load_rows8_buffer(const __amdgpu_buffer_rsrc_t r
         reg[c >> 2][c & 3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, lane_off + (kb + c) * ks_bytes, 0, 0));
 }
 
+// two rows (tid / 4 and tid / 4 + 64 of the tile), four consecutive k each, of an operand plane whose rows are
+// contiguous in k: A(row, k) = plane[row * rs + k].  K4 (K a multiple of four): a piece of sixteen bytes never runs
+// over the end of its row, so it is one load; otherwise element by element.  No branch either way: the generic form
+// of this load sits inside tests of the row and of the row's end, and the compiler waits for every load at the end of
+// its branch (26368 x 256 -> 256: 29 us, the waves waiting 38 % of it; 25 us with this form).
+template <bool K4>
+__device__ __forceinline__ void load_kcontig_buffer(const __amdgpu_buffer_rsrc_t rsrc, uint32_t rs_bytes, int row0, int nrows, int k0, int K,
+                                                    int tid, v4f (&reg)[2]) {
+    const int k = k0 + (tid & 3) * 4;
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int row = row0 + (tid >> 2) + it * 64;
+        const uint32_t at = row < nrows ? static_cast<uint32_t>(row) * rs_bytes + static_cast<uint32_t>(k) * 4u : OUTSIDE;
+        if (K4) {
+            const v4i raw = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, k < K ? at : OUTSIDE, 0, 0));
+            reg[it] = __builtin_bit_cast(v4f, raw);
+        } else {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                reg[it][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, k + c < K ? at + 4u * c : OUTSIDE, 0, 0));
+        }
+    }
+}
+
 // The finished accumulators of one wave to a dense plane C[m * ld + n] through a buffer resource over the plane.
 template <bool STREAM_C>
 __device__ __forceinline__ void store_acc_buffer(const __amdgpu_buffer_rsrc_t rsrc, uint32_t ld_bytes, int N, float alpha,
@@ -604,9 +628,10 @@ __device__ __forceinline__ void store_acc_buffer(const __amdgpu_buffer_rsrc_t rs
     }
 }
 
-template <int MODE, bool SPLIT_C, bool STREAM_C, bool FAST_IO = false>
+template <int MODE, bool SPLIT_C, bool STREAM_C, bool FAST_IO = false, bool K4 = true>
 __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
-    static_assert(!FAST_IO || (MODE == LOAD_ROW_CONTIG && !SPLIT_C), "buffer addressing: contiguous rows, dense output");
+    static_assert(!FAST_IO || ((MODE == LOAD_ROW_CONTIG || MODE == LOAD_K_CONTIG) && !SPLIT_C),
+                  "buffer addressing: rows contiguous in themselves or in k, dense output");
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * SPLIT_PLANE];
     __shared__ __attribute__((aligned(16))) uint8_t lds_b[3 * SPLIT_PLANE];
 
@@ -638,12 +663,17 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
     // FAST_IO: one buffer resource per operand plane and for the output plane (sizes checked by the launcher)
     __amdgpu_buffer_rsrc_t rsrc_a, rsrc_b, rsrc_c;
     if (FAST_IO) {
-        rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, static_cast<int>(p.K * p.a_ks * 4), 0x00020000);
-        rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, static_cast<int>(p.K * p.b_ks * 4), 0x00020000);
+        const int64_t a_plane = MODE == LOAD_K_CONTIG ? (p.M - 1) * p.a_rs + p.K : p.K * p.a_ks;     // floats from the plane's base to its end
+        const int64_t b_plane = MODE == LOAD_K_CONTIG ? (p.N - 1) * p.b_rs + p.K : p.K * p.b_ks;
+        rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, static_cast<int>(a_plane * 4), 0x00020000);
+        rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, static_cast<int>(b_plane * 4), 0x00020000);
         rsrc_c = __builtin_amdgcn_make_buffer_rsrc(C, 0, static_cast<int>(p.M * p.c_mi * 4), 0x00020000);
     }
     const auto load_both = [&](int k0) {
-        if (FAST_IO) {
+        if (FAST_IO && MODE == LOAD_K_CONTIG) {
+            load_kcontig_buffer<K4>(rsrc_a, static_cast<uint32_t>(p.a_rs) * 4u, m0, p.M, k0, p.K, tid, ra);
+            load_kcontig_buffer<K4>(rsrc_b, static_cast<uint32_t>(p.b_rs) * 4u, n0, p.N, k0, p.K, tid, rb);
+        } else if (FAST_IO) {
             load_rows8_buffer(rsrc_a, static_cast<uint32_t>(p.a_ks) * 4u, m0, p.M, k0, tid, ra);
             load_rows8_buffer(rsrc_b, static_cast<uint32_t>(p.b_ks) * 4u, n0, p.N, k0, tid, rb);
         } else if (MODE == LOAD_ROW_CONTIG) {
@@ -694,6 +724,130 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
 
     if (FAST_IO) store_acc_buffer<STREAM_C>(rsrc_c, static_cast<uint32_t>(p.c_mi) * 4u, p.N, p.alpha, acc, m0 + wm, n0 + wn, lane);
     else store_acc<SPLIT_C, STREAM_C, false, false>(p, C, acc, m0 + wm, n0 + wn, lane);
+}
+
+// ------------------------------------------------------------------------------------------
+// The same contraction with the work of a work-group divided between two sets of waves.  In gemm_bf16x3_kernel a wave
+// splits its share of a 16-k chunk (vector pipe), waits at a barrier, and then issues the chunk's matrix work (matrix
+// pipe): with at most one work-group per CU -- a LinearLayer-shaped contraction of a few hundred tiles, or a small
+// square one -- the two pipes take turns and the K loop costs 1.2 us per chunk whatever the problem's size
+// (408 x 256 -> 16 and 26368 x 256 -> 128 both took 19 to 20 us).  Here waves 4..7 of a work-group of eight only load
+// and split (chunk k + 1, into the other half of a double buffer, from loads issued three chunks ahead: they hold no
+// accumulators, so the registers are there), and waves 0..3 only read fragments and issue MFMAs (chunk k); one barrier
+// per chunk.  Every SIMD hosts one wave of each kind, so the vector and the matrix pipe work at the same time.  Same
+// thread-to-element mapping, same fragments, same order of the products as gemm_bf16x3_kernel: same bits.  Buffer
+// addressing throughout (the launcher's conditions for it).  Measured, us, this / gemm_bf16x3_kernel: 408 x 256 -> 16
+// 13.5 / 19.1, 26368 x 256 -> 16 .. 128 15.0 - 16.9 / 20.3, 10609 x 256 -> 128 14.7 / 19.6, 1024^3 41 / 65; with
+// more tiles than CUs (26368 x 256 -> 256 and wider, the many-plane contractions) the work-groups of a CU overlap
+// each other anyway and the two forms measure the same: the launcher takes this one up to one tile per CU.
+constexpr int PC_AHEAD = 3;                       // chunks a producer wave has in flight
+template <int MODE, bool STREAM_C, bool K4>
+__global__ __launch_bounds__(512) void gemm_bf16x3_pc_kernel(const GemmParams p) {
+    static_assert(MODE == LOAD_ROW_CONTIG || MODE == LOAD_K_CONTIG, "buffer addressing");
+    constexpr int STAGE = 3 * SPLIT_PLANE;            // the three planes of one operand's chunk
+    __shared__ __attribute__((aligned(16))) uint8_t lds_ab[2][2 * STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const bool producer = wave >= 4;
+    const int ptid = tid & 255;                         // a producer's number in gemm_bf16x3_kernel's thread-to-element mapping
+    const int cw = wave & 3;
+    const int wm = (cw >> 1) * 64, wn = (cw & 1) * 64;
+
+    int plane, m0, n0;
+    tile_of_group(p, plane, m0, n0);
+    const int p2 = plane % p.np2, p3 = plane / p.np2;
+    const float* A = p.A + p2 * p.a_p2 + p3 * p.a_p3;
+    const float* B = p.B + (p2 / p.b_div2) * p.b_p2 + (p3 / p.b_div3) * p.b_p3;
+    float* C = p.C + p2 * p.c_p2 + p3 * p.c_p3;
+    const int chunks = (p.K + BK - 1) / BK;
+
+    const int64_t a_plane = MODE == LOAD_K_CONTIG ? (p.M - 1) * p.a_rs + p.K : p.K * p.a_ks;
+    const int64_t b_plane = MODE == LOAD_K_CONTIG ? (p.N - 1) * p.b_rs + p.K : p.K * p.b_ks;
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, static_cast<int>(a_plane * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, static_cast<int>(b_plane * 4), 0x00020000);
+
+    // Both kinds of wave pass chunks + 1 barriers in their loops: barrier i + 1 says "chunk i is in LDS" and "chunk
+    // i - 1 has been read".
+    int fired = 0;
+    if (producer) {
+        v4f ra[PC_AHEAD][2], rb[PC_AHEAD][2];
+        const auto load_both = [&](int c, v4f (&xa)[2], v4f (&xb)[2]) {
+            if (MODE == LOAD_K_CONTIG) {
+                load_kcontig_buffer<K4>(rsrc_a, static_cast<uint32_t>(p.a_rs) * 4u, m0, p.M, c * BK, p.K, ptid, xa);
+                load_kcontig_buffer<K4>(rsrc_b, static_cast<uint32_t>(p.b_rs) * 4u, n0, p.N, c * BK, p.K, ptid, xb);
+            } else {
+                load_rows8_buffer(rsrc_a, static_cast<uint32_t>(p.a_ks) * 4u, m0, p.M, c * BK, ptid, xa);
+                load_rows8_buffer(rsrc_b, static_cast<uint32_t>(p.b_ks) * 4u, n0, p.N, c * BK, ptid, xb);
+            }
+        };
+#pragma unroll
+        for (int d = 0; d < PC_AHEAD; ++d)
+            if (d < chunks) load_both(d, ra[d], rb[d]);
+        SplitGuard guard;
+        // chunk c goes to half c % 2 while the other waves contract chunk c - 1 out of the other half; the register
+        // sets take turns by name (the loop body is written out PC_AHEAD times)
+        for (int cg = 0; cg < chunks; cg += PC_AHEAD) {
+#pragma unroll
+            for (int d = 0; d < PC_AHEAD; ++d) {
+                const int c = cg + d;
+                if (c >= chunks) break;                 // uniform
+                uint8_t* half = lds_ab[c & 1];
+                split_store<MODE>(half, ptid, ra[d], guard);
+                split_store<MODE>(half + STAGE, ptid, rb[d], guard);
+                if (c + PC_AHEAD < chunks) load_both(c + PC_AHEAD, ra[d], rb[d]);
+                __syncthreads();
+            }
+        }
+        __syncthreads();                                // (the other waves' last chunk)
+        fired = guard.fired() ? 1 : 0;
+    }
+
+    v16f acc[2][2];
+    if (!producer) {
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj) {
+            const int n = n0 + wn + tj * 32 + j;
+            const float b0 = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+#pragma unroll
+            for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[ti][tj][r] = b0;
+        }
+        const int frag_a = (wm + j) * SPLIT_PITCH + hh * 16;
+        const int frag_b = STAGE + (wn + j) * SPLIT_PITCH + hh * 16;
+        __syncthreads();                                // chunk 0 is in LDS
+        for (int c = 0; c < chunks; ++c) {
+            const uint8_t* half = lds_ab[c & 1];
+            v8bf fa[2][3], fb[2][3];
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int s = 0; s < 3; ++s) {
+                    fa[t][s] = *reinterpret_cast<const v8bf*>(half + frag_a + s * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
+                    fb[t][s] = *reinterpret_cast<const v8bf*>(half + frag_b + s * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
+                }
+#pragma unroll
+            for (int q = 0; q < 6; ++q)
+#pragma unroll
+                for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+                    for (int tj = 0; tj < 2; ++tj)
+                        acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][SPLIT_TERMS[q][0]], fb[tj][SPLIT_TERMS[q][1]], acc[ti][tj], 0, 0, 0);
+            __syncthreads();                            // chunk c has been read; chunk c + 1 is in LDS
+        }
+    }
+
+    // an operand of this tile that the split could not carry: the whole tile again, the reference's way
+    if (__syncthreads_or(fired)) {
+        if (tid < 256) plain_tile(p, A, B, C, m0, n0, BM, BN, tid);
+        return;
+    }
+    if (!producer) {
+        const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(C, 0, static_cast<int>(p.M * p.c_mi * 4), 0x00020000);
+        store_acc_buffer<STREAM_C>(rsrc_c, static_cast<uint32_t>(p.c_mi) * 4u, p.N, p.alpha, acc, m0 + wm, n0 + wn, lane);
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1432,6 +1586,9 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
             return rc;
         }
     }
+    // few tiles and a K loop worth it: the work-group divided into loading / splitting and contracting waves
+    // (gemm_bf16x3_pc_kernel), where buffer addressing applies
+    const bool two_sets = total <= device_cu_count() && p.K > 3 * BK;
 #define PPML_LAUNCH_BF16(MODE, SPLIT)                                                                 \
     do {                                                                                              \
         if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_kernel<MODE, SPLIT, true>), grid, block, 0, stream, p);  \
@@ -1487,12 +1644,32 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
                 return check_launch(what);
             }
         }
-        if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_kernel<LOAD_ROW_CONTIG, false, true, true>), grid, block, 0, stream, p);
+        if (two_sets) {
+            if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_pc_kernel<LOAD_ROW_CONTIG, true, true>), grid, dim3(512), 0, stream, p);
+            else hipLaunchKernelGGL((gemm_bf16x3_pc_kernel<LOAD_ROW_CONTIG, false, true>), grid, dim3(512), 0, stream, p);
+        }
+        else if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_kernel<LOAD_ROW_CONTIG, false, true, true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((gemm_bf16x3_kernel<LOAD_ROW_CONTIG, false, false, true>), grid, block, 0, stream, p);
     }
     else if (!p.clamp && !p.f16_in) {
         // binary32 operands without the finite guard: the contraction runs on the bf16 matrix pipe
-        if (mode == LOAD_K_CONTIG)        { if (split) PPML_LAUNCH_BF16(LOAD_K_CONTIG, true);   else PPML_LAUNCH_BF16(LOAD_K_CONTIG, false); }
+        // rows contiguous in k, dense output planes, every plane below 2 GiB: buffer addressing (see load_kcontig_buffer)
+        const bool k_fast = mode == LOAD_K_CONTIG && !split && p.c_ni == 1 && p.a_lm == 0 &&
+                            ((p.M - 1) * p.a_rs + p.K) * 4 < (1LL << 31) && ((p.N - 1) * p.b_rs + p.K) * 4 < (1LL << 31) &&
+                            p.M * p.c_mi * 4 < (1LL << 31) && p.c_mi < (1 << 22) && p.a_rs < (1 << 22) && p.b_rs < (1 << 22);
+        if (k_fast && two_sets) {
+#define PPML_KPC(STREAM_, K4_) hipLaunchKernelGGL((gemm_bf16x3_pc_kernel<LOAD_K_CONTIG, STREAM_, K4_>), grid, dim3(512), 0, stream, p)
+            if (p.K % 4 == 0) { if (p.stream_c) PPML_KPC(true, true); else PPML_KPC(false, true); }
+            else              { if (p.stream_c) PPML_KPC(true, false); else PPML_KPC(false, false); }
+#undef PPML_KPC
+        }
+        else if (k_fast) {
+#define PPML_KFAST(STREAM_, K4_) hipLaunchKernelGGL((gemm_bf16x3_kernel<LOAD_K_CONTIG, false, STREAM_, true, K4_>), grid, block, 0, stream, p)
+            if (p.K % 4 == 0) { if (p.stream_c) PPML_KFAST(true, true); else PPML_KFAST(false, true); }
+            else              { if (p.stream_c) PPML_KFAST(true, false); else PPML_KFAST(false, false); }
+#undef PPML_KFAST
+        }
+        else if (mode == LOAD_K_CONTIG)   { if (split) PPML_LAUNCH_BF16(LOAD_K_CONTIG, true);   else PPML_LAUNCH_BF16(LOAD_K_CONTIG, false); }
         else if (mode == LOAD_ROW_CONTIG) { if (split) PPML_LAUNCH_BF16(LOAD_ROW_CONTIG, true); else PPML_LAUNCH_BF16(LOAD_ROW_CONTIG, false); }
         else                              { if (split) PPML_LAUNCH_BF16(LOAD_STRIDED, true);    else PPML_LAUNCH_BF16(LOAD_STRIDED, false); }
     }
