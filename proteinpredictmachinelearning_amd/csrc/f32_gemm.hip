@@ -1520,7 +1520,10 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
     const int64_t planes_groups = static_cast<int64_t>((p.M + PBM - 1) / PBM) * p.tiles_n;
     const int chunks = (p.K + BK - 1) / BK;
     int slices = 1;
-    if (planes_groups < PLANES_MIN_GROUPS) {
+    // (K slices are for problems that leave most CUs without a tile -- the outer-product-mean backward has 96 --; with
+    // a tile per CU or so the split ahead of the matrix work costs more than the slices win: 26368 x 512 -> 256, 206
+    // work-groups, took 107 us in two slices against 48 on operands split in the tile loop)
+    if (planes_groups < PLANES_MIN_GROUPS / 4) {
         const int64_t want = (PLANES_MIN_GROUPS + planes_groups - 1) / planes_groups;
         const int64_t most = chunks / PLANES_MIN_SLICE_CHUNKS;
         slices = static_cast<int>(want < most ? want : most);
