@@ -850,6 +850,148 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_kernel(const GemmParams p)
     }
 }
 
+// The same again for contractions with one NARROW side: at most 32 rows of A (SIDE_M: the second contraction of the
+// attention chain, out_prod_tt_hip with the head dimension for its rows) or of B (SIDE_N: a LinearLayer with up to 32
+// output features -- the bias projections onto the heads, the 256 -> 16 projections of the outer-product-mean).  A 128 x
+// 128 tile is three quarters padding there: matrix work, split and LDS traffic for rows that do not exist.  Here the
+// tile is 128 along the long side and 32 along the narrow one; each of the four contracting waves takes 32 rows of the
+// long operand against the one fragment of the narrow operand, six MFMAs per 16-k chunk; of the loading waves all
+// four split the long operand and two of them the narrow one.  Operands contiguous in k, buffer addressing, same
+// products in the same order as the other forms: same bits.
+constexpr int SIDE_M = 1, SIDE_N = 2;
+template <int SIDE, bool STREAM_C, bool K4>
+__global__ __launch_bounds__(512) void gemm_bf16x3_pc_narrow_kernel(const GemmParams p) {
+    static_assert(SIDE == SIDE_M || SIDE == SIDE_N, "which operand is the narrow one");
+    constexpr int LONG_STAGE = 3 * SPLIT_PLANE;                  // three planes of 128 rows
+    constexpr int NARROW_PLANE = 32 * SPLIT_PITCH;
+    constexpr int STAGE = LONG_STAGE + 3 * NARROW_PLANE;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_ab[2][STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const bool producer = wave >= 4;
+    const int ptid = tid & 255;
+    const int cw = wave & 3;
+
+    // the tile list runs along the long side only (the launcher sets tiles_m or tiles_n to 1 for the narrow side)
+    int plane, m0, n0;
+    tile_of_group(p, plane, m0, n0);
+    const int p2 = plane % p.np2, p3 = plane / p.np2;
+    const float* A = p.A + p2 * p.a_p2 + p3 * p.a_p3;
+    const float* B = p.B + (p2 / p.b_div2) * p.b_p2 + (p3 / p.b_div3) * p.b_p3;
+    float* C = p.C + p2 * p.c_p2 + p3 * p.c_p3;
+    const int chunks = (p.K + BK - 1) / BK;
+
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, static_cast<int>(((p.M - 1) * p.a_rs + p.K) * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, static_cast<int>(((p.N - 1) * p.b_rs + p.K) * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t& rsrc_long = SIDE == SIDE_M ? rsrc_b : rsrc_a;
+    const __amdgpu_buffer_rsrc_t& rsrc_narrow = SIDE == SIDE_M ? rsrc_a : rsrc_b;
+    const uint32_t long_rs = static_cast<uint32_t>(SIDE == SIDE_M ? p.b_rs : p.a_rs) * 4u;
+    const uint32_t narrow_rs = static_cast<uint32_t>(SIDE == SIDE_M ? p.a_rs : p.b_rs) * 4u;
+    const int long_row0 = SIDE == SIDE_M ? n0 : m0, long_rows = SIDE == SIDE_M ? p.N : p.M;
+    const int narrow_rows = SIDE == SIDE_M ? p.M : p.N;
+
+    // (barriers: chunks + 1 in either loop, as in gemm_bf16x3_pc_kernel)
+    int fired = 0;
+    if (producer) {
+        v4f rl[PC_AHEAD][2];                            // the long operand: two row pieces per thread
+        v4f rn[PC_AHEAD];                               // the narrow one: one piece per thread of the first two loading waves
+        const bool has_narrow = wave < 6;               // rows ptid / 4 < 32
+        const auto load_both = [&](int c, v4f (&xl)[2], v4f& xn) {
+            load_kcontig_buffer<K4>(rsrc_long, long_rs, long_row0, long_rows, c * BK, p.K, ptid, xl);
+            if (has_narrow) {
+                const int k = c * BK + (ptid & 3) * 4;
+                const int row = ptid >> 2;
+                const uint32_t at = row < narrow_rows ? static_cast<uint32_t>(row) * narrow_rs + static_cast<uint32_t>(k) * 4u : OUTSIDE;
+                if (K4) {
+                    xn = __builtin_bit_cast(v4f, __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_narrow, k < p.K ? at : OUTSIDE, 0, 0)));
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        xn[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_narrow, k + e < p.K ? at + 4u * e : OUTSIDE, 0, 0));
+                }
+            }
+        };
+#pragma unroll
+        for (int d = 0; d < PC_AHEAD; ++d)
+            if (d < chunks) load_both(d, rl[d], rn[d]);
+        SplitGuard guard;
+        for (int cg = 0; cg < chunks; cg += PC_AHEAD) {
+#pragma unroll
+            for (int d = 0; d < PC_AHEAD; ++d) {
+                const int c = cg + d;
+                if (c >= chunks) break;                 // uniform
+                uint8_t* half = lds_ab[c & 1];
+                split_store<LOAD_K_CONTIG>(half, ptid, rl[d], guard);
+                if (has_narrow) {
+                    uint2 parts[3];
+                    split4(rn[d], parts, guard);
+                    uint8_t* dst = half + LONG_STAGE + (ptid >> 2) * SPLIT_PITCH + (ptid & 3) * 8;
+#pragma unroll
+                    for (int s3 = 0; s3 < 3; ++s3) *reinterpret_cast<uint2*>(dst + s3 * NARROW_PLANE) = parts[s3];
+                }
+                if (c + PC_AHEAD < chunks) load_both(c + PC_AHEAD, rl[d], rn[d]);
+                __syncthreads();
+            }
+        }
+        __syncthreads();
+        fired = guard.fired() ? 1 : 0;
+    }
+
+    v16f acc;
+    if (!producer) {
+        {
+            const int n = SIDE == SIDE_M ? n0 + cw * 32 + j : j;
+            const float b0 = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = b0;
+        }
+        const int frag_long = (cw * 32 + j) * SPLIT_PITCH + hh * 16;
+        const int frag_narrow = LONG_STAGE + j * SPLIT_PITCH + hh * 16;
+        __syncthreads();                                // chunk 0 is in LDS
+        for (int c = 0; c < chunks; ++c) {
+            const uint8_t* half = lds_ab[c & 1];
+            v8bf fl[3], fn[3];
+#pragma unroll
+            for (int s3 = 0; s3 < 3; ++s3) {
+                fl[s3] = *reinterpret_cast<const v8bf*>(half + frag_long + s3 * SPLIT_PLANE);
+                fn[s3] = *reinterpret_cast<const v8bf*>(half + frag_narrow + s3 * NARROW_PLANE);
+            }
+#pragma unroll
+            for (int q = 0; q < 6; ++q) {
+                // (part of a, part of b): a is the narrow operand with SIDE_M, the long one with SIDE_N
+                const v8bf& fa = SIDE == SIDE_M ? fn[SPLIT_TERMS[q][0]] : fl[SPLIT_TERMS[q][0]];
+                const v8bf& fb = SIDE == SIDE_M ? fl[SPLIT_TERMS[q][1]] : fn[SPLIT_TERMS[q][1]];
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+            }
+            __syncthreads();
+        }
+    }
+
+    if (__syncthreads_or(fired)) {
+        // the whole tile again, the reference's way: 128 along the long side, the narrow side in full
+        if (tid < 256) plain_tile(p, A, B, C, SIDE == SIDE_M ? 0 : m0, SIDE == SIDE_M ? n0 : 0, SIDE == SIDE_M ? 32 : BM, SIDE == SIDE_M ? BN : 32, tid);
+        return;
+    }
+    if (!producer) {
+        const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(C, 0, static_cast<int>(p.M * p.c_mi * 4), 0x00020000);
+        const uint32_t ld_bytes = static_cast<uint32_t>(p.c_mi) * 4u;
+        const int m_base = SIDE == SIDE_M ? 0 : m0 + cw * 32;
+        const int n = SIDE == SIDE_M ? n0 + cw * 32 + j : j;
+        const uint32_t first = static_cast<uint32_t>(m_base + 4 * hh);
+        // rows past the matrix fall outside the plane by themselves (offset >= M * ld bytes)
+        const uint32_t base = n < p.N ? first * ld_bytes + static_cast<uint32_t>(n) * 4u : OUTSIDE;
+        const bool scale = p.alpha != 1.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float v = acc[r];
+            if (scale) v *= p.alpha;
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rsrc_c, base + (8 * (r >> 2) + (r & 3)) * ld_bytes, 0, STREAM_C ? 3 : 0);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // Batched contractions with a short K (at most 32: the attention logits, K = head dimension) on operands whose
 // rows are contiguous, into dense output planes.  Per output tile there are two 16-k chunks of matrix work and
@@ -1660,7 +1802,21 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
         const bool k_fast = mode == LOAD_K_CONTIG && !split && p.c_ni == 1 && p.a_lm == 0 &&
                             ((p.M - 1) * p.a_rs + p.K) * 4 < (1LL << 31) && ((p.N - 1) * p.b_rs + p.K) * 4 < (1LL << 31) &&
                             p.M * p.c_mi * 4 < (1LL << 31) && p.c_mi < (1 << 22) && p.a_rs < (1 << 22) && p.b_rs < (1 << 22);
-        if (k_fast && two_sets) {
+        if (k_fast && p.K > 3 * BK && (p.N <= 32 || p.M <= 32)) {
+            // one narrow side: tiles of 128 x 32 along the other (gemm_bf16x3_pc_narrow_kernel)
+            const bool side_n = p.N <= 32;
+            const int64_t tiles_long = side_n ? p.tiles_m : p.tiles_n;
+            if (side_n) p.tiles_n = 1; else p.tiles_m = 1;
+            const dim3 ngrid(static_cast<unsigned>(tiles_long * p.np2 * p.np3));
+#define PPML_KNARROW(SIDE_, STREAM_, K4_) hipLaunchKernelGGL((gemm_bf16x3_pc_narrow_kernel<SIDE_, STREAM_, K4_>), ngrid, dim3(512), 0, stream, p)
+            const bool k4 = p.K % 4 == 0;
+            if (side_n) { if (k4) { if (p.stream_c) PPML_KNARROW(SIDE_N, true, true); else PPML_KNARROW(SIDE_N, false, true); }
+                          else    { if (p.stream_c) PPML_KNARROW(SIDE_N, true, false); else PPML_KNARROW(SIDE_N, false, false); } }
+            else        { if (k4) { if (p.stream_c) PPML_KNARROW(SIDE_M, true, true); else PPML_KNARROW(SIDE_M, false, true); }
+                          else    { if (p.stream_c) PPML_KNARROW(SIDE_M, true, false); else PPML_KNARROW(SIDE_M, false, false); } }
+#undef PPML_KNARROW
+        }
+        else if (k_fast && two_sets) {
 #define PPML_KPC(STREAM_, K4_) hipLaunchKernelGGL((gemm_bf16x3_pc_kernel<LOAD_K_CONTIG, STREAM_, K4_>), grid, dim3(512), 0, stream, p)
             if (p.K % 4 == 0) { if (p.stream_c) PPML_KPC(true, true); else PPML_KPC(false, true); }
             else              { if (p.stream_c) PPML_KPC(true, false); else PPML_KPC(false, false); }

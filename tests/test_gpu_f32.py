@@ -792,3 +792,42 @@ def test_out_prod_of_the_unpermuted_operands_has_the_bits_of_out_prod_on_the_cop
         assert torch.equal(got.view(torch.int32), exp.view(torch.int32))
     with pytest.raises(ValueError):
         ops.out_prod_tt(ad, _dev(np.ones((1, planes, D, Lk + 1), np.float32)))
+
+
+@pytest.mark.parametrize("M,K,N", [(1000, 256, 16), (130, 64, 32), (26368, 256, 8), (300, 100, 4), (257, 130, 1), (5, 512, 32)])
+def test_linear_layers_with_few_output_features_take_narrow_tiles_with_the_same_bits(ops, oracle, M, K, N):
+    """mul_mat with at most 32 output features (the bias projections onto the heads, the 256 -> 16 projections of the
+    outer-product-mean; src/model/Embedding.cpp:120-153) runs on 128 x 32 tiles: the bits of the same contraction with
+    the weight padded to 64 rows of zeros (which takes the ordinary tiles), the oracle within the f32 bar, bias first,
+    and the reference's infinities."""
+    rng = np.random.default_rng(M + N)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    b = rng.standard_normal((N, K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    ad = _dev(a)
+    got = ops.mul_mat(ad, _dev(b), _dev(bias))
+    padded_b = np.zeros((64, K), np.float32)
+    padded_b[:N] = b
+    padded_bias = np.zeros(64, np.float32)
+    padded_bias[:N] = bias
+    wide = ops.mul_mat(ad, _dev(padded_b), _dev(padded_bias))
+    assert torch.equal(got.view(torch.int32), wide[:, :N].contiguous().view(torch.int32))
+    if M <= 1000:
+        want = oracle.mul_mat_f32(a, b, bias)
+        absprod = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64).T + np.abs(bias)
+        assert (np.abs(got.cpu().numpy().astype(np.float64) - want) <= RTOL * absprod).all()
+        a_inf = a.copy()
+        a_inf[M // 2, K // 3] = np.inf
+        got_inf = ops.mul_mat(_dev(a_inf), _dev(b), _dev(bias)).cpu().numpy()
+        with np.errstate(invalid="ignore", over="ignore"):
+            want_inf = oracle.mul_mat_f32(a_inf, b, bias)
+        assert np.array_equal(np.isnan(got_inf), np.isnan(want_inf))
+        assert np.array_equal(got_inf[np.isinf(want_inf)], want_inf[np.isinf(want_inf)])
+    # sentinels around C
+    buf = torch.full((M * N + 512,), 3.5, device="cuda")
+    out = buf[256:256 + M * N].view(M, N)
+    import ctypes as C
+    p = lambda t: C.c_void_p(t.data_ptr())  # noqa: E731
+    bd, biasd = _dev(b), _dev(bias)
+    assert ops._lib().mul_mat_hip(p(ad), p(bd), p(out), M, K, N, p(biasd), None) == 0
+    assert torch.equal(out.view(torch.int32), got.view(torch.int32)) and (buf[:256] == 3.5).all() and (buf[256 + M * N:] == 3.5).all()
