@@ -992,6 +992,171 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_narrow_kernel(const GemmPa
     }
 }
 
+// A long, tall operand with compound indices against a small one (the outer-product-mean backward: the gradient
+// tensor [d1][d2][i][j], 12288 x 12288 at the configured size, against 256 columns).  Splitting the tall operand ahead,
+// as gemm_planes_kernel wants it, reads it element by element and moves 2.5 times its bytes before the matrix work
+// starts -- as long as the matrix work itself.  Here only the SMALL operand is split ahead (split_operand_kernel, any
+// strides); the contracting waves read its fragments straight from memory (L2), HS_AHEAD chunks ahead, one wave per 32
+// columns, and the loading waves split the tall operand as in gemm_bf16x3_pc_kernel, from loads that follow its runs:
+// the compound index is resolved once per lane for the rows (a byte offset) and by a scalar cursor for the chunks
+// (run number and place within the run of a chunk's first k), so a load is one add.  HS_KRUN: the contraction index
+// runs along memory (sixteen bytes per load); HS_RRUN: the row index does (eight loads, each contiguous across the
+// lanes).  GEN: runs of any length (a pair tensor of 103 residues): a chunk may then pass from one run into the next and
+// end behind the last one, so every element takes its own load, whose offset is picked between the two runs' bases.
+// The K loop is cut into slices (tile numbering: the slice is the plane; one slice is allowed): raw sums go to
+// partial[slice][m][n] for reduce_slices_kernel, which adds them in slice order, applies bias, factor and the output's
+// addressing, and computes the rows and columns flagged here (fired_a, one per 32 rows) or by the small operand's split
+// (fired_b) the reference's way.
+constexpr int HS_KRUN = 0, HS_RRUN = 1;
+constexpr int HS_AHEAD = 2;
+template <int AMODE, bool GEN>
+__global__ __launch_bounds__(512, 2) void gemm_bf16x3_half_split_kernel(const GemmParams p, const uint8_t* __restrict__ wb, int nb_pad, int chunks,
+                                                                        int slice_chunks, float* __restrict__ partial, int ma_pad,
+                                                                        int* __restrict__ fired_a, uint32_t a_span_bytes) {
+    constexpr int STAGE = 3 * SPLIT_PLANE;
+    constexpr int SMODE = AMODE == HS_KRUN ? LOAD_K_CONTIG : LOAD_ROW_CONTIG;     // the thread-to-element mapping of the split
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[2][STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const bool producer = wave >= 4;
+    const int ptid = tid & 255;
+    const int wn = (wave & 3) * 32;
+
+    int slice, m0, n0;
+    tile_of_group(p, slice, m0, n0);
+    const int c_begin = slice * slice_chunks;
+    const int c_end = c_begin + slice_chunks < chunks ? c_begin + slice_chunks : chunks;
+    const int nch = c_end - c_begin;
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.A), 0, static_cast<int>(a_span_bytes), 0x00020000);
+
+    // (barriers: nch + 1 in either loop, as in gemm_bf16x3_pc_kernel)
+    if (producer) {
+        // byte offsets of this lane's rows (and, HS_KRUN, of its four k within a chunk); 2^31 for rows past the matrix
+        uint32_t roff[2];
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+            const int row = AMODE == HS_KRUN ? m0 + (ptid >> 2) + it * 64 : m0 + (ptid & 127);
+            const int64_t el = static_cast<int64_t>(row / p.a_lm) * p.a_mo + static_cast<int64_t>(row % p.a_lm) * p.a_mi;
+            roff[it] = row < p.M ? static_cast<uint32_t>(el) * 4u + (AMODE == HS_KRUN ? (ptid & 3) * 16u : 0u) : OUTSIDE;
+        }
+        // the chunk the next load is for: run number and place within the run of its first k
+        int kd = (c_begin * BK) / p.a_lk, kr = (c_begin * BK) % p.a_lk;
+        const int nruns = p.K / p.a_lk;
+        const int oct = __builtin_amdgcn_readfirstlane(ptid >> 7) * 8;
+        const auto load = [&](v4f (&x)[2]) {
+            if (!GEN) {                                 // runs of whole chunks
+                if (AMODE == HS_KRUN) {
+                    const uint32_t koff = static_cast<uint32_t>(static_cast<int64_t>(kd) * p.a_ko + kr) * 4u;
+#pragma unroll
+                    for (int it = 0; it < 2; ++it) x[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, roff[it] + koff, 0, 0));
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
+                        const uint32_t koff = static_cast<uint32_t>(static_cast<int64_t>(kd) * p.a_ko + static_cast<int64_t>(kr + oct + c) * p.a_ki) * 4u;
+                        x[c >> 2][c & 3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_a, roff[0] + koff, 0, 0));
+                    }
+                }
+            } else {
+                // element u places behind the chunk's first k lies in this run while kr + u < run length, else in the next
+                // one (a run is at least a chunk long: the launcher's rule); a run behind the last one is outside: 2^30,
+                // which with the operand's span (at most 2^30 bytes in this form) and with a row's 2^31 stays outside
+                constexpr uint32_t NO_RUN = 0x40000000u;
+                const uint32_t here = kd < nruns ? static_cast<uint32_t>(static_cast<int64_t>(kd) * p.a_ko + static_cast<int64_t>(kr) * p.a_ki) * 4u : NO_RUN;
+                const uint32_t next = kd + 1 < nruns ? static_cast<uint32_t>(static_cast<int64_t>(kd + 1) * p.a_ko + static_cast<int64_t>(kr - p.a_lk) * p.a_ki) * 4u : NO_RUN;
+                const int left = p.a_lk - kr;             // elements of the chunk that lie in this run
+                if (AMODE == HS_KRUN) {
+                    const int u0 = (ptid & 3) * 4;
+#pragma unroll
+                    for (int it = 0; it < 2; ++it)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {       // (k step 1: the place within the chunk is part of roff)
+                            const uint32_t base = u0 + e < left ? here : next;
+                            x[it][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_a, roff[it] + base + 4u * e, 0, 0));
+                        }
+                } else {
+                    const uint32_t step = static_cast<uint32_t>(p.a_ki) * 4u;
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
+                        const uint32_t koff = (oct + c < left ? here : next) + static_cast<uint32_t>(oct + c) * step;
+                        x[c >> 2][c & 3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_a, roff[0] + koff, 0, 0));
+                    }
+                }
+            }
+            kr += BK;
+            if (kr >= p.a_lk) { kr -= p.a_lk; ++kd; }
+        };
+        v4f ra[PC_AHEAD][2];
+#pragma unroll
+        for (int d = 0; d < PC_AHEAD; ++d)
+            if (d < nch) load(ra[d]);
+        SplitGuard guard;
+        for (int cg = 0; cg < nch; cg += PC_AHEAD) {
+#pragma unroll
+            for (int d = 0; d < PC_AHEAD; ++d) {
+                const int c = cg + d;
+                if (c >= nch) break;                    // uniform
+                split_store<SMODE>(lds_a[c & 1], ptid, ra[d], guard);
+                if (c + PC_AHEAD < nch) load(ra[d]);
+                __syncthreads();
+            }
+        }
+        __syncthreads();
+        if (guard.fired()) {                            // (every writer writes the same value)
+            if (AMODE == HS_KRUN) { fired_a[(m0 + (ptid >> 2)) >> 5] = 1; fired_a[(m0 + (ptid >> 2) + 64) >> 5] = 1; }
+            else fired_a[(m0 + (ptid & 127)) >> 5] = 1;
+        }
+        return;
+    }
+
+    v16f acc[4];
+    {
+#pragma unroll
+        for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][r] = 0.0f;
+        const size_t b_chunk = static_cast<size_t>(nb_pad) * 32, b_part = b_chunk * chunks;
+        const uint8_t* bfrag = wb + static_cast<size_t>(n0 + wn) * 32 + lane * 16 + c_begin * b_chunk;
+        const int frag_a = j * SPLIT_PITCH + hh * 16;
+        v8bf fb[HS_AHEAD + 1][3];                       // sets that take turns by name (the loop body is written out three times)
+        const auto load_fb = [&](v8bf (&f)[3], int c) {
+#pragma unroll
+            for (int s3 = 0; s3 < 3; ++s3) f[s3] = *reinterpret_cast<const v8bf*>(bfrag + s3 * b_part + c * b_chunk);
+        };
+#pragma unroll
+        for (int d = 0; d < HS_AHEAD; ++d)
+            if (d < nch) load_fb(fb[d], d);
+        __syncthreads();                                // chunk 0 of the tall operand is in LDS
+        for (int cg = 0; cg < nch; cg += HS_AHEAD + 1) {
+#pragma unroll
+            for (int u = 0; u < HS_AHEAD + 1; ++u) {
+                const int c = cg + u;
+                if (c >= nch) break;                    // uniform
+                if (c + HS_AHEAD < nch) load_fb(fb[(u + HS_AHEAD) % (HS_AHEAD + 1)], c + HS_AHEAD);
+                const uint8_t* half = lds_a[c & 1];
+#pragma unroll
+                for (int ti = 0; ti < 4; ++ti) {
+                    v8bf fa[3];
+#pragma unroll
+                    for (int s3 = 0; s3 < 3; ++s3) fa[s3] = *reinterpret_cast<const v8bf*>(half + frag_a + s3 * SPLIT_PLANE + ti * 32 * SPLIT_PITCH);
+#pragma unroll
+                    for (int q = 0; q < 6; ++q)
+                        acc[ti] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[SPLIT_TERMS[q][0]], fb[u][SPLIT_TERMS[q][1]], acc[ti], 0, 0, 0);
+                }
+                __syncthreads();
+            }
+        }
+    }
+
+    // raw sums of this slice: the padded workspace takes every row and column of the tile
+    float* dst = partial + (static_cast<size_t>(slice) * ma_pad + m0 + 4 * hh) * nb_pad + n0 + wn + j;
+#pragma unroll
+    for (int ti = 0; ti < 4; ++ti)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dst[static_cast<size_t>(ti * 32 + 8 * (r >> 2) + (r & 3)) * nb_pad] = acc[ti][r];
+}
+
 // ------------------------------------------------------------------------------------------
 // Batched contractions with a short K (at most 32: the attention logits, K = head dimension) on operands whose
 // rows are contiguous, into dense output planes.  Per output tile there are two 16-k chunks of matrix work and
@@ -1628,6 +1793,74 @@ int f32_arithmetic() {
 // `fixed_ws` / `fixed_cap`: a workspace the caller brings (the static array of the entry point that allocates
 // nothing).  With one, the pool is never touched: a contraction that wants more workspace than `fixed_cap`
 // is refused, one that wants none runs as it always does.
+// gemm_bf16x3_half_split_kernel for a single-plane contraction whose tall operand A has compound indices; -1 when the
+// contraction is not of that kind (the caller goes on to the other forms).  p.tiles_m / p.tiles_n / p.stream_c are set.
+int try_half_split(const GemmParams& p, hipStream_t stream, const char* what) {
+    if (p.a_lm <= 0 || p.np2 * p.np3 != 1 || p.clamp || p.f16_in || !(p.c_lm >= p.M && p.c_ln >= p.N)) return -1;
+    if (p.a_lk < BK || p.K % p.a_lk != 0 || p.tiles_n > 16 || p.tiles_m < 3) return -1;
+    const bool gen = p.a_lk % BK != 0;                  // runs that are not whole chunks (that form: a span of at most 2^30 bytes)
+    const int amode = p.a_ki == 1 ? HS_KRUN : p.a_mi == 1 ? HS_RRUN : -1;
+    if (amode < 0) return -1;
+    // 32-bit byte offsets: the tall operand's span and the dense output below 2 GiB
+    const int64_t a_span = static_cast<int64_t>((p.M - 1) / p.a_lm) * p.a_mo + static_cast<int64_t>(p.a_lm - 1) * p.a_mi +
+                           static_cast<int64_t>((p.K - 1) / p.a_lk) * p.a_ko + static_cast<int64_t>(p.a_lk - 1) * p.a_ki + 1;
+    if (p.a_mo < 0 || p.a_mi < 0 || p.a_ko < 0 || p.a_ki < 0 || a_span * 4 >= (1LL << 31) || (gen && a_span * 4 > (1LL << 30))) return -1;
+    const int chunks = (p.K + BK - 1) / BK;
+    const int groups = p.tiles_m * p.tiles_n, cus = device_cu_count();
+    // K slices until the work-groups come out even over the CUs (a CU's rate does not depend on how many it holds);
+    // a slice is at least PLANES_MIN_SLICE_CHUNKS chunks long
+    int slices = 1;
+    {
+        const int most = chunks / PLANES_MIN_SLICE_CHUNKS < 16 ? chunks / PLANES_MIN_SLICE_CHUNKS : 16;
+        double best = 1e30;
+        for (int sl = 1; sl <= (most > 1 ? most : 1); ++sl) {
+            const int64_t wgs = static_cast<int64_t>(groups) * sl;
+            const double waste = static_cast<double>((wgs + cus - 1) / cus * cus) / static_cast<double>(wgs);
+            if (waste < best - 0.02) { best = waste; slices = sl; }
+        }
+    }
+    const int slice_chunks = (chunks + slices - 1) / slices;
+    slices = (chunks + slice_chunks - 1) / slice_chunks;
+    const int ma_pad = p.tiles_m * BM, nb_pad = p.tiles_n * BN;
+    const size_t b_bytes = static_cast<size_t>(3) * chunks * nb_pad * 32;
+    const size_t part_bytes = static_cast<size_t>(slices) * ma_pad * nb_pad * 4;
+    const int n_flags = ma_pad / 32 + nb_pad / 32;
+    const size_t flag_bytes = (static_cast<size_t>(n_flags) * 4 + 255) / 256 * 256;
+    uint8_t* ws = nullptr;
+    hipMemPool_t pool = workspace_pool();
+    if (!pool || hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), b_bytes + part_bytes + flag_bytes, pool, stream) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    float* partial = reinterpret_cast<float*>(ws + b_bytes);
+    int* fired_a = reinterpret_cast<int*>(ws + b_bytes + part_bytes);
+    int* fired_b = fired_a + ma_pad / 32;
+    GemmParams q = p;
+    q.np2 = slices;                                      // the tile numbering walks the slices as planes
+    const dim3 grid(static_cast<unsigned>(groups * slices)), block(512);
+    hipLaunchKernelGGL(clear_flags_kernel, dim3((n_flags + 255) / 256), dim3(256), 0, stream, fired_a, n_flags);
+    int rc = check_launch(what);
+    const SplitJob jb{p.B, ws, p.N, nb_pad, p.K, chunks, p.b_rs, p.b_ks, 0, 0, 0, 0, 0, 0, fired_b};
+    if (rc == RC_OK) rc = launch_split(jb, stream);
+    if (rc == RC_OK) {
+        const uint32_t span_bytes = static_cast<uint32_t>(a_span * 4);
+#define PPML_HS(AMODE_, GEN_) hipLaunchKernelGGL((gemm_bf16x3_half_split_kernel<AMODE_, GEN_>), grid, block, 0, stream, q, ws, nb_pad, chunks, slice_chunks, \
+                                                 partial, ma_pad, fired_a, span_bytes)
+        if (amode == HS_KRUN) { if (gen) PPML_HS(HS_KRUN, true); else PPML_HS(HS_KRUN, false); }
+        else                  { if (gen) PPML_HS(HS_RRUN, true); else PPML_HS(HS_RRUN, false); }
+#undef PPML_HS
+        rc = check_launch(what);
+    }
+    if (rc == RC_OK) {
+        const int64_t threads = static_cast<int64_t>(p.M) * ((p.N + 3) / 4);
+        hipLaunchKernelGGL((reduce_slices_kernel<false>), dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream, p, partial, slices,
+                           ma_pad, nb_pad, fired_a, fired_b);
+        rc = check_launch(what);
+    }
+    if (hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();
+    return rc;
+}
+
 int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fixed_ws = nullptr, size_t fixed_cap = 0) {
     p.tiles_m = (p.M + BM - 1) / BM;
     p.tiles_n = (p.N + BN - 1) / BN;
@@ -1673,6 +1906,10 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
     }
     const bool planes_fit = slices > 1 ? planes_groups * slices >= PLANES_MIN_GROUPS / 2 && static_cast<int64_t>(p.M) * p.N >= (1 << 20)
                                        : p.tiles_m >= PLANES_MIN_TILES && p.tiles_n >= PLANES_MIN_TILES && planes_groups >= PLANES_MIN_GROUPS;
+    if (!fp32_pipe && !fixed_ws && p.a_lm > 0) {
+        const int rc = try_half_split(p, stream, what);
+        if (rc >= 0) return rc;
+    }
     if (!fp32_pipe && !p.clamp && !p.f16_in && p.np2 * p.np3 == 1 && planes_fit) {
         const int tiles_m = (p.M + PBM - 1) / PBM;
         const int ma_pad = tiles_m * PBM, nb_pad = p.tiles_n * BN;

@@ -741,7 +741,11 @@ def test_tri_mul_back(ops, oracle, D, I, J, K, Bt, outgoing):
     assert none is None and np.array_equal(gr.cpu().numpy(), wr)
 
 
-@pytest.mark.parametrize("D,L,N,Bt", [(3, 4, 8, 2), (16, 40, 64, 1), (4, 103, 37, 1), (32, 64, 512, 1)])   # the last: K slices
+# (3, 4, 8), (8, 48, 64, 2): the generic kernel (a short pair tensor; a batch); the others: the gradient tensor split in
+# the tile loop -- runs of whole 16-k chunks (L a multiple of 16) and of any length (103, 50, 40), ragged rows (2176 =
+# 17 tiles) and columns, two to eight K slices, up to four column tiles
+@pytest.mark.parametrize("D,L,N,Bt", [(3, 4, 8, 2), (16, 40, 64, 1), (4, 103, 37, 1), (32, 64, 512, 1), (8, 48, 64, 1), (8, 272, 200, 1),
+                                      (32, 64, 256, 1), (8, 48, 64, 2), (16, 50, 100, 1), (8, 103, 200, 1)])
 def test_outer_prod_mean_back(ops, oracle, D, L, N, Bt):
     rng = np.random.default_rng(D + L)
     left = rng.standard_normal(D * L * N * Bt).astype(np.float32)
@@ -760,6 +764,80 @@ def test_outer_prod_mean_back(ops, oracle, D, L, N, Bt):
         assert none is None and np.array_equal(gl.cpu().numpy(), wl)
         none, gr = ops.outer_prod_mean_back(_dev(gi), _dev(li), _dev(ri), D, L, N, Bt, want_left=False)
         assert none is None and np.array_equal(gr.cpu().numpy(), wr)
+
+
+@pytest.mark.parametrize("L", [48, 51])
+@pytest.mark.parametrize("kind", ["inf", "tiny"])
+def test_outer_prod_mean_back_carries_what_the_split_cannot(ops, oracle, kind, L):
+    """Non-finite elements of the gradient tensor or of an operand, and elements whose low bits lie below bf16's
+    range (2^-128 against 2^100), at a size where the gradient tensor is split in the tile loop and the K loop is cut
+    into slices: infinities and NaNs stand where the reference's loop puts them (src/backend/CPUKernels.cpp:1034-1105),
+    the small elements keep all their bits, and the other outputs are what they are without them.  L = 51: runs that
+    are not whole 16-k chunks."""
+    D, N = 8, 64
+    rng = np.random.default_rng(11)
+    left = rng.standard_normal(D * L * N).astype(np.float32)
+    right = rng.standard_normal(D * L * N).astype(np.float32)
+    grad = rng.standard_normal(D * D * L * L).astype(np.float32)
+    clean_l, clean_r = (t.cpu().numpy().reshape(D, L, N) for t in ops.outer_prod_mean_back(_dev(grad), _dev(left), _dev(right), D, L, N, 1))
+    g4, l3, r3 = grad.reshape(D, D, L, L), left.reshape(D, L, N), right.reshape(D, L, N)
+    if kind == "inf":
+        g4[5, 3, 7, 9] = np.inf                     # row (d1 = 5, i = 7) of gleft, row (d2 = 3, j = 9) of gright
+        g4[1, 6, 40, 2] = -np.inf
+        r3[2, 11, 5] = np.inf                       # column 5 of gleft
+    else:
+        g4[5, :, 7, :] = (rng.standard_normal((D, L)) * 2.0 ** -128).astype(np.float32)
+        g4[:, 3, :, 9] = (rng.standard_normal((D, L)) * 2.0 ** -128).astype(np.float32)
+        r3[:, :, 5] *= np.float32(2.0 ** 100)
+        l3[:, :, 6] *= np.float32(2.0 ** 100)
+    want_l, want_r = (a.reshape(D, L, N) for a in oracle.outer_prod_mean_back(grad, left, right, D, L, N, 1))
+    got_l, got_r = (t.cpu().numpy().reshape(D, L, N) for t in ops.outer_prod_mean_back(_dev(grad), _dev(left), _dev(right), D, L, N, 1))
+    with np.errstate(invalid="ignore", over="ignore"):
+        abs_l = np.einsum("abij,bjn->ain", np.nan_to_num(np.abs(g4.astype(np.float64)), posinf=0.0), np.nan_to_num(np.abs(r3.astype(np.float64)), posinf=0.0)) / N
+        abs_r = np.einsum("abij,ain->bjn", np.nan_to_num(np.abs(g4.astype(np.float64)), posinf=0.0), np.nan_to_num(np.abs(l3.astype(np.float64)), posinf=0.0)) / N
+    for got, want, absprod in ((got_l, want_l, abs_l), (got_r, want_r, abs_r)):
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(np.isinf(got), np.isinf(want))
+        assert np.array_equal(got[np.isinf(want)], want[np.isinf(want)])
+        fin = np.isfinite(want)
+        assert np.all(np.abs(got[fin].astype(np.float64) - want[fin]) <= 1e-5 * absprod[fin] + 1e-44)
+    if kind == "inf":
+        cols = np.arange(N) != 5                    # (column 5 of gleft meets the infinite element of `right` as well: inf - inf there)
+        assert np.isinf(got_l[5, 7][cols]).all() and np.isinf(got_r[3, 9]).all() and np.isinf(got_l[1, 40][cols]).all() and np.isinf(got_r[6, 2]).all()
+        # tiles of 128 rows / groups of 32 columns that hold none of the planted elements are bit for bit what they were
+        far = np.ones((D * L, N), bool)
+        for m in (5 * L + 7, 1 * L + 40):
+            far[(m // 128) * 128:(m // 128 + 1) * 128] = False
+        far[:, 0:32] = False
+        assert np.array_equal(got_l.reshape(D * L, N)[far].view(np.int32), clean_l.reshape(D * L, N)[far].view(np.int32))
+        far = np.ones((D * L, N), bool)
+        for m in (3 * L + 9, 6 * L + 2):
+            far[(m // 32) * 32:(m // 32 + 1) * 32] = False
+        assert np.array_equal(got_r.reshape(D * L, N)[far].view(np.int32), clean_r.reshape(D * L, N)[far].view(np.int32))
+    else:
+        assert got_l[5, 7, 5] != 0.0 and got_r[3, 9, 6] != 0.0
+
+
+def test_outer_prod_mean_back_configured_size_sampled_rows(ops):
+    """D = 32, L = 384, N = 256 (12288 x 12288 gradient elements against 256 columns, the size bench.py times): rows of
+    both gradients against float64 sums of the same operands, within (K + 2) * 2^-24 * sum|a||b|."""
+    D, L, N = 32, 384, 256
+    torch.manual_seed(5)
+    grad = torch.randn(D * D * L * L, device="cuda")
+    left = torch.randn(D * L * N, device="cuda")
+    right = torch.randn(D * L * N, device="cuda")
+    gl, gr = ops.outer_prod_mean_back(grad, left, right, D, L, N, 1)
+    g4 = grad.view(D, D, L, L)
+    K = D * L
+    for (d, i) in ((0, 0), (7, 133), (31, 383), (16, 200)):
+        a = g4[d, :, i, :].reshape(-1).double()                     # k = (d2, j)
+        want = (a[:, None] * right.view(K, N).double()).sum(0) / N
+        bound = (a.abs()[:, None] * right.view(K, N).double().abs()).sum(0) / N * (K + 2) * 2.0 ** -24
+        assert bool(((gl.view(D, L, N)[d, i].double() - want).abs() <= bound).all())
+        a = g4[:, d, :, i].reshape(-1).double()                     # k = (d1, i)
+        want = (a[:, None] * left.view(K, N).double()).sum(0) / N
+        bound = (a.abs()[:, None] * left.view(K, N).double().abs()).sum(0) / N * (K + 2) * 2.0 ** -24
+        assert bool(((gr.view(D, L, N)[d, i].double() - want).abs() <= bound).all())
 
 
 @pytest.mark.parametrize("planes,Lq,Lk,D", [(3, 20, 20, 16), (7, 51, 51, 32), (412, 103, 103, 32), (60, 256, 256, 32), (5, 70, 33, 8)])
