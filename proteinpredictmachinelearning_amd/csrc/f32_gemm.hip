@@ -850,6 +850,112 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_kernel(const GemmParams p)
     }
 }
 
+// gemm_bf16x3_pc_kernel for a few output tiles under a long K (a LinearLayer's weight gradient: 256 x 768 outputs over
+// 26368 tokens -- twelve tiles): the K loop is cut into slices, one work-group per (tile, slice) -- the tile numbering
+// takes the slice for the plane --, raw sums go to partial[slice][m][n] and reduce_slices_kernel adds them in slice
+// order, applies bias, factor and the output's addressing.  A slice whose split could not carry an operand flags the
+// tile's rows (fired_a, one per 32 rows) and reduce_slices_kernel computes those the reference's way.
+template <int MODE, bool K4>
+__global__ __launch_bounds__(512) void gemm_bf16x3_pc_slices_kernel(const GemmParams p, int chunks, int slice_chunks, float* __restrict__ partial,
+                                                                    int ma_pad, int nb_pad, int* __restrict__ fired_a) {
+    static_assert(MODE == LOAD_ROW_CONTIG || MODE == LOAD_K_CONTIG, "buffer addressing");
+    constexpr int STAGE = 3 * SPLIT_PLANE;
+    __shared__ __attribute__((aligned(16))) uint8_t lds_ab[2][2 * STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const bool producer = wave >= 4;
+    const int ptid = tid & 255;
+    const int cw = wave & 3;
+    const int wm = (cw >> 1) * 64, wn = (cw & 1) * 64;
+
+    int slice, m0, n0;
+    tile_of_group(p, slice, m0, n0);
+    const int c_begin = slice * slice_chunks;
+    const int c_end = c_begin + slice_chunks < chunks ? c_begin + slice_chunks : chunks;
+    const int nch = c_end - c_begin;
+
+    const int64_t a_plane = MODE == LOAD_K_CONTIG ? (p.M - 1) * p.a_rs + p.K : p.K * p.a_ks;
+    const int64_t b_plane = MODE == LOAD_K_CONTIG ? (p.N - 1) * p.b_rs + p.K : p.K * p.b_ks;
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.A), 0, static_cast<int>(a_plane * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.B), 0, static_cast<int>(b_plane * 4), 0x00020000);
+
+    // (barriers: nch + 1 in either loop, as in gemm_bf16x3_pc_kernel)
+    if (producer) {
+        v4f ra[PC_AHEAD][2], rb[PC_AHEAD][2];
+        const auto load_both = [&](int c, v4f (&xa)[2], v4f (&xb)[2]) {
+            if (MODE == LOAD_K_CONTIG) {
+                load_kcontig_buffer<K4>(rsrc_a, static_cast<uint32_t>(p.a_rs) * 4u, m0, p.M, c * BK, p.K, ptid, xa);
+                load_kcontig_buffer<K4>(rsrc_b, static_cast<uint32_t>(p.b_rs) * 4u, n0, p.N, c * BK, p.K, ptid, xb);
+            } else {
+                load_rows8_buffer(rsrc_a, static_cast<uint32_t>(p.a_ks) * 4u, m0, p.M, c * BK, ptid, xa);
+                load_rows8_buffer(rsrc_b, static_cast<uint32_t>(p.b_ks) * 4u, n0, p.N, c * BK, ptid, xb);
+            }
+        };
+#pragma unroll
+        for (int d = 0; d < PC_AHEAD; ++d)
+            if (d < nch) load_both(c_begin + d, ra[d], rb[d]);
+        SplitGuard guard;
+        for (int cg = 0; cg < nch; cg += PC_AHEAD) {
+#pragma unroll
+            for (int d = 0; d < PC_AHEAD; ++d) {
+                const int c = cg + d;
+                if (c >= nch) break;                    // uniform
+                uint8_t* half = lds_ab[c & 1];
+                split_store<MODE>(half, ptid, ra[d], guard);
+                split_store<MODE>(half + STAGE, ptid, rb[d], guard);
+                if (c + PC_AHEAD < nch) load_both(c_begin + c + PC_AHEAD, ra[d], rb[d]);
+                __syncthreads();
+            }
+        }
+        __syncthreads();
+        if (guard.fired()) {                            // (either operand: the tile's rows; every writer writes the same value)
+#pragma unroll
+            for (int i = 0; i < BM / 32; ++i) fired_a[(m0 >> 5) + i] = 1;
+        }
+        return;
+    }
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
+    const int frag_a = (wm + j) * SPLIT_PITCH + hh * 16;
+    const int frag_b = STAGE + (wn + j) * SPLIT_PITCH + hh * 16;
+    __syncthreads();                                    // chunk 0 is in LDS
+    for (int c = 0; c < nch; ++c) {
+        const uint8_t* half = lds_ab[c & 1];
+        v8bf fa[2][3], fb[2][3];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s3 = 0; s3 < 3; ++s3) {
+                fa[t][s3] = *reinterpret_cast<const v8bf*>(half + frag_a + s3 * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
+                fb[t][s3] = *reinterpret_cast<const v8bf*>(half + frag_b + s3 * SPLIT_PLANE + t * 32 * SPLIT_PITCH);
+            }
+#pragma unroll
+        for (int q = 0; q < 6; ++q)
+#pragma unroll
+            for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < 2; ++tj)
+                    acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][SPLIT_TERMS[q][0]], fb[tj][SPLIT_TERMS[q][1]], acc[ti][tj], 0, 0, 0);
+        __syncthreads();                                // chunk c has been read; chunk c + 1 is in LDS
+    }
+    // raw sums of this slice: the padded workspace takes every row and column of the tile
+    float* dst = partial + (static_cast<size_t>(slice) * ma_pad + m0 + wm + 4 * hh) * nb_pad + n0 + wn + j;
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dst[static_cast<size_t>(ti * 32 + 8 * (r >> 2) + (r & 3)) * nb_pad + tj * 32] = acc[ti][tj][r];
+}
+
 // The same again for contractions with one NARROW side: at most 32 rows of A (SIDE_M: the second contraction of the
 // attention chain, out_prod_tt_hip with the head dimension for its rows) or of B (SIDE_N: a LinearLayer with up to 32
 // output features -- the bias projections onto the heads, the 256 -> 16 projections of the outer-product-mean).  A 128 x
@@ -1793,6 +1899,22 @@ int f32_arithmetic() {
 // `fixed_ws` / `fixed_cap`: a workspace the caller brings (the static array of the entry point that allocates
 // nothing).  With one, the pool is never touched: a contraction that wants more workspace than `fixed_cap`
 // is refused, one that wants none runs as it always does.
+// How many K slices make `groups` output tiles come out even over the CUs (a CU's rate does not depend on how many
+// work-groups it holds): the smallest count within 2 % of the best, slices of at least PLANES_MIN_SLICE_CHUNKS chunks.
+int even_slices(int groups, int chunks, int most_slices) {
+    const int cus = device_cu_count();
+    int most = chunks / PLANES_MIN_SLICE_CHUNKS < most_slices ? chunks / PLANES_MIN_SLICE_CHUNKS : most_slices;
+    if (most < 1) most = 1;
+    int slices = 1;
+    double best = 1e30;
+    for (int sl = 1; sl <= most; ++sl) {
+        const int64_t wgs = static_cast<int64_t>(groups) * sl;
+        const double waste = static_cast<double>((wgs + cus - 1) / cus * cus) / static_cast<double>(wgs);
+        if (waste < best - 0.02) { best = waste; slices = sl; }
+    }
+    return slices;
+}
+
 // gemm_bf16x3_half_split_kernel for a single-plane contraction whose tall operand A has compound indices; -1 when the
 // contraction is not of that kind (the caller goes on to the other forms).  p.tiles_m / p.tiles_n / p.stream_c are set.
 int try_half_split(const GemmParams& p, hipStream_t stream, const char* what) {
@@ -1806,19 +1928,8 @@ int try_half_split(const GemmParams& p, hipStream_t stream, const char* what) {
                            static_cast<int64_t>((p.K - 1) / p.a_lk) * p.a_ko + static_cast<int64_t>(p.a_lk - 1) * p.a_ki + 1;
     if (p.a_mo < 0 || p.a_mi < 0 || p.a_ko < 0 || p.a_ki < 0 || a_span * 4 >= (1LL << 31) || (gen && a_span * 4 > (1LL << 30))) return -1;
     const int chunks = (p.K + BK - 1) / BK;
-    const int groups = p.tiles_m * p.tiles_n, cus = device_cu_count();
-    // K slices until the work-groups come out even over the CUs (a CU's rate does not depend on how many it holds);
-    // a slice is at least PLANES_MIN_SLICE_CHUNKS chunks long
-    int slices = 1;
-    {
-        const int most = chunks / PLANES_MIN_SLICE_CHUNKS < 16 ? chunks / PLANES_MIN_SLICE_CHUNKS : 16;
-        double best = 1e30;
-        for (int sl = 1; sl <= (most > 1 ? most : 1); ++sl) {
-            const int64_t wgs = static_cast<int64_t>(groups) * sl;
-            const double waste = static_cast<double>((wgs + cus - 1) / cus * cus) / static_cast<double>(wgs);
-            if (waste < best - 0.02) { best = waste; slices = sl; }
-        }
-    }
+    const int groups = p.tiles_m * p.tiles_n;
+    int slices = even_slices(groups, chunks, 16);
     const int slice_chunks = (chunks + slices - 1) / slices;
     slices = (chunks + slice_chunks - 1) / slice_chunks;
     const int ma_pad = p.tiles_m * BM, nb_pad = p.tiles_n * BN;
@@ -1859,6 +1970,60 @@ int try_half_split(const GemmParams& p, hipStream_t stream, const char* what) {
     }
     if (hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();
     return rc;
+}
+
+// gemm_bf16x3_pc_slices_kernel for a single dense plane with few output tiles under a long K; -1 when the contraction
+// is not of that kind or no workspace is to be had (the caller goes on to the unsliced forms).
+template <int MODE>
+int try_pc_slices(const GemmParams& p, hipStream_t stream, const char* what) {
+    const int chunks = (p.K + BK - 1) / BK;
+    const int groups = p.tiles_m * p.tiles_n;
+    // (three launches and a workspace: about 28 us before the first chunk; measured even with the unsliced form at K = 515
+    // on one tile (23 against 33 us), ahead of it at K = 1000 on nine tiles (32 against 41))
+    if (p.np2 * p.np3 != 1 || groups * 2 > device_cu_count() || chunks < 3 * PLANES_MIN_SLICE_CHUNKS) return -1;
+    int slices = even_slices(groups, chunks, 128);
+    if (slices < 2) return -1;
+    const int slice_chunks = (chunks + slices - 1) / slices;
+    slices = (chunks + slice_chunks - 1) / slice_chunks;
+    const int ma_pad = p.tiles_m * BM, nb_pad = p.tiles_n * BN;
+    const size_t part_bytes = static_cast<size_t>(slices) * ma_pad * nb_pad * 4;
+    const int n_flags = ma_pad / 32 + nb_pad / 32;
+    const size_t flag_bytes = (static_cast<size_t>(n_flags) * 4 + 255) / 256 * 256;
+    uint8_t* ws = nullptr;
+    hipMemPool_t pool = workspace_pool();
+    if (!pool || hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), part_bytes + flag_bytes, pool, stream) != hipSuccess) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    float* partial = reinterpret_cast<float*>(ws);
+    int* fired_a = reinterpret_cast<int*>(ws + part_bytes);
+    int* fired_b = fired_a + ma_pad / 32;               // (stays clear: the kernel flags rows for either operand)
+    GemmParams q = p;
+    q.np2 = slices;                                      // the tile numbering walks the slices as planes
+    const dim3 grid(static_cast<unsigned>(groups * slices)), block(512);
+    hipLaunchKernelGGL(clear_flags_kernel, dim3((n_flags + 255) / 256), dim3(256), 0, stream, fired_a, n_flags);
+    int rc = check_launch(what);
+    if (rc == RC_OK) {
+        if (MODE == LOAD_K_CONTIG && p.K % 4 != 0)
+            hipLaunchKernelGGL((gemm_bf16x3_pc_slices_kernel<MODE, false>), grid, block, 0, stream, q, chunks, slice_chunks, partial, ma_pad, nb_pad, fired_a);
+        else
+            hipLaunchKernelGGL((gemm_bf16x3_pc_slices_kernel<MODE, true>), grid, block, 0, stream, q, chunks, slice_chunks, partial, ma_pad, nb_pad, fired_a);
+        rc = check_launch(what);
+    }
+    if (rc == RC_OK) {
+        const int64_t threads = static_cast<int64_t>(p.M) * ((p.N + 3) / 4);
+        hipLaunchKernelGGL((reduce_slices_kernel<false>), dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream, p, partial, slices,
+                           ma_pad, nb_pad, fired_a, fired_b);
+        rc = check_launch(what);
+    }
+    if (hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();
+    return rc;
+}
+
+template <int MODE>
+bool try_pc_slices_done(const GemmParams& p, hipStream_t stream, const char* what, int& rc) {
+    rc = try_pc_slices<MODE>(p, stream, what);
+    return rc >= 0;
 }
 
 int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fixed_ws = nullptr, size_t fixed_cap = 0) {
@@ -2026,6 +2191,10 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
                 return check_launch(what);
             }
         }
+        if (!fixed_ws) {
+            const int rc = try_pc_slices<LOAD_ROW_CONTIG>(p, stream, what);
+            if (rc >= 0) return rc;
+        }
         if (two_sets) {
             if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_pc_kernel<LOAD_ROW_CONTIG, true, true>), grid, dim3(512), 0, stream, p);
             else hipLaunchKernelGGL((gemm_bf16x3_pc_kernel<LOAD_ROW_CONTIG, false, true>), grid, dim3(512), 0, stream, p);
@@ -2036,9 +2205,12 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
     else if (!p.clamp && !p.f16_in) {
         // binary32 operands without the finite guard: the contraction runs on the bf16 matrix pipe
         // rows contiguous in k, dense output planes, every plane below 2 GiB: buffer addressing (see load_kcontig_buffer)
+        int slices_rc = -1;
         const bool k_fast = mode == LOAD_K_CONTIG && !split && p.c_ni == 1 && p.a_lm == 0 &&
                             ((p.M - 1) * p.a_rs + p.K) * 4 < (1LL << 31) && ((p.N - 1) * p.b_rs + p.K) * 4 < (1LL << 31) &&
                             p.M * p.c_mi * 4 < (1LL << 31) && p.c_mi < (1 << 22) && p.a_rs < (1 << 22) && p.b_rs < (1 << 22);
+        // few tiles under a long K (a LinearLayer's weight gradient) go in K slices, whatever their width
+        if (k_fast && !fixed_ws && try_pc_slices_done<LOAD_K_CONTIG>(p, stream, what, slices_rc)) return slices_rc;
         if (k_fast && p.K > 3 * BK && (p.N <= 32 || p.M <= 32)) {
             // one narrow side: tiles of 128 x 32 along the other (gemm_bf16x3_pc_narrow_kernel)
             const bool side_n = p.N <= 32;

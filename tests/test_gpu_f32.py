@@ -766,6 +766,41 @@ def test_outer_prod_mean_back(ops, oracle, D, L, N, Bt):
         assert none is None and np.array_equal(gr.cpu().numpy(), wr)
 
 
+@pytest.mark.parametrize("T,K,N", [(26368, 256, 768), (10609, 128, 512), (5000, 100, 130), (3001, 33, 7), (1000, 300, 300), (26368, 256, 16)])
+def test_weight_gradients_of_linear_layers_go_in_k_slices(ops, oracle, T, K, N):
+    """dW = X^T dY of a LinearLayer (src/core/ComputeGraph.cpp:708-773: `mat_transpose` of both, then `mul_mat`): a few
+    output tiles under a contraction as long as the token count.  Both formulations -- on the operands as they lie
+    (mul_mat_tn) and on the transposed copies (mul_mat) -- are cut into the same K slices and give the same bits;
+    against float64 within (T + 2) * 2^-24 * sum|a||b|; a non-finite or sub-range element ends where the reference's
+    loop puts it."""
+    torch.manual_seed(T + N)
+    x = torch.randn(T, K, device="cuda")
+    dy = torch.randn(T, N, device="cuda")
+    got = ops.mul_mat_tn(x, dy)
+    want = x.double().t() @ dy.double()
+    bound = (x.double().abs().t() @ dy.double().abs()) * (T + 2) * 2.0 ** -24
+    assert bool(((got.double() - want).abs() <= bound).all())
+    xt, dyt = x.t().contiguous(), dy.t().contiguous()
+    copies = ops.mul_mat(xt, dyt)
+    assert torch.equal(got.view(torch.int32), copies.view(torch.int32))
+    if T <= 5000:
+        ref = oracle.mul_mat_f32(xt.cpu().numpy(), dyt.cpu().numpy())
+        np.testing.assert_allclose(got.cpu().numpy(), ref, rtol=0, atol=float(bound.max()))
+        x2, dy2 = x.clone(), dy.clone()
+        x2[T // 3, 5] = float("inf")
+        x2[T // 2, 9] = 3e-41
+        dy2[T - 1, N - 1] = -float("inf")
+        dy2[7, 2] = 1e-44
+        got2 = ops.mul_mat_tn(x2, dy2).cpu().numpy()
+        with np.errstate(invalid="ignore", over="ignore"):
+            ref2 = oracle.mul_mat_f32(x2.t().contiguous().cpu().numpy(), dy2.t().contiguous().cpu().numpy())
+        assert np.array_equal(np.isnan(got2), np.isnan(ref2)) and np.array_equal(np.isinf(got2), np.isinf(ref2))
+        assert np.array_equal(got2[np.isinf(ref2)], ref2[np.isinf(ref2)])
+        fin = np.isfinite(ref2)
+        assert np.all(np.abs(got2[fin].astype(np.float64) - ref2[fin]) <= bound.cpu().numpy()[fin] * 2 + 1e-30)
+        assert np.isinf(got2[5, :N - 1]).all() and np.isinf(np.delete(got2[:, N - 1], 5)).all()      # (where the two meet: inf - inf)
+
+
 @pytest.mark.parametrize("L", [48, 51])
 @pytest.mark.parametrize("kind", ["inf", "tiny"])
 def test_outer_prod_mean_back_carries_what_the_split_cannot(ops, oracle, kind, L):

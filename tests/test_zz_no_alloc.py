@@ -45,7 +45,9 @@ def test_no_alloc_entry_point_matches_the_allocating_one_on_calls_in_a_row():
             assert _call(lib.mul_mat_tn_noalloc_hip, a, b, got, M, K, N, 1.0 / K) == 0, cabi.last_error()
     torch.cuda.synchronize()
     free_after, _total = torch.cuda.mem_get_info()
-    assert free_after == free_before, "device memory changed hands during calls that must not allocate"
+    # (free memory may grow meanwhile -- the runtime hands back what earlier tests of this process let go of --, but a
+    # call that allocates would shrink it)
+    assert free_after >= free_before, "device memory was taken during calls that must not allocate"
     for M, K, N, a, b, want, got in cases:
         assert torch.equal(got, want), (M, K, N)
         # and the result is the contraction: a sample against float64
