@@ -9,7 +9,7 @@
 // dst[j0,j1,j2,j3] = sum over k0 < r0, k1 < r1, k2 < r2, k3 < r3 of src[j0 + k0*d0, j1 + k1*d1, j2 + k2*d2, j3 + k3*d3]
 // with dimension 0 innermost in both tensors.  The reference adds the terms one at a time with k3 running
 // fastest; here the same sequence is cut into `slices` consecutive runs that are summed side by side and then
-// added in run order, so the result is a fixed function of the shapes (no atomics), equal to the reference's
+// added in a fixed pattern, so the result is a fixed function of the shapes (no atomics), equal to the reference's
 // up to the rounding of a differently bracketed binary32 sum.
 #include "common.hpp"
 
@@ -25,14 +25,18 @@ struct RepeatBackJob {
     int64_t total;                   // d0 * d1 * d2 * d3
     int64_t reps;                    // r0 * r1 * r2 * r3
     int64_t per_slice;               // terms per run
+    int64_t slices;                  // runs (1: `out` is dst itself)
 };
 
-// One thread per (destination element, run).  Neighbouring threads hold neighbouring j0, so for every term
-// a wave reads one contiguous stretch of the source.
+// One thread per (run, destination element), the element fastest.  Neighbouring threads hold neighbouring j0, so for
+// every term a wave reads one contiguous stretch of the source.  The terms are requested eight at a time and added in their
+// order (one load in flight per wave had a bias gradient of 26368 x 768 wait 104 us for 81 MB); the element's place
+// moves from term to term by the strides of the four copy counters, no product per term.
 __global__ __launch_bounds__(256) void repeat_back_kernel(const RepeatBackJob jb) {
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (idx >= jb.total) return;
-    const int64_t slice = blockIdx.y;
+    const int64_t gidx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (gidx >= jb.total * jb.slices) return;
+    const int64_t slice = gidx / jb.total;
+    const int64_t idx = gidx - slice * jb.total;
     int64_t t = idx;
     const int64_t j0 = t % jb.d0; t /= jb.d0;
     const int64_t j1 = t % jb.d1; t /= jb.d1;
@@ -46,28 +50,48 @@ __global__ __launch_bounds__(256) void repeat_back_kernel(const RepeatBackJob jb
     int64_t k2 = q % jb.r2; q /= jb.r2;
     int64_t k1 = q % jb.r1; q /= jb.r1;
     int64_t k0 = q;
-    float sum = 0.0f;
-    for (int64_t term = begin; term < end; ++term) {
-        const int64_t i0 = j0 + k0 * jb.d0, i1 = j1 + k1 * jb.d1, i2 = j2 + k2 * jb.d2, i3 = j3 + k3 * jb.d3;
-        sum += jb.src[((i3 * jb.s2 + i2) * jb.s1 + i1) * jb.s0 + i0];
+    // a step of each counter in elements of the source, and what its wrap takes back
+    const int64_t st0 = jb.d0, st1 = jb.d1 * jb.s0, st2 = jb.d2 * jb.s1 * jb.s0, st3 = jb.d3 * jb.s2 * jb.s1 * jb.s0;
+    const int64_t back3 = jb.r3 * st3, back2 = jb.r2 * st2, back1 = jb.r1 * st1;
+    const float* at = jb.src + (((j3 + k3 * jb.d3) * jb.s2 + (j2 + k2 * jb.d2)) * jb.s1 + (j1 + k1 * jb.d1)) * jb.s0 + (j0 + k0 * jb.d0);
+    const auto step = [&]() {
+        at += st3;
         if (++k3 == jb.r3) {
-            k3 = 0;
+            k3 = 0; at += st2 - back3;
             if (++k2 == jb.r2) {
-                k2 = 0;
-                if (++k1 == jb.r1) { k1 = 0; ++k0; }
+                k2 = 0; at += st1 - back2;
+                if (++k1 == jb.r1) { k1 = 0; at += st0 - back1; }
             }
         }
+    };
+    float sum = 0.0f;
+    int64_t term = begin;
+    for (; term + 8 <= end; term += 8) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { v[i] = *at; step(); }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += v[i];
     }
-    jb.out[slice * jb.total + idx] = sum;
+    for (; term < end; ++term) { sum += *at; step(); }
+    jb.out[idx * jb.slices + slice] = sum;              // an element's runs side by side, for the wave that adds them
 }
 
+// The runs of one destination element, added by one wave: lane l takes runs l, l + 64, ... in their order, then the
+// lanes' sums meet in a fixed butterfly -- a fixed function of the shapes, like everything else here.  (One thread
+// per element walking its runs one load at a time took longer than the sums themselves: 341 runs for a bias
+// gradient of 768 elements.)
 __global__ __launch_bounds__(256) void repeat_back_fold_kernel(const float* __restrict__ partial, float* __restrict__ dst,
                                                                int64_t total, int slices) {
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-    if (idx >= total) return;
-    float sum = partial[idx];
-    for (int s = 1; s < slices; ++s) sum += partial[static_cast<int64_t>(s) * total + idx];
-    dst[idx] = sum;
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * 4 + (threadIdx.x >> 6);
+    if (idx >= total) return;                           // wave-uniform
+    const int lane = threadIdx.x & 63;
+    const float* runs = partial + idx * slices;
+    float sum = 0.0f;
+    for (int s = lane; s < slices; s += 64) sum += runs[s];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) sum += __shfl_xor(sum, d, 64);
+    if (lane == 0) dst[idx] = sum;
 }
 
 }  // namespace
@@ -105,9 +129,9 @@ extern "C" int repeat_back_hip(const float* src, float* dst,
     const int64_t blocks = (jb.total + 255) / 256;
     if (blocks > 0x7fffffffLL) { set_error("repeat_back_hip: destination too large"); return RC_BAD_ARGS; }
     // Few destination elements and many copies (a bias gradient: 768 sums of 26368 terms) would leave most of
-    // the chip idle: cut the sum into runs until about eight waves per CU have work, at least 32 terms a run.
+    // the chip idle: cut the sum into runs until about sixteen waves per CU have work, at least 32 terms a run.
     int64_t slices = 1;
-    const int64_t want_threads = 256LL * 8 * 64;
+    const int64_t want_threads = 256LL * 16 * 64;
     if (jb.total < want_threads && jb.reps >= 64) {
         slices = (want_threads + jb.total - 1) / jb.total;
         if (slices > jb.reps / 32) slices = jb.reps / 32;
@@ -116,6 +140,7 @@ extern "C" int repeat_back_hip(const float* src, float* dst,
     }
     jb.per_slice = (jb.reps + slices - 1) / slices;
     slices = (jb.reps + jb.per_slice - 1) / jb.per_slice;
+    if (slices > 0x7fffffff / 256 || (jb.total * slices + 255) / 256 > 0x7fffffffLL) { set_error("repeat_back_hip: destination too large"); return RC_BAD_ARGS; }
     float* partial = nullptr;
     if (slices > 1) {
         hipMemPool_t pool = workspace_pool();
@@ -127,11 +152,12 @@ extern "C" int repeat_back_hip(const float* src, float* dst,
         }
     }
     jb.out = partial ? partial : dst;
-    hipLaunchKernelGGL(repeat_back_kernel, dim3(static_cast<unsigned>(blocks), static_cast<unsigned>(slices)), dim3(256), 0, s, jb);
+    jb.slices = slices;
+    hipLaunchKernelGGL(repeat_back_kernel, dim3(static_cast<unsigned>((jb.total * slices + 255) / 256)), dim3(256), 0, s, jb);
     int rc = check_launch("repeat_back_kernel");
     if (partial) {
         if (rc == RC_OK) {
-            hipLaunchKernelGGL(repeat_back_fold_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, s, partial, dst, jb.total,
+            hipLaunchKernelGGL(repeat_back_fold_kernel, dim3(static_cast<unsigned>((jb.total + 3) / 4)), dim3(256), 0, s, partial, dst, jb.total,
                                static_cast<int>(slices));
             rc = check_launch("repeat_back_fold_kernel");
         }
