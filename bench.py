@@ -490,6 +490,26 @@ def main() -> int:
         steps, warm = 20, 5
         f32_case(opm_back, (2 * 12288 * 12288 + 4 * 12288 * 256) * 4, 4.0 * 12288 * 12288 * 256,
                  "opm_backward_D32_L384_N256", pipe="bf16x3")
+
+        def weight_grad():
+            # dW = X^T dY of the headline projection's f32 twin (src/core/ComputeGraph.cpp:708-773): 256 x 768 outputs,
+            # contraction over the 26368 tokens, cut into K slices
+            ns = 3
+            xs = [torch.randn(26368, 256, device=dev, generator=gen) for _ in range(ns)]
+            dys = [torch.randn(26368, 768, device=dev, generator=gen) for _ in range(ns)]
+            keep.append((xs, dys))
+            return (lambda i: ops.mul_mat_tn(xs[i], dys[i])), ns
+        steps, warm = 50, 10
+        f32_case(weight_grad, (26368 * 256 + 26368 * 768 + 256 * 768) * 4, 2.0 * 26368 * 256 * 768,
+                 "linear_weight_gradient_26368x256_768", pipe="bf16x3")
+
+        def bias_grad():
+            # dbias[n] = sum over the tokens of dY[token][n] (OP_REPEAT_BACK, src/backend/CPUKernels.cpp:2091-2148)
+            ns = 6
+            dys = [torch.randn(26368, 768, device=dev, generator=gen) for _ in range(ns)]
+            keep.append(dys)
+            return (lambda i: ops.repeat_back(dys[i], (768,))), ns
+        f32_case(bias_grad, (26368 * 768 + 768) * 4, 0.0, "linear_bias_gradient_26368x768")
         out["extra"] = extra
 
     if args.copy_calibration:

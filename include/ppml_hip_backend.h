@@ -84,6 +84,11 @@ void ppml_hip_backend_set_fuse_attention_chain(ppml_hip_backend *b, int on);
  *     same bits, two copies less. */
 void ppml_hip_backend_set_fuse_add_into_soft_max(ppml_hip_backend *b, int on);
 void ppml_hip_backend_set_fuse_permutes_into_out_prod(ppml_hip_backend *b, int on);
+/*   permutes_into_mul_mat (default 1): an F32 OP_MUL_MAT without bias whose operands are both matrix transpositions
+ *     nobody else reads -- the weight gradient of a LinearLayer, mul_mat(mat_transpose(grad), mat_transpose(x)),
+ *     src/core/ComputeGraph.cpp:733-738 -- contracts the untransposed matrices over their rows; same bits, and the
+ *     copies of the activations and of their gradient are not made. */
+void ppml_hip_backend_set_fuse_permutes_into_mul_mat(ppml_hip_backend *b, int on);
 /* how many nodes the last graph_compute folded into a neighbour and did not execute */
 int ppml_hip_backend_nodes_fused_away(const ppml_hip_backend *b);
 /* Matrix pipe of this backend's f32 contractions for the length of each graph_compute: 0 = bf16 pipe through

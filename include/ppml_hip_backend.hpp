@@ -185,6 +185,13 @@ public:
     bool fuse_add_into_soft_max() const { return fuse_add_into_soft_max_; }
     void set_fuse_permutes_into_out_prod(bool v) { fuse_permutes_into_out_prod_ = v; }
     bool fuse_permutes_into_out_prod() const { return fuse_permutes_into_out_prod_; }
+    // The same for the weight gradient of a LinearLayer, dW = mul_mat(mat_transpose(grad), mat_transpose(x))
+    // (src/core/ComputeGraph.cpp:733-738): an F32 OP_MUL_MAT without bias both of whose operands are matrix
+    // transpositions nobody else reads contracts the untransposed matrices over their rows (mul_mat_tn_hip); the two
+    // copies -- of the activations and of their gradient, the largest tensors of the backward pass -- are not made.
+    // ON by default; same bits as the nodes run one by one.
+    void set_fuse_permutes_into_mul_mat(bool v) { fuse_permutes_into_mul_mat_ = v; }
+    bool fuse_permutes_into_mul_mat() const { return fuse_permutes_into_mul_mat_; }
     // Off by default.  On: the reference's default attention chain (src/modules/Attention.cpp:264-281)
     //   out_prod(K, Q) -> scale -> [add bias] -> softmax -> permute{1,0,2,3} ; permute{1,0,2,3}(V) -> out_prod
     // whose intermediates have no other reader runs as one fused attention launch on the graph's own layouts
@@ -240,12 +247,14 @@ private:
     bool fuse_attention_chain_ = false;
     bool fuse_add_into_soft_max_ = true;
     bool fuse_permutes_into_out_prod_ = true;
+    bool fuse_permutes_into_mul_mat_ = true;
     size_t nodes_fused_away_ = 0;
     int attn_layout_ = 0;                                // layout bits of the attention node being dispatched
     bool relu_in_quantizer_ = false;                     // the matmul being dispatched applies a fused-away ReLU
     float out_prod_alpha_ = 1.0f;                        // scale of a fused-away OP_SCALE behind the out_prod being dispatched
     bool out_prod_scaled_ = false;
     bool out_prod_transposed_ = false;                   // the out_prod being dispatched reads the sources of two fused-away permutations
+    bool mul_mat_transposed_ = false;                    // the same for the mul_mat being dispatched
     const Tensor* soft_max_bias_ = nullptr;              // second operand of a fused-away OP_ADD in front of the softmax being dispatched
     std::string error_;
     std::vector<std::unique_ptr<Buffer>> owned_;         // node outputs allocated here, packed weights

@@ -127,6 +127,11 @@ class Backend:
         """On by default: an OP_OUT_PROD of two {1,0,2,3} permutations nobody else reads contracts the unpermuted tensors."""
         self._lib.ppml_hip_backend_set_fuse_permutes_into_out_prod(self.handle, int(on))
 
+    def set_fuse_permutes_into_mul_mat(self, on: bool) -> None:
+        """On by default: an F32 OP_MUL_MAT of two matrix transpositions nobody else reads (a LinearLayer's weight
+        gradient) contracts the untransposed matrices over their rows."""
+        self._lib.ppml_hip_backend_set_fuse_permutes_into_mul_mat(self.handle, int(on))
+
     def set_fuse_attention_chain(self, on: bool) -> None:
         self._lib.ppml_hip_backend_set_fuse_attention_chain(self.handle, int(on))
 

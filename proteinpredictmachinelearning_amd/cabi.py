@@ -93,6 +93,7 @@ BACKEND_SIGNATURES = {
     "ppml_hip_backend_set_fuse_scale_into_out_prod": (None, [_vp, _i]),
     "ppml_hip_backend_set_fuse_add_into_soft_max": (None, [_vp, _i]),
     "ppml_hip_backend_set_fuse_permutes_into_out_prod": (None, [_vp, _i]),
+    "ppml_hip_backend_set_fuse_permutes_into_mul_mat": (None, [_vp, _i]),
     "ppml_hip_backend_set_fuse_attention_chain": (None, [_vp, _i]),
     "ppml_hip_backend_nodes_fused_away": (_i, [_vp]),
     "ppml_hip_backend_set_f32_arithmetic": (None, [_vp, _i]),
@@ -149,6 +150,12 @@ def load() -> C.CDLL:
         raise ImportError(
             f"{LIB_PATH} is missing: build it with `make -C proteinpredictmachinelearning_amd/csrc` "
             "(or __graft_entry__.build()); this backend has no CPU fallback")
+    # A process holds one HIP runtime: the first one loaded.  PyTorch ships its own and does not find the GPU through
+    # another, so where PyTorch is installed it is imported first and this library binds to the runtime it brought.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in list(SIGNATURES.items()) + list(BACKEND_SIGNATURES.items()) + list(WEIGHTS_SIGNATURES.items()):
         fn = getattr(lib, name)          # AttributeError if the library lacks a declared symbol

@@ -342,6 +342,18 @@ Status HipBackend::kernel_mul_mat(Tensor* node) {
     Tensor* s0 = node->src[0];
     Tensor* s1 = node->src[1];
     if (!s0 || !s1) return fail(Status::NOT_SUPPORTED, "mul_mat: missing source");
+    if (mul_mat_transposed_) {
+        // s0, s1 are the sources of the two folded transpositions: [M, K] and [N, K] in the reference's order of
+        // dimensions, i.e. K rows of M and of N elements; the node is [N, M]
+        const int64_t M = node->dims[1], N = node->dims[0], K = s0->dims[1];
+        if (s0->type != TENSOR_TYPE_F32 || s1->type != TENSOR_TYPE_F32 || node->type != TENSOR_TYPE_F32 || node->src[2] ||
+            s0->dims[0] != M || s1->dims[0] != N || s1->dims[1] != K || s0->numel() != M * K || s1->numel() != N * K)
+            return fail(Status::ABORTED, "mul_mat: the folded transpositions do not fit the node");
+        const int rc = mul_mat_tn_hip(static_cast<const float*>(s0->data), static_cast<const float*>(s1->data), static_cast<float*>(node->data),
+                                      static_cast<int>(M), static_cast<int>(K), static_cast<int>(N), 1.0f, nullptr);
+        if (rc != 0) return fail(status_of_rc(rc), std::string("mul_mat: ") + ppml_hip_last_error());
+        return Status::SUCCESS;
+    }
     const int64_t M = node->dims[1], N = node->dims[0], K = s0->dims[0];
     if (s1->dims[0] != K) return fail(Status::NOT_SUPPORTED, "mul_mat: inner dimensions differ");
     if (s0->numel() != M * K || s1->numel() != N * K)
@@ -696,7 +708,7 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         Tensor* relu = nullptr;
         Tensor* out_prod = nullptr;         // OP_SCALE node that runs as the (skipped) out_prod it reads, scaled
         Tensor* added = nullptr;            // OP_SOFT_MAX node that adds the second operand of this (skipped) OP_ADD on its way in
-        bool transposed = false;            // OP_OUT_PROD that reads the sources of its two (skipped) {1,0,2,3} permutations
+        bool transposed = false;            // OP_OUT_PROD / OP_MUL_MAT that reads the sources of its two (skipped) {1,0,2,3} permutations
         bool chain = false;                 // out_prod(attn_t, V_t) that runs as the whole attention chain
         Tensor *q = nullptr, *k = nullptr, *v = nullptr, *bias = nullptr;
         float scale = 1.0f;
@@ -705,7 +717,7 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
     std::unordered_set<const Tensor*> skipped;
     nodes_fused_away_ = 0;
     if (fuse_attention_bridges_ || fuse_relu_into_q8_ || fuse_scale_into_out_prod_ || fuse_attention_chain_ ||
-        fuse_add_into_soft_max_ || fuse_permutes_into_out_prod_) {
+        fuse_add_into_soft_max_ || fuse_permutes_into_out_prod_ || fuse_permutes_into_mul_mat_) {
         std::unordered_map<const Tensor*, int> uses, position;
         std::unordered_map<const Tensor*, Tensor*> single_user;
         int pos = 0;
@@ -867,6 +879,28 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
                 skipped.insert(p1);
             }
         }
+
+        // (7) the two matrix transpositions in front of a LinearLayer's weight gradient,
+        // mul_mat(mat_transpose(grad), mat_transpose(x)) (src/core/ComputeGraph.cpp:733-738; mat_transpose is a
+        // permutation copy of dims[0] and dims[1], src/core/ComputeGraphHelper.cpp:375-382)
+        if (fuse_permutes_into_mul_mat_) {
+            const auto is_mat_t = [](const Tensor* t) {
+                if (!t || (t->op != OP_PERMUTE && t->op != OP_TRANSPOSE) || t->ndim < 2 || t->type != TENSOR_TYPE_F32 || t->view_src) return false;
+                const Tensor* s = t->src[0];
+                if (!s || s->type != TENSOR_TYPE_F32 || s->ndim != t->ndim || s->numel() != t->numel()) return false;
+                for (int d = 2; d < t->ndim; ++d) if (t->op_params[d] != d || t->dims[d] != 1) return false;       // one matrix
+                return t->op_params[0] == 1 && t->op_params[1] == 0 && s->dims[0] == t->dims[1] && s->dims[1] == t->dims[0];
+            };
+            for (Tensor* n : *graph) {
+                if (!n || n->op != OP_MUL_MAT || n->type != TENSOR_TYPE_F32 || n->src[2] || skipped.count(n) || !node_supported(n)) continue;
+                Tensor* p0 = n->src[0];
+                Tensor* p1 = n->src[1];
+                if (p0 == p1 || !is_mat_t(p0) || !is_mat_t(p1) || !private_to(p0, n) || !private_to(p1, n)) continue;
+                plans[n].transposed = true;
+                skipped.insert(p0);
+                skipped.insert(p1);
+            }
+        }
         nodes_fused_away_ = skipped.size();
     }
 
@@ -899,6 +933,7 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         relu_in_quantizer_ = false;
         out_prod_scaled_ = false;
         out_prod_transposed_ = false;
+        mul_mat_transposed_ = false;
         soft_max_bias_ = nullptr;
         const auto plan = plans.find(node);
         if (plan != plans.end()) {
@@ -943,7 +978,8 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
             if (pl.transposed) {
                 rewired.src[0] = node->src[0]->src[0];
                 rewired.src[1] = node->src[1]->src[0];
-                out_prod_transposed_ = true;
+                if (node->op == OP_MUL_MAT) mul_mat_transposed_ = true;
+                else out_prod_transposed_ = true;
             }
             if (pl.chain) {
                 // src/core/ComputeGraphHelper.cpp:450-484: Q, K, V, bias in src 0..3; scale, causal, eps, Br, Bc
@@ -1004,6 +1040,7 @@ Status HipBackend::graph_compute(ComputeGraph* graph) {
         relu_in_quantizer_ = false;
         out_prod_scaled_ = false;
         out_prod_transposed_ = false;
+        mul_mat_transposed_ = false;
         soft_max_bias_ = nullptr;
         if (st != Status::SUCCESS) return st;
         const hipError_t e = hipGetLastError();
@@ -1158,6 +1195,9 @@ void ppml_hip_backend_set_fuse_scale_into_out_prod(ppml_hip_backend* b, int on) 
 }
 void ppml_hip_backend_set_fuse_add_into_soft_max(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_fuse_add_into_soft_max(on != 0);
+}
+void ppml_hip_backend_set_fuse_permutes_into_mul_mat(ppml_hip_backend* b, int on) {
+    if (b) b->impl.set_fuse_permutes_into_mul_mat(on != 0);
 }
 void ppml_hip_backend_set_fuse_permutes_into_out_prod(ppml_hip_backend* b, int on) {
     if (b) b->impl.set_fuse_permutes_into_out_prod(on != 0);

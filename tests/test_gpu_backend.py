@@ -491,6 +491,47 @@ def test_backward_of_a_biased_linear_stays_on_the_device(be, oracle):
     assert np.array_equal(be.download(db), oracle.repeat_back(G, (N,)))
 
 
+@pytest.mark.parametrize("T,K,N", [(2601, 128, 256), (10609, 128, 512), (300, 40, 24)])
+def test_weight_gradient_reads_the_untransposed_matrices(be, T, K, N):
+    """dW = mul_mat(mat_transpose(grad), mat_transpose(x)) (src/core/ComputeGraph.cpp:733-738): the two transpositions
+    are not executed when nobody else reads them, the contraction runs over the rows of grad and x as they lie, and the
+    result has the bits of the three nodes run one by one.  A transposition somebody else reads stays a node."""
+    rng = np.random.default_rng(T)
+    X = rng.standard_normal((T, K)).astype(np.float32)
+    G = rng.standard_normal((T, N)).astype(np.float32)
+
+    def build(extra_reader):
+        x, g = _leaf(be, X), _leaf(be, G)
+        gt = B.Tensor((T, N), B.F32, B.OP_PERMUTE, [g]); gt.set_param(0, 1).set_param(1, 0)
+        xt = B.Tensor((T, K), B.F32, B.OP_PERMUTE, [x]); xt.set_param(0, 1).set_param(1, 0)
+        dW = B.Tensor((K, N), B.F32, B.OP_MUL_MAT, [gt, xt])
+        nodes = [gt, xt, dW]
+        if extra_reader:
+            other = B.Tensor((T, K), B.F32, B.OP_SCALE, [xt]).set_param(0, 2.0)
+            nodes.append(other)
+        return nodes, dW, xt
+
+    results = {}
+    for fused in (True, False):
+        be.set_fuse_permutes_into_mul_mat(fused)
+        try:
+            nodes, dW, xt = build(False)
+            assert be.graph_compute(nodes) == B.SUCCESS, be.last_error
+            assert be.nodes_fused_away == (2 if fused else 0)
+            results[fused] = be.download(dW).reshape(N, K)
+        finally:
+            be.set_fuse_permutes_into_mul_mat(True)
+    assert np.array_equal(results[True].view(np.int32), results[False].view(np.int32))
+    want = G.astype(np.float64).T @ X.astype(np.float64)
+    bound = (np.abs(G.astype(np.float64)).T @ np.abs(X.astype(np.float64))) * (T + 2) * 2.0 ** -24
+    assert np.all(np.abs(results[True] - want) <= bound)
+    nodes, dW, xt = build(True)
+    assert be.graph_compute(nodes) == B.SUCCESS, be.last_error
+    assert be.nodes_fused_away == 0
+    assert np.array_equal(be.download(dW).reshape(N, K).view(np.int32), results[False].view(np.int32))
+    assert np.array_equal(be.download(xt).reshape(K, T), X.T)
+
+
 def test_f32_arithmetic_is_a_field_of_the_backend(be, oracle):
     # two backends with different pipes do not disturb each other or the calling thread's own setting
     import torch
