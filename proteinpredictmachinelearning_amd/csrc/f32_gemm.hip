@@ -962,12 +962,15 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_slices_kernel(const GemmPa
 // 128 tile is three quarters padding there: matrix work, split and LDS traffic for rows that do not exist.  Here the
 // tile is 128 along the long side and 32 along the narrow one; each of the four contracting waves takes 32 rows of the
 // long operand against the one fragment of the narrow operand, six MFMAs per 16-k chunk; of the loading waves all
-// four split the long operand and two of them the narrow one.  Operands contiguous in k, buffer addressing, same
-// products in the same order as the other forms: same bits.
+// four split the long operand and two of them (one, with contiguous rows) the narrow one.  Operands contiguous in k
+// (MODE LOAD_K_CONTIG) or in their rows (LOAD_ROW_CONTIG: the backward of the attention logits, out_prod(grad,
+// mat_transpose(Q)), 256 x 32 per plane under K = 256), buffer addressing, same products in the same order as the other
+// forms: same bits.
 constexpr int SIDE_M = 1, SIDE_N = 2;
-template <int SIDE, bool STREAM_C, bool K4>
+template <int MODE, int SIDE, bool STREAM_C, bool K4>
 __global__ __launch_bounds__(512) void gemm_bf16x3_pc_narrow_kernel(const GemmParams p) {
     static_assert(SIDE == SIDE_M || SIDE == SIDE_N, "which operand is the narrow one");
+    static_assert(MODE == LOAD_ROW_CONTIG || MODE == LOAD_K_CONTIG, "buffer addressing");
     constexpr int LONG_STAGE = 3 * SPLIT_PLANE;                  // three planes of 128 rows
     constexpr int NARROW_PLANE = 32 * SPLIT_PITCH;
     constexpr int STAGE = LONG_STAGE + 3 * NARROW_PLANE;
@@ -989,33 +992,48 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_narrow_kernel(const GemmPa
     float* C = p.C + p2 * p.c_p2 + p3 * p.c_p3;
     const int chunks = (p.K + BK - 1) / BK;
 
-    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, static_cast<int>(((p.M - 1) * p.a_rs + p.K) * 4), 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, static_cast<int>(((p.N - 1) * p.b_rs + p.K) * 4), 0x00020000);
+    const int64_t a_plane = MODE == LOAD_K_CONTIG ? (p.M - 1) * p.a_rs + p.K : p.K * p.a_ks;
+    const int64_t b_plane = MODE == LOAD_K_CONTIG ? (p.N - 1) * p.b_rs + p.K : p.K * p.b_ks;
+    const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, static_cast<int>(a_plane * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, static_cast<int>(b_plane * 4), 0x00020000);
     const __amdgpu_buffer_rsrc_t& rsrc_long = SIDE == SIDE_M ? rsrc_b : rsrc_a;
     const __amdgpu_buffer_rsrc_t& rsrc_narrow = SIDE == SIDE_M ? rsrc_a : rsrc_b;
-    const uint32_t long_rs = static_cast<uint32_t>(SIDE == SIDE_M ? p.b_rs : p.a_rs) * 4u;
-    const uint32_t narrow_rs = static_cast<uint32_t>(SIDE == SIDE_M ? p.a_rs : p.b_rs) * 4u;
+    // the step between rows (k-contiguous operands) or between k (row-contiguous ones), in bytes
+    const uint32_t long_rs = static_cast<uint32_t>(MODE == LOAD_K_CONTIG ? (SIDE == SIDE_M ? p.b_rs : p.a_rs) : (SIDE == SIDE_M ? p.b_ks : p.a_ks)) * 4u;
+    const uint32_t narrow_rs = static_cast<uint32_t>(MODE == LOAD_K_CONTIG ? (SIDE == SIDE_M ? p.a_rs : p.b_rs) : (SIDE == SIDE_M ? p.a_ks : p.b_ks)) * 4u;
     const int long_row0 = SIDE == SIDE_M ? n0 : m0, long_rows = SIDE == SIDE_M ? p.N : p.M;
     const int narrow_rows = SIDE == SIDE_M ? p.M : p.N;
 
     // (barriers: chunks + 1 in either loop, as in gemm_bf16x3_pc_kernel)
     int fired = 0;
     if (producer) {
-        v4f rl[PC_AHEAD][2];                            // the long operand: two row pieces per thread
-        v4f rn[PC_AHEAD];                               // the narrow one: one piece per thread of the first two loading waves
-        const bool has_narrow = wave < 6;               // rows ptid / 4 < 32
-        const auto load_both = [&](int c, v4f (&xl)[2], v4f& xn) {
-            load_kcontig_buffer<K4>(rsrc_long, long_rs, long_row0, long_rows, c * BK, p.K, ptid, xl);
-            if (has_narrow) {
-                const int k = c * BK + (ptid & 3) * 4;
-                const int row = ptid >> 2;
-                const uint32_t at = row < narrow_rows ? static_cast<uint32_t>(row) * narrow_rs + static_cast<uint32_t>(k) * 4u : OUTSIDE;
-                if (K4) {
-                    xn = __builtin_bit_cast(v4f, __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_narrow, k < p.K ? at : OUTSIDE, 0, 0)));
-                } else {
+        v4f rl[PC_AHEAD][2];                            // the long operand: two row pieces per thread (one row, eight k, with contiguous rows)
+        v4f rn[PC_AHEAD][2];                            // the narrow one: one piece per thread of the first two loading waves (eight k per thread of the first)
+        const bool has_narrow = MODE == LOAD_K_CONTIG ? wave < 6 : wave < 5;     // rows ptid / 4 < 32; row ptid % 32, k half ptid / 32 of 64 threads
+        const auto load_both = [&](int c, v4f (&xl)[2], v4f (&xn)[2]) {
+            if (MODE == LOAD_K_CONTIG) {
+                load_kcontig_buffer<K4>(rsrc_long, long_rs, long_row0, long_rows, c * BK, p.K, ptid, xl);
+                if (has_narrow) {
+                    const int k = c * BK + (ptid & 3) * 4;
+                    const int row = ptid >> 2;
+                    const uint32_t at = row < narrow_rows ? static_cast<uint32_t>(row) * narrow_rs + static_cast<uint32_t>(k) * 4u : OUTSIDE;
+                    if (K4) {
+                        xn[0] = __builtin_bit_cast(v4f, __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_narrow, k < p.K ? at : OUTSIDE, 0, 0)));
+                    } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        xn[e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_narrow, k + e < p.K ? at + 4u * e : OUTSIDE, 0, 0));
+                        for (int e = 0; e < 4; ++e)
+                            xn[0][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_narrow, k + e < p.K ? at + 4u * e : OUTSIDE, 0, 0));
+                    }
+                }
+            } else {
+                load_rows8_buffer(rsrc_long, long_rs, long_row0, long_rows, c * BK, ptid, xl);
+                if (has_narrow) {
+                    const int row = ptid & 31;
+                    const uint32_t lane_off = row < narrow_rows ? static_cast<uint32_t>(row) * 4u : OUTSIDE;
+                    const uint32_t kb = static_cast<uint32_t>(c * BK + (ptid >> 5) * 8);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)     // (k past the end: outside the plane, whose size is K steps)
+                        xn[e >> 2][e & 3] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc_narrow, lane_off + (kb + e) * narrow_rs, 0, 0));
                 }
             }
         };
@@ -1029,13 +1047,22 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_narrow_kernel(const GemmPa
                 const int c = cg + d;
                 if (c >= chunks) break;                 // uniform
                 uint8_t* half = lds_ab[c & 1];
-                split_store<LOAD_K_CONTIG>(half, ptid, rl[d], guard);
+                split_store<MODE>(half, ptid, rl[d], guard);
                 if (has_narrow) {
-                    uint2 parts[3];
-                    split4(rn[d], parts, guard);
-                    uint8_t* dst = half + LONG_STAGE + (ptid >> 2) * SPLIT_PITCH + (ptid & 3) * 8;
+                    if (MODE == LOAD_K_CONTIG) {
+                        uint2 parts[3];
+                        split4(rn[d][0], parts, guard);
+                        uint8_t* dst = half + LONG_STAGE + (ptid >> 2) * SPLIT_PITCH + (ptid & 3) * 8;
 #pragma unroll
-                    for (int s3 = 0; s3 < 3; ++s3) *reinterpret_cast<uint2*>(dst + s3 * NARROW_PLANE) = parts[s3];
+                        for (int s3 = 0; s3 < 3; ++s3) *reinterpret_cast<uint2*>(dst + s3 * NARROW_PLANE) = parts[s3];
+                    } else {
+                        uint2 lo[3], hi[3];
+                        split4(rn[d][0], lo, guard);
+                        split4(rn[d][1], hi, guard);
+                        uint8_t* dst = half + LONG_STAGE + (ptid & 31) * SPLIT_PITCH + (ptid >> 5) * 16;
+#pragma unroll
+                        for (int s3 = 0; s3 < 3; ++s3) *reinterpret_cast<uint4*>(dst + s3 * NARROW_PLANE) = uint4{lo[s3].x, lo[s3].y, hi[s3].x, hi[s3].y};
+                    }
                 }
                 if (c + PC_AHEAD < chunks) load_both(c + PC_AHEAD, rl[d], rn[d]);
                 __syncthreads();
@@ -2195,6 +2222,18 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
             const int rc = try_pc_slices<LOAD_ROW_CONTIG>(p, stream, what);
             if (rc >= 0) return rc;
         }
+        if (p.K > 3 * BK && (p.N <= 32) != (p.M <= 32)) {
+            // one narrow side: tiles of 128 x 32 along the other (gemm_bf16x3_pc_narrow_kernel)
+            const bool side_n = p.N <= 32;
+            const int64_t tiles_long = side_n ? p.tiles_m : p.tiles_n;
+            if (side_n) p.tiles_n = 1; else p.tiles_m = 1;
+            const dim3 ngrid(static_cast<unsigned>(tiles_long * p.np2 * p.np3));
+#define PPML_RNARROW(SIDE_, STREAM_) hipLaunchKernelGGL((gemm_bf16x3_pc_narrow_kernel<LOAD_ROW_CONTIG, SIDE_, STREAM_, true>), ngrid, dim3(512), 0, stream, p)
+            if (side_n) { if (p.stream_c) PPML_RNARROW(SIDE_N, true); else PPML_RNARROW(SIDE_N, false); }
+            else        { if (p.stream_c) PPML_RNARROW(SIDE_M, true); else PPML_RNARROW(SIDE_M, false); }
+#undef PPML_RNARROW
+            return check_launch(what);
+        }
         if (two_sets) {
             if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_pc_kernel<LOAD_ROW_CONTIG, true, true>), grid, dim3(512), 0, stream, p);
             else hipLaunchKernelGGL((gemm_bf16x3_pc_kernel<LOAD_ROW_CONTIG, false, true>), grid, dim3(512), 0, stream, p);
@@ -2217,7 +2256,7 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
             const int64_t tiles_long = side_n ? p.tiles_m : p.tiles_n;
             if (side_n) p.tiles_n = 1; else p.tiles_m = 1;
             const dim3 ngrid(static_cast<unsigned>(tiles_long * p.np2 * p.np3));
-#define PPML_KNARROW(SIDE_, STREAM_, K4_) hipLaunchKernelGGL((gemm_bf16x3_pc_narrow_kernel<SIDE_, STREAM_, K4_>), ngrid, dim3(512), 0, stream, p)
+#define PPML_KNARROW(SIDE_, STREAM_, K4_) hipLaunchKernelGGL((gemm_bf16x3_pc_narrow_kernel<LOAD_K_CONTIG, SIDE_, STREAM_, K4_>), ngrid, dim3(512), 0, stream, p)
             const bool k4 = p.K % 4 == 0;
             if (side_n) { if (k4) { if (p.stream_c) PPML_KNARROW(SIDE_N, true, true); else PPML_KNARROW(SIDE_N, false, true); }
                           else    { if (p.stream_c) PPML_KNARROW(SIDE_N, true, false); else PPML_KNARROW(SIDE_N, false, false); } }

@@ -766,6 +766,39 @@ def test_outer_prod_mean_back(ops, oracle, D, L, N, Bt):
         assert none is None and np.array_equal(gr.cpu().numpy(), wr)
 
 
+@pytest.mark.parametrize("planes,K,ne00,ne10", [(824, 256, 256, 32), (412, 103, 103, 32), (7, 70, 300, 5), (3, 200, 33, 32), (50, 64, 128, 16),
+                                                (5, 90, 20, 200), (2, 1000, 129, 31)])
+def test_out_prod_with_a_narrow_side_takes_narrow_tiles_with_the_same_bits(ops, planes, K, ne00, ne10):
+    """out_prod with at most 32 rows on one side (the backward of the attention logits, out_prod(grad, mat_transpose(Q)):
+    head dimension x keys per plane, src/core/ComputeGraph.cpp:769-773) runs on tiles of 128 x 32: the bits of the same
+    contraction on 128 x 128 tiles (the narrow operand padded with zero columns), float64 within 1e-4, and an infinite
+    or sub-range element ends where it does there."""
+    torch.manual_seed(planes + K)
+    a = torch.randn(1, planes, K, ne00, device="cuda")
+    b = torch.randn(1, planes, K, ne10, device="cuda")
+
+    def wide(x, y):
+        # the narrow one of the two padded to 64 columns: wide tiles; the padding's outputs are cut off again
+        if y.shape[-1] <= 32:
+            yp = torch.zeros(*y.shape[:-1], 64, device="cuda"); yp[..., :y.shape[-1]] = y
+            return ops.out_prod(x, yp)[:, :, :y.shape[-1], :].contiguous()
+        xp = torch.zeros(*x.shape[:-1], 64, device="cuda"); xp[..., :x.shape[-1]] = x
+        return ops.out_prod(xp, y)[:, :, :, :x.shape[-1]].contiguous()
+
+    got = ops.out_prod(a, b)
+    assert torch.equal(got.view(torch.int32), wide(a, b).view(torch.int32))
+    want = torch.einsum("pkm,pkn->pnm", a[0].double(), b[0].double())
+    assert float((got[0].double() - want).abs().max()) <= 1e-4 * float(want.abs().max())
+    a2, b2 = a.clone(), b.clone()
+    a2[0, planes // 2, K // 3, ne00 // 2] = float("inf")
+    b2[0, planes - 1, K - 1, ne10 - 1] = 1e-42
+    b2[0, 0, 0, 0] = -float("inf")
+    got2, wide2 = ops.out_prod(a2, b2), wide(a2, b2)
+    assert torch.equal(got2.isnan(), wide2.isnan())
+    assert torch.equal(torch.nan_to_num(got2, nan=0.0).view(torch.int32), torch.nan_to_num(wide2, nan=0.0).view(torch.int32))
+    assert bool(got2[0, planes // 2, :, ne00 // 2].isinf().all()) and bool(got2[0, 0, 0, :].isinf().all())
+
+
 @pytest.mark.parametrize("T,K,N", [(26368, 256, 768), (10609, 128, 512), (5000, 100, 130), (3001, 33, 7), (1000, 300, 300), (26368, 256, 16)])
 def test_weight_gradients_of_linear_layers_go_in_k_slices(ops, oracle, T, K, N):
     """dW = X^T dY of a LinearLayer (src/core/ComputeGraph.cpp:708-773: `mat_transpose` of both, then `mul_mat`): a few
