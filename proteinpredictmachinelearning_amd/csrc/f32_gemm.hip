@@ -1964,12 +1964,9 @@ int try_half_split(const GemmParams& p, hipStream_t stream, const char* what) {
     const size_t part_bytes = static_cast<size_t>(slices) * ma_pad * nb_pad * 4;
     const int n_flags = ma_pad / 32 + nb_pad / 32;
     const size_t flag_bytes = (static_cast<size_t>(n_flags) * 4 + 255) / 256 * 256;
-    uint8_t* ws = nullptr;
-    hipMemPool_t pool = workspace_pool();
-    if (!pool || hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), b_bytes + part_bytes + flag_bytes, pool, stream) != hipSuccess) {
-        (void)hipGetLastError();
-        return -1;
-    }
+    const Workspace held = workspace_take(b_bytes + part_bytes + flag_bytes, stream);
+    uint8_t* ws = held.ptr;
+    if (!ws) return -1;
     float* partial = reinterpret_cast<float*>(ws + b_bytes);
     int* fired_a = reinterpret_cast<int*>(ws + b_bytes + part_bytes);
     int* fired_b = fired_a + ma_pad / 32;
@@ -1995,7 +1992,7 @@ int try_half_split(const GemmParams& p, hipStream_t stream, const char* what) {
                            ma_pad, nb_pad, fired_a, fired_b);
         rc = check_launch(what);
     }
-    if (hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();
+    workspace_give(held, stream);
     return rc;
 }
 
@@ -2016,12 +2013,9 @@ int try_pc_slices(const GemmParams& p, hipStream_t stream, const char* what) {
     const size_t part_bytes = static_cast<size_t>(slices) * ma_pad * nb_pad * 4;
     const int n_flags = ma_pad / 32 + nb_pad / 32;
     const size_t flag_bytes = (static_cast<size_t>(n_flags) * 4 + 255) / 256 * 256;
-    uint8_t* ws = nullptr;
-    hipMemPool_t pool = workspace_pool();
-    if (!pool || hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), part_bytes + flag_bytes, pool, stream) != hipSuccess) {
-        (void)hipGetLastError();
-        return -1;
-    }
+    const Workspace held = workspace_take(part_bytes + flag_bytes, stream);
+    uint8_t* ws = held.ptr;
+    if (!ws) return -1;
     float* partial = reinterpret_cast<float*>(ws);
     int* fired_a = reinterpret_cast<int*>(ws + part_bytes);
     int* fired_b = fired_a + ma_pad / 32;               // (stays clear: the kernel flags rows for either operand)
@@ -2043,7 +2037,7 @@ int try_pc_slices(const GemmParams& p, hipStream_t stream, const char* what) {
                            ma_pad, nb_pad, fired_a, fired_b);
         rc = check_launch(what);
     }
-    if (hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();
+    workspace_give(held, stream);
     return rc;
 }
 
@@ -2113,6 +2107,7 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
         const size_t flag_bytes = (static_cast<size_t>(n_flags) * 4 + 255) / 256 * 256;
         const size_t ws_bytes = a_bytes + b_bytes + part_bytes + flag_bytes;
         uint8_t* ws = nullptr;
+        Workspace held;
         if (fixed_ws) {
             if (ws_bytes > fixed_cap) {
                 set_error("%s: this contraction needs %zu bytes of workspace, the static one holds %zu", what, ws_bytes, fixed_cap);
@@ -2120,11 +2115,8 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
             }
             ws = fixed_ws;
         } else {
-            hipMemPool_t pool = workspace_pool();
-            if (pool && hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws), ws_bytes, pool, stream) != hipSuccess) {
-                (void)hipGetLastError();
-                ws = nullptr;
-            }
+            held = workspace_take(ws_bytes, stream);
+            ws = held.ptr;
         }
         if (ws) {
             GemmParams q = p;
@@ -2156,7 +2148,7 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
                 else       hipLaunchKernelGGL((reduce_slices_kernel<false>), rgrid, block, 0, stream, p, partial, slices, ma_pad, nb_pad, fired_a, fired_b);
                 rc = check_launch(what);
             }
-            if (!fixed_ws && hipFreeAsync(ws, stream) != hipSuccess) (void)hipGetLastError();
+            if (!fixed_ws) workspace_give(held, stream);
             return rc;
         }
     }

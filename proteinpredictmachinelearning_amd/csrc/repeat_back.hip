@@ -142,11 +142,11 @@ extern "C" int repeat_back_hip(const float* src, float* dst,
     slices = (jb.reps + jb.per_slice - 1) / jb.per_slice;
     if (slices > 0x7fffffff / 256 || (jb.total * slices + 255) / 256 > 0x7fffffffLL) { set_error("repeat_back_hip: destination too large"); return RC_BAD_ARGS; }
     float* partial = nullptr;
+    Workspace held;
     if (slices > 1) {
-        hipMemPool_t pool = workspace_pool();
-        if (!pool || hipMallocFromPoolAsync(reinterpret_cast<void**>(&partial), static_cast<size_t>(slices) * jb.total * 4, pool, s) != hipSuccess) {
-            (void)hipGetLastError();
-            partial = nullptr;
+        held = workspace_take(static_cast<size_t>(slices) * jb.total * 4, s);
+        partial = reinterpret_cast<float*>(held.ptr);
+        if (!partial) {
             slices = 1;                               // no workspace: one run per element, slower and just as right
             jb.per_slice = jb.reps;
         }
@@ -161,7 +161,7 @@ extern "C" int repeat_back_hip(const float* src, float* dst,
                                static_cast<int>(slices));
             rc = check_launch("repeat_back_fold_kernel");
         }
-        if (hipFreeAsync(partial, s) != hipSuccess) (void)hipGetLastError();
+        workspace_give(held, s);
     }
     return rc;
 }

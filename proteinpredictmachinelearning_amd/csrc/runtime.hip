@@ -210,6 +210,51 @@ hipMemPool_t workspace_pool() {
     return pools[dev];
 }
 
+Workspace workspace_take(size_t bytes, hipStream_t stream) {
+    Workspace ws;
+    hipMemPool_t pool = workspace_pool();
+    if (!pool || bytes == 0) return ws;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (stream != nullptr && stream != hipStreamPerThread && hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+        (void)hipGetLastError();
+        capturing = hipStreamCaptureStatusActive;        // (cannot tell: treat it as the careful case)
+    }
+    if (stream == hipStreamPerThread || capturing != hipStreamCaptureStatusNone) {
+        // one name for many streams, or an allocation that would be baked into a graph: allocate for this call only
+        if (hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws.ptr), bytes, pool, stream) != hipSuccess) { (void)hipGetLastError(); ws.ptr = nullptr; }
+        ws.call_owned = ws.ptr != nullptr;
+        return ws;
+    }
+    struct Kept { uint8_t* ptr = nullptr; size_t cap = 0; std::mutex turn; };
+    static std::mutex mu;
+    static std::map<std::pair<int, hipStream_t>, Kept> kept;       // (nodes of a map stay where they are)
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return ws; }
+    Kept* entry;
+    {
+        std::lock_guard<std::mutex> guard(mu);
+        entry = &kept[{dev, stream}];
+    }
+    Kept& k = *entry;
+    k.turn.lock();                                       // until workspace_give()
+    if (k.cap < bytes) {
+        if (k.ptr && hipFreeAsync(k.ptr, stream) != hipSuccess) (void)hipGetLastError();
+        k.ptr = nullptr; k.cap = 0;
+        const size_t want = (bytes + (bytes >> 2) + ((1u << 20) - 1)) & ~static_cast<size_t>((1u << 20) - 1);    // a quarter more, whole MiB
+        if (hipMallocFromPoolAsync(reinterpret_cast<void**>(&k.ptr), want, pool, stream) == hipSuccess) k.cap = want;
+        else { (void)hipGetLastError(); k.ptr = nullptr; }
+    }
+    ws.ptr = k.ptr;
+    if (ws.ptr) ws.turn = &k.turn;
+    else k.turn.unlock();
+    return ws;
+}
+
+void workspace_give(const Workspace& ws, hipStream_t stream) {
+    if (ws.call_owned && ws.ptr && hipFreeAsync(ws.ptr, stream) != hipSuccess) (void)hipGetLastError();
+    if (ws.turn) static_cast<std::mutex*>(ws.turn)->unlock();
+}
+
 // compute units of the device the library first ran on (256 on the part this library is built for)
 int device_cu_count() {
     static const int cus = [] {
