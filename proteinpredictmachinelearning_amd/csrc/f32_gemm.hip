@@ -1927,10 +1927,10 @@ int f32_arithmetic() {
 // nothing).  With one, the pool is never touched: a contraction that wants more workspace than `fixed_cap`
 // is refused, one that wants none runs as it always does.
 // How many K slices make `groups` output tiles come out even over the CUs (a CU's rate does not depend on how many
-// work-groups it holds): the smallest count within 2 % of the best, slices of at least PLANES_MIN_SLICE_CHUNKS chunks.
-int even_slices(int groups, int chunks, int most_slices) {
+// work-groups it holds): the smallest count within 2 % of the best, slices of at least `least_chunks` chunks.
+int even_slices(int groups, int chunks, int most_slices, int least_chunks = PLANES_MIN_SLICE_CHUNKS) {
     const int cus = device_cu_count();
-    int most = chunks / PLANES_MIN_SLICE_CHUNKS < most_slices ? chunks / PLANES_MIN_SLICE_CHUNKS : most_slices;
+    int most = chunks / least_chunks < most_slices ? chunks / least_chunks : most_slices;
     if (most < 1) most = 1;
     int slices = 1;
     double best = 1e30;
@@ -2002,10 +2002,12 @@ template <int MODE>
 int try_pc_slices(const GemmParams& p, hipStream_t stream, const char* what) {
     const int chunks = (p.K + BK - 1) / BK;
     const int groups = p.tiles_m * p.tiles_n;
-    // (three launches and a workspace: about 28 us before the first chunk; measured even with the unsliced form at K = 515
-    // on one tile (23 against 33 us), ahead of it at K = 1000 on nine tiles (32 against 41))
-    if (p.np2 * p.np3 != 1 || groups * 2 > device_cu_count() || chunks < 3 * PLANES_MIN_SLICE_CHUNKS) return -1;
-    int slices = even_slices(groups, chunks, 128);
+    // (three launches: about 12 us before the first chunk.  us over K for one to nine tiles, unsliced: 256 12, 400 16.5,
+    // 512 20, 640 24, 752 27; in slices: 784 and 1024 16.5-17, 2048 18-19)
+    constexpr int LEAST = 8;                            // chunks a slice is long at least
+    // (64 tiles of 128 x 128 under K = 512 measured 23.0 against 20.4 unsliced, under K = 784 24.7 against 28.9)
+    if (p.np2 * p.np3 != 1 || groups * 2 > device_cu_count() || chunks < (groups * 4 <= device_cu_count() ? 4 * LEAST : 6 * LEAST)) return -1;
+    int slices = even_slices(groups, chunks, 128, LEAST);
     if (slices < 2) return -1;
     const int slice_chunks = (chunks + slices - 1) / slices;
     slices = (chunks + slice_chunks - 1) / slice_chunks;
