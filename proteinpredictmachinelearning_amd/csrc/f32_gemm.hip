@@ -741,9 +741,12 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
 // more tiles than CUs (26368 x 256 -> 256 and wider, the many-plane contractions) the work-groups of a CU overlap
 // each other anyway and the two forms measure the same: the launcher takes this one up to one tile per CU.
 constexpr int PC_AHEAD = 3;                       // chunks a producer wave has in flight
-template <int MODE, bool STREAM_C, bool K4>
+template <int MODE, bool STREAM_C, bool K4, int BMODE = MODE>
 __global__ __launch_bounds__(512) void gemm_bf16x3_pc_kernel(const GemmParams p) {
+    // (MODE: how A lies; BMODE: how B lies -- the backward of the triangle multiplication contracts a gradient that is
+    // contiguous in k with an operand that is contiguous in its rows)
     static_assert(MODE == LOAD_ROW_CONTIG || MODE == LOAD_K_CONTIG, "buffer addressing");
+    static_assert(BMODE == LOAD_ROW_CONTIG || BMODE == LOAD_K_CONTIG, "buffer addressing");
     constexpr int STAGE = 3 * SPLIT_PLANE;            // the three planes of one operand's chunk
     __shared__ __attribute__((aligned(16))) uint8_t lds_ab[2][2 * STAGE];
 
@@ -764,7 +767,7 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_kernel(const GemmParams p)
     const int chunks = (p.K + BK - 1) / BK;
 
     const int64_t a_plane = MODE == LOAD_K_CONTIG ? (p.M - 1) * p.a_rs + p.K : p.K * p.a_ks;
-    const int64_t b_plane = MODE == LOAD_K_CONTIG ? (p.N - 1) * p.b_rs + p.K : p.K * p.b_ks;
+    const int64_t b_plane = BMODE == LOAD_K_CONTIG ? (p.N - 1) * p.b_rs + p.K : p.K * p.b_ks;
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, static_cast<int>(a_plane * 4), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, static_cast<int>(b_plane * 4), 0x00020000);
 
@@ -774,13 +777,10 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_kernel(const GemmParams p)
     if (producer) {
         v4f ra[PC_AHEAD][2], rb[PC_AHEAD][2];
         const auto load_both = [&](int c, v4f (&xa)[2], v4f (&xb)[2]) {
-            if (MODE == LOAD_K_CONTIG) {
-                load_kcontig_buffer<K4>(rsrc_a, static_cast<uint32_t>(p.a_rs) * 4u, m0, p.M, c * BK, p.K, ptid, xa);
-                load_kcontig_buffer<K4>(rsrc_b, static_cast<uint32_t>(p.b_rs) * 4u, n0, p.N, c * BK, p.K, ptid, xb);
-            } else {
-                load_rows8_buffer(rsrc_a, static_cast<uint32_t>(p.a_ks) * 4u, m0, p.M, c * BK, ptid, xa);
-                load_rows8_buffer(rsrc_b, static_cast<uint32_t>(p.b_ks) * 4u, n0, p.N, c * BK, ptid, xb);
-            }
+            if (MODE == LOAD_K_CONTIG) load_kcontig_buffer<K4>(rsrc_a, static_cast<uint32_t>(p.a_rs) * 4u, m0, p.M, c * BK, p.K, ptid, xa);
+            else load_rows8_buffer(rsrc_a, static_cast<uint32_t>(p.a_ks) * 4u, m0, p.M, c * BK, ptid, xa);
+            if (BMODE == LOAD_K_CONTIG) load_kcontig_buffer<K4>(rsrc_b, static_cast<uint32_t>(p.b_rs) * 4u, n0, p.N, c * BK, p.K, ptid, xb);
+            else load_rows8_buffer(rsrc_b, static_cast<uint32_t>(p.b_ks) * 4u, n0, p.N, c * BK, ptid, xb);
         };
 #pragma unroll
         for (int d = 0; d < PC_AHEAD; ++d)
@@ -795,7 +795,7 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_kernel(const GemmParams p)
                 if (c >= chunks) break;                 // uniform
                 uint8_t* half = lds_ab[c & 1];
                 split_store<MODE>(half, ptid, ra[d], guard);
-                split_store<MODE>(half + STAGE, ptid, rb[d], guard);
+                split_store<BMODE>(half + STAGE, ptid, rb[d], guard);
                 if (c + PC_AHEAD < chunks) load_both(c + PC_AHEAD, ra[d], rb[d]);
                 __syncthreads();
             }
@@ -2270,6 +2270,16 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
             else              { if (p.stream_c) PPML_KFAST(true, false); else PPML_KFAST(false, false); }
 #undef PPML_KFAST
         }
+        // A contiguous in k, B contiguous in its rows, dense output planes below 2 GiB (the backward of the triangle
+        // multiplication): the loading / contracting form with a loader per operand, whatever the number of tiles
+        else if (p.a_ks == 1 && p.b_rs == 1 && p.a_lm == 0 && !split && p.c_ni == 1 && p.K > BK &&
+                 ((p.M - 1) * p.a_rs + p.K) * 4 < (1LL << 31) && p.K * p.b_ks * 4 < (1LL << 31) && p.M * p.c_mi * 4 < (1LL << 31) &&
+                 p.c_mi < (1 << 22) && p.a_rs < (1 << 22) && p.b_ks < (1 << 24)) {
+#define PPML_MIXED(STREAM_, K4_) hipLaunchKernelGGL((gemm_bf16x3_pc_kernel<LOAD_K_CONTIG, STREAM_, K4_, LOAD_ROW_CONTIG>), grid, dim3(512), 0, stream, p)
+            if (p.K % 4 == 0) { if (p.stream_c) PPML_MIXED(true, true); else PPML_MIXED(false, true); }
+            else              { if (p.stream_c) PPML_MIXED(true, false); else PPML_MIXED(false, false); }
+#undef PPML_MIXED
+        }
         else if (mode == LOAD_K_CONTIG)   { if (split) PPML_LAUNCH_BF16(LOAD_K_CONTIG, true);   else PPML_LAUNCH_BF16(LOAD_K_CONTIG, false); }
         else if (mode == LOAD_ROW_CONTIG) { if (split) PPML_LAUNCH_BF16(LOAD_ROW_CONTIG, true); else PPML_LAUNCH_BF16(LOAD_ROW_CONTIG, false); }
         else                              { if (split) PPML_LAUNCH_BF16(LOAD_STRIDED, true);    else PPML_LAUNCH_BF16(LOAD_STRIDED, false); }
@@ -2569,13 +2579,17 @@ extern "C" int tri_mul_back_hip(const float* grad, const float* left, const floa
                             int64_t a_p3, int64_t b_p3, int64_t c_p3) {
         StatsScope stat("hip/tri_mul_back", M, Kc, N, static_cast<hipStream_t>(stream));
         GemmParams p = plain_params();
-        p.A = a; p.B = b; p.C = c;
-        p.M = static_cast<int>(M); p.N = static_cast<int>(N); p.K = static_cast<int>(Kc);
-        p.a_rs = a_rs * B; p.a_ks = a_ks * B; p.b_rs = b_rs * B; p.b_ks = b_ks * B;
-        p.c_mi = c_mi * B; p.c_ni = c_ni * B;
+        // an output whose ROW index runs along memory is the dense plane of the transposed product: the operands trade
+        // places (the fast forms of the contraction store dense planes)
+        const bool swap = c_mi == 1 && c_ni != 1;
+        p.A = swap ? b : a; p.B = swap ? a : b; p.C = c;
+        p.M = static_cast<int>(swap ? N : M); p.N = static_cast<int>(swap ? M : N); p.K = static_cast<int>(Kc);
+        p.a_rs = (swap ? b_rs : a_rs) * B; p.a_ks = (swap ? b_ks : a_ks) * B;
+        p.b_rs = (swap ? a_rs : b_rs) * B; p.b_ks = (swap ? a_ks : b_ks) * B;
+        p.c_mi = (swap ? c_ni : c_mi) * B; p.c_ni = (swap ? c_mi : c_ni) * B;
         p.np2 = static_cast<int>(B); p.np3 = static_cast<int>(D);
         p.a_p2 = 1; p.b_p2 = 1; p.c_p2 = 1;
-        p.a_p3 = a_p3 * B; p.b_p3 = b_p3 * B; p.c_p3 = c_p3 * B;
+        p.a_p3 = (swap ? b_p3 : a_p3) * B; p.b_p3 = (swap ? a_p3 : b_p3) * B; p.c_p3 = c_p3 * B;
         p.alpha = inv_L;
         return launch_gemm(p, static_cast<hipStream_t>(stream), "tri_mul_back_hip");
     };
