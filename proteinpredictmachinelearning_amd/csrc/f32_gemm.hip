@@ -630,8 +630,8 @@ __device__ __forceinline__ void store_acc_buffer(const __amdgpu_buffer_rsrc_t rs
 
 template <int MODE, bool SPLIT_C, bool STREAM_C, bool FAST_IO = false, bool K4 = true>
 __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
-    static_assert(!FAST_IO || ((MODE == LOAD_ROW_CONTIG || MODE == LOAD_K_CONTIG) && !SPLIT_C),
-                  "buffer addressing: rows contiguous in themselves or in k, dense output");
+    // (FAST_IO with SPLIT_C: buffer-addressed loads, the output by its compound addressing)
+    static_assert(!FAST_IO || MODE == LOAD_ROW_CONTIG || MODE == LOAD_K_CONTIG, "buffer addressing: rows contiguous in themselves or in k");
     __shared__ __attribute__((aligned(16))) uint8_t lds_a[3 * SPLIT_PLANE];
     __shared__ __attribute__((aligned(16))) uint8_t lds_b[3 * SPLIT_PLANE];
 
@@ -667,7 +667,7 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
         const int64_t b_plane = MODE == LOAD_K_CONTIG ? (p.N - 1) * p.b_rs + p.K : p.K * p.b_ks;
         rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, static_cast<int>(a_plane * 4), 0x00020000);
         rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, static_cast<int>(b_plane * 4), 0x00020000);
-        rsrc_c = __builtin_amdgcn_make_buffer_rsrc(C, 0, static_cast<int>(p.M * p.c_mi * 4), 0x00020000);
+        if (!SPLIT_C) rsrc_c = __builtin_amdgcn_make_buffer_rsrc(C, 0, static_cast<int>(p.M * p.c_mi * 4), 0x00020000);
     }
     const auto load_both = [&](int k0) {
         if (FAST_IO && MODE == LOAD_K_CONTIG) {
@@ -722,7 +722,7 @@ __global__ __launch_bounds__(256) void gemm_bf16x3_kernel(const GemmParams p) {
         return;
     }
 
-    if (FAST_IO) store_acc_buffer<STREAM_C>(rsrc_c, static_cast<uint32_t>(p.c_mi) * 4u, p.N, p.alpha, acc, m0 + wm, n0 + wn, lane);
+    if (FAST_IO && !SPLIT_C) store_acc_buffer<STREAM_C>(rsrc_c, static_cast<uint32_t>(p.c_mi) * 4u, p.N, p.alpha, acc, m0 + wm, n0 + wn, lane);
     else store_acc<SPLIT_C, STREAM_C, false, false>(p, C, acc, m0 + wm, n0 + wn, lane);
 }
 
@@ -2269,6 +2269,20 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
             if (p.K % 4 == 0) { if (p.stream_c) PPML_KFAST(true, true); else PPML_KFAST(false, true); }
             else              { if (p.stream_c) PPML_KFAST(true, false); else PPML_KFAST(false, false); }
 #undef PPML_KFAST
+        }
+        // an output with compound addressing (the outer-product-mean in its graph and value forms) over operand planes
+        // below 2 GiB that are contiguous in k or in their rows: buffer-addressed loads, the generic store
+        else if (split && p.a_lm == 0 && mode == LOAD_K_CONTIG && ((p.M - 1) * p.a_rs + p.K) * 4 < (1LL << 31) &&
+                 ((p.N - 1) * p.b_rs + p.K) * 4 < (1LL << 31) && p.a_rs < (1 << 22) && p.b_rs < (1 << 22)) {
+#define PPML_KFAST_SPLIT(STREAM_, K4_) hipLaunchKernelGGL((gemm_bf16x3_kernel<LOAD_K_CONTIG, true, STREAM_, true, K4_>), grid, block, 0, stream, p)
+            if (p.K % 4 == 0) { if (p.stream_c) PPML_KFAST_SPLIT(true, true); else PPML_KFAST_SPLIT(false, true); }
+            else              { if (p.stream_c) PPML_KFAST_SPLIT(true, false); else PPML_KFAST_SPLIT(false, false); }
+#undef PPML_KFAST_SPLIT
+        }
+        else if (split && p.a_lm == 0 && mode == LOAD_ROW_CONTIG && p.K * p.a_ks * 4 < (1LL << 31) && p.K * p.b_ks * 4 < (1LL << 31) &&
+                 p.a_ks < (1 << 24) && p.b_ks < (1 << 24)) {
+            if (p.stream_c) hipLaunchKernelGGL((gemm_bf16x3_kernel<LOAD_ROW_CONTIG, true, true, true>), grid, block, 0, stream, p);
+            else hipLaunchKernelGGL((gemm_bf16x3_kernel<LOAD_ROW_CONTIG, true, false, true>), grid, block, 0, stream, p);
         }
         // A contiguous in k, B contiguous in its rows, dense output planes below 2 GiB (the backward of the triangle
         // multiplication): the loading / contracting form with a loader per operand, whatever the number of tiles
