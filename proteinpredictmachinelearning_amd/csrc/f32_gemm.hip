@@ -853,11 +853,12 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_kernel(const GemmParams p)
 // gemm_bf16x3_pc_kernel for a few output tiles under a long K (a LinearLayer's weight gradient: 256 x 768 outputs over
 // 26368 tokens -- twelve tiles): the K loop is cut into slices, one work-group per (tile, slice) -- the tile numbering
 // takes the slice for the plane --, raw sums go to partial[slice][m][n] and reduce_slices_kernel adds them in slice
-// order, applies bias, factor and the output's addressing.  A slice whose split could not carry an operand flags the
-// tile's rows (fired_a, one per 32 rows) and reduce_slices_kernel computes those the reference's way.
+// order, applies bias, factor and the output's addressing.  A slice whose split could not carry an operand leaves NaN
+// for its whole tile, and reduce_slices_kernel computes every output whose sum is NaN the reference's way (no flags to
+// clear ahead: one launch less).
 template <int MODE, bool K4>
 __global__ __launch_bounds__(512) void gemm_bf16x3_pc_slices_kernel(const GemmParams p, int chunks, int slice_chunks, float* __restrict__ partial,
-                                                                    int ma_pad, int nb_pad, int* __restrict__ fired_a) {
+                                                                    int ma_pad, int nb_pad) {
     static_assert(MODE == LOAD_ROW_CONTIG || MODE == LOAD_K_CONTIG, "buffer addressing");
     constexpr int STAGE = 3 * SPLIT_PLANE;
     __shared__ __attribute__((aligned(16))) uint8_t lds_ab[2][2 * STAGE];
@@ -882,6 +883,8 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_slices_kernel(const GemmPa
     const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.B), 0, static_cast<int>(b_plane * 4), 0x00020000);
 
     // (barriers: nch + 1 in either loop, as in gemm_bf16x3_pc_kernel)
+    int fired = 0;
+    v16f acc[2][2];
     if (producer) {
         v4f ra[PC_AHEAD][2], rb[PC_AHEAD][2];
         const auto load_both = [&](int c, v4f (&xa)[2], v4f (&xb)[2]) {
@@ -910,14 +913,8 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_slices_kernel(const GemmPa
             }
         }
         __syncthreads();
-        if (guard.fired()) {                            // (either operand: the tile's rows; every writer writes the same value)
-#pragma unroll
-            for (int i = 0; i < BM / 32; ++i) fired_a[(m0 >> 5) + i] = 1;
-        }
-        return;
-    }
-
-    v16f acc[2][2];
+        fired = guard.fired() ? 1 : 0;
+    } else {
 #pragma unroll
     for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
@@ -946,14 +943,18 @@ __global__ __launch_bounds__(512) void gemm_bf16x3_pc_slices_kernel(const GemmPa
                     acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][SPLIT_TERMS[q][0]], fb[tj][SPLIT_TERMS[q][1]], acc[ti][tj], 0, 0, 0);
         __syncthreads();                                // chunk c has been read; chunk c + 1 is in LDS
     }
-    // raw sums of this slice: the padded workspace takes every row and column of the tile
+    }
+    const bool again = __syncthreads_or(fired) != 0;    // an operand of this tile and slice that the split could not carry
+    if (producer) return;
+    // raw sums of this slice (NaN for a tile to be computed again): the padded workspace takes every row and column of the tile
     float* dst = partial + (static_cast<size_t>(slice) * ma_pad + m0 + wm + 4 * hh) * nb_pad + n0 + wn + j;
+    const float nan = __builtin_nanf("");
 #pragma unroll
     for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
         for (int tj = 0; tj < 2; ++tj)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) dst[static_cast<size_t>(ti * 32 + 8 * (r >> 2) + (r & 3)) * nb_pad + tj * 32] = acc[ti][tj][r];
+            for (int r = 0; r < 16; ++r) dst[static_cast<size_t>(ti * 32 + 8 * (r >> 2) + (r & 3)) * nb_pad + tj * 32] = again ? nan : acc[ti][tj][r];
 }
 
 // The same again for contractions with one NARROW side: at most 32 rows of A (SIDE_M: the second contraction of the
@@ -1883,9 +1884,11 @@ __global__ __launch_bounds__(256) void reduce_slices_kernel(const GemmParams p, 
     }
     const float* src = partial + static_cast<size_t>(m) * nb_pad + n4;          // nb_pad is a multiple of 128
     for (int s = 0; s < slices; ++s) sum += *reinterpret_cast<const v4f*>(src + static_cast<size_t>(s) * ma_pad * nb_pad);
-    if (fired_a[m >> 5] | fired_b[n4 >> 5]) {           // operands the split could not carry: these four again, the reference's way
+    // operands the split could not carry: these four again, the reference's way -- by the flags of the splits, or
+    // (callers that pass none) wherever the slices' sum is NaN, which is what a slice leaves for such a tile
+    if (fired_a ? (fired_a[m >> 5] | fired_b[n4 >> 5]) != 0 : (sum[0] != sum[0] || sum[1] != sum[1] || sum[2] != sum[2] || sum[3] != sum[3])) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) if (n4 + c < p.N) sum[c] = plain_dot(p, p.A, p.B, m, n4 + c);
+        for (int c = 0; c < 4; ++c) if (n4 + c < p.N && (fired_a || sum[c] != sum[c])) sum[c] = plain_dot(p, p.A, p.B, m, n4 + c);
     }
     int64_t roff;
     if (SPLIT_C) roff = static_cast<int64_t>(m / p.c_lm) * p.c_mo + static_cast<int64_t>(m % p.c_lm) * p.c_mi;
@@ -2002,10 +2005,10 @@ template <int MODE>
 int try_pc_slices(const GemmParams& p, hipStream_t stream, const char* what) {
     const int chunks = (p.K + BK - 1) / BK;
     const int groups = p.tiles_m * p.tiles_n;
-    // (three launches: about 12 us before the first chunk.  us over K for one to nine tiles, unsliced: 256 12, 400 16.5,
-    // 512 20, 640 24, 752 27; in slices: 784 and 1024 16.5-17, 2048 18-19)
-    constexpr int LEAST = 8;                            // chunks a slice is long at least
-    // (64 tiles of 128 x 128 under K = 512 measured 23.0 against 20.4 unsliced, under K = 784 24.7 against 28.9)
+    // (two launches: about 10 us before the first chunk.  us over K for one to nine tiles, unsliced: 256 12, 400 16.5,
+    // 512 20, 640 24, 752 27; in slices: 512 ... 1024 12.8-14, 2048 15-19)
+    constexpr int LEAST = 6;                            // chunks a slice is long at least
+    // (64 tiles of 128 x 128 under K = 512 measured 21.6 against 20.4 unsliced, under K = 640 22.7 against 24.3)
     if (p.np2 * p.np3 != 1 || groups * 2 > device_cu_count() || chunks < (groups * 4 <= device_cu_count() ? 4 * LEAST : 6 * LEAST)) return -1;
     int slices = even_slices(groups, chunks, 128, LEAST);
     if (slices < 2) return -1;
@@ -2013,30 +2016,22 @@ int try_pc_slices(const GemmParams& p, hipStream_t stream, const char* what) {
     slices = (chunks + slice_chunks - 1) / slice_chunks;
     const int ma_pad = p.tiles_m * BM, nb_pad = p.tiles_n * BN;
     const size_t part_bytes = static_cast<size_t>(slices) * ma_pad * nb_pad * 4;
-    const int n_flags = ma_pad / 32 + nb_pad / 32;
-    const size_t flag_bytes = (static_cast<size_t>(n_flags) * 4 + 255) / 256 * 256;
-    const Workspace held = workspace_take(part_bytes + flag_bytes, stream);
+    const Workspace held = workspace_take(part_bytes, stream);
     uint8_t* ws = held.ptr;
     if (!ws) return -1;
     float* partial = reinterpret_cast<float*>(ws);
-    int* fired_a = reinterpret_cast<int*>(ws + part_bytes);
-    int* fired_b = fired_a + ma_pad / 32;               // (stays clear: the kernel flags rows for either operand)
     GemmParams q = p;
     q.np2 = slices;                                      // the tile numbering walks the slices as planes
     const dim3 grid(static_cast<unsigned>(groups * slices)), block(512);
-    hipLaunchKernelGGL(clear_flags_kernel, dim3((n_flags + 255) / 256), dim3(256), 0, stream, fired_a, n_flags);
+    if (MODE == LOAD_K_CONTIG && p.K % 4 != 0)
+        hipLaunchKernelGGL((gemm_bf16x3_pc_slices_kernel<MODE, false>), grid, block, 0, stream, q, chunks, slice_chunks, partial, ma_pad, nb_pad);
+    else
+        hipLaunchKernelGGL((gemm_bf16x3_pc_slices_kernel<MODE, true>), grid, block, 0, stream, q, chunks, slice_chunks, partial, ma_pad, nb_pad);
     int rc = check_launch(what);
-    if (rc == RC_OK) {
-        if (MODE == LOAD_K_CONTIG && p.K % 4 != 0)
-            hipLaunchKernelGGL((gemm_bf16x3_pc_slices_kernel<MODE, false>), grid, block, 0, stream, q, chunks, slice_chunks, partial, ma_pad, nb_pad, fired_a);
-        else
-            hipLaunchKernelGGL((gemm_bf16x3_pc_slices_kernel<MODE, true>), grid, block, 0, stream, q, chunks, slice_chunks, partial, ma_pad, nb_pad, fired_a);
-        rc = check_launch(what);
-    }
     if (rc == RC_OK) {
         const int64_t threads = static_cast<int64_t>(p.M) * ((p.N + 3) / 4);
         hipLaunchKernelGGL((reduce_slices_kernel<false>), dim3(static_cast<unsigned>((threads + 255) / 256)), dim3(256), 0, stream, p, partial, slices,
-                           ma_pad, nb_pad, fired_a, fired_b);
+                           ma_pad, nb_pad, static_cast<const int*>(nullptr), static_cast<const int*>(nullptr));
         rc = check_launch(what);
     }
     workspace_give(held, stream);
