@@ -1319,7 +1319,7 @@ __global__ __launch_bounds__(512, 2) void gemm_bf16x3_half_split_kernel(const Ge
 // sixteen bytes per lane, a store instruction writing two 512-byte runs instead of two lines.
 constexpr int C_ORDINARY = 0, C_STREAM = 1, C_FLAT = 2, C_ROWS = 3;
 template <int TM, int C_FORM>
-__global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmParams p, int total_tiles) {
+__global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmParams p, int total_tiles, uint32_t launch_mark) {
     static_assert(TM == 64 || TM == 128, "tile side");
     constexpr int WT = TM / 2;                        // a wave's square of the tile
     constexpr int NT = WT / 32;                       // 32 x 32 accumulator tiles per side of it
@@ -1328,14 +1328,17 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
     constexpr int LOADS = TM == 128 ? 2 : 1;          // 16-k chunks a thread loads separately (at 64 rows one pass covers K = 32)
     static_assert(2 * OPERAND >= (TM * TM + 32) * 4, "a whole tile of C, shifted by up to a line, fits the operands' LDS");
     __shared__ __attribute__((aligned(128))) uint8_t lds_ab[2 * OPERAND];
-    // "A SplitGuard fired for tile t": a thread whose guard fires writes t + 1 into the word of t's turn, and after the
-    // barrier everybody compares.  Within a launch a tile number never comes back to a work-group.  LDS keeps what
-    // earlier kernels left there, and work-groups land on the same CUs launch after launch: a mark left behind would
-    // match the same tile number in every later launch of the shape and send that tile down the plain path each time
-    // (right results, fifteen times the time).  So a work-group that saw a mark clears both words before it ends; a
-    // word that happens to hold a tile number for any other reason costs one needless pass and is cleared by it.
-    // (Clearing them when the kernel starts takes a barrier in front of the first split: 0.3 us per launch.)
-    __shared__ int lds_guard[2];
+    // "A SplitGuard fired for tile t": a thread whose guard fires writes a mark into the word of t's turn, and after
+    // the barrier everybody compares.  LDS keeps what earlier kernels left there -- this kernel's own marks
+    // (work-groups land on the same CUs launch after launch) and whatever other kernels kept at these addresses, which
+    // may well look like a tile number: a word taken for a mark sends its tile down the plain path (right results, the
+    // other path's bits, fifteen times the time).  So a mark is a word that nothing else writes -- a scrambled count
+    // of the host's launches (the kernel's last argument) with the tile's number folded in --, and a work-group that
+    // saw one clears the words before it ends (a captured graph replays the same launch number).  What is left is one
+    // chance in 2^32 per tile that leftover data is taken for a mark: that tile then has the other path's bits, once.
+    // (Clearing the words when the kernel starts takes a barrier in front of the first split, or a mark written behind
+    // the split's barrier: 0.2 to 0.35 us per launch either way; a second word to compare, about as much.)
+    __shared__ uint32_t lds_guard[2];
     uint8_t* const lds_a = lds_ab;
     uint8_t* const lds_b = lds_ab + OPERAND;
 
@@ -1392,7 +1395,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
         }
     };
     // a lane's share goes to the three planes of its chunk: row lrow, bytes 16 * (octet % 2) of the row's 32
-    const auto split_to_lds = [&](int* fired, int mark) {
+    const auto split_to_lds = [&](uint32_t* fired, uint32_t mark) {
         SplitGuard guard;
 #pragma unroll
         for (int l = 0; l < LOADS; ++l) {
@@ -1431,8 +1434,9 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
         // That keeps the test and the other path's code out of the chain load -> split -> MFMA -> store that a
         // work-group with one tile consists of (decided ahead of the matrix work it cost half a microsecond per
         // launch; with the other path inline behind the stores, a third).
-        int* const mark_word = &lds_guard[turn];
-        split_to_lds(mark_word, t + 1);
+        uint32_t* const mark_word = &lds_guard[turn];
+        const uint32_t mark = launch_mark ^ static_cast<uint32_t>(t + 1);
+        split_to_lds(mark_word, mark);
         __syncthreads();
         turn ^= 1;
         const int t_next = t + groups;
@@ -1468,7 +1472,7 @@ __global__ __launch_bounds__(256, 2) void gemm_bf16x3_shortk_kernel(const GemmPa
                         acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ti][SPLIT_TERMS[q][0]], fb[tj][SPLIT_TERMS[q][1]], acc[ti][tj], 0, 0, 0);
         }
         __syncthreads();                                // the planes may be overwritten
-        if (__builtin_amdgcn_readfirstlane(*mark_word) == t + 1) fired_its |= 1ull << (it < 63 ? it : 63);   // uniform over the work-group
+        if (__builtin_amdgcn_readfirstlane(*mark_word) == mark) fired_its |= 1ull << (it < 63 ? it : 63);   // uniform over the work-group
         ++it;
         // ---- stores of this tile: younger than the next tile's loads
         if (C_FORM == C_FLAT) {
@@ -2199,7 +2203,11 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
                 // rows that one tile spans lose the round trip: 2000 planes of 128 x 128 30.2 / 31.4, 100 of them 4.8 / 5.5).
                 const bool rows = p.stream_c && big && p.N > tm;
                 const int form = rows ? C_ROWS : p.stream_c ? C_STREAM : flat ? C_FLAT : C_ORDINARY;
-#define PPML_SHORTK(TM_, FORM_) hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<TM_, FORM_>), pgrid, block, 0, stream, p, static_cast<int>(tiles))
+                // (the number of this launch: see lds_guard in the kernel)
+                static std::atomic<uint64_t> launches{0};
+                const uint64_t launch = launches.fetch_add(1, std::memory_order_relaxed) + 1;
+                const uint32_t launch_mark = (static_cast<uint32_t>(launch) ^ static_cast<uint32_t>(launch >> 32)) * 0x9e3779b1u ^ 0x85ebca6bu;
+#define PPML_SHORTK(TM_, FORM_) hipLaunchKernelGGL((gemm_bf16x3_shortk_kernel<TM_, FORM_>), pgrid, block, 0, stream, p, static_cast<int>(tiles), launch_mark)
                 if (form == C_ROWS) PPML_SHORTK(128, C_ROWS);
                 else if (big) { if (form == C_STREAM) PPML_SHORTK(128, C_STREAM); else if (form == C_FLAT) PPML_SHORTK(128, C_FLAT); else PPML_SHORTK(128, C_ORDINARY); }
                 else     { if (form == C_STREAM) PPML_SHORTK(64, C_STREAM);  else if (form == C_FLAT) PPML_SHORTK(64, C_FLAT);  else PPML_SHORTK(64, C_ORDINARY); }
