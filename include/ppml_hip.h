@@ -69,8 +69,10 @@ int ppml_hip_set_f32_arithmetic(int mode);
  * loop): +-inf, NaN and the bits down to 2^-149 come out as the reference's.  The fused attention kernels
  * (flash_attn_*_hip) split without that check; ppml_hip_set_f32_arithmetic(1) selects the fp32 pipe, which
  * carries every operand, for all of them.  Contractions of at
- * least 512 work-groups of 256 x 128 outputs take a workspace of 6 bytes per operand element from a
- * stream-ordered pool (allocated and freed on `stream`); no other launcher allocates. */
+ * least 512 work-groups of 256 x 128 outputs (6 bytes per operand element) and contractions of few output
+ * tiles under a long K (the partial sums of their K slices) use a workspace from a stream-ordered pool of
+ * the library's; a stream keeps one such buffer between calls (a stream under capture and the per-thread
+ * default stream allocate and release per call). */
 int mul_mat_hip(const float *A, const float *B, float *C, int M, int K, int N,
                 const float *bias, ppml_hip_stream_t stream);
 
@@ -285,8 +287,8 @@ int permute_hip(const float *src, float *dst, int64_t total, int ndim,
  * is the node the backward of a biased mul_mat emits for the bias: grad [N, M] -> dbias [N]
  * (src/core/ComputeGraph.cpp:742).  The reference adds the copies one at a time, k3 fastest; here that
  * sequence is cut into consecutive runs summed side by side and added in run order (a fixed bracketing,
- * no atomics).  With few destination elements and many copies the partial sums take a workspace from the
- * library's stream-ordered pool.  returns 0 ok, 1 bad arguments (a copy outside the source), 6 launch error. */
+ * no atomics).  With few destination elements and many copies the partial sums take the stream's workspace
+ * (see mul_mat_hip).  returns 0 ok, 1 bad arguments (a copy outside the source), 6 launch error. */
 int repeat_back_hip(const float *src, float *dst,
                     int64_t s0, int64_t s1, int64_t s2, int64_t s3,
                     int64_t d0, int64_t d1, int64_t d2, int64_t d3,
