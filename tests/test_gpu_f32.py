@@ -834,6 +834,47 @@ def test_weight_gradients_of_linear_layers_go_in_k_slices(ops, oracle, T, K, N):
         assert np.isinf(got2[5, :N - 1]).all() and np.isinf(np.delete(got2[:, N - 1], 5)).all()      # (where the two meet: inf - inf)
 
 
+def test_workspace_users_from_several_threads_and_streams(ops):
+    """The launchers that use a workspace keep one buffer per stream between calls: calls from several host threads, each
+    on a stream of its own, and from two threads that share one stream, with sizes that make the buffer grow and shrink
+    in turn, all give the results of the same calls made one after the other."""
+    import threading
+    torch.manual_seed(21)
+    cases = []
+    for T, K, N in ((5000, 100, 130), (26368, 64, 48), (3001, 33, 7), (9000, 256, 256)):
+        x, dy = torch.randn(T, K, device="cuda"), torch.randn(T, N, device="cuda")
+        cases.append((x, dy, ops.mul_mat_tn(x, dy).clone()))
+    g = torch.randn(26368, 96, device="cuda")
+    bias_ref = ops.repeat_back(g, (96,)).clone()
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    errors = []
+
+    def work(stream, seed):
+        try:
+            rng = np.random.default_rng(seed)
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    i = int(rng.integers(len(cases)))
+                    x, dy, ref = cases[i]
+                    out = ops.mul_mat_tn(x, dy)
+                    db = ops.repeat_back(g, (96,))
+                    stream.synchronize()
+                    if not torch.equal(out, ref) or not torch.equal(db, bias_ref):
+                        errors.append((seed, i))
+        except Exception as e:                         # noqa: BLE001 -- reported below
+            errors.append((seed, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(streams[0], 1)), threading.Thread(target=work, args=(streams[1], 2)),
+               threading.Thread(target=work, args=(streams[2], 3)), threading.Thread(target=work, args=(streams[2], 4))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+
+
 @pytest.mark.parametrize("L", [48, 51])
 @pytest.mark.parametrize("kind", ["inf", "tiny"])
 def test_outer_prod_mean_back_carries_what_the_split_cannot(ops, oracle, kind, L):
