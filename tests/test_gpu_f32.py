@@ -834,6 +834,37 @@ def test_weight_gradients_of_linear_layers_go_in_k_slices(ops, oracle, T, K, N):
         assert np.isinf(got2[5, :N - 1]).all() and np.isinf(np.delete(got2[:, N - 1], 5)).all()      # (where the two meet: inf - inf)
 
 
+def test_operands_at_any_four_byte_alignment(ops):
+    """Operand and output buffers that start one, two or three floats behind a 16-byte boundary (views into larger
+    allocations): the same bits as on aligned copies, for the launchers whose kernels load sixteen bytes at a time."""
+    torch.manual_seed(8)
+
+    def shifted(t, off):
+        flat = torch.empty(t.numel() + 4, device="cuda")
+        v = flat[off:off + t.numel()].view(t.shape)
+        v.copy_(t)
+        assert v.data_ptr() % 16 == (t.data_ptr() + 4 * off) % 16
+        return v
+
+    for off in (1, 2, 3):
+        for M, K, N in ((300, 256, 200), (26368, 256, 16), (130, 64, 32), (2000, 100, 7)):
+            a, b, bias = torch.randn(M, K, device="cuda"), torch.randn(N, K, device="cuda"), torch.randn(N, device="cuda")
+            want = ops.mul_mat(a, b, bias)
+            got = ops.mul_mat(shifted(a, off), shifted(b, (off + 1) % 4), shifted(bias, off))
+            assert torch.equal(got.view(torch.int32), want.view(torch.int32)), (off, M, K, N)
+        x, dy = torch.randn(5000, 100, device="cuda"), torch.randn(5000, 130, device="cuda")
+        assert torch.equal(ops.mul_mat_tn(shifted(x, off), shifted(dy, off)).view(torch.int32), ops.mul_mat_tn(x, dy).view(torch.int32))
+        D, L, N = 8, 48, 64
+        g, l, r = torch.randn(D * D * L * L, device="cuda"), torch.randn(D * L * N, device="cuda"), torch.randn(D * L * N, device="cuda")
+        wl, wr = ops.outer_prod_mean_back(g, l, r, D, L, N, 1)
+        gl, gr = ops.outer_prod_mean_back(shifted(g, off), shifted(l, off), shifted(r, (off + 2) % 4), D, L, N, 1)
+        assert torch.equal(gl.view(torch.int32), wl.view(torch.int32)) and torch.equal(gr.view(torch.int32), wr.view(torch.int32))
+        k, q = torch.randn(1, 40, 32, 103, device="cuda"), torch.randn(1, 40, 32, 103, device="cuda")
+        assert torch.equal(ops.out_prod(shifted(k, off), shifted(q, off), scale=0.25).view(torch.int32), ops.out_prod(k, q, scale=0.25).view(torch.int32))
+        a3, v3 = torch.rand(1, 7, 51, 51, device="cuda"), torch.randn(1, 7, 32, 51, device="cuda")
+        assert torch.equal(ops.out_prod_tt(shifted(a3, off), shifted(v3, off)).view(torch.int32), ops.out_prod_tt(a3, v3).view(torch.int32))
+
+
 def test_workspace_users_from_several_threads_and_streams(ops):
     """The launchers that use a workspace keep one buffer per stream between calls: calls from several host threads, each
     on a stream of its own, and from two threads that share one stream, with sizes that make the buffer grow and shrink
