@@ -296,6 +296,8 @@ def main() -> int:
                            "GBps": round(nbytes / e_ / 1e9, 1), "hbm_frac": round(nbytes / e_ / 1e9 / HBM_PEAK_GBS, 4)}
             if pipe == "bf16x3":
                 extra[name]["bf16_mfma_frac"] = round(6.0 * flops / e_ / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4)
+            elif pipe == "f16":                         # halves straight to the matrix pipe (same published peak as bf16)
+                extra[name]["f16_mfma_frac"] = round(flops / e_ / 1e12 / BF16_MFMA_PEAK_TFLOPS, 4)
             else:
                 extra[name]["fp32_mfma_frac"] = round(flops / e_ / 1e12 / FP32_MFMA_PEAK_TFLOPS, 4)
             if rw is not None:                          # (bytes read, bytes written) of an HBM-bound shape
@@ -502,6 +504,16 @@ def main() -> int:
         steps, warm = 50, 10
         f32_case(weight_grad, (26368 * 256 + 26368 * 768 + 256 * 768) * 4, 2.0 * 26368 * 256 * 768,
                  "linear_weight_gradient_26368x256_768", pipe="bf16x3")
+
+        def f16_linear():
+            # the headline projection with both operands in halves (F16 x F16 -> F32, src/backend/CPUKernels.cpp:646-672)
+            ns = 8
+            xs = [torch.randn(26368, 256, device=dev, generator=gen).half() for _ in range(ns)]
+            w16 = (torch.randn(768, 256, device=dev, generator=gen) * 0.05).half()
+            keep.append((xs, w16))
+            return (lambda i: ops.mul_mat_f16(xs[i], w16)), ns
+        f32_case(f16_linear, 26368 * 256 * 2 + 768 * 256 * 2 + 26368 * 768 * 4, 2.0 * 26368 * 256 * 768,
+                 "mul_mat_f16_26368x256_768", pipe="f16")
 
         def bias_grad():
             # dbias[n] = sum over the tokens of dY[token][n] (OP_REPEAT_BACK, src/backend/CPUKernels.cpp:2091-2148)

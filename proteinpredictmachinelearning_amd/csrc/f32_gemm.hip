@@ -604,9 +604,12 @@ __device__ __forceinline__ void load_kcontig_buffer(const __amdgpu_buffer_rsrc_t
 }
 
 // The finished accumulators of one wave to a dense plane C[m * ld + n] through a buffer resource over the plane.
-template <bool STREAM_C>
+// (TAIL: tail[tj] joins the finished sums of the lane's column in tile column tj -- a bias that is added last; the
+// caller has loaded it long before: a load here would be waited for with a count that every earlier store is part of)
+template <bool STREAM_C, bool TAIL = false>
 __device__ __forceinline__ void store_acc_buffer(const __amdgpu_buffer_rsrc_t rsrc, uint32_t ld_bytes, int N, float alpha,
-                                                 const v16f (&acc)[2][2], int m_base, int n_base, int lane) {
+                                                 const v16f (&acc)[2][2], int m_base, int n_base, int lane,
+                                                 float tail0 = 0.0f, float tail1 = 0.0f) {
     const int j = lane & 31;
     const bool scale = alpha != 1.0f;
 #pragma unroll
@@ -617,10 +620,12 @@ __device__ __forceinline__ void store_acc_buffer(const __amdgpu_buffer_rsrc_t rs
             const int n = n_base + tj * 32 + j;
             // rows past the matrix fall outside the plane by themselves (offset >= M * ld bytes)
             const uint32_t base = n < N ? first * ld_bytes + static_cast<uint32_t>(n) * 4u : OUTSIDE;
+            const float tail = tj ? tail1 : tail0;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 float v = acc[ti][tj][r];
                 if (scale) v *= alpha;
+                if (TAIL) v += tail;
                 __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rsrc, base + (8 * (r >> 2) + (r & 3)) * ld_bytes, 0,
                                                       STREAM_C ? 3 : 0);
             }
@@ -1683,6 +1688,151 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const GemmParams p) {
     store_acc<false, STREAM_C, true, false>(p, p.C, acc, m0 + wm, n0 + wn, lane);
 }
 
+// The same contraction as a stream of tiles through resident work-groups whose waves divide the work: waves 4..7 only
+// load (global -> registers, F16P_AHEAD stages of 64 k ahead, -> the other half of a double buffer in LDS) and waves
+// 0..3 only read fragments, issue MFMAs and store finished tiles.  In gemm_f16_kernel every work-group of a round
+// loads, contracts and stores at the same time as all the others, so the memory system sees a burst of loads and then
+// a burst of stores, and a tile's four stages of K = 256 are four exposed round trips; here the loading waves run on
+// into the next tile while the contracting waves store (they issue no loads, so nothing of theirs ever waits for a
+// store), and a CU holds two such work-groups.  Tiles go to the XCDs in eight contiguous ranges, inside a range in
+// bands of eight tile rows, so that the work-groups resident on an XCD at one time share operand panels in its L2.
+// Same fragments, same order of the products, zero start and bias last as in gemm_f16_kernel: same bits.
+// Conditions (the launcher's): K, both row pitches and both base addresses multiples of eight halves -- every load
+// is sixteen bytes that lie inside one row or entirely past K --, operands and the dense output each below 2 GiB
+// (buffer addressing: what lies outside reads as zero and is not stored), a grid that is a multiple of eight.
+constexpr int F16P_AHEAD = 2;    // (three measured the same or 0.5 us slower: a longer start and end per work-group)
+constexpr int F16P_STAGE = (BM + BN) * F16_PITCH;     // A's tile, then B's
+template <bool STREAM_C>
+__global__ __launch_bounds__(512, 2) void gemm_f16_pc_kernel(const GemmParams p, int total_tiles) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][F16P_STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool producer = wave >= 4;
+    const int chunks = (p.K + F16_BK - 1) / F16_BK;
+
+    // this work-group's tiles: first, first + step, ... below hi
+    const int xcd = blockIdx.x & 7, step = gridDim.x >> 3;
+    const int lo = static_cast<int>(static_cast<int64_t>(total_tiles) * xcd / 8);
+    const int hi = static_cast<int>(static_cast<int64_t>(total_tiles) * (xcd + 1) / 8);
+    const int first = lo + static_cast<int>(blockIdx.x >> 3);
+    const int my_tiles = first < hi ? (hi - first + step - 1) / step : 0;
+    const int total = my_tiles * chunks;              // stages this work-group contracts ...
+    const int padded = (total + F16P_AHEAD - 1) / F16P_AHEAD * F16P_AHEAD;   // ... and passes
+    const auto tile_origin = [&](int t, int& m0, int& n0) {
+        const int band_rows = 8;
+        const int band = t / (band_rows * p.tiles_n);
+        t -= band * band_rows * p.tiles_n;
+        const int rows_here = (p.tiles_m - band * band_rows) < band_rows ? (p.tiles_m - band * band_rows) : band_rows;
+        m0 = (band * band_rows + t % rows_here) * BM;
+        n0 = (t / rows_here) * BN;
+    };
+
+    // Both kinds of wave pass padded + 1 barriers: barrier g + 1 says "stage g is in LDS" and "stage g - 1 has been read".
+    if (producer) {
+        const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(p.A), 0, static_cast<int>(((p.M - 1) * p.a_rs + p.K) * 2), 0x00020000);
+        const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(p.B), 0, static_cast<int>(((p.N - 1) * p.b_rs + p.K) * 2), 0x00020000);
+        const uint32_t a_rs_bytes = static_cast<uint32_t>(p.a_rs) * 2u, b_rs_bytes = static_cast<uint32_t>(p.b_rs) * 2u;
+        // a thread's share of a stage: rows ptid / 8 + 32 i of both tiles, eight halves from k = 8 (ptid % 8) on --
+        // eight lanes read a row's 128 bytes
+        const int ptid = tid & 255;
+        const int prow = ptid >> 3, pk = (ptid & 7) * 8;
+        const int put = prow * F16_PITCH + pk * 2;
+        v4i ra[F16P_AHEAD][4], rb[F16P_AHEAD][4];
+        int it = 0, ic = 0, m0 = 0, n0 = 0;             // the next stage to request: tile `it` of mine, stage ic of it
+        if (my_tiles > 0) tile_origin(first, m0, n0);
+        // (Past the last stage a request asks for nothing -- every offset outside -- but is still made: the count of
+        // loads in flight that the wait for a stage names is then the same in every iteration, and the compiler
+        // waits for that stage alone -- vmcnt(15) .. vmcnt(8) for its eight loads; with requests under a condition
+        // it waited for all of them.)
+        const auto request = [&](v4i (&xa)[4], v4i (&xb)[4]) {
+            const int k = ic * F16_BK + pk;
+            const uint32_t kb = static_cast<uint32_t>(k) * 2u;
+            const bool live = it < my_tiles && k < p.K;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int ar = m0 + prow + 32 * i, br = n0 + prow + 32 * i;
+                const uint32_t at = (live && ar < p.M) ? static_cast<uint32_t>(ar) * a_rs_bytes + kb : OUTSIDE;
+                const uint32_t bt = (live && br < p.N) ? static_cast<uint32_t>(br) * b_rs_bytes + kb : OUTSIDE;
+                xa[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, at, 0, 0));
+                xb[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, bt, 0, 0));
+            }
+            if (++ic == chunks) {
+                ic = 0;
+                if (++it < my_tiles) tile_origin(first + it * step, m0, n0);
+            }
+        };
+#pragma unroll
+        for (int d = 0; d < F16P_AHEAD; ++d) { request(ra[d], rb[d]); __builtin_amdgcn_sched_barrier(0); }   // (in this order)
+        // The register sets take turns by name: the loop body is written out F16P_AHEAD times, and runs whole -- the
+        // stages past the last one move zeros, and the other waves pass their barriers (a way out of the middle of
+        // the body joins the loop's back edge in the compiled code, and the wait at the loop's head then allows
+        // for a set that has only just been requested: it waits for every load in flight).
+        for (int g0 = 0; g0 < padded; g0 += F16P_AHEAD) {
+#pragma unroll
+            for (int d = 0; d < F16P_AHEAD; ++d) {
+                const int g = g0 + d;
+                uint8_t* half = lds[g & 1];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    *reinterpret_cast<v4i*>(half + put + i * 32 * F16_PITCH) = ra[d][i];
+                    *reinterpret_cast<v4i*>(half + BM * F16_PITCH + put + i * 32 * F16_PITCH) = rb[d][i];
+                }
+                request(ra[d], rb[d]);
+                __syncthreads();
+            }
+        }
+        __syncthreads();                                // (the other waves' last stage)
+    } else {
+        const int j = lane & 31, hh = lane >> 5;
+        const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+        const int frag_a = (wm + j) * F16_PITCH + hh * 16;
+        const int frag_b = (BM + wn + j) * F16_PITCH + hh * 16;
+        const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(p.C, 0, static_cast<int>(p.M * p.c_mi * 4), 0x00020000);
+        __syncthreads();                                // stage 0 is in LDS
+        int g = 0;
+        for (int it = 0; it < my_tiles; ++it) {
+            int m0, n0;
+            tile_origin(first + it * step, m0, n0);
+            float tail[2];
+#pragma unroll
+            for (int tj = 0; tj < 2; ++tj) {
+                const int n = n0 + wn + tj * 32 + j;
+                tail[tj] = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
+            }
+            v16f acc[2][2];
+#pragma unroll
+            for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+                for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
+            for (int c = 0; c < chunks; ++c, ++g) {
+                const uint8_t* half = lds[g & 1];
+#pragma unroll
+                for (int s = 0; s < F16_BK / 16; ++s) {
+                    v8h fa[2], fb[2];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        fa[t] = *reinterpret_cast<const v8h*>(half + frag_a + t * 32 * F16_PITCH + s * 32);
+                        fb[t] = *reinterpret_cast<const v8h*>(half + frag_b + t * 32 * F16_PITCH + s * 32);
+                    }
+#pragma unroll
+                    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+                        for (int tj = 0; tj < 2; ++tj)
+                            acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[ti], fb[tj], acc[ti][tj], 0, 0, 0);
+                }
+                __syncthreads();                        // stage g has been read; stage g + 1 is in LDS
+            }
+            store_acc_buffer<STREAM_C, true>(rsrc_c, static_cast<uint32_t>(p.c_mi) * 4u, p.N, p.alpha, acc, m0 + wm, n0 + wn, lane, tail[0], tail[1]);
+        }
+        for (; g < padded; ++g) __syncthreads();
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // Large contractions split their operands once, ahead of the matrix work, instead of in every
 // work-group that reads them (a 128-row panel of A is read by every tile column): the planes go to a
@@ -2316,7 +2466,19 @@ int launch_gemm(GemmParams p, hipStream_t stream, const char* what, uint8_t* fix
     }
     else {
         if (split || p.np2 * p.np3 != 1 || p.a_ks != 1 || p.b_ks != 1) { set_error("%s: no F16 instance for this addressing", what); return RC_BAD_ARGS; }
-        if (p.stream_c) hipLaunchKernelGGL((gemm_f16_kernel<true>), grid, block, 0, stream, p);
+        // the streaming form where every load is sixteen aligned bytes and 32-bit offsets reach everything
+        const bool aligned8 = p.K % 8 == 0 && p.a_rs % 8 == 0 && p.b_rs % 8 == 0 &&
+                              ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0;
+        const bool in_reach = ((p.M - 1) * p.a_rs + p.K) * 2 < (1LL << 31) && ((p.N - 1) * p.b_rs + p.K) * 2 < (1LL << 31) &&
+                              p.c_ni == 1 && p.M * p.c_mi * 4 < (1LL << 31) && p.c_mi < (1 << 22);
+        if (aligned8 && in_reach) {
+            const int64_t resident = 2LL * device_cu_count() / 8 * 8;      // two work-groups per CU (LDS: 72 KB each)
+            const int64_t wgs = std::max<int64_t>(8, std::min<int64_t>((total + 7) / 8 * 8, resident));
+            const dim3 pgrid(static_cast<unsigned>(wgs));
+            if (p.stream_c) hipLaunchKernelGGL((gemm_f16_pc_kernel<true>), pgrid, dim3(512), 0, stream, p, static_cast<int>(total));
+            else hipLaunchKernelGGL((gemm_f16_pc_kernel<false>), pgrid, dim3(512), 0, stream, p, static_cast<int>(total));
+        }
+        else if (p.stream_c) hipLaunchKernelGGL((gemm_f16_kernel<true>), grid, block, 0, stream, p);
         else hipLaunchKernelGGL((gemm_f16_kernel<false>), grid, block, 0, stream, p);
     }
 #undef PPML_LAUNCH_BF16

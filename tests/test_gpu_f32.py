@@ -111,6 +111,45 @@ def test_mul_mat_f16_exact_on_small_integers(ops, oracle):
         ops.mul_mat_f16(_dev(a), _dev(b[:, :39]))
 
 
+@pytest.mark.parametrize("M,K,N,bias", [(26368, 256, 768, True), (300, 72, 260, False), (129, 8, 127, True),
+                                        (1000, 1032, 130, False), (5, 64, 3, True), (1, 8, 1, False), (2050, 192, 1030, True)])
+def test_mul_mat_f16_streaming_form_gives_the_general_kernels_bits(ops, oracle, M, K, N, bias):
+    """Operands whose rows start on sixteen bytes (K a multiple of eight halves, aligned base) take the kernel that
+    streams tiles through resident work-groups; the same values at an address two bytes further on take the general
+    kernel.  Same products in the same order: the same bits, non-finite values included -- and the oracle's result
+    on a sample of rows."""
+    rng = np.random.default_rng(M + 7 * K + 13 * N)
+    a = rng.standard_normal((M, K)).astype(np.float16)
+    b = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    if M >= 129:
+        a[M // 2, K // 3] = np.inf
+        a[M - 1, K - 1] = np.nan
+        b[N // 2, 0] = -np.inf
+    bv = rng.standard_normal(N).astype(np.float32) if bias else None
+    da, db = _dev(a), _dev(b)
+    assert da.data_ptr() % 16 == 0 and db.data_ptr() % 16 == 0
+
+    def shifted(t):
+        flat = torch.empty(t.numel() + 1, dtype=torch.float16, device="cuda")
+        view = flat[1:].view(t.shape)
+        view.copy_(t)
+        assert view.data_ptr() % 16 == 2 and view.is_contiguous()
+        return view
+
+    dbias = None if bv is None else _dev(bv)
+    got = ops.mul_mat_f16(da, db, dbias).cpu().numpy()
+    general = ops.mul_mat_f16(shifted(da), shifted(db), dbias).cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), general.view(np.uint32))
+    rows = np.unique(np.concatenate([np.arange(min(M, 40)), np.arange(max(0, M - 40), M), [M // 2]]))
+    want = oracle.mul_mat_f16(a[rows], b, bv)
+    with np.errstate(invalid="ignore"):
+        absprod = np.abs(a[rows]).astype(np.float64) @ np.abs(b).astype(np.float64).T + (np.abs(bv)[None, :] if bias else 0)
+    finite = np.isfinite(want)
+    assert np.array_equal(np.isnan(got[rows]), np.isnan(want))
+    assert np.array_equal(got[rows][~finite & ~np.isnan(want)], want[~finite & ~np.isnan(want)])
+    _check(np.where(finite, got[rows], 0), np.where(finite, want, 0), np.where(finite, absprod, 1.0))
+
+
 # ----------------------------------------------------------------------------- out_prod
 def test_out_prod_reference_small_inputs_exact(ops, oracle):
     # tests/test_cuda.cpp:207-245
