@@ -113,7 +113,12 @@ int q8_weight_pack_hip(const void *W, int wtype, int M, int K, void *packed,
  * *path_out (may be NULL) receives what the reference would report for the call (MulMatQ8Kernel.cu:493-496):
  * 1 when PPML_MMQ is not 0 and N reaches PPML_MMQ_MIN_N (default 16) or the weight is repacked (wtype 2, 3),
  * else 0; 0 on every error.  It names the reference's kernels, not this library's (ppml_hip_q8_last_path
- * does that): every path gives the same numbers. */
+ * does that): every path gives the same numbers.
+ * A packed weight (wtype 3) too large for the weight-stationary kernels, under enough tokens and features for
+ * sixteen tiles of 128 x 256, takes the tiled kernel: the activations are quantized once into a workspace
+ * (1.06 bytes per element, fragment order) from the stream-ordered pool mul_mat_hip describes -- the only
+ * kernel family of this entry point that uses memory beyond its arguments; without a workspace the general
+ * kernel serves the call. */
 int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
                    int c_trans, int *path_out, ppml_hip_stream_t stream);
 
@@ -123,7 +128,7 @@ int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K,
  *   flags bit 1: quantize X with the Q8_1 rule of quantize_rows_q8_1_hip instead of the Q8_0 rule:
  *                the numbers mul_mat_q8_cuda itself produces (src/cuda/MulMatQ8Kernel.cu:520-527
  *                quantizes activations to Q8_1 and settles with their d).
- *   flags bits 2..7 (PPML_Q8_FLAG_*): restrict the choice among the kernels that serve a Q8_0M weight, all
+ *   flags bits 2..8 (PPML_Q8_FLAG_*): restrict the choice among the kernels that serve a Q8_0M weight, all
  *                of which give the same bits; for tests and measurements.  (With c_trans = 0 the choice is
  *                between the weight-stationary kernel without column parts and the general one.)
  *   xq_dump  (may be NULL): receives the Q8_0 blocks the kernel made of X, [N][K/32] block_q8_0
@@ -137,7 +142,8 @@ enum {
     PPML_Q8_FLAG_LOW_LATENCY_16 = 32,      /* ... of 16 tokens */
     PPML_Q8_FLAG_LOW_LATENCY_32 = 48,      /* ... of 32 tokens (both bits; K = 512 only) */
     PPML_Q8_FLAG_COLUMN_PARTS = 64,        /* weight-stationary kernel: work-groups share a token tile, a part of the columns each, wherever there is an instance */
-    PPML_Q8_FLAG_NO_COLUMN_PARTS = 128     /* ... never */
+    PPML_Q8_FLAG_NO_COLUMN_PARTS = 128,    /* ... never */
+    PPML_Q8_FLAG_NO_TILED = 256            /* do not take the tiled kernel (large weights under many tokens) */
 };
 int mul_mat_q8_ex_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
                       int c_trans, int flags, void *xq_dump, int32_t *sums_dump,
@@ -368,7 +374,8 @@ void ppml_hip_mulmat_stats_reset(void);
 enum {
     PPML_Q8_PATH_GENERAL = 0,           /* one token tile per work-group, any shape and weight layout */
     PPML_Q8_PATH_WEIGHT_STATIONARY = 1, /* persistent work-groups, weight fragments resident in registers */
-    PPML_Q8_PATH_LOW_LATENCY = 2        /* few token tiles per CU: many small work-groups, weights through L2 */
+    PPML_Q8_PATH_LOW_LATENCY = 2,       /* few token tiles per CU: many small work-groups, weights through L2 */
+    PPML_Q8_PATH_TILED = 3              /* large weights under many tokens: activations quantized ahead, 128 x 256 tiles */
 };
 int ppml_hip_q8_last_path(void);
 

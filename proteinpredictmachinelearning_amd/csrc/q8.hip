@@ -1642,6 +1642,274 @@ extern "C" int dequantize_q8_1_hip(const void* x, float* y, int64_t ne, ppml_hip
     return check_launch("dequantize_q8_1_kernel") ? RC_BAD_ARGS : RC_OK;
 }
 
+namespace ppmlhip {
+namespace {
+
+// ------------------------------------------------------------------------------------------
+// Tiled form of the same linear, for Q8_0M weights too large for the weight-stationary kernel under many
+// tokens (K from 1024 on, or more columns than its instances hold).  The general kernel gives a work-group 32
+// tokens and streams the WHOLE weight through it: 4096 tokens x 4096 -> 4096 reads the 16 MB weight 128 times
+// (900 us, 0.03 of the int8 matrix peak).  Here the problem is cut like a GEMM:
+//
+//   1. the activations are quantized once, into a workspace, in the layout the packed weight has: per tile of
+//      32 tokens and block of 32 k the 64 lanes' sixteen quants (1 KB, an MFMA operand as it lies), and a plane
+//      of fp16 scales [tile][block][32] (q8_quantize_fragments_kernel: the arithmetic of quantize_block_lane,
+//      tokens past the end quantize zeros);
+//   2. q8_tiled_kernel: one work-group of eight waves per 128 tokens x 256 features; wave (wr, wc) owns 64 x 64
+//      of it (2 x 2 accumulator tiles).  K is walked in stages of two blocks: every thread copies sixteen
+//      bytes of activation fragments and thirty-two of weight fragments (plus the scales) from memory to the
+//      other half of a double buffer in LDS -- requested one stage ahead, into registers --, one barrier per
+//      stage.  Per stage and accumulator tile: two v_mfma_i32_32x32x32_i8 that start from 1.5 * 2^23 (exact
+//      block sums, read as floats), two v_mfma_f32_32x32x8_bf16 that take the offset off, one
+//      v_mfma_f32_32x32x4_2b_f16 for the two scale tables d_a[token] * d_w[feature] (each entry the exact
+//      product of two halves), and 2 x 16 fma on the vector pipe:
+//          acc = fma(float(sumi), d_w * d_a, acc)        blocks ascending
+//      -- the settlement of every other kernel of this file: same bits.
+//
+// c_trans = 0 (C [M][N]) swaps the operands of the MFMAs, as the weight-stationary kernel does.
+// ------------------------------------------------------------------------------------------
+constexpr int QT_TOK_TILES = 4, QT_COL_TILES = 8;          // a work-group's tile in units of 32: 128 tokens x 256 features
+constexpr int QT_A = QT_TOK_TILES * 2 * 1024;              // a stage: activation fragments [token tile][block of the pair][1 KB]
+constexpr int QT_W = QT_COL_TILES * 2 * 1024;              //          weight fragments [column tile][block][1 KB]
+constexpr int QT_DA = QT_TOK_TILES * 2 * 32 * 2;           //          activation scales [token tile][block][32] fp16
+constexpr int QT_DW = QT_COL_TILES * 2 * 32 * 2;           //          weight scales [column tile][block][32] fp16
+constexpr int QT_STAGE = QT_A + QT_W + QT_DA + QT_DW;
+constexpr uint32_t QT_OUTSIDE = 0x80000000u;               // an offset no buffer of this kernel reaches
+
+// One wave per (token tile, its upper or lower sixteen tokens, block): four lanes hold a block in element order.
+template <bool Q81>
+__global__ __launch_bounds__(256) void q8_quantize_fragments_kernel(const float* __restrict__ X, uint8_t* __restrict__ xq,
+                                                                    uint16_t* __restrict__ xd, int N, int nblk, int relu, int total_waves) {
+    const int lane = threadIdx.x & 63;
+    const int gw = __builtin_amdgcn_readfirstlane(static_cast<int>(blockIdx.x) * 4 + static_cast<int>(threadIdx.x >> 6));
+    if (gw >= total_waves) return;                      // wave-uniform
+    const int b = gw % nblk, rest = gw / nblk;
+    const int half = rest & 1, tile = rest >> 1;
+    const int c4 = lane & 3, r = half * 16 + (lane >> 2);
+    const int row = tile * 32 + r;
+    v4f x0 = {0.f, 0.f, 0.f, 0.f}, x1 = {0.f, 0.f, 0.f, 0.f};
+    if (row < N) {
+        const float* src = X + (static_cast<int64_t>(row) * nblk + b) * QK + c4 * 8;
+        x0 = *reinterpret_cast<const v4f_u*>(src);
+        x1 = *reinterpret_cast<const v4f_u*>(src + 4);
+    }
+    const BlockQuant bq = (relu & 1) ? quantize_block_lane<Q81, true>(x0, x1) : quantize_block_lane<Q81, false>(x0, x1);
+    const size_t frag = static_cast<size_t>(tile) * nblk + b;
+    *reinterpret_cast<uint2*>(xq + (frag << 10) + (((c4 >> 1) * 32 + r) << 4) + ((c4 & 1) << 3)) = uint2{bq.q_lo, bq.q_hi};
+    if (c4 == 0) xd[frag * 32 + r] = bq.d_bits;
+}
+
+template <bool CT0>
+__global__ __launch_bounds__(512) void q8_tiled_kernel(const uint8_t* __restrict__ xq, const uint16_t* __restrict__ xd,
+                                                       const uint8_t* __restrict__ W, float* __restrict__ C, int M, int N, int nblk,
+                                                       int ntt_pad, int mct_pad, int tiles_t, int tiles_c) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][QT_STAGE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 31, hh = lane >> 5;
+    const int wr = wave >> 2, wc = wave & 3;
+
+    // work-group -> tile: bands of eight token tiles, the column tiles of a band side by side in one XCD's L2
+    int tile_t, tile_c;
+    {
+        int t = xcd_contiguous_index(static_cast<int>(blockIdx.x), tiles_t * tiles_c);
+        const int band_rows = 8;
+        const int band = t / (band_rows * tiles_c);
+        t -= band * band_rows * tiles_c;
+        const int rows_here = (tiles_t - band * band_rows) < band_rows ? (tiles_t - band * band_rows) : band_rows;
+        tile_t = band * band_rows + t % rows_here;
+        tile_c = t / rows_here;
+    }
+    const int tt0 = tile_t * QT_TOK_TILES, ct0 = tile_c * QT_COL_TILES;
+    const int stages = nblk / 2;
+
+    const __amdgpu_buffer_rsrc_t rsrc_xq = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(xq), 0, ntt_pad * nblk * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_xd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(xd), 0, ntt_pad * nblk * 64, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_wq = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(W), 0, mct_pad * nblk * 1024, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_wd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(W) + static_cast<size_t>(mct_pad) * nblk * 1024, 0,
+                                                                             mct_pad * nblk * 64, 0x00020000);
+    // this thread's shares of a stage (the two blocks of a pair lie side by side in memory: 2 KB of fragments, 128
+    // bytes of scales per tile).  Column tiles past the weight's padded end repeat the last one; never stored.
+    const auto col_tile = [&](int c) { return c < mct_pad ? c : mct_pad - 1; };
+    uint32_t a_off = static_cast<uint32_t>((tt0 + (tid >> 7)) * nblk) * 1024u + static_cast<uint32_t>(tid & 127) * 16u;
+    uint32_t w_off[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) w_off[i] = static_cast<uint32_t>(col_tile(ct0 + (tid >> 7) + 4 * i) * nblk) * 1024u + static_cast<uint32_t>(tid & 127) * 16u;
+    // scales: threads 0..31 the activations' (four tiles x 128 bytes), threads 64..127 the weight's (eight x 128);
+    // the others request nothing (an offset outside), so every wave counts the same loads
+    uint32_t da_off = tid < 32 ? static_cast<uint32_t>((tt0 + (tid >> 3)) * nblk) * 64u + static_cast<uint32_t>(tid & 7) * 16u : QT_OUTSIDE;
+    uint32_t dw_off = (tid >= 64 && tid < 128) ? static_cast<uint32_t>(col_tile(ct0 + ((tid - 64) >> 3)) * nblk) * 64u + static_cast<uint32_t>(tid & 7) * 16u
+                                               : QT_OUTSIDE;
+    v4i ra, rw[2], rda, rdw;
+    const auto request = [&](int s) {                   // (s past the last stage: outside, zeros)
+        const uint32_t fo = static_cast<uint32_t>(s) * 2048u, so = static_cast<uint32_t>(s) * 128u;
+        const bool live = s < stages;
+        ra = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_xq, live ? a_off + fo : QT_OUTSIDE, 0, 0));
+#pragma unroll
+        for (int i = 0; i < 2; ++i) rw[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_wq, live ? w_off[i] + fo : QT_OUTSIDE, 0, 0));
+        rda = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_xd, (live && tid < 32) ? da_off + so : QT_OUTSIDE, 0, 0));
+        rdw = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_wd, (live && tid >= 64 && tid < 128) ? dw_off + so : QT_OUTSIDE, 0, 0));
+    };
+    const auto deposit = [&](uint8_t* stage) {
+        *reinterpret_cast<v4i*>(stage + tid * 16) = ra;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) *reinterpret_cast<v4i*>(stage + QT_A + (tid + 512 * i) * 16) = rw[i];
+        if (tid < 32) *reinterpret_cast<v4i*>(stage + QT_A + QT_W + tid * 16) = rda;
+        if (tid >= 64 && tid < 128) *reinterpret_cast<v4i*>(stage + QT_A + QT_W + QT_DA + (tid - 64) * 16) = rdw;
+    };
+
+    // (see the weight-stationary kernel: block sums leave the matrix pipe as floats)
+    v16i magic_i;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) magic_i[r] = WS_MAGIC_BITS;
+    asm volatile("" : "+v"(magic_i));
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    v4s unbias_a = {static_cast<short>(0xCAC0), 0, 0, 0};   // bf16 -0.75 * 2^23
+    v4s unbias_b = {static_cast<short>(0x3F80), 0, 0, 0};   // bf16 1
+    asm volatile("" : "+v"(unbias_a), "+v"(unbias_b));
+    v32f zero_f2;
+#pragma unroll
+    for (int r = 0; r < 32; ++r) zero_f2[r] = 0.0f;
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
+
+    request(0);
+    for (int s = 0; s < stages; ++s) {
+        uint8_t* stage = lds[s & 1];
+        deposit(stage);
+        request(s + 1);
+        __syncthreads();                                // stage s is in LDS; every wave has left stage s - 1
+        // this wave's operands of the stage
+        v4i a[2][2], w[2][2];
+        uint2 da[2], dw[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk) {
+                a[t][blk] = *reinterpret_cast<const v4i*>(stage + (((2 * wr + t) * 2 + blk) << 10) + lane * 16);
+                w[t][blk] = *reinterpret_cast<const v4i*>(stage + QT_A + (((2 * wc + t) * 2 + blk) << 10) + lane * 16);
+            }
+            // lanes 0..31: the rows (columns) of the pair's first block, lanes 32..63: of its second; the scale in the
+            // first of a lane's four k slots, zeros in the others
+            da[t] = uint2{*reinterpret_cast<const uint16_t*>(stage + QT_A + QT_W + ((2 * wr + t) * 2 + hh) * 64 + j * 2), 0u};
+            dw[t] = uint2{*reinterpret_cast<const uint16_t*>(stage + QT_A + QT_W + QT_DA + ((2 * wc + t) * 2 + hh) * 64 + j * 2), 0u};
+        }
+        // The four accumulator tiles in turn, the matrix pipe one block ahead of the vector pipe (the order of the
+        // weight-stationary kernel's steps): the block sum of a tile's second block is issued, then the first block is
+        // settled while it runs; the first block sum and the scale tables of the NEXT tile are issued in front of the
+        // settlement of the second block.  The barriers keep the compiler from sinking every MFMA next to its
+        // consumer, where each settlement would wait out a whole MFMA.
+        const auto block_sum = [&](int c, int blk) {
+            const int ti = c >> 1, tj = c & 1;
+            if constexpr (CT0) return __builtin_amdgcn_mfma_i32_32x32x32_i8(w[tj][blk], a[ti][blk], magic_i, 0, 0, 0);
+            else return __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ti][blk], w[tj][blk], magic_i, 0, 0, 0);
+        };
+        const auto to_float = [&](const v16i& biased) {     // 1.5 * 2^23 + sum -> float(sum), on the matrix pipe
+            return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(unbias_a, unbias_b, __builtin_bit_cast(v16f, biased), 0, 0, 0);
+        };
+        const auto scale_tables = [&](int c) {             // d_a[token] * d_w[feature] of both blocks of tile c
+            const int ti = c >> 1, tj = c & 1;
+            if constexpr (CT0) return __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, dw[tj]), __builtin_bit_cast(v4h, da[ti]), zero_f2, 0, 0, 0);
+            else return __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, da[ti]), __builtin_bit_cast(v4h, dw[tj]), zero_f2, 0, 0, 0);
+        };
+        v16i sum_a = block_sum(0, 0), sum_b;
+        v32f scl[2];                                       // the tables of this tile and of the next one, taking turns by name
+        scl[0] = scale_tables(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int ti = c >> 1, tj = c & 1;
+            const v16f flt_a = to_float(sum_a);
+            sum_b = block_sum(c, 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = __builtin_fmaf(flt_a[r], scl[c & 1][r], acc[ti][tj][r]);
+            __builtin_amdgcn_sched_barrier(0);
+            const v16f flt_b = to_float(sum_b);
+            if (c < 3) {
+                sum_a = block_sum(c + 1, 0);
+                scl[(c + 1) & 1] = scale_tables(c + 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = __builtin_fmaf(flt_b[r], scl[c & 1][16 + r], acc[ti][tj][r]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // the finished tile: a half-wave store is one 128-byte run of a C row; what lies outside C is dropped by the buffer
+    // (rows past the end lie behind it, columns past the end start from 2^31: the launcher keeps C below that)
+    const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(C, 0, static_cast<int>(static_cast<int64_t>(M) * N * 4), 0x00020000);
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti) {
+#pragma unroll
+        for (int tj = 0; tj < 2; ++tj) {
+            const int tok0 = (tt0 + 2 * wr + ti) * 32, m0 = (ct0 + 2 * wc + tj) * 32;
+            uint32_t off;
+            int pitch;
+            if constexpr (CT0) {       // rows of C are features, the lane's token picks the column
+                off = (tok0 + j < N && m0 < mct_pad * 32) ? (static_cast<uint32_t>(m0 + 4 * hh) * N + (tok0 + j)) * 4u : QT_OUTSIDE;
+                pitch = N * 4;
+            } else {
+                off = m0 + j < M ? (static_cast<uint32_t>(tok0 + 4 * hh) * M + (m0 + j)) * 4u : QT_OUTSIDE;
+                pitch = M * 4;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[ti][tj][r]), rsrc_c, off, 0, WS_STORE_AUX);
+                off += ((r & 3) == 3 ? 5 : 1) * pitch;  // rows 8 * (r / 4) + r % 4 (+ 4 in the upper half-wave)
+            }
+        }
+    }
+}
+
+// -1: not a problem for this form, or no workspace to be had (the caller goes on to the general kernel)
+template <bool Q81>
+int try_q8_tiled(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans, int relu, hipStream_t stream) {
+    if (nblk % 2 != 0) return -1;                       // stages are pairs of blocks
+    const int ntt = (N + 31) / 32, ntt_pad = (ntt + QT_TOK_TILES - 1) / QT_TOK_TILES * QT_TOK_TILES;
+    const int mct = (M + 31) / 32, mct_pad = packed_tiles(M);
+    const int tiles_t = ntt_pad / QT_TOK_TILES, tiles_c = (mct + QT_COL_TILES - 1) / QT_COL_TILES;
+    // Where it pays: from sixteen work-groups on (a work-group walks the whole K by itself), at least half a tile of
+    // features.  Measured, us, general kernel / this form: 4096 x 4096 -> 4096  900 / 200, 8192 x 1024 -> 8192  555 /
+    // 217, 408 x 4096 -> 4096  905 / 80, 128 x 1024 -> 4096  199 / 23, 2048 x 1024 -> 1024  52 / 26, 16384 x 512 ->
+    // 4096  186 / 118, 2601 x 1024 -> 512  30 / 26, 26368 x 1024 -> 1024  116 / 112; eight work-groups: 1024 x 1024 ->
+    // 256  19 / 24.
+    if (M < 128 || static_cast<int64_t>(tiles_t) * tiles_c < 16) return -1;
+    // 32-bit byte offsets everywhere: the fragments of both operands and C with the rows of its last, ragged tile
+    const int64_t xq_bytes = static_cast<int64_t>(ntt_pad) * nblk * 1024, xd_bytes = static_cast<int64_t>(ntt_pad) * nblk * 64;
+    const int64_t wq_bytes = static_cast<int64_t>(mct_pad) * nblk * 1024;
+    const int64_t c_reach = c_trans ? static_cast<int64_t>(ntt_pad * 32 + 4) * M * 4 : static_cast<int64_t>(tiles_c * QT_COL_TILES * 32 + 4) * N * 4;
+    if (xq_bytes >= 0x7fff0000LL || wq_bytes >= 0x7fff0000LL || c_reach >= 0x7fff0000LL) return -1;
+    if (static_cast<int64_t>(tiles_t) * tiles_c > 0x7fffffffLL) return -1;
+    const Workspace held = workspace_take(static_cast<size_t>(xq_bytes + xd_bytes), stream);
+    if (!held.ptr) return -1;
+    uint8_t* xq = held.ptr;
+    uint16_t* xd = reinterpret_cast<uint16_t*>(held.ptr + xq_bytes);
+    const int total_waves = ntt_pad * 2 * nblk;
+    hipLaunchKernelGGL((q8_quantize_fragments_kernel<Q81>), dim3((total_waves + 3) / 4), dim3(256), 0, stream, X, xq, xd, N, nblk, relu, total_waves);
+    int rc = check_launch("q8_quantize_fragments_kernel");
+    if (rc == RC_OK) {
+        const dim3 grid(static_cast<unsigned>(tiles_t * tiles_c)), block(512);
+        if (c_trans) hipLaunchKernelGGL((q8_tiled_kernel<false>), grid, block, 0, stream, xq, xd, static_cast<const uint8_t*>(W), C, M, N, nblk, ntt_pad, mct_pad, tiles_t, tiles_c);
+        else hipLaunchKernelGGL((q8_tiled_kernel<true>), grid, block, 0, stream, xq, xd, static_cast<const uint8_t*>(W), C, M, N, nblk, ntt_pad, mct_pad, tiles_t, tiles_c);
+        rc = check_launch("q8_tiled_kernel");
+    }
+    workspace_give(held, stream);
+    return rc;
+}
+
+}  // namespace
+}  // namespace ppmlhip
+
 extern "C" size_t q8_weight_packed_bytes_hip(int M, int K) {
     if (M <= 0 || K <= 0 || (K % QK) != 0) return 0;
     const size_t tiles = static_cast<size_t>(packed_tiles(M));
@@ -1693,6 +1961,11 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
                          : (act & 2) ? try_q8_linear_ws<true>(W, X, C, M, N, nblk, c_trans, relu, csplit, xq_dump, sums_dump, s)
                                      : try_q8_linear_ws<false>(W, X, C, M, N, nblk, c_trans, relu, csplit, xq_dump, sums_dump, s);
             if (rc >= 0) { set_q8_path(PPML_Q8_PATH_WEIGHT_STATIONARY); stat.set_path("hip/q8-weight-stationary"); return rc; }
+            // (the diagnostic buffers are the general kernel's; PPML_Q8_FLAG_NO_TILED keeps a call there too)
+            const int rt = ((flags & PPML_Q8_FLAG_NO_TILED) || xq_dump || sums_dump) ? -1
+                         : (act & 2) ? try_q8_tiled<true>(W, X, C, M, N, nblk, c_trans, relu, s)
+                                     : try_q8_tiled<false>(W, X, C, M, N, nblk, c_trans, relu, s);
+            if (rt >= 0) { set_q8_path(PPML_Q8_PATH_TILED); stat.set_path("hip/q8-tiled"); return rt; }
             return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         }
         default: set_error("mul_mat_q8_hip: unsupported wtype %d", wtype); return RC_WTYPE;

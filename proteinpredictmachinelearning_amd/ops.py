@@ -47,7 +47,7 @@ def _ptr(t) -> C.c_void_p:
     return C.c_void_p(0 if t is None else t.data_ptr())
 
 
-Q8_PATH_NAMES = {0: "general", 1: "weight-stationary", 2: "low-latency"}
+Q8_PATH_NAMES = {0: "general", 1: "weight-stationary", 2: "low-latency", 3: "tiled"}
 
 
 def last_q8_path() -> str:
@@ -476,7 +476,7 @@ class Q8Weight:
         return Q8Weight(out, self.M, self.K, WTYPE_Q8_0M)
 
 
-_Q8_PATH_FLAGS = {"auto": 0, "weight-stationary": 4, "general": 4 | 8, "low-latency": 0, "low-latency-8": 16, "low-latency-16": 32, "low-latency-32": 48,
+_Q8_PATH_FLAGS = {"auto": 0, "weight-stationary": 4, "general": 4 | 8 | 256, "tiled": 4 | 8, "low-latency": 0, "low-latency-8": 16, "low-latency-16": 32, "low-latency-32": 48,
                   "weight-stationary-column-parts": 4 | 64, "weight-stationary-whole": 4 | 128}
 
 
@@ -488,7 +488,8 @@ def mul_mat_q8(w: Q8Weight, x: torch.Tensor, c_trans: int = 1, relu: bool = Fals
     ``act`` selects the rule the activations are quantized with: "q8_0" (the CPU contract) or
     "q8_1" (what the reference's CUDA launcher does, src/cuda/MulMatQ8Kernel.cu:483-527).
     ``path`` restricts the kernel choice for a packed weight ("weight-stationary": not the low-latency kernel;
-    "general": neither of the two; "low-latency-8" / "-16" / "-32": that unit size wherever an instance exists (32: K = 512 only);
+    "general": the general kernel only; "tiled": neither the low-latency nor the weight-stationary kernel, i.e. the tiled
+    one wherever the problem is large enough for it; "low-latency-8" / "-16" / "-32": that unit size wherever an instance exists (32: K = 512 only);
     "weight-stationary-column-parts" / "-whole": that kernel with the columns shared out between work-groups
     wherever an instance exists / never); every choice gives the same bits.
     ``out``: a contiguous f32 device tensor of the result's shape to write into instead of a new one."""

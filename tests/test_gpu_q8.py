@@ -253,6 +253,12 @@ def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packe
         assert ops.last_q8_path() == "general"
 
 
+def _takes_tiled(N, K, M):
+    """The tiled kernel's own conditions: blocks in pairs, half a tile of features, sixteen work-groups."""
+    tok_tiles, col_tiles = (N + 31) // 32, (M + 31) // 32
+    return (K // 32) % 2 == 0 and M >= 128 and ((tok_tiles + 3) // 4) * ((col_tiles + 7) // 8) >= 16
+
+
 def _has_resident_weight_instance(K, M):
     tiles, nblk = (M + 31) // 32, K // 32
     tpw = (tiles + 7) // 8
@@ -336,14 +342,73 @@ def test_projections_wider_than_a_work_group_holds_go_in_column_parts(ops, oracl
     assert (got == oracle.mul_mat_q8(wq, np.maximum(x, 0.0), wtype=0, c_trans=1, fma=1)).all()
     got = ops.mul_mat_q8(W, _dev(x), act="q8_1").cpu().numpy()
     assert (got == oracle.mul_mat_q8_act(wq, x, act=1, c_trans=1)).all()
-    # told not to share the columns out, the call falls to the general kernel: same bits
+    # told not to share the columns out, the call falls to the tiled kernel where there are sixteen tiles of 128 x 256
+    # for it, else to the general one: same bits
     got = ops.mul_mat_q8(W, _dev(x), path="weight-stationary-whole")
-    assert ops.last_q8_path() == "general" and (got.cpu().numpy() == want).all()
+    assert ops.last_q8_path() == ("tiled" if _takes_tiled(N, K, M) else "general") and (got.cpu().numpy() == want).all()
     # sentinels around C
     buf = torch.full((N * M + 2048,), 7.5, device="cuda")
     ops.mul_mat_q8(W, _dev(x), out=buf[1024:1024 + N * M].view(N, M))
     assert (buf[1024:1024 + N * M].view(N, M).cpu().numpy() == want).all()
     assert (buf[:1024] == 7.5).all() and (buf[1024 + N * M:] == 7.5).all()
+
+
+# ----------------------------------------------------------------------------- tiled kernel (large weights)
+@pytest.mark.parametrize("N,K,M", [(300, 256, 2100),      # ragged tokens and features, 27 work-groups
+                                   (650, 1088, 600),      # 34 blocks; the last column tile of the last work-group is padding
+                                   (2048, 64, 130)])      # one stage; five column tiles, three of a work-group's eight repeat the last
+def test_tiled_kernel_bit_exact_against_the_oracle(ops, oracle, N, K, M):
+    """A packed weight under enough tokens and features for sixteen tiles of 128 x 256: the activations are quantized
+    ahead into fragment order and the contraction is cut like a GEMM.  Same block sums, same settlement, blocks
+    ascending: the oracle's bits, in both output orientations, with ReLU and with the Q8_1 rule."""
+    x, w = _inputs(3 * N + K + M, N, K, M)
+    x[N // 2, :32] = 0.0                                # an all-zero block: scale 0, reciprocal replaced by 0
+    wq = oracle.quantize_q8_0(w)
+    W = ops.Q8Weight(_dev(wq.reshape(-1)), M, K, ops.WTYPE_Q8_0).pack()
+    for c_trans in (1, 0):
+        want = oracle.mul_mat_q8(wq, x, wtype=0, c_trans=c_trans, fma=1)
+        got = ops.mul_mat_q8(W, _dev(x), c_trans=c_trans, path="tiled")
+        assert ops.last_q8_path() == "tiled"
+        assert (got.cpu().numpy() == want).all(), c_trans
+        got = ops.mul_mat_q8(W, _dev(x), c_trans=c_trans, relu=True, path="tiled").cpu().numpy()
+        assert (got == oracle.mul_mat_q8(wq, np.maximum(x, 0.0), wtype=0, c_trans=c_trans, fma=1)).all(), c_trans
+        got = ops.mul_mat_q8(W, _dev(x), c_trans=c_trans, act="q8_1", path="tiled").cpu().numpy()
+        assert ops.last_q8_path() == "tiled"
+        assert (got == oracle.mul_mat_q8_act(wq, x, act=1, c_trans=c_trans)).all(), c_trans
+    # sentinels around C, ragged last tiles in both directions
+    buf = torch.full((N * M + 4096,), 7.5, device="cuda")
+    ops.mul_mat_q8(W, _dev(x), out=buf[2048:2048 + N * M].view(N, M), path="tiled")
+    assert ops.last_q8_path() == "tiled"
+    assert (buf[2048:2048 + N * M].view(N, M).cpu().numpy() == oracle.mul_mat_q8(wq, x, wtype=0, c_trans=1, fma=1)).all()
+    assert (buf[:2048] == 7.5).all() and (buf[2048 + N * M:] == 7.5).all()
+    # the diagnostic buffers are the general kernel's, and so is the call when that kernel is asked for
+    ops.mul_mat_q8(W, _dev(x), dump=True, path="tiled")
+    assert ops.last_q8_path() == "general"
+    ops.mul_mat_q8(W, _dev(x), path="general")
+    assert ops.last_q8_path() == "general"
+
+
+def test_tiled_kernel_is_the_librarys_choice_for_large_weights(ops):
+    """Where the weight-stationary kernels have no instance (K = 2048; 4096 features under K = 512) the library
+    takes the tiled kernel from sixteen work-groups on, and its bits are the general kernel's; an odd number of
+    blocks, few work-groups or a weight that is not packed stay with the general kernel."""
+    rng = np.random.default_rng(11)
+    for N, K, M, want_path in [(408, 2048, 2048, "tiled"), (4096, 512, 4096, "tiled"), (1000, 2080, 512, "general"),
+                               (1024, 1024, 256, "general"), (2048, 1024, 64, "general")]:
+        x = _dev(rng.standard_normal((N, K)).astype(np.float32))
+        w = _dev((rng.standard_normal((M, K)) * 0.02).astype(np.float32))
+        W = ops.Q8Weight.from_f32(w)
+        ref = ops.mul_mat_q8(W, x)
+        assert ops.last_q8_path() == "general"          # the unpacked weight
+        Wp = W.pack()
+        for c_trans in (1, 0):
+            got = ops.mul_mat_q8(Wp, x, c_trans=c_trans)
+            assert ops.last_q8_path() == want_path, (N, K, M)
+            gen = ops.mul_mat_q8(Wp, x, c_trans=c_trans, path="general")
+            assert ops.last_q8_path() == "general"
+            assert torch.equal(got.view(torch.int32), gen.view(torch.int32)), (N, K, M, c_trans)
+            if c_trans:
+                assert torch.equal(got.view(torch.int32), ref.view(torch.int32)), (N, K, M)
 
 
 @pytest.mark.parametrize("key", sorted(WS_INSTANCE_SHAPES))
