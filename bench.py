@@ -283,6 +283,16 @@ def main() -> int:
             if cpu_pair is not None:
                 extra[name]["cpu_baseline"] = q8_cpu(w_dev, x_dev, relu, no, f"the whole {r}x{k}->{n} workload")
 
+        # a compute-bound shape of the same operator (no shape of the reference's model is one: its quantized
+        # projections all have K <= 512): large weights take the tiled kernel, measured against the int8 matrix peak
+        if not args.configured_shapes_only:
+            r, k, n = 4096, 4096, 4096
+            f, ns, nb, no, _ = q8_case(r, k, n)
+            w_, e_ = time_op(f, ns, max(10, steps // 4), 3)
+            extra["q8_linear_large_4096x4096_4096"] = {"us": round(e_ * 1e6, 2), "TOPS": round(no / e_ / 1e12, 2),
+                                                       "int8_mfma_frac": round(no / e_ / 1e12 / INT8_PEAK_TOPS, 4),
+                                                       "kernel": ops.last_q8_path(), "event_steps": time_op.last["event_steps"]}
+
         rest = {"skip": False}
 
         def f32_case(make, nbytes, flops, name, pipe="fp32", rw=None, cpu=None):
