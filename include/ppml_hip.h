@@ -115,7 +115,7 @@ int q8_weight_pack_hip(const void *W, int wtype, int M, int K, void *packed,
  * else 0; 0 on every error.  It names the reference's kernels, not this library's (ppml_hip_q8_last_path
  * does that): every path gives the same numbers.
  * A packed weight (wtype 3) too large for the weight-stationary kernels, under enough tokens and features for
- * sixteen tiles of 128 x 256, takes the tiled kernel: the activations are quantized once into a workspace
+ * sixteen tiles of 128 x 256 (or 128 x 128), takes the tiled kernel: the activations are quantized once into a workspace
  * (1.06 bytes per element, fragment order) from the stream-ordered pool mul_mat_hip describes -- the only
  * kernel family of this entry point that uses memory beyond its arguments; without a workspace the general
  * kernel serves the call. */

@@ -1656,7 +1656,8 @@ namespace {
 //      of fp16 scales [tile][block][32] (q8_quantize_fragments_kernel: the arithmetic of quantize_block_lane,
 //      tokens past the end quantize zeros);
 //   2. q8_tiled_kernel: one work-group of eight waves per 128 tokens x 256 features; wave (wr, wc) owns 64 x 64
-//      of it (2 x 2 accumulator tiles).  K is walked in stages of two blocks: every thread copies sixteen
+//      of it (2 x 2 accumulator tiles) -- or, where that leaves CUs without work or in a thin last round, per 128 x
+//      128, a wave 64 x 32 (the launcher's rule).  K is walked in stages of two blocks: every thread copies sixteen
 //      bytes of activation fragments and thirty-two of weight fragments (plus the scales) from memory to the
 //      other half of a double buffer in LDS -- requested one stage ahead, into registers --, one barrier per
 //      stage.  Per stage and accumulator tile: two v_mfma_i32_32x32x32_i8 that start from 1.5 * 2^23 (exact
@@ -1668,12 +1669,15 @@ namespace {
 //
 // c_trans = 0 (C [M][N]) swaps the operands of the MFMAs, as the weight-stationary kernel does.
 // ------------------------------------------------------------------------------------------
-constexpr int QT_TOK_TILES = 4, QT_COL_TILES = 8;          // a work-group's tile in units of 32: 128 tokens x 256 features
-constexpr int QT_A = QT_TOK_TILES * 2 * 1024;              // a stage: activation fragments [token tile][block of the pair][1 KB]
-constexpr int QT_W = QT_COL_TILES * 2 * 1024;              //          weight fragments [column tile][block][1 KB]
-constexpr int QT_DA = QT_TOK_TILES * 2 * 32 * 2;           //          activation scales [token tile][block][32] fp16
-constexpr int QT_DW = QT_COL_TILES * 2 * 32 * 2;           //          weight scales [column tile][block][32] fp16
-constexpr int QT_STAGE = QT_A + QT_W + QT_DA + QT_DW;
+constexpr int QT_TOK_TILES = 4;                            // a work-group's tile in units of 32: 128 tokens x (128 TJ) features,
+template <int TJ> struct QTile {                           // TJ = column tiles per wave (2: the wide form, 1: the narrow one)
+    static constexpr int COL_TILES = 4 * TJ;
+    static constexpr int A = QT_TOK_TILES * 2 * 1024;      // a stage: activation fragments [token tile][block of the pair][1 KB]
+    static constexpr int W = COL_TILES * 2 * 1024;         //          weight fragments [column tile][block][1 KB]
+    static constexpr int DA = QT_TOK_TILES * 2 * 32 * 2;   //          activation scales [token tile][block][32] fp16
+    static constexpr int DW = COL_TILES * 2 * 32 * 2;      //          weight scales [column tile][block][32] fp16
+    static constexpr int STAGE = A + W + DA + DW;
+};
 constexpr uint32_t QT_OUTSIDE = 0x80000000u;               // an offset no buffer of this kernel reaches
 
 // One wave per (token tile, its upper or lower sixteen tokens, block): four lanes hold a block in element order.
@@ -1699,11 +1703,12 @@ __global__ __launch_bounds__(256) void q8_quantize_fragments_kernel(const float*
     if (c4 == 0) xd[frag * 32 + r] = bq.d_bits;
 }
 
-template <bool CT0>
+template <bool CT0, int TJ>
 __global__ __launch_bounds__(512) void q8_tiled_kernel(const uint8_t* __restrict__ xq, const uint16_t* __restrict__ xd,
                                                        const uint8_t* __restrict__ W, float* __restrict__ C, int M, int N, int nblk,
                                                        int ntt_pad, int mct_pad, int tiles_t, int tiles_c) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2][QT_STAGE];
+    using T = QTile<TJ>;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2][T::STAGE];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1721,7 +1726,7 @@ __global__ __launch_bounds__(512) void q8_tiled_kernel(const uint8_t* __restrict
         tile_t = band * band_rows + t % rows_here;
         tile_c = t / rows_here;
     }
-    const int tt0 = tile_t * QT_TOK_TILES, ct0 = tile_c * QT_COL_TILES;
+    const int tt0 = tile_t * QT_TOK_TILES, ct0 = tile_c * T::COL_TILES;
     const int stages = nblk / 2;
 
     const __amdgpu_buffer_rsrc_t rsrc_xq = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(xq), 0, ntt_pad * nblk * 1024, 0x00020000);
@@ -1733,30 +1738,31 @@ __global__ __launch_bounds__(512) void q8_tiled_kernel(const uint8_t* __restrict
     // bytes of scales per tile).  Column tiles past the weight's padded end repeat the last one; never stored.
     const auto col_tile = [&](int c) { return c < mct_pad ? c : mct_pad - 1; };
     uint32_t a_off = static_cast<uint32_t>((tt0 + (tid >> 7)) * nblk) * 1024u + static_cast<uint32_t>(tid & 127) * 16u;
-    uint32_t w_off[2];
+    uint32_t w_off[TJ];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) w_off[i] = static_cast<uint32_t>(col_tile(ct0 + (tid >> 7) + 4 * i) * nblk) * 1024u + static_cast<uint32_t>(tid & 127) * 16u;
-    // scales: threads 0..31 the activations' (four tiles x 128 bytes), threads 64..127 the weight's (eight x 128);
-    // the others request nothing (an offset outside), so every wave counts the same loads
+    for (int i = 0; i < TJ; ++i) w_off[i] = static_cast<uint32_t>(col_tile(ct0 + (tid >> 7) + 4 * i) * nblk) * 1024u + static_cast<uint32_t>(tid & 127) * 16u;
+    // scales: threads 0..31 the activations' (four tiles x 128 bytes), threads 64 .. 63 + 32 TJ the weight's (128 bytes
+    // per column tile); the others request nothing (an offset outside), so every wave counts the same loads
+    const bool dw_thread = tid >= 64 && tid < 64 + 32 * TJ;
     uint32_t da_off = tid < 32 ? static_cast<uint32_t>((tt0 + (tid >> 3)) * nblk) * 64u + static_cast<uint32_t>(tid & 7) * 16u : QT_OUTSIDE;
-    uint32_t dw_off = (tid >= 64 && tid < 128) ? static_cast<uint32_t>(col_tile(ct0 + ((tid - 64) >> 3)) * nblk) * 64u + static_cast<uint32_t>(tid & 7) * 16u
+    uint32_t dw_off = dw_thread ? static_cast<uint32_t>(col_tile(ct0 + ((tid - 64) >> 3)) * nblk) * 64u + static_cast<uint32_t>(tid & 7) * 16u
                                                : QT_OUTSIDE;
-    v4i ra, rw[2], rda, rdw;
+    v4i ra, rw[TJ], rda, rdw;
     const auto request = [&](int s) {                   // (s past the last stage: outside, zeros)
         const uint32_t fo = static_cast<uint32_t>(s) * 2048u, so = static_cast<uint32_t>(s) * 128u;
         const bool live = s < stages;
         ra = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_xq, live ? a_off + fo : QT_OUTSIDE, 0, 0));
 #pragma unroll
-        for (int i = 0; i < 2; ++i) rw[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_wq, live ? w_off[i] + fo : QT_OUTSIDE, 0, 0));
+        for (int i = 0; i < TJ; ++i) rw[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_wq, live ? w_off[i] + fo : QT_OUTSIDE, 0, 0));
         rda = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_xd, (live && tid < 32) ? da_off + so : QT_OUTSIDE, 0, 0));
-        rdw = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_wd, (live && tid >= 64 && tid < 128) ? dw_off + so : QT_OUTSIDE, 0, 0));
+        rdw = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_wd, (live && dw_thread) ? dw_off + so : QT_OUTSIDE, 0, 0));
     };
     const auto deposit = [&](uint8_t* stage) {
         *reinterpret_cast<v4i*>(stage + tid * 16) = ra;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) *reinterpret_cast<v4i*>(stage + QT_A + (tid + 512 * i) * 16) = rw[i];
-        if (tid < 32) *reinterpret_cast<v4i*>(stage + QT_A + QT_W + tid * 16) = rda;
-        if (tid >= 64 && tid < 128) *reinterpret_cast<v4i*>(stage + QT_A + QT_W + QT_DA + (tid - 64) * 16) = rdw;
+        for (int i = 0; i < TJ; ++i) *reinterpret_cast<v4i*>(stage + T::A + (tid + 512 * i) * 16) = rw[i];
+        if (tid < 32) *reinterpret_cast<v4i*>(stage + T::A + T::W + tid * 16) = rda;
+        if (dw_thread) *reinterpret_cast<v4i*>(stage + T::A + T::W + T::DA + (tid - 64) * 16) = rdw;
     };
 
     // (see the weight-stationary kernel: block sums leave the matrix pipe as floats)
@@ -1773,11 +1779,11 @@ __global__ __launch_bounds__(512) void q8_tiled_kernel(const uint8_t* __restrict
 #pragma unroll
     for (int r = 0; r < 32; ++r) zero_f2[r] = 0.0f;
 
-    v16f acc[2][2];
+    v16f acc[2][TJ];
 #pragma unroll
     for (int ti = 0; ti < 2; ++ti)
 #pragma unroll
-        for (int tj = 0; tj < 2; ++tj)
+        for (int tj = 0; tj < TJ; ++tj)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[ti][tj][r] = 0.0f;
 
@@ -1787,28 +1793,26 @@ __global__ __launch_bounds__(512) void q8_tiled_kernel(const uint8_t* __restrict
         deposit(stage);
         request(s + 1);
         __syncthreads();                                // stage s is in LDS; every wave has left stage s - 1
-        // this wave's operands of the stage
-        v4i a[2][2], w[2][2];
-        uint2 da[2], dw[2];
+        // this wave's operands of the stage: fragments a[token tile][block], w[column tile][block]; scales da / dw: lanes
+        // 0..31 hold the rows (columns) of the pair's first block, lanes 32..63 of its second, the scale in the first of a
+        // lane's four k slots, zeros in the others
+        v4i a[2][2], w[TJ][2];
+        uint2 da[2], dw[TJ];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
 #pragma unroll
-            for (int blk = 0; blk < 2; ++blk) {
-                a[t][blk] = *reinterpret_cast<const v4i*>(stage + (((2 * wr + t) * 2 + blk) << 10) + lane * 16);
-                w[t][blk] = *reinterpret_cast<const v4i*>(stage + QT_A + (((2 * wc + t) * 2 + blk) << 10) + lane * 16);
-            }
-            // lanes 0..31: the rows (columns) of the pair's first block, lanes 32..63: of its second; the scale in the
-            // first of a lane's four k slots, zeros in the others
-            da[t] = uint2{*reinterpret_cast<const uint16_t*>(stage + QT_A + QT_W + ((2 * wr + t) * 2 + hh) * 64 + j * 2), 0u};
-            dw[t] = uint2{*reinterpret_cast<const uint16_t*>(stage + QT_A + QT_W + QT_DA + ((2 * wc + t) * 2 + hh) * 64 + j * 2), 0u};
+            for (int blk = 0; blk < 2; ++blk) a[t][blk] = *reinterpret_cast<const v4i*>(stage + (((2 * wr + t) * 2 + blk) << 10) + lane * 16);
+            da[t] = uint2{*reinterpret_cast<const uint16_t*>(stage + T::A + T::W + ((2 * wr + t) * 2 + hh) * 64 + j * 2), 0u};
         }
-        // The four accumulator tiles in turn, the matrix pipe one block ahead of the vector pipe (the order of the
-        // weight-stationary kernel's steps): the block sum of a tile's second block is issued, then the first block is
-        // settled while it runs; the first block sum and the scale tables of the NEXT tile are issued in front of the
-        // settlement of the second block.  The barriers keep the compiler from sinking every MFMA next to its
-        // consumer, where each settlement would wait out a whole MFMA.
+#pragma unroll
+        for (int t = 0; t < TJ; ++t) {
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk) w[t][blk] = *reinterpret_cast<const v4i*>(stage + T::A + (((TJ * wc + t) * 2 + blk) << 10) + lane * 16);
+            dw[t] = uint2{*reinterpret_cast<const uint16_t*>(stage + T::A + T::W + T::DA + ((TJ * wc + t) * 2 + hh) * 64 + j * 2), 0u};
+        }
+        // accumulator tile c of the wave: token tile c / TJ, column tile c % TJ
         const auto block_sum = [&](int c, int blk) {
-            const int ti = c >> 1, tj = c & 1;
+            const int ti = c / TJ, tj = c % TJ;
             if constexpr (CT0) return __builtin_amdgcn_mfma_i32_32x32x32_i8(w[tj][blk], a[ti][blk], magic_i, 0, 0, 0);
             else return __builtin_amdgcn_mfma_i32_32x32x32_i8(a[ti][blk], w[tj][blk], magic_i, 0, 0, 0);
         };
@@ -1816,31 +1820,48 @@ __global__ __launch_bounds__(512) void q8_tiled_kernel(const uint8_t* __restrict
             return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(unbias_a, unbias_b, __builtin_bit_cast(v16f, biased), 0, 0, 0);
         };
         const auto scale_tables = [&](int c) {             // d_a[token] * d_w[feature] of both blocks of tile c
-            const int ti = c >> 1, tj = c & 1;
+            const int ti = c / TJ, tj = c % TJ;
             if constexpr (CT0) return __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, dw[tj]), __builtin_bit_cast(v4h, da[ti]), zero_f2, 0, 0, 0);
             else return __builtin_amdgcn_mfma_f32_32x32x4f16(__builtin_bit_cast(v4h, da[ti]), __builtin_bit_cast(v4h, dw[tj]), zero_f2, 0, 0, 0);
         };
-        v16i sum_a = block_sum(0, 0), sum_b;
-        v32f scl[2];                                       // the tables of this tile and of the next one, taking turns by name
+        // The stage's 4 TJ units (accumulator tile u / 2, block u % 2) with the matrix pipe ahead of the vector pipe, the
+        // order of the weight-stationary kernel's steps; the barriers keep the compiler from sinking every MFMA next to
+        // its consumer, where each settlement would wait out a whole MFMA.  The wide form, with 64 accumulator registers,
+        // has room for two buffers of block sums: while unit u is settled, the block sum of unit u + 1 runs, and the
+        // offset comes off it right in front of its settlement.  The narrow form has room for three: the matrix pipe is
+        // two units ahead, and a settlement reads nothing that was issued less than a whole unit ago.  (Neither makes the
+        // two pipes overlap: their times add up in both.)
+        constexpr int UNITS = 4 * TJ, DEPTH = TJ == 2 ? 1 : 2;
+        v16i sum[DEPTH + 1];
+        v16f flt[DEPTH + 1];
+        v32f scl[2];                                       // the tables of a tile and of the next one, taking turns by name
+        sum[0] = block_sum(0, 0);
         scl[0] = scale_tables(0);
+        if constexpr (DEPTH == 2) {
+            sum[1] = block_sum(0, 1);
+            flt[0] = to_float(sum[0]);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int ti = c >> 1, tj = c & 1;
-            const v16f flt_a = to_float(sum_a);
-            sum_b = block_sum(c, 1);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = __builtin_fmaf(flt_a[r], scl[c & 1][r], acc[ti][tj][r]);
-            __builtin_amdgcn_sched_barrier(0);
-            const v16f flt_b = to_float(sum_b);
-            if (c < 3) {
-                sum_a = block_sum(c + 1, 0);
-                scl[(c + 1) & 1] = scale_tables(c + 1);
+        for (int u = 0; u < UNITS; ++u) {
+            const int c = u >> 1, ti = c / TJ, tj = c % TJ;
+            if constexpr (DEPTH == 1) {
+                flt[u & 1] = to_float(sum[u & 1]);
+                if (u + 1 < UNITS) {
+                    sum[(u + 1) & 1] = block_sum((u + 1) >> 1, (u + 1) & 1);
+                    if (((u + 1) & 1) == 0) scl[((u + 1) >> 1) & 1] = scale_tables((u + 1) >> 1);
+                }
+            } else {
+                if (u + 2 < UNITS) {
+                    sum[(u + 2) % 3] = block_sum((u + 2) >> 1, (u + 2) & 1);
+                    if (((u + 2) & 1) == 0) scl[((u + 2) >> 1) & 1] = scale_tables((u + 2) >> 1);
+                }
+                if (u + 1 < UNITS) flt[(u + 1) % 3] = to_float(sum[(u + 1) % 3]);
             }
             __builtin_amdgcn_sched_barrier(0);
+            const v16f& f = flt[u % (DEPTH + 1)];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = __builtin_fmaf(flt_b[r], scl[c & 1][16 + r], acc[ti][tj][r]);
+            for (int r = 0; r < 16; ++r) acc[ti][tj][r] = __builtin_fmaf(f[r], scl[c & 1][(u & 1) * 16 + r], acc[ti][tj][r]);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -1851,8 +1872,8 @@ __global__ __launch_bounds__(512) void q8_tiled_kernel(const uint8_t* __restrict
 #pragma unroll
     for (int ti = 0; ti < 2; ++ti) {
 #pragma unroll
-        for (int tj = 0; tj < 2; ++tj) {
-            const int tok0 = (tt0 + 2 * wr + ti) * 32, m0 = (ct0 + 2 * wc + tj) * 32;
+        for (int tj = 0; tj < TJ; ++tj) {
+            const int tok0 = (tt0 + 2 * wr + ti) * 32, m0 = (ct0 + TJ * wc + tj) * 32;
             uint32_t off;
             int pitch;
             if constexpr (CT0) {       // rows of C are features, the lane's token picks the column
@@ -1877,17 +1898,28 @@ int try_q8_tiled(const void* W, const float* X, float* C, int M, int N, int nblk
     if (nblk % 2 != 0) return -1;                       // stages are pairs of blocks
     const int ntt = (N + 31) / 32, ntt_pad = (ntt + QT_TOK_TILES - 1) / QT_TOK_TILES * QT_TOK_TILES;
     const int mct = (M + 31) / 32, mct_pad = packed_tiles(M);
-    const int tiles_t = ntt_pad / QT_TOK_TILES, tiles_c = (mct + QT_COL_TILES - 1) / QT_COL_TILES;
-    // Where it pays: from sixteen work-groups on (a work-group walks the whole K by itself), at least half a tile of
-    // features.  Measured, us, general kernel / this form: 4096 x 4096 -> 4096  900 / 200, 8192 x 1024 -> 8192  555 /
-    // 217, 408 x 4096 -> 4096  905 / 80, 128 x 1024 -> 4096  199 / 23, 2048 x 1024 -> 1024  52 / 26, 16384 x 512 ->
-    // 4096  186 / 118, 2601 x 1024 -> 512  30 / 26, 26368 x 1024 -> 1024  116 / 112; eight work-groups: 1024 x 1024 ->
-    // 256  19 / 24.
-    if (M < 128 || static_cast<int64_t>(tiles_t) * tiles_c < 16) return -1;
+    const int tiles_t = ntt_pad / QT_TOK_TILES;
+    // The form: tiles 256 features wide (two column tiles per wave) or 128 wide (one).  A CU holds one work-group of
+    // either; a wide one takes 1.8 times as long as a narrow one for twice the outputs, so the form with the cheaper
+    // rounds wins: us, wide / narrow, with the work-groups of each: 4096 x 4096 -> 4096  199 / 222 (512, 1024), 8192 x
+    // 1024 -> 8192  216 / 233, 16384 x 512 -> 4096  118 / 131, 5000 x 2048 -> 1000  55 / 60 (160, 320), 26368 x 1024 ->
+    // 256  44 / 47 (206, 412); 408 x 4096 -> 4096  80 / 51 (64, 128), 2048 x 1024 -> 1024  26 / 19, 512 x 1024 -> 1024
+    // 24 / 16, 2601 x 1024 -> 512  26 / 19, 10609 x 1024 -> 128  31 / 23, 10609 x 512 -> 1024  35 / 32 (332, 664),
+    // 26368 x 512 -> 1024  65 / 63.
+    const int cus = device_cu_count();
+    const int64_t wgs_wide = static_cast<int64_t>(tiles_t) * ((mct + 7) / 8), wgs_narrow = static_cast<int64_t>(tiles_t) * ((mct + 3) / 4);
+    const bool narrow = static_cast<double>((wgs_narrow + cus - 1) / cus) < 1.8 * static_cast<double>((wgs_wide + cus - 1) / cus);
+    const int ctiles = narrow ? 4 : 8;
+    const int tiles_c = (mct + ctiles - 1) / ctiles;
+    // Where it pays at all: from sixteen work-groups on (a work-group walks the whole K by itself), at least half a
+    // narrow tile of features.  us, general kernel / this one: 4096 x 4096 -> 4096  900 / 199, 408 x 4096 -> 4096  905 /
+    // 51, 128 x 1024 -> 4096  199 / 15, 2048 x 1024 -> 1024  52 / 19, 1024 x 1024 -> 256  19 / 16, 26368 x 1024 -> 1024
+    // 116 / 108.
+    if (M < 64 || static_cast<int64_t>(tiles_t) * tiles_c < 16) return -1;
     // 32-bit byte offsets everywhere: the fragments of both operands and C with the rows of its last, ragged tile
     const int64_t xq_bytes = static_cast<int64_t>(ntt_pad) * nblk * 1024, xd_bytes = static_cast<int64_t>(ntt_pad) * nblk * 64;
     const int64_t wq_bytes = static_cast<int64_t>(mct_pad) * nblk * 1024;
-    const int64_t c_reach = c_trans ? static_cast<int64_t>(ntt_pad * 32 + 4) * M * 4 : static_cast<int64_t>(tiles_c * QT_COL_TILES * 32 + 4) * N * 4;
+    const int64_t c_reach = c_trans ? static_cast<int64_t>(ntt_pad * 32 + 4) * M * 4 : static_cast<int64_t>(tiles_c * ctiles * 32 + 4) * N * 4;
     if (xq_bytes >= 0x7fff0000LL || wq_bytes >= 0x7fff0000LL || c_reach >= 0x7fff0000LL) return -1;
     if (static_cast<int64_t>(tiles_t) * tiles_c > 0x7fffffffLL) return -1;
     const Workspace held = workspace_take(static_cast<size_t>(xq_bytes + xd_bytes), stream);
@@ -1899,8 +1931,11 @@ int try_q8_tiled(const void* W, const float* X, float* C, int M, int N, int nblk
     int rc = check_launch("q8_quantize_fragments_kernel");
     if (rc == RC_OK) {
         const dim3 grid(static_cast<unsigned>(tiles_t * tiles_c)), block(512);
-        if (c_trans) hipLaunchKernelGGL((q8_tiled_kernel<false>), grid, block, 0, stream, xq, xd, static_cast<const uint8_t*>(W), C, M, N, nblk, ntt_pad, mct_pad, tiles_t, tiles_c);
-        else hipLaunchKernelGGL((q8_tiled_kernel<true>), grid, block, 0, stream, xq, xd, static_cast<const uint8_t*>(W), C, M, N, nblk, ntt_pad, mct_pad, tiles_t, tiles_c);
+#define PPML_QT(CT0_, TJ_) hipLaunchKernelGGL((q8_tiled_kernel<CT0_, TJ_>), grid, block, 0, stream, xq, xd, static_cast<const uint8_t*>(W), C, M, N, nblk, \
+                                              ntt_pad, mct_pad, tiles_t, tiles_c)
+        if (narrow) { if (c_trans) PPML_QT(false, 1); else PPML_QT(true, 1); }
+        else        { if (c_trans) PPML_QT(false, 2); else PPML_QT(true, 2); }
+#undef PPML_QT
         rc = check_launch("q8_tiled_kernel");
     }
     workspace_give(held, stream);

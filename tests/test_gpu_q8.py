@@ -254,9 +254,14 @@ def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packe
 
 
 def _takes_tiled(N, K, M):
-    """The tiled kernel's own conditions: blocks in pairs, half a tile of features, sixteen work-groups."""
-    tok_tiles, col_tiles = (N + 31) // 32, (M + 31) // 32
-    return (K // 32) % 2 == 0 and M >= 128 and ((tok_tiles + 3) // 4) * ((col_tiles + 7) // 8) >= 16
+    """The tiled kernel's own conditions: blocks in pairs, half a narrow tile of features, sixteen work-groups of the
+    form it picks (tiles of 128 tokens x 128 features where their rounds over the CUs come cheaper than those of
+    tiles twice as wide, which take 1.8 times as long each)."""
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    tiles_t, col_tiles = ((N + 31) // 32 + 3) // 4, (M + 31) // 32
+    wide, narrow = tiles_t * ((col_tiles + 7) // 8), tiles_t * ((col_tiles + 3) // 4)
+    takes_narrow = -(-narrow // cus) < 1.8 * -(-wide // cus)
+    return (K // 32) % 2 == 0 and M >= 64 and (narrow if takes_narrow else wide) >= 16
 
 
 def _has_resident_weight_instance(K, M):
@@ -354,9 +359,10 @@ def test_projections_wider_than_a_work_group_holds_go_in_column_parts(ops, oracl
 
 
 # ----------------------------------------------------------------------------- tiled kernel (large weights)
-@pytest.mark.parametrize("N,K,M", [(300, 256, 2100),      # ragged tokens and features, 27 work-groups
+@pytest.mark.parametrize("N,K,M", [(300, 256, 2100),      # ragged tokens and features; narrow tiles (51 work-groups in one round)
                                    (650, 1088, 600),      # 34 blocks; the last column tile of the last work-group is padding
-                                   (2048, 64, 130)])      # one stage; five column tiles, three of a work-group's eight repeat the last
+                                   (2048, 64, 130),       # one stage; five column tiles, of a work-group's tiles some repeat the last
+                                   (5000, 128, 1000)])    # wide tiles: 160 work-groups of 128 x 256 in one round (320 narrow ones would take two)
 def test_tiled_kernel_bit_exact_against_the_oracle(ops, oracle, N, K, M):
     """A packed weight under enough tokens and features for sixteen tiles of 128 x 256: the activations are quantized
     ahead into fragment order and the contraction is cut like a GEMM.  Same block sums, same settlement, blocks
@@ -390,11 +396,12 @@ def test_tiled_kernel_bit_exact_against_the_oracle(ops, oracle, N, K, M):
 
 def test_tiled_kernel_is_the_librarys_choice_for_large_weights(ops):
     """Where the weight-stationary kernels have no instance (K = 2048; 4096 features under K = 512) the library
-    takes the tiled kernel from sixteen work-groups on, and its bits are the general kernel's; an odd number of
-    blocks, few work-groups or a weight that is not packed stay with the general kernel."""
+    takes the tiled kernel from sixteen work-groups on -- in tiles of 128 x 256 or of 128 x 128, whichever has the
+    cheaper rounds over the CUs -- and its bits are the general kernel's; an odd number of blocks, few work-groups,
+    fewer than 64 features or a weight that is not packed stay with the general kernel."""
     rng = np.random.default_rng(11)
     for N, K, M, want_path in [(408, 2048, 2048, "tiled"), (4096, 512, 4096, "tiled"), (1000, 2080, 512, "general"),
-                               (1024, 1024, 256, "general"), (2048, 1024, 64, "general")]:
+                               (1024, 1024, 256, "tiled"), (512, 1024, 256, "general"), (2048, 1024, 32, "general")]:
         x = _dev(rng.standard_normal((N, K)).astype(np.float32))
         w = _dev((rng.standard_normal((M, K)) * 0.02).astype(np.float32))
         W = ops.Q8Weight.from_f32(w)
