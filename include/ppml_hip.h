@@ -71,8 +71,10 @@ int ppml_hip_set_f32_arithmetic(int mode);
  * carries every operand, for all of them.  Contractions of at
  * least 512 work-groups of 256 x 128 outputs (6 bytes per operand element) and contractions of few output
  * tiles under a long K (the partial sums of their K slices) use a workspace from a stream-ordered pool of
- * the library's; a stream keeps one such buffer between calls (a stream under capture and the per-thread
- * default stream allocate and release per call). */
+ * the library's; a stream keeps one such buffer between calls (the per-thread default stream allocates and
+ * releases per call).  A stream under capture gets no workspace -- an allocation made while a graph is recorded
+ * is gone before the graph runs -- and its calls take the forms that need none; mul_mat_tn_noalloc_hip brings the
+ * sliced forms to recorded code. */
 int mul_mat_hip(const float *A, const float *B, float *C, int M, int K, int N,
                 const float *bias, ppml_hip_stream_t stream);
 

@@ -41,9 +41,9 @@ hipMemPool_t workspace_pool();         // the library's stream-ordered pool on t
 // Device memory for the work a launcher is about to issue on `stream`, valid until that work has run: the stream keeps
 // one buffer from the pool between calls (the next taker's work is ordered behind this one's on the same stream, so it
 // may have the same memory), which saves an allocation and a release per call -- 10 us on this stack.  Null when none
-// is to be had.  workspace_give() after the last launch that uses it: it releases what was allocated for this call only
-// (a stream under capture and the per-thread default stream keep nothing) and lets the next host thread that issues
-// work on the same stream have the buffer (two threads' launches must not interleave on it).
+// is to be had -- always so on a stream under capture.  workspace_give() after the last launch that uses it: it releases
+// what was allocated for this call only (the per-thread default stream keeps nothing) and lets the next host thread that
+// issues work on the same stream have the buffer (two threads' launches must not interleave on it).
 struct Workspace { uint8_t* ptr = nullptr; bool call_owned = false; void* turn = nullptr; };
 Workspace workspace_take(size_t bytes, hipStream_t stream);
 void workspace_give(const Workspace& ws, hipStream_t stream);

@@ -212,15 +212,21 @@ hipMemPool_t workspace_pool() {
 
 Workspace workspace_take(size_t bytes, hipStream_t stream) {
     Workspace ws;
-    hipMemPool_t pool = workspace_pool();
-    if (!pool || bytes == 0) return ws;
+    if (bytes == 0) return ws;
+    // A stream under capture gets no workspace, and nothing here touches the pool for it: an allocation made while the
+    // graph is recorded is released again before the graph ever runs, and the recorded kernels would keep its address
+    // (a replay then reads and writes memory that is not theirs -- an illegal access on the device).  The caller takes
+    // the form of its operation that needs no workspace; mul_mat_tn_noalloc_hip brings the forms that do to recorded code.
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (stream != nullptr && stream != hipStreamPerThread && hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
         (void)hipGetLastError();
         capturing = hipStreamCaptureStatusActive;        // (cannot tell: treat it as the careful case)
     }
-    if (stream == hipStreamPerThread || capturing != hipStreamCaptureStatusNone) {
-        // one name for many streams, or an allocation that would be baked into a graph: allocate for this call only
+    if (capturing != hipStreamCaptureStatusNone) return ws;
+    hipMemPool_t pool = workspace_pool();
+    if (!pool) return ws;
+    if (stream == hipStreamPerThread) {
+        // one name for many streams: allocate for this call only
         if (hipMallocFromPoolAsync(reinterpret_cast<void**>(&ws.ptr), bytes, pool, stream) != hipSuccess) { (void)hipGetLastError(); ws.ptr = nullptr; }
         ws.call_owned = ws.ptr != nullptr;
         return ws;

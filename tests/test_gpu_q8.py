@@ -418,6 +418,30 @@ def test_tiled_kernel_is_the_librarys_choice_for_large_weights(ops):
                 assert torch.equal(got.view(torch.int32), ref.view(torch.int32)), (N, K, M)
 
 
+def test_a_call_on_a_capturing_stream_takes_no_workspace(ops):
+    """The tiled kernel's workspace comes from the stream-ordered pool, and a stream under capture gets none (what is
+    allocated while a graph is recorded is gone before the graph runs): a call recorded into a graph takes the
+    general kernel.  The graph is recorded and dropped, never run."""
+    g = torch.Generator(device="cuda").manual_seed(9)
+    N, K, M = 600, 1024, 1024
+    W = ops.Q8Weight.from_f32(torch.randn(M, K, device="cuda", generator=g) * 0.02).pack()
+    x = torch.randn(N, K, device="cuda", generator=g)
+    out = torch.empty(N, M, device="cuda")
+    ops.mul_mat_q8(W, x, out=out, path="general")        # eager first: nothing is set up for the first time under capture
+    ops.mul_mat_q8(W, x, out=out)
+    assert ops.last_q8_path() == "tiled"
+    want = out.clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.mul_mat_q8(W, x, out=out)
+        recorded_path = ops.last_q8_path()
+    del graph
+    assert recorded_path == "general"
+    ops.mul_mat_q8(W, x, out=out)                        # and the stream's kept buffer serves eager calls as before
+    assert ops.last_q8_path() == "tiled" and torch.equal(out, want)
+
+
 @pytest.mark.parametrize("key", sorted(WS_INSTANCE_SHAPES))
 def test_features_outermost_output_on_the_weight_stationary_kernel(ops, oracle, key):
     """c_trans = 0 (the quantized weight was src[0], src/backend/CUDAKernels.cpp:761-777: C is [M][N]) with a packed
