@@ -120,7 +120,8 @@ int q8_weight_pack_hip(const void *W, int wtype, int M, int K, void *packed,
  * sixteen tiles of 128 x 256 (or 128 x 128), takes the tiled kernel: the activations are quantized once into a workspace
  * (1.06 bytes per element, fragment order) from the stream-ordered pool mul_mat_hip describes -- the only
  * kernel family of this entry point that uses memory beyond its arguments; without a workspace the general
- * kernel serves the call. */
+ * kernel serves the call.  A weight of wtype 0, 1 or 2 beyond 256 Ki elements takes it too, packed into the same
+ * workspace on the way (1.06 bytes per element more). */
 int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
                    int c_trans, int *path_out, ppml_hip_stream_t stream);
 

@@ -1642,6 +1642,9 @@ extern "C" int dequantize_q8_1_hip(const void* x, float* y, int64_t ne, ppml_hip
     return check_launch("dequantize_q8_1_kernel") ? RC_BAD_ARGS : RC_OK;
 }
 
+extern "C" size_t q8_weight_packed_bytes_hip(int M, int K);
+extern "C" int q8_weight_pack_hip(const void* W, int wtype, int M, int K, void* packed, ppml_hip_stream_t stream);
+
 namespace ppmlhip {
 namespace {
 
@@ -1893,8 +1896,10 @@ __global__ __launch_bounds__(512) void q8_tiled_kernel(const uint8_t* __restrict
 }
 
 // -1: not a problem for this form, or no workspace to be had (the caller goes on to the general kernel)
+// `wtype` other than PPML_WTYPE_Q8_0M: the weight is packed into the workspace first, per call (one pass over it: 4096 x
+// 4096 in 10 us, against the 700 us that the general kernel loses on such a weight).
 template <bool Q81>
-int try_q8_tiled(const void* W, const float* X, float* C, int M, int N, int nblk, int c_trans, int relu, hipStream_t stream) {
+int try_q8_tiled(const void* W, int wtype, const float* X, float* C, int M, int N, int nblk, int c_trans, int relu, hipStream_t stream) {
     if (nblk % 2 != 0) return -1;                       // stages are pairs of blocks
     const int ntt = (N + 31) / 32, ntt_pad = (ntt + QT_TOK_TILES - 1) / QT_TOK_TILES * QT_TOK_TILES;
     const int mct = (M + 31) / 32, mct_pad = packed_tiles(M);
@@ -1922,13 +1927,22 @@ int try_q8_tiled(const void* W, const float* X, float* C, int M, int N, int nblk
     const int64_t c_reach = c_trans ? static_cast<int64_t>(ntt_pad * 32 + 4) * M * 4 : static_cast<int64_t>(tiles_c * ctiles * 32 + 4) * N * 4;
     if (xq_bytes >= 0x7fff0000LL || wq_bytes >= 0x7fff0000LL || c_reach >= 0x7fff0000LL) return -1;
     if (static_cast<int64_t>(tiles_t) * tiles_c > 0x7fffffffLL) return -1;
-    const Workspace held = workspace_take(static_cast<size_t>(xq_bytes + xd_bytes), stream);
+    const size_t wp_bytes = wtype == PPML_WTYPE_Q8_0M ? 0 : (q8_weight_packed_bytes_hip(M, nblk * QK) + 1023) / 1024 * 1024;
+    const Workspace held = workspace_take(static_cast<size_t>(xq_bytes + xd_bytes) + wp_bytes, stream);
     if (!held.ptr) return -1;
     uint8_t* xq = held.ptr;
     uint16_t* xd = reinterpret_cast<uint16_t*>(held.ptr + xq_bytes);
+    int rc = RC_OK;
+    if (wp_bytes) {
+        uint8_t* wp = held.ptr + xq_bytes + xd_bytes;
+        rc = q8_weight_pack_hip(W, wtype, M, nblk * QK, wp, stream);
+        W = wp;
+    }
     const int total_waves = ntt_pad * 2 * nblk;
-    hipLaunchKernelGGL((q8_quantize_fragments_kernel<Q81>), dim3((total_waves + 3) / 4), dim3(256), 0, stream, X, xq, xd, N, nblk, relu, total_waves);
-    int rc = check_launch("q8_quantize_fragments_kernel");
+    if (rc == RC_OK) {
+        hipLaunchKernelGGL((q8_quantize_fragments_kernel<Q81>), dim3((total_waves + 3) / 4), dim3(256), 0, stream, X, xq, xd, N, nblk, relu, total_waves);
+        rc = check_launch("q8_quantize_fragments_kernel");
+    }
     if (rc == RC_OK) {
         const dim3 grid(static_cast<unsigned>(tiles_t * tiles_c)), block(512);
 #define PPML_QT(CT0_, TJ_) hipLaunchKernelGGL((q8_tiled_kernel<CT0_, TJ_>), grid, block, 0, stream, xq, xd, static_cast<const uint8_t*>(W), C, M, N, nblk, \
@@ -1979,6 +1993,15 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
     hipStream_t s = static_cast<hipStream_t>(stream);
     StatsScope stat("hip/q8-general", M, K, N, s);
     set_q8_path(PPML_Q8_PATH_GENERAL);
+    // A weight of the reference's own layouts that is large (beyond what stays resident even when packed) takes the tiled
+    // kernel too, packed into the workspace on the way; the diagnostic buffers and PPML_Q8_FLAG_NO_TILED keep a call with
+    // the general kernel.
+    if (wtype != PPML_WTYPE_Q8_0M && (wtype == PPML_WTYPE_Q8_0 || wtype == PPML_WTYPE_Q8_1 || wtype == PPML_WTYPE_Q8_0R) &&
+        static_cast<int64_t>(M) * K > (256 << 10) && !(flags & PPML_Q8_FLAG_NO_TILED) && !xq_dump && !sums_dump) {
+        const int rt = (act & 2) ? try_q8_tiled<true>(W, wtype, X, C, M, N, nblk, c_trans, relu, s)
+                                 : try_q8_tiled<false>(W, wtype, X, C, M, N, nblk, c_trans, relu, s);
+        if (rt >= 0) { set_q8_path(PPML_Q8_PATH_TILED); stat.set_path("hip/q8-tiled"); return rt; }
+    }
     switch (wtype) {
         case PPML_WTYPE_Q8_0:  return dispatch_q8_linear<PPML_WTYPE_Q8_0>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_1:  return dispatch_q8_linear<PPML_WTYPE_Q8_1>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
@@ -1998,8 +2021,8 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
             if (rc >= 0) { set_q8_path(PPML_Q8_PATH_WEIGHT_STATIONARY); stat.set_path("hip/q8-weight-stationary"); return rc; }
             // (the diagnostic buffers are the general kernel's; PPML_Q8_FLAG_NO_TILED keeps a call there too)
             const int rt = ((flags & PPML_Q8_FLAG_NO_TILED) || xq_dump || sums_dump) ? -1
-                         : (act & 2) ? try_q8_tiled<true>(W, X, C, M, N, nblk, c_trans, relu, s)
-                                     : try_q8_tiled<false>(W, X, C, M, N, nblk, c_trans, relu, s);
+                         : (act & 2) ? try_q8_tiled<true>(W, wtype, X, C, M, N, nblk, c_trans, relu, s)
+                                     : try_q8_tiled<false>(W, wtype, X, C, M, N, nblk, c_trans, relu, s);
             if (rt >= 0) { set_q8_path(PPML_Q8_PATH_TILED); stat.set_path("hip/q8-tiled"); return rt; }
             return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         }

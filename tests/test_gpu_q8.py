@@ -405,8 +405,13 @@ def test_tiled_kernel_is_the_librarys_choice_for_large_weights(ops):
         x = _dev(rng.standard_normal((N, K)).astype(np.float32))
         w = _dev((rng.standard_normal((M, K)) * 0.02).astype(np.float32))
         W = ops.Q8Weight.from_f32(w)
-        ref = ops.mul_mat_q8(W, x)
-        assert ops.last_q8_path() == "general"          # the unpacked weight
+        ref = ops.mul_mat_q8(W, x, path="general")
+        assert ops.last_q8_path() == "general"
+        # the weight as the reference stores it: tiled too where it is larger than anything that stays resident (it is
+        # packed into the workspace on the way), else the general kernel
+        got = ops.mul_mat_q8(W, x)
+        assert ops.last_q8_path() == (want_path if M * K > 256 * 1024 else "general"), (N, K, M)
+        assert torch.equal(got.view(torch.int32), ref.view(torch.int32)), (N, K, M)
         Wp = W.pack()
         for c_trans in (1, 0):
             got = ops.mul_mat_q8(Wp, x, c_trans=c_trans)
@@ -416,6 +421,25 @@ def test_tiled_kernel_is_the_librarys_choice_for_large_weights(ops):
             assert torch.equal(got.view(torch.int32), gen.view(torch.int32)), (N, K, M, c_trans)
             if c_trans:
                 assert torch.equal(got.view(torch.int32), ref.view(torch.int32)), (N, K, M)
+
+
+def test_tiled_kernel_on_the_references_weight_layouts(ops, oracle):
+    """Q8_0, Q8_1 and Q8_0R weights (include/ppml/QuantBlocks.h:33-41, 123-133) beyond 256 Ki elements take the tiled
+    kernel through a per-call repack into the workspace: the oracle's bits in both orientations."""
+    N, K, M = 300, 512, 1000
+    x, w = _inputs(77, N, K, M)
+    wq = oracle.quantize_q8_0(w)
+    want = oracle.mul_mat_q8(wq, x, wtype=0, c_trans=1, fma=1)
+    layouts = {ops.WTYPE_Q8_0: wq.reshape(-1), ops.WTYPE_Q8_1: _q8_1_from_q8_0(wq).reshape(-1), ops.WTYPE_Q8_0R: oracle.repack_q8_0(wq)}
+    for wtype, data in layouts.items():
+        W = ops.Q8Weight(_dev(data), M, K, wtype)
+        got = ops.mul_mat_q8(W, _dev(x), c_trans=1)
+        assert ops.last_q8_path() == "tiled", wtype
+        assert (got.cpu().numpy() == want).all(), wtype
+        got = ops.mul_mat_q8(W, _dev(x), c_trans=0)
+        assert ops.last_q8_path() == "tiled" and (got.cpu().numpy() == want.T).all(), wtype
+        out, xq, sums = ops.mul_mat_q8(W, _dev(x), c_trans=1, dump=True)       # the diagnostic buffers: the general kernel
+        assert ops.last_q8_path() == "general" and (out.cpu().numpy() == want).all(), wtype
 
 
 def test_a_call_on_a_capturing_stream_takes_no_workspace(ops):
