@@ -121,7 +121,8 @@ int q8_weight_pack_hip(const void *W, int wtype, int M, int K, void *packed,
  * (1.06 bytes per element, fragment order) from the stream-ordered pool mul_mat_hip describes -- the only
  * kernel family of this entry point that uses memory beyond its arguments; without a workspace the general
  * kernel serves the call.  A weight of wtype 0, 1 or 2 beyond 256 Ki elements takes it too, packed into the same
- * workspace on the way (1.06 bytes per element more). */
+ * workspace on the way (1.06 bytes per element more); a smaller one, under 1024 tokens or more, is packed into the
+ * workspace per call as well (one launch) and served by the kernels of wtype 3 where they have an instance. */
 int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
                    int c_trans, int *path_out, ppml_hip_stream_t stream);
 
@@ -131,8 +132,9 @@ int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K,
  *   flags bit 1: quantize X with the Q8_1 rule of quantize_rows_q8_1_hip instead of the Q8_0 rule:
  *                the numbers mul_mat_q8_cuda itself produces (src/cuda/MulMatQ8Kernel.cu:520-527
  *                quantizes activations to Q8_1 and settles with their d).
- *   flags bits 2..8 (PPML_Q8_FLAG_*): restrict the choice among the kernels that serve a Q8_0M weight, all
- *                of which give the same bits; for tests and measurements.  (With c_trans = 0 the choice is
+ *   flags bits 2..8 (PPML_Q8_FLAG_*): restrict the choice among the kernels that serve a Q8_0M weight (and a weight
+ *                of another layout that is packed per call, below), all of which give the same bits; for tests and
+ *                measurements.  (With c_trans = 0 the choice is
  *                between the weight-stationary kernel without column parts and the general one.)
  *   xq_dump  (may be NULL): receives the Q8_0 blocks the kernel made of X, [N][K/32] block_q8_0
  *   sums_dump(may be NULL): receives the per-block int32 sums, [(n*M+m)*(K/32)+ib]            */

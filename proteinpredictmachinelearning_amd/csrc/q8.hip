@@ -1993,37 +1993,61 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
     hipStream_t s = static_cast<hipStream_t>(stream);
     StatsScope stat("hip/q8-general", M, K, N, s);
     set_q8_path(PPML_Q8_PATH_GENERAL);
-    // A weight of the reference's own layouts that is large (beyond what stays resident even when packed) takes the tiled
-    // kernel too, packed into the workspace on the way; the diagnostic buffers and PPML_Q8_FLAG_NO_TILED keep a call with
-    // the general kernel.
-    if (wtype != PPML_WTYPE_Q8_0M && (wtype == PPML_WTYPE_Q8_0 || wtype == PPML_WTYPE_Q8_1 || wtype == PPML_WTYPE_Q8_0R) &&
-        static_cast<int64_t>(M) * K > (256 << 10) && !(flags & PPML_Q8_FLAG_NO_TILED) && !xq_dump && !sums_dump) {
-        const int rt = (act & 2) ? try_q8_tiled<true>(W, wtype, X, C, M, N, nblk, c_trans, relu, s)
+    // the kernel families that want the packed layout and keep the weight resident or close by; -1: none of them ran
+    const auto resident_families = [&](const void* Wp) -> int {
+        const int ll_bits = flags & (PPML_Q8_FLAG_LOW_LATENCY_8 | PPML_Q8_FLAG_LOW_LATENCY_16);
+        const int force_ll = ll_bits == PPML_Q8_FLAG_LOW_LATENCY_32 ? 32 : ll_bits == PPML_Q8_FLAG_LOW_LATENCY_8 ? 8 :
+                             ll_bits == PPML_Q8_FLAG_LOW_LATENCY_16 ? 16 : 0;
+        const int rl = (flags & PPML_Q8_FLAG_NO_LOW_LATENCY) ? -1
+                     : (act & 2) ? try_q8_linear_ll<true>(Wp, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s)
+                                 : try_q8_linear_ll<false>(Wp, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s);
+        if (rl >= 0) { set_q8_path(PPML_Q8_PATH_LOW_LATENCY); stat.set_path("hip/q8-low-latency"); return rl; }
+        const int csplit = (flags & PPML_Q8_FLAG_COLUMN_PARTS) ? 1 : (flags & PPML_Q8_FLAG_NO_COLUMN_PARTS) ? -1 : 0;
+        const int rc = (flags & PPML_Q8_FLAG_NO_WEIGHT_STATIONARY) ? -1
+                     : (act & 2) ? try_q8_linear_ws<true>(Wp, X, C, M, N, nblk, c_trans, relu, csplit, xq_dump, sums_dump, s)
+                                 : try_q8_linear_ws<false>(Wp, X, C, M, N, nblk, c_trans, relu, csplit, xq_dump, sums_dump, s);
+        if (rc >= 0) { set_q8_path(PPML_Q8_PATH_WEIGHT_STATIONARY); stat.set_path("hip/q8-weight-stationary"); return rc; }
+        return -1;
+    };
+    // (the diagnostic buffers are the general kernel's; PPML_Q8_FLAG_NO_TILED keeps a call there too)
+    const auto tiled = [&]() -> int {
+        const int rt = ((flags & PPML_Q8_FLAG_NO_TILED) || xq_dump || sums_dump) ? -1
+                     : (act & 2) ? try_q8_tiled<true>(W, wtype, X, C, M, N, nblk, c_trans, relu, s)
                                  : try_q8_tiled<false>(W, wtype, X, C, M, N, nblk, c_trans, relu, s);
-        if (rt >= 0) { set_q8_path(PPML_Q8_PATH_TILED); stat.set_path("hip/q8-tiled"); return rt; }
+        if (rt >= 0) { set_q8_path(PPML_Q8_PATH_TILED); stat.set_path("hip/q8-tiled"); }
+        return rt;
+    };
+    // A weight in one of the reference's own layouts (include/ppml/QuantBlocks.h:33-41, 123-133) need not wait for its
+    // owner to adopt the packed one.  Beyond what stays resident it takes the tiled kernel, which packs it into its
+    // workspace on the way.  Up to that size, under 1024 tokens or more, it is packed into the stream's workspace here
+    // (one launch, a few microseconds) and served by the kernels of the packed layout: us on a Q8_0 weight, general
+    // kernel / this way (timed through the Python operator, 9 us of host time per call): 26368 x 256 -> 768  60 / 26,
+    // 26368 x 256 -> 256  28 / 13, 26368 x 512 -> 128  30 / 19, 10609 x 128 -> 512  16 / 12, 10609 x 256 -> 768  32 / 14.
+    // With fewer tokens the launch costs what the better kernel saves.  No workspace (a stream under capture): the
+    // general kernel, as before.
+    if (wtype == PPML_WTYPE_Q8_0 || wtype == PPML_WTYPE_Q8_1 || wtype == PPML_WTYPE_Q8_0R) {
+        if (static_cast<int64_t>(M) * K > (256 << 10)) {
+            const int rt = tiled();
+            if (rt >= 0) return rt;
+        } else if (N >= 1024 && !xq_dump && !sums_dump &&
+                   (flags & (PPML_Q8_FLAG_NO_LOW_LATENCY | PPML_Q8_FLAG_NO_WEIGHT_STATIONARY)) != (PPML_Q8_FLAG_NO_LOW_LATENCY | PPML_Q8_FLAG_NO_WEIGHT_STATIONARY)) {
+            const Workspace held = workspace_take(q8_weight_packed_bytes_hip(M, K), s);
+            if (held.ptr) {
+                const int rc = q8_weight_pack_hip(W, wtype, M, K, held.ptr, stream) == RC_OK ? resident_families(held.ptr) : -1;
+                workspace_give(held, s);
+                if (rc >= 0) return rc;
+            }
+        }
     }
     switch (wtype) {
         case PPML_WTYPE_Q8_0:  return dispatch_q8_linear<PPML_WTYPE_Q8_0>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_1:  return dispatch_q8_linear<PPML_WTYPE_Q8_1>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0R: return dispatch_q8_linear<PPML_WTYPE_Q8_0R>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         case PPML_WTYPE_Q8_0M: {
-            const int ll_bits = flags & (PPML_Q8_FLAG_LOW_LATENCY_8 | PPML_Q8_FLAG_LOW_LATENCY_16);
-            const int force_ll = ll_bits == PPML_Q8_FLAG_LOW_LATENCY_32 ? 32 : ll_bits == PPML_Q8_FLAG_LOW_LATENCY_8 ? 8 :
-                                 ll_bits == PPML_Q8_FLAG_LOW_LATENCY_16 ? 16 : 0;
-            const int rl = (flags & PPML_Q8_FLAG_NO_LOW_LATENCY) ? -1
-                         : (act & 2) ? try_q8_linear_ll<true>(W, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s)
-                                     : try_q8_linear_ll<false>(W, X, C, M, N, nblk, c_trans, relu, force_ll, xq_dump, sums_dump, s);
-            if (rl >= 0) { set_q8_path(PPML_Q8_PATH_LOW_LATENCY); stat.set_path("hip/q8-low-latency"); return rl; }
-            const int csplit = (flags & PPML_Q8_FLAG_COLUMN_PARTS) ? 1 : (flags & PPML_Q8_FLAG_NO_COLUMN_PARTS) ? -1 : 0;
-            const int rc = (flags & PPML_Q8_FLAG_NO_WEIGHT_STATIONARY) ? -1
-                         : (act & 2) ? try_q8_linear_ws<true>(W, X, C, M, N, nblk, c_trans, relu, csplit, xq_dump, sums_dump, s)
-                                     : try_q8_linear_ws<false>(W, X, C, M, N, nblk, c_trans, relu, csplit, xq_dump, sums_dump, s);
-            if (rc >= 0) { set_q8_path(PPML_Q8_PATH_WEIGHT_STATIONARY); stat.set_path("hip/q8-weight-stationary"); return rc; }
-            // (the diagnostic buffers are the general kernel's; PPML_Q8_FLAG_NO_TILED keeps a call there too)
-            const int rt = ((flags & PPML_Q8_FLAG_NO_TILED) || xq_dump || sums_dump) ? -1
-                         : (act & 2) ? try_q8_tiled<true>(W, wtype, X, C, M, N, nblk, c_trans, relu, s)
-                                     : try_q8_tiled<false>(W, wtype, X, C, M, N, nblk, c_trans, relu, s);
-            if (rt >= 0) { set_q8_path(PPML_Q8_PATH_TILED); stat.set_path("hip/q8-tiled"); return rt; }
+            const int rr = resident_families(W);
+            if (rr >= 0) return rr;
+            const int rt = tiled();
+            if (rt >= 0) return rt;
             return dispatch_q8_linear<PPML_WTYPE_Q8_0M>(W, X, C, M, N, nblk, c_trans, act, xq_dump, sums_dump, s);
         }
         default: set_error("mul_mat_q8_hip: unsupported wtype %d", wtype); return RC_WTYPE;

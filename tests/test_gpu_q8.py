@@ -226,6 +226,15 @@ def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packe
     fast = ops.mul_mat_q8(W, _dev(x), c_trans=1).cpu().numpy()
     assert (fast == out).all()
     if not packed:
+        # a weight as the reference stores it: under 1024 tokens or more it is packed into the stream's workspace per call
+        # and served by the kernels of the packed layout, where they have an instance; else the general kernel
+        if N >= 1024 and _has_low_latency_instance(K, M) and N <= 4096:
+            assert ops.last_q8_path() == "low-latency"
+        elif N >= 1024 and _has_resident_weight_instance(K, M):
+            assert ops.last_q8_path() == "weight-stationary"
+        else:
+            assert ops.last_q8_path() == "general"
+        assert (ops.mul_mat_q8(W, _dev(x), c_trans=1, path="general").cpu().numpy() == out).all()
         assert ops.last_q8_path() == "general"
         return
     # a packed weight: every kernel family that has an instance for the shape, dump form and fast form
