@@ -169,11 +169,13 @@ def main() -> int:
                 best = ev_ if best is None else min(best, ev_)
         return round(best * 1e6, 2)
 
-    def q8_case(rows, K, N, relu=False):
+    def q8_case(rows, K, N, relu=False, packed=True):
         nbytes = q8_bytes(rows, K, N)
         nsets = max(2, int(640e6 // nbytes) + 1)
         w = torch.randn(N, K, device=dev, generator=gen) * 0.02
-        W = ops.Q8Weight.from_f32(w).pack()
+        W = ops.Q8Weight.from_f32(w)                    # block_q8_0 records, as the reference's loader leaves them
+        if packed:
+            W = W.pack()
         xs = [torch.randn(rows, K, device=dev, generator=gen) for _ in range(nsets)]
         ys = [torch.empty(rows, N, device=dev) for _ in range(nsets)]
         lib, cabi = ops._lib(), ops.cabi
@@ -282,6 +284,15 @@ def main() -> int:
                            "bytes_only_us": bytes_only_us(r * k * 4 + n * k * 34 // 32, r * n * 4, steps, warm)}
             if cpu_pair is not None:
                 extra[name]["cpu_baseline"] = q8_cpu(w_dev, x_dev, relu, no, f"the whole {r}x{k}->{n} workload")
+
+        # the headline shape on a weight in the reference's own layout (block_q8_0 records): the library packs it into
+        # its workspace per call and runs the same kernel
+        if not args.configured_shapes_only:
+            f, ns, nb, no, _ = q8_case(26368, 256, 768, packed=False)
+            w_, e_ = time_op(f, ns, steps, warm)
+            extra["msa_qkv_on_a_block_q8_0_weight_26368x256_768"] = {
+                "us": round(e_ * 1e6, 2), "TOPS": round(no / e_ / 1e12, 2), "GBps": round(nb / e_ / 1e9, 1),
+                "hbm_frac": round(nb / e_ / 1e9 / HBM_PEAK_GBS, 4), "kernel": ops.last_q8_path(), "event_steps": time_op.last["event_steps"]}
 
         # a compute-bound shape of the same operator (no shape of the reference's model is one: its quantized
         # projections all have K <= 512): large weights take the tiled kernel, measured against the int8 matrix peak
