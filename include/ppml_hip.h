@@ -121,8 +121,9 @@ int q8_weight_pack_hip(const void *W, int wtype, int M, int K, void *packed,
  * (1.06 bytes per element, fragment order) from the stream-ordered pool mul_mat_hip describes -- the only
  * kernel family of this entry point that uses memory beyond its arguments; without a workspace the general
  * kernel serves the call.  A weight of wtype 0, 1 or 2 beyond 256 Ki elements takes it too, packed into the same
- * workspace on the way (1.06 bytes per element more); a smaller one, under 1024 tokens or more, is packed into the
- * workspace per call as well (one launch) and served by the kernels of wtype 3 where they have an instance. */
+ * workspace on the way (1.06 bytes per element more); a smaller one is packed into the workspace per call as well
+ * (one launch, 3.7 us) and served by the kernels of wtype 3, where they have an instance and the call is large enough
+ * for that launch to pay (2^27 products; 64 Ki weight elements with K >= 512 or 768 features at any token count). */
 int mul_mat_q8_hip(const void *W, const float *X, float *C, int M, int N, int K, int wtype,
                    int c_trans, int *path_out, ppml_hip_stream_t stream);
 

@@ -2019,18 +2019,20 @@ extern "C" int mul_mat_q8_ex_hip(const void* W, const float* X, float* C, int M,
     };
     // A weight in one of the reference's own layouts (include/ppml/QuantBlocks.h:33-41, 123-133) need not wait for its
     // owner to adopt the packed one.  Beyond what stays resident it takes the tiled kernel, which packs it into its
-    // workspace on the way.  Up to that size, under 1024 tokens or more, it is packed into the stream's workspace here
-    // (one launch, a few microseconds) and served by the kernels of the packed layout: us on a Q8_0 weight, general
-    // kernel / this way (timed through the Python operator, 9 us of host time per call): 26368 x 256 -> 768  60 / 26,
-    // 26368 x 256 -> 256  28 / 13, 26368 x 512 -> 128  30 / 19, 10609 x 128 -> 512  16 / 12, 10609 x 256 -> 768  32 / 14.
-    // Through this entry point directly the first of these takes 22.9 us, against 20.8 on a weight packed at load.
-    // With fewer tokens the launch costs what the better kernel saves.  No workspace (a stream under capture): the
-    // general kernel, as before.
+    // workspace on the way.  Up to that size it is packed into the stream's workspace here (one launch: 3.7 us more
+    // than the call on a packed weight) and served by the kernels of the packed layout, wherever that launch costs less
+    // than the general kernel loses: from 2^27 products on, and for weights of 64 Ki elements with K >= 512 or 768
+    // features whatever the token count.  us on a Q8_0 weight, general kernel / this way: 26368 x 256 -> 768  60 / 22.9
+    // (20.8 on a weight packed at load), 26368 x 256 -> 256  26.8 / 12.3, 105472 x 64 -> 256  39.6 / 21.9, 10609 x 64 ->
+    // 256  8.1 / 7.1, 2601 x 256 -> 256  8.4 / 7.0, 64 x 512 -> 128  14.0 / 7.8, 128 x 256 -> 768  16.7 / 9.8; below the
+    // rule: 5000 x 64 -> 256  5.5 / 6.9, 26368 x 64 -> 64  6.6 / 7.2, 1024 x 128 -> 128  5.6 / 7.8.  No workspace (a stream
+    // under capture): the general kernel, as before.
     if (wtype == PPML_WTYPE_Q8_0 || wtype == PPML_WTYPE_Q8_1 || wtype == PPML_WTYPE_Q8_0R) {
         if (static_cast<int64_t>(M) * K > (256 << 10)) {
             const int rt = tiled();
             if (rt >= 0) return rt;
-        } else if (N >= 1024 && !xq_dump && !sums_dump &&
+        } else if ((static_cast<int64_t>(N) * M * K >= (1LL << 27) || (static_cast<int64_t>(M) * K >= (64 << 10) && (K >= 512 || M >= 768))) &&
+                   !xq_dump && !sums_dump &&
                    (flags & (PPML_Q8_FLAG_NO_LOW_LATENCY | PPML_Q8_FLAG_NO_WEIGHT_STATIONARY)) != (PPML_Q8_FLAG_NO_LOW_LATENCY | PPML_Q8_FLAG_NO_WEIGHT_STATIONARY)) {
             const Workspace held = workspace_take(q8_weight_packed_bytes_hip(M, K), s);
             if (held.ptr) {

@@ -226,11 +226,13 @@ def test_fused_linear_bit_exact_internals_and_output(ops, oracle, N, K, M, packe
     fast = ops.mul_mat_q8(W, _dev(x), c_trans=1).cpu().numpy()
     assert (fast == out).all()
     if not packed:
-        # a weight as the reference stores it: under 1024 tokens or more it is packed into the stream's workspace per call
-        # and served by the kernels of the packed layout, where they have an instance; else the general kernel
-        if N >= 1024 and _has_low_latency_instance(K, M) and N <= 4096:
+        # a weight as the reference stores it: where one more launch costs less than the general kernel loses (from 2^27
+        # products on; weights of 64 Ki elements with K >= 512 or 768 features at any token count) it is packed into the
+        # stream's workspace per call and served by the kernels of the packed layout, where they have an instance
+        repacked = N * M * K >= 2 ** 27 or (M * K >= 64 * 1024 and (K >= 512 or M >= 768))
+        if repacked and _has_low_latency_instance(K, M) and N <= 4096:
             assert ops.last_q8_path() == "low-latency"
-        elif N >= 1024 and _has_resident_weight_instance(K, M):
+        elif repacked and _has_resident_weight_instance(K, M):
             assert ops.last_q8_path() == "weight-stationary"
         else:
             assert ops.last_q8_path() == "general"
@@ -700,8 +702,10 @@ def test_fused_linear_with_q8_1_activations(ops, oracle, wname, N, K, M, c_trans
     # without the dump, and the two rules really differ
     y2 = ops.mul_mat_q8(W, _dev(x), c_trans=c_trans, act="q8_1").cpu().numpy()
     assert (y2 == want).all()
-    # a packed weight gets the resident-weight kernels under this rule too, in either orientation
-    assert (ops.last_q8_path() != "general") == (wname == "packed")
+    # a packed weight gets the resident-weight kernels under this rule too, in either orientation -- and so does a weight in
+    # one of the reference's layouts where the library packs it per call (here: K = 512, and 768 features)
+    repacked = N * M * K >= 2 ** 27 or (M * K >= 64 * 1024 and (K >= 512 or M >= 768))
+    assert (ops.last_q8_path() != "general") == (wname == "packed" or repacked)
     if wname == "packed" and c_trans == 1:
         for fam in ("weight-stationary", "weight-stationary-column-parts", "low-latency-8", "low-latency-16", "low-latency-32"):
             if fam.startswith("low") and (not _has_low_latency_instance(K, M) or (fam.endswith("32") and K != 512)):
