@@ -84,3 +84,28 @@ def test_mulmat_stats_switch_and_empty_table_need_no_gpu():
     finally:
         lib.ppml_hip_mulmat_stats_enable(before)
     assert ctypes.sizeof(cabi.MulMatStat) == 32 + 4 * 8 + 8
+
+
+def test_q8_path_and_flag_constants_match_the_header():
+    """The Python operator's names for the kernel families and its flag words are the header's enumerators."""
+    from proteinpredictmachinelearning_amd import ops
+
+    text = open(os.path.join(ROOT, "include", "ppml_hip.h")).read()
+    enums = {name: int(value) for name, value in re.findall(r"\b(PPML_Q8_(?:PATH|FLAG)_\w+)\s*=\s*(\d+)", text)}
+    paths = {v: k for k, v in enums.items() if k.startswith("PPML_Q8_PATH_")}
+    assert sorted(paths) == sorted(ops.Q8_PATH_NAMES) == [0, 1, 2, 3]
+    for value, name in ops.Q8_PATH_NAMES.items():
+        assert paths[value] == "PPML_Q8_PATH_" + name.upper().replace("-", "_"), (value, name)
+    flag = lambda n: enums["PPML_Q8_FLAG_" + n]
+    fl = ops._Q8_PATH_FLAGS
+    assert fl["auto"] == 0
+    assert fl["weight-stationary"] == flag("NO_LOW_LATENCY")
+    assert fl["tiled"] == flag("NO_LOW_LATENCY") | flag("NO_WEIGHT_STATIONARY")
+    assert fl["general"] == flag("NO_LOW_LATENCY") | flag("NO_WEIGHT_STATIONARY") | flag("NO_TILED")
+    assert (fl["low-latency-8"], fl["low-latency-16"], fl["low-latency-32"]) == (flag("LOW_LATENCY_8"), flag("LOW_LATENCY_16"), flag("LOW_LATENCY_32"))
+    assert fl["weight-stationary-column-parts"] == flag("NO_LOW_LATENCY") | flag("COLUMN_PARTS")
+    assert fl["weight-stationary-whole"] == flag("NO_LOW_LATENCY") | flag("NO_COLUMN_PARTS")
+    # every flag is its own bit (the three-way low-latency field aside), none collides with ReLU or the Q8_1 rule
+    singles = [flag(n) for n in ("RELU", "Q8_1_ACTIVATIONS", "NO_LOW_LATENCY", "NO_WEIGHT_STATIONARY", "LOW_LATENCY_8", "LOW_LATENCY_16",
+                                 "COLUMN_PARTS", "NO_COLUMN_PARTS", "NO_TILED")]
+    assert sorted(singles) == [1 << i for i in range(9)]
