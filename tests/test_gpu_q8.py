@@ -453,6 +453,51 @@ def test_tiled_kernel_on_the_references_weight_layouts(ops, oracle):
         assert ops.last_q8_path() == "general" and (out.cpu().numpy() == want).all(), wtype
 
 
+def test_workspace_paths_from_several_threads_and_streams(ops):
+    """The tiled kernel's quantized activations and the per-call repack of a weight in the reference's layouts live in the
+    stream's kept workspace: calls from several host threads, each on a stream of its own, and from two threads that
+    share one stream, with sizes that make the buffer grow and shrink in turn, give the bits of the same calls made one
+    after the other."""
+    import threading
+    g = torch.Generator(device="cuda").manual_seed(31)
+    cases = []
+    for N, K, M, pack in ((600, 1024, 1024, True), (3000, 256, 768, False), (408, 2048, 2048, False), (300, 256, 256, True),
+                          (2100, 128, 2050, True)):
+        W = ops.Q8Weight.from_f32(torch.randn(M, K, device="cuda", generator=g) * 0.02)
+        if pack:
+            W = W.pack()
+        x = torch.randn(N, K, device="cuda", generator=g)
+        ref = ops.mul_mat_q8(W, x).clone()
+        cases.append((W, x, ref, ops.last_q8_path()))
+    assert [c[3] for c in cases] == ["tiled", "weight-stationary", "tiled", "low-latency", "weight-stationary"]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    errors = []
+
+    def work(stream, seed):
+        try:
+            rng = np.random.default_rng(seed)
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    i = int(rng.integers(len(cases)))
+                    W, x, ref, _ = cases[i]
+                    out = ops.mul_mat_q8(W, x)
+                    stream.synchronize()
+                    if not torch.equal(out.view(torch.int32), ref.view(torch.int32)):
+                        errors.append((seed, i))
+        except Exception as e:                         # noqa: BLE001 -- reported below
+            errors.append((seed, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(streams[0], 1)), threading.Thread(target=work, args=(streams[1], 2)),
+               threading.Thread(target=work, args=(streams[2], 3)), threading.Thread(target=work, args=(streams[2], 4))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+
+
 def test_a_call_on_a_capturing_stream_takes_no_workspace(ops):
     """The tiled kernel's workspace comes from the stream-ordered pool, and a stream under capture gets none (what is
     allocated while a graph is recorded is gone before the graph runs): a call recorded into a graph takes the
