@@ -312,7 +312,8 @@ def test_every_weight_stationary_instance_has_a_shape_in_the_suite():
     assert len(WS_INSTANCE_SHAPES) == 13
 
 
-@pytest.mark.parametrize("N,K,M", [(408, 256, 256), (100, 96, 100), (70, 128, 800)])
+@pytest.mark.parametrize("N,K,M", [(408, 256, 256), (100, 96, 100), (70, 128, 800),
+                                   (300, 512, 128), (2100, 256, 768)])      # the last two: packed per call by the library
 def test_weight_layouts_and_output_orientations_agree(ops, oracle, N, K, M):
     x, w = _inputs(11 * N + M, N, K, M)
     wq = oracle.quantize_q8_0(w)
@@ -323,9 +324,11 @@ def test_weight_layouts_and_output_orientations_agree(ops, oracle, N, K, M):
         ops.WTYPE_Q8_1: _q8_1_from_q8_0(wq).reshape(-1),
         ops.WTYPE_Q8_0R: oracle.repack_q8_0(wq),
     }
+    repacked = N * M * K >= 2 ** 27 or (M * K >= 64 * 1024 and (K >= 512 or M >= 768))
     for wtype, data in layouts.items():
         W = ops.Q8Weight(_dev(data), M, K, wtype)
         assert (ops.mul_mat_q8(W, xd, c_trans=1).cpu().numpy() == want).all(), wtype
+        assert (ops.last_q8_path() != "general") == repacked, wtype
         assert (ops.mul_mat_q8(W, xd, c_trans=0).cpu().numpy() == want.T).all(), wtype
         Wm = W.pack()
         tiles = (((M + 31) // 32) + 1) // 2 * 2          # the packed layout holds an even number of 32-row tiles
